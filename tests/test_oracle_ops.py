@@ -218,9 +218,9 @@ def test_adamw_vs_torch_and_clip_rule():
     big = 3 * r(n)
     nrm = np.linalg.norm(big)
     b2 = big.copy()
-    ret = oracle.lib(P).or_clip_grad_norm(b2.ctypes.data, oracle.C.c_size_t(n), oracle.C.c_float(1.0))
+    ret = op(P, "or_clip_grad_norm", b2, SZ(n), 1.0)
     assert abs(ret - nrm) < 1e-12 and abs(np.linalg.norm(b2) - 1.0) < 1e-6
     small = big / (2 * nrm)
     s2 = small.copy()
-    oracle.lib(P).or_clip_grad_norm(s2.ctypes.data, oracle.C.c_size_t(n), oracle.C.c_float(1.0))
+    op(P, "or_clip_grad_norm", s2, SZ(n), 1.0)
     assert np.array_equal(s2, small)                        # norm <= 1: untouched
