@@ -1,0 +1,136 @@
+/*
+ * fast_hip.h — C ABI of the MI355X (gfx950) backend for llm.metal's fast
+ * training pipelines.
+ *
+ * This is the drop-in boundary: it exports the symbols the reference's
+ * src/nn/fast_metal.h declares (same names, argument order and meaning as the
+ * reference CALL SITES use them), implemented by hand-written HIP kernels on
+ * one in-order stream.  Reference callers (src/nn/wmat.c, fast_sft.c,
+ * fast_grpo.c) link against this library instead of fast_metal.m.
+ *
+ * Conventions kept from the reference (src/nn/fast_metal.m):
+ *   - fast_metal_init returns 0 / -1 and is reference counted (:69-76,171);
+ *     every other function is void and silent;
+ *   - enqueues execute in program order, each seeing the previous one's
+ *     writes (:231-233); metal_flush blocks until everything has run (:235-249);
+ *   - in == out aliasing is allowed where the reference relies on it
+ *     (rms_norm, rms_norm_backward, silu/gelu_mul_backward with dgate == dout).
+ * Differences forced by a discrete GPU are listed at metal_buf_ptr.
+ *
+ * Not exported yet: the 16 inference-only enqueues (q8_matvec, f16_matvec,
+ * f16_batch_matvec, rms_norm (single), per_head_rms_norm, rope,
+ * kv_cache_store, attention and the _off variants; src/nn/fast_metal.h:20-80).
+ */
+#ifndef FAST_HIP_H
+#define FAST_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* src/nn/fast_metal.h:8-9.  Fails (-1, message on stderr) when no gfx950
+ * device is present; there is no CPU fallback. */
+int  fast_metal_init(void);
+void fast_metal_shutdown(void);
+
+/* src/nn/fast_metal.h:12-17 */
+typedef struct MetalBuf MetalBuf;
+MetalBuf *metal_buf_create(size_t size);                    /* uninitialised device memory */
+MetalBuf *metal_buf_from_data(const void *data, size_t sz); /* copies; caller keeps `data` */
+void      metal_buf_free(MetalBuf *b);                      /* NULL is a no-op */
+/* Returns a CPU pointer valid for the buffer's lifetime and coherent at
+ * metal_flush boundaries, as the reference's shared-storage buffers are.
+ * On first use the buffer MIGRATES to pinned, device-mapped host memory and
+ * stays there: kernels then reach it over the host link.  Meant for the small
+ * CPU-touched buffers (inputs, targets, losses, GRPO actions); for bulk data
+ * use metal_buf_read / metal_buf_write, which leave the buffer in HBM. */
+void     *metal_buf_ptr(MetalBuf *b);
+
+/* Extensions (no counterpart in the reference): explicit staging that keeps
+ * the buffer in HBM.  Both order themselves after all enqueued work. */
+void   metal_buf_read(MetalBuf *b, size_t offset, void *dst, size_t n);
+void   metal_buf_write(MetalBuf *b, size_t offset, const void *src, size_t n);
+size_t metal_buf_size(MetalBuf *b);
+/* Non-owning window [offset, offset+size) of another buffer. */
+MetalBuf *metal_buf_view(MetalBuf *parent, size_t offset, size_t size);
+
+/* src/nn/fast_metal.h:83 */
+void metal_flush(void);
+
+/* ---- enqueues shared with inference (src/nn/fast_metal.h:36-61) ---- */
+void metal_enqueue_rms_norm_batched(MetalBuf *x, MetalBuf *gamma, MetalBuf *out,
+                                    int dim, float eps, int B);
+void metal_enqueue_silu_mul(MetalBuf *gate, MetalBuf *up, int n);
+void metal_enqueue_gelu_mul(MetalBuf *gate, MetalBuf *up, int n);
+void metal_enqueue_residual_add(MetalBuf *x, MetalBuf *y, int n);
+
+/* ---- training enqueues (src/nn/fast_metal.h:88-188) ----
+ * Argument ORDER follows the reference's implementation and call sites
+ * (src/nn/fast_metal.m:562-594, src/nn/fast_sft.c:638): the first buffer is the
+ * fp32 activation, the second the F16 weight, whatever the header names say. */
+
+/* C[M,N] fp32 = A[M,K] fp32 * W[N,K]^T, W F16 row-major. */
+void metal_enqueue_f16_matmul(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, int N, int K);
+/* C[M,K] fp32 = A[M,N] fp32 * W[N,K], W F16 row-major. */
+void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, int N, int K);
+void metal_enqueue_transpose_heads_fwd(MetalBuf *src, MetalBuf *dst, int seq_len, int n_heads, int head_dim);
+void metal_enqueue_transpose_heads_rev(MetalBuf *src, MetalBuf *dst, int seq_len, int n_heads, int head_dim);
+void metal_enqueue_repeat_kv(MetalBuf *src, MetalBuf *dst, int n_kv, int seq_len, int head_dim, int group_ratio);
+void metal_enqueue_rope_train(MetalBuf *q, MetalBuf *k, int Hq, int Hkv, int hd, int seq_len, float theta);
+void metal_enqueue_silu_mul_backward(MetalBuf *dout, MetalBuf *gate, MetalBuf *up,
+                                     MetalBuf *dgate, MetalBuf *dup, int n);
+void metal_enqueue_gelu_mul_backward(MetalBuf *dout, MetalBuf *gate, MetalBuf *up,
+                                     MetalBuf *dgate, MetalBuf *dup, int n);
+void metal_enqueue_rms_norm_backward(MetalBuf *x, MetalBuf *dy, MetalBuf *gamma, MetalBuf *dx,
+                                     int batch, int dim, float eps);
+void metal_enqueue_scale(MetalBuf *x, float alpha, int n);
+void metal_enqueue_add_scaled(MetalBuf *y, MetalBuf *x, float alpha, int n);
+void metal_enqueue_softmax_ce(MetalBuf *logits, MetalBuf *targets, MetalBuf *losses,
+                              MetalBuf *dlogits, int batch, int vocab_size);
+void metal_enqueue_attn_train_fwd(MetalBuf *Q, MetalBuf *K, MetalBuf *V, MetalBuf *out, MetalBuf *probs,
+                                  int H, int N, int D, float scale);
+void metal_enqueue_attn_bwd_dq(MetalBuf *d_out, MetalBuf *probs, MetalBuf *V, MetalBuf *K,
+                               MetalBuf *d_score, MetalBuf *dQ, int H, int N, int D, float scale);
+void metal_enqueue_attn_bwd_dkv(MetalBuf *d_score, MetalBuf *Q, MetalBuf *probs, MetalBuf *d_out,
+                                MetalBuf *dK, MetalBuf *dV, int H, int N, int D);
+void metal_enqueue_repeat_kv_bwd(MetalBuf *d_expanded, MetalBuf *d_kv,
+                                 int n_kv, int seq_len, int head_dim, int group_ratio);
+void metal_enqueue_rope_train_bwd(MetalBuf *q, MetalBuf *k, int Hq, int Hkv, int hd, int seq_len, float theta);
+/* fp32 LoRA products: C[M,N] = A[M,K] W[N,K]^T;  C[M,N] = A[K,M]^T B[K,N];  C[M,K] = A[M,N] W[N,K]. */
+void metal_enqueue_float_matmul(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, int N, int K);
+void metal_enqueue_float_matmul_tn(MetalBuf *A, MetalBuf *B, MetalBuf *C, int M, int N, int K);
+void metal_enqueue_float_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, int N, int K);
+void metal_enqueue_copy(MetalBuf *src, MetalBuf *dst, int n);
+void metal_enqueue_clamp(MetalBuf *x, float max_val, int n);
+/* W[M,N] F16 -= lr * dY[K,M]^T X[K,N] */
+void metal_enqueue_f16_sgd_fused(MetalBuf *W, MetalBuf *dY, MetalBuf *X, int M, int K, int N, float lr);
+void metal_enqueue_grpo_policy_grad(MetalBuf *logits, MetalBuf *actions, MetalBuf *old_lp, MetalBuf *advs,
+                                    MetalBuf *new_lp, MetalBuf *dlogits, int N, int V, float clip_eps);
+/* G[M,N] F16 += dY[K,M]^T X[K,N], one rounding per call */
+void metal_enqueue_f16_grad_accum(MetalBuf *G, MetalBuf *dY, MetalBuf *X, int M, int K, int N);
+void metal_enqueue_f16_sgd_apply(MetalBuf *W, MetalBuf *G, int n, float lr);
+
+/* ---- extensions used by the weight container ---- */
+/* dst F16 [n] = round-to-nearest-even(src fp32 [n]); wmat_create_f16, src/nn/wmat.c:63-75 */
+void hip_enqueue_f32_to_f16(MetalBuf *src, MetalBuf *dst, size_t n);
+/* dst Q8_0 blocks (34 B each) from src fp32 [rows, cols]; quantize_row_q8, src/nn/wmat.c:19-44 */
+void hip_enqueue_q8_quantize(MetalBuf *src, MetalBuf *dst, int rows, int cols);
+/* dst fp32 [rows, cols] = float(scale) * code; src/data/gguf.c:225-253 */
+void hip_enqueue_q8_dequant(MetalBuf *src, MetalBuf *dst, int rows, int cols);
+/* dst F16 [rows, cols] = half(float(scale) * code): the values the dequant-fused GEMM multiplies with */
+void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
+
+/* Timing aid for benchmarks: when enabled, every launch of the weight-streaming
+ * GEMM is bracketed by HIP events on the library's stream.  hip_gemm_profile_read
+ * (after metal_flush) returns the number of launches recorded since the last
+ * enable and adds up their durations (ms) and weight bytes. */
+void hip_gemm_profile_enable(int on);
+int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FAST_HIP_H */

@@ -1,0 +1,138 @@
+/*
+ * sft_hip.h — host API of the fused LoRA SFT step on MI355X.
+ *
+ * Keeps the reference's C host API for this path: the weight container of
+ * src/nn/wmat.h and the SFTState functions of src/nn/fast_sft.h, with the same
+ * names, argument meaning and error behaviour (constructors return NULL when
+ * the backend cannot start; everything else is silent).  What differs:
+ *
+ *  - State is built from the reference's own model-independent description
+ *    (LayerWeightRef, src/nn/wmat.h:39-56) wrapped in SFTModelRef, not from
+ *    Qwen3Model / Gemma3Model: those structs belong to the reference's CPU
+ *    tensor runtime.  The two-line adapters that fill an SFTModelRef from them
+ *    are shown in INTEGRATION.md.
+ *  - `batch` sequences per step (the reference has batch 1): RoPE positions and
+ *    causal attention restart at every sequence.
+ *  - Embedding gather, loss scaling, global-norm clipping and AdamW run on the
+ *    device; the host touches only tokens, targets and the per-row losses.
+ */
+#ifndef SFT_HIP_H
+#define SFT_HIP_H
+
+#include "fast_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- src/nn/wmat.h:10-78 ---- */
+typedef enum { MODEL_QWEN3, MODEL_GEMMA3 } ModelType;
+
+typedef struct WMat {
+    MetalBuf *mbuf;
+    int rows, cols, nb;            /* nb = cols/32, Q8_0 only */
+} WMat;
+
+typedef struct {
+    WMat *q_proj, *k_proj, *v_proj, *o_proj;
+    WMat *gate_proj, *up_proj, *down_proj;
+    MetalBuf *input_norm_g, *post_attn_norm_g;
+    MetalBuf *pre_ff_norm_g, *post_ff_norm_g;   /* Gemma3 only */
+    MetalBuf *q_norm_g, *k_norm_g;
+} LayerW;
+
+typedef struct { const float *data; int rows, cols; } WeightRef;
+
+typedef struct {
+    WeightRef q_proj, k_proj, v_proj, o_proj;
+    WeightRef gate_proj, up_proj, down_proj;
+    const float *input_norm_g;
+    const float *post_attn_norm_g;
+    const float *pre_ff_norm_g;    /* Gemma3 only */
+    const float *post_ff_norm_g;   /* Gemma3 only */
+    const float *q_norm_g;
+    const float *k_norm_g;
+    int d_model;
+    int head_dim;
+} LayerWeightRef;
+
+WMat *wmat_create_f16(const float *src, int rows, int cols);   /* src/nn/wmat.c:63-75, bit-identical */
+WMat *wmat_create_q8(const float *src, int rows, int cols);    /* src/nn/wmat.c:46-61, bit-identical */
+void  wmat_free(WMat *w);
+LayerW *layers_convert_upload(const LayerWeightRef *refs, int n_layers, int use_fp16);
+void  layers_free(LayerW *layers, int n_layers);
+WMat *wmat_convert(const float *data, int rows, int cols, int use_fp16);
+MetalBuf *norm_upload(const float *gamma, int dim);
+
+/* ---- model description (replaces the Qwen3Model / Gemma3Model arguments of
+ *      sft_state_create*, src/nn/fast_sft.c:171-396) ---- */
+typedef struct {
+    ModelType model_type;
+    int n_layers, d_model, n_q_heads, n_kv_heads, head_dim, intermediate_size, vocab_size;
+    const float *rope_thetas;          /* [n_layers]; Gemma3: global on layers with L % 6 == 0 */
+    const LayerWeightRef *layers;      /* [n_layers], fp32 host arrays */
+    const float *token_emb;            /* [vocab, d_model] fp32 */
+    const float *lm_head;              /* [vocab, d_model] fp32; Gemma3 passes token_emb (tied) */
+    const float *final_norm_g;         /* [d_model] */
+    /* optional initial adapters, flat per layer A_q[R,D] | B_q[Hq*hd,R] | A_v[R,D] | B_v[Hkv*hd,R];
+     * NULL: A ~ U(-1,1)/sqrt(D) from rand(), B = 0 (src/nn/fast_sft.c:89-131) */
+    const float *lora_init;
+} SFTModelRef;
+
+typedef struct SFTState SFTState;
+
+/* weight_format: 1 = F16 frozen weights, 0 = Q8_0 (quantised with the reference's
+ * algorithm; the GEMMs multiply with the dequantised values). */
+SFTState *sft_state_create_from_ref(const SFTModelRef *model, int batch, int seq_len,
+                                    int lora_rank, float lora_alpha, int weight_format);
+void sft_state_free(SFTState *state);
+
+/* src/nn/fast_sft.h:43-49; tokens are [batch*seq_len] */
+float sft_train_step(SFTState *state, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr);
+
+/* src/nn/fast_sft.h:57-63: embeddings must be in sft_get_x_cpu's buffer */
+void forward_to_logits(SFTState *state);
+void sft_backward(SFTState *state);            /* consumes sft_get_dlogits (fp32 [BN, V]) */
+void sft_lora_update(SFTState *state, float lr);
+
+MetalBuf *sft_get_logits(SFTState *state);
+MetalBuf *sft_get_dlogits(SFTState *state);
+float *sft_get_x_cpu(SFTState *state);
+float *sft_get_losses_cpu(SFTState *state);
+int sft_get_seq_len(SFTState *state);          /* rows per step = batch * seq_len, as callers size by it */
+int sft_get_vocab_size(SFTState *state);
+int sft_get_d_model(SFTState *state);
+int sft_get_lora_rank(SFTState *state);
+int sft_get_n_layers(SFTState *state);
+float sft_get_emb_scale(SFTState *state);
+int sft_get_step_count(SFTState *state);
+void sft_set_step_count(SFTState *state, int step);
+int sft_get_n_lora_grad_bufs(SFTState *state);
+float *sft_get_lora_grad_ptr(SFTState *state, int idx, int *out_size);
+void sft_set_lora_grad(SFTState *state, int idx, const float *data, int size);
+MetalBuf *sft_get_lora_weight_buf(SFTState *state, int layer, int sub);
+float sft_get_lora_scaling(SFTState *state);
+ModelType sft_get_model_type(SFTState *state);
+int sft_get_n_q_heads(SFTState *state);
+int sft_get_n_kv_heads(SFTState *state);
+int sft_get_head_dim(SFTState *state);
+int sft_get_intermediate_size(SFTState *state);
+const float *sft_get_rope_thetas(SFTState *state);
+int sft_is_full_param(SFTState *state);
+/* "LORA" adapter file, src/nn/fast_sft.c:1255-1285 */
+void sft_save_lora(SFTState *state, const char *path);
+
+/* Extensions: bulk copies that leave the adapters in HBM (flat layout as lora_init). */
+size_t sft_lora_numel(SFTState *state);
+void sft_copy_lora(SFTState *state, float *dst);
+void sft_copy_lora_grads(SFTState *state, float *dst);
+void sft_set_lora(SFTState *state, const float *src);
+float sft_get_last_grad_norm(SFTState *state);
+/* Enqueue forward + loss + backward + update without waiting (sft_train_step = this + flush + mean). */
+void sft_enqueue_train_step(SFTState *state, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr);
+float sft_finish_train_step(SFTState *state);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SFT_HIP_H */

@@ -1,0 +1,53 @@
+// Internal header of the HIP backend: buffer handle layout, the library's one
+// stream, scratch arenas and launch-time checks shared by the translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include "../../include/fast_hip.h"
+
+struct MetalBuf {
+    void   *dev;          // address kernels use (HBM, or the device view of pinned host memory)
+    void   *host;         // pinned host allocation once metal_buf_ptr has been called, else NULL
+    size_t  size;
+    int     owns;         // 0 for views
+    MetalBuf *parent;     // views: the buffer whose allocation this window lies in
+    size_t  parent_off;
+    // lazily built transposed F16 copy used by metal_enqueue_f16_matmul_nt
+    void   *t_dev;
+    int     t_rows, t_cols;
+    uint64_t t_version;   // version of `dev` contents the copy was made from
+    uint64_t version;     // bumped by every enqueue that writes this buffer
+};
+
+namespace lmhip {
+
+hipStream_t stream();
+int  initialized();
+int  num_cus();
+void die(const char *what, hipError_t e, const char *file, int line);
+
+// Grow-only device scratch, one arena per purpose; contents are only valid
+// within the enqueue that asked for them.
+enum ScratchSlot { SCR_A16 = 0, SCR_SCALE, SCR_PARTIAL, SCR_MISC, SCR_COUNT };
+void *scratch(ScratchSlot slot, size_t bytes);
+
+// Device address of a buffer; views resolve through their parent so that they
+// follow it when metal_buf_ptr migrates the allocation to host memory.
+inline void *dptr(const MetalBuf *b) { return b->parent ? (void *)((char *)b->parent->dev + b->parent_off) : b->dev; }
+template <typename T> inline T *dptr_as(const MetalBuf *b) { return (T *)dptr(b); }
+
+inline void mark_written(MetalBuf *b) { if (b) { b->version++; if (b->parent) b->parent->version++; } }
+
+}  // namespace lmhip
+
+#define LMHIP_API extern "C" __attribute__((visibility("default")))
+#define HIP_CHECK(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) lmhip::die(#expr, e_, __FILE__, __LINE__); } while (0)
+
+// Host-side guard against launching on operands smaller than the kernel will touch.
+#define REQUIRE_BYTES(buf, bytes, fn) do { \
+    if (!(buf) || (buf)->size < (size_t)(bytes)) { \
+        fprintf(stderr, "[fast_hip] %s: buffer %s too small (%zu < %zu bytes); launch skipped\n", \
+                fn, #buf, (buf) ? (buf)->size : (size_t)0, (size_t)(bytes)); \
+        return; } } while (0)

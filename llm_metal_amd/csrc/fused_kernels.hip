@@ -1,0 +1,712 @@
+// Fused row / head kernels of the SFT step.  Each one sits between two
+// weight-streaming GEMMs: it sums the producer GEMM's K-split partial planes on
+// load, does the reference's per-row arithmetic in fp32 (shaders/q8_kernels.metal,
+// cited per kernel) and writes what the next GEMM reads as a scaled fp16 row.
+// One launch here replaces between 3 and 12 dispatches of the reference's
+// forward_to_logits / sft_backward_ex (src/nn/fast_sft.c:616-982).
+#include "fused.h"
+
+namespace lmhip {
+namespace {
+
+constexpr int TB = 256;
+
+__device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
+{
+    float s = 0.f;
+    const float *p = P.p + row * P.ld + col;
+    for (int i = 0; i < P.S; i++) s += p[(size_t)i * P.stride];
+    return s;
+}
+
+__device__ __forceinline__ void write_f16_row(const float *vals, int n, half_t *out, int ld, float s)
+{
+    for (int i = threadIdx.x; i < ld; i += blockDim.x) out[i] = (i < n) ? f2h(vals[i] * s) : (half_t)0;
+}
+
+// ------------------------------------------------------------------ forward rows
+// x = (gathered embedding | x_prev) [+ branch | + RN(branch; g_branch)];  ln = RN(x; g_norm).
+// rms_norm: shaders/q8_kernels.metal:133-158; residual_add :369-375; the Gemma3
+// ordering (norm the branch, then add) is src/nn/fast_sft.c:698-705, 732-736.
+__global__ __launch_bounds__(TB) void k_norm_rows(NormRowsArgs a)
+{
+    extern __shared__ float lds[];
+    float *row = lds, *brow = lds + a.D;
+    __shared__ float sm[16];
+    const size_t r = blockIdx.x;
+    const int D = a.D;
+    if (a.emb) {
+        const float *e = a.emb + (size_t)a.tokens[r] * D;
+        for (int i = threadIdx.x; i < D; i += TB) row[i] = (a.emb_scale != 1.0f) ? e[i] * a.emb_scale : e[i];
+    } else {
+        for (int i = threadIdx.x; i < D; i += TB) row[i] = a.x_prev[r * D + i];
+    }
+    if (a.branch.S > 0) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < D; i += TB) { const float b = planes_at(a.branch, r, i); brow[i] = b; ss += b * b; }
+        if (a.g_branch) {
+            ss = block_sum(ss, sm);
+            const float inv = rsqrtf(ss / (float)D + a.eps);
+            for (int i = threadIdx.x; i < D; i += TB) {
+                if (a.branch_raw_out) a.branch_raw_out[r * D + i] = brow[i];
+                row[i] += brow[i] * inv * a.g_branch[i];
+            }
+        } else {
+            for (int i = threadIdx.x; i < D; i += TB) row[i] += brow[i];
+        }
+    }
+    if (a.x_out) for (int i = threadIdx.x; i < D; i += TB) a.x_out[r * D + i] = row[i];
+    if (!a.g_norm) return;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < D; i += TB) ss += row[i] * row[i];
+    ss = block_sum(ss, sm);
+    const float inv = rsqrtf(ss / (float)D + a.eps);
+    float amax = 0.f;
+    for (int i = threadIdx.x; i < D; i += TB) { const float v = row[i] * inv * a.g_norm[i]; brow[i] = v; amax = fmaxf(amax, fabsf(v)); }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    write_f16_row(brow, D, a.ln16 + r * a.ld16, a.ld16, s);   // each thread re-reads only what it wrote
+    if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
+}
+
+// ------------------------------------------------------------------ QKV epilogue
+// One wave per (row, head): sums the fused QKV GEMM planes, adds the LoRA term
+// sc * (x A^T) B^T (add_scaled, src/nn/fast_sft.c:639-644, 651-656), saves the
+// pre-norm head, applies the per-head RMSNorm (src/nn/fast_sft.c:668-669) and the
+// half-split RoPE (rope_train, shaders/q8_kernels.metal:495-538).  Works on the
+// [rows][H*hd] layout, so the reference's three head transposes, repeat_kv and
+// five buffer copies disappear.  A lane owns the pairs (d, d + hd/2).
+constexpr int MAXP = 4;                                   // pairs per lane: hd <= 512
+__global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int HT = a.Hq + 2 * a.Hkv;
+    const size_t task = (size_t)blockIdx.x * 4 + wave;
+    if (task >= (size_t)a.rows * HT) return;            // whole wave leaves together; no block barrier below
+    const size_t row = task / HT;
+    const int slot = (int)(task % HT);
+    const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd;
+    const int kind = slot < a.Hq ? 0 : (slot < a.Hq + a.Hkv ? 1 : 2);     // 0 q, 1 k, 2 v
+    const int h = kind == 0 ? slot : (kind == 1 ? slot - a.Hq : slot - a.Hq - a.Hkv);
+    const int col0 = kind == 0 ? h * hd : (kind == 1 ? qd + h * hd : qd + kd + h * hd);
+    const int t0 = qd + 2 * kd + (kind == 2 ? a.R : 0);
+    const bool lora = a.R > 0 && kind != 1;
+    const float *B = kind == 0 ? a.Bq : a.Bv;
+
+    float tval = 0.f;
+    if (lora && lane < a.R) tval = planes_at(a.qkv, row, t0 + lane);
+    if (lora && h == 0 && lane < a.R) (kind == 0 ? a.tq : a.tv)[row * a.R + lane] = tval;
+
+    float x0[MAXP], x1[MAXP];
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < MAXP; p++) {
+        const int d = lane + 64 * p;
+        x0[p] = x1[p] = 0.f;
+        if (d < half) {
+            x0[p] = planes_at(a.qkv, row, col0 + d);
+            x1[p] = planes_at(a.qkv, row, col0 + d + half);
+        }
+        if (lora) {                                           // uniform branch: shuffles stay convergent
+            float acc0 = 0.f, acc1 = 0.f;
+            for (int r = 0; r < a.R; r++) {
+                const float t = __shfl(tval, r, WAVE);
+                if (d < half) {
+                    acc0 += t * B[(size_t)(h * hd + d) * a.R + r];
+                    acc1 += t * B[(size_t)(h * hd + d + half) * a.R + r];
+                }
+            }
+            x0[p] += a.sc * acc0;
+            x1[p] += a.sc * acc1;
+        }
+        ss += x0[p] * x0[p] + x1[p] * x1[p];
+    }
+    if (kind == 2) {
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int d = lane + 64 * p;
+            if (d < half) { a.v_out[row * kd + h * hd + d] = x0[p]; a.v_out[row * kd + h * hd + d + half] = x1[p]; }
+        }
+        return;
+    }
+    ss = wave_sum(ss);
+    const float inv = rsqrtf(ss / (float)hd + a.eps);
+    const float *g = kind == 0 ? a.g_q : a.g_k;
+    float *pre = kind == 0 ? a.q_pre : a.k_pre, *fin = kind == 0 ? a.q_fin : a.k_fin;
+    const int W = kind == 0 ? qd : kd;
+    const int pos = (int)(row % a.seq);
+#pragma unroll
+    for (int p = 0; p < MAXP; p++) {
+        const int d = lane + 64 * p;
+        if (d >= half) continue;
+        const size_t o = row * W + h * hd + d;
+        pre[o] = x0[p];
+        pre[o + half] = x1[p];
+        const float n0 = x0[p] * inv * g[d], n1 = x1[p] * inv * g[d + half];
+        const float freq = 1.0f / powf(a.theta, (float)(2 * d) / (float)hd);
+        float s, c;
+        sincosf((float)pos * freq, &s, &c);
+        fin[o] = n0 * c - n1 * s;
+        fin[o + half] = n0 * s + n1 * c;
+    }
+}
+
+// ------------------------------------------------------------------ attention
+// attn_train_fwd, shaders/q8_kernels.metal:769-851, on [rows][H*hd] activations
+// with the KV head picked as h / ratio (repeat_kv, :476-492) and one wave per
+// (head, query, sequence).  Output goes straight to the O-projection's fp16 operand.
+__global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
+{
+    extern __shared__ float sc[];                        // [seq] scores/probs, [hd] query
+    const int N = a.seq, hd = a.hd;
+    float *qs = sc + N;
+    const int h = blockIdx.x, i = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int qd = a.Hq * hd, kd = a.Hkv * hd, hk = h / (a.Hq / a.Hkv);
+    const size_t r0 = (size_t)b * N;
+    const float *q = a.q + (r0 + i) * qd + h * hd;
+    for (int d = lane; d < hd; d += 64) qs[d] = q[d];
+    __syncthreads();
+    float mx = -1e30f;
+    for (int j = lane; j <= i; j += 64) {
+        const float4 *kr = reinterpret_cast<const float4 *>(a.k + (r0 + j) * kd + hk * hd);
+        float dot = 0.f;
+        for (int d4 = 0; d4 < hd / 4; d4++) {
+            const float4 kv = kr[d4];
+            dot += qs[4 * d4] * kv.x + qs[4 * d4 + 1] * kv.y + qs[4 * d4 + 2] * kv.z + qs[4 * d4 + 3] * kv.w;
+        }
+        dot *= a.scale;
+        sc[j] = dot;
+        mx = fmaxf(mx, dot);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int j = lane; j <= i; j += 64) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+    float *pr = a.probs + (((size_t)b * a.Hq + h) * N + i) * N;
+    for (int j = lane; j < N; j += 64) {
+        const float p = (j <= i) ? sc[j] * inv : 0.f;
+        sc[j] = p;
+        pr[j] = p;
+    }
+    __syncthreads();
+    for (int d = lane; d < hd; d += 64) {
+        float acc = 0.f;
+        for (int j = 0; j <= i; j++) acc += sc[j] * a.v[(r0 + j) * kd + hk * hd + d];
+        a.out16[(r0 + i) * a.ld16 + h * hd + d] = f2h(acc);
+    }
+}
+
+// attn_bwd_dq, shaders/q8_kernels.metal:857-925.  Also leaves the plane-summed dO
+// row in dO_red for the dK/dV kernel.
+__global__ __launch_bounds__(64) void k_attn_bwd_dq(AttnBwdArgs a)
+{
+    extern __shared__ float dr[];                        // [seq] d_raw/ds, [hd] dO row
+    const int N = a.seq, hd = a.hd;
+    float *dos = dr + N;
+    const int h = blockIdx.x, i = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int qd = a.Hq * hd, kd = a.Hkv * hd, hk = h / (a.Hq / a.Hkv);
+    const size_t r0 = (size_t)b * N;
+    for (int d = lane; d < hd; d += 64) {
+        const float v = planes_at(a.dO, r0 + i, h * hd + d);
+        dos[d] = v;
+        a.dO_red[(r0 + i) * qd + h * hd + d] = v;
+    }
+    __syncthreads();
+    const float *pr = a.probs + (((size_t)b * a.Hq + h) * N + i) * N;
+    float dp = 0.f;
+    for (int j = lane; j <= i; j += 64) {
+        const float4 *vr = reinterpret_cast<const float4 *>(a.v + (r0 + j) * kd + hk * hd);
+        float dot = 0.f;
+        for (int d4 = 0; d4 < hd / 4; d4++) {
+            const float4 vv = vr[d4];
+            dot += dos[4 * d4] * vv.x + dos[4 * d4 + 1] * vv.y + dos[4 * d4 + 2] * vv.z + dos[4 * d4 + 3] * vv.w;
+        }
+        dr[j] = dot;
+        dp += pr[j] * dot;
+    }
+    dp = wave_sum(dp);
+    float *ds = a.dscore + (((size_t)b * a.Hq + h) * N + i) * N;
+    for (int j = lane; j < N; j += 64) {
+        const float v = (j <= i) ? pr[j] * (dr[j] - dp) * a.scale : 0.f;
+        dr[j] = v;
+        ds[j] = v;
+    }
+    __syncthreads();
+    for (int d = lane; d < hd; d += 64) {
+        float acc = 0.f;
+        for (int j = 0; j <= i; j++) acc += dr[j] * a.k[(r0 + j) * kd + hk * hd + d];
+        a.dq[(r0 + i) * qd + h * hd + d] = acc;
+    }
+}
+
+// attn_bwd_dkv + repeat_kv_bwd, shaders/q8_kernels.metal:931-992: one wave per
+// (kv head, key, sequence) sums over the query heads of its group.
+__global__ __launch_bounds__(64) void k_attn_bwd_dkv(AttnBwdArgs a)
+{
+    const int N = a.seq, hd = a.hd, ratio = a.Hq / a.Hkv;
+    const int hk = blockIdx.x, j = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int qd = a.Hq * hd, kd = a.Hkv * hd;
+    const size_t r0 = (size_t)b * N;
+    for (int d = lane; d < hd; d += 64) {
+        float dk = 0.f, dv = 0.f;
+        for (int g = 0; g < ratio; g++) {
+            const int h = hk * ratio + g;
+            const size_t pbase = ((size_t)b * a.Hq + h) * N * N;
+            for (int i = j; i < N; i++) {
+                const float ds = a.dscore[pbase + (size_t)i * N + j];
+                const float p = a.probs[pbase + (size_t)i * N + j];
+                dk += ds * a.q[(r0 + i) * qd + h * hd + d];
+                dv += p * a.dO_red[(r0 + i) * qd + h * hd + d];
+            }
+        }
+        a.dk[(r0 + j) * kd + hk * hd + d] = dk;
+        a.dv[(r0 + j) * kd + hk * hd + d] = dv;
+    }
+}
+
+// ------------------------------------------------------------------ QKV backward rows
+// Per row: inverse RoPE (rope_train_bwd, shaders/q8_kernels.metal:997-1038), QK-norm
+// backward (rms_norm_train_backward :584-625 on rows of hd), dh = sc * dq B
+// (float_matmul_nt + scale, src/nn/fast_sft.c:950-951, 964-965), then the whole
+// row [dq | dk | dv | dh_q | dh_v] as one scaled fp16 operand so that a single GEMM
+// against [Wq; Wk; Wv; A_q; A_v]^T yields dq Wq + dk Wk + dv Wv + dh_q A_q + dh_v A_v
+// (src/nn/fast_sft.c:953-971).
+__global__ __launch_bounds__(TB) void k_qkv_bwd_rows(QkvBwdArgs a)
+{
+    extern __shared__ float buf[];                       // [qd + 2kd + 2R]
+    __shared__ float sm[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row = blockIdx.x;
+    const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd;
+    const int pos = (int)(row % a.seq);
+    for (int slot = wave; slot < a.Hq + a.Hkv; slot += 4) {
+        const int isk = slot >= a.Hq, h = isk ? slot - a.Hq : slot;
+        const int W = isk ? kd : qd;
+        const float *gin = (isk ? a.dk : a.dq) + row * W + h * hd;
+        const float *xp = (isk ? a.k_pre : a.q_pre) + row * W + h * hd;
+        const float *g = isk ? a.g_k : a.g_q;
+        float y0[MAXP], y1[MAXP], p0[MAXP], p1[MAXP];
+        float ss = 0.f, dot = 0.f;
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int d = lane + 64 * p;
+            y0[p] = y1[p] = p0[p] = p1[p] = 0.f;
+            if (d < half) {
+                const float g0 = gin[d], g1 = gin[d + half];
+                const float freq = 1.0f / powf(a.theta, (float)(2 * d) / (float)hd);
+                float s, c;
+                sincosf((float)pos * freq, &s, &c);
+                y0[p] = g0 * c + g1 * s;
+                y1[p] = -g0 * s + g1 * c;
+                p0[p] = xp[d];
+                p1[p] = xp[d + half];
+                ss += p0[p] * p0[p] + p1[p] * p1[p];
+                dot += y0[p] * g[d] * p0[p] + y1[p] * g[d + half] * p1[p];
+            }
+        }
+        ss = wave_sum(ss);
+        dot = wave_sum(dot);
+        const float inv = rsqrtf(ss / (float)hd + a.eps);
+        const float coeff = dot * inv * inv / (float)hd;
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int d = lane + 64 * p;
+            if (d >= half) continue;
+            const float d0 = (g[d] * y0[p] - coeff * p0[p]) * inv;
+            const float d1 = (g[d + half] * y1[p] - coeff * p1[p]) * inv;
+            const int c0 = (isk ? qd : 0) + h * hd + d;
+            buf[c0] = d0;
+            buf[c0 + half] = d1;
+            if (!isk) { a.dq_f[row * qd + h * hd + d] = d0; a.dq_f[row * qd + h * hd + d + half] = d1; }
+        }
+    }
+    for (int c = threadIdx.x; c < kd; c += TB) buf[qd + kd + c] = a.dv[row * kd + c];
+    __syncthreads();
+    const int R = a.R;
+    for (int r = wave; r < 2 * R; r += 4) {
+        const int isv = r >= R, rr = isv ? r - R : r;
+        const float *src = buf + (isv ? qd + kd : 0);
+        const float *B = isv ? a.Bv : a.Bq;
+        const int width = isv ? kd : qd;
+        float acc = 0.f;
+        for (int c = lane; c < width; c += 64) acc += src[c] * B[(size_t)c * R + rr];
+        acc = wave_sum(acc) * a.sc;
+        if (lane == 0) { buf[qd + 2 * kd + r] = acc; a.dh[row * 2 * R + r] = acc; }
+    }
+    __syncthreads();
+    const int n = qd + 2 * kd + 2 * R;
+    float amax = 0.f;
+    for (int c = threadIdx.x; c < n; c += TB) amax = fmaxf(amax, fabsf(buf[c]));
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    write_f16_row(buf, n, a.out16 + row * a.ld16, a.ld16, s);
+    if (threadIdx.x == 0) a.inv_scale[row] = 1.0f / s;
+}
+
+// ------------------------------------------------------------------ LoRA gradients
+// dB = sc * dY^T t, dA = dh^T ln1 (float_matmul_tn + scale, src/nn/fast_sft.c:948-952,
+// 962-966): one thread per gradient element, looping over the rows.  Each
+// workgroup also leaves the sum of squares of what it wrote (for the global norm).
+__global__ __launch_bounds__(TB) void k_lora_grads(LoraGradArgs a)
+{
+    __shared__ float sm[16];
+    const size_t idx = (size_t)blockIdx.x * TB + threadIdx.x;
+    const size_t nA = (size_t)a.R * a.D, nBq = (size_t)a.qd * a.R, nBv = (size_t)a.kd * a.R;
+    float gval = 0.f;
+    if (idx < 2 * nA + nBq + nBv) {
+        size_t o = idx;
+        int which;                                        // 0 dA_q, 1 dB_q, 2 dA_v, 3 dB_v
+        if (o < nA) which = 0;
+        else if ((o -= nA) < nBq) which = 1;
+        else if ((o -= nBq) < nA) which = 2;
+        else { o -= nA; which = 3; }
+        float s = 0.f;
+        if (which == 0 || which == 2) {
+            const int r = (int)(o / a.D), d = (int)(o % a.D);
+            const int hc = (which == 2 ? a.R : 0) + r;
+            for (int i = 0; i < a.rows; i++)
+                s += a.dh[(size_t)i * 2 * a.R + hc] * (h2f(a.ln16[(size_t)i * a.ld16 + d]) * a.ln_inv_scale[i]);
+        } else {
+            const int c = (int)(o / a.R), r = (int)(o % a.R);
+            const float *dy = which == 1 ? a.dq_f : a.dv_f;
+            const float *t = which == 1 ? a.tq : a.tv;
+            const int W = which == 1 ? a.qd : a.kd;
+            for (int i = 0; i < a.rows; i++) s += dy[(size_t)i * W + c] * t[(size_t)i * a.R + r];
+            s *= a.sc;
+        }
+        a.grad[idx] = s;
+        gval = s;
+    }
+    const float sq = block_sum(gval * gval, sm);
+    if (threadIdx.x == 0) a.sq_slots[blockIdx.x] = sq;
+}
+
+// ------------------------------------------------------------------ gated FFN rows
+__device__ __forceinline__ float gelu_inner(float g)
+{
+    const float in = 0.7978845608f * (g + 0.044715f * g * g * g);
+    return fminf(fmaxf(in, -15.0f), 15.0f);
+}
+__device__ __forceinline__ float act_fwd(float g, int gelu)
+{
+    return gelu ? 0.5f * g * (1.0f + tanhf(gelu_inner(g))) : g / (1.0f + expf(-g));
+}
+
+// silu_mul / gelu_mul, shaders/q8_kernels.metal:337-362, with the gate/up saves of
+// src/nn/fast_sft.c:715-718.  Two passes over the row: amax, then the scaled write.
+__global__ __launch_bounds__(TB) void k_glu_fwd(GluArgs a)
+{
+    __shared__ float sm[16];
+    const size_t r = blockIdx.x;
+    const int IS = a.IS;
+    float amax = 0.f;
+    for (int i = threadIdx.x; i < IS; i += TB) {
+        const float g = planes_at(a.in, r, i), u = planes_at(a.in, r, IS + i);
+        a.gate_pre[r * IS + i] = g;
+        a.up_val[r * IS + i] = u;
+        amax = fmaxf(amax, fabsf(act_fwd(g, a.gelu) * u));
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    half_t *o = a.out16 + r * a.ld16;
+    for (int i = threadIdx.x; i < a.ld16; i += TB) {
+        half_t hv = (half_t)0;
+        if (i < IS) hv = f2h(act_fwd(a.gate_pre[r * IS + i], a.gelu) * a.up_val[r * IS + i] * s);
+        o[i] = hv;
+    }
+    if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
+}
+
+__device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, float &dg, float &du)
+{
+    if (gelu) {                                           // gelu_mul_backward, shaders/q8_kernels.metal:561-580
+        const float t = tanhf(gelu_inner(g));
+        const float grad = 0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * 0.7978845608f * (1.0f + 3.0f * 0.044715f * g * g);
+        dg = dy * u * grad;
+        du = dy * (0.5f * g * (1.0f + t));
+    } else {                                              // silu_mul_backward, :540-556
+        const float sig = 1.0f / (1.0f + expf(-g));
+        dg = dy * u * (sig * (1.0f + g * (1.0f - sig)));
+        du = dy * (g * sig);
+    }
+}
+
+__global__ __launch_bounds__(TB) void k_glu_bwd(GluArgs a)
+{
+    __shared__ float sm[16];
+    const size_t r = blockIdx.x;
+    const int IS = a.IS;
+    float amax = 0.f;
+    for (int i = threadIdx.x; i < IS; i += TB) {
+        float dg, du;
+        act_bwd(planes_at(a.in, r, i), a.gate_pre[r * IS + i], a.up_val[r * IS + i], a.gelu, dg, du);
+        amax = fmaxf(amax, fmaxf(fabsf(dg), fabsf(du)));
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    half_t *o = a.out16 + r * a.ld16;
+    for (int i = threadIdx.x; i < IS; i += TB) {
+        float dg, du;
+        act_bwd(planes_at(a.in, r, i), a.gate_pre[r * IS + i], a.up_val[r * IS + i], a.gelu, dg, du);
+        o[i] = f2h(dg * s);
+        o[IS + i] = f2h(du * s);
+    }
+    for (int i = 2 * IS + threadIdx.x; i < a.ld16; i += TB) o[i] = (half_t)0;
+    if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
+}
+
+// ------------------------------------------------------------------ backward rows
+// dx_out = dx_prev + RNB(x_saved, sum(dy planes); g), clamped (rms_norm_train_backward,
+// shaders/q8_kernels.metal:584-625; residual_add; clamp_tensor :1155-1161;
+// src/nn/fast_sft.c:870-874, 975-980).  The operand of the next dX GEMM is dx_out
+// itself (Qwen3) or RNB(branch_raw, dx_out; g_branch) (Gemma3's post-norms,
+// src/nn/fast_sft.c:798-802, 877-881).
+__global__ __launch_bounds__(TB) void k_norm_bwd_rows(NormBwdArgs a)
+{
+    extern __shared__ float lds[];
+    float *dyb = lds, *dxn = lds + a.D;
+    __shared__ float sm[16];
+    const size_t r = blockIdx.x;
+    const int D = a.D;
+    float ss = 0.f, dot = 0.f;
+    for (int i = threadIdx.x; i < D; i += TB) {
+        const float dy = planes_at(a.dy, r, i), x = a.x_saved[r * D + i];
+        dyb[i] = dy;
+        ss += x * x;
+        dot += dy * a.g[i] * x;
+    }
+    ss = block_sum(ss, sm);
+    dot = block_sum(dot, sm);
+    const float inv = rsqrtf(ss / (float)D + a.eps);
+    const float coeff = dot * inv * inv / (float)D;
+    for (int i = threadIdx.x; i < D; i += TB) {
+        float t = (a.g[i] * dyb[i] - coeff * a.x_saved[r * D + i]) * inv;
+        if (a.dx_prev) t += a.dx_prev[r * D + i];
+        if (a.clamp > 0.f) t = fminf(fmaxf(t, -a.clamp), a.clamp);
+        a.dx_out[r * D + i] = t;
+        dxn[i] = t;
+    }
+    if (!a.d16) return;
+    float amax = 0.f;
+    if (a.branch_raw) {
+        float ssb = 0.f, dotb = 0.f;
+        for (int i = threadIdx.x; i < D; i += TB) {
+            const float xb = a.branch_raw[r * D + i];
+            ssb += xb * xb;
+            dotb += dxn[i] * a.g_branch[i] * xb;
+        }
+        ssb = block_sum(ssb, sm);
+        dotb = block_sum(dotb, sm);
+        const float invb = rsqrtf(ssb / (float)D + a.eps);
+        const float cb = dotb * invb * invb / (float)D;
+        for (int i = threadIdx.x; i < D; i += TB) {
+            const float v = (a.g_branch[i] * dxn[i] - cb * a.branch_raw[r * D + i]) * invb;
+            dyb[i] = v;
+            amax = fmaxf(amax, fabsf(v));
+        }
+    } else {
+        for (int i = threadIdx.x; i < D; i += TB) { dyb[i] = dxn[i]; amax = fmaxf(amax, fabsf(dxn[i])); }
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    write_f16_row(dyb, D, a.d16 + r * a.ld16, a.ld16, s);
+    if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
+}
+
+// ------------------------------------------------------------------ loss rows
+// softmax_ce_train + scale(1/BN), shaders/q8_kernels.metal:646-690 and
+// src/nn/fast_sft.c:754-760.  The gradient is written once, as the lm_head dX GEMM's
+// fp16 operand: (softmax - onehot) * 1024 with row factor (1/BN) / 1024.
+__global__ __launch_bounds__(1024) void k_ce_rows(CeArgs a)
+{
+    __shared__ float sm[16];
+    const size_t r = blockIdx.x;
+    const int V = a.V;
+    const float *lg = a.logits + r * V;
+    const uint32_t tgt = a.targets[r];
+    float mx = -1e30f;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, lg[i]);
+    mx = block_max(mx, sm);
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) sum += expf(lg[i] - mx);
+    sum = block_sum(sum, sm);
+    const float lse = logf(sum) + mx;
+    if (threadIdx.x == 0) {
+        a.losses[r] = lse - lg[tgt];
+        a.inv_scale[r] = (1.0f / (float)a.rows_total) * (1.0f / 1024.0f);
+    }
+    half_t *o = a.dl16 + r * a.ld16;
+    for (int i = threadIdx.x; i < a.ld16; i += blockDim.x) {
+        half_t hv = (half_t)0;
+        if (i < V) hv = f2h((expf(lg[i] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f);
+        o[i] = hv;
+    }
+}
+
+// ------------------------------------------------------------------ optimiser
+// clip_grad_norm + adamw_update, src/nn/fast_sft.c:1045-1107, in one pass over the
+// flat LoRA arena: the global norm comes from the per-workgroup sums of squares
+// (double accumulator, as the reference), gradients are rescaled in place when
+// the norm exceeds max_norm, and the fp16 images of A_q / A_v inside the fused
+// QKV weight (and its transpose) are refreshed for the next step's GEMMs.
+__global__ __launch_bounds__(1024) void k_grad_norm(const float *__restrict__ slots, int n, float *out)
+{
+    __shared__ double sd[16];
+    double s = 0.0;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) s += (double)slots[i];
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, WAVE);
+    if ((threadIdx.x & 63) == 0) sd[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int i = 0; i < (int)(blockDim.x >> 6); i++) t += sd[i];
+        out[0] = (float)sqrt(t);
+    }
+}
+
+__device__ __forceinline__ void shadow_store(const AdamArgs &a, size_t idx, float pv)
+{
+    const size_t L = idx / a.layer_size;
+    size_t o = idx % a.layer_size;
+    const size_t nA = (size_t)a.R * a.D, nBq = (size_t)a.qd * a.R;
+    int rbase;
+    if (o < nA) rbase = 0;
+    else if (o >= nA + nBq && o < 2 * nA + nBq) { o -= nA + nBq; rbase = a.R; }
+    else return;
+    const int r = (int)(o / a.D), d = (int)(o % a.D);
+    const int rowx = a.qd + 2 * a.kd + rbase + r;
+    const half_t hv = f2h(pv);
+    a.wqkv[L * a.wqkv_layer_stride + (size_t)rowx * a.D + d] = hv;
+    a.wqkvT[L * a.wqkvT_layer_stride + (size_t)d * a.ldT + rowx] = hv;
+}
+
+__global__ __launch_bounds__(TB) void k_adamw(AdamArgs a)
+{
+    const float lr = a.hyper[0], bc1 = a.hyper[1], bc2 = a.hyper[2];
+    const float norm = a.grad_norm_out[0];
+    const float gscale = (norm > a.max_norm) ? a.max_norm / norm : 1.0f;
+    const bool clip = norm > a.max_norm;
+    for (size_t i = (size_t)blockIdx.x * TB + threadIdx.x; i < a.n; i += (size_t)gridDim.x * TB) {
+        float g = a.g[i];
+        if (clip) { g *= gscale; a.g[i] = g; }
+        const float m = a.b1 * a.m[i] + (1.0f - a.b1) * g;
+        const float v = a.b2 * a.v[i] + (1.0f - a.b2) * g * g;
+        a.m[i] = m;
+        a.v[i] = v;
+        const float mh = m / bc1, vh = v / bc2;
+        float p = a.p[i];
+        p -= lr * (mh / (sqrtf(vh) + a.eps) + a.wd * p);
+        a.p[i] = p;
+        shadow_store(a, i, p);
+    }
+}
+
+__global__ __launch_bounds__(TB) void k_lora_shadow(AdamArgs a)
+{
+    for (size_t i = (size_t)blockIdx.x * TB + threadIdx.x; i < a.n; i += (size_t)gridDim.x * TB)
+        shadow_store(a, i, a.p[i]);
+}
+
+__global__ void k_fill_f32(float *p, float v, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * TB + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+#define LAUNCH(kern, grid, block, lds, ...) do { \
+    hipLaunchKernelGGL(kern, grid, block, lds, stream(), __VA_ARGS__); HIP_CHECK(hipGetLastError()); } while (0)
+
+void require(bool ok, const char *what)
+{
+    if (!ok) { fprintf(stderr, "[fast_hip] unsupported shape: %s\n", what); abort(); }
+}
+
+}  // namespace
+
+void launch_norm_rows(const NormRowsArgs &a, int rows)
+{
+    require(a.D > 0 && (size_t)a.D * 8 <= 64 * 1024, "norm_rows: hidden size must be <= 8192");
+    LAUNCH(k_norm_rows, dim3(rows), dim3(TB), (size_t)a.D * 8, a);
+}
+
+void launch_qkv_post(const QkvPostArgs &a, int rows)
+{
+    require(a.hd % 2 == 0 && a.hd <= 2 * 64 * MAXP && a.R <= 64 && a.Hq % a.Hkv == 0, "qkv_post: head_dim <= 512, rank <= 64");
+    const size_t tasks = (size_t)rows * (a.Hq + 2 * a.Hkv);
+    QkvPostArgs b = a;
+    b.rows = rows;
+    LAUNCH(k_qkv_post, dim3((unsigned)((tasks + 3) / 4)), dim3(TB), 0, b);
+}
+
+void launch_attn_fwd(const AttnFwdArgs &a)
+{
+    require(a.hd % 4 == 0 && a.seq <= 4096, "attn_fwd: head_dim % 4, seq <= 4096");
+    LAUNCH(k_attn_fwd, dim3(a.Hq, a.seq, a.batch), dim3(64), (size_t)(a.seq + a.hd) * 4, a);
+}
+
+void launch_attn_bwd(const AttnBwdArgs &a)
+{
+    require(a.hd % 4 == 0 && a.seq <= 4096, "attn_bwd: head_dim % 4, seq <= 4096");
+    LAUNCH(k_attn_bwd_dq, dim3(a.Hq, a.seq, a.batch), dim3(64), (size_t)(a.seq + a.hd) * 4, a);
+    LAUNCH(k_attn_bwd_dkv, dim3(a.Hkv, a.seq, a.batch), dim3(64), 0, a);
+}
+
+void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
+{
+    const size_t n = (size_t)(a.Hq + 2 * a.Hkv) * a.hd + 2 * a.R;
+    require(a.hd <= 2 * 64 * MAXP && n * 4 <= 64 * 1024, "qkv_bwd: row of dq|dk|dv must fit 64 KB of LDS");
+    LAUNCH(k_qkv_bwd_rows, dim3(rows), dim3(TB), n * 4, a);
+}
+
+int lora_grad_blocks(int D, int qd, int kd, int R)
+{
+    const size_t n = (size_t)2 * R * D + (size_t)qd * R + (size_t)kd * R;
+    return (int)((n + TB - 1) / TB);
+}
+
+void launch_lora_grads(const LoraGradArgs &a)
+{
+    LAUNCH(k_lora_grads, dim3(lora_grad_blocks(a.D, a.qd, a.kd, a.R)), dim3(TB), 0, a);
+}
+
+void launch_glu_fwd(const GluArgs &a, int rows) { LAUNCH(k_glu_fwd, dim3(rows), dim3(TB), 0, a); }
+void launch_glu_bwd(const GluArgs &a, int rows) { LAUNCH(k_glu_bwd, dim3(rows), dim3(TB), 0, a); }
+
+void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
+{
+    require(a.D > 0 && (size_t)a.D * 8 <= 64 * 1024, "norm_bwd_rows: hidden size must be <= 8192");
+    LAUNCH(k_norm_bwd_rows, dim3(rows), dim3(TB), (size_t)a.D * 8, a);
+}
+
+void launch_ce_rows(const CeArgs &a, int rows) { LAUNCH(k_ce_rows, dim3(rows), dim3(a.V >= 4096 ? 1024 : 256), 0, a); }
+
+void launch_adamw(const AdamArgs &a)
+{
+    if (!a.n) return;
+    LAUNCH(k_grad_norm, dim3(1), dim3(1024), 0, a.sq_slots, a.n_slots, a.grad_norm_out);
+    size_t blocks = (a.n + TB - 1) / TB;
+    if (blocks > 4096) blocks = 4096;
+    LAUNCH(k_adamw, dim3((unsigned)blocks), dim3(TB), 0, a);
+}
+
+void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
+                        size_t wqkvT_layer_stride, int ldT, int D, int qd, int kd, int R, size_t layer_size)
+{
+    if (!n) return;
+    AdamArgs a{};
+    a.p = const_cast<float *>(p); a.n = n; a.wqkv = wqkv; a.wqkv_layer_stride = wqkv_layer_stride;
+    a.wqkvT = wqkvT; a.wqkvT_layer_stride = wqkvT_layer_stride; a.ldT = ldT;
+    a.D = D; a.qd = qd; a.kd = kd; a.R = R; a.layer_size = layer_size;
+    size_t blocks = (n + TB - 1) / TB;
+    if (blocks > 4096) blocks = 4096;
+    LAUNCH(k_lora_shadow, dim3((unsigned)blocks), dim3(TB), 0, a);
+}
+
+void launch_fill_f32(float *p, float v, size_t n)
+{
+    if (!n) return;
+    LAUNCH(k_fill_f32, dim3((unsigned)((n + TB - 1) / TB)), dim3(TB), 0, p, v, n);
+}
+
+}  // namespace lmhip

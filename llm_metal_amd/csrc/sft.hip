@@ -1,0 +1,646 @@
+// Host pipeline of the fused LoRA SFT step: state, forward, loss, backward,
+// update.  Restates the sequencing of the reference's src/nn/fast_sft.c
+// (forward_to_logits :616-752, sft_apply_ce_loss :754-760, sft_backward_ex
+// :766-982, lora_update :1090-1107, sft_train_step :1113-1157) as ~20 launches
+// per layer on one stream instead of ~82:
+//   * Q, K, V and the two LoRA down-projections are ONE GEMM against the fused
+//     weight [Wq; Wk; Wv; A_q; A_v]; gate and up are one GEMM against [Wg; Wu];
+//   * every dX product of the backward uses a transposed copy of the weight made
+//     at start-up, so it runs through the same weight-streaming kernel; the QKV
+//     backward is one GEMM whose operand row is [dq | dk | dv | dh_q | dh_v];
+//   * GEMM outputs stay as K-split partial planes that the next row kernel sums;
+//   * saved activations are simply where the forward wrote them (no copies).
+#include "backend.h"
+#include "devutil.h"
+#include "gemm.h"
+#include "fused.h"
+#include "../../include/sft_hip.h"
+#include <math.h>
+#include <string.h>
+#include <vector>
+
+using namespace lmhip;
+
+struct SFTState {
+    int D, Hq, Hkv, hd, IS, V, NL, N, B, BN;
+    int qd, kd, R, nq_ext, ldq;          // nq_ext = qd + 2kd + 2R rows of the fused QKV weight; ldq its padded length as a K
+    float eps, lora_scaling, emb_scale;
+    ModelType model_type;
+    int step_count, weight_format;
+    std::vector<float> rope_thetas;
+
+    // frozen weights, F16, one arena per matrix kind with a fixed layer stride
+    MetalBuf *wqkv, *wqkvT, *wo, *woT, *wgu, *wguT, *wd, *wdT, *wlm, *wlmT;
+    MetalBuf *q8_blocks;                 // Q8_0 mode: the quantised bytes of every matrix, in upload order
+    MetalBuf *g_in, *g_post_attn, *g_pre_ff, *g_post_ff, *g_q, *g_k, *g_final;
+    MetalBuf *emb;                       // fp32 [V, D]
+    std::vector<LayerW> layer_views;     // WMat/MetalBuf windows handed out by sft_get_layers-style accessors
+
+    // LoRA arena and optimiser state (fp32, device)
+    size_t lsz, lora_n;
+    MetalBuf *lora, *lora_grad, *adam_m, *adam_v, *sq_slots, *grad_norm;
+    int slots_per_layer;
+    std::vector<MetalBuf *> lora_views, grad_views;
+
+    // host-visible small buffers
+    MetalBuf *tokens, *targets, *losses, *hyper, *x_in_host;
+    uint32_t *tokens_cpu, *targets_cpu;
+    float *losses_cpu, *hyper_cpu, *x_cpu;
+
+    // saved activations (layer-strided arenas)
+    MetalBuf *xs;                        // [2*NL + 1][BN*D]: x_in[L] = 2L, x_mid[L] = 2L+1, x_final = 2NL
+    MetalBuf *ln1_16, *ln1_inv;          // [NL][BN*D] f16, [NL][BN]
+    MetalBuf *q_pre, *k_pre, *q_fin, *k_fin, *v_sav, *probs, *gate_pre, *up_val, *tq, *tv, *o_raw, *ff_raw;
+    // transients
+    MetalBuf *a16, *a16_inv;             // largest fp16 operand (BN x max K) and its row factors
+    MetalBuf *ones;                      // [BN] of 1.0f
+    MetalBuf *planes;
+    MetalBuf *logits, *dlogits, *dl16, *dl_inv;
+    MetalBuf *dx[2], *dO_red, *dscore, *dq, *dk, *dv, *dq_f, *dh;
+    size_t planes_cap;
+};
+
+namespace {
+
+inline int round8(int x) { return (x + 7) & ~7; }
+inline MetalBuf *fbuf(size_t n) { return metal_buf_create(n * sizeof(float)); }
+inline MetalBuf *hbuf(size_t n) { return metal_buf_create(n * sizeof(half_t)); }
+template <typename T> inline T *at(MetalBuf *b, size_t elem_off = 0) { return dptr_as<T>(b) + elem_off; }
+
+// Upload one fp32 matrix and store it as F16 rows [row0, row0+rows) of a row-major arena slice
+// whose row length is `cols`.  Q8_0 mode quantises first and stores the dequantised values.
+void put_matrix(SFTState *s, MetalBuf *arena, size_t elem_off, const float *src, int rows, int cols,
+                std::vector<MetalBuf *> &q8_keep)
+{
+    const size_t n = (size_t)rows * cols;
+    MetalBuf *stage = metal_buf_from_data(src, n * sizeof(float));
+    MetalBuf *dst = metal_buf_view(arena, elem_off * sizeof(half_t), n * sizeof(half_t));
+    if (s->weight_format) {
+        hip_enqueue_f32_to_f16(stage, dst, n);
+    } else {
+        MetalBuf *q8 = metal_buf_create((size_t)rows * (cols / 32) * 34);
+        hip_enqueue_q8_quantize(stage, q8, rows, cols);
+        hip_enqueue_q8_to_f16(q8, dst, rows, cols);
+        q8_keep.push_back(q8);
+    }
+    metal_buf_free(dst);
+    metal_buf_free(stage);
+}
+
+size_t max_planes_elems(SFTState *s)
+{
+    struct Sh { int N, K; };
+    const Sh shapes[] = {{s->nq_ext, s->D}, {s->D, s->qd}, {2 * s->IS, s->D}, {s->D, s->IS}, {s->V, s->D},
+                         {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->ldq}};
+    size_t mx = 0;
+    for (const Sh &sh : shapes) {
+        GemmPlan p = plan_gemm(s->BN, sh.N, sh.K);
+        const size_t e = (size_t)p.S * s->BN * sh.N;
+        if (e > mx) mx = e;
+    }
+    return mx;
+}
+
+// P = A16 * W^T as K-split planes in the state's plane buffer
+Planes gemm(SFTState *s, const half_t *A, int lda, const float *inv, const half_t *W, int ldw, int N, int K,
+            float *out = nullptr)
+{
+    GemmPlan p = plan_gemm(s->BN, N, K);
+    float *P = out ? out : at<float>(s->planes);
+    const size_t stride = (size_t)s->BN * N;
+    if (!out && (size_t)p.S * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
+    if (out && p.S != 1) { fprintf(stderr, "[fast_sft] direct GEMM output needs S == 1\n"); abort(); }
+    launch_gemm(A, lda, inv, W, ldw, P, N, stride, s->BN, N, K, p);
+    return Planes{P, p.S, stride, N};
+}
+
+void forward_impl(SFTState *s, bool gather)
+{
+    const int BN = s->BN, D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R;
+    const size_t xsz = (size_t)BN * D;
+    half_t *a16 = at<half_t>(s->a16);
+    float *ainv = at<float>(s->a16_inv);
+    const bool gemma = s->model_type == MODEL_GEMMA3;
+    Planes pending{nullptr, 0, 0, 0};                    // FFN output of the previous layer, not yet added
+
+    for (int L = 0; L < s->NL; L++) {
+        float *x_in = at<float>(s->xs, (size_t)(2 * L) * xsz), *x_mid = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
+        half_t *ln1 = at<half_t>(s->ln1_16, (size_t)L * xsz);
+        float *ln1inv = at<float>(s->ln1_inv, (size_t)L * BN);
+
+        // x_in = x (+ previous FFN branch); ln1 = RN(x_in; g_in)        [src/nn/fast_sft.c:631-635, 732-740]
+        NormRowsArgs n1{};
+        if (L == 0) {
+            if (gather) { n1.emb = at<float>(s->emb); n1.tokens = at<uint32_t>(s->tokens); n1.emb_scale = s->emb_scale; }
+            else n1.x_prev = at<float>(s->x_in_host);
+        } else {
+            n1.x_prev = at<float>(s->xs, (size_t)(2 * L - 1) * xsz);
+            n1.branch = pending;
+            if (gemma) { n1.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); n1.branch_raw_out = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); }
+        }
+        n1.x_out = x_in;
+        n1.g_norm = at<float>(s->g_in, (size_t)L * D);
+        n1.ln16 = ln1; n1.ld16 = D; n1.inv_scale = ln1inv; n1.D = D; n1.eps = s->eps;
+        launch_norm_rows(n1, BN);
+
+        // [q | k | v | tq | tv] = ln1 [Wq; Wk; Wv; A_q; A_v]^T                 [:638-656]
+        Planes pq = gemm(s, ln1, D, ln1inv, at<half_t>(s->wqkv, (size_t)L * s->nq_ext * D), D, s->nq_ext, D);
+        QkvPostArgs qa{};
+        qa.qkv = pq;
+        qa.Bq = at<float>(s->lora, L * s->lsz + (size_t)R * D);
+        qa.Bv = at<float>(s->lora, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
+        qa.R = R; qa.sc = s->lora_scaling;
+        qa.g_q = at<float>(s->g_q, (size_t)L * s->hd); qa.g_k = at<float>(s->g_k, (size_t)L * s->hd);
+        qa.eps = s->eps; qa.theta = s->rope_thetas[L];
+        qa.Hq = s->Hq; qa.Hkv = s->Hkv; qa.hd = s->hd; qa.seq = s->N;
+        qa.q_pre = at<float>(s->q_pre, (size_t)L * BN * qd); qa.k_pre = at<float>(s->k_pre, (size_t)L * BN * kd);
+        qa.q_fin = at<float>(s->q_fin, (size_t)L * BN * qd); qa.k_fin = at<float>(s->k_fin, (size_t)L * BN * kd);
+        qa.v_out = at<float>(s->v_sav, (size_t)L * BN * kd);
+        qa.tq = at<float>(s->tq, (size_t)L * BN * (R ? R : 1)); qa.tv = at<float>(s->tv, (size_t)L * BN * (R ? R : 1));
+        launch_qkv_post(qa, BN);
+
+        // causal GQA attention                                               [:678-689]
+        AttnFwdArgs aa{};
+        aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
+        aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
+        aa.scale = 1.0f / sqrtf((float)s->hd);
+        aa.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
+        aa.out16 = a16; aa.ld16 = qd;
+        launch_attn_fwd(aa);
+
+        // o = attn Wo^T; x_mid = x_in + o (Qwen3) | x_in + RN(o; g_post_attn) (Gemma3); ln2 = RN(x_mid; g_ffn_in)   [:696-711]
+        Planes po = gemm(s, a16, qd, at<float>(s->ones), at<half_t>(s->wo, (size_t)L * D * qd), qd, D, qd);
+        NormRowsArgs n2{};
+        n2.x_prev = x_in; n2.branch = po;
+        if (gemma) { n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); n2.branch_raw_out = at<float>(s->o_raw, (size_t)L * xsz); }
+        n2.x_out = x_mid;
+        n2.g_norm = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
+        n2.ln16 = a16; n2.ld16 = D; n2.inv_scale = ainv; n2.D = D; n2.eps = s->eps;
+        launch_norm_rows(n2, BN);
+
+        // [gate | up] = ln2 [Wg; Wu]^T; act = silu|gelu(gate) * up              [:715-725]
+        Planes pg = gemm(s, a16, D, ainv, at<half_t>(s->wgu, (size_t)L * 2 * IS * D), D, 2 * IS, D);
+        GluArgs ga{};
+        ga.in = pg; ga.IS = IS; ga.gelu = gemma;
+        ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
+        ga.out16 = a16; ga.ld16 = IS; ga.inv_scale = ainv;
+        launch_glu_fwd(ga, BN);
+
+        // ff = act Wd^T, added by the next row kernel                          [:730-740]
+        pending = gemm(s, a16, IS, ainv, at<half_t>(s->wd, (size_t)L * D * IS), IS, D, IS);
+    }
+
+    // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
+    NormRowsArgs nf{};
+    const int L = s->NL;
+    nf.x_prev = at<float>(s->xs, (size_t)(2 * L - 1) * xsz);
+    nf.branch = pending;
+    if (gemma) { nf.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); nf.branch_raw_out = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); }
+    nf.x_out = at<float>(s->xs, (size_t)(2 * L) * xsz);
+    nf.g_norm = at<float>(s->g_final);
+    nf.ln16 = a16; nf.ld16 = D; nf.inv_scale = ainv; nf.D = D; nf.eps = s->eps;
+    launch_norm_rows(nf, BN);
+    GemmPlan pl = plan_gemm(BN, s->V, D);
+    if (pl.S == 1) {
+        gemm(s, a16, D, ainv, at<half_t>(s->wlm), D, s->V, D, at<float>(s->logits));
+    } else {
+        Planes p = gemm(s, a16, D, ainv, at<half_t>(s->wlm), D, s->V, D);
+        launch_reduce_planes(p.p, p.S, p.stride, p.ld, at<float>(s->logits), BN, s->V);
+    }
+}
+
+// Backward from the fp16 loss gradient in dl16 / dl_inv.
+void backward_impl(SFTState *s)
+{
+    const int BN = s->BN, D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R, NL = s->NL;
+    const size_t xsz = (size_t)BN * D;
+    half_t *a16 = at<half_t>(s->a16);
+    float *ainv = at<float>(s->a16_inv);
+    const bool gemma = s->model_type == MODEL_GEMMA3;
+    int cur = 0;                                          // dx ping-pong
+
+    // dx = RNB(x_final, dlogits Wlm; g_final)                                [:777-790]
+    Planes p = gemm(s, at<half_t>(s->dl16), round8(s->V), at<float>(s->dl_inv), at<half_t>(s->wlmT), round8(s->V), D, round8(s->V));
+    NormBwdArgs nb{};
+    nb.dy = p; nb.x_saved = at<float>(s->xs, (size_t)(2 * NL) * xsz); nb.g = at<float>(s->g_final);
+    nb.eps = s->eps; nb.D = D; nb.dx_prev = nullptr; nb.dx_out = at<float>(s->dx[cur]); nb.clamp = 0.f;
+    if (gemma) { nb.branch_raw = at<float>(s->ff_raw, (size_t)(NL - 1) * xsz); nb.g_branch = at<float>(s->g_post_ff, (size_t)(NL - 1) * D); }
+    nb.d16 = a16; nb.ld16 = D; nb.inv_scale = ainv;
+    launch_norm_bwd_rows(nb, BN);
+
+    for (int L = NL - 1; L >= 0; L--) {
+        // FFN: d act = d Wd; (dgate, dup); dln2 = dgate Wg + dup Wu; dx += RNB(x_mid, dln2)   [:798-874]
+        Planes pd = gemm(s, a16, D, ainv, at<half_t>(s->wdT, (size_t)L * IS * D), D, IS, D);
+        GluArgs gb{};
+        gb.in = pd; gb.IS = IS; gb.gelu = gemma;
+        gb.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); gb.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
+        gb.out16 = a16; gb.ld16 = 2 * IS; gb.inv_scale = ainv;
+        launch_glu_bwd(gb, BN);
+        Planes pgu = gemm(s, a16, 2 * IS, ainv, at<half_t>(s->wguT, (size_t)L * D * 2 * IS), 2 * IS, D, 2 * IS);
+        NormBwdArgs n2{};
+        n2.dy = pgu; n2.x_saved = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
+        n2.g = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
+        n2.eps = s->eps; n2.D = D; n2.dx_prev = at<float>(s->dx[cur]); n2.dx_out = at<float>(s->dx[cur ^ 1]); n2.clamp = 0.f;
+        if (gemma) { n2.branch_raw = at<float>(s->o_raw, (size_t)L * xsz); n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); }
+        n2.d16 = a16; n2.ld16 = D; n2.inv_scale = ainv;
+        launch_norm_bwd_rows(n2, BN);
+        cur ^= 1;
+
+        // attention: dO = d Wo; dq, dk, dv                                    [:877-911]
+        Planes pdo = gemm(s, a16, D, ainv, at<half_t>(s->woT, (size_t)L * qd * D), D, qd, D);
+        AttnBwdArgs ab{};
+        ab.dO = pdo;
+        ab.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
+        ab.q = at<float>(s->q_fin, (size_t)L * BN * qd); ab.k = at<float>(s->k_fin, (size_t)L * BN * kd);
+        ab.v = at<float>(s->v_sav, (size_t)L * BN * kd);
+        ab.Hq = s->Hq; ab.Hkv = s->Hkv; ab.hd = s->hd; ab.seq = s->N; ab.batch = s->B;
+        ab.scale = 1.0f / sqrtf((float)s->hd);
+        ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore);
+        ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv);
+        launch_attn_bwd(ab);
+
+        // inverse RoPE, QK-norm backward, dh; LoRA gradients                  [:912-966]
+        QkvBwdArgs qb{};
+        qb.dq = ab.dq; qb.dk = ab.dk; qb.dv = ab.dv;
+        qb.q_pre = at<float>(s->q_pre, (size_t)L * BN * qd); qb.k_pre = at<float>(s->k_pre, (size_t)L * BN * kd);
+        qb.g_q = at<float>(s->g_q, (size_t)L * s->hd); qb.g_k = at<float>(s->g_k, (size_t)L * s->hd);
+        qb.eps = s->eps; qb.theta = s->rope_thetas[L];
+        qb.Bq = at<float>(s->lora, L * s->lsz + (size_t)R * D);
+        qb.Bv = at<float>(s->lora, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
+        qb.R = R; qb.sc = s->lora_scaling;
+        qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
+        qb.dq_f = at<float>(s->dq_f); qb.dv_f = nullptr; qb.dh = at<float>(s->dh);
+        qb.out16 = a16; qb.ld16 = s->ldq; qb.inv_scale = ainv;
+        launch_qkv_bwd(qb, BN);
+        if (R > 0) {
+            LoraGradArgs lg{};
+            lg.dq_f = qb.dq_f; lg.dv_f = ab.dv; lg.tq = at<float>(s->tq, (size_t)L * BN * R); lg.tv = at<float>(s->tv, (size_t)L * BN * R);
+            lg.dh = qb.dh;
+            lg.ln16 = at<half_t>(s->ln1_16, (size_t)L * xsz); lg.ld16 = D; lg.ln_inv_scale = at<float>(s->ln1_inv, (size_t)L * BN);
+            lg.rows = BN; lg.D = D; lg.qd = qd; lg.kd = kd; lg.R = R; lg.sc = s->lora_scaling;
+            lg.grad = at<float>(s->lora_grad, L * s->lsz);
+            lg.sq_slots = at<float>(s->sq_slots, (size_t)L * s->slots_per_layer);
+            launch_lora_grads(lg);
+        }
+
+        // dln1 = [dq|dk|dv|dh] [Wq;Wk;Wv;A_q;A_v]; dx += RNB(x_in, dln1; g_in); clamp     [:956-980]
+        Planes pl = gemm(s, a16, s->ldq, ainv, at<half_t>(s->wqkvT, (size_t)L * D * s->ldq), s->ldq, D, s->ldq);
+        NormBwdArgs n1{};
+        n1.dy = pl; n1.x_saved = at<float>(s->xs, (size_t)(2 * L) * xsz); n1.g = at<float>(s->g_in, (size_t)L * D);
+        n1.eps = s->eps; n1.D = D; n1.dx_prev = at<float>(s->dx[cur]); n1.dx_out = at<float>(s->dx[cur ^ 1]); n1.clamp = 1e6f;
+        if (L > 0) {
+            if (gemma) { n1.branch_raw = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); n1.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); }
+            n1.d16 = a16; n1.ld16 = D; n1.inv_scale = ainv;
+        }
+        launch_norm_bwd_rows(n1, BN);
+        cur ^= 1;
+    }
+}
+
+void write_hyper(SFTState *s, float lr, int step)
+{
+    s->hyper_cpu[0] = lr;
+    s->hyper_cpu[1] = 1.0f - powf(0.9f, (float)step);     // bias corrections as adamw_update forms them, src/nn/fast_sft.c:1048-1049
+    s->hyper_cpu[2] = 1.0f - powf(0.999f, (float)step);
+}
+
+void enqueue_update(SFTState *s)
+{
+    if (!s->R) return;
+    AdamArgs a{};
+    a.p = at<float>(s->lora); a.g = at<float>(s->lora_grad); a.m = at<float>(s->adam_m); a.v = at<float>(s->adam_v);
+    a.n = s->lora_n;
+    a.sq_slots = at<float>(s->sq_slots); a.n_slots = s->slots_per_layer * s->NL;
+    a.hyper = at<float>(s->hyper);
+    a.b1 = 0.9f; a.b2 = 0.999f; a.eps = 1e-8f; a.wd = 0.01f; a.max_norm = 1.0f;      // src/nn/fast_sft.c:1091-1094
+    a.wqkv = at<half_t>(s->wqkv); a.wqkv_layer_stride = (size_t)s->nq_ext * s->D;
+    a.wqkvT = at<half_t>(s->wqkvT); a.wqkvT_layer_stride = (size_t)s->D * s->ldq; a.ldT = s->ldq;
+    a.NL = s->NL; a.D = s->D; a.qd = s->qd; a.kd = s->kd; a.R = s->R; a.layer_size = s->lsz;
+    a.grad_norm_out = at<float>(s->grad_norm);
+    launch_adamw(a);
+}
+
+void refresh_shadow(SFTState *s)
+{
+    if (!s->R) return;
+    launch_lora_shadow(at<float>(s->lora), s->lora_n, at<half_t>(s->wqkv), (size_t)s->nq_ext * s->D,
+                       at<half_t>(s->wqkvT), (size_t)s->D * s->ldq, s->ldq, s->D, s->qd, s->kd, s->R, s->lsz);
+}
+
+MetalBuf *host_buf(size_t bytes, void **cpu)
+{
+    MetalBuf *b = metal_buf_create(bytes);
+    *cpu = metal_buf_ptr(b);
+    memset(*cpu, 0, bytes);
+    return b;
+}
+
+}  // namespace
+
+extern "C" {
+
+SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len, int lora_rank, float lora_alpha,
+                                    int weight_format)
+{
+    if (fast_metal_init() != 0) {
+        fprintf(stderr, "[FastSFT] HIP backend init failed\n");
+        return nullptr;
+    }
+    SFTState *s = new SFTState();
+    s->model_type = m->model_type;
+    s->D = m->d_model; s->Hq = m->n_q_heads; s->Hkv = m->n_kv_heads; s->hd = m->head_dim;
+    s->IS = m->intermediate_size; s->V = m->vocab_size; s->NL = m->n_layers;
+    s->N = seq_len; s->B = batch; s->BN = batch * seq_len;
+    s->qd = s->Hq * s->hd; s->kd = s->Hkv * s->hd; s->R = lora_rank;
+    s->nq_ext = s->qd + 2 * s->kd + 2 * s->R;
+    s->ldq = round8(s->nq_ext);
+    s->eps = 1e-6f;                                        // src/nn/fast_sft.c:190
+    s->lora_scaling = lora_rank > 0 ? lora_alpha / (float)lora_rank : 0.f;
+    s->emb_scale = m->model_type == MODEL_GEMMA3 ? sqrtf((float)m->d_model) : 1.0f;   // :302
+    s->step_count = 0;
+    s->weight_format = weight_format;
+    s->rope_thetas.assign(m->rope_thetas, m->rope_thetas + s->NL);
+    const int D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R, NL = s->NL, BN = s->BN, V = s->V;
+    if ((D & 7) || (qd & 7) || (kd & 7) || (IS & 7) || (s->nq_ext & 7) || (s->hd & 3) || (!weight_format && ((D & 31) || (IS & 31) || (qd & 31)))) {
+        fprintf(stderr, "[FastSFT] unsupported dims: d_model, head widths, FFN width and 2*rank must be multiples of 8 "
+                        "(32 for Q8_0)\n");
+        delete s;
+        fast_metal_shutdown();
+        return nullptr;
+    }
+
+    // ---- frozen weights: F16 arenas plus transposed copies for the dX products ----
+    s->wqkv = hbuf((size_t)NL * s->nq_ext * D);  s->wqkvT = hbuf((size_t)NL * D * s->ldq);
+    s->wo = hbuf((size_t)NL * D * qd);           s->woT = hbuf((size_t)NL * qd * D);
+    s->wgu = hbuf((size_t)NL * 2 * IS * D);      s->wguT = hbuf((size_t)NL * D * 2 * IS);
+    s->wd = hbuf((size_t)NL * D * IS);           s->wdT = hbuf((size_t)NL * IS * D);
+    s->wlm = hbuf((size_t)V * D);                s->wlmT = hbuf((size_t)D * round8(V));
+    HIP_CHECK(hipMemsetAsync(dptr(s->wqkv), 0, s->wqkv->size, stream()));
+    HIP_CHECK(hipMemsetAsync(dptr(s->wqkvT), 0, s->wqkvT->size, stream()));
+    HIP_CHECK(hipMemsetAsync(dptr(s->wlmT), 0, s->wlmT->size, stream()));
+    std::vector<MetalBuf *> q8_keep;
+    s->g_in = fbuf((size_t)NL * D); s->g_post_attn = fbuf((size_t)NL * D);
+    s->g_pre_ff = fbuf((size_t)NL * D); s->g_post_ff = fbuf((size_t)NL * D);
+    s->g_q = fbuf((size_t)NL * s->hd); s->g_k = fbuf((size_t)NL * s->hd);
+    for (int L = 0; L < NL; L++) {
+        const LayerWeightRef *r = &m->layers[L];
+        const size_t oq = (size_t)L * s->nq_ext * D;
+        put_matrix(s, s->wqkv, oq, r->q_proj.data, qd, D, q8_keep);
+        put_matrix(s, s->wqkv, oq + (size_t)qd * D, r->k_proj.data, kd, D, q8_keep);
+        put_matrix(s, s->wqkv, oq + (size_t)(qd + kd) * D, r->v_proj.data, kd, D, q8_keep);
+        put_matrix(s, s->wo, (size_t)L * D * qd, r->o_proj.data, D, qd, q8_keep);
+        put_matrix(s, s->wgu, (size_t)L * 2 * IS * D, r->gate_proj.data, IS, D, q8_keep);
+        put_matrix(s, s->wgu, (size_t)L * 2 * IS * D + (size_t)IS * D, r->up_proj.data, IS, D, q8_keep);
+        put_matrix(s, s->wd, (size_t)L * D * IS, r->down_proj.data, D, IS, q8_keep);
+        metal_buf_write(s->g_in, (size_t)L * D * 4, r->input_norm_g, (size_t)D * 4);
+        metal_buf_write(s->g_post_attn, (size_t)L * D * 4, r->post_attn_norm_g, (size_t)D * 4);
+        if (r->pre_ff_norm_g) metal_buf_write(s->g_pre_ff, (size_t)L * D * 4, r->pre_ff_norm_g, (size_t)D * 4);
+        if (r->post_ff_norm_g) metal_buf_write(s->g_post_ff, (size_t)L * D * 4, r->post_ff_norm_g, (size_t)D * 4);
+        metal_buf_write(s->g_q, (size_t)L * s->hd * 4, r->q_norm_g, (size_t)s->hd * 4);
+        metal_buf_write(s->g_k, (size_t)L * s->hd * 4, r->k_norm_g, (size_t)s->hd * 4);
+        launch_transpose_f16(at<half_t>(s->wo, (size_t)L * D * qd), at<half_t>(s->woT, (size_t)L * qd * D), D, qd, D);
+        launch_transpose_f16(at<half_t>(s->wgu, (size_t)L * 2 * IS * D), at<half_t>(s->wguT, (size_t)L * D * 2 * IS), 2 * IS, D, 2 * IS);
+        launch_transpose_f16(at<half_t>(s->wd, (size_t)L * D * IS), at<half_t>(s->wdT, (size_t)L * IS * D), D, IS, D);
+    }
+    put_matrix(s, s->wlm, 0, m->lm_head, V, D, q8_keep);
+    launch_transpose_f16(at<half_t>(s->wlm), at<half_t>(s->wlmT), V, D, round8(V));
+    s->g_final = metal_buf_from_data(m->final_norm_g, (size_t)D * 4);
+    s->emb = metal_buf_from_data(m->token_emb, (size_t)V * D * 4);
+    s->q8_blocks = nullptr;
+    for (MetalBuf *b : q8_keep) metal_buf_free(b);       // the bytes were only needed to form the values
+
+    // ---- LoRA arena, gradients, optimiser state ----
+    s->lsz = (size_t)2 * R * D + (size_t)qd * R + (size_t)kd * R;
+    s->lora_n = s->lsz * NL;
+    s->slots_per_layer = R ? lora_grad_blocks(D, qd, kd, R) : 1;
+    s->lora = fbuf(s->lora_n ? s->lora_n : 1); s->lora_grad = fbuf(s->lora_n ? s->lora_n : 1);
+    s->adam_m = fbuf(s->lora_n ? s->lora_n : 1); s->adam_v = fbuf(s->lora_n ? s->lora_n : 1);
+    s->sq_slots = fbuf((size_t)s->slots_per_layer * NL); s->grad_norm = fbuf(4);
+    HIP_CHECK(hipMemsetAsync(dptr(s->lora_grad), 0, s->lora_grad->size, stream()));
+    HIP_CHECK(hipMemsetAsync(dptr(s->adam_m), 0, s->adam_m->size, stream()));
+    HIP_CHECK(hipMemsetAsync(dptr(s->adam_v), 0, s->adam_v->size, stream()));
+    HIP_CHECK(hipMemsetAsync(dptr(s->sq_slots), 0, s->sq_slots->size, stream()));
+    HIP_CHECK(hipMemsetAsync(dptr(s->grad_norm), 0, s->grad_norm->size, stream()));
+    if (s->lora_n) {
+        if (m->lora_init) {
+            metal_buf_write(s->lora, 0, m->lora_init, s->lora_n * 4);
+        } else {                                           // init_lora_layer, src/nn/fast_sft.c:100-123
+            std::vector<float> tmp(s->lora_n, 0.f);
+            const float std_a = 1.0f / sqrtf((float)D);
+            for (int L = 0; L < NL; L++) {
+                float *aq = tmp.data() + L * s->lsz, *av = aq + (size_t)R * D + (size_t)qd * R;
+                for (size_t j = 0; j < (size_t)R * D; j++) aq[j] = ((float)rand() / (float)RAND_MAX - 0.5f) * 2.0f * std_a;
+                for (size_t j = 0; j < (size_t)R * D; j++) av[j] = ((float)rand() / (float)RAND_MAX - 0.5f) * 2.0f * std_a;
+            }
+            metal_buf_write(s->lora, 0, tmp.data(), s->lora_n * 4);
+        }
+    }
+    for (int L = 0; L < NL && R; L++) {
+        const size_t o = L * s->lsz * 4;
+        const size_t sz[4] = {(size_t)R * D * 4, (size_t)qd * R * 4, (size_t)R * D * 4, (size_t)kd * R * 4};
+        size_t off = o;
+        for (int k = 0; k < 4; k++) {
+            s->lora_views.push_back(metal_buf_view(s->lora, off, sz[k]));
+            s->grad_views.push_back(metal_buf_view(s->lora_grad, off, sz[k]));
+            off += sz[k];
+        }
+    }
+
+    // ---- host-visible small buffers ----
+    s->tokens = host_buf((size_t)BN * 4, (void **)&s->tokens_cpu);
+    s->targets = host_buf((size_t)BN * 4, (void **)&s->targets_cpu);
+    s->losses = host_buf((size_t)BN * 4, (void **)&s->losses_cpu);
+    s->hyper = host_buf(64, (void **)&s->hyper_cpu);
+    s->x_in_host = nullptr; s->x_cpu = nullptr;
+
+    // ---- saved activations and transients ----
+    const size_t xsz = (size_t)BN * D;
+    s->xs = fbuf((size_t)(2 * NL + 1) * xsz);
+    s->ln1_16 = hbuf((size_t)NL * xsz); s->ln1_inv = fbuf((size_t)NL * BN);
+    s->q_pre = fbuf((size_t)NL * BN * qd); s->k_pre = fbuf((size_t)NL * BN * kd);
+    s->q_fin = fbuf((size_t)NL * BN * qd); s->k_fin = fbuf((size_t)NL * BN * kd); s->v_sav = fbuf((size_t)NL * BN * kd);
+    s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
+    s->gate_pre = fbuf((size_t)NL * BN * IS); s->up_val = fbuf((size_t)NL * BN * IS);
+    s->tq = fbuf((size_t)NL * BN * (R ? R : 1)); s->tv = fbuf((size_t)NL * BN * (R ? R : 1));
+    const bool gemma = s->model_type == MODEL_GEMMA3;
+    s->o_raw = gemma ? fbuf((size_t)NL * xsz) : nullptr; s->ff_raw = gemma ? fbuf((size_t)NL * xsz) : nullptr;
+    int maxk = D;
+    if (qd > maxk) maxk = qd;
+    if (2 * IS > maxk) maxk = 2 * IS;
+    if (s->ldq > maxk) maxk = s->ldq;
+    s->a16 = hbuf((size_t)BN * maxk); s->a16_inv = fbuf(BN);
+    s->ones = fbuf(BN);
+    launch_fill_f32(at<float>(s->ones), 1.0f, BN);
+    s->planes_cap = max_planes_elems(s);
+    s->planes = fbuf(s->planes_cap);
+    s->logits = fbuf((size_t)BN * V); s->dlogits = nullptr;
+    s->dl16 = hbuf((size_t)BN * round8(V)); s->dl_inv = fbuf(BN);
+    s->dx[0] = fbuf(xsz); s->dx[1] = fbuf(xsz);
+    s->dO_red = fbuf((size_t)BN * qd); s->dscore = fbuf((size_t)s->B * s->Hq * s->N * s->N);
+    s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf((size_t)BN * kd);
+    s->dq_f = fbuf((size_t)BN * qd); s->dh = fbuf((size_t)BN * (R ? 2 * R : 1));
+
+    // the fused QKV weight carries fp16 images of A_q, A_v; its transpose follows from it
+    refresh_shadow(s);
+    for (int L = 0; L < NL; L++)
+        launch_transpose_f16(at<half_t>(s->wqkv, (size_t)L * s->nq_ext * D), at<half_t>(s->wqkvT, (size_t)L * D * s->ldq),
+                             s->nq_ext, D, s->ldq);
+    metal_flush();
+    return s;
+}
+
+void sft_state_free(SFTState *s)
+{
+    if (!s) return;
+    metal_flush();
+    for (MetalBuf *b : s->lora_views) metal_buf_free(b);
+    for (MetalBuf *b : s->grad_views) metal_buf_free(b);
+    MetalBuf *all[] = {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT, s->q8_blocks,
+                       s->g_in, s->g_post_attn, s->g_pre_ff, s->g_post_ff, s->g_q, s->g_k, s->g_final, s->emb,
+                       s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
+                       s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
+                       s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
+                       s->gate_pre, s->up_val, s->tq, s->tv, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->ones, s->planes,
+                       s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
+                       s->dq, s->dk, s->dv, s->dq_f, s->dh};
+    for (MetalBuf *b : all) metal_buf_free(b);
+    delete s;
+    fast_metal_shutdown();
+}
+
+void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr)
+{
+    memcpy(s->tokens_cpu, input_tokens, (size_t)s->BN * 4);
+    memcpy(s->targets_cpu, target_tokens, (size_t)s->BN * 4);
+    if (s->R) { s->step_count++; write_hyper(s, lr, s->step_count); }
+    forward_impl(s, true);
+    CeArgs ce{};
+    ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
+    ce.dl16 = at<half_t>(s->dl16); ce.ld16 = round8(s->V); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
+    launch_ce_rows(ce, s->BN);
+    backward_impl(s);
+    enqueue_update(s);
+}
+
+float sft_finish_train_step(SFTState *s)
+{
+    metal_flush();
+    float tot = 0.f;
+    for (int i = 0; i < s->BN; i++) tot += s->losses_cpu[i];
+    return tot / (float)s->BN;
+}
+
+float sft_train_step(SFTState *s, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr)
+{
+    sft_enqueue_train_step(s, input_tokens, target_tokens, lr);
+    return sft_finish_train_step(s);
+}
+
+void forward_to_logits(SFTState *s)
+{
+    if (!s->x_in_host) sft_get_x_cpu(s);
+    forward_impl(s, false);
+}
+
+void sft_backward(SFTState *s)
+{
+    MetalBuf *dl = sft_get_dlogits(s);
+    launch_rows_to_f16(at<float>(dl), s->V, at<half_t>(s->dl16), round8(s->V), at<float>(s->dl_inv), s->BN, s->V);
+    backward_impl(s);
+}
+
+void sft_lora_update(SFTState *s, float lr)
+{
+    // the caller has set the step count (src/nn/fast_grpo.c:488-490); gradients may have been replaced
+    // through sft_set_lora_grad, so the sums of squares are recomputed from the gradient arena
+    write_hyper(s, lr, s->step_count);
+    std::vector<float> g(s->lora_n);
+    metal_buf_read(s->lora_grad, 0, g.data(), s->lora_n * 4);
+    std::vector<float> slots((size_t)s->slots_per_layer * s->NL, 0.f);
+    double sq = 0;
+    for (float v : g) sq += (double)v * v;
+    slots[0] = (float)sq;
+    metal_buf_write(s->sq_slots, 0, slots.data(), slots.size() * 4);
+    enqueue_update(s);
+    metal_flush();
+}
+
+MetalBuf *sft_get_logits(SFTState *s) { return s->logits; }
+MetalBuf *sft_get_dlogits(SFTState *s)
+{
+    if (!s->dlogits) s->dlogits = fbuf((size_t)s->BN * s->V);
+    return s->dlogits;
+}
+float *sft_get_x_cpu(SFTState *s)
+{
+    if (!s->x_in_host) s->x_in_host = host_buf((size_t)s->BN * s->D * 4, (void **)&s->x_cpu);
+    return s->x_cpu;
+}
+float *sft_get_losses_cpu(SFTState *s) { return s->losses_cpu; }
+int sft_get_seq_len(SFTState *s) { return s->BN; }
+int sft_get_vocab_size(SFTState *s) { return s->V; }
+int sft_get_d_model(SFTState *s) { return s->D; }
+int sft_get_lora_rank(SFTState *s) { return s->R; }
+int sft_get_n_layers(SFTState *s) { return s->NL; }
+float sft_get_emb_scale(SFTState *s) { return s->emb_scale; }
+int sft_get_step_count(SFTState *s) { return s->step_count; }
+void sft_set_step_count(SFTState *s, int step) { s->step_count = step; }
+int sft_get_n_lora_grad_bufs(SFTState *s) { return (int)s->grad_views.size(); }
+float *sft_get_lora_grad_ptr(SFTState *s, int idx, int *out_size)
+{
+    if (idx < 0 || idx >= (int)s->grad_views.size()) return nullptr;
+    if (out_size) *out_size = (int)(s->grad_views[idx]->size / 4);
+    return (float *)metal_buf_ptr(s->grad_views[idx]);     // migrates the gradient arena to host memory
+}
+void sft_set_lora_grad(SFTState *s, int idx, const float *data, int size)
+{
+    if (idx < 0 || idx >= (int)s->grad_views.size()) return;
+    metal_buf_write(s->grad_views[idx], 0, data, (size_t)size * 4);
+}
+MetalBuf *sft_get_lora_weight_buf(SFTState *s, int layer, int sub)
+{
+    const size_t i = (size_t)layer * 4 + sub;
+    return i < s->lora_views.size() ? s->lora_views[i] : nullptr;
+}
+float sft_get_lora_scaling(SFTState *s) { return s->lora_scaling; }
+ModelType sft_get_model_type(SFTState *s) { return s->model_type; }
+int sft_get_n_q_heads(SFTState *s) { return s->Hq; }
+int sft_get_n_kv_heads(SFTState *s) { return s->Hkv; }
+int sft_get_head_dim(SFTState *s) { return s->hd; }
+int sft_get_intermediate_size(SFTState *s) { return s->IS; }
+const float *sft_get_rope_thetas(SFTState *s) { return s->rope_thetas.data(); }
+int sft_is_full_param(SFTState *s) { (void)s; return 0; }
+
+size_t sft_lora_numel(SFTState *s) { return s->lora_n; }
+void sft_copy_lora(SFTState *s, float *dst) { if (s->lora_n) metal_buf_read(s->lora, 0, dst, s->lora_n * 4); }
+void sft_copy_lora_grads(SFTState *s, float *dst) { if (s->lora_n) metal_buf_read(s->lora_grad, 0, dst, s->lora_n * 4); }
+void sft_set_lora(SFTState *s, const float *src)
+{
+    if (!s->lora_n) return;
+    metal_buf_write(s->lora, 0, src, s->lora_n * 4);
+    refresh_shadow(s);
+    metal_flush();
+}
+float sft_get_last_grad_norm(SFTState *s)
+{
+    float v = 0.f;
+    metal_buf_read(s->grad_norm, 0, &v, 4);
+    return v;
+}
+
+// "LORA" adapter file: u32 magic 0x4C4F5241, i32 n_layers, i32 rank, then per layer
+// A_q, B_q, A_v, B_v as fp32 (src/nn/fast_sft.c:1255-1285) — exactly the arena order.
+void sft_save_lora(SFTState *s, const char *path)
+{
+    FILE *f = fopen(path, "wb");
+    if (!f) { fprintf(stderr, "[FastSFT] Cannot open %s for writing\n", path); return; }
+    const uint32_t magic = 0x4C4F5241u;
+    const int32_t nl = s->NL, rank = s->R;
+    fwrite(&magic, 4, 1, f); fwrite(&nl, 4, 1, f); fwrite(&rank, 4, 1, f);
+    std::vector<float> w(s->lora_n);
+    sft_copy_lora(s, w.data());
+    fwrite(w.data(), 4, w.size(), f);
+    fclose(f);
+}
+
+}  // extern "C"

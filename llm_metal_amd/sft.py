@@ -1,0 +1,175 @@
+"""Python mirror of the C host API of the SFT step (include/sft_hip.h), used by
+tests and bench.py: device buffers as thin handles, the SFT state as a class.
+Every method is one call into libllm_metal_hip.so."""
+import ctypes as C
+
+import numpy as np
+
+from . import lib as _lib
+from .configs import SFTConfig
+
+
+def _vp(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Backend:
+    """fast_metal_init / fast_metal_shutdown as a context manager."""
+
+    def __init__(self):
+        self.L = _lib.load()
+        if self.L.fast_metal_init() != 0:
+            raise RuntimeError("fast_metal_init failed: no gfx950 device (this library has no CPU path)")
+
+    def close(self):
+        if self.L is not None:
+            self.L.fast_metal_shutdown()
+            self.L = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # -- buffers
+    def buf(self, arr):
+        arr = np.ascontiguousarray(arr)
+        return Buf(self.L, self.L.metal_buf_from_data(_vp(arr), arr.nbytes), arr.nbytes)
+
+    def empty(self, nbytes):
+        return Buf(self.L, self.L.metal_buf_create(nbytes), nbytes)
+
+    def flush(self):
+        self.L.metal_flush()
+
+
+class Buf:
+    def __init__(self, L, handle, nbytes, owned=True):
+        if not handle:
+            raise RuntimeError("buffer creation failed")
+        self.L, self.h, self.nbytes, self.owned = L, handle, nbytes, owned
+
+    def read(self, dtype, shape=None):
+        out = np.empty(self.nbytes // np.dtype(dtype).itemsize, dtype=dtype)
+        self.L.metal_buf_read(self.h, 0, _vp(out), out.nbytes)
+        return out.reshape(shape) if shape is not None else out
+
+    def write(self, arr):
+        arr = np.ascontiguousarray(arr)
+        self.L.metal_buf_write(self.h, 0, _vp(arr), arr.nbytes)
+
+    def free(self):
+        if self.owned and self.h:
+            self.L.metal_buf_free(self.h)
+        self.h = None
+
+
+def _layer_refs(c: SFTConfig, model, keep):
+    refs = (_lib.LayerWeightRef * c.NL)()
+    names = {"q_proj": "wq", "k_proj": "wk", "v_proj": "wv", "o_proj": "wo",
+             "gate_proj": "wg", "up_proj": "wu", "down_proj": "wd"}
+    gam = {"input_norm_g": "g_in", "post_attn_norm_g": "g_post_attn", "pre_ff_norm_g": "g_pre_ff",
+           "post_ff_norm_g": "g_post_ff", "q_norm_g": "g_q", "k_norm_g": "g_k"}
+    for L in range(c.NL):
+        for field, key in names.items():
+            a = np.ascontiguousarray(model[key][L], dtype=np.float32)
+            keep.append(a)
+            setattr(refs[L], field, _lib.WeightRef(a.ctypes.data, a.shape[0], a.shape[1]))
+        for field, key in gam.items():
+            g = model[key][L]
+            if g is None:
+                setattr(refs[L], field, None)
+            else:
+                a = np.ascontiguousarray(g, dtype=np.float32)
+                keep.append(a)
+                setattr(refs[L], field, a.ctypes.data)
+        refs[L].d_model = c.D
+        refs[L].head_dim = c.hd
+    return refs
+
+
+class SFTState:
+    """sft_state_create_from_ref ... sft_state_free."""
+
+    def __init__(self, c: SFTConfig, model, lora_init=True):
+        self.L = _lib.load()
+        self.c = c
+        keep = []
+        refs = _layer_refs(c, model, keep)
+        thetas = np.asarray(c.rope_thetas(), dtype=np.float32)
+        emb = np.ascontiguousarray(model["token_emb"], dtype=np.float32)
+        head = emb if model["lm_head"] is model["token_emb"] else np.ascontiguousarray(model["lm_head"], dtype=np.float32)
+        gf = np.ascontiguousarray(model["g_final"], dtype=np.float32)
+        lora = np.ascontiguousarray(model["lora"], dtype=np.float32) if (lora_init and c.R) else None
+        m = _lib.SFTModelRef(c.model_type, c.NL, c.D, c.Hq, c.Hkv, c.hd, c.IS, c.V, thetas.ctypes.data, refs,
+                             emb.ctypes.data, head.ctypes.data, gf.ctypes.data,
+                             lora.ctypes.data if lora is not None else None)
+        self.h = self.L.sft_state_create_from_ref(C.byref(m), c.batch, c.seq, c.R, c.alpha,
+                                                  1 if c.weight_format == "f16" else 0)
+        if not self.h:
+            raise RuntimeError("sft_state_create_from_ref failed (no gfx950 device or unsupported dims)")
+
+    def train_step(self, tok, tgt, lr):
+        tok = np.ascontiguousarray(tok, dtype=np.uint32)
+        tgt = np.ascontiguousarray(tgt, dtype=np.uint32)
+        return float(self.L.sft_train_step(self.h, _vp(tok), _vp(tgt), lr))
+
+    def enqueue_train_step(self, tok, tgt, lr):
+        self.L.sft_enqueue_train_step(self.h, _vp(tok), _vp(tgt), lr)
+
+    def finish_train_step(self):
+        return float(self.L.sft_finish_train_step(self.h))
+
+    def lora(self):
+        out = np.empty(self.L.sft_lora_numel(self.h), dtype=np.float32)
+        self.L.sft_copy_lora(self.h, _vp(out))
+        return out
+
+    def lora_grads(self):
+        out = np.empty(self.L.sft_lora_numel(self.h), dtype=np.float32)
+        self.L.sft_copy_lora_grads(self.h, _vp(out))
+        return out
+
+    def set_lora(self, arr):
+        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        assert arr.size == self.L.sft_lora_numel(self.h)
+        self.L.sft_set_lora(self.h, _vp(arr))
+
+    def logits(self):
+        b = Buf(self.L, self.L.sft_get_logits(self.h), self.c.BN * self.c.V * 4, owned=False)
+        return b.read(np.float32, (self.c.BN, self.c.V))
+
+    def losses(self):
+        p = self.L.sft_get_losses_cpu(self.h)
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_float)), shape=(self.c.BN,)).copy()
+
+    def grad_norm(self):
+        return float(self.L.sft_get_last_grad_norm(self.h))
+
+    def step_count(self):
+        return self.L.sft_get_step_count(self.h)
+
+    def x_cpu(self):
+        p = self.L.sft_get_x_cpu(self.h)
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_float)), shape=(self.c.BN, self.c.D))
+
+    def dlogits_buf(self):
+        return Buf(self.L, self.L.sft_get_dlogits(self.h), self.c.BN * self.c.V * 4, owned=False)
+
+    def forward_to_logits(self):
+        self.L.forward_to_logits(self.h)
+
+    def backward(self):
+        self.L.sft_backward(self.h)
+
+    def free(self):
+        if self.h:
+            self.L.sft_state_free(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.free()

@@ -1,0 +1,44 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every function that
+include/*.h declares, and refuses to start without a GPU (no compute calls here)."""
+import os
+
+import pytest
+
+from llm_metal_amd import lib
+
+
+@pytest.fixture(scope="module")
+def L():
+    if not os.path.exists(lib.LIB_PATH):
+        lib.build()
+    return lib.load()
+
+
+def test_every_declared_symbol_is_exported(L):
+    decl = lib.declared_symbols()
+    assert len(decl) >= 90
+    missing = [n for n in decl if not hasattr(L, n)]
+    assert not missing, missing
+
+
+def test_reference_abi_names_present(L):
+    # the 33 symbols of src/nn/fast_metal.h the LoRA SFT step uses, plus the 3 of the GRPO accumulate path
+    names = """fast_metal_init fast_metal_shutdown metal_buf_create metal_buf_from_data metal_buf_free metal_buf_ptr
+    metal_flush metal_enqueue_rms_norm_batched metal_enqueue_silu_mul metal_enqueue_gelu_mul metal_enqueue_residual_add
+    metal_enqueue_f16_matmul metal_enqueue_f16_matmul_nt metal_enqueue_transpose_heads_fwd
+    metal_enqueue_transpose_heads_rev metal_enqueue_repeat_kv metal_enqueue_rope_train metal_enqueue_silu_mul_backward
+    metal_enqueue_gelu_mul_backward metal_enqueue_rms_norm_backward metal_enqueue_scale metal_enqueue_add_scaled
+    metal_enqueue_softmax_ce metal_enqueue_attn_train_fwd metal_enqueue_attn_bwd_dq metal_enqueue_attn_bwd_dkv
+    metal_enqueue_repeat_kv_bwd metal_enqueue_rope_train_bwd metal_enqueue_float_matmul metal_enqueue_float_matmul_tn
+    metal_enqueue_float_matmul_nt metal_enqueue_copy metal_enqueue_clamp metal_enqueue_f16_sgd_fused
+    metal_enqueue_grpo_policy_grad metal_enqueue_f16_grad_accum metal_enqueue_f16_sgd_apply""".split()
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def test_init_fails_loudly_without_a_gpu(L):
+    import torch
+    if torch.cuda.device_count() > 0:
+        pytest.skip("a GPU is present")
+    assert L.fast_metal_init() == -1
+    assert not L.metal_buf_create(16)          # refused before init, returns NULL
