@@ -6,6 +6,8 @@ N(0, 0.01) for parity runs (a zero B makes the first-step dA exactly zero),
 tokens uniform on [0, V), target = next token with the last wrapping to the
 first (main.c:471-477).
 """
+import os
+
 import numpy as np
 from .configs import SFTConfig, GEMMA3
 
@@ -24,15 +26,40 @@ def _normal(rng, shape, std):
     return a
 
 
-def make_model(c: SFTConfig, seed=0, gamma_jitter=0.0, lora_b_std=0.01):
+def make_model(c: SFTConfig, seed=0, gamma_jitter=0.0, lora_b_std=0.01, threads=None):
     """Returns a dict of fp32 numpy arrays: per-layer lists for the 7 matrices and
     the norm gammas, token_emb, lm_head (same object when tied), g_final, lora
-    (flat [NL * lora_layer_size]: A_q | B_q | A_v | B_v per layer)."""
-    rng = np.random.default_rng(seed)
+    (flat [NL * lora_layer_size]: A_q | B_q | A_v | B_v per layer).  Every array has
+    its own generator derived from (seed, index), so the result does not depend on
+    how many threads filled it."""
+    from concurrent.futures import ThreadPoolExecutor
     shp = mat_shapes(c)
-    m = {k: [] for k in MATS}
-    for k in ("g_in", "g_post_attn", "g_pre_ff", "g_post_ff", "g_q", "g_k"):
-        m[k] = []
+    m = {k: [None] * c.NL for k in MATS}
+    jobs = []                                              # (dict, key/index, shape)
+    for L in range(c.NL):
+        for k in MATS:
+            jobs.append((m[k], L, shp[k]))
+    m["token_emb"] = None
+    jobs.append((m, "token_emb", (c.V, c.D)))
+    if not c.tied:
+        jobs.append((m, "lm_head", (c.V, c.D)))
+    seqs = np.random.SeedSequence(seed).spawn(len(jobs) + 2)
+
+    def fill(i):
+        dst, key, shape = jobs[i]
+        dst[key] = _normal(np.random.default_rng(seqs[i]), shape, 0.02)
+
+    big = sum(int(np.prod(j[2])) for j in jobs) > 50_000_000
+    if big:
+        with ThreadPoolExecutor(threads or min(16, (os.cpu_count() or 8))) as ex:
+            list(ex.map(fill, range(len(jobs))))
+    else:
+        for i in range(len(jobs)):
+            fill(i)
+    if c.tied:
+        m["lm_head"] = m["token_emb"]
+
+    rng = np.random.default_rng(seqs[-2])
 
     def gamma(n):
         g = np.ones(n, dtype=np.float32)
@@ -40,9 +67,9 @@ def make_model(c: SFTConfig, seed=0, gamma_jitter=0.0, lora_b_std=0.01):
             g += _normal(rng, n, gamma_jitter)
         return g
 
+    for k in ("g_in", "g_post_attn", "g_pre_ff", "g_post_ff", "g_q", "g_k"):
+        m[k] = []
     for _ in range(c.NL):
-        for k in MATS:
-            m[k].append(_normal(rng, shp[k], 0.02))
         m["g_in"].append(gamma(c.D))
         m["g_post_attn"].append(gamma(c.D))
         m["g_pre_ff"].append(gamma(c.D) if c.model_type == GEMMA3 else None)
@@ -50,9 +77,7 @@ def make_model(c: SFTConfig, seed=0, gamma_jitter=0.0, lora_b_std=0.01):
         m["g_q"].append(gamma(c.hd))
         m["g_k"].append(gamma(c.hd))
     m["g_final"] = gamma(c.D)
-    m["token_emb"] = _normal(rng, (c.V, c.D), 0.02)
-    m["lm_head"] = m["token_emb"] if c.tied else _normal(rng, (c.V, c.D), 0.02)
-    m["lora"] = make_lora(c, rng, lora_b_std)
+    m["lora"] = make_lora(c, np.random.default_rng(seqs[-1]), lora_b_std)
     return m
 
 

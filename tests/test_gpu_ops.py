@@ -269,16 +269,19 @@ def test_softmax_ce_and_grpo(dev, B, V):
     losses, dl = dev.empty(B * 4), dev.empty(B * V * 4)
     lgb, tb = dev.up(lg), dev.up(tgt)
     dev.L.metal_enqueue_softmax_ce(lgb.h, tb.h, losses.h, dl.h, B, V)
-    rl, rd = np.zeros(B, F), np.zeros((B, V), F)
-    op("f32", "or_softmax_ce", lg, tgt, rl, rd, B, V)
+    # reference in double: a sequential fp32 sum over 151936 terms is itself only good to ~2e-5
+    rl, rd = np.zeros(B), np.zeros((B, V))
+    op("f64", "or_softmax_ce", lg.astype(np.float64), tgt, rl, rd, B, V)
     assert maxrel(losses.read(F), rl) < 1e-5 and maxrel(dl.read(F, (B, V)), rd) < 1e-5
     assert np.abs(dl.read(F, (B, V)).sum(-1)).max() < 1e-4
+    rl = rl.astype(F)
     old = (-rl + rng.uniform(-0.4, 0.4, B)).astype(F)       # ratios on both sides of the clip band
     adv = rnd(rng, B)
     new_lp = dev.empty(B * 4)
     dev.L.metal_enqueue_grpo_policy_grad(lgb.h, tb.h, dev.up(old).h, dev.up(adv).h, new_lp.h, dl.h, B, V, 0.2)
-    rn, rg = np.zeros(B, F), np.zeros((B, V), F)
-    op("f32", "or_grpo_policy_grad", lg, tgt, old, adv, rn, rg, B, V, 0.2)
+    rn, rg = np.zeros(B), np.zeros((B, V))
+    op("f64", "or_grpo_policy_grad", lg.astype(np.float64), tgt, old.astype(np.float64), adv.astype(np.float64),
+       rn, rg, B, V, 0.2)
     assert maxrel(new_lp.read(F), rn) < 1e-5
     got = dl.read(F, (B, V))
     same_gate = (np.abs(got).sum(-1) > 0) == (np.abs(rg).sum(-1) > 0)
