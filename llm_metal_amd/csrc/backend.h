@@ -14,10 +14,9 @@ struct MetalBuf {
     int     owns;         // 0 for views
     MetalBuf *parent;     // views: the buffer whose allocation this window lies in
     size_t  parent_off;
-    // lazily built transposed F16 copy used by metal_enqueue_f16_matmul_nt
-    void   *t_dev;
-    int     t_rows, t_cols;
-    uint64_t t_version;   // version of `dev` contents the copy was made from
+    // lazily built tiled images of an F16 weight held in this buffer ([0] as is, [1] transposed),
+    // used by metal_enqueue_f16_matmul / _nt
+    struct Tiled { void *dev; int rows, cols; uint64_t version; } tiled[2];
     uint64_t version;     // bumped by every enqueue that writes this buffer
 };
 

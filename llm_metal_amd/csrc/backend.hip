@@ -120,7 +120,7 @@ void metal_buf_free(MetalBuf *b)
 {
     if (!b) return;
     if (g_stream) hipStreamSynchronize(g_stream);
-    if (b->t_dev) hipFree(b->t_dev);
+    for (auto &t : b->tiled) if (t.dev) hipFree(t.dev);
     if (b->owns) {
         if (b->host) hipHostFree(b->host);
         else if (b->dev) hipFree(b->dev);

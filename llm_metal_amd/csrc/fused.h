@@ -5,6 +5,7 @@
 #pragma once
 #include "backend.h"
 #include "devutil.h"
+#include "gemm.h"
 
 namespace lmhip {
 
@@ -24,7 +25,7 @@ struct NormRowsArgs {
     Planes branch; const float *g_branch; float *branch_raw_out;
     float *x_out;                 // new residual stream row (may be null when nothing was added)
     const float *g_norm;          // null: no normalised output wanted
-    half_t *ln16; int ld16; float *inv_scale;
+    half_t *ln16; float *inv_scale;   // tiled [rows, D]
     int D; float eps;
 };
 void launch_norm_rows(const NormRowsArgs &a, int rows);
@@ -33,19 +34,22 @@ struct QkvPostArgs {
     Planes qkv;                   // [rows][q | k | v | tq(R) | tv(R)]
     const float *Bq, *Bv;         // LoRA B, [Hq*hd][R], [Hkv*hd][R]
     int R; float sc;
-    const float *g_q, *g_k; float eps, theta;
+    const float *g_q, *g_k; float eps;
+    const float2 *rope;           // [seq][hd/2] (cos, sin) of this layer's theta
     int Hq, Hkv, hd, seq;
     float *q_pre, *k_pre, *q_fin, *k_fin, *v_out;   // [rows][H*hd]
     float *tq, *tv;               // [rows][R]
     int rows;
 };
 void launch_qkv_post(const QkvPostArgs &a, int rows);
+// tab[pos][d] = (cos, sin)(pos * theta^(-2d/hd)), pos < seq, d < hd/2
+void launch_rope_table(float2 *tab, int seq, int hd, float theta);
 
 // Causal GQA attention over [rows][H*hd] row-major activations, probabilities saved.
 struct AttnFwdArgs {
     const float *q, *k, *v; int Hq, Hkv, hd, seq, batch; float scale;
     float *probs;                 // [batch][Hq][seq][seq]
-    half_t *out16; int ld16;      // [rows][Hq*hd], unit scale
+    half_t *out16;                // tiled [rows, Hq*hd], unit scale
 };
 void launch_attn_fwd(const AttnFwdArgs &a);
 
@@ -59,18 +63,19 @@ void launch_attn_bwd(const AttnBwdArgs &a);
 
 struct QkvBwdArgs {
     const float *dq, *dk, *dv;    // post-RoPE-domain gradients
-    const float *q_pre, *k_pre, *g_q, *g_k; float eps, theta;
+    const float *q_pre, *k_pre, *g_q, *g_k; float eps;
+    const float2 *rope;
     const float *Bq, *Bv; int R; float sc;
     int Hq, Hkv, hd, seq;
     float *dq_f, *dv_f;           // pre-norm-domain dq [rows][Hq*hd], dv copy [rows][Hkv*hd] (for dB)
     float *dh;                    // [rows][2R] = sc * dq B_q | sc * dv B_v
-    half_t *out16; int ld16; float *inv_scale;      // [rows][dq | dk | dv | dh_q | dh_v | 0-pad]
+    half_t *out16; float *inv_scale;                // tiled [rows, dq | dk | dv | dh_q | dh_v]
 };
 void launch_qkv_bwd(const QkvBwdArgs &a, int rows);
 
 struct LoraGradArgs {
     const float *dq_f, *dv_f, *tq, *tv, *dh;
-    const half_t *ln16; int ld16; const float *ln_inv_scale;
+    const half_t *ln16; const float *ln_inv_scale;  // tiled [rows, D]
     int rows, D, qd, kd, R; float sc;
     float *grad;                  // this layer's arena: dA_q | dB_q | dA_v | dB_v
     float *sq_slots;              // one partial sum of squares per workgroup
@@ -82,7 +87,7 @@ struct GluArgs {
     Planes in;                    // fwd: [rows][gate | up]; bwd: [rows][d act]
     int IS, gelu;
     float *gate_pre, *up_val;     // fwd: written; bwd: read
-    half_t *out16; int ld16; float *inv_scale;      // fwd: act [rows][IS]; bwd: [rows][dgate | dup]
+    half_t *out16; float *inv_scale;                // tiled; fwd: act [rows, IS]; bwd: [rows, dgate | dup]
 };
 void launch_glu_fwd(const GluArgs &a, int rows);
 void launch_glu_bwd(const GluArgs &a, int rows);
@@ -91,13 +96,13 @@ struct NormBwdArgs {
     Planes dy; const float *x_saved, *g; float eps; int D;
     const float *dx_prev; float *dx_out; float clamp;   // clamp <= 0: none
     const float *branch_raw, *g_branch;                 // Gemma3: next GEMM input is RNB(branch_raw, dx_out)
-    half_t *d16; int ld16; float *inv_scale;            // may be null on the last kernel of the backward
+    half_t *d16; float *inv_scale;                      // tiled [rows, D]; may be null on the last kernel of the backward
 };
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows);
 
 struct CeArgs {
     const float *logits; int V; const uint32_t *targets; float *losses;
-    half_t *dl16; int ld16; float *inv_scale; int rows_total;
+    half_t *dl16; float *inv_scale; int rows_total;     // tiled [rows, V]
 };
 void launch_ce_rows(const CeArgs &a, int rows);
 
@@ -107,7 +112,7 @@ struct AdamArgs {
     const float *hyper;           // device-visible: [0] lr, [1] 1-b1^t, [2] 1-b2^t, written by the host per step
     float b1, b2, eps, wd, max_norm;
     // fp16 shadows of A_q / A_v inside the fused QKV weight and its transpose
-    half_t *wqkv; size_t wqkv_layer_stride; half_t *wqkvT; size_t wqkvT_layer_stride; int ldT;
+    half_t *wqkv; size_t wqkv_layer_stride; half_t *wqkvT; size_t wqkvT_layer_stride;   // tiled
     int NL, D, qd, kd, R; size_t layer_size;
     float *grad_norm_out;         // [1]
 };
@@ -115,7 +120,7 @@ void launch_adamw(const AdamArgs &a);
 
 // fp16 shadow refresh only (after LoRA weights were written from outside)
 void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
-                        size_t wqkvT_layer_stride, int ldT, int D, int qd, int kd, int R, size_t layer_size);
+                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size);
 
 void launch_fill_f32(float *p, float v, size_t n);
 

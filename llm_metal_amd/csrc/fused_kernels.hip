@@ -1,15 +1,22 @@
 // Fused row / head kernels of the SFT step.  Each one sits between two
 // weight-streaming GEMMs: it sums the producer GEMM's K-split partial planes on
 // load, does the reference's per-row arithmetic in fp32 (shaders/q8_kernels.metal,
-// cited per kernel) and writes what the next GEMM reads as a scaled fp16 row.
-// One launch here replaces between 3 and 12 dispatches of the reference's
-// forward_to_logits / sft_backward_ex (src/nn/fast_sft.c:616-982).
+// cited per kernel) and writes what the next GEMM reads as a scaled fp16 row in
+// the GEMM's tiled layout.  One launch here replaces between 3 and 12 dispatches
+// of the reference's forward_to_logits / sft_backward_ex (src/nn/fast_sft.c:616-982).
+//
+// With 64..160 rows per step these kernels are latency bound, not bandwidth
+// bound: a row gets one 1024-thread workgroup, every thread keeps its few float4
+// of the row in registers between the reductions, and all plane loads of a
+// thread are independent so they are in flight together.
 #include "fused.h"
 
 namespace lmhip {
 namespace {
 
 constexpr int TB = 256;
+constexpr int RB = 1024;                                  // threads of a row workgroup
+constexpr int MAXV = 3;                                   // float4 per thread: rows up to 12288 wide
 
 __device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
 {
@@ -19,54 +26,138 @@ __device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
     return s;
 }
 
-__device__ __forceinline__ void write_f16_row(const float *vals, int n, half_t *out, int ld, float s)
+// Sum of the planes at four consecutive columns (col % 4 == 0, ld % 4 == 0).
+__device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int col)
 {
-    for (int i = threadIdx.x; i < ld; i += blockDim.x) out[i] = (i < n) ? f2h(vals[i] * s) : (half_t)0;
+    const float *p = P.p + row * P.ld + col;
+    float4 s = *reinterpret_cast<const float4 *>(p);
+    int i = 1;
+    for (; i + 1 < P.S; i += 2) {
+        const float4 a = *reinterpret_cast<const float4 *>(p + (size_t)i * P.stride);
+        const float4 b = *reinterpret_cast<const float4 *>(p + (size_t)(i + 1) * P.stride);
+        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+    }
+    if (i < P.S) {
+        const float4 a = *reinterpret_cast<const float4 *>(p + (size_t)i * P.stride);
+        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+    }
+    return s;
+}
+
+__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
+__device__ __forceinline__ float sumsq4(float4 v) { return v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+
+// four consecutive elements (k % 4 == 0) of row `row` of a tiled fp16 operand
+__device__ __forceinline__ void st_tiled4(half_t *out, size_t row, int k, int Kb, float4 v, float s)
+{
+    half4 h = {f2h(v.x * s), f2h(v.y * s), f2h(v.z * s), f2h(v.w * s)};
+    *reinterpret_cast<half4 *>(out + tiled_index((int)row, k, Kb)) = h;
+}
+
+// zero the K padding [n, Kb*64) of a tiled row
+__device__ __forceinline__ void zero_tiled_pad(half_t *out, size_t row, int n, int Kb)
+{
+    for (int i = n + threadIdx.x; i < Kb * 64; i += blockDim.x) out[tiled_index((int)row, i, Kb)] = (half_t)0;
+}
+
+// Row `row` of a tiled fp16 operand [*, n] from fp32 values in LDS, scaled by s.
+__device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t *out, size_t row, float s)
+{
+    const int Kb = tiled_kb(n);
+    for (int c = threadIdx.x; c < Kb * 8; c += blockDim.x) {
+        half8 hv;
+#pragma unroll
+        for (int e = 0; e < 8; e++) { const int i = c * 8 + e; hv[e] = (i < n) ? f2h(vals[i] * s) : (half_t)0; }
+        *reinterpret_cast<half8 *>(out + tiled_index((int)row, c * 8, Kb)) = hv;
+    }
 }
 
 // ------------------------------------------------------------------ forward rows
 // x = (gathered embedding | x_prev) [+ branch | + RN(branch; g_branch)];  ln = RN(x; g_norm).
 // rms_norm: shaders/q8_kernels.metal:133-158; residual_add :369-375; the Gemma3
 // ordering (norm the branch, then add) is src/nn/fast_sft.c:698-705, 732-736.
-__global__ __launch_bounds__(TB) void k_norm_rows(NormRowsArgs a)
+__global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
-    extern __shared__ float lds[];
-    float *row = lds, *brow = lds + a.D;
     __shared__ float sm[16];
     const size_t r = blockIdx.x;
-    const int D = a.D;
-    if (a.emb) {
-        const float *e = a.emb + (size_t)a.tokens[r] * D;
-        for (int i = threadIdx.x; i < D; i += TB) row[i] = (a.emb_scale != 1.0f) ? e[i] * a.emb_scale : e[i];
-    } else {
-        for (int i = threadIdx.x; i < D; i += TB) row[i] = a.x_prev[r * D + i];
-    }
-    if (a.branch.S > 0) {
-        float ss = 0.f;
-        for (int i = threadIdx.x; i < D; i += TB) { const float b = planes_at(a.branch, r, i); brow[i] = b; ss += b * b; }
-        if (a.g_branch) {
-            ss = block_sum(ss, sm);
-            const float inv = rsqrtf(ss / (float)D + a.eps);
-            for (int i = threadIdx.x; i < D; i += TB) {
-                if (a.branch_raw_out) a.branch_raw_out[r * D + i] = brow[i];
-                row[i] += brow[i] * inv * a.g_branch[i];
-            }
-        } else {
-            for (int i = threadIdx.x; i < D; i += TB) row[i] += brow[i];
+    const int D = a.D, nv = D >> 2;
+    float4 x[MAXV], b[MAXV];
+    const float *base = a.emb ? a.emb + (size_t)a.tokens[r] * D : a.x_prev + r * D;
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        x[t] = b[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) {
+            x[t] = ld4(base + 4 * v);
+            if (a.emb && a.emb_scale != 1.0f) { x[t].x *= a.emb_scale; x[t].y *= a.emb_scale; x[t].z *= a.emb_scale; x[t].w *= a.emb_scale; }
+            if (a.branch.S > 0) b[t] = planes_at4(a.branch, r, 4 * v);
         }
     }
-    if (a.x_out) for (int i = threadIdx.x; i < D; i += TB) a.x_out[r * D + i] = row[i];
+    if (a.branch.S > 0) {
+        float inv = 1.0f;
+        if (a.g_branch) {
+            float ss = 0.f;
+#pragma unroll
+            for (int t = 0; t < MAXV; t++) ss += sumsq4(b[t]);
+            ss = block_sum(ss, sm);
+            inv = rsqrtf(ss / (float)D + a.eps);
+        }
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const int v = threadIdx.x + t * RB;
+            if (v >= nv) continue;
+            if (a.g_branch) {
+                if (a.branch_raw_out) st4(a.branch_raw_out + r * D + 4 * v, b[t]);
+                const float4 g = ld4(a.g_branch + 4 * v);
+                x[t].x += b[t].x * inv * g.x; x[t].y += b[t].y * inv * g.y;
+                x[t].z += b[t].z * inv * g.z; x[t].w += b[t].w * inv * g.w;
+            } else {
+                x[t].x += b[t].x; x[t].y += b[t].y; x[t].z += b[t].z; x[t].w += b[t].w;
+            }
+        }
+    }
+    if (a.x_out) {
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st4(a.x_out + r * D + 4 * v, x[t]); }
+    }
     if (!a.g_norm) return;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < D; i += TB) ss += row[i] * row[i];
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) ss += sumsq4(x[t]);
     ss = block_sum(ss, sm);
     const float inv = rsqrtf(ss / (float)D + a.eps);
     float amax = 0.f;
-    for (int i = threadIdx.x; i < D; i += TB) { const float v = row[i] * inv * a.g_norm[i]; brow[i] = v; amax = fmaxf(amax, fabsf(v)); }
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        if (v >= nv) continue;
+        const float4 g = ld4(a.g_norm + 4 * v);
+        x[t].x = x[t].x * inv * g.x; x[t].y = x[t].y * inv * g.y; x[t].z = x[t].z * inv * g.z; x[t].w = x[t].w * inv * g.w;
+        amax = fmaxf(amax, amax4(x[t]));
+    }
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
-    write_f16_row(brow, D, a.ln16 + r * a.ld16, a.ld16, s);   // each thread re-reads only what it wrote
+    const int Kb = tiled_kb(D);
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st_tiled4(a.ln16, r, 4 * v, Kb, x[t], s); }
+    zero_tiled_pad(a.ln16, r, D, Kb);
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
+}
+
+// cos/sin of pos * theta^(-2d/hd), exactly as rope_train forms them
+// (shaders/q8_kernels.metal:527-530): table[pos][d] = (cos, sin), d < hd/2.
+__global__ void k_rope_table(float2 *tab, int seq, int half, int hd, float theta)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= seq * half) return;
+    const int pos = idx / half, d = idx % half;
+    const float freq = 1.0f / powf(theta, (float)(2 * d) / (float)hd);
+    float s, c;
+    sincosf((float)pos * freq, &s, &c);
+    tab[idx] = make_float2(c, s);
 }
 
 // ------------------------------------------------------------------ QKV epilogue
@@ -109,12 +200,11 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
         }
         if (lora) {                                           // uniform branch: shuffles stay convergent
             float acc0 = 0.f, acc1 = 0.f;
+            const float *b0 = B + (size_t)(h * hd + (d < half ? d : 0)) * a.R;
+            const float *b1 = b0 + (size_t)half * a.R;
             for (int r = 0; r < a.R; r++) {
                 const float t = __shfl(tval, r, WAVE);
-                if (d < half) {
-                    acc0 += t * B[(size_t)(h * hd + d) * a.R + r];
-                    acc1 += t * B[(size_t)(h * hd + d + half) * a.R + r];
-                }
+                if (d < half) { acc0 += t * b0[r]; acc1 += t * b1[r]; }
             }
             x0[p] += a.sc * acc0;
             x1[p] += a.sc * acc1;
@@ -143,11 +233,9 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
         pre[o] = x0[p];
         pre[o + half] = x1[p];
         const float n0 = x0[p] * inv * g[d], n1 = x1[p] * inv * g[d + half];
-        const float freq = 1.0f / powf(a.theta, (float)(2 * d) / (float)hd);
-        float s, c;
-        sincosf((float)pos * freq, &s, &c);
-        fin[o] = n0 * c - n1 * s;
-        fin[o + half] = n0 * s + n1 * c;
+        const float2 cs = a.rope[(size_t)pos * half + d];
+        fin[o] = n0 * cs.x - n1 * cs.y;
+        fin[o + half] = n0 * cs.y + n1 * cs.x;
     }
 }
 
@@ -170,6 +258,7 @@ __global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
     for (int j = lane; j <= i; j += 64) {
         const float4 *kr = reinterpret_cast<const float4 *>(a.k + (r0 + j) * kd + hk * hd);
         float dot = 0.f;
+#pragma unroll 8
         for (int d4 = 0; d4 < hd / 4; d4++) {
             const float4 kv = kr[d4];
             dot += qs[4 * d4] * kv.x + qs[4 * d4 + 1] * kv.y + qs[4 * d4 + 2] * kv.z + qs[4 * d4 + 3] * kv.w;
@@ -190,11 +279,15 @@ __global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
         pr[j] = p;
     }
     __syncthreads();
+    const int Kb = tiled_kb(qd);
     for (int d = lane; d < hd; d += 64) {
         float acc = 0.f;
+#pragma unroll 8
         for (int j = 0; j <= i; j++) acc += sc[j] * a.v[(r0 + j) * kd + hk * hd + d];
-        a.out16[(r0 + i) * a.ld16 + h * hd + d] = f2h(acc);
+        a.out16[tiled_index((int)(r0 + i), h * hd + d, Kb)] = f2h(acc);
     }
+    if (h == a.Hq - 1)                                    // zero the K padding of this row once
+        for (int c = qd + lane; c < Kb * 64; c += 64) a.out16[tiled_index((int)(r0 + i), c, Kb)] = (half_t)0;
 }
 
 // attn_bwd_dq, shaders/q8_kernels.metal:857-925.  Also leaves the plane-summed dO
@@ -218,6 +311,7 @@ __global__ __launch_bounds__(64) void k_attn_bwd_dq(AttnBwdArgs a)
     for (int j = lane; j <= i; j += 64) {
         const float4 *vr = reinterpret_cast<const float4 *>(a.v + (r0 + j) * kd + hk * hd);
         float dot = 0.f;
+#pragma unroll 8
         for (int d4 = 0; d4 < hd / 4; d4++) {
             const float4 vv = vr[d4];
             dot += dos[4 * d4] * vv.x + dos[4 * d4 + 1] * vv.y + dos[4 * d4 + 2] * vv.z + dos[4 * d4 + 3] * vv.w;
@@ -235,33 +329,49 @@ __global__ __launch_bounds__(64) void k_attn_bwd_dq(AttnBwdArgs a)
     __syncthreads();
     for (int d = lane; d < hd; d += 64) {
         float acc = 0.f;
+#pragma unroll 8
         for (int j = 0; j <= i; j++) acc += dr[j] * a.k[(r0 + j) * kd + hk * hd + d];
         a.dq[(r0 + i) * qd + h * hd + d] = acc;
     }
 }
 
-// attn_bwd_dkv + repeat_kv_bwd, shaders/q8_kernels.metal:931-992: one wave per
-// (kv head, key, sequence) sums over the query heads of its group.
-__global__ __launch_bounds__(64) void k_attn_bwd_dkv(AttnBwdArgs a)
+// attn_bwd_dkv + repeat_kv_bwd, shaders/q8_kernels.metal:931-992: one workgroup per
+// (kv head, key, sequence); the four waves split the queries i >= j between them (the sum
+// also runs over the query heads of the group) and add their partial rows through LDS.
+__global__ __launch_bounds__(TB) void k_attn_bwd_dkv(AttnBwdArgs a)
 {
+    extern __shared__ float part[];                      // [4 waves][2][hd]
     const int N = a.seq, hd = a.hd, ratio = a.Hq / a.Hkv;
-    const int hk = blockIdx.x, j = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int hk = blockIdx.x, j = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int qd = a.Hq * hd, kd = a.Hkv * hd;
     const size_t r0 = (size_t)b * N;
-    for (int d = lane; d < hd; d += 64) {
+    for (int d0 = 0; d0 < hd; d0 += 64) {
+        const int d = d0 + lane;
         float dk = 0.f, dv = 0.f;
-        for (int g = 0; g < ratio; g++) {
-            const int h = hk * ratio + g;
-            const size_t pbase = ((size_t)b * a.Hq + h) * N * N;
-            for (int i = j; i < N; i++) {
-                const float ds = a.dscore[pbase + (size_t)i * N + j];
-                const float p = a.probs[pbase + (size_t)i * N + j];
-                dk += ds * a.q[(r0 + i) * qd + h * hd + d];
-                dv += p * a.dO_red[(r0 + i) * qd + h * hd + d];
+        if (d < hd) {
+            for (int g = 0; g < ratio; g++) {
+                const int h = hk * ratio + g;
+                const float *dsp = a.dscore + ((size_t)b * a.Hq + h) * N * N + j;
+                const float *pp = a.probs + ((size_t)b * a.Hq + h) * N * N + j;
+                const float *qp = a.q + r0 * qd + h * hd + d;
+                const float *dop = a.dO_red + r0 * qd + h * hd + d;
+#pragma unroll 4
+                for (int i = j + wave; i < N; i += 4) {
+                    dk += dsp[(size_t)i * N] * qp[(size_t)i * qd];
+                    dv += pp[(size_t)i * N] * dop[(size_t)i * qd];
+                }
             }
+            part[(wave * 2 + 0) * hd + d] = dk;
+            part[(wave * 2 + 1) * hd + d] = dv;
         }
-        a.dk[(r0 + j) * kd + hk * hd + d] = dk;
-        a.dv[(r0 + j) * kd + hk * hd + d] = dv;
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < 2 * hd; d += TB) {
+        const int which = d / hd, dd = d % hd;
+        const float s = part[(0 * 2 + which) * hd + dd] + part[(1 * 2 + which) * hd + dd]
+                      + part[(2 * 2 + which) * hd + dd] + part[(3 * 2 + which) * hd + dd];
+        (which ? a.dv : a.dk)[(r0 + j) * kd + hk * hd + dd] = s;
     }
 }
 
@@ -272,15 +382,17 @@ __global__ __launch_bounds__(64) void k_attn_bwd_dkv(AttnBwdArgs a)
 // row [dq | dk | dv | dh_q | dh_v] as one scaled fp16 operand so that a single GEMM
 // against [Wq; Wk; Wv; A_q; A_v]^T yields dq Wq + dk Wk + dv Wv + dh_q A_q + dh_v A_v
 // (src/nn/fast_sft.c:953-971).
-__global__ __launch_bounds__(TB) void k_qkv_bwd_rows(QkvBwdArgs a)
+__global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
 {
-    extern __shared__ float buf[];                       // [qd + 2kd + 2R]
+    extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [16 waves][32] partials
     __shared__ float sm[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t row = blockIdx.x;
-    const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd;
+    const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd, R = a.R;
+    const int n = qd + 2 * kd + 2 * R;
+    float *dhp = buf + n;
     const int pos = (int)(row % a.seq);
-    for (int slot = wave; slot < a.Hq + a.Hkv; slot += 4) {
+    for (int slot = wave; slot < a.Hq + a.Hkv; slot += RB / 64) {
         const int isk = slot >= a.Hq, h = isk ? slot - a.Hq : slot;
         const int W = isk ? kd : qd;
         const float *gin = (isk ? a.dk : a.dq) + row * W + h * hd;
@@ -294,11 +406,9 @@ __global__ __launch_bounds__(TB) void k_qkv_bwd_rows(QkvBwdArgs a)
             y0[p] = y1[p] = p0[p] = p1[p] = 0.f;
             if (d < half) {
                 const float g0 = gin[d], g1 = gin[d + half];
-                const float freq = 1.0f / powf(a.theta, (float)(2 * d) / (float)hd);
-                float s, c;
-                sincosf((float)pos * freq, &s, &c);
-                y0[p] = g0 * c + g1 * s;
-                y1[p] = -g0 * s + g1 * c;
+                const float2 cs = a.rope[(size_t)pos * half + d];
+                y0[p] = g0 * cs.x + g1 * cs.y;
+                y1[p] = -g0 * cs.y + g1 * cs.x;
                 p0[p] = xp[d];
                 p1[p] = xp[d + half];
                 ss += p0[p] * p0[p] + p1[p] * p1[p];
@@ -321,26 +431,45 @@ __global__ __launch_bounds__(TB) void k_qkv_bwd_rows(QkvBwdArgs a)
             if (!isk) { a.dq_f[row * qd + h * hd + d] = d0; a.dq_f[row * qd + h * hd + d + half] = d1; }
         }
     }
-    for (int c = threadIdx.x; c < kd; c += TB) buf[qd + kd + c] = a.dv[row * kd + c];
+    for (int c = threadIdx.x; c < kd; c += RB) buf[qd + kd + c] = a.dv[row * kd + c];
     __syncthreads();
-    const int R = a.R;
-    for (int r = wave; r < 2 * R; r += 4) {
-        const int isv = r >= R, rr = isv ? r - R : r;
-        const float *src = buf + (isv ? qd + kd : 0);
-        const float *B = isv ? a.Bv : a.Bq;
-        const int width = isv ? kd : qd;
-        float acc = 0.f;
-        for (int c = lane; c < width; c += 64) acc += src[c] * B[(size_t)c * R + rr];
-        acc = wave_sum(acc) * a.sc;
-        if (lane == 0) { buf[qd + 2 * kd + r] = acc; a.dh[row * 2 * R + r] = acc; }
+    // dh[r] = sc * sum_c d[c] * B[c][r]: a thread walks whole rows of B (R contiguous floats)
+    if (R > 0) {
+        float acc[32];
+#pragma unroll
+        for (int r = 0; r < 32; r++) acc[r] = 0.f;
+        for (int c = threadIdx.x; c < qd + kd; c += RB) {
+            const int isv = c >= qd;
+            const float x = buf[isv ? c + kd : c];
+            const float *Br = isv ? a.Bv + (size_t)(c - qd) * R : a.Bq + (size_t)c * R;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float bv = (r < R) ? Br[r] : 0.f;
+                if (isv) acc[16 + r] += x * bv; else acc[r] += x * bv;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 32; r++) acc[r] = wave_sum(acc[r]);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < 32; r++) dhp[wave * 32 + r] = acc[r];
+        }
+        __syncthreads();
+        if (threadIdx.x < 2 * R) {
+            const int isv = threadIdx.x >= R, rr = isv ? threadIdx.x - R : threadIdx.x;
+            float s = 0.f;
+            for (int w = 0; w < RB / 64; w++) s += dhp[w * 32 + (isv ? 16 : 0) + rr];
+            s *= a.sc;
+            buf[qd + 2 * kd + threadIdx.x] = s;
+            a.dh[row * 2 * R + threadIdx.x] = s;
+        }
+        __syncthreads();
     }
-    __syncthreads();
-    const int n = qd + 2 * kd + 2 * R;
     float amax = 0.f;
-    for (int c = threadIdx.x; c < n; c += TB) amax = fmaxf(amax, fabsf(buf[c]));
+    for (int c = threadIdx.x; c < n; c += RB) amax = fmaxf(amax, fabsf(buf[c]));
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
-    write_f16_row(buf, n, a.out16 + row * a.ld16, a.ld16, s);
+    write_f16_tiled(buf, n, a.out16, row, s);
     if (threadIdx.x == 0) a.inv_scale[row] = 1.0f / s;
 }
 
@@ -365,13 +494,16 @@ __global__ __launch_bounds__(TB) void k_lora_grads(LoraGradArgs a)
         if (which == 0 || which == 2) {
             const int r = (int)(o / a.D), d = (int)(o % a.D);
             const int hc = (which == 2 ? a.R : 0) + r;
+            const int Kb = tiled_kb(a.D);
+#pragma unroll 8
             for (int i = 0; i < a.rows; i++)
-                s += a.dh[(size_t)i * 2 * a.R + hc] * (h2f(a.ln16[(size_t)i * a.ld16 + d]) * a.ln_inv_scale[i]);
+                s += a.dh[(size_t)i * 2 * a.R + hc] * (h2f(a.ln16[tiled_index(i, d, Kb)]) * a.ln_inv_scale[i]);
         } else {
             const int c = (int)(o / a.R), r = (int)(o % a.R);
             const float *dy = which == 1 ? a.dq_f : a.dv_f;
             const float *t = which == 1 ? a.tq : a.tv;
             const int W = which == 1 ? a.qd : a.kd;
+#pragma unroll 8
             for (int i = 0; i < a.rows; i++) s += dy[(size_t)i * W + c] * t[(size_t)i * a.R + r];
             s *= a.sc;
         }
@@ -394,27 +526,33 @@ __device__ __forceinline__ float act_fwd(float g, int gelu)
 }
 
 // silu_mul / gelu_mul, shaders/q8_kernels.metal:337-362, with the gate/up saves of
-// src/nn/fast_sft.c:715-718.  Two passes over the row: amax, then the scaled write.
-__global__ __launch_bounds__(TB) void k_glu_fwd(GluArgs a)
+// src/nn/fast_sft.c:715-718.
+__global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
 {
     __shared__ float sm[16];
     const size_t r = blockIdx.x;
-    const int IS = a.IS;
+    const int IS = a.IS, nv = IS >> 2;
+    float4 act[MAXV];
     float amax = 0.f;
-    for (int i = threadIdx.x; i < IS; i += TB) {
-        const float g = planes_at(a.in, r, i), u = planes_at(a.in, r, IS + i);
-        a.gate_pre[r * IS + i] = g;
-        a.up_val[r * IS + i] = u;
-        amax = fmaxf(amax, fabsf(act_fwd(g, a.gelu) * u));
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        act[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) {
+            const float4 g = planes_at4(a.in, r, 4 * v), u = planes_at4(a.in, r, IS + 4 * v);
+            st4(a.gate_pre + r * IS + 4 * v, g);
+            st4(a.up_val + r * IS + 4 * v, u);
+            act[t] = make_float4(act_fwd(g.x, a.gelu) * u.x, act_fwd(g.y, a.gelu) * u.y,
+                                 act_fwd(g.z, a.gelu) * u.z, act_fwd(g.w, a.gelu) * u.w);
+            amax = fmaxf(amax, amax4(act[t]));
+        }
     }
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
-    half_t *o = a.out16 + r * a.ld16;
-    for (int i = threadIdx.x; i < a.ld16; i += TB) {
-        half_t hv = (half_t)0;
-        if (i < IS) hv = f2h(act_fwd(a.gate_pre[r * IS + i], a.gelu) * a.up_val[r * IS + i] * s);
-        o[i] = hv;
-    }
+    const int Kb = tiled_kb(IS);
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st_tiled4(a.out16, r, 4 * v, Kb, act[t], s); }
+    zero_tiled_pad(a.out16, r, IS, Kb);
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
 
@@ -432,27 +570,35 @@ __device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, fl
     }
 }
 
-__global__ __launch_bounds__(TB) void k_glu_bwd(GluArgs a)
+__global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
 {
     __shared__ float sm[16];
     const size_t r = blockIdx.x;
-    const int IS = a.IS;
+    const int IS = a.IS, nv = IS >> 2;
+    float4 dg[MAXV], du[MAXV];
     float amax = 0.f;
-    for (int i = threadIdx.x; i < IS; i += TB) {
-        float dg, du;
-        act_bwd(planes_at(a.in, r, i), a.gate_pre[r * IS + i], a.up_val[r * IS + i], a.gelu, dg, du);
-        amax = fmaxf(amax, fmaxf(fabsf(dg), fabsf(du)));
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        dg[t] = du[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) {
+            const float4 dy = planes_at4(a.in, r, 4 * v), g = ld4(a.gate_pre + r * IS + 4 * v), u = ld4(a.up_val + r * IS + 4 * v);
+            act_bwd(dy.x, g.x, u.x, a.gelu, dg[t].x, du[t].x);
+            act_bwd(dy.y, g.y, u.y, a.gelu, dg[t].y, du[t].y);
+            act_bwd(dy.z, g.z, u.z, a.gelu, dg[t].z, du[t].z);
+            act_bwd(dy.w, g.w, u.w, a.gelu, dg[t].w, du[t].w);
+            amax = fmaxf(amax, fmaxf(amax4(dg[t]), amax4(du[t])));
+        }
     }
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
-    half_t *o = a.out16 + r * a.ld16;
-    for (int i = threadIdx.x; i < IS; i += TB) {
-        float dg, du;
-        act_bwd(planes_at(a.in, r, i), a.gate_pre[r * IS + i], a.up_val[r * IS + i], a.gelu, dg, du);
-        o[i] = f2h(dg * s);
-        o[IS + i] = f2h(du * s);
+    const int Kb = tiled_kb(2 * IS);
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        if (v < nv) { st_tiled4(a.out16, r, 4 * v, Kb, dg[t], s); st_tiled4(a.out16, r, IS + 4 * v, Kb, du[t], s); }
     }
-    for (int i = 2 * IS + threadIdx.x; i < a.ld16; i += TB) o[i] = (half_t)0;
+    zero_tiled_pad(a.out16, r, 2 * IS, Kb);
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
 
@@ -462,55 +608,77 @@ __global__ __launch_bounds__(TB) void k_glu_bwd(GluArgs a)
 // src/nn/fast_sft.c:870-874, 975-980).  The operand of the next dX GEMM is dx_out
 // itself (Qwen3) or RNB(branch_raw, dx_out; g_branch) (Gemma3's post-norms,
 // src/nn/fast_sft.c:798-802, 877-881).
-__global__ __launch_bounds__(TB) void k_norm_bwd_rows(NormBwdArgs a)
+__global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
-    extern __shared__ float lds[];
-    float *dyb = lds, *dxn = lds + a.D;
     __shared__ float sm[16];
     const size_t r = blockIdx.x;
-    const int D = a.D;
+    const int D = a.D, nv = D >> 2;
+    float4 dy[MAXV], x[MAXV], g[MAXV];
     float ss = 0.f, dot = 0.f;
-    for (int i = threadIdx.x; i < D; i += TB) {
-        const float dy = planes_at(a.dy, r, i), x = a.x_saved[r * D + i];
-        dyb[i] = dy;
-        ss += x * x;
-        dot += dy * a.g[i] * x;
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        dy[t] = x[t] = g[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) {
+            dy[t] = planes_at4(a.dy, r, 4 * v);
+            x[t] = ld4(a.x_saved + r * D + 4 * v);
+            g[t] = ld4(a.g + 4 * v);
+            ss += sumsq4(x[t]);
+            dot += dy[t].x * g[t].x * x[t].x + dy[t].y * g[t].y * x[t].y + dy[t].z * g[t].z * x[t].z + dy[t].w * g[t].w * x[t].w;
+        }
     }
     ss = block_sum(ss, sm);
     dot = block_sum(dot, sm);
     const float inv = rsqrtf(ss / (float)D + a.eps);
     const float coeff = dot * inv * inv / (float)D;
-    for (int i = threadIdx.x; i < D; i += TB) {
-        float t = (a.g[i] * dyb[i] - coeff * a.x_saved[r * D + i]) * inv;
-        if (a.dx_prev) t += a.dx_prev[r * D + i];
-        if (a.clamp > 0.f) t = fminf(fmaxf(t, -a.clamp), a.clamp);
-        a.dx_out[r * D + i] = t;
-        dxn[i] = t;
+    float4 dx[MAXV];
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        const int v = threadIdx.x + t * RB;
+        dx[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v >= nv) continue;
+        dx[t] = make_float4((g[t].x * dy[t].x - coeff * x[t].x) * inv, (g[t].y * dy[t].y - coeff * x[t].y) * inv,
+                            (g[t].z * dy[t].z - coeff * x[t].z) * inv, (g[t].w * dy[t].w - coeff * x[t].w) * inv);
+        if (a.dx_prev) { const float4 p = ld4(a.dx_prev + r * D + 4 * v); dx[t].x += p.x; dx[t].y += p.y; dx[t].z += p.z; dx[t].w += p.w; }
+        if (a.clamp > 0.f) {
+            dx[t].x = fminf(fmaxf(dx[t].x, -a.clamp), a.clamp); dx[t].y = fminf(fmaxf(dx[t].y, -a.clamp), a.clamp);
+            dx[t].z = fminf(fmaxf(dx[t].z, -a.clamp), a.clamp); dx[t].w = fminf(fmaxf(dx[t].w, -a.clamp), a.clamp);
+        }
+        st4(a.dx_out + r * D + 4 * v, dx[t]);
     }
     if (!a.d16) return;
     float amax = 0.f;
     if (a.branch_raw) {
         float ssb = 0.f, dotb = 0.f;
-        for (int i = threadIdx.x; i < D; i += TB) {
-            const float xb = a.branch_raw[r * D + i];
-            ssb += xb * xb;
-            dotb += dxn[i] * a.g_branch[i] * xb;
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const int v = threadIdx.x + t * RB;
+            if (v >= nv) continue;
+            x[t] = ld4(a.branch_raw + r * D + 4 * v);
+            g[t] = ld4(a.g_branch + 4 * v);
+            ssb += sumsq4(x[t]);
+            dotb += dx[t].x * g[t].x * x[t].x + dx[t].y * g[t].y * x[t].y + dx[t].z * g[t].z * x[t].z + dx[t].w * g[t].w * x[t].w;
         }
         ssb = block_sum(ssb, sm);
         dotb = block_sum(dotb, sm);
         const float invb = rsqrtf(ssb / (float)D + a.eps);
         const float cb = dotb * invb * invb / (float)D;
-        for (int i = threadIdx.x; i < D; i += TB) {
-            const float v = (a.g_branch[i] * dxn[i] - cb * a.branch_raw[r * D + i]) * invb;
-            dyb[i] = v;
-            amax = fmaxf(amax, fabsf(v));
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const int v = threadIdx.x + t * RB;
+            if (v >= nv) continue;
+            dx[t] = make_float4((g[t].x * dx[t].x - cb * x[t].x) * invb, (g[t].y * dx[t].y - cb * x[t].y) * invb,
+                                (g[t].z * dx[t].z - cb * x[t].z) * invb, (g[t].w * dx[t].w - cb * x[t].w) * invb);
         }
-    } else {
-        for (int i = threadIdx.x; i < D; i += TB) { dyb[i] = dxn[i]; amax = fmaxf(amax, fabsf(dxn[i])); }
     }
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) amax = fmaxf(amax, amax4(dx[t]));
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
-    write_f16_row(dyb, D, a.d16 + r * a.ld16, a.ld16, s);
+    const int Kb = tiled_kb(D);
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st_tiled4(a.d16, r, 4 * v, Kb, dx[t], s); }
+    zero_tiled_pad(a.d16, r, D, Kb);
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
 
@@ -525,22 +693,30 @@ __global__ __launch_bounds__(1024) void k_ce_rows(CeArgs a)
     const int V = a.V;
     const float *lg = a.logits + r * V;
     const uint32_t tgt = a.targets[r];
+    const int nv = V >> 2;                                // V % 4 == 0 is checked by the launcher
     float mx = -1e30f;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, lg[i]);
+    for (int v = threadIdx.x; v < nv; v += blockDim.x) { const float4 x = ld4(lg + 4 * v); mx = fmaxf(mx, fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w))); }
     mx = block_max(mx, sm);
     float sum = 0.f;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) sum += expf(lg[i] - mx);
+    for (int v = threadIdx.x; v < nv; v += blockDim.x) {
+        const float4 x = ld4(lg + 4 * v);
+        sum += expf(x.x - mx) + expf(x.y - mx) + expf(x.z - mx) + expf(x.w - mx);
+    }
     sum = block_sum(sum, sm);
     const float lse = logf(sum) + mx;
     if (threadIdx.x == 0) {
         a.losses[r] = lse - lg[tgt];
         a.inv_scale[r] = (1.0f / (float)a.rows_total) * (1.0f / 1024.0f);
     }
-    half_t *o = a.dl16 + r * a.ld16;
-    for (int i = threadIdx.x; i < a.ld16; i += blockDim.x) {
-        half_t hv = (half_t)0;
-        if (i < V) hv = f2h((expf(lg[i] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f);
-        o[i] = hv;
+    const int Kb = tiled_kb(V);
+    for (int c = threadIdx.x; c < Kb * 8; c += blockDim.x) {
+        half8 hv;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int i = c * 8 + e;
+            hv[e] = (i < V) ? f2h((expf(lg[i] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
+        }
+        *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
     }
 }
 
@@ -577,8 +753,8 @@ __device__ __forceinline__ void shadow_store(const AdamArgs &a, size_t idx, floa
     const int r = (int)(o / a.D), d = (int)(o % a.D);
     const int rowx = a.qd + 2 * a.kd + rbase + r;
     const half_t hv = f2h(pv);
-    a.wqkv[L * a.wqkv_layer_stride + (size_t)rowx * a.D + d] = hv;
-    a.wqkvT[L * a.wqkvT_layer_stride + (size_t)d * a.ldT + rowx] = hv;
+    a.wqkv[L * a.wqkv_layer_stride + tiled_index(rowx, d, tiled_kb(a.D))] = hv;
+    a.wqkvT[L * a.wqkvT_layer_stride + tiled_index(d, rowx, tiled_kb(a.qd + 2 * a.kd + 2 * a.R))] = hv;
 }
 
 __global__ __launch_bounds__(TB) void k_adamw(AdamArgs a)
@@ -626,8 +802,15 @@ void require(bool ok, const char *what)
 
 void launch_norm_rows(const NormRowsArgs &a, int rows)
 {
-    require(a.D > 0 && (size_t)a.D * 8 <= 64 * 1024, "norm_rows: hidden size must be <= 8192");
-    LAUNCH(k_norm_rows, dim3(rows), dim3(TB), (size_t)a.D * 8, a);
+    require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV, "norm_rows: hidden size must be a multiple of 4, <= 12288");
+    require(a.branch.S == 0 || a.branch.ld % 4 == 0, "norm_rows: plane row length must be a multiple of 4");
+    LAUNCH(k_norm_rows, dim3(rows), dim3(RB), 0, a);
+}
+
+void launch_rope_table(float2 *tab, int seq, int hd, float theta)
+{
+    const int n = seq * (hd / 2);
+    LAUNCH(k_rope_table, dim3((n + 255) / 256), dim3(256), 0, tab, seq, hd / 2, hd, theta);
 }
 
 void launch_qkv_post(const QkvPostArgs &a, int rows)
@@ -649,14 +832,14 @@ void launch_attn_bwd(const AttnBwdArgs &a)
 {
     require(a.hd % 4 == 0 && a.seq <= 4096, "attn_bwd: head_dim % 4, seq <= 4096");
     LAUNCH(k_attn_bwd_dq, dim3(a.Hq, a.seq, a.batch), dim3(64), (size_t)(a.seq + a.hd) * 4, a);
-    LAUNCH(k_attn_bwd_dkv, dim3(a.Hkv, a.seq, a.batch), dim3(64), 0, a);
+    LAUNCH(k_attn_bwd_dkv, dim3(a.Hkv, a.seq, a.batch), dim3(TB), (size_t)8 * a.hd * 4, a);
 }
 
 void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
 {
-    const size_t n = (size_t)(a.Hq + 2 * a.Hkv) * a.hd + 2 * a.R;
-    require(a.hd <= 2 * 64 * MAXP && n * 4 <= 64 * 1024, "qkv_bwd: row of dq|dk|dv must fit 64 KB of LDS");
-    LAUNCH(k_qkv_bwd_rows, dim3(rows), dim3(TB), n * 4, a);
+    const size_t n = (size_t)(a.Hq + 2 * a.Hkv) * a.hd + 2 * a.R + 16 * 32;
+    require(a.hd <= 2 * 64 * MAXP && n * 4 <= 64 * 1024 && a.R <= 16, "qkv_bwd: row of dq|dk|dv must fit 64 KB of LDS, rank <= 16");
+    LAUNCH(k_qkv_bwd_rows, dim3(rows), dim3(RB), n * 4, a);
 }
 
 int lora_grad_blocks(int D, int qd, int kd, int R)
@@ -670,16 +853,28 @@ void launch_lora_grads(const LoraGradArgs &a)
     LAUNCH(k_lora_grads, dim3(lora_grad_blocks(a.D, a.qd, a.kd, a.R)), dim3(TB), 0, a);
 }
 
-void launch_glu_fwd(const GluArgs &a, int rows) { LAUNCH(k_glu_fwd, dim3(rows), dim3(TB), 0, a); }
-void launch_glu_bwd(const GluArgs &a, int rows) { LAUNCH(k_glu_bwd, dim3(rows), dim3(TB), 0, a); }
+void launch_glu_fwd(const GluArgs &a, int rows)
+{
+    require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_fwd: FFN width must be a multiple of 4, <= 12288");
+    LAUNCH(k_glu_fwd, dim3(rows), dim3(RB), 0, a);
+}
+void launch_glu_bwd(const GluArgs &a, int rows)
+{
+    require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_bwd: FFN width must be a multiple of 4, <= 12288");
+    LAUNCH(k_glu_bwd, dim3(rows), dim3(RB), 0, a);
+}
 
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
 {
-    require(a.D > 0 && (size_t)a.D * 8 <= 64 * 1024, "norm_bwd_rows: hidden size must be <= 8192");
-    LAUNCH(k_norm_bwd_rows, dim3(rows), dim3(TB), (size_t)a.D * 8, a);
+    require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV && a.dy.ld % 4 == 0, "norm_bwd_rows: hidden size must be a multiple of 4, <= 12288");
+    LAUNCH(k_norm_bwd_rows, dim3(rows), dim3(RB), 0, a);
 }
 
-void launch_ce_rows(const CeArgs &a, int rows) { LAUNCH(k_ce_rows, dim3(rows), dim3(a.V >= 4096 ? 1024 : 256), 0, a); }
+void launch_ce_rows(const CeArgs &a, int rows)
+{
+    require(a.V % 4 == 0, "ce_rows: vocabulary size must be a multiple of 4");
+    LAUNCH(k_ce_rows, dim3(rows), dim3(a.V >= 4096 ? 1024 : 256), 0, a);
+}
 
 void launch_adamw(const AdamArgs &a)
 {
@@ -691,12 +886,12 @@ void launch_adamw(const AdamArgs &a)
 }
 
 void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
-                        size_t wqkvT_layer_stride, int ldT, int D, int qd, int kd, int R, size_t layer_size)
+                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size)
 {
     if (!n) return;
     AdamArgs a{};
     a.p = const_cast<float *>(p); a.n = n; a.wqkv = wqkv; a.wqkv_layer_stride = wqkv_layer_stride;
-    a.wqkvT = wqkvT; a.wqkvT_layer_stride = wqkvT_layer_stride; a.ldT = ldT;
+    a.wqkvT = wqkvT; a.wqkvT_layer_stride = wqkvT_layer_stride;
     a.D = D; a.qd = qd; a.kd = kd; a.R = R; a.layer_size = layer_size;
     size_t blocks = (n + TB - 1) / TB;
     if (blocks > 4096) blocks = 4096;

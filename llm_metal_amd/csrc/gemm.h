@@ -1,28 +1,51 @@
-// Internal interface of the weight-streaming GEMM (gemm.hip).
+// Internal interface of the weight-streaming GEMM (gemm.hip) and of the tiled
+// fp16 operand layout it reads.
 #pragma once
 #include "backend.h"
 #include "devutil.h"
 
 namespace lmhip {
 
+// ---- tiled fp16 operand layout ------------------------------------------------
+// A matrix [R, K] is cut into tiles of 32 rows x 64 columns (4 KB).  Inside a
+// tile the order is [j = 0..3][lane = 0..63][e = 0..7] with
+//     row = lane & 31,   col = (lane >> 5) * 32 + 8 * j + e,
+// i.e. exactly the registers lane `lane` feeds to the j-th v_mfma_f32_32x32x16_f16
+// of a 64-wide K step (the K order inside a step is permuted the same way for
+// both operands, which a dot product does not see).  Tiles are stored
+// [row block][K block].  One wave-wide 16-byte load therefore reads 1 KB of
+// contiguous memory.  R is padded to 32 and K to 64; padding must hold zeros
+// in K (rows beyond R may hold anything: their outputs are never stored).
+__host__ __device__ inline int tiled_kb(int K) { return (K + 63) >> 6; }
+__host__ __device__ inline int tiled_rb(int R) { return (R + 31) >> 5; }
+__host__ __device__ inline size_t tiled_elems(int R, int K) { return (size_t)tiled_rb(R) * tiled_kb(K) * 2048; }
+__host__ __device__ inline size_t tiled_index(int r, int k, int Kb)
+{
+    const int c = k & 63;
+    const size_t tile = (size_t)(r >> 5) * Kb + (k >> 6);
+    return ((tile * 4 + ((c & 31) >> 3)) * 64 + ((c >> 5) << 5) + (r & 31)) * 8 + (c & 7);
+}
+
 struct GemmPlan {
     int nb;        // 32-row weight blocks per wave (1 or 2)
     int S;         // K chunks = partial planes written
-    int k_chunk;   // elements of K per chunk (multiple of 256)
+    int steps;     // 64-wide K steps per chunk
     int n_tiles, m_tiles;
 };
 
 GemmPlan plan_gemm(int M, int N, int K);
 
 // P[s][m][n] (s < plan.S, plane s at P + s*plane_stride, row stride ldp) =
-//   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k]
-void launch_gemm(const half_t *A, int lda, const float *a_inv_scale, const half_t *W, int ldw,
+//   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k],  A and W in the tiled layout
+void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const half_t *W_tiled,
                  float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p);
 
-// out[m][0..ldo) = fp16(X[m][k] * s_m) (zero beyond K), inv_scale[m] = 1/s_m
-void launch_rows_to_f16(const float *X, int ldx, half_t *out, int ldo, float *inv_scale, int M, int K);
+// out (tiled [M, K]) = fp16(X[m][k] * s_m), zero in the K padding; inv_scale[m] = 1/s_m
+void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_scale, int M, int K);
 void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, float *C, int M, int N);
-void launch_transpose_f16(const half_t *src, half_t *dst, int rows, int cols, int ld_dst);
-void gemm_f32a(const float *A, const half_t *W, int ldw, float *C, int M, int N, int K);
+// dst (tiled, Kb_dst K blocks) <- src row-major F16 [rows, cols]:
+//   element (r, c) goes to tiled(row_off + r, k_off + c), or tiled(row_off + c, k_off + r) when transposed
+void launch_tile_f16(const half_t *src, int rows, int cols, half_t *dst_tiled, int Kb_dst,
+                     int row_off, int k_off, int transpose);
 
 }  // namespace lmhip

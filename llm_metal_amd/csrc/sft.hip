@@ -23,13 +23,17 @@ using namespace lmhip;
 
 struct SFTState {
     int D, Hq, Hkv, hd, IS, V, NL, N, B, BN;
-    int qd, kd, R, nq_ext, ldq;          // nq_ext = qd + 2kd + 2R rows of the fused QKV weight; ldq its padded length as a K
+    int qd, kd, R, nq_ext;               // nq_ext = qd + 2kd + 2R rows of the fused QKV weight
+    size_t st_qkv, st_qkvT, st_o, st_oT, st_gu, st_guT, st_d, st_dT, st_ln1;   // layer strides (elements) of the tiled weight arenas
     float eps, lora_scaling, emb_scale;
     ModelType model_type;
     int step_count, weight_format;
     std::vector<float> rope_thetas;
+    MetalBuf *rope_tabs;                 // one (cos, sin) table [seq][hd/2] per distinct theta
+    std::vector<int> rope_slot;          // layer -> table index
 
-    // frozen weights, F16, one arena per matrix kind with a fixed layer stride
+    // frozen weights, F16 in the GEMM's tiled layout, one arena per matrix kind with a fixed layer stride;
+    // the ...T arenas hold the transposed matrices for the dX products
     MetalBuf *wqkv, *wqkvT, *wo, *woT, *wgu, *wguT, *wd, *wdT, *wlm, *wlmT;
     MetalBuf *q8_blocks;                 // Q8_0 mode: the quantised bytes of every matrix, in upload order
     MetalBuf *g_in, *g_post_attn, *g_pre_ff, *g_post_ff, *g_q, *g_k, *g_final;
@@ -62,28 +66,31 @@ struct SFTState {
 
 namespace {
 
-inline int round8(int x) { return (x + 7) & ~7; }
 inline MetalBuf *fbuf(size_t n) { return metal_buf_create(n * sizeof(float)); }
 inline MetalBuf *hbuf(size_t n) { return metal_buf_create(n * sizeof(half_t)); }
 template <typename T> inline T *at(MetalBuf *b, size_t elem_off = 0) { return dptr_as<T>(b) + elem_off; }
 
-// Upload one fp32 matrix and store it as F16 rows [row0, row0+rows) of a row-major arena slice
-// whose row length is `cols`.  Q8_0 mode quantises first and stores the dequantised values.
-void put_matrix(SFTState *s, MetalBuf *arena, size_t elem_off, const float *src, int rows, int cols,
-                std::vector<MetalBuf *> &q8_keep)
+struct Dest { MetalBuf *arena; size_t elem_off; int Kb; int row_off, k_off, transpose; };
+
+// Upload one fp32 matrix [rows, cols], round it to F16 (Q8_0 mode: quantise, then take the
+// dequantised values) and scatter it into tiled weight arenas: `a` as is, `b` transposed.
+void put_matrix(SFTState *s, const float *src, int rows, int cols, const Dest &a, const Dest &b)
 {
     const size_t n = (size_t)rows * cols;
     MetalBuf *stage = metal_buf_from_data(src, n * sizeof(float));
-    MetalBuf *dst = metal_buf_view(arena, elem_off * sizeof(half_t), n * sizeof(half_t));
+    MetalBuf *rm = metal_buf_create(n * sizeof(half_t));
+    MetalBuf *q8 = nullptr;
     if (s->weight_format) {
-        hip_enqueue_f32_to_f16(stage, dst, n);
+        hip_enqueue_f32_to_f16(stage, rm, n);
     } else {
-        MetalBuf *q8 = metal_buf_create((size_t)rows * (cols / 32) * 34);
+        q8 = metal_buf_create((size_t)rows * (cols / 32) * 34);
         hip_enqueue_q8_quantize(stage, q8, rows, cols);
-        hip_enqueue_q8_to_f16(q8, dst, rows, cols);
-        q8_keep.push_back(q8);
+        hip_enqueue_q8_to_f16(q8, rm, rows, cols);
     }
-    metal_buf_free(dst);
+    for (const Dest *d : {&a, &b})
+        launch_tile_f16(at<half_t>(rm), rows, cols, at<half_t>(d->arena, d->elem_off), d->Kb, d->row_off, d->k_off, d->transpose);
+    metal_buf_free(rm);                                   // synchronises the stream first
+    metal_buf_free(q8);
     metal_buf_free(stage);
 }
 
@@ -91,7 +98,7 @@ size_t max_planes_elems(SFTState *s)
 {
     struct Sh { int N, K; };
     const Sh shapes[] = {{s->nq_ext, s->D}, {s->D, s->qd}, {2 * s->IS, s->D}, {s->D, s->IS}, {s->V, s->D},
-                         {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->ldq}};
+                         {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->nq_ext}};
     size_t mx = 0;
     for (const Sh &sh : shapes) {
         GemmPlan p = plan_gemm(s->BN, sh.N, sh.K);
@@ -101,16 +108,15 @@ size_t max_planes_elems(SFTState *s)
     return mx;
 }
 
-// P = A16 * W^T as K-split planes in the state's plane buffer
-Planes gemm(SFTState *s, const half_t *A, int lda, const float *inv, const half_t *W, int ldw, int N, int K,
-            float *out = nullptr)
+// P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
+Planes gemm(SFTState *s, const half_t *A, const float *inv, const half_t *W, int N, int K, float *out = nullptr)
 {
     GemmPlan p = plan_gemm(s->BN, N, K);
     float *P = out ? out : at<float>(s->planes);
     const size_t stride = (size_t)s->BN * N;
     if (!out && (size_t)p.S * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
     if (out && p.S != 1) { fprintf(stderr, "[fast_sft] direct GEMM output needs S == 1\n"); abort(); }
-    launch_gemm(A, lda, inv, W, ldw, P, N, stride, s->BN, N, K, p);
+    launch_gemm(A, inv, W, P, N, stride, s->BN, N, K, p);
     return Planes{P, p.S, stride, N};
 }
 
@@ -125,7 +131,7 @@ void forward_impl(SFTState *s, bool gather)
 
     for (int L = 0; L < s->NL; L++) {
         float *x_in = at<float>(s->xs, (size_t)(2 * L) * xsz), *x_mid = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
-        half_t *ln1 = at<half_t>(s->ln1_16, (size_t)L * xsz);
+        half_t *ln1 = at<half_t>(s->ln1_16, (size_t)L * s->st_ln1);
         float *ln1inv = at<float>(s->ln1_inv, (size_t)L * BN);
 
         // x_in = x (+ previous FFN branch); ln1 = RN(x_in; g_in)        [src/nn/fast_sft.c:631-635, 732-740]
@@ -140,18 +146,18 @@ void forward_impl(SFTState *s, bool gather)
         }
         n1.x_out = x_in;
         n1.g_norm = at<float>(s->g_in, (size_t)L * D);
-        n1.ln16 = ln1; n1.ld16 = D; n1.inv_scale = ln1inv; n1.D = D; n1.eps = s->eps;
+        n1.ln16 = ln1; n1.inv_scale = ln1inv; n1.D = D; n1.eps = s->eps;
         launch_norm_rows(n1, BN);
 
         // [q | k | v | tq | tv] = ln1 [Wq; Wk; Wv; A_q; A_v]^T                 [:638-656]
-        Planes pq = gemm(s, ln1, D, ln1inv, at<half_t>(s->wqkv, (size_t)L * s->nq_ext * D), D, s->nq_ext, D);
+        Planes pq = gemm(s, ln1, ln1inv, at<half_t>(s->wqkv, L * s->st_qkv), s->nq_ext, D);
         QkvPostArgs qa{};
         qa.qkv = pq;
         qa.Bq = at<float>(s->lora, L * s->lsz + (size_t)R * D);
         qa.Bv = at<float>(s->lora, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
         qa.R = R; qa.sc = s->lora_scaling;
         qa.g_q = at<float>(s->g_q, (size_t)L * s->hd); qa.g_k = at<float>(s->g_k, (size_t)L * s->hd);
-        qa.eps = s->eps; qa.theta = s->rope_thetas[L];
+        qa.eps = s->eps; qa.rope = at<float2>(s->rope_tabs, (size_t)s->rope_slot[L] * s->N * (s->hd / 2));
         qa.Hq = s->Hq; qa.Hkv = s->Hkv; qa.hd = s->hd; qa.seq = s->N;
         qa.q_pre = at<float>(s->q_pre, (size_t)L * BN * qd); qa.k_pre = at<float>(s->k_pre, (size_t)L * BN * kd);
         qa.q_fin = at<float>(s->q_fin, (size_t)L * BN * qd); qa.k_fin = at<float>(s->k_fin, (size_t)L * BN * kd);
@@ -165,29 +171,29 @@ void forward_impl(SFTState *s, bool gather)
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
         aa.scale = 1.0f / sqrtf((float)s->hd);
         aa.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
-        aa.out16 = a16; aa.ld16 = qd;
+        aa.out16 = a16;
         launch_attn_fwd(aa);
 
         // o = attn Wo^T; x_mid = x_in + o (Qwen3) | x_in + RN(o; g_post_attn) (Gemma3); ln2 = RN(x_mid; g_ffn_in)   [:696-711]
-        Planes po = gemm(s, a16, qd, at<float>(s->ones), at<half_t>(s->wo, (size_t)L * D * qd), qd, D, qd);
+        Planes po = gemm(s, a16, at<float>(s->ones), at<half_t>(s->wo, L * s->st_o), D, qd);
         NormRowsArgs n2{};
         n2.x_prev = x_in; n2.branch = po;
         if (gemma) { n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); n2.branch_raw_out = at<float>(s->o_raw, (size_t)L * xsz); }
         n2.x_out = x_mid;
         n2.g_norm = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
-        n2.ln16 = a16; n2.ld16 = D; n2.inv_scale = ainv; n2.D = D; n2.eps = s->eps;
+        n2.ln16 = a16; n2.inv_scale = ainv; n2.D = D; n2.eps = s->eps;
         launch_norm_rows(n2, BN);
 
         // [gate | up] = ln2 [Wg; Wu]^T; act = silu|gelu(gate) * up              [:715-725]
-        Planes pg = gemm(s, a16, D, ainv, at<half_t>(s->wgu, (size_t)L * 2 * IS * D), D, 2 * IS, D);
+        Planes pg = gemm(s, a16, ainv, at<half_t>(s->wgu, L * s->st_gu), 2 * IS, D);
         GluArgs ga{};
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
         ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
-        ga.out16 = a16; ga.ld16 = IS; ga.inv_scale = ainv;
+        ga.out16 = a16; ga.inv_scale = ainv;
         launch_glu_fwd(ga, BN);
 
         // ff = act Wd^T, added by the next row kernel                          [:730-740]
-        pending = gemm(s, a16, IS, ainv, at<half_t>(s->wd, (size_t)L * D * IS), IS, D, IS);
+        pending = gemm(s, a16, ainv, at<half_t>(s->wd, L * s->st_d), D, IS);
     }
 
     // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
@@ -198,13 +204,13 @@ void forward_impl(SFTState *s, bool gather)
     if (gemma) { nf.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); nf.branch_raw_out = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); }
     nf.x_out = at<float>(s->xs, (size_t)(2 * L) * xsz);
     nf.g_norm = at<float>(s->g_final);
-    nf.ln16 = a16; nf.ld16 = D; nf.inv_scale = ainv; nf.D = D; nf.eps = s->eps;
+    nf.ln16 = a16; nf.inv_scale = ainv; nf.D = D; nf.eps = s->eps;
     launch_norm_rows(nf, BN);
     GemmPlan pl = plan_gemm(BN, s->V, D);
     if (pl.S == 1) {
-        gemm(s, a16, D, ainv, at<half_t>(s->wlm), D, s->V, D, at<float>(s->logits));
+        gemm(s, a16, ainv, at<half_t>(s->wlm), s->V, D, at<float>(s->logits));
     } else {
-        Planes p = gemm(s, a16, D, ainv, at<half_t>(s->wlm), D, s->V, D);
+        Planes p = gemm(s, a16, ainv, at<half_t>(s->wlm), s->V, D);
         launch_reduce_planes(p.p, p.S, p.stride, p.ld, at<float>(s->logits), BN, s->V);
     }
 }
@@ -220,34 +226,34 @@ void backward_impl(SFTState *s)
     int cur = 0;                                          // dx ping-pong
 
     // dx = RNB(x_final, dlogits Wlm; g_final)                                [:777-790]
-    Planes p = gemm(s, at<half_t>(s->dl16), round8(s->V), at<float>(s->dl_inv), at<half_t>(s->wlmT), round8(s->V), D, round8(s->V));
+    Planes p = gemm(s, at<half_t>(s->dl16), at<float>(s->dl_inv), at<half_t>(s->wlmT), D, s->V);
     NormBwdArgs nb{};
     nb.dy = p; nb.x_saved = at<float>(s->xs, (size_t)(2 * NL) * xsz); nb.g = at<float>(s->g_final);
     nb.eps = s->eps; nb.D = D; nb.dx_prev = nullptr; nb.dx_out = at<float>(s->dx[cur]); nb.clamp = 0.f;
     if (gemma) { nb.branch_raw = at<float>(s->ff_raw, (size_t)(NL - 1) * xsz); nb.g_branch = at<float>(s->g_post_ff, (size_t)(NL - 1) * D); }
-    nb.d16 = a16; nb.ld16 = D; nb.inv_scale = ainv;
+    nb.d16 = a16; nb.inv_scale = ainv;
     launch_norm_bwd_rows(nb, BN);
 
     for (int L = NL - 1; L >= 0; L--) {
         // FFN: d act = d Wd; (dgate, dup); dln2 = dgate Wg + dup Wu; dx += RNB(x_mid, dln2)   [:798-874]
-        Planes pd = gemm(s, a16, D, ainv, at<half_t>(s->wdT, (size_t)L * IS * D), D, IS, D);
+        Planes pd = gemm(s, a16, ainv, at<half_t>(s->wdT, L * s->st_dT), IS, D);
         GluArgs gb{};
         gb.in = pd; gb.IS = IS; gb.gelu = gemma;
         gb.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); gb.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
-        gb.out16 = a16; gb.ld16 = 2 * IS; gb.inv_scale = ainv;
+        gb.out16 = a16; gb.inv_scale = ainv;
         launch_glu_bwd(gb, BN);
-        Planes pgu = gemm(s, a16, 2 * IS, ainv, at<half_t>(s->wguT, (size_t)L * D * 2 * IS), 2 * IS, D, 2 * IS);
+        Planes pgu = gemm(s, a16, ainv, at<half_t>(s->wguT, L * s->st_guT), D, 2 * IS);
         NormBwdArgs n2{};
         n2.dy = pgu; n2.x_saved = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
         n2.g = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
         n2.eps = s->eps; n2.D = D; n2.dx_prev = at<float>(s->dx[cur]); n2.dx_out = at<float>(s->dx[cur ^ 1]); n2.clamp = 0.f;
         if (gemma) { n2.branch_raw = at<float>(s->o_raw, (size_t)L * xsz); n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); }
-        n2.d16 = a16; n2.ld16 = D; n2.inv_scale = ainv;
+        n2.d16 = a16; n2.inv_scale = ainv;
         launch_norm_bwd_rows(n2, BN);
         cur ^= 1;
 
         // attention: dO = d Wo; dq, dk, dv                                    [:877-911]
-        Planes pdo = gemm(s, a16, D, ainv, at<half_t>(s->woT, (size_t)L * qd * D), D, qd, D);
+        Planes pdo = gemm(s, a16, ainv, at<half_t>(s->woT, L * s->st_oT), qd, D);
         AttnBwdArgs ab{};
         ab.dO = pdo;
         ab.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
@@ -264,19 +270,19 @@ void backward_impl(SFTState *s)
         qb.dq = ab.dq; qb.dk = ab.dk; qb.dv = ab.dv;
         qb.q_pre = at<float>(s->q_pre, (size_t)L * BN * qd); qb.k_pre = at<float>(s->k_pre, (size_t)L * BN * kd);
         qb.g_q = at<float>(s->g_q, (size_t)L * s->hd); qb.g_k = at<float>(s->g_k, (size_t)L * s->hd);
-        qb.eps = s->eps; qb.theta = s->rope_thetas[L];
+        qb.eps = s->eps; qb.rope = at<float2>(s->rope_tabs, (size_t)s->rope_slot[L] * s->N * (s->hd / 2));
         qb.Bq = at<float>(s->lora, L * s->lsz + (size_t)R * D);
         qb.Bv = at<float>(s->lora, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
         qb.R = R; qb.sc = s->lora_scaling;
         qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
         qb.dq_f = at<float>(s->dq_f); qb.dv_f = nullptr; qb.dh = at<float>(s->dh);
-        qb.out16 = a16; qb.ld16 = s->ldq; qb.inv_scale = ainv;
+        qb.out16 = a16; qb.inv_scale = ainv;
         launch_qkv_bwd(qb, BN);
         if (R > 0) {
             LoraGradArgs lg{};
             lg.dq_f = qb.dq_f; lg.dv_f = ab.dv; lg.tq = at<float>(s->tq, (size_t)L * BN * R); lg.tv = at<float>(s->tv, (size_t)L * BN * R);
             lg.dh = qb.dh;
-            lg.ln16 = at<half_t>(s->ln1_16, (size_t)L * xsz); lg.ld16 = D; lg.ln_inv_scale = at<float>(s->ln1_inv, (size_t)L * BN);
+            lg.ln16 = at<half_t>(s->ln1_16, (size_t)L * s->st_ln1); lg.ln_inv_scale = at<float>(s->ln1_inv, (size_t)L * BN);
             lg.rows = BN; lg.D = D; lg.qd = qd; lg.kd = kd; lg.R = R; lg.sc = s->lora_scaling;
             lg.grad = at<float>(s->lora_grad, L * s->lsz);
             lg.sq_slots = at<float>(s->sq_slots, (size_t)L * s->slots_per_layer);
@@ -284,13 +290,13 @@ void backward_impl(SFTState *s)
         }
 
         // dln1 = [dq|dk|dv|dh] [Wq;Wk;Wv;A_q;A_v]; dx += RNB(x_in, dln1; g_in); clamp     [:956-980]
-        Planes pl = gemm(s, a16, s->ldq, ainv, at<half_t>(s->wqkvT, (size_t)L * D * s->ldq), s->ldq, D, s->ldq);
+        Planes pl = gemm(s, a16, ainv, at<half_t>(s->wqkvT, L * s->st_qkvT), D, s->nq_ext);
         NormBwdArgs n1{};
         n1.dy = pl; n1.x_saved = at<float>(s->xs, (size_t)(2 * L) * xsz); n1.g = at<float>(s->g_in, (size_t)L * D);
         n1.eps = s->eps; n1.D = D; n1.dx_prev = at<float>(s->dx[cur]); n1.dx_out = at<float>(s->dx[cur ^ 1]); n1.clamp = 1e6f;
         if (L > 0) {
             if (gemma) { n1.branch_raw = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); n1.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); }
-            n1.d16 = a16; n1.ld16 = D; n1.inv_scale = ainv;
+            n1.d16 = a16; n1.inv_scale = ainv;
         }
         launch_norm_bwd_rows(n1, BN);
         cur ^= 1;
@@ -313,8 +319,8 @@ void enqueue_update(SFTState *s)
     a.sq_slots = at<float>(s->sq_slots); a.n_slots = s->slots_per_layer * s->NL;
     a.hyper = at<float>(s->hyper);
     a.b1 = 0.9f; a.b2 = 0.999f; a.eps = 1e-8f; a.wd = 0.01f; a.max_norm = 1.0f;      // src/nn/fast_sft.c:1091-1094
-    a.wqkv = at<half_t>(s->wqkv); a.wqkv_layer_stride = (size_t)s->nq_ext * s->D;
-    a.wqkvT = at<half_t>(s->wqkvT); a.wqkvT_layer_stride = (size_t)s->D * s->ldq; a.ldT = s->ldq;
+    a.wqkv = at<half_t>(s->wqkv); a.wqkv_layer_stride = s->st_qkv;
+    a.wqkvT = at<half_t>(s->wqkvT); a.wqkvT_layer_stride = s->st_qkvT;
     a.NL = s->NL; a.D = s->D; a.qd = s->qd; a.kd = s->kd; a.R = s->R; a.layer_size = s->lsz;
     a.grad_norm_out = at<float>(s->grad_norm);
     launch_adamw(a);
@@ -323,8 +329,8 @@ void enqueue_update(SFTState *s)
 void refresh_shadow(SFTState *s)
 {
     if (!s->R) return;
-    launch_lora_shadow(at<float>(s->lora), s->lora_n, at<half_t>(s->wqkv), (size_t)s->nq_ext * s->D,
-                       at<half_t>(s->wqkvT), (size_t)s->D * s->ldq, s->ldq, s->D, s->qd, s->kd, s->R, s->lsz);
+    launch_lora_shadow(at<float>(s->lora), s->lora_n, at<half_t>(s->wqkv), s->st_qkv,
+                       at<half_t>(s->wqkvT), s->st_qkvT, s->D, s->qd, s->kd, s->R, s->lsz);
 }
 
 MetalBuf *host_buf(size_t bytes, void **cpu)
@@ -353,7 +359,6 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->N = seq_len; s->B = batch; s->BN = batch * seq_len;
     s->qd = s->Hq * s->hd; s->kd = s->Hkv * s->hd; s->R = lora_rank;
     s->nq_ext = s->qd + 2 * s->kd + 2 * s->R;
-    s->ldq = round8(s->nq_ext);
     s->eps = 1e-6f;                                        // src/nn/fast_sft.c:190
     s->lora_scaling = lora_rank > 0 ? lora_alpha / (float)lora_rank : 0.f;
     s->emb_scale = m->model_type == MODEL_GEMMA3 ? sqrtf((float)m->d_model) : 1.0f;   // :302
@@ -361,53 +366,66 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->weight_format = weight_format;
     s->rope_thetas.assign(m->rope_thetas, m->rope_thetas + s->NL);
     const int D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R, NL = s->NL, BN = s->BN, V = s->V;
-    if ((D & 7) || (qd & 7) || (kd & 7) || (IS & 7) || (s->nq_ext & 7) || (s->hd & 3) || (!weight_format && ((D & 31) || (IS & 31) || (qd & 31)))) {
-        fprintf(stderr, "[FastSFT] unsupported dims: d_model, head widths, FFN width and 2*rank must be multiples of 8 "
-                        "(32 for Q8_0)\n");
+    if ((s->hd & 3) || (s->Hq % s->Hkv) || (D & 3) || (IS & 3) || (V & 3) || (lora_rank & 1) || lora_rank > 16 || (!weight_format && ((D & 31) || (IS & 31) || (qd & 31)))) {
+        fprintf(stderr, "[FastSFT] unsupported dims: d_model, FFN width, vocab, head_dim must be multiples of 4, Hq of Hkv, rank even and <= 16 "
+                        "(and every matrix width a multiple of 32 for Q8_0)\n");
         delete s;
         fast_metal_shutdown();
         return nullptr;
     }
 
-    // ---- frozen weights: F16 arenas plus transposed copies for the dX products ----
-    s->wqkv = hbuf((size_t)NL * s->nq_ext * D);  s->wqkvT = hbuf((size_t)NL * D * s->ldq);
-    s->wo = hbuf((size_t)NL * D * qd);           s->woT = hbuf((size_t)NL * qd * D);
-    s->wgu = hbuf((size_t)NL * 2 * IS * D);      s->wguT = hbuf((size_t)NL * D * 2 * IS);
-    s->wd = hbuf((size_t)NL * D * IS);           s->wdT = hbuf((size_t)NL * IS * D);
-    s->wlm = hbuf((size_t)V * D);                s->wlmT = hbuf((size_t)D * round8(V));
-    HIP_CHECK(hipMemsetAsync(dptr(s->wqkv), 0, s->wqkv->size, stream()));
-    HIP_CHECK(hipMemsetAsync(dptr(s->wqkvT), 0, s->wqkvT->size, stream()));
-    HIP_CHECK(hipMemsetAsync(dptr(s->wlmT), 0, s->wlmT->size, stream()));
-    std::vector<MetalBuf *> q8_keep;
+    // ---- frozen weights: tiled F16 arenas plus transposed images for the dX products ----
+    s->st_qkv = tiled_elems(s->nq_ext, D); s->st_qkvT = tiled_elems(D, s->nq_ext);
+    s->st_o = tiled_elems(D, qd);          s->st_oT = tiled_elems(qd, D);
+    s->st_gu = tiled_elems(2 * IS, D);     s->st_guT = tiled_elems(D, 2 * IS);
+    s->st_d = tiled_elems(D, IS);          s->st_dT = tiled_elems(IS, D);
+    s->st_ln1 = tiled_elems(BN, D);
+    s->wqkv = hbuf(NL * s->st_qkv); s->wqkvT = hbuf(NL * s->st_qkvT);
+    s->wo = hbuf(NL * s->st_o);     s->woT = hbuf(NL * s->st_oT);
+    s->wgu = hbuf(NL * s->st_gu);   s->wguT = hbuf(NL * s->st_guT);
+    s->wd = hbuf(NL * s->st_d);     s->wdT = hbuf(NL * s->st_dT);
+    s->wlm = hbuf(tiled_elems(V, D)); s->wlmT = hbuf(tiled_elems(D, V));
+    for (MetalBuf *b : {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT})
+        HIP_CHECK(hipMemsetAsync(dptr(b), 0, b->size, stream()));        // row and K padding must read as zero
     s->g_in = fbuf((size_t)NL * D); s->g_post_attn = fbuf((size_t)NL * D);
     s->g_pre_ff = fbuf((size_t)NL * D); s->g_post_ff = fbuf((size_t)NL * D);
     s->g_q = fbuf((size_t)NL * s->hd); s->g_k = fbuf((size_t)NL * s->hd);
+    const int kbD = tiled_kb(D), kbQ = tiled_kb(qd), kbI = tiled_kb(IS), kb2I = tiled_kb(2 * IS), kbX = tiled_kb(s->nq_ext);
     for (int L = 0; L < NL; L++) {
         const LayerWeightRef *r = &m->layers[L];
-        const size_t oq = (size_t)L * s->nq_ext * D;
-        put_matrix(s, s->wqkv, oq, r->q_proj.data, qd, D, q8_keep);
-        put_matrix(s, s->wqkv, oq + (size_t)qd * D, r->k_proj.data, kd, D, q8_keep);
-        put_matrix(s, s->wqkv, oq + (size_t)(qd + kd) * D, r->v_proj.data, kd, D, q8_keep);
-        put_matrix(s, s->wo, (size_t)L * D * qd, r->o_proj.data, D, qd, q8_keep);
-        put_matrix(s, s->wgu, (size_t)L * 2 * IS * D, r->gate_proj.data, IS, D, q8_keep);
-        put_matrix(s, s->wgu, (size_t)L * 2 * IS * D + (size_t)IS * D, r->up_proj.data, IS, D, q8_keep);
-        put_matrix(s, s->wd, (size_t)L * D * IS, r->down_proj.data, D, IS, q8_keep);
+        put_matrix(s, r->q_proj.data, qd, D, {s->wqkv, L * s->st_qkv, kbD, 0, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, 0, 1});
+        put_matrix(s, r->k_proj.data, kd, D, {s->wqkv, L * s->st_qkv, kbD, qd, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, qd, 1});
+        put_matrix(s, r->v_proj.data, kd, D, {s->wqkv, L * s->st_qkv, kbD, qd + kd, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, qd + kd, 1});
+        put_matrix(s, r->o_proj.data, D, qd, {s->wo, L * s->st_o, kbQ, 0, 0, 0}, {s->woT, L * s->st_oT, kbD, 0, 0, 1});
+        put_matrix(s, r->gate_proj.data, IS, D, {s->wgu, L * s->st_gu, kbD, 0, 0, 0}, {s->wguT, L * s->st_guT, kb2I, 0, 0, 1});
+        put_matrix(s, r->up_proj.data, IS, D, {s->wgu, L * s->st_gu, kbD, IS, 0, 0}, {s->wguT, L * s->st_guT, kb2I, 0, IS, 1});
+        put_matrix(s, r->down_proj.data, D, IS, {s->wd, L * s->st_d, kbI, 0, 0, 0}, {s->wdT, L * s->st_dT, kbD, 0, 0, 1});
         metal_buf_write(s->g_in, (size_t)L * D * 4, r->input_norm_g, (size_t)D * 4);
         metal_buf_write(s->g_post_attn, (size_t)L * D * 4, r->post_attn_norm_g, (size_t)D * 4);
         if (r->pre_ff_norm_g) metal_buf_write(s->g_pre_ff, (size_t)L * D * 4, r->pre_ff_norm_g, (size_t)D * 4);
         if (r->post_ff_norm_g) metal_buf_write(s->g_post_ff, (size_t)L * D * 4, r->post_ff_norm_g, (size_t)D * 4);
         metal_buf_write(s->g_q, (size_t)L * s->hd * 4, r->q_norm_g, (size_t)s->hd * 4);
         metal_buf_write(s->g_k, (size_t)L * s->hd * 4, r->k_norm_g, (size_t)s->hd * 4);
-        launch_transpose_f16(at<half_t>(s->wo, (size_t)L * D * qd), at<half_t>(s->woT, (size_t)L * qd * D), D, qd, D);
-        launch_transpose_f16(at<half_t>(s->wgu, (size_t)L * 2 * IS * D), at<half_t>(s->wguT, (size_t)L * D * 2 * IS), 2 * IS, D, 2 * IS);
-        launch_transpose_f16(at<half_t>(s->wd, (size_t)L * D * IS), at<half_t>(s->wdT, (size_t)L * IS * D), D, IS, D);
     }
-    put_matrix(s, s->wlm, 0, m->lm_head, V, D, q8_keep);
-    launch_transpose_f16(at<half_t>(s->wlm), at<half_t>(s->wlmT), V, D, round8(V));
+    put_matrix(s, m->lm_head, V, D, {s->wlm, 0, kbD, 0, 0, 0}, {s->wlmT, 0, tiled_kb(V), 0, 0, 1});
     s->g_final = metal_buf_from_data(m->final_norm_g, (size_t)D * 4);
     s->emb = metal_buf_from_data(m->token_emb, (size_t)V * D * 4);
     s->q8_blocks = nullptr;
-    for (MetalBuf *b : q8_keep) metal_buf_free(b);       // the bytes were only needed to form the values
+
+    // ---- RoPE tables: one per distinct theta (Gemma3 has two) ----
+    {
+        std::vector<float> distinct;
+        for (int L = 0; L < NL; L++) {
+            int slot = -1;
+            for (size_t k = 0; k < distinct.size(); k++) if (distinct[k] == s->rope_thetas[L]) slot = (int)k;
+            if (slot < 0) { slot = (int)distinct.size(); distinct.push_back(s->rope_thetas[L]); }
+            s->rope_slot.push_back(slot);
+        }
+        const size_t per = (size_t)s->N * (s->hd / 2);
+        s->rope_tabs = metal_buf_create(distinct.size() * per * sizeof(float2));
+        for (size_t k = 0; k < distinct.size(); k++)
+            launch_rope_table(at<float2>(s->rope_tabs, k * per), s->N, s->hd, distinct[k]);
+    }
 
     // ---- LoRA arena, gradients, optimiser state ----
     s->lsz = (size_t)2 * R * D + (size_t)qd * R + (size_t)kd * R;
@@ -456,7 +474,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     // ---- saved activations and transients ----
     const size_t xsz = (size_t)BN * D;
     s->xs = fbuf((size_t)(2 * NL + 1) * xsz);
-    s->ln1_16 = hbuf((size_t)NL * xsz); s->ln1_inv = fbuf((size_t)NL * BN);
+    s->ln1_16 = hbuf((size_t)NL * s->st_ln1); s->ln1_inv = fbuf((size_t)NL * BN);
     s->q_pre = fbuf((size_t)NL * BN * qd); s->k_pre = fbuf((size_t)NL * BN * kd);
     s->q_fin = fbuf((size_t)NL * BN * qd); s->k_fin = fbuf((size_t)NL * BN * kd); s->v_sav = fbuf((size_t)NL * BN * kd);
     s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
@@ -467,24 +485,21 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     int maxk = D;
     if (qd > maxk) maxk = qd;
     if (2 * IS > maxk) maxk = 2 * IS;
-    if (s->ldq > maxk) maxk = s->ldq;
-    s->a16 = hbuf((size_t)BN * maxk); s->a16_inv = fbuf(BN);
+    if (s->nq_ext > maxk) maxk = s->nq_ext;
+    s->a16 = hbuf(tiled_elems(BN, maxk)); s->a16_inv = fbuf(BN);
     s->ones = fbuf(BN);
     launch_fill_f32(at<float>(s->ones), 1.0f, BN);
     s->planes_cap = max_planes_elems(s);
     s->planes = fbuf(s->planes_cap);
     s->logits = fbuf((size_t)BN * V); s->dlogits = nullptr;
-    s->dl16 = hbuf((size_t)BN * round8(V)); s->dl_inv = fbuf(BN);
+    s->dl16 = hbuf(tiled_elems(BN, V)); s->dl_inv = fbuf(BN);
     s->dx[0] = fbuf(xsz); s->dx[1] = fbuf(xsz);
     s->dO_red = fbuf((size_t)BN * qd); s->dscore = fbuf((size_t)s->B * s->Hq * s->N * s->N);
     s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf((size_t)BN * kd);
     s->dq_f = fbuf((size_t)BN * qd); s->dh = fbuf((size_t)BN * (R ? 2 * R : 1));
 
-    // the fused QKV weight carries fp16 images of A_q, A_v; its transpose follows from it
+    // the fused QKV weight and its transpose carry fp16 images of A_q, A_v
     refresh_shadow(s);
-    for (int L = 0; L < NL; L++)
-        launch_transpose_f16(at<half_t>(s->wqkv, (size_t)L * s->nq_ext * D), at<half_t>(s->wqkvT, (size_t)L * D * s->ldq),
-                             s->nq_ext, D, s->ldq);
     metal_flush();
     return s;
 }
@@ -496,7 +511,7 @@ void sft_state_free(SFTState *s)
     for (MetalBuf *b : s->lora_views) metal_buf_free(b);
     for (MetalBuf *b : s->grad_views) metal_buf_free(b);
     MetalBuf *all[] = {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT, s->q8_blocks,
-                       s->g_in, s->g_post_attn, s->g_pre_ff, s->g_post_ff, s->g_q, s->g_k, s->g_final, s->emb,
+                       s->rope_tabs, s->g_in, s->g_post_attn, s->g_pre_ff, s->g_post_ff, s->g_q, s->g_k, s->g_final, s->emb,
                        s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
@@ -516,7 +531,7 @@ void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uin
     forward_impl(s, true);
     CeArgs ce{};
     ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
-    ce.dl16 = at<half_t>(s->dl16); ce.ld16 = round8(s->V); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
+    ce.dl16 = at<half_t>(s->dl16); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
     launch_ce_rows(ce, s->BN);
     backward_impl(s);
     enqueue_update(s);
@@ -545,7 +560,7 @@ void forward_to_logits(SFTState *s)
 void sft_backward(SFTState *s)
 {
     MetalBuf *dl = sft_get_dlogits(s);
-    launch_rows_to_f16(at<float>(dl), s->V, at<half_t>(s->dl16), round8(s->V), at<float>(s->dl_inv), s->BN, s->V);
+    launch_rows_to_f16(at<float>(dl), s->V, at<half_t>(s->dl16), at<float>(s->dl_inv), s->BN, s->V);
     backward_impl(s);
 }
 
