@@ -55,6 +55,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c3_qwen3_4b_f16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the library's plain copy kernel (1 GiB in, 1 GiB out, 5 launches): "
+                         "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the step has no multi-GPU path); use --gpus 1",
@@ -65,6 +68,21 @@ def main():
     from llm_metal_amd import lib
     from llm_metal_amd.sft import SFTState
     L = lib.load()
+
+    if args.copy_calibration:
+        if L.fast_metal_init() != 0:
+            sys.exit("no gfx950 device")
+        n = 1 << 28                                        # floats: 1 GiB read + 1 GiB written per launch
+        src, dst = L.metal_buf_create(4 * n), L.metal_buf_create(4 * n)
+        L.metal_enqueue_scale(src, 0.0, n)                 # touch the source once
+        for _ in range(5):
+            L.metal_enqueue_copy(src, dst, n)
+        L.metal_flush()
+        L.metal_buf_free(src), L.metal_buf_free(dst)
+        L.fast_metal_shutdown()
+        print(json.dumps({"copy_calibration": {"kernel": "k_copy", "bytes_read_per_launch": 4 * n,
+                                               "bytes_written_per_launch": 4 * n, "launches": 5}}))
+        return
 
     t0 = time.perf_counter()
     model = make_model(cfg, seed=0, lora_b_std=0.0)          # timing runs: B = 0 as the reference initialises it

@@ -202,9 +202,20 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
             float acc0 = 0.f, acc1 = 0.f;
             const float *b0 = B + (size_t)(h * hd + (d < half ? d : 0)) * a.R;
             const float *b1 = b0 + (size_t)half * a.R;
-            for (int r = 0; r < a.R; r++) {
-                const float t = __shfl(tval, r, WAVE);
-                if (d < half) { acc0 += t * b0[r]; acc1 += t * b1[r]; }
+            if ((a.R & 3) == 0) {                              // whole rows of B as independent 16-byte loads
+                for (int r4 = 0; r4 < a.R; r4 += 4) {
+                    float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w1 = w0;
+                    if (d < half) { w0 = ld4(b0 + r4); w1 = ld4(b1 + r4); }
+                    const float t0 = __shfl(tval, r4, WAVE), t1 = __shfl(tval, r4 + 1, WAVE);
+                    const float t2 = __shfl(tval, r4 + 2, WAVE), t3 = __shfl(tval, r4 + 3, WAVE);
+                    acc0 += t0 * w0.x; acc0 += t1 * w0.y; acc0 += t2 * w0.z; acc0 += t3 * w0.w;
+                    acc1 += t0 * w1.x; acc1 += t1 * w1.y; acc1 += t2 * w1.z; acc1 += t3 * w1.w;
+                }
+            } else {
+                for (int r = 0; r < a.R; r++) {
+                    const float t = __shfl(tval, r, WAVE);
+                    if (d < half) { acc0 += t * b0[r]; acc1 += t * b1[r]; }
+                }
             }
             x0[p] += a.sc * acc0;
             x1[p] += a.sc * acc1;
@@ -336,31 +347,36 @@ __global__ __launch_bounds__(64) void k_attn_bwd_dq(AttnBwdArgs a)
 }
 
 // attn_bwd_dkv + repeat_kv_bwd, shaders/q8_kernels.metal:931-992: one workgroup per
-// (kv head, key, sequence); the four waves split the queries i >= j between them (the sum
-// also runs over the query heads of the group) and add their partial rows through LDS.
+// (kv head, key j, sequence).  The column j of dS and P for every query head of the group
+// is first gathered into LDS (one round of independent loads), then the four waves split
+// the (head, query) pairs and stream the matching q / dO rows; partial rows meet in LDS.
 __global__ __launch_bounds__(TB) void k_attn_bwd_dkv(AttnBwdArgs a)
 {
-    extern __shared__ float part[];                      // [4 waves][2][hd]
+    extern __shared__ float lds[];                       // [ratio*N] ds column, [ratio*N] p column, [4][2][hd] partials
     const int N = a.seq, hd = a.hd, ratio = a.Hq / a.Hkv;
     const int hk = blockIdx.x, j = blockIdx.y, b = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int qd = a.Hq * hd, kd = a.Hkv * hd;
     const size_t r0 = (size_t)b * N;
+    float *dsc = lds, *pc = lds + ratio * N, *part = lds + 2 * ratio * N;
+    const int npair = ratio * (N - j);                   // pairs (g, i) with i >= j
+    for (int t = threadIdx.x; t < npair; t += TB) {
+        const int g = t / (N - j), i = j + t % (N - j);
+        const size_t o = (((size_t)b * a.Hq + hk * ratio + g) * N + i) * N + j;
+        dsc[t] = a.dscore[o];
+        pc[t] = a.probs[o];
+    }
+    __syncthreads();
     for (int d0 = 0; d0 < hd; d0 += 64) {
         const int d = d0 + lane;
         float dk = 0.f, dv = 0.f;
         if (d < hd) {
-            for (int g = 0; g < ratio; g++) {
-                const int h = hk * ratio + g;
-                const float *dsp = a.dscore + ((size_t)b * a.Hq + h) * N * N + j;
-                const float *pp = a.probs + ((size_t)b * a.Hq + h) * N * N + j;
-                const float *qp = a.q + r0 * qd + h * hd + d;
-                const float *dop = a.dO_red + r0 * qd + h * hd + d;
-#pragma unroll 4
-                for (int i = j + wave; i < N; i += 4) {
-                    dk += dsp[(size_t)i * N] * qp[(size_t)i * qd];
-                    dv += pp[(size_t)i * N] * dop[(size_t)i * qd];
-                }
+#pragma unroll 8
+            for (int t = wave; t < npair; t += 4) {
+                const int g = t / (N - j), i = j + t % (N - j);
+                const size_t o = (r0 + i) * qd + (hk * ratio + g) * hd + d;
+                dk += dsc[t] * a.q[o];
+                dv += pc[t] * a.dO_red[o];
             }
             part[(wave * 2 + 0) * hd + d] = dk;
             part[(wave * 2 + 1) * hd + d] = dv;
@@ -442,11 +458,20 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
             const int isv = c >= qd;
             const float x = buf[isv ? c + kd : c];
             const float *Br = isv ? a.Bv + (size_t)(c - qd) * R : a.Bq + (size_t)c * R;
+            float bv[16];
+            if ((R & 3) == 0) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float bv = (r < R) ? Br[r] : 0.f;
-                if (isv) acc[16 + r] += x * bv; else acc[r] += x * bv;
+                for (int r4 = 0; r4 < 16; r4 += 4) {
+                    float4 w = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (r4 < R) w = ld4(Br + r4);
+                    bv[r4] = w.x; bv[r4 + 1] = w.y; bv[r4 + 2] = w.z; bv[r4 + 3] = w.w;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) bv[r] = (r < R) ? Br[r] : 0.f;
             }
+#pragma unroll
+            for (int r = 0; r < 16; r++) { if (isv) acc[16 + r] += x * bv[r]; else acc[r] += x * bv[r]; }
         }
 #pragma unroll
         for (int r = 0; r < 32; r++) acc[r] = wave_sum(acc[r]);
@@ -832,7 +857,9 @@ void launch_attn_bwd(const AttnBwdArgs &a)
 {
     require(a.hd % 4 == 0 && a.seq <= 4096, "attn_bwd: head_dim % 4, seq <= 4096");
     LAUNCH(k_attn_bwd_dq, dim3(a.Hq, a.seq, a.batch), dim3(64), (size_t)(a.seq + a.hd) * 4, a);
-    LAUNCH(k_attn_bwd_dkv, dim3(a.Hkv, a.seq, a.batch), dim3(TB), (size_t)8 * a.hd * 4, a);
+    const size_t dkv_lds = ((size_t)2 * (a.Hq / a.Hkv) * a.seq + 8 * a.hd) * 4;
+    require(dkv_lds <= 64 * 1024, "attn_bwd: (Hq/Hkv) * seq too large for the dK/dV kernel");
+    LAUNCH(k_attn_bwd_dkv, dim3(a.Hkv, a.seq, a.batch), dim3(TB), dkv_lds, a);
 }
 
 void launch_qkv_bwd(const QkvBwdArgs &a, int rows)

@@ -42,7 +42,7 @@ __device__ __forceinline__ void load_stage(Stage<NB> &st, const half8 *const (&a
 #pragma unroll
     for (int j = 0; j < 4; j++) {
 #pragma unroll
-        for (int b = 0; b < NB; b++) st.w[b][j] = wp[b][o + j * 64];
+        for (int b = 0; b < NB; b++) st.w[b][j] = __builtin_nontemporal_load(&wp[b][o + j * 64]);   // streamed once: keep L2 for A
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) st.a[mb][j] = ap[mb][o + j * 64];
     }
