@@ -9,12 +9,13 @@
 
 namespace lmhip {
 
-// K-split partial planes of a GEMM output: value(row, col) = sum_s p[s*stride + row*ld + col]
+// K-split partial planes of a GEMM output: value(row, col) = row_scale[row] * sum_s p[s*stride + row*ld + col]
 struct Planes {
     const float *p;
     int S;
     size_t stride;
     int ld;
+    const float *row_scale;   // value(row, col) is multiplied by row_scale[row] when non-null
 };
 
 struct NormRowsArgs {

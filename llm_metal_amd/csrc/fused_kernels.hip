@@ -23,7 +23,7 @@ __device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
     float s = 0.f;
     const float *p = P.p + row * P.ld + col;
     for (int i = 0; i < P.S; i++) s += p[(size_t)i * P.stride];
-    return s;
+    return P.row_scale ? s * P.row_scale[row] : s;
 }
 
 // Sum of the planes at four consecutive columns (col % 4 == 0, ld % 4 == 0).
@@ -42,6 +42,7 @@ __device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int co
         const float4 a = *reinterpret_cast<const float4 *>(p + (size_t)i * P.stride);
         s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
     }
+    if (P.row_scale) { const float f = P.row_scale[row]; s.x *= f; s.y *= f; s.z *= f; s.w *= f; }
     return s;
 }
 

@@ -31,18 +31,21 @@ struct GemmPlan {
     int S;         // K chunks = partial planes written
     int steps;     // 64-wide K steps per chunk
     int n_tiles, m_tiles;
+    int rotate;    // start each workgroup at a different K step of its chunk
 };
 
 GemmPlan plan_gemm(int M, int N, int K);
 
 // P[s][m][n] (s < plan.S, plane s at P + s*plane_stride, row stride ldp) =
-//   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k],  A and W in the tiled layout
+//   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k],  A and W in the tiled layout.
+// Pass a_inv_scale = null to leave the row factors to the consumer of the planes.
 void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const half_t *W_tiled,
                  float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p);
 
 // out (tiled [M, K]) = fp16(X[m][k] * s_m), zero in the K padding; inv_scale[m] = 1/s_m
 void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_scale, int M, int K);
-void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, float *C, int M, int N);
+// C[m][n] = row_scale[m] * sum_s P[s][m][n] (row_scale may be null)
+void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, const float *row_scale, float *C, int M, int N);
 // dst (tiled, Kb_dst K blocks) <- src row-major F16 [rows, cols]:
 //   element (r, c) goes to tiled(row_off + r, k_off + c), or tiled(row_off + c, k_off + r) when transposed
 void launch_tile_f16(const half_t *src, int rows, int cols, half_t *dst_tiled, int Kb_dst,

@@ -24,114 +24,10 @@
 #include "backend.h"
 #include "devutil.h"
 #include "gemm.h"
+#include "gemm_kernel.h"
 #include <vector>
 
 namespace {
-
-template <int NB>
-struct Stage {
-    half8 a[2][4];
-    half8 w[NB][4];
-};
-
-template <int NB>
-__device__ __forceinline__ void load_stage(Stage<NB> &st, const half8 *const (&ap)[2],
-                                           const half8 *const (&wp)[NB], int kb)
-{
-    const size_t o = (size_t)kb * 256;                   // 4 x 64 half8 per K step
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-#pragma unroll
-        for (int b = 0; b < NB; b++) st.w[b][j] = __builtin_nontemporal_load(&wp[b][o + j * 64]);   // streamed once: keep L2 for A
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++) st.a[mb][j] = ap[mb][o + j * 64];
-    }
-}
-
-template <int NB>
-__device__ __forceinline__ void mma_stage(const Stage<NB> &st, float16v (&acc)[2][NB])
-{
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int b = 0; b < NB; b++)
-                acc[mb][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(st.a[mb][j], st.w[b][j], acc[mb][b], 0, 0, 0);
-}
-
-// grid: x = ceil(Nb / NB) weight-row tiles, y = S (K chunks), z = ceil(M / 64); block = 256.
-// Kb = number of 64-wide K steps of the (padded) reduction; Nb, Mb = 32-row blocks of W and A.
-template <int NB>
-__global__ __launch_bounds__(256, 2) void gemm_tiled_f16(
-    const half8 *__restrict__ A, const float *__restrict__ a_inv_scale, const half8 *__restrict__ W,
-    float *__restrict__ P, int ldp, size_t plane_stride,
-    int M, int N, int Mb, int Nb, int Kb, int steps_per_chunk)
-{
-    extern __shared__ float red[];                       // [4 waves][2*NB*16 regs][64 lanes]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 31, h = lane >> 5;
-    const int nb0 = blockIdx.x * NB, mb0 = blockIdx.z * 2;
-    const int kb_beg = blockIdx.y * steps_per_chunk;
-    const int kb_end = min(Kb, kb_beg + steps_per_chunk);
-
-    const half8 *wp[NB];
-    const half8 *ap[2];
-#pragma unroll
-    for (int b = 0; b < NB; b++) wp[b] = W + (size_t)min(nb0 + b, Nb - 1) * Kb * 256 + lane;
-#pragma unroll
-    for (int mb = 0; mb < 2; mb++) ap[mb] = A + (size_t)min(mb0 + mb, Mb - 1) * Kb * 256 + lane;
-
-    float16v acc[2][NB];
-#pragma unroll
-    for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[mb][b][v] = 0.f;
-
-    // wave w takes the K steps w, w+4, w+8, ... of this workgroup's chunk
-    int kb = kb_beg + wave;
-    Stage<NB> s0, s1;
-    if (kb < kb_end) load_stage<NB>(s0, ap, wp, kb);
-    while (kb < kb_end) {
-        if (kb + 4 < kb_end) load_stage<NB>(s1, ap, wp, kb + 4);
-        mma_stage<NB>(s0, acc);
-        kb += 4;
-        if (kb >= kb_end) break;
-        if (kb + 4 < kb_end) load_stage<NB>(s0, ap, wp, kb + 4);
-        mma_stage<NB>(s1, acc);
-        kb += 4;
-    }
-
-    // add the four waves' accumulators: red[wave][reg][lane], lane fastest => conflict-free
-    constexpr int REGS = 2 * NB * 16;
-#pragma unroll
-    for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-#pragma unroll
-            for (int v = 0; v < 16; v++)
-                red[(wave * REGS + (mb * NB + b) * 16 + v) * 64 + lane] = acc[mb][b][v];
-    __syncthreads();
-
-    float *Pp = P + (size_t)blockIdx.y * plane_stride;
-#pragma unroll
-    for (int i = 0; i < REGS / 4; i++) {
-        const int reg = wave + 4 * i;                      // this thread finishes (reg, lane)
-        float s = red[(0 * REGS + reg) * 64 + lane] + red[(1 * REGS + reg) * 64 + lane]
-                + red[(2 * REGS + reg) * 64 + lane] + red[(3 * REGS + reg) * 64 + lane];
-        const int v = reg & 15, blk = reg >> 4;
-        const int b = blk % NB, mb = blk / NB;
-        // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4
-        const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-        const int n = (nb0 + b) * 32 + r;
-        if (m < M && n < N) {
-            if (a_inv_scale) s *= a_inv_scale[m];
-            Pp[(size_t)m * ldp + n] = s;
-        }
-    }
-}
 
 // One workgroup per row: fp32 row -> tiled fp16 row scaled by a power of two, plus 1/scale.
 __global__ __launch_bounds__(256) void rows_to_f16_scaled(
@@ -150,14 +46,14 @@ __global__ __launch_bounds__(256) void rows_to_f16_scaled(
 }
 
 __global__ void reduce_planes(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
-                              float *__restrict__ C, int M, int N)
+                              const float *__restrict__ row_scale, float *__restrict__ C, int M, int N)
 {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)M * N) return;
     const int m = (int)(idx / N), n = (int)(idx % N);
     float s = 0.f;
     for (int p = 0; p < S; p++) s += P[p * plane_stride + (size_t)m * ldp + n];
-    C[idx] = s;
+    C[idx] = row_scale ? s * row_scale[m] : s;
 }
 
 // Row-major F16 [rows, cols] -> tiled layout, optionally transposed; 64x64 element tiles via LDS
@@ -193,27 +89,32 @@ int g_force_nb = 0, g_force_S = 0;
 
 namespace lmhip {
 
-// Tile height and K split.  Measured on MI355X at M = 64: one 32-row block per wave (lower
-// register use, three resident workgroups per CU) beats two at every shape of the step, and
-// the kernel wants at least ~2.5 workgroups per CU even when that leaves each with only a
-// couple of K steps per wave; beyond that, splitting K only adds partial-plane traffic.
+// Tile height and K split, from measurements on MI355X at M = 64: two 32-row blocks per wave
+// (activation bytes through L1/L2 = weight bytes), about three workgroups per CU, chunks of at
+// least 4 and at most 40 K steps (long chunks gain nothing and short ones spread the
+// activation reads over more L2 lines); beyond that, splitting K only adds plane traffic.
 GemmPlan plan_gemm(int M, int N, int K)
 {
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), m_tiles = (M + 63) / 64;
     const int cus = num_cus() > 0 ? num_cus() : 256;
     GemmPlan p{};
-    p.nb = g_force_nb ? g_force_nb : 1;
+    p.nb = g_force_nb ? g_force_nb : (Nb >= 2 ? 2 : 1);
     p.n_tiles = (Nb + p.nb - 1) / p.nb;
     p.m_tiles = m_tiles;
     const int base = p.n_tiles * m_tiles;
-    int S = g_force_S ? g_force_S : (5 * cus / 2 + base - 1) / base;
-    const int max_s = Kb >= 8 ? Kb / 8 : 1;                // at least two K steps per wave
-    if (!g_force_S && S > max_s) S = max_s;
+    int S = g_force_S ? g_force_S : (3 * cus + base - 1) / base;
     if (S < 1) S = 1;
     int steps = (Kb + S - 1) / S;
+    if (!g_force_S) {
+        if (steps < 4) steps = 4;
+        if (steps > 40) steps = 40;
+    }
     steps = (steps + 3) & ~3;                              // whole steps for each of the four waves
+    if (steps > Kb) steps = Kb;
     p.steps = steps;
     p.S = (Kb + steps - 1) / steps;
+    // rotate the K order unless the activation matrix is too big to stay in an XCD's L2
+    p.rotate = (size_t)tiled_rb(M) * 32 * Kb * 64 * 2 <= (size_t)4 << 20;
     return p;
 }
 
@@ -228,7 +129,7 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const half_t *W,
     }
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
     dim3 grid(p.n_tiles, p.S, p.m_tiles), block(256);
-    const size_t lds = (size_t)4 * (2 * p.nb * 16) * 64 * sizeof(float);
+    const size_t lds = (size_t)2 * (2 * p.nb * 16) * 64 * sizeof(float);
     ProfRec rec{};
     if (g_prof_on) {
         HIP_CHECK(hipEventCreate(&rec.a));
@@ -237,12 +138,13 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const half_t *W,
         HIP_CHECK(hipEventRecord(rec.a, stream()));
     }
     const half8 *A8 = reinterpret_cast<const half8 *>(A), *W8 = reinterpret_cast<const half8 *>(W);
-    if (p.nb == 2)
-        hipLaunchKernelGGL(gemm_tiled_f16<2>, grid, block, lds, stream(), A8, a_inv_scale, W8,
-                           P, ldp, plane_stride, M, N, Mb, Nb, Kb, p.steps);
-    else
-        hipLaunchKernelGGL(gemm_tiled_f16<1>, grid, block, lds, stream(), A8, a_inv_scale, W8,
-                           P, ldp, plane_stride, M, N, Mb, Nb, Kb, p.steps);
+#define GEMM_LAUNCH(NBV, ROT, SC) hipLaunchKernelGGL((gemm_tiled_f16<NBV, ROT, SC>), grid, block, lds, stream(), A8, a_inv_scale, W8, \
+                                                    P, ldp, plane_stride, M, N, Mb, Nb, Kb, p.steps)
+#define GEMM_PICK(NBV, ROT) do { if (a_inv_scale) GEMM_LAUNCH(NBV, ROT, 1); else GEMM_LAUNCH(NBV, ROT, 0); } while (0)
+    if (p.nb == 2) { if (p.rotate) GEMM_PICK(2, 1); else GEMM_PICK(2, 0); }
+    else           { if (p.rotate) GEMM_PICK(1, 1); else GEMM_PICK(1, 0); }
+#undef GEMM_PICK
+#undef GEMM_LAUNCH
     HIP_CHECK(hipGetLastError());
     if (g_prof_on) {
         HIP_CHECK(hipEventRecord(rec.b, stream()));
@@ -256,11 +158,11 @@ void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_s
     HIP_CHECK(hipGetLastError());
 }
 
-void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, float *C, int M, int N)
+void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, const float *row_scale, float *C, int M, int N)
 {
     const size_t n = (size_t)M * N;
     hipLaunchKernelGGL(reduce_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(),
-                       P, S, plane_stride, ldp, C, M, N);
+                       P, S, plane_stride, ldp, row_scale, C, M, N);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -321,8 +223,8 @@ void gemm_f32a(const float *A, const half_t *Wt, float *C, int M, int Nout, int 
     } else {
         const size_t plane = (size_t)M * Nout;
         float *P = (float *)scratch(SCR_PARTIAL, plane * p.S * sizeof(float));
-        launch_gemm(a16, inv, Wt, P, Nout, plane, M, Nout, Kred, p);
-        launch_reduce_planes(P, p.S, plane, Nout, C, M, Nout);
+        launch_gemm(a16, nullptr, Wt, P, Nout, plane, M, Nout, Kred, p);
+        launch_reduce_planes(P, p.S, plane, Nout, inv, C, M, Nout);
     }
 }
 
@@ -398,10 +300,10 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int S, int iters, int *u
     HIP_CHECK(hipEventCreate(&e0)); HIP_CHECK(hipEventCreate(&e1));
     const int saved = g_prof_on;
     g_prof_on = 0;
-    for (int i = 0; i < 3; i++) launch_gemm((half_t *)A, (float *)inv, (half_t *)W, (float *)P, N, (size_t)M * N, M, N, K, p);
+    for (int i = 0; i < 3; i++) launch_gemm((half_t *)A, nullptr, (half_t *)W, (float *)P, N, (size_t)M * N, M, N, K, p);
     HIP_CHECK(hipEventRecord(e0, stream()));
     for (int i = 0; i < iters; i++)
-        launch_gemm((half_t *)A, (float *)inv, (half_t *)((char *)W + (size_t)(i % nbuf) * wb), (float *)P, N, (size_t)M * N, M, N, K, p);
+        launch_gemm((half_t *)A, nullptr, (half_t *)((char *)W + (size_t)(i % nbuf) * wb), (float *)P, N, (size_t)M * N, M, N, K, p);
     HIP_CHECK(hipEventRecord(e1, stream()));
     HIP_CHECK(hipStreamSynchronize(stream()));
     g_prof_on = saved;

@@ -116,8 +116,9 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const half_t *W, int
     const size_t stride = (size_t)s->BN * N;
     if (!out && (size_t)p.S * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
     if (out && p.S != 1) { fprintf(stderr, "[fast_sft] direct GEMM output needs S == 1\n"); abort(); }
-    launch_gemm(A, inv, W, P, N, stride, s->BN, N, K, p);
-    return Planes{P, p.S, stride, N};
+    // a direct (final) output gets its row factors in the GEMM epilogue; planes leave them to the consumer
+    launch_gemm(A, out ? inv : nullptr, W, P, N, stride, s->BN, N, K, p);
+    return Planes{P, p.S, stride, N, out ? nullptr : inv};
 }
 
 void forward_impl(SFTState *s, bool gather)
@@ -127,7 +128,7 @@ void forward_impl(SFTState *s, bool gather)
     half_t *a16 = at<half_t>(s->a16);
     float *ainv = at<float>(s->a16_inv);
     const bool gemma = s->model_type == MODEL_GEMMA3;
-    Planes pending{nullptr, 0, 0, 0};                    // FFN output of the previous layer, not yet added
+    Planes pending{nullptr, 0, 0, 0, nullptr};                    // FFN output of the previous layer, not yet added
 
     for (int L = 0; L < s->NL; L++) {
         float *x_in = at<float>(s->xs, (size_t)(2 * L) * xsz), *x_mid = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
@@ -211,7 +212,7 @@ void forward_impl(SFTState *s, bool gather)
         gemm(s, a16, ainv, at<half_t>(s->wlm), s->V, D, at<float>(s->logits));
     } else {
         Planes p = gemm(s, a16, ainv, at<half_t>(s->wlm), s->V, D);
-        launch_reduce_planes(p.p, p.S, p.stride, p.ld, at<float>(s->logits), BN, s->V);
+        launch_reduce_planes(p.p, p.S, p.stride, p.ld, p.row_scale, at<float>(s->logits), BN, s->V);
     }
 }
 
