@@ -39,7 +39,10 @@ def cpu_baseline(cfg, budget_s=20.0):
     lora = model["lora"].copy()
     m, vv = np.zeros_like(lora), np.zeros_like(lora)
     t0 = time.perf_counter()
-    oracle.sft_train_step(small, used, lora, m, vv, 0, tok, tgt, 1e-4)
+    if cfg.R:
+        oracle.sft_train_step(small, used, lora, m, vv, 0, tok, tgt, 1e-4)
+    else:                                                  # full-parameter: forward + backward with F16 gradient accumulation
+        oracle.full_param_pass(small, used, oracle.new_grad_accum(used), tok=tok, tgt=tgt)
     dt = time.perf_counter() - t0
     scale = cfg.frozen_params / small.frozen_params
     est = dt * scale
@@ -93,23 +96,44 @@ def main():
     batches = [make_batch(cfg, seed=100 + i) for i in range(4)]
     lr = 1e-4
 
+    grpo = cfg.R == 0
+    if grpo:
+        # GRPO phases 3-4 (src/nn/fast_grpo.c:376-495): 4 completions of 128 tokens after a 32-token prompt,
+        # group-normalised N(0,1) advantages, old log-probabilities = the policy's own (ratio 1, clip inactive)
+        rng = np.random.default_rng(7)
+        G, p_len = 4, 32
+        prompt = rng.integers(0, cfg.V, p_len).astype(np.uint32)
+        comps = [rng.integers(0, cfg.V, cfg.seq - p_len).astype(np.uint32) for _ in range(G)]
+        r = rng.standard_normal(G).astype(np.float32)
+        adv = (r - r.mean()) / (r.std() + 1e-8)
+        zeros = [np.zeros(cfg.seq - p_len, dtype=np.float32) for _ in range(G)]
+        new_lp = st.grpo_apply_completions(prompt, comps, zeros, np.zeros(G, dtype=np.float32), 0.2, 0.0)
+        old = [new_lp[i, p_len:].copy() for i in range(G)]
+        lr = 1e-5
+        step = lambda i: st.grpo_apply_completions(prompt, comps, old, adv, 0.2, lr)
+        rows_per_step = G * cfg.seq
+    else:
+        step = lambda i: st.train_step(*batches[i % 4], lr)
+        rows_per_step = cfg.BN
     for i in range(args.warmup):
-        st.train_step(*batches[i % 4], lr)
+        step(i)
     L.metal_flush()
     t1 = time.perf_counter()
     loss = 0.0
     for i in range(args.steps):
-        loss = st.train_step(*batches[i % 4], lr)
+        loss = step(i)
     L.metal_flush()
     dt = time.perf_counter() - t1
     ms = dt / args.steps * 1e3
-    toks = cfg.BN * args.steps / dt
+    toks = rows_per_step * args.steps / dt
+    if grpo:
+        loss = float(np.mean(loss[:, 32:]))                # mean log-probability of the sampled tokens
 
     # dominant kernel: the weight-streaming GEMM, timed launch by launch with HIP events on the library's stream
     prof_steps = max(1, min(5, args.steps))
     L.hip_gemm_profile_enable(1)
     for i in range(prof_steps):
-        st.train_step(*batches[i % 4], lr)
+        step(i)
     import ctypes as C
     tms, wb = C.c_double(0), C.c_double(0)
     n = L.hip_gemm_profile_read(C.byref(tms), C.byref(wb))
@@ -117,17 +141,19 @@ def main():
     gbs = wb.value / (tms.value * 1e-3) / 1e9 if tms.value > 0 else 0.0
     roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "gemm_skinny_f16", "launches_per_step": n // prof_steps,
+                "kernel": "gemm_tiled_f16", "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                 "weight_bytes_per_step": wb.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}
     st.free()
 
-    out = {"metric": "SFT train tokens/s, Qwen3-4B LoRA r16 seq64; % of HBM-BW / MFMA peak",
+    metric = ("SFT train tokens/s, Qwen3-4B LoRA r16 seq64; % of HBM-BW / MFMA peak" if cfg.name == "c3_qwen3_4b_f16" else
+              "GRPO train tokens/s, full-parameter F16 accumulate + apply" if grpo else "SFT train tokens/s")
+    out = {"metric": metric,
            "value": round(toks, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "f16 weights x f16 activations, f32 accumulate", "data": "synthetic",
-           "config": {"workload": cfg.name, "rows_per_step": cfg.BN, "layers": cfg.NL, "lora_rank": cfg.R,
+           "config": {"workload": cfg.name, "rows_per_step": rows_per_step, "layers": cfg.NL, "lora_rank": cfg.R,
                       "frozen_params": cfg.frozen_params, "weight_format": cfg.weight_format},
            "roofline": roofline, "final_loss": round(float(loss), 5),
            "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}

@@ -118,7 +118,37 @@ int sft_get_n_kv_heads(SFTState *state);
 int sft_get_head_dim(SFTState *state);
 int sft_get_intermediate_size(SFTState *state);
 const float *sft_get_rope_thetas(SFTState *state);
-int sft_is_full_param(SFTState *state);
+int sft_is_full_param(SFTState *state);          /* 1 when the state was created with lora_rank 0 (sft_state_create_full) */
+const float *sft_get_token_emb(SFTState *state);  /* the caller's fp32 table, borrowed: it must outlive the state */
+MetalBuf *sft_get_final_norm_g(SFTState *state);
+/* Weight sharing accessors (src/nn/fast_sft.h:98-101).  The state keeps its matrices in the GEMM's own
+ * operand layout, so these hand out row-major F16 COPIES, refreshed on every call. */
+LayerW *sft_get_layers(SFTState *state);
+WMat *sft_get_lm_head(SFTState *state);
+
+/* ---- full-parameter mode (src/nn/fast_sft.h:20-39).  sft_train_step then runs forward, loss and
+ *      sft_backward_sgd(lr) (or accumulates, once sft_alloc_grad_accum was called); no AdamW. ---- */
+void sft_backward_sgd(SFTState *state, float lr);   /* W = half(W - lr dY^T X) per matrix, inside the backward */
+void sft_alloc_grad_accum(SFTState *state);         /* zeroed F16 accumulators mirroring every weight */
+void sft_backward_accum(SFTState *state);           /* G = half(G + dY^T X), weights untouched */
+void sft_apply_grad_sgd(SFTState *state, float lr); /* W = half(W - lr G), G = 0; flushes */
+void sft_save_full_checkpoint(SFTState *state, const char *path);   /* "FULL" file, src/nn/fast_sft.c:1286-1340 */
+/* Extension: row-major F16 bits of one matrix.  which: 0..6 = q, k, v, o, gate, up, down of `layer`,
+ * 7 = lm_head.  source: 0 = the weight, 1 = its transposed image (same values), 2 = the accumulator. */
+void sft_copy_matrix_f16(SFTState *state, int layer, int which, int source, uint16_t *dst);
+
+/* ---- GRPO phases 3-4 (src/nn/fast_grpo.c:376-495) over completions sampled elsewhere ---- */
+typedef struct {
+    const uint32_t *prompt; int prompt_len;
+    int group_size;                       /* G */
+    const uint32_t *const *gen_tokens;    /* [G] arrays of gen_lengths[i] sampled tokens */
+    const int *gen_lengths;
+    const float *const *gen_logprobs;     /* log-probabilities at sampling time */
+    const float *advantages;              /* [G], group-normalised */
+    float clip_eps;
+    int accurate;                         /* full-parameter only: 1 = accumulate, apply once; 0 = SGD per completion with lr/G */
+} GRPOCompletions;
+void grpo_apply_completions(SFTState *state, const GRPOCompletions *c, float lr, float *new_logprobs);
 /* "LORA" adapter file, src/nn/fast_sft.c:1255-1285 */
 void sft_save_lora(SFTState *state, const char *path);
 

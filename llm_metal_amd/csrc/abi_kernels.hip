@@ -387,6 +387,10 @@ __global__ __launch_bounds__(256) void k_float_matmul(const float *__restrict__ 
     if (row < M && col < N) C[(size_t)row * N + col] = s;
 }
 
+// The F16 update rules below are separate fp32 operations (multiply, add, one rounding to F16);
+// a fused multiply-add would change results at rounding ties.
+#pragma clang fp contract(off)
+
 // f16_sgd_fused / f16_grad_accum, shaders/q8_kernels.metal:1097-1125, 1164-1190:
 // T[M,N] (F16) = half(float(T) + alpha * sum_k dY[k,M] X[k,N])
 __global__ __launch_bounds__(256) void k_f16_rank_update(half_t *__restrict__ T, const float *__restrict__ dY,

@@ -1,0 +1,244 @@
+// Full-parameter mode: weight gradients dW = dY^T X on the matrix cores, straight
+// into the tiled F16 images the GEMMs read.
+//
+// Replaces f16_grad_accum / f16_sgd_fused / f16_sgd_apply of
+// shaders/q8_kernels.metal:1097-1125, 1164-1206 as the fused pipeline uses them
+// (src/nn/fast_sft.c:778-946, 1021-1039).
+//
+// The contraction of a weight gradient runs over the tokens, so both operands are
+// first transposed: the token-major fp16 operand rows that the backward already
+// holds (each with its own row factor) become feature-major rows with one
+// power-of-two factor per FEATURE — factors of the output's row and column, which
+// can be taken out of the sum.  k_wgrad then forms 64 x 64 blocks of dW per wave
+// with v_mfma_f32_32x32x16_f16 and does the read-modify-write of the F16 target
+// (accumulator G or weight W) in the operand layout of gemm.h, 8 bytes per lane,
+// 512 contiguous bytes per wave instruction.  The kernel is bound by that
+// read-modify-write: 4 bytes of HBM traffic per weight and call.
+#include "backend.h"
+#include "devutil.h"
+#include "gemm.h"
+#include "fused.h"
+
+using namespace lmhip;
+
+// The F16 update rules are specified as separate fp32 operations (multiply, then add, then one
+// rounding to F16); a fused multiply-add would change results at rounding ties.
+#pragma clang fp contract(off)
+
+namespace {
+
+#define LAUNCH(kern, grid, block, lds, ...) do { \
+    hipLaunchKernelGGL(kern, grid, block, lds, stream(), __VA_ARGS__); HIP_CHECK(hipGetLastError()); } while (0)
+
+// in:  tiled [T tokens, F features] fp16, value(t, f) = in[t][f] * in_inv[t]
+// out: tiled [F, T] fp16, value(f, t) = out[f][t] * out_inv[f]; zero in the K (token) padding and in
+//      rows >= F; out_inv has room for a multiple of 64 entries and gets 0 beyond F.
+// One workgroup per block of 64 features; two sweeps over the tokens (row maxima, then the data).
+__global__ __launch_bounds__(256) void k_transpose_scaled(const half8 *__restrict__ in, const float *__restrict__ in_inv,
+                                                           int T, int F, half8 *__restrict__ out, float *__restrict__ out_inv)
+{
+    __shared__ float amax[64], scl[64];
+    __shared__ half_t t[64][72];
+    const int tid = threadIdx.x, fb = blockIdx.x;
+    const int KbIn = tiled_kb(F), TbIn = tiled_rb(T), KbOut = tiled_kb(T), FbOut = tiled_rb(F);
+    if (tid < 64) amax[tid] = 0.f;
+    __syncthreads();
+    {
+        const int j = tid >> 6, lp = tid & 63, f0 = (lp >> 5) * 32 + 8 * j;
+        for (int tb = 0; tb < TbIn; tb++) {
+            const int token = tb * 32 + (lp & 31);
+            const half8 h = in[((size_t)tb * KbIn + fb) * 256 + tid];
+            const float s = token < T ? in_inv[token] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v = fabsf(h2f(h[e]) * s);
+                if (v > 0.f) atomicMax(reinterpret_cast<unsigned *>(&amax[f0 + e]), __float_as_uint(v));
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < 64) {
+        const int f = fb * 64 + tid;
+        const float s = f < F ? row_scale_for(amax[tid]) : 0.f;
+        scl[tid] = s;
+        out_inv[f] = f < F ? 1.0f / s : 0.f;
+    }
+    __syncthreads();
+    for (int tb2 = 0; tb2 < KbOut; tb2++) {
+        for (int q = tid; q < 512; q += 256) {
+            const int th = q >> 8, qq = q & 255, tile = tb2 * 2 + th;
+            const int j = qq >> 6, lp = qq & 63, tl = th * 32 + (lp & 31), f0 = (lp >> 5) * 32 + 8 * j;
+            const int token = tb2 * 64 + tl;
+            half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
+            float s = 0.f;
+            if (tile < TbIn && token < T) { h = in[((size_t)tile * KbIn + fb) * 256 + qq]; s = in_inv[token]; }
+#pragma unroll
+            for (int e = 0; e < 8; e++) t[tl][f0 + e] = f2h(h2f(h[e]) * s * scl[f0 + e]);
+        }
+        __syncthreads();
+        for (int q = tid; q < 512; q += 256) {
+            const int th = q >> 8, qq = q & 255, rowtile = fb * 2 + th;
+            if (rowtile >= FbOut) continue;
+            const int j = qq >> 6, lp = qq & 63, fl = th * 32 + (lp & 31), k0 = (lp >> 5) * 32 + 8 * j;
+            half8 o;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = t[k0 + e][fl];
+            out[((size_t)rowtile * KbOut + tb2) * 256 + qq] = o;
+        }
+        __syncthreads();
+    }
+}
+
+// Target[m][n] (tiled [M_out, N_in] F16) <- half(float(Target) + alpha * sum_t Y[t][m] X[t][n])
+// with XT = tiled [N_in, T], YT = tiled [M_out, T] and their row factors.  SGD: alpha = -lr, else 1.
+// grid: x = ceil(Kb / 4) (each wave one 64-wide column block), y = ceil(Mb / 2); block 256.
+// The MFMA's first operand supplies the rows of its result, so feeding X there puts four
+// consecutive n into each lane's registers: exactly the 8-byte groups of the tiled target.
+template <int SGD>
+__global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, const float *__restrict__ x_inv,
+                                               const half8 *__restrict__ YT, const float *__restrict__ y_inv,
+                                               half_t *__restrict__ target, int M_out, int N_in, int Kt, float lr)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l31 = lane & 31, h = lane >> 5;
+    const int KbG = tiled_kb(N_in), MbG = tiled_rb(M_out), NbX = tiled_rb(N_in);
+    const int nk = blockIdx.x * 4 + wave, mb0 = blockIdx.y * 2;
+    if (nk >= KbG) return;
+    const half8 *xp[2], *yp[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        xp[i] = XT + (size_t)min(nk * 2 + i, NbX - 1) * Kt * 256 + lane;
+        yp[i] = YT + (size_t)min(mb0 + i, MbG - 1) * Kt * 256 + lane;
+    }
+    float16v acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+    for (int kt = 0; kt < Kt; kt++) {
+        const size_t o = (size_t)kt * 256;
+        half8 x[2][4], y[2][4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) { x[i][j] = xp[i][o + j * 64]; y[i][j] = yp[i][o + j * 64]; }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int nh = 0; nh < 2; nh++)
+                    acc[mt][nh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[nh][j], y[mt][j], acc[mt][nh], 0, 0, 0);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+        const int m = (mb0 + mt) * 32 + l31;
+        if (mb0 + mt >= MbG || m >= M_out) continue;
+        const float sy = y_inv[m];
+#pragma unroll
+        for (int nh = 0; nh < 2; nh++)
+#pragma unroll
+            for (int j4 = 0; j4 < 4; j4++) {
+                const int n0 = nk * 64 + nh * 32 + 8 * j4 + 4 * h;
+                if (n0 >= N_in) continue;
+                const size_t addr = ((((size_t)(mb0 + mt) * KbG + nk) * 4 + j4) * 64 + nh * 32 + l31) * 8 + 4 * h;
+                half4 g = *reinterpret_cast<half4 *>(target + addr);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    if (n0 + i >= N_in) continue;
+                    const float a = acc[mt][nh][4 * j4 + i] * sy * x_inv[n0 + i];
+                    g[i] = SGD ? f2h(h2f(g[i]) - lr * a) : f2h(h2f(g[i]) + a);        // contraction is off in this file
+                }
+                *reinterpret_cast<half4 *>(target + addr) = g;
+            }
+    }
+}
+
+// 64 x 64 blocks of W (tiled [Mo, Ni]):  if G: W = half(W - lr * G), G = 0 (f16_sgd_apply);
+// then the block is written, transposed, into WT (tiled [Ni, Mo]).
+// grid: x = K blocks of W, y = ceil(row tiles / 2); block 256.
+__global__ __launch_bounds__(256) void k_apply_retile(half8 *__restrict__ W, half8 *__restrict__ G, half8 *__restrict__ WT,
+                                                       int Mo, int Ni, float lr)
+{
+    __shared__ half_t t[64][72];
+    const int tid = threadIdx.x, bx = blockIdx.x, by = blockIdx.y;
+    const int KbW = tiled_kb(Ni), MbW = tiled_rb(Mo), KbT = tiled_kb(Mo), NbT = tiled_rb(Ni);
+    for (int q = tid; q < 512; q += 256) {
+        const int th = q >> 8, qq = q & 255, mbt = by * 2 + th;
+        const int j = qq >> 6, lp = qq & 63, ml = th * 32 + (lp & 31), n0 = (lp >> 5) * 32 + 8 * j;
+        half8 w = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (mbt < MbW) {
+            const size_t a = ((size_t)mbt * KbW + bx) * 256 + qq;
+            w = W[a];
+            if (G) {
+                const half8 g = G[a];
+#pragma unroll
+                for (int e = 0; e < 8; e++) w[e] = f2h(h2f(w[e]) - lr * h2f(g[e]));   // two roundings: contraction is off
+                W[a] = w;
+                const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                G[a] = z;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[ml][n0 + e] = w[e];
+    }
+    __syncthreads();
+    for (int q = tid; q < 512; q += 256) {
+        const int th = q >> 8, qq = q & 255, nbt = bx * 2 + th;
+        if (nbt >= NbT) continue;
+        const int j = qq >> 6, lp = qq & 63, nl = th * 32 + (lp & 31), m0 = (lp >> 5) * 32 + 8 * j;
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = t[m0 + e][nl];
+        WT[((size_t)nbt * KbT + by) * 256 + qq] = o;
+    }
+}
+
+// dst row-major F16 [rows, cols] <- tiled image: element (r, c) from tiled(row_off + r, k_off + c),
+// or from tiled(row_off + c, k_off + r) when the image holds the transposed matrix.
+__global__ void k_untile_f16(const half_t *__restrict__ src, int Kb, int row_off, int k_off, int transpose,
+                             int rows, int cols, half_t *__restrict__ dst)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)rows * cols) return;
+    const int r = (int)(idx / cols), c = (int)(idx % cols);
+    dst[idx] = transpose ? src[tiled_index(row_off + c, k_off + r, Kb)] : src[tiled_index(row_off + r, k_off + c, Kb)];
+}
+
+}  // namespace
+
+namespace lmhip {
+
+void launch_transpose_scaled(const half_t *in_tiled, const float *in_inv, int T, int F, half_t *out_tiled, float *out_inv)
+{
+    if (T <= 0 || F <= 0) return;
+    LAUNCH(k_transpose_scaled, dim3(tiled_kb(F)), dim3(256), 0, reinterpret_cast<const half8 *>(in_tiled), in_inv, T, F,
+           reinterpret_cast<half8 *>(out_tiled), out_inv);
+}
+
+void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,
+                  int M_out, int N_in, int T, int sgd, float lr)
+{
+    if (M_out <= 0 || N_in <= 0 || T <= 0) return;
+    const dim3 grid((tiled_kb(N_in) + 3) / 4, (tiled_rb(M_out) + 1) / 2);
+    const half8 *x8 = reinterpret_cast<const half8 *>(XT), *y8 = reinterpret_cast<const half8 *>(YT);
+    if (sgd) LAUNCH(k_wgrad<1>, grid, dim3(256), 0, x8, x_inv, y8, y_inv, target_tiled, M_out, N_in, tiled_kb(T), lr);
+    else     LAUNCH(k_wgrad<0>, grid, dim3(256), 0, x8, x_inv, y8, y_inv, target_tiled, M_out, N_in, tiled_kb(T), lr);
+}
+
+void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr)
+{
+    if (M_out <= 0 || N_in <= 0) return;
+    LAUNCH(k_apply_retile, dim3(tiled_kb(N_in), (tiled_rb(M_out) + 1) / 2), dim3(256), 0, reinterpret_cast<half8 *>(W_tiled),
+           reinterpret_cast<half8 *>(G_tiled), reinterpret_cast<half8 *>(WT_tiled), M_out, N_in, lr);
+}
+
+void launch_untile_f16(const half_t *src_tiled, int Kb, int row_off, int k_off, int transpose, int rows, int cols, half_t *dst)
+{
+    const size_t n = (size_t)rows * cols;
+    if (!n) return;
+    LAUNCH(k_untile_f16, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, src_tiled, Kb, row_off, k_off, transpose, rows, cols, dst);
+}
+
+}  // namespace lmhip

@@ -21,6 +21,7 @@ struct Planes {
 struct NormRowsArgs {
     // source of the residual stream row: token gather (emb != null) or x_prev
     const float *emb; const uint32_t *tokens; float emb_scale;
+    int n_valid;                  // gather only: rows >= n_valid read as zero (0 = every row is valid)
     const float *x_prev;
     // optional branch added to it: planes, optionally RMS-normalised with g_branch first
     Planes branch; const float *g_branch; float *branch_raw_out;
@@ -104,6 +105,8 @@ void launch_norm_bwd_rows(const NormBwdArgs &a, int rows);
 struct CeArgs {
     const float *logits; int V; const uint32_t *targets; float *losses;
     half_t *dl16; float *inv_scale; int rows_total;     // tiled [rows, V]
+    // policy-gradient variant (grpo != 0): targets are the sampled actions; losses is not written
+    int grpo; const float *old_lp, *advs; float *new_lp; float clip_eps, dl_scale;
 };
 void launch_ce_rows(const CeArgs &a, int rows);
 
@@ -124,5 +127,16 @@ void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_laye
                         size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size);
 
 void launch_fill_f32(float *p, float v, size_t n);
+
+// ---- full-parameter mode (fullparam.hip) ----
+// out (tiled [F, T]) and out_inv[F] <- transposed in (tiled [T, F]) with in_inv[T]; out_inv needs tiled_kb(F)*64 floats
+void launch_transpose_scaled(const half_t *in_tiled, const float *in_inv, int T, int F, half_t *out_tiled, float *out_inv);
+// target (tiled [M_out, N_in] F16) <- half(target + alpha * Y^T X), XT/YT = transposed operands over T tokens;
+// sgd: alpha = -lr (f16_sgd_fused), else alpha = 1 (f16_grad_accum)
+void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,
+                  int M_out, int N_in, int T, int sgd, float lr);
+// G != null: W = half(W - lr G), G = 0 (f16_sgd_apply); always: WT (tiled [N_in, M_out]) <- W^T
+void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr);
+void launch_untile_f16(const half_t *src_tiled, int Kb, int row_off, int k_off, int transpose, int rows, int cols, half_t *dst);
 
 }  // namespace lmhip

@@ -86,13 +86,14 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
     const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
-    const float *base = a.emb ? a.emb + (size_t)a.tokens[r] * D : a.x_prev + r * D;
+    const bool padded = a.emb && a.n_valid > 0 && (int)r >= a.n_valid;      // zero rows past the sequence
+    const float *base = a.emb ? a.emb + (size_t)(padded ? 0u : a.tokens[r]) * D : a.x_prev + r * D;
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         const int v = threadIdx.x + t * RB;
         x[t] = b[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (v < nv) {
-            x[t] = ld4(base + 4 * v);
+            if (!padded) x[t] = ld4(base + 4 * v);
             if (a.emb && a.emb_scale != 1.0f) { x[t].x *= a.emb_scale; x[t].y *= a.emb_scale; x[t].z *= a.emb_scale; x[t].w *= a.emb_scale; }
             if (a.branch.S > 0) b[t] = planes_at4(a.branch, r, 4 * v);
         }
@@ -711,7 +712,8 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 // ------------------------------------------------------------------ loss rows
 // softmax_ce_train + scale(1/BN), shaders/q8_kernels.metal:646-690 and
 // src/nn/fast_sft.c:754-760.  The gradient is written once, as the lm_head dX GEMM's
-// fp16 operand: (softmax - onehot) * 1024 with row factor (1/BN) / 1024.
+// fp16 operand: (softmax - onehot) * 1024 with row factor (1/BN) / 1024.  With a.grpo the row
+// factor carries the policy-gradient weight instead (src/nn/fast_grpo.c:437-452).
 __global__ __launch_bounds__(1024) void k_ce_rows(CeArgs a)
 {
     __shared__ float sm[16];
@@ -730,10 +732,21 @@ __global__ __launch_bounds__(1024) void k_ce_rows(CeArgs a)
     }
     sum = block_sum(sum, sm);
     const float lse = logf(sum) + mx;
-    if (threadIdx.x == 0) {
+    // coefficient of (softmax - onehot): 1/BN for the cross-entropy; w * ratio * dl_scale for the
+    // PPO-clip policy gradient (grpo_policy_grad, shaders/q8_kernels.metal:741-760)
+    float coef = 1.0f / (float)a.rows_total;
+    if (a.grpo) {
+        const float new_lp = lg[tgt] - lse;
+        const float ratio = expf(new_lp - a.old_lp[r]);
+        const float clipped = fminf(fmaxf(ratio, 1.0f - a.clip_eps), 1.0f + a.clip_eps);
+        const float adv = a.advs[r];
+        const float w = (adv >= 0.f) ? ((ratio <= clipped) ? -adv : 0.f) : ((ratio >= clipped) ? -adv : 0.f);
+        coef = w * ratio * a.dl_scale;
+        if (threadIdx.x == 0) a.new_lp[r] = new_lp;
+    } else if (threadIdx.x == 0) {
         a.losses[r] = lse - lg[tgt];
-        a.inv_scale[r] = (1.0f / (float)a.rows_total) * (1.0f / 1024.0f);
     }
+    if (threadIdx.x == 0) a.inv_scale[r] = coef * (1.0f / 1024.0f);
     const int Kb = tiled_kb(V);
     for (int c = threadIdx.x; c < Kb * 8; c += blockDim.x) {
         half8 hv;

@@ -62,7 +62,25 @@ struct SFTState {
     MetalBuf *logits, *dlogits, *dl16, *dl_inv;
     MetalBuf *dx[2], *dO_red, *dscore, *dq, *dk, *dv, *dq_f, *dh;
     size_t planes_cap;
+
+    // full-parameter mode (lora_rank == 0): the GEMM operands of the forward are kept per layer, because
+    // every one of them is the X of a weight gradient dW = dY^T X
+    int full_param;
+    const float *token_emb_host;         // the caller's table, borrowed (src/nn/fast_sft.c:239)
+    MetalBuf *ln2_16, *ln2_inv, *act16, *act_inv, *attn16, *lnf16, *lnf_inv;
+    size_t st_act, st_attn;
+    MetalBuf *xT, *xT_inv, *yT, *yT_inv; // transposed operands of the weight gradient being formed
+    MetalBuf *gqkv, *go, *ggu, *gd, *glm;   // F16 gradient accumulators, tiled like the weights (sft_alloc_grad_accum)
+    MetalBuf *grpo_old_lp, *grpo_advs, *grpo_new_lp;   // host-visible [BN] inputs/outputs of the policy gradient
+    float *grpo_old_lp_cpu, *grpo_advs_cpu, *grpo_new_lp_cpu;
+    MetalBuf *lora_acc;                  // LoRA gradients summed over the completions of a GRPO group
+    std::vector<LayerW> layers_out;      // row-major F16 copies handed out by sft_get_layers
+    std::vector<WMat> wmats_out;
+    std::vector<MetalBuf *> views_out;
+    WMat lm_head_out;
 };
+
+enum { BWD_LORA = 0, BWD_ACCUM = 1, BWD_SGD = 2 };
 
 namespace {
 
@@ -121,7 +139,7 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const half_t *W, int
     return Planes{P, p.S, stride, N, out ? nullptr : inv};
 }
 
-void forward_impl(SFTState *s, bool gather)
+void forward_impl(SFTState *s, bool gather, int n_valid = 0)
 {
     const int BN = s->BN, D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R;
     const size_t xsz = (size_t)BN * D;
@@ -138,7 +156,7 @@ void forward_impl(SFTState *s, bool gather)
         // x_in = x (+ previous FFN branch); ln1 = RN(x_in; g_in)        [src/nn/fast_sft.c:631-635, 732-740]
         NormRowsArgs n1{};
         if (L == 0) {
-            if (gather) { n1.emb = at<float>(s->emb); n1.tokens = at<uint32_t>(s->tokens); n1.emb_scale = s->emb_scale; }
+            if (gather) { n1.emb = at<float>(s->emb); n1.tokens = at<uint32_t>(s->tokens); n1.emb_scale = s->emb_scale; n1.n_valid = n_valid; }
             else n1.x_prev = at<float>(s->x_in_host);
         } else {
             n1.x_prev = at<float>(s->xs, (size_t)(2 * L - 1) * xsz);
@@ -172,29 +190,35 @@ void forward_impl(SFTState *s, bool gather)
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
         aa.scale = 1.0f / sqrtf((float)s->hd);
         aa.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
-        aa.out16 = a16;
+        // full-parameter mode keeps the three FFN/attention GEMM operands of every layer
+        half_t *attn16 = s->full_param ? at<half_t>(s->attn16, L * s->st_attn) : a16;
+        half_t *ln2 = s->full_param ? at<half_t>(s->ln2_16, L * s->st_ln1) : a16;
+        float *ln2inv = s->full_param ? at<float>(s->ln2_inv, (size_t)L * BN) : ainv;
+        half_t *act16 = s->full_param ? at<half_t>(s->act16, L * s->st_act) : a16;
+        float *actinv = s->full_param ? at<float>(s->act_inv, (size_t)L * BN) : ainv;
+        aa.out16 = attn16;
         launch_attn_fwd(aa);
 
         // o = attn Wo^T; x_mid = x_in + o (Qwen3) | x_in + RN(o; g_post_attn) (Gemma3); ln2 = RN(x_mid; g_ffn_in)   [:696-711]
-        Planes po = gemm(s, a16, at<float>(s->ones), at<half_t>(s->wo, L * s->st_o), D, qd);
+        Planes po = gemm(s, attn16, at<float>(s->ones), at<half_t>(s->wo, L * s->st_o), D, qd);
         NormRowsArgs n2{};
         n2.x_prev = x_in; n2.branch = po;
         if (gemma) { n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); n2.branch_raw_out = at<float>(s->o_raw, (size_t)L * xsz); }
         n2.x_out = x_mid;
         n2.g_norm = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
-        n2.ln16 = a16; n2.inv_scale = ainv; n2.D = D; n2.eps = s->eps;
+        n2.ln16 = ln2; n2.inv_scale = ln2inv; n2.D = D; n2.eps = s->eps;
         launch_norm_rows(n2, BN);
 
         // [gate | up] = ln2 [Wg; Wu]^T; act = silu|gelu(gate) * up              [:715-725]
-        Planes pg = gemm(s, a16, ainv, at<half_t>(s->wgu, L * s->st_gu), 2 * IS, D);
+        Planes pg = gemm(s, ln2, ln2inv, at<half_t>(s->wgu, L * s->st_gu), 2 * IS, D);
         GluArgs ga{};
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
         ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
-        ga.out16 = a16; ga.inv_scale = ainv;
+        ga.out16 = act16; ga.inv_scale = actinv;
         launch_glu_fwd(ga, BN);
 
         // ff = act Wd^T, added by the next row kernel                          [:730-740]
-        pending = gemm(s, a16, ainv, at<half_t>(s->wd, L * s->st_d), D, IS);
+        pending = gemm(s, act16, actinv, at<half_t>(s->wd, L * s->st_d), D, IS);
     }
 
     // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
@@ -205,19 +229,41 @@ void forward_impl(SFTState *s, bool gather)
     if (gemma) { nf.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); nf.branch_raw_out = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); }
     nf.x_out = at<float>(s->xs, (size_t)(2 * L) * xsz);
     nf.g_norm = at<float>(s->g_final);
-    nf.ln16 = a16; nf.inv_scale = ainv; nf.D = D; nf.eps = s->eps;
+    half_t *lnf = s->full_param ? at<half_t>(s->lnf16) : a16;
+    float *lnfinv = s->full_param ? at<float>(s->lnf_inv) : ainv;
+    nf.ln16 = lnf; nf.inv_scale = lnfinv; nf.D = D; nf.eps = s->eps;
     launch_norm_rows(nf, BN);
     GemmPlan pl = plan_gemm(BN, s->V, D);
     if (pl.S == 1) {
-        gemm(s, a16, ainv, at<half_t>(s->wlm), s->V, D, at<float>(s->logits));
+        gemm(s, lnf, lnfinv, at<half_t>(s->wlm), s->V, D, at<float>(s->logits));
     } else {
-        Planes p = gemm(s, a16, ainv, at<half_t>(s->wlm), s->V, D);
+        Planes p = gemm(s, lnf, lnfinv, at<half_t>(s->wlm), s->V, D);
         launch_reduce_planes(p.p, p.S, p.stride, p.ld, p.row_scale, at<float>(s->logits), BN, s->V);
     }
 }
 
-// Backward from the fp16 loss gradient in dl16 / dl_inv.
-void backward_impl(SFTState *s)
+// dW = dY^T X for one (fused) matrix [M_out, N_in] at element offsets w_off / wt_off of its arenas:
+// added into the accumulator (BWD_ACCUM) or applied at once to both weight images (BWD_SGD).
+void weight_grad(SFTState *s, int mode, float lr, const half_t *dY16, const float *dy_inv, int M_out,
+                 const half_t *X16, const float *x_inv, int N_in,
+                 MetalBuf *W, MetalBuf *WT, MetalBuf *G, size_t w_off, size_t wt_off)
+{
+    if (mode == BWD_ACCUM && !G) { fprintf(stderr, "[fast_sft] gradient accumulators are not allocated\n"); abort(); }
+    launch_transpose_scaled(dY16, dy_inv, s->BN, M_out, at<half_t>(s->yT), at<float>(s->yT_inv));
+    launch_transpose_scaled(X16, x_inv, s->BN, N_in, at<half_t>(s->xT), at<float>(s->xT_inv));
+    if (mode == BWD_ACCUM) {
+        launch_wgrad(at<half_t>(s->xT), at<float>(s->xT_inv), at<half_t>(s->yT), at<float>(s->yT_inv),
+                     at<half_t>(G, w_off), M_out, N_in, s->BN, 0, 0.f);
+    } else {
+        launch_wgrad(at<half_t>(s->xT), at<float>(s->xT_inv), at<half_t>(s->yT), at<float>(s->yT_inv),
+                     at<half_t>(W, w_off), M_out, N_in, s->BN, 1, lr);
+        launch_apply_retile(at<half_t>(W, w_off), nullptr, at<half_t>(WT, wt_off), M_out, N_in, 0.f);
+    }
+}
+
+// Backward from the fp16 loss gradient in dl16 / dl_inv.  mode: BWD_LORA (adapter gradients),
+// BWD_ACCUM / BWD_SGD (full-parameter: sft_backward_accum / sft_backward_sgd, src/nn/fast_sft.c:984-986).
+void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
 {
     const int BN = s->BN, D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R, NL = s->NL;
     const size_t xsz = (size_t)BN * D;
@@ -228,6 +274,9 @@ void backward_impl(SFTState *s)
 
     // dx = RNB(x_final, dlogits Wlm; g_final)                                [:777-790]
     Planes p = gemm(s, at<half_t>(s->dl16), at<float>(s->dl_inv), at<half_t>(s->wlmT), D, s->V);
+    if (mode != BWD_LORA)                                                     // [:778-786]
+        weight_grad(s, mode, lr, at<half_t>(s->dl16), at<float>(s->dl_inv), s->V, at<half_t>(s->lnf16), at<float>(s->lnf_inv), D,
+                    s->wlm, s->wlmT, s->glm, 0, 0);
     NormBwdArgs nb{};
     nb.dy = p; nb.x_saved = at<float>(s->xs, (size_t)(2 * NL) * xsz); nb.g = at<float>(s->g_final);
     nb.eps = s->eps; nb.D = D; nb.dx_prev = nullptr; nb.dx_out = at<float>(s->dx[cur]); nb.clamp = 0.f;
@@ -238,12 +287,18 @@ void backward_impl(SFTState *s)
     for (int L = NL - 1; L >= 0; L--) {
         // FFN: d act = d Wd; (dgate, dup); dln2 = dgate Wg + dup Wu; dx += RNB(x_mid, dln2)   [:798-874]
         Planes pd = gemm(s, a16, ainv, at<half_t>(s->wdT, L * s->st_dT), IS, D);
+        if (mode != BWD_LORA)                                                 // [:804-811, 842-849]
+            weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->act16, L * s->st_act), at<float>(s->act_inv, (size_t)L * BN), IS,
+                        s->wd, s->wdT, s->gd, L * s->st_d, L * s->st_dT);
         GluArgs gb{};
         gb.in = pd; gb.IS = IS; gb.gelu = gemma;
         gb.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); gb.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
         gb.out16 = a16; gb.inv_scale = ainv;
         launch_glu_bwd(gb, BN);
         Planes pgu = gemm(s, a16, ainv, at<half_t>(s->wguT, L * s->st_guT), D, 2 * IS);
+        if (mode != BWD_LORA)                                                 // gate and up as one matrix [:817-833, 853-869]
+            weight_grad(s, mode, lr, a16, ainv, 2 * IS, at<half_t>(s->ln2_16, L * s->st_ln1), at<float>(s->ln2_inv, (size_t)L * BN), D,
+                        s->wgu, s->wguT, s->ggu, L * s->st_gu, L * s->st_guT);
         NormBwdArgs n2{};
         n2.dy = pgu; n2.x_saved = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
         n2.g = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
@@ -255,6 +310,9 @@ void backward_impl(SFTState *s)
 
         // attention: dO = d Wo; dq, dk, dv                                    [:877-911]
         Planes pdo = gemm(s, a16, ainv, at<half_t>(s->woT, L * s->st_oT), qd, D);
+        if (mode != BWD_LORA)                                                 // [:883-901]
+            weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->attn16, L * s->st_attn), at<float>(s->ones), qd,
+                        s->wo, s->woT, s->go, L * s->st_o, L * s->st_oT);
         AttnBwdArgs ab{};
         ab.dO = pdo;
         ab.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
@@ -289,6 +347,12 @@ void backward_impl(SFTState *s)
             lg.sq_slots = at<float>(s->sq_slots, (size_t)L * s->slots_per_layer);
             launch_lora_grads(lg);
         }
+
+        // full-parameter: W_q, W_k, W_v are updated BEFORE the dX product, which then multiplies with the
+        // new weights in SGD mode, as the reference does                       [:922-946]
+        if (mode != BWD_LORA)
+            weight_grad(s, mode, lr, a16, ainv, s->nq_ext, at<half_t>(s->ln1_16, (size_t)L * s->st_ln1), at<float>(s->ln1_inv, (size_t)L * BN), D,
+                        s->wqkv, s->wqkvT, s->gqkv, L * s->st_qkv, L * s->st_qkvT);
 
         // dln1 = [dq|dk|dv|dh] [Wq;Wk;Wv;A_q;A_v]; dx += RNB(x_in, dln1; g_in); clamp     [:956-980]
         Planes pl = gemm(s, a16, ainv, at<half_t>(s->wqkvT, L * s->st_qkvT), D, s->nq_ext);
@@ -365,6 +429,8 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->emb_scale = m->model_type == MODEL_GEMMA3 ? sqrtf((float)m->d_model) : 1.0f;   // :302
     s->step_count = 0;
     s->weight_format = weight_format;
+    s->full_param = lora_rank == 0;                        // sft_state_create_full, src/nn/fast_sft.c:402-410
+    s->token_emb_host = m->token_emb;
     s->rope_thetas.assign(m->rope_thetas, m->rope_thetas + s->NL);
     const int D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R, NL = s->NL, BN = s->BN, V = s->V;
     if ((s->hd & 3) || (s->Hq % s->Hkv) || (D & 3) || (IS & 3) || (V & 3) || (lora_rank & 1) || lora_rank > 16 || (!weight_format && ((D & 31) || (IS & 31) || (qd & 31)))) {
@@ -499,6 +565,22 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf((size_t)BN * kd);
     s->dq_f = fbuf((size_t)BN * qd); s->dh = fbuf((size_t)BN * (R ? 2 * R : 1));
 
+    // ---- full-parameter mode: kept GEMM operands and the transposed pair of one weight gradient ----
+    s->st_act = tiled_elems(BN, IS); s->st_attn = tiled_elems(BN, qd);
+    if (s->full_param) {
+        s->ln2_16 = hbuf((size_t)NL * s->st_ln1); s->ln2_inv = fbuf((size_t)NL * BN);
+        s->act16 = hbuf((size_t)NL * s->st_act);  s->act_inv = fbuf((size_t)NL * BN);
+        s->attn16 = hbuf((size_t)NL * s->st_attn);
+        s->lnf16 = hbuf(s->st_ln1); s->lnf_inv = fbuf(BN);
+        int maxy = V > 2 * IS ? V : 2 * IS;
+        if (s->nq_ext > maxy) maxy = s->nq_ext;
+        if (D > maxy) maxy = D;
+        int maxx = IS > qd ? IS : qd;
+        if (D > maxx) maxx = D;
+        s->yT = hbuf(tiled_elems(maxy, BN)); s->yT_inv = fbuf((size_t)tiled_kb(maxy) * 64);
+        s->xT = hbuf(tiled_elems(maxx, BN)); s->xT_inv = fbuf((size_t)tiled_kb(maxx) * 64);
+    }
+
     // the fused QKV weight and its transpose carry fp16 images of A_q, A_v
     refresh_shadow(s);
     metal_flush();
@@ -518,8 +600,13 @@ void sft_state_free(SFTState *s)
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
                        s->gate_pre, s->up_val, s->tq, s->tv, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->ones, s->planes,
                        s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
-                       s->dq, s->dk, s->dv, s->dq_f, s->dh};
+                       s->dq, s->dk, s->dv, s->dq_f, s->dh,
+                       s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
+                       s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
+                       s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf};
+    for (MetalBuf *b : s->views_out) metal_buf_free(b);
     for (MetalBuf *b : all) metal_buf_free(b);
+    for (WMat &w : s->wmats_out) metal_buf_free(w.mbuf);
     delete s;
     fast_metal_shutdown();
 }
@@ -534,7 +621,8 @@ void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uin
     ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
     ce.dl16 = at<half_t>(s->dl16); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
     launch_ce_rows(ce, s->BN);
-    backward_impl(s);
+    if (s->full_param) backward_impl(s, s->gqkv ? BWD_ACCUM : BWD_SGD, lr);     // src/nn/fast_sft.c:1136-1140 with :778-786
+    else backward_impl(s);
     enqueue_update(s);
 }
 
@@ -558,11 +646,97 @@ void forward_to_logits(SFTState *s)
     forward_impl(s, false);
 }
 
-void sft_backward(SFTState *s)
+static void backward_from_dlogits(SFTState *s, int mode, float lr)
 {
     MetalBuf *dl = sft_get_dlogits(s);
     launch_rows_to_f16(at<float>(dl), s->V, at<half_t>(s->dl16), at<float>(s->dl_inv), s->BN, s->V);
-    backward_impl(s);
+    backward_impl(s, mode, lr);
+}
+
+// sft_backward / sft_backward_sgd / sft_backward_accum, src/nn/fast_sft.c:984-986: all three run
+// sft_backward_ex, whose branch depends on the state (LoRA | accumulators allocated | fused SGD).
+void sft_backward(SFTState *s) { backward_from_dlogits(s, !s->full_param ? BWD_LORA : (s->gqkv ? BWD_ACCUM : BWD_SGD), 0.f); }
+void sft_backward_sgd(SFTState *s, float lr) { backward_from_dlogits(s, !s->full_param ? BWD_LORA : (s->gqkv ? BWD_ACCUM : BWD_SGD), lr); }
+void sft_backward_accum(SFTState *s) { sft_backward(s); }
+
+// sft_alloc_grad_accum, src/nn/fast_sft.c:996-1019: zeroed F16 accumulators mirroring every weight.
+void sft_alloc_grad_accum(SFTState *s)
+{
+    if (s->gqkv || !s->full_param) return;
+    s->gqkv = hbuf(s->NL * s->st_qkv); s->go = hbuf(s->NL * s->st_o);
+    s->ggu = hbuf(s->NL * s->st_gu);   s->gd = hbuf(s->NL * s->st_d);
+    s->glm = hbuf(tiled_elems(s->V, s->D));
+    for (MetalBuf *b : {s->gqkv, s->go, s->ggu, s->gd, s->glm}) HIP_CHECK(hipMemsetAsync(dptr(b), 0, b->size, stream()));
+    const double mb = 2.0 * ((double)s->NL * (s->st_qkv + s->st_o + s->st_gu + s->st_d) + (double)tiled_elems(s->V, s->D)) / (1024.0 * 1024.0);
+    printf("[FastSFT] Grad accum buffers allocated: %.2f MB\n", mb);
+}
+
+// sft_apply_grad_sgd, src/nn/fast_sft.c:1021-1039: W = half(W - lr G), G = 0, then flush.  Both images
+// of every weight (as stored and transposed) are rewritten.
+void sft_apply_grad_sgd(SFTState *s, float lr)
+{
+    if (!s->gqkv) return;
+    for (int L = 0; L < s->NL; L++) {
+        launch_apply_retile(at<half_t>(s->wqkv, L * s->st_qkv), at<half_t>(s->gqkv, L * s->st_qkv), at<half_t>(s->wqkvT, L * s->st_qkvT), s->nq_ext, s->D, lr);
+        launch_apply_retile(at<half_t>(s->wo, L * s->st_o), at<half_t>(s->go, L * s->st_o), at<half_t>(s->woT, L * s->st_oT), s->D, s->qd, lr);
+        launch_apply_retile(at<half_t>(s->wgu, L * s->st_gu), at<half_t>(s->ggu, L * s->st_gu), at<half_t>(s->wguT, L * s->st_guT), 2 * s->IS, s->D, lr);
+        launch_apply_retile(at<half_t>(s->wd, L * s->st_d), at<half_t>(s->gd, L * s->st_d), at<half_t>(s->wdT, L * s->st_dT), s->D, s->IS, lr);
+    }
+    launch_apply_retile(at<half_t>(s->wlm), at<half_t>(s->glm), at<half_t>(s->wlmT), s->V, s->D, lr);
+    metal_flush();
+}
+
+// Row-major F16 copy of one matrix: which = 0..6 (q, k, v, o, gate, up, down of `layer`) or 7 (lm_head);
+// source = 0 the image the forward multiplies with, 1 its transposed twin (must hold the same values),
+// 2 the gradient accumulator.
+void sft_copy_matrix_f16(SFTState *s, int layer, int which, int source, uint16_t *dst)
+{
+    const int D = s->D, IS = s->IS, qd = s->qd, kd = s->kd;
+    struct Sel { MetalBuf *W, *WT, *G; size_t st, stT; int M, N, row_off, rows; } sel;
+    switch (which) {
+    case 0: sel = {s->wqkv, s->wqkvT, s->gqkv, s->st_qkv, s->st_qkvT, s->nq_ext, D, 0, qd}; break;
+    case 1: sel = {s->wqkv, s->wqkvT, s->gqkv, s->st_qkv, s->st_qkvT, s->nq_ext, D, qd, kd}; break;
+    case 2: sel = {s->wqkv, s->wqkvT, s->gqkv, s->st_qkv, s->st_qkvT, s->nq_ext, D, qd + kd, kd}; break;
+    case 3: sel = {s->wo, s->woT, s->go, s->st_o, s->st_oT, D, qd, 0, D}; break;
+    case 4: sel = {s->wgu, s->wguT, s->ggu, s->st_gu, s->st_guT, 2 * IS, D, 0, IS}; break;
+    case 5: sel = {s->wgu, s->wguT, s->ggu, s->st_gu, s->st_guT, 2 * IS, D, IS, IS}; break;
+    case 6: sel = {s->wd, s->wdT, s->gd, s->st_d, s->st_dT, D, IS, 0, D}; break;
+    case 7: sel = {s->wlm, s->wlmT, s->glm, 0, 0, s->V, D, 0, s->V}; layer = 0; break;
+    default: return;
+    }
+    if (layer < 0 || layer >= s->NL || (source == 2 && !sel.G)) return;
+    const size_t n = (size_t)sel.rows * sel.N;
+    MetalBuf *tmp = hbuf(n);
+    if (source == 1)
+        launch_untile_f16(at<half_t>(sel.WT, layer * sel.stT), tiled_kb(sel.M), 0, sel.row_off, 1, sel.rows, sel.N, at<half_t>(tmp));
+    else
+        launch_untile_f16(at<half_t>(source == 2 ? sel.G : sel.W, layer * sel.st), tiled_kb(sel.N), sel.row_off, 0, 0, sel.rows, sel.N, at<half_t>(tmp));
+    metal_buf_read(tmp, 0, dst, n * 2);
+    metal_buf_free(tmp);
+}
+
+// "FULL" checkpoint, src/nn/fast_sft.c:1286-1340: nine u32 header words, then per layer
+// q, k, v, o, gate, up, down and finally lm_head as row-major F16.
+void sft_save_full_checkpoint(SFTState *s, const char *path)
+{
+    FILE *fp = fopen(path, "wb");
+    if (!fp) { fprintf(stderr, "[FastSFT] Failed to open %s for writing\n", path); return; }
+    const uint32_t hdr[9] = {0x46554C4Cu, (uint32_t)s->model_type, (uint32_t)s->NL, (uint32_t)s->D, (uint32_t)s->Hq,
+                             (uint32_t)s->Hkv, (uint32_t)s->hd, (uint32_t)s->IS, (uint32_t)s->V};
+    fwrite(hdr, 4, 9, fp);
+    const size_t sizes[8] = {(size_t)s->qd * s->D, (size_t)s->kd * s->D, (size_t)s->kd * s->D, (size_t)s->D * s->qd,
+                             (size_t)s->IS * s->D, (size_t)s->IS * s->D, (size_t)s->D * s->IS, (size_t)s->V * s->D};
+    std::vector<uint16_t> buf;
+    size_t total = 0;
+    for (int L = 0; L <= s->NL; L++)
+        for (int w = (L < s->NL ? 0 : 7); w < (L < s->NL ? 7 : 8); w++) {
+            buf.resize(sizes[w]);
+            sft_copy_matrix_f16(s, L < s->NL ? L : 0, w, 0, buf.data());
+            fwrite(buf.data(), 2, sizes[w], fp);
+            total += sizes[w] * 2;
+        }
+    fclose(fp);
+    printf("[FastSFT] Full checkpoint saved to %s (%.2f MB)\n", path, (float)total / (1024.0f * 1024.0f));
 }
 
 void sft_lora_update(SFTState *s, float lr)
@@ -625,7 +799,9 @@ int sft_get_n_kv_heads(SFTState *s) { return s->Hkv; }
 int sft_get_head_dim(SFTState *s) { return s->hd; }
 int sft_get_intermediate_size(SFTState *s) { return s->IS; }
 const float *sft_get_rope_thetas(SFTState *s) { return s->rope_thetas.data(); }
-int sft_is_full_param(SFTState *s) { (void)s; return 0; }
+int sft_is_full_param(SFTState *s) { return s->full_param; }
+const float *sft_get_token_emb(SFTState *s) { return s->token_emb_host; }
+MetalBuf *sft_get_final_norm_g(SFTState *s) { return s->g_final; }
 
 size_t sft_lora_numel(SFTState *s) { return s->lora_n; }
 void sft_copy_lora(SFTState *s, float *dst) { if (s->lora_n) metal_buf_read(s->lora, 0, dst, s->lora_n * 4); }
@@ -642,6 +818,127 @@ float sft_get_last_grad_norm(SFTState *s)
     float v = 0.f;
     metal_buf_read(s->grad_norm, 0, &v, 4);
     return v;
+}
+
+// Row-major F16 copies of the seven matrices of every layer (refreshed on every call, since
+// full-parameter training changes them) plus windows on the norm gammas: what
+// inference_state_create_from_sft borrows (src/nn/fast_inference.c:596-603).  The copies are F16 also
+// when the state was built from Q8_0 weights (they hold the dequantised values).
+LayerW *sft_get_layers(SFTState *s)
+{
+    const int NL = s->NL, D = s->D, IS = s->IS, qd = s->qd, kd = s->kd;
+    const int rows[7] = {qd, kd, kd, D, IS, IS, D}, cols[7] = {D, D, D, qd, D, D, IS};
+    if (s->layers_out.empty()) {
+        s->wmats_out.resize((size_t)7 * NL);
+        s->layers_out.resize(NL);
+        for (int L = 0; L < NL; L++) {
+            for (int w = 0; w < 7; w++) {
+                WMat &m = s->wmats_out[(size_t)L * 7 + w];
+                m.rows = rows[w]; m.cols = cols[w]; m.nb = cols[w] / 32;
+                m.mbuf = hbuf((size_t)rows[w] * cols[w]);
+            }
+            WMat *m = &s->wmats_out[(size_t)L * 7];
+            auto view = [&](MetalBuf *arena, int dim) -> MetalBuf * {
+                if (!arena) return nullptr;
+                MetalBuf *v = metal_buf_view(arena, (size_t)L * dim * 4, (size_t)dim * 4);
+                s->views_out.push_back(v);
+                return v;
+            };
+            const bool gemma = s->model_type == MODEL_GEMMA3;
+            s->layers_out[L] = LayerW{m, m + 1, m + 2, m + 3, m + 4, m + 5, m + 6,
+                                      view(s->g_in, D), view(s->g_post_attn, D),
+                                      gemma ? view(s->g_pre_ff, D) : nullptr, gemma ? view(s->g_post_ff, D) : nullptr,
+                                      view(s->g_q, s->hd), view(s->g_k, s->hd)};
+        }
+    }
+    for (int L = 0; L < NL; L++) {
+        struct Src { MetalBuf *W; size_t st; int N, row_off; };
+        const Src src[7] = {{s->wqkv, s->st_qkv, D, 0}, {s->wqkv, s->st_qkv, D, qd}, {s->wqkv, s->st_qkv, D, qd + kd},
+                            {s->wo, s->st_o, qd, 0}, {s->wgu, s->st_gu, D, 0}, {s->wgu, s->st_gu, D, IS}, {s->wd, s->st_d, IS, 0}};
+        for (int w = 0; w < 7; w++)
+            launch_untile_f16(at<half_t>(src[w].W, L * src[w].st), tiled_kb(src[w].N), src[w].row_off, 0, 0, rows[w], cols[w],
+                              at<half_t>(s->wmats_out[(size_t)L * 7 + w].mbuf));
+    }
+    return s->layers_out.data();
+}
+
+WMat *sft_get_lm_head(SFTState *s)
+{
+    WMat &m = s->lm_head_out;
+    if (!m.mbuf) { m.rows = s->V; m.cols = s->D; m.nb = s->D / 32; m.mbuf = hbuf((size_t)s->V * s->D); }
+    launch_untile_f16(at<half_t>(s->wlm), tiled_kb(s->D), 0, 0, 0, s->V, s->D, at<half_t>(m.mbuf));
+    return &m;
+}
+
+// Phases 3 and 4 of grpo_train_step (src/nn/fast_grpo.c:376-495) for a group of completions that
+// has already been sampled and scored: per completion build [prompt tail | completion | zero rows],
+// forward, PPO-clip policy gradient scaled by 1/G, backward; then apply.
+//   full-parameter + accurate: accumulate F16 gradients, one sft_apply_grad_sgd(lr) at the end;
+//   full-parameter otherwise:  fused SGD with lr/G after every completion;
+//   LoRA:                      sum the adapter gradients over the group, step_count++, AdamW.
+// new_logprobs (optional, [G][rows]) receives the policy's log-probabilities of the actions.
+void grpo_apply_completions(SFTState *s, const GRPOCompletions *c, float lr, float *new_logprobs)
+{
+    if (s->B != 1) { fprintf(stderr, "[FastGRPO] the state must be built with batch 1\n"); return; }
+    const int G = c->group_size, seq_len = s->BN;
+    if (G <= 0) return;
+    const bool accurate = s->full_param && c->accurate;
+    if (accurate) sft_alloc_grad_accum(s);
+    if (!s->grpo_old_lp) {
+        s->grpo_old_lp = host_buf((size_t)seq_len * 4, (void **)&s->grpo_old_lp_cpu);
+        s->grpo_advs = host_buf((size_t)seq_len * 4, (void **)&s->grpo_advs_cpu);
+        s->grpo_new_lp = host_buf((size_t)seq_len * 4, (void **)&s->grpo_new_lp_cpu);
+    }
+    if (!s->full_param) {
+        if (!s->lora_acc) s->lora_acc = fbuf(s->lora_n);
+        HIP_CHECK(hipMemsetAsync(dptr(s->lora_acc), 0, s->lora_n * 4, stream()));
+    }
+    for (int i = 0; i < G; i++) {
+        int comp_len = c->gen_lengths[i];                  // [:388-400]
+        if (comp_len > seq_len) comp_len = seq_len;
+        int prompt_use = seq_len - comp_len;
+        if (prompt_use > c->prompt_len) prompt_use = c->prompt_len;
+        if (prompt_use < 0) prompt_use = 0;
+        int total = prompt_use + comp_len;
+        if (total > seq_len) { comp_len = seq_len - prompt_use; total = seq_len; }
+        if (new_logprobs) memset(new_logprobs + (size_t)i * seq_len, 0, (size_t)seq_len * 4);
+        if (total <= 0) continue;                          // nothing but zero rows: no gradient
+        const int prompt_start = c->prompt_len - prompt_use;
+        memset(s->tokens_cpu, 0, (size_t)seq_len * 4);
+        memset(s->targets_cpu, 0, (size_t)seq_len * 4);    // actions                      [:430-443]
+        memset(s->grpo_old_lp_cpu, 0, (size_t)seq_len * 4);
+        memset(s->grpo_advs_cpu, 0, (size_t)seq_len * 4);
+        for (int t = 0; t < prompt_use; t++) s->tokens_cpu[t] = c->prompt[prompt_start + t];
+        for (int t = 0; t < comp_len; t++) {
+            const int pos = prompt_use + t;
+            s->tokens_cpu[pos] = c->gen_tokens[i][t];
+            s->targets_cpu[pos] = c->gen_tokens[i][t];
+            s->grpo_old_lp_cpu[pos] = c->gen_logprobs[i][t];
+            s->grpo_advs_cpu[pos] = c->advantages[i];
+        }
+        forward_impl(s, true, total < seq_len ? total : 0);
+        CeArgs ce{};
+        ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
+        ce.dl16 = at<half_t>(s->dl16); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
+        ce.grpo = 1; ce.old_lp = at<float>(s->grpo_old_lp); ce.advs = at<float>(s->grpo_advs); ce.new_lp = at<float>(s->grpo_new_lp);
+        ce.clip_eps = c->clip_eps; ce.dl_scale = 1.0f / (float)G;                 // [:445-452]
+        launch_ce_rows(ce, s->BN);
+        if (s->full_param) {
+            backward_impl(s, s->gqkv ? BWD_ACCUM : BWD_SGD, lr / (float)G);       // [:454-461]
+        } else {
+            backward_impl(s);                                                     // [:462-473]
+            metal_enqueue_add_scaled(s->lora_acc, s->lora_grad, 1.0f, (int)s->lora_n);
+        }
+        metal_flush();
+        if (new_logprobs) memcpy(new_logprobs + (size_t)i * seq_len, s->grpo_new_lp_cpu, (size_t)seq_len * 4);
+    }
+    if (accurate) {                                                               // [:479-481]
+        sft_apply_grad_sgd(s, lr);
+    } else if (!s->full_param) {                                                  // [:482-491]
+        metal_enqueue_copy(s->lora_acc, s->lora_grad, (int)s->lora_n);
+        s->step_count++;
+        sft_lora_update(s, lr);
+    }
 }
 
 // "LORA" adapter file: u32 magic 0x4C4F5241, i32 n_layers, i32 rank, then per layer

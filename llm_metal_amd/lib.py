@@ -56,6 +56,19 @@ class WMat(C.Structure):
     _fields_ = [("mbuf", C.c_void_p), ("rows", C.c_int), ("cols", C.c_int), ("nb", C.c_int)]
 
 
+class LayerW(C.Structure):
+    _fields_ = [(k, C.POINTER(WMat)) for k in ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")] + \
+               [(k, C.c_void_p) for k in ("input_norm_g", "post_attn_norm_g", "pre_ff_norm_g", "post_ff_norm_g",
+                                          "q_norm_g", "k_norm_g")]
+
+
+class GRPOCompletions(C.Structure):
+    _fields_ = [("prompt", C.c_void_p), ("prompt_len", C.c_int), ("group_size", C.c_int),
+                ("gen_tokens", C.POINTER(C.c_void_p)), ("gen_lengths", C.c_void_p),
+                ("gen_logprobs", C.POINTER(C.c_void_p)), ("advantages", C.c_void_p),
+                ("clip_eps", C.c_float), ("accurate", C.c_int)]
+
+
 def load():
     global _lib
     if _lib is not None:
@@ -112,6 +125,12 @@ def load():
         "sft_get_rope_thetas": (vp, [vp]), "sft_is_full_param": (i, [vp]), "sft_save_lora": (None, [vp, C.c_char_p]),
         "sft_lora_numel": (sz, [vp]), "sft_copy_lora": (None, [vp, vp]), "sft_copy_lora_grads": (None, [vp, vp]),
         "sft_set_lora": (None, [vp, vp]), "sft_get_last_grad_norm": (f, [vp]),
+        "sft_get_token_emb": (vp, [vp]), "sft_get_final_norm_g": (vp, [vp]),
+        "sft_get_layers": (C.POINTER(LayerW), [vp]), "sft_get_lm_head": (C.POINTER(WMat), [vp]),
+        "sft_backward_sgd": (None, [vp, f]), "sft_alloc_grad_accum": (None, [vp]), "sft_backward_accum": (None, [vp]),
+        "sft_apply_grad_sgd": (None, [vp, f]), "sft_save_full_checkpoint": (None, [vp, C.c_char_p]),
+        "sft_copy_matrix_f16": (None, [vp, i, i, i, vp]),
+        "grpo_apply_completions": (None, [vp, C.POINTER(GRPOCompletions), f, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)

@@ -109,6 +109,7 @@ class SFTState:
                                                   1 if c.weight_format == "f16" else 0)
         if not self.h:
             raise RuntimeError("sft_state_create_from_ref failed (no gfx950 device or unsupported dims)")
+        self._emb = emb                                    # sft_get_token_emb hands out this (borrowed) table
 
     def train_step(self, tok, tgt, lr):
         tok = np.ascontiguousarray(tok, dtype=np.uint32)
@@ -162,6 +163,56 @@ class SFTState:
 
     def backward(self):
         self.L.sft_backward(self.h)
+
+    # -- full-parameter mode (lora_rank 0)
+    MATRICES = ("wq", "wk", "wv", "wo", "wg", "wu", "wd", "lm_head")
+
+    def matrix_shape(self, which):
+        c = self.c
+        return {"wq": (c.Hq * c.hd, c.D), "wk": (c.Hkv * c.hd, c.D), "wv": (c.Hkv * c.hd, c.D), "wo": (c.D, c.Hq * c.hd),
+                "wg": (c.IS, c.D), "wu": (c.IS, c.D), "wd": (c.D, c.IS), "lm_head": (c.V, c.D)}[which]
+
+    def matrix_f16(self, layer, which, source=0):
+        """F16 bit pattern (uint16, row-major) of one matrix: source 0 = weight, 1 = its transposed image,
+        2 = gradient accumulator."""
+        out = np.zeros(self.matrix_shape(which), dtype=np.uint16)
+        self.L.sft_copy_matrix_f16(self.h, layer, self.MATRICES.index(which), source, _vp(out))
+        return out
+
+    def is_full_param(self):
+        return bool(self.L.sft_is_full_param(self.h))
+
+    def alloc_grad_accum(self):
+        self.L.sft_alloc_grad_accum(self.h)
+
+    def backward_accum(self):
+        self.L.sft_backward_accum(self.h)
+
+    def backward_sgd(self, lr):
+        self.L.sft_backward_sgd(self.h, lr)
+
+    def apply_grad_sgd(self, lr):
+        self.L.sft_apply_grad_sgd(self.h, lr)
+
+    def save_full_checkpoint(self, path):
+        self.L.sft_save_full_checkpoint(self.h, path.encode())
+
+    def grpo_apply_completions(self, prompt, gen_tokens, gen_logprobs, advantages, clip_eps, lr, accurate=True):
+        """Phases 3-4 of a GRPO step over already sampled completions.  Returns the policy's
+        log-probabilities of the actions, [G, rows] (zero outside the completion positions)."""
+        G = len(gen_tokens)
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        toks = [np.ascontiguousarray(t, dtype=np.uint32) for t in gen_tokens]
+        lps = [np.ascontiguousarray(p, dtype=np.float32) for p in gen_logprobs]
+        lens = np.asarray([len(t) for t in toks], dtype=np.int32)
+        adv = np.ascontiguousarray(advantages, dtype=np.float32)
+        tp = (C.c_void_p * G)(*[t.ctypes.data for t in toks])
+        lp = (C.c_void_p * G)(*[p.ctypes.data for p in lps])
+        c = _lib.GRPOCompletions(prompt.ctypes.data, len(prompt), G, tp, lens.ctypes.data, lp, adv.ctypes.data,
+                                 clip_eps, 1 if accurate else 0)
+        new_lp = np.zeros((G, self.c.BN), dtype=np.float32)
+        self.L.grpo_apply_completions(self.h, C.byref(c), lr, _vp(new_lp))
+        return new_lp
 
     def free(self):
         if self.h:

@@ -38,6 +38,15 @@ class OrWeights(C.Structure):
                 ("token_emb", C.POINTER(C.c_float)), ("rope_theta", C.POINTER(C.c_float))]
 
 
+_PU16 = C.POINTER(C.POINTER(C.c_uint16))
+
+
+class OrFull(C.Structure):
+    _fields_ = [("accum", C.c_int), ("lr", C.c_float)] + \
+               [(k, _PU16) for k in ("gq", "gk", "gv", "go", "gg", "gu", "gd")] + \
+               [("glm", C.POINTER(C.c_uint16))]
+
+
 def lib(precision="f32"):
     if precision not in _LIBS:
         path = os.path.join(_HERE, f"liboracle_{precision}.so")
@@ -46,6 +55,7 @@ def lib(precision="f32"):
         L = C.CDLL(path)
         L.or_sft_loss.restype = C.c_double
         L.or_sft_train_step.restype = C.c_double
+        L.or_full_param_pass.restype = C.c_double
         L.or_clip_grad_norm.restype = C.c_double
         L.or_lora_layer_size.restype = C.c_size_t
         L.or_f32_to_f16_bits.restype = C.c_uint16
@@ -183,6 +193,84 @@ def sft_train_step(c, used, lora, m, v, step, tok, tgt, lr, do_update=True, prec
     if want_dx:
         out["dx"] = dx
     return out
+
+
+# ---------------------------------------------------------------- full-parameter mode
+
+_GA_KEYS = (("gq", "wq"), ("gk", "wk"), ("gv", "wv"), ("go", "wo"), ("gg", "wg"), ("gu", "wu"), ("gd", "wd"))
+
+
+def new_grad_accum(used):
+    """Zeroed F16 (bit pattern) accumulators shaped like the matrices of `used`
+    (sft_alloc_grad_accum, src/nn/fast_sft.c:996-1019)."""
+    ga = {g: [np.zeros(w.shape, dtype=np.uint16) for w in used[k]] for g, k in _GA_KEYS}
+    ga["glm"] = np.zeros(used["lm_head"].shape, dtype=np.uint16)
+    return ga
+
+
+def _full(c, ga, lr):
+    f = OrFull()
+    keep = []
+    f.accum = 1 if ga is not None else 0
+    f.lr = lr
+    if ga is not None:
+        for g, _ in _GA_KEYS:
+            tbl = (C.POINTER(C.c_uint16) * c.NL)(*[a.ctypes.data_as(C.POINTER(C.c_uint16)) for a in ga[g]])
+            keep.append(tbl)
+            setattr(f, g, C.cast(tbl, _PU16))
+        f.glm = ga["glm"].ctypes.data_as(C.POINTER(C.c_uint16))
+    return f, keep
+
+
+def full_param_pass(c, used, ga, lr=0.0, tok=None, x_rows=None, tgt=None, grpo=None, precision="f32",
+                    want_logits=False, want_dx=False, lora=None):
+    """Forward + full-parameter backward.  ga = accumulators (sft_backward_accum) or
+    None (sft_backward_sgd with lr: the float32 matrices of `used` are updated in
+    place).  grpo = dict(actions, old_lp, advs, clip_eps, dl_scale) switches the
+    loss to the policy gradient.  With lora (flat adapters, c.R > 0) the backward is the
+    LoRA one instead and the result carries "grad".  Returns dict(loss[, logits, new_lp, dx, grad])."""
+    assert (c.R == 0) == (lora is None)
+    L = lib(precision)
+    dt = real_dtype(precision)
+    pk = _Packed(c, used)
+    full, keep = _full(c, ga, lr)
+    fullp = C.byref(full) if lora is None else None
+    lora_a = np.ascontiguousarray(lora, dtype=dt) if lora is not None else None
+    grad = np.zeros_like(lora_a) if lora is not None else None
+    lp, gp = (_p(lora_a), _p(grad)) if lora is not None else (None, None)
+    logits = np.zeros((c.BN, c.V), dtype=dt) if want_logits else None
+    dx = np.zeros((c.BN, c.D), dtype=dt) if want_dx else None
+    new_lp = np.zeros(c.BN, dtype=dt)
+    tokp = _p(np.ascontiguousarray(tok, dtype=np.uint32)) if tok is not None else None
+    xr = np.ascontiguousarray(x_rows, dtype=dt) if x_rows is not None else None
+    if grpo is None:
+        tg = np.ascontiguousarray(tgt, dtype=np.uint32)
+        loss = L.or_full_param_pass(C.byref(_cfg(c)), C.byref(pk.w), fullp, lp, gp, tokp, _p(xr) if xr is not None else None,
+                                    C.c_int(0), _p(tg), None, None, C.c_float(0), C.c_float(0),
+                                    _p(logits) if want_logits else None, None, _p(dx) if want_dx else None)
+    else:
+        act = np.ascontiguousarray(grpo["actions"], dtype=np.uint32)
+        olp = np.ascontiguousarray(grpo["old_lp"], dtype=dt)
+        adv = np.ascontiguousarray(grpo["advs"], dtype=dt)
+        loss = L.or_full_param_pass(C.byref(_cfg(c)), C.byref(pk.w), fullp, lp, gp, tokp, _p(xr) if xr is not None else None,
+                                    C.c_int(1), _p(act), _p(olp), _p(adv), C.c_float(grpo["clip_eps"]),
+                                    C.c_float(grpo["dl_scale"]),
+                                    _p(logits) if want_logits else None, _p(new_lp), _p(dx) if want_dx else None)
+    out = {"loss": loss, "new_lp": new_lp}
+    if want_logits:
+        out["logits"] = logits
+    if want_dx:
+        out["dx"] = dx
+    if grad is not None:
+        out["grad"] = grad
+    return out
+
+
+def apply_grad_sgd(c, used, ga, lr):
+    """W = half(W - lr G), G = 0 on every matrix (sft_apply_grad_sgd)."""
+    pk = _Packed(c, used)
+    full, keep = _full(c, ga, lr)
+    lib().or_apply_grad_sgd(C.byref(_cfg(c)), C.byref(pk.w), C.byref(full), C.c_float(lr))
 
 
 # ---------------------------------------------------------------- single ops

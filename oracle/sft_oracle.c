@@ -640,6 +640,7 @@ OR_API size_t or_lora_layer_size(const OrCfg *c)
 typedef struct {
     real *x_in, *ln1, *q_pre, *k_pre, *q_fin, *k_exp, *v_exp, *probs;
     real *x_mid, *ln2, *gate_pre, *up_val, *tq, *tv, *o_out, *ff_raw;
+    real *act, *attn_flat;   /* save_gate_act, save_attn_flat: inputs of down_proj / o_proj (weight gradients) */
 } OrSave;
 
 typedef struct {
@@ -667,6 +668,7 @@ static OrRun *run_alloc(const OrCfg *c)
         s->gate_pre = ralloc(BN * c->IS); s->up_val = ralloc(BN * c->IS);
         s->tq = ralloc(BN * (c->R ? c->R : 1)); s->tv = ralloc(BN * (c->R ? c->R : 1));
         s->o_out = ralloc(BN * c->D); s->ff_raw = ralloc(BN * c->D);
+        s->act = ralloc(BN * c->IS);  s->attn_flat = ralloc(BN * qd);
     }
     r->x_final = ralloc(BN * c->D); r->ln_final = ralloc(BN * c->D);
     r->logits = ralloc(BN * c->V);  r->dlogits = ralloc(BN * c->V);
@@ -681,6 +683,7 @@ static void run_free(OrRun *r)
         free(s->x_in); free(s->ln1); free(s->q_pre); free(s->k_pre); free(s->q_fin);
         free(s->k_exp); free(s->v_exp); free(s->probs); free(s->x_mid); free(s->ln2);
         free(s->gate_pre); free(s->up_val); free(s->tq); free(s->tv); free(s->o_out); free(s->ff_raw);
+        free(s->act); free(s->attn_flat);
     }
     free(r->sv); free(r->x_final); free(r->ln_final); free(r->logits); free(r->dlogits); free(r->losses);
     free(r);
@@ -743,6 +746,7 @@ static void forward(OrRun *r, const OrWeights *w, const real *lora, real *x)
             or_transpose_heads_rev(ao, af + ro * qd, N, Hq, hd);
         }
 
+        memcpy(s->attn_flat, af, sizeof(real) * BN * qd);
         or_wmatmul(af, w->wo[L], x2, BN, D, qd);
         if (c->model_type == 1) {                      /* src/nn/fast_sft.c:698-705 */
             memcpy(s->o_out, x2, sizeof(real) * BN * D);
@@ -763,6 +767,7 @@ static void forward(OrRun *r, const OrWeights *w, const real *lora, real *x)
         memcpy(s->up_val, up, sizeof(real) * BN * IS);
         if (c->model_type == 1) or_gelu_mul(gate, up, (size_t)BN * IS);
         else                    or_silu_mul(gate, up, (size_t)BN * IS);
+        memcpy(s->act, gate, sizeof(real) * BN * IS);
         or_wmatmul(gate, w->wd[L], ff, BN, D, IS);
         if (c->model_type == 1) {                      /* src/nn/fast_sft.c:732-736 */
             memcpy(s->ff_raw, ff, sizeof(real) * BN * D);
@@ -779,10 +784,38 @@ static void forward(OrRun *r, const OrWeights *w, const real *lora, real *x)
     free(ao); free(af); free(x2); free(gate); free(up); free(ff);
 }
 
-/* sft_backward_ex (LoRA branch), src/nn/fast_sft.c:766-982.  r->dlogits must
+/* Full-parameter mode of sft_backward_ex (src/nn/fast_sft.c:778-786, 804-811,
+ * 817-833, 883-901, 922-946).  Every frozen matrix gets dW = dY^T X either added
+ * into an F16 accumulator (accum = 1, f16_grad_accum) or applied at once as
+ * W = half(W - lr dW) (accum = 0, f16_sgd_fused).  The matrices of OrWeights hold
+ * F16 values widened to float; in SGD mode they are updated in place (the const
+ * of OrWeights is cast away) and stay F16-representable. */
+typedef struct {
+    int accum;
+    float lr;
+    uint16_t *const *gq, *const *gk, *const *gv, *const *go, *const *gg, *const *gu, *const *gd;   /* [NL] F16 bits */
+    uint16_t *glm;
+} OrFull;
+
+static void weight_grad(const OrFull *fp, const float *W_const, uint16_t *G,
+                        const real *dY, const real *X, int M, int K, int N)
+{
+    if (fp->accum) { or_f16_grad_accum(G, dY, X, M, K, N); return; }
+    float *W = (float *)W_const;
+    for (int m = 0; m < M; m++)
+        for (int n = 0; n < N; n++) {                   /* f16_sgd_fused on widened values */
+            real s = 0;
+            for (int k = 0; k < K; k++) s += dY[(size_t)k * M + m] * X[(size_t)k * N + n];
+            size_t idx = (size_t)m * N + n;
+            W[idx] = or_f16_bits_to_f32(or_f32_to_f16_bits(W[idx] - fp->lr * (float)s));
+        }
+}
+
+/* sft_backward_ex, src/nn/fast_sft.c:766-982: the LoRA branch when fp is NULL,
+ * the full-parameter branch (c->R must be 0) otherwise.  r->dlogits must
  * hold the loss gradient.  Writes the LoRA gradients (overwritten, never
  * accumulated) and, if dx_out is given, the gradient w.r.t. the embedded input. */
-static void backward(OrRun *r, const OrWeights *w, const real *lora, real *grad, real *dx_out)
+static void backward(OrRun *r, const OrWeights *w, const real *lora, real *grad, real *dx_out, const OrFull *fp)
 {
     const OrCfg *c = &r->c;
     int BN = c->batch * c->seq, N = c->seq, D = c->D, Hq = c->Hq, Hkv = c->Hkv, hd = c->hd;
@@ -799,6 +832,7 @@ static void backward(OrRun *r, const OrWeights *w, const real *lora, real *grad,
     real *dh = ralloc((size_t)BN * (R ? R : 1)), *lo = ralloc((size_t)BN * D);
 
     or_wmatmul_nt(r->dlogits, w->lm_head, dx, BN, c->V, D);
+    if (fp) weight_grad(fp, w->lm_head, fp->glm, r->dlogits, r->ln_final, c->V, BN, D);
     or_rms_norm_backward(r->x_final, dx, w->g_final, dx2, BN, D, c->eps);
     memcpy(dx, dx2, sizeof(real) * BN * D);
 
@@ -816,10 +850,13 @@ static void backward(OrRun *r, const OrWeights *w, const real *lora, real *grad,
             d = dx2;
         }
         or_wmatmul_nt(d, w->wd[L], gate, BN, D, IS);
+        if (fp) weight_grad(fp, w->wd[L], fp->accum ? fp->gd[L] : NULL, d, s->act, D, BN, IS);
         if (c->model_type == 1) or_gelu_mul_backward(gate, s->gate_pre, s->up_val, gate, up, (size_t)BN * IS);
         else                    or_silu_mul_backward(gate, s->gate_pre, s->up_val, gate, up, (size_t)BN * IS);
         or_wmatmul_nt(gate, w->wg[L], ln, BN, IS, D);
+        if (fp) weight_grad(fp, w->wg[L], fp->accum ? fp->gg[L] : NULL, gate, s->ln2, IS, BN, D);
         or_wmatmul_nt(up, w->wu[L], x2, BN, IS, D);
+        if (fp) weight_grad(fp, w->wu[L], fp->accum ? fp->gu[L] : NULL, up, s->ln2, IS, BN, D);
         or_residual_add(ln, x2, (size_t)BN * D);
         or_rms_norm_backward(s->x_mid, ln, c->model_type == 1 ? w->g_pre_ff[L] : w->g_post_attn[L],
                              dx2, BN, D, c->eps);
@@ -832,6 +869,7 @@ static void backward(OrRun *r, const OrWeights *w, const real *lora, real *grad,
             d = dx2;
         }
         or_wmatmul_nt(d, w->wo[L], af, BN, D, qd);
+        if (fp) weight_grad(fp, w->wo[L], fp->accum ? fp->go[L] : NULL, d, s->attn_flat, D, BN, qd);
 
         /* attention core, src/nn/fast_sft.c:905-920 */
         for (int b = 0; b < c->batch; b++) {
@@ -848,6 +886,14 @@ static void backward(OrRun *r, const OrWeights *w, const real *lora, real *grad,
             or_transpose_heads_rev(qt, dq + ro * qd, N, Hq, hd);
             or_transpose_heads_rev(kt, dk + ro * kd, N, Hkv, hd);
             or_transpose_heads_rev(vt, dv + ro * kd, N, Hkv, hd);
+        }
+
+        /* full-parameter: the three weight updates come BEFORE the dX products, which therefore see
+         * the new weights in SGD mode (src/nn/fast_sft.c:922-946) */
+        if (fp) {
+            weight_grad(fp, w->wq[L], fp->accum ? fp->gq[L] : NULL, dq, s->ln1, qd, BN, D);
+            weight_grad(fp, w->wk[L], fp->accum ? fp->gk[L] : NULL, dk, s->ln1, kd, BN, D);
+            weight_grad(fp, w->wv[L], fp->accum ? fp->gv[L] : NULL, dv, s->ln1, kd, BN, D);
         }
 
         /* LoRA Q, base Q/K, LoRA V, base V: src/nn/fast_sft.c:948-971 */
@@ -932,7 +978,7 @@ OR_API double or_sft_train_step(const OrCfg *c, const OrWeights *w, real *lora, 
     forward(r, w, lora, x);
     or_softmax_ce(r->logits, targets, r->losses, r->dlogits, BN, c->V);
     or_scale(r->dlogits, 1.0f / (float)BN, (size_t)BN * c->V);
-    backward(r, w, lora, grad, dx_out);
+    backward(r, w, lora, grad, dx_out, NULL);
     real tot = 0;
     for (int i = 0; i < BN; i++) tot += r->losses[i];
     double loss = (double)(tot / (real)BN);
@@ -950,4 +996,80 @@ OR_API double or_sft_train_step(const OrCfg *c, const OrWeights *w, real *lora, 
     }
     free(x); run_free(r);
     return loss;
+}
+
+/* One forward + backward on one batch of rows, in full-parameter mode (full != NULL,
+ * c->R == 0) or in LoRA mode (full == NULL: lora holds the adapters and grad receives
+ * their gradients, overwritten).
+ *   kind 0: cross-entropy against `targets`, dlogits / BN — sft_train_step with
+ *           s->full_param (src/nn/fast_sft.c:1129-1139); returns the mean loss.
+ *   kind 1: GRPO — grpo_policy_grad(actions = targets, old_lp, advs, clip_eps),
+ *           dlogits * dl_scale (1/G), src/nn/fast_grpo.c:437-452; new_lp_out gets the
+ *           log-probabilities; returns 0.
+ * x_rows, when given, is the embedded input [BN, D] (GRPO zero-pads rows past the
+ * sequence, src/nn/fast_grpo.c:420-422) and `tokens` is ignored.
+ * full->accum selects sft_backward_accum or sft_backward_sgd(lr). */
+OR_API double or_full_param_pass(const OrCfg *c, const OrWeights *w, const OrFull *full,
+                                 const real *lora, real *grad,
+                                 const uint32_t *tokens, const real *x_rows, int kind,
+                                 const uint32_t *targets, const real *old_lp, const real *advs,
+                                 float clip_eps, float dl_scale,
+                                 real *logits_out, real *new_lp_out, real *dx_out)
+{
+    OrRun *r = run_alloc(c);
+    int BN = c->batch * c->seq;
+    real *x;
+    if (x_rows) {
+        x = ralloc((size_t)BN * c->D);
+        memcpy(x, x_rows, sizeof(real) * BN * c->D);
+    } else {
+        x = embed(c, w, tokens);
+    }
+    forward(r, w, lora, x);
+    if (logits_out) memcpy(logits_out, r->logits, sizeof(real) * BN * c->V);
+    double ret = 0;
+    if (kind == 0) {
+        or_softmax_ce(r->logits, targets, r->losses, r->dlogits, BN, c->V);
+        or_scale(r->dlogits, 1.0f / (float)BN, (size_t)BN * c->V);
+        real tot = 0;
+        for (int i = 0; i < BN; i++) tot += r->losses[i];
+        ret = (double)(tot / (real)BN);
+    } else {
+        real *nl = ralloc(BN);
+        or_grpo_policy_grad(r->logits, targets, old_lp, advs, nl, r->dlogits, BN, c->V, clip_eps);
+        or_scale(r->dlogits, dl_scale, (size_t)BN * c->V);
+        if (new_lp_out) memcpy(new_lp_out, nl, sizeof(real) * BN);
+        free(nl);
+    }
+    backward(r, w, lora, grad, dx_out, full);
+    free(x); run_free(r);
+    return ret;
+}
+
+/* sft_apply_grad_sgd, src/nn/fast_sft.c:1021-1039, on widened weights:
+ * W = half(W - lr * G), G = 0 for the seven matrices of every layer and lm_head. */
+OR_API void or_apply_grad_sgd(const OrCfg *c, const OrWeights *w, const OrFull *full, float lr)
+{
+    size_t qd = (size_t)c->Hq * c->hd, kd = (size_t)c->Hkv * c->hd, D = c->D, IS = c->IS;
+    for (int L = 0; L <= c->NL; L++) {
+        const float *W[7]; uint16_t *G[7]; size_t n[7]; int cnt = 7;
+        if (L < c->NL) {
+            W[0] = w->wq[L]; G[0] = full->gq[L]; n[0] = qd * D;
+            W[1] = w->wk[L]; G[1] = full->gk[L]; n[1] = kd * D;
+            W[2] = w->wv[L]; G[2] = full->gv[L]; n[2] = kd * D;
+            W[3] = w->wo[L]; G[3] = full->go[L]; n[3] = D * qd;
+            W[4] = w->wg[L]; G[4] = full->gg[L]; n[4] = IS * D;
+            W[5] = w->wu[L]; G[5] = full->gu[L]; n[5] = IS * D;
+            W[6] = w->wd[L]; G[6] = full->gd[L]; n[6] = D * IS;
+        } else {
+            W[0] = w->lm_head; G[0] = full->glm; n[0] = (size_t)c->V * D; cnt = 1;
+        }
+        for (int j = 0; j < cnt; j++) {
+            float *Wm = (float *)W[j];
+            for (size_t i = 0; i < n[j]; i++) {
+                Wm[i] = or_f16_bits_to_f32(or_f32_to_f16_bits(Wm[i] - lr * or_f16_bits_to_f32(G[j][i])));
+                G[j][i] = 0;
+            }
+        }
+    }
 }

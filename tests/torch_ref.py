@@ -27,8 +27,29 @@ def rope_hf(x, theta):
     return x * cos + torch.cat([-x2, x1], -1) * sin
 
 
-def forward_loss(c, used, lora_flat, tok, tgt, x_embed=None):
-    """lora_flat: torch fp64 leaf tensor.  Returns (mean CE loss, logits)."""
+class _LinearUpdatedFirst(torch.autograd.Function):
+    """y = x W^T whose backward first forms dW, applies W' = half(W - lr dW) and only then
+    propagates dx = dy W' — the order in which the reference's full-parameter SGD mode treats
+    the Q, K and V projections (src/nn/fast_sft.c:922-946)."""
+
+    @staticmethod
+    def forward(ctx, x, W, lr):
+        ctx.save_for_backward(x, W)
+        ctx.lr = lr
+        return x @ W.T
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, W = ctx.saved_tensors
+        dW = dy.reshape(-1, dy.shape[-1]).T @ x.reshape(-1, x.shape[-1])
+        W_new = (W.float() - torch.tensor(ctx.lr, dtype=torch.float32) * dW.float()).half().double()
+        return dy @ W_new, dW, None
+
+
+def forward_loss(c, used, lora_flat, tok, tgt, x_embed=None, params=None, qkv_lr=None):
+    """lora_flat: torch fp64 leaf tensor.  Returns (mean CE loss, logits).
+    params (optional): {name: [per-layer leaf tensors]} + "lm_head" used in place of `used`'s matrices;
+    qkv_lr: route the Q/K/V projections through _LinearUpdatedFirst with this learning rate."""
     B, N, D, Hq, Hkv, hd = c.batch, c.seq, c.D, c.Hq, c.Hkv, c.hd
     lv = lora_views(c, lora_flat) if c.R else None
     thetas = c.rope_thetas()
@@ -41,11 +62,16 @@ def forward_loss(c, used, lora_flat, tok, tgt, x_embed=None):
     x = x.reshape(B, N, D)
     sc = c.lora_scaling if c.R else 0.0
     for L in range(c.NL):
-        g = lambda k: _t(used[k][L])
+        g = lambda k: params[k][L] if (params is not None and k in params) else _t(used[k][L])
         ln = F.rms_norm(x, (D,), g("g_in"), c.eps)
-        q = ln @ g("wq").T
-        k = ln @ g("wk").T
-        v = ln @ g("wv").T
+        if qkv_lr is None:
+            q = ln @ g("wq").T
+            k = ln @ g("wk").T
+            v = ln @ g("wv").T
+        else:
+            q = _LinearUpdatedFirst.apply(ln, g("wq"), qkv_lr)
+            k = _LinearUpdatedFirst.apply(ln, g("wk"), qkv_lr)
+            v = _LinearUpdatedFirst.apply(ln, g("wv"), qkv_lr)
         if c.R:
             q = q + sc * (ln @ lv[L]["A_q"].T) @ lv[L]["B_q"].T
             v = v + sc * (ln @ lv[L]["A_v"].T) @ lv[L]["B_v"].T
@@ -67,7 +93,8 @@ def forward_loss(c, used, lora_flat, tok, tgt, x_embed=None):
             a = F.silu(ln @ g("wg").T) * (ln @ g("wu").T)
             x = x + a @ g("wd").T
     ln = F.rms_norm(x, (D,), _t(used["g_final"]), c.eps)
-    logits = ln.reshape(B * N, D) @ _t(used["lm_head"]).T
+    lm = params["lm_head"] if params is not None else _t(used["lm_head"])
+    logits = ln.reshape(B * N, D) @ lm.T
     loss = F.cross_entropy(logits, torch.as_tensor(tgt.astype(np.int64)), reduction="mean")
     return loss, logits
 
@@ -90,3 +117,18 @@ def train_steps(c, used, lora0, batches, lr, clip=True):
         out.append({"loss": float(loss.detach()), "grad": g.numpy().copy(), "grad_norm": gn,
                     "lora": p.detach().numpy().copy(), "logits": logits.detach().numpy().copy()})
     return out
+
+
+MATS = ("wq", "wk", "wv", "wo", "wg", "wu", "wd")
+
+
+def full_param_grads(c, used, tok, tgt, qkv_lr=None):
+    """Autograd gradients of the mean CE loss w.r.t. every frozen matrix (R = 0).
+    Returns ({name: [per-layer arrays]} + "lm_head", loss, logits)."""
+    params = {k: [_t(w).requires_grad_(True) for w in used[k]] for k in MATS}
+    params["lm_head"] = _t(used["lm_head"]).requires_grad_(True)
+    loss, logits = forward_loss(c, used, None, tok, tgt, params=params, qkv_lr=qkv_lr)
+    loss.backward()
+    grads = {k: [p.grad.numpy().copy() for p in params[k]] for k in MATS}
+    grads["lm_head"] = params["lm_head"].grad.numpy().copy()
+    return grads, float(loss.detach()), logits.detach().numpy().copy()
