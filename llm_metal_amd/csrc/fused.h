@@ -55,6 +55,16 @@ struct AttnFwdArgs {
 };
 void launch_attn_fwd(const AttnFwdArgs &a);
 
+// QKV epilogue + attention in one launch, one workgroup per (sequence, query head); see attn_fused.hip.
+struct AttnFusedFwdArgs {
+    QkvPostArgs q;                // q.rows is not used
+    int batch; float scale;
+    float *probs;                 // [batch][Hq][seq][seq]
+    half_t *out16;                // tiled [rows, Hq*hd], unit scale
+};
+bool attn_fused_fwd_supported(const QkvPostArgs &a);
+void launch_attn_fused_fwd(const AttnFusedFwdArgs &a);
+
 struct AttnBwdArgs {
     Planes dO;                    // [rows][Hq*hd]
     const float *probs, *q, *k, *v; int Hq, Hkv, hd, seq, batch; float scale;

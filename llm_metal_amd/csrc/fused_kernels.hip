@@ -10,6 +10,7 @@
 // of the row in registers between the reductions, and all plane loads of a
 // thread are independent so they are in flight together.
 #include "fused.h"
+#include "planes.h"
 
 namespace lmhip {
 namespace {
@@ -17,39 +18,6 @@ namespace {
 constexpr int TB = 256;
 constexpr int RB = 1024;                                  // threads of a row workgroup
 constexpr int MAXV = 3;                                   // float4 per thread: rows up to 12288 wide
-
-__device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
-{
-    float s = 0.f;
-    const float *p = P.p + row * P.ld + col;
-    for (int i = 0; i < P.S; i++) s += p[(size_t)i * P.stride];
-    return P.row_scale ? s * P.row_scale[row] : s;
-}
-
-// Sum of the planes at four consecutive columns (col % 4 == 0, ld % 4 == 0).
-__device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int col)
-{
-    const float *p = P.p + row * P.ld + col;
-    float4 s = *reinterpret_cast<const float4 *>(p);
-    int i = 1;
-    for (; i + 1 < P.S; i += 2) {
-        const float4 a = *reinterpret_cast<const float4 *>(p + (size_t)i * P.stride);
-        const float4 b = *reinterpret_cast<const float4 *>(p + (size_t)(i + 1) * P.stride);
-        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
-        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
-    }
-    if (i < P.S) {
-        const float4 a = *reinterpret_cast<const float4 *>(p + (size_t)i * P.stride);
-        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
-    }
-    if (P.row_scale) { const float f = P.row_scale[row]; s.x *= f; s.y *= f; s.z *= f; s.w *= f; }
-    return s;
-}
-
-__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
-__device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
-__device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
-__device__ __forceinline__ float sumsq4(float4 v) { return v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
 
 // four consecutive elements (k % 4 == 0) of row `row` of a tiled fp16 operand
 __device__ __forceinline__ void st_tiled4(half_t *out, size_t row, int k, int Kb, float4 v, float s)

@@ -28,6 +28,7 @@ __host__ __device__ inline size_t tiled_index(int r, int k, int Kb)
 
 struct GemmPlan {
     int nb;        // 32-row weight blocks per wave (1 or 2)
+    int nw;        // waves per workgroup (4, 8 or 16): they split the workgroup's K chunk
     int S;         // K chunks = partial planes written
     int steps;     // 64-wide K steps per chunk
     int n_tiles, m_tiles;

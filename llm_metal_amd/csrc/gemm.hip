@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void tile_f16(const half_t *__restrict__ src, 
 struct ProfRec { hipEvent_t a, b; double wbytes; };
 int g_prof_on = 0;
 std::vector<ProfRec> g_prof;
-int g_force_nb = 0, g_force_S = 0;
+int g_force_nb = 0, g_force_S = 0, g_force_nw = 0;
 
 }  // namespace
 
@@ -100,17 +100,19 @@ GemmPlan plan_gemm(int M, int N, int K)
     const int cus = num_cus() > 0 ? num_cus() : 256;
     GemmPlan p{};
     p.nb = g_force_nb ? g_force_nb : (Nb >= 2 ? 2 : 1);
+    p.nw = g_force_nw ? g_force_nw : 4;
     p.n_tiles = (Nb + p.nb - 1) / p.nb;
     p.m_tiles = m_tiles;
     const int base = p.n_tiles * m_tiles;
-    int S = g_force_S ? g_force_S : (3 * cus + base - 1) / base;
+    // about twelve waves per CU in flight, whatever the workgroup size
+    int S = g_force_S ? g_force_S : (12 * cus / p.nw + base - 1) / base;
     if (S < 1) S = 1;
     int steps = (Kb + S - 1) / S;
     if (!g_force_S) {
-        if (steps < 4) steps = 4;
-        if (steps > 40) steps = 40;
+        if (steps < p.nw) steps = p.nw;
+        if (steps > 10 * p.nw) steps = 10 * p.nw;
     }
-    steps = (steps + 3) & ~3;                              // whole steps for each of the four waves
+    steps = (steps + p.nw - 1) / p.nw * p.nw;              // whole steps for each wave
     if (steps > Kb) steps = Kb;
     p.steps = steps;
     p.S = (Kb + steps - 1) / steps;
@@ -123,14 +125,14 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const half_t *W,
                  float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p)
 {
     if (M <= 0 || N <= 0 || K <= 0) return;
-    if (ldp < N || p.S < 1 || p.steps < 1 || (p.nb != 1 && p.nb != 2)) {
+    if (ldp < N || p.S < 1 || p.steps < 1 || (p.nb != 1 && p.nb != 2) || (p.nw != 4 && p.nw != 8 && p.nw != 16)) {
         fprintf(stderr, "[fast_hip] gemm: bad launch M=%d N=%d K=%d ldp=%d plan(nb=%d S=%d steps=%d)\n",
                 M, N, K, ldp, p.nb, p.S, p.steps);
         abort();
     }
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
-    dim3 grid(p.n_tiles, p.S, p.m_tiles), block(256);
-    const size_t lds = (size_t)2 * (2 * p.nb * 16) * 64 * sizeof(float);
+    dim3 grid(p.n_tiles, p.S, p.m_tiles), block(p.nw * 64);
+    const size_t lds = (size_t)(p.nw / 2) * (2 * p.nb * 16) * 64 * sizeof(float);
     // When profiling, the events ride on the dispatch itself (hipExtLaunchKernelGGL), so their
     // difference is the kernel's own execution time without the gaps a separate record adds.
     ProfRec rec{};
@@ -142,12 +144,23 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const half_t *W,
         ev_a = rec.a; ev_b = rec.b;
     }
     const half8 *A8 = reinterpret_cast<const half8 *>(A), *W8 = reinterpret_cast<const half8 *>(W);
-#define GEMM_LAUNCH(NBV, ROT, SC) hipExtLaunchKernelGGL((gemm_tiled_f16<NBV, ROT, SC>), grid, block, lds, stream(), ev_a, ev_b, 0, \
-                                                       A8, a_inv_scale, W8, P, ldp, plane_stride, M, N, Mb, Nb, Kb, p.steps)
-#define GEMM_PICK(NBV, ROT) do { if (a_inv_scale) GEMM_LAUNCH(NBV, ROT, 1); else GEMM_LAUNCH(NBV, ROT, 0); } while (0)
-    if (p.nb == 2) { if (p.rotate) GEMM_PICK(2, 1); else GEMM_PICK(2, 0); }
-    else           { if (p.rotate) GEMM_PICK(1, 1); else GEMM_PICK(1, 0); }
-#undef GEMM_PICK
+    // every instantiation may use more than the default 64 KB of dynamic LDS
+#define GEMM_LAUNCH(NBV, NWV, ROT, SC) do { \
+        static bool attr_set = false; \
+        if (!attr_set) { \
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tiled_f16<NBV, NWV, ROT, SC>), \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (NWV / 2) * (2 * NBV * 16) * 64 * 4)); \
+            attr_set = true; \
+        } \
+        hipExtLaunchKernelGGL((gemm_tiled_f16<NBV, NWV, ROT, SC>), grid, block, lds, stream(), ev_a, ev_b, 0, \
+                              A8, a_inv_scale, W8, P, ldp, plane_stride, M, N, Mb, Nb, Kb, p.steps); } while (0)
+#define GEMM_PICK_SC(NBV, NWV, ROT) do { if (a_inv_scale) GEMM_LAUNCH(NBV, NWV, ROT, 1); else GEMM_LAUNCH(NBV, NWV, ROT, 0); } while (0)
+#define GEMM_PICK_ROT(NBV, NWV) do { if (p.rotate) GEMM_PICK_SC(NBV, NWV, 1); else GEMM_PICK_SC(NBV, NWV, 0); } while (0)
+#define GEMM_PICK_NW(NBV) do { if (p.nw == 4) GEMM_PICK_ROT(NBV, 4); else if (p.nw == 8) GEMM_PICK_ROT(NBV, 8); else GEMM_PICK_ROT(NBV, 16); } while (0)
+    if (p.nb == 2) GEMM_PICK_NW(2); else GEMM_PICK_NW(1);
+#undef GEMM_PICK_NW
+#undef GEMM_PICK_ROT
+#undef GEMM_PICK_SC
 #undef GEMM_LAUNCH
     HIP_CHECK(hipGetLastError());
     if (g_prof_on) g_prof.push_back(rec);
@@ -281,13 +294,13 @@ int hip_gemm_profile_read(double *total_ms, double *total_weight_bytes)
 }
 
 // Times `iters` launches of the GEMM alone on synthetic tiled operands of the given shape
-// (HIP events on the library's stream).  nb / S = 0 let the planner choose; otherwise they
-// force the tile height and K split.  Returns the average milliseconds per launch.
-double hip_gemm_time_shape(int M, int N, int K, int nb, int S, int iters, int *used_nb, int *used_S)
+// (HIP events on the library's stream).  nb / nw / S = 0 let the planner choose; otherwise they
+// force the tile height, the waves per workgroup and the K split.  Returns the average milliseconds per launch.
+double hip_gemm_time_shape(int M, int N, int K, int nb, int nw, int S, int iters, int *used_nb, int *used_S)
 {
-    g_force_nb = nb; g_force_S = S;
+    g_force_nb = nb; g_force_S = S; g_force_nw = nw;
     GemmPlan p = plan_gemm(M, N, K);
-    g_force_nb = 0; g_force_S = 0;
+    g_force_nb = 0; g_force_S = 0; g_force_nw = 0;
     if (used_nb) *used_nb = p.nb;
     if (used_S) *used_S = p.S;
     void *A = nullptr, *W = nullptr, *P = nullptr, *inv = nullptr;

@@ -4,7 +4,7 @@
 
 namespace lmhip {
 
-// grid: x = ceil(Nb / NB) weight-row tiles, y = S (K chunks), z = ceil(M / 64); block = 256.
+// grid: x = ceil(Nb / NB) weight-row tiles, y = S (K chunks), z = ceil(M / 64); block = NW waves of 64.
 // Kb = number of 64-wide K steps of the (padded) reduction; Nb, Mb = 32-row blocks of W and A.
 //
 // Each wave loads one K step (NB weight tiles + 2 activation tiles), waits, issues its MFMAs and
@@ -14,13 +14,16 @@ namespace lmhip {
 // it all workgroups of a chunk ask L2 for the same activation lines at the same moment.
 // SCALE: multiply row m of the result by a_inv_scale[m] here (used when the output is final, S == 1);
 // otherwise the consumer of the partial planes applies the row factors.
-template <int NB, int ROTATE, int SCALE>
-__global__ __launch_bounds__(256, 2) void gemm_tiled_f16(
+// NW (4, 8 or 16 waves) trades partial planes for workgroup size: the waves of a workgroup split its K chunk
+// and add their accumulators through LDS, so a larger workgroup covers a longer chunk and the launch writes
+// fewer planes for the same number of waves in flight.
+template <int NB, int NW, int ROTATE, int SCALE>
+__global__ __launch_bounds__(NW * 64, 2) void gemm_tiled_f16(
     const half8 *__restrict__ A, const float *__restrict__ a_inv_scale, const half8 *__restrict__ W,
     float *__restrict__ P, int ldp, size_t plane_stride,
     int M, int N, int Mb, int Nb, int Kb, int steps_per_chunk)
 {
-    extern __shared__ float red[];                       // [2][2*NB*16 regs][64 lanes]
+    extern __shared__ float red[];                       // [NW/2][2*NB*16 regs][64 lanes]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb0 = blockIdx.x * NB, mb0 = blockIdx.z * 2;
@@ -55,9 +58,9 @@ __global__ __launch_bounds__(256, 2) void gemm_tiled_f16(
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[mb][b][v] = 0.f;
 
-    // wave w takes the K steps w, w+4, w+8, ... of this workgroup's chunk (rotated)
+    // wave w takes the K steps w, w+NW, w+2NW, ... of this workgroup's chunk (rotated)
     const int rot = ROTATE ? (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)nsteps) : 0;
-    for (int i = wave; i < nsteps; i += 4) {
+    for (int i = wave; i < nsteps; i += NW) {
         int kk = i + rot;
         if (kk >= nsteps) kk -= nsteps;
         const size_t o = (size_t)(kb_beg + kk) * 256;    // 4 x 64 half8 per K step
@@ -78,37 +81,32 @@ __global__ __launch_bounds__(256, 2) void gemm_tiled_f16(
                     acc[mb][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mb][j], w[b][j], acc[mb][b], 0, 0, 0);
     }
 
-    // add the four waves' accumulators in two rounds through LDS (lane fastest => conflict-free):
-    // waves 2,3 park theirs and waves 0,1 add them; then wave 1 parks and wave 0 adds and stores.
+    // add the waves' accumulators in log2(NW) rounds through LDS (lane fastest => conflict-free):
+    // in every round the upper half of the remaining waves parks its registers and the lower half adds them
     constexpr int REGS = 2 * NB * 16;
-    float *slot = red + (size_t)(wave & 1) * REGS * 64;
-    if (wave >= 2) {
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+    for (int half = NW / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
+            float *slot = red + (size_t)(wave - half) * REGS * 64;
 #pragma unroll
-            for (int b = 0; b < NB; b++)
+            for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) slot[((mb * NB + b) * 16 + v) * 64 + lane] = acc[mb][b][v];
+                for (int b = 0; b < NB; b++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) slot[((mb * NB + b) * 16 + v) * 64 + lane] = acc[mb][b][v];
+        }
+        __syncthreads();
+        if (wave < half) {
+            const float *slot = red + (size_t)wave * REGS * 64;
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                for (int b = 0; b < NB; b++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[mb][b][v] += slot[((mb * NB + b) * 16 + v) * 64 + lane];
+        }
+        if (half > 1) __syncthreads();
     }
-    __syncthreads();
-    if (wave < 2) {
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int b = 0; b < NB; b++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) acc[mb][b][v] += slot[((mb * NB + b) * 16 + v) * 64 + lane];
-    }
-    __syncthreads();
-    if (wave == 1) {
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int b = 0; b < NB; b++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) red[((mb * NB + b) * 16 + v) * 64 + lane] = acc[mb][b][v];
-    }
-    __syncthreads();
     if (wave != 0) return;
     float *Pp = P + (size_t)blockIdx.y * plane_stride;
 #pragma unroll
@@ -117,7 +115,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tiled_f16(
         for (int b = 0; b < NB; b++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                float sres = acc[mb][b][v] + red[((mb * NB + b) * 16 + v) * 64 + lane];
+                float sres = acc[mb][b][v];
                 // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4
                 const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
                 const int n = (nb0 + b) * 32 + r;

@@ -1,0 +1,40 @@
+// Device helpers shared by the row kernels: reading a GEMM result that is still
+// split into K-chunk planes, and 16-byte loads/stores.
+#pragma once
+#include "fused.h"
+
+namespace lmhip {
+
+__device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
+{
+    float s = 0.f;
+    const float *p = P.p + row * P.ld + col;
+    for (int i = 0; i < P.S; i++) s += p[(size_t)i * P.stride];
+    return P.row_scale ? s * P.row_scale[row] : s;
+}
+
+// Sum of the planes at four consecutive columns (col % 4 == 0, ld % 4 == 0), added in plane order.
+// The loads of up to eight planes are issued together, so their latency is paid once.
+__device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int col)
+{
+    const float *p = P.p + row * P.ld + col;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i0 = 0; i0 < P.S; i0 += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            v[i] = (i0 + i < P.S) ? *reinterpret_cast<const float4 *>(p + (size_t)(i0 + i) * P.stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < 8; i++) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
+    }
+    if (P.row_scale) { const float f = P.row_scale[row]; s.x *= f; s.y *= f; s.z *= f; s.w *= f; }
+    return s;
+}
+
+__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
+__device__ __forceinline__ float sumsq4(float4 v) { return v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+
+
+}  // namespace lmhip

@@ -182,22 +182,27 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         qa.q_fin = at<float>(s->q_fin, (size_t)L * BN * qd); qa.k_fin = at<float>(s->k_fin, (size_t)L * BN * kd);
         qa.v_out = at<float>(s->v_sav, (size_t)L * BN * kd);
         qa.tq = at<float>(s->tq, (size_t)L * BN * (R ? R : 1)); qa.tv = at<float>(s->tv, (size_t)L * BN * (R ? R : 1));
-        launch_qkv_post(qa, BN);
-
         // causal GQA attention                                               [:678-689]
-        AttnFwdArgs aa{};
-        aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
-        aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
-        aa.scale = 1.0f / sqrtf((float)s->hd);
-        aa.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
-        // full-parameter mode keeps the three FFN/attention GEMM operands of every layer
         half_t *attn16 = s->full_param ? at<half_t>(s->attn16, L * s->st_attn) : a16;
+        float *probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
+        const float attn_scale = 1.0f / sqrtf((float)s->hd);
+        if (attn_fused_fwd_supported(qa)) {
+            AttnFusedFwdArgs fa{};
+            fa.q = qa; fa.batch = s->B; fa.scale = attn_scale; fa.probs = probs; fa.out16 = attn16;
+            launch_attn_fused_fwd(fa);
+        } else {
+            launch_qkv_post(qa, BN);
+            AttnFwdArgs aa{};
+            aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
+            aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
+            aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16;
+            launch_attn_fwd(aa);
+        }
+        // full-parameter mode keeps the FFN GEMM operands of every layer as well
         half_t *ln2 = s->full_param ? at<half_t>(s->ln2_16, L * s->st_ln1) : a16;
         float *ln2inv = s->full_param ? at<float>(s->ln2_inv, (size_t)L * BN) : ainv;
         half_t *act16 = s->full_param ? at<half_t>(s->act16, L * s->st_act) : a16;
         float *actinv = s->full_param ? at<float>(s->act_inv, (size_t)L * BN) : ainv;
-        aa.out16 = attn16;
-        launch_attn_fwd(aa);
 
         // o = attn Wo^T; x_mid = x_in + o (Qwen3) | x_in + RN(o; g_post_attn) (Gemma3); ln2 = RN(x_mid; g_ffn_in)   [:696-711]
         Planes po = gemm(s, attn16, at<float>(s->ones), at<half_t>(s->wo, L * s->st_o), D, qd);

@@ -27,6 +27,9 @@ CASES = [
     C1.with_(name="wide_head", NL=1, D=512, Hq=2, Hkv=1, hd=256, IS=512, V=1024, seq=16),   # Gemma-sized heads
     TINY_GEMMA3.with_(name="gemma_seq160", NL=2, seq=160),                # config 5's non-power-of-two length
     C1.with_(name="c1_q8", weight_format="q8_0"),                         # Q8_0 frozen weights
+    C1.with_(name="hd128", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),       # config 3's head shape
+    C1.with_(name="ragged_seq40", NL=2, batch=2, seq=40, R=4, alpha=8.0),                    # rows past the sequence in a 64-row block
+    C1.with_(name="seq17_mqa", NL=1, Hq=4, Hkv=1, seq=17, V=1024),                           # one KV head, odd length
 ]
 
 
