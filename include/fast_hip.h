@@ -130,9 +130,10 @@ void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
 void hip_gemm_profile_enable(int on);
 int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
 /* Microbenchmark of the GEMM alone at one shape (M rows, N x K weight) on synthetic operands,
- * rotating through > 1 GB of distinct weight images.  nb / nw / S = 0: planner's choice, else forced
- * tile height (1, 2), waves per workgroup (4, 8, 16) and K split.  Returns average ms per launch. */
-double hip_gemm_time_shape(int M, int N, int K, int nb, int nw, int S, int iters, int *used_nb, int *used_S);
+ * rotating through > 1 GB of distinct weight images.  nb / S = 0: planner's choice, else forced
+ * tile height (1, 2) and K split.  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
+ * 2 Q8_0 with column scales (transposed image).  Returns average ms per launch. */
+double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S);
 
 #ifdef __cplusplus
 }

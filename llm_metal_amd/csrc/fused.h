@@ -55,16 +55,6 @@ struct AttnFwdArgs {
 };
 void launch_attn_fwd(const AttnFwdArgs &a);
 
-// QKV epilogue + attention in one launch, one workgroup per (sequence, query head); see attn_fused.hip.
-struct AttnFusedFwdArgs {
-    QkvPostArgs q;                // q.rows is not used
-    int batch; float scale;
-    float *probs;                 // [batch][Hq][seq][seq]
-    half_t *out16;                // tiled [rows, Hq*hd], unit scale
-};
-bool attn_fused_fwd_supported(const QkvPostArgs &a);
-void launch_attn_fused_fwd(const AttnFusedFwdArgs &a);
-
 struct AttnBwdArgs {
     Planes dO;                    // [rows][Hq*hd]
     const float *probs, *q, *k, *v; int Hq, Hkv, hd, seq, batch; float scale;
@@ -125,8 +115,10 @@ struct AdamArgs {
     const float *sq_slots; int n_slots;
     const float *hyper;           // device-visible: [0] lr, [1] 1-b1^t, [2] 1-b2^t, written by the host per step
     float b1, b2, eps, wd, max_norm;
-    // fp16 shadows of A_q / A_v inside the fused QKV weight and its transpose
-    half_t *wqkv; size_t wqkv_layer_stride; half_t *wqkvT; size_t wqkvT_layer_stride;   // tiled
+    // fp16 shadows of A_q / A_v: rows a_row0.. of the tiled image wqkv ([*, D]) and columns a_row0.. of the
+    // transposed image wqkvT (kbT K blocks per row block)
+    half_t *wqkv; size_t wqkv_layer_stride; half_t *wqkvT; size_t wqkvT_layer_stride;
+    int a_row0, kbT;
     int NL, D, qd, kd, R; size_t layer_size;
     float *grad_norm_out;         // [1]
 };
@@ -134,7 +126,7 @@ void launch_adamw(const AdamArgs &a);
 
 // fp16 shadow refresh only (after LoRA weights were written from outside)
 void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
-                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size);
+                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size, int a_row0, int kbT);
 
 void launch_fill_f32(float *p, float v, size_t n);
 

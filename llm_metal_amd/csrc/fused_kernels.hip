@@ -758,10 +758,10 @@ __device__ __forceinline__ void shadow_store(const AdamArgs &a, size_t idx, floa
     else if (o >= nA + nBq && o < 2 * nA + nBq) { o -= nA + nBq; rbase = a.R; }
     else return;
     const int r = (int)(o / a.D), d = (int)(o % a.D);
-    const int rowx = a.qd + 2 * a.kd + rbase + r;
+    const int rowx = a.a_row0 + rbase + r;
     const half_t hv = f2h(pv);
     a.wqkv[L * a.wqkv_layer_stride + tiled_index(rowx, d, tiled_kb(a.D))] = hv;
-    a.wqkvT[L * a.wqkvT_layer_stride + tiled_index(d, rowx, tiled_kb(a.qd + 2 * a.kd + 2 * a.R))] = hv;
+    a.wqkvT[L * a.wqkvT_layer_stride + tiled_index(d, rowx, a.kbT)] = hv;
 }
 
 __global__ __launch_bounds__(TB) void k_adamw(AdamArgs a)
@@ -895,13 +895,13 @@ void launch_adamw(const AdamArgs &a)
 }
 
 void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
-                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size)
+                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size, int a_row0, int kbT)
 {
     if (!n) return;
     AdamArgs a{};
     a.p = const_cast<float *>(p); a.n = n; a.wqkv = wqkv; a.wqkv_layer_stride = wqkv_layer_stride;
     a.wqkvT = wqkvT; a.wqkvT_layer_stride = wqkvT_layer_stride;
-    a.D = D; a.qd = qd; a.kd = kd; a.R = R; a.layer_size = layer_size;
+    a.D = D; a.qd = qd; a.kd = kd; a.R = R; a.layer_size = layer_size; a.a_row0 = a_row0; a.kbT = kbT;
     size_t blocks = (n + TB - 1) / TB;
     if (blocks > 4096) blocks = 4096;
     LAUNCH(k_lora_shadow, dim3((unsigned)blocks), dim3(TB), 0, a);

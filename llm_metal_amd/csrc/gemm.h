@@ -26,22 +26,51 @@ __host__ __device__ inline size_t tiled_index(int r, int k, int Kb)
     return ((tile * 4 + ((c & 31) >> 3)) * 64 + ((c >> 5) << 5) + (r & 31)) * 8 + (c & 7);
 }
 
+// Weight operand of the GEMM.  fmt 0: F16 tiles in w16.  fmt 1 / 2: Q8_0 (GGML blocks of 32 int8 with
+// one fp16 scale, src/nn/wmat.c:9-44) re-laid for the kernel: `q` holds the int8 of a 32 x 64 tile as
+// [2][64 lanes][16 bytes] (lane, j, e as in the F16 tile, j = 2 * half + byte / 8), `d` 64 scales per tile.
+//   fmt 1: scales belong to (row, 32-column block): d[tile][lane] is the one scale of that lane's 32 weights;
+//          row blocks from nbq on are F16 tiles in w16 (row block index - nbq).
+//   fmt 2: the transposed image of a Q8_0 matrix: scales belong to (column, 32-row block), d[tile][column];
+//          K steps from kbq on are F16 tiles in w16 ([row block][Kb - kbq]).
+struct WeightOp {
+    const half_t *w16;
+    const uint8_t *q;
+    const half_t *d;
+    int fmt, nbq, kbq;
+};
+inline WeightOp weight_f16(const half_t *w) { return WeightOp{w, nullptr, nullptr, 0, 0, 0}; }
+
 struct GemmPlan {
     int nb;        // 32-row weight blocks per wave (1 or 2)
-    int nw;        // waves per workgroup (4, 8 or 16): they split the workgroup's K chunk
+    int nw;        // waves per workgroup (4): they split the workgroup's K chunk
     int S;         // K chunks = partial planes written
     int steps;     // 64-wide K steps per chunk
     int n_tiles, m_tiles;
     int rotate;    // start each workgroup at a different K step of its chunk
 };
 
-GemmPlan plan_gemm(int M, int N, int K);
+// nbq: Q8_0 row blocks of a fmt-1 operand (an odd count forces one row block per wave)
+GemmPlan plan_gemm(int M, int N, int K, int nbq = 0);
 
 // P[s][m][n] (s < plan.S, plane s at P + s*plane_stride, row stride ldp) =
 //   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k],  A and W in the tiled layout.
 // Pass a_inv_scale = null to leave the row factors to the consumer of the planes.
-void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const half_t *W_tiled,
+void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W,
                  float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p);
+inline void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const half_t *W_tiled,
+                        float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p)
+{
+    launch_gemm(A_tiled, a_inv_scale, weight_f16(W_tiled), P, ldp, plane_stride, M, N, K, p);
+}
+// bytes of weight data one launch streams for an [N, K] operand (2 per F16 weight, 34 per 32 Q8_0 weights)
+double weight_stream_bytes(const WeightOp &W, int N, int K);
+// Q8_0 blocks in the reference's row-major layout ([rows][cols/32] blocks of 34 bytes) -> kernel tiles.
+// Element (r, c) goes to tiled (row_off + r, k_off + c) with row scales (fmt 1), or, transposed, to
+// (row_off + c, k_off + r) with column scales (fmt 2).  Kb_dst = K blocks per row block of the destination.
+// row_off must be a multiple of 32 and k_off of 32 (fmt 1); cols a multiple of 32.
+void launch_tile_q8(const uint8_t *blocks, int rows, int cols, uint8_t *q_tiles, half_t *d_tiles, int Kb_dst,
+                    int row_off, int k_off, int transpose);
 
 // out (tiled [M, K]) = fp16(X[m][k] * s_m), zero in the K padding; inv_scale[m] = 1/s_m
 void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_scale, int M, int K);
@@ -51,5 +80,9 @@ void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, c
 //   element (r, c) goes to tiled(row_off + r, k_off + c), or tiled(row_off + c, k_off + r) when transposed
 void launch_tile_f16(const half_t *src, int rows, int cols, half_t *dst_tiled, int Kb_dst,
                      int row_off, int k_off, int transpose);
+
+// dst (row-major F16 [rows, cols]) <- half(d * q) of a window of a Q8_0 tiled operand (fmt 1 or 2), optionally transposed
+void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, int Kb, int row_off, int k_off, int transpose,
+                      int rows, int cols, half_t *dst);
 
 }  // namespace lmhip

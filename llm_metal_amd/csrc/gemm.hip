@@ -81,10 +81,52 @@ __global__ __launch_bounds__(256) void tile_f16(const half_t *__restrict__ src, 
     }
 }
 
+// Q8_0 blocks (34 bytes: fp16 scale, 32 int8; row-major [rows][cols/32]) -> GEMM tiles, see WeightOp in gemm.h.
+// One thread per source block.
+__global__ __launch_bounds__(256) void tile_q8(const uint8_t *__restrict__ blocks, int rows, int nbk,
+                                                uint8_t *__restrict__ qt, half_t *__restrict__ dt, int Kb_dst,
+                                                int row_off, int k_off, int transpose)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)rows * nbk) return;
+    const int r = (int)(idx / nbk), b = (int)(idx % nbk);
+    const uint8_t *p = blocks + idx * 34;
+    const half_t d = __builtin_bit_cast(half_t, (uint16_t)(p[0] | (p[1] << 8)));
+    for (int i = 0; i < 32; i++) {
+        const int c = b * 32 + i;
+        const int R = transpose ? row_off + c : row_off + r, Kc = transpose ? k_off + r : k_off + c;
+        const size_t tile = (size_t)(R >> 5) * Kb_dst + (Kc >> 6);
+        const int cc = Kc & 63, j = (cc & 31) >> 3, lane = (cc >> 5) * 32 + (R & 31);
+        qt[((tile * 2 + (j >> 1)) * 64 + lane) * 16 + (j & 1) * 8 + (cc & 7)] = p[2 + i];
+        if (transpose && i == 0) dt[tile * 64 + cc] = d;            // one scale per (column Kc, 32-row block)
+    }
+    if (!transpose) {
+        const int R = row_off + r, Kc = k_off + b * 32;
+        const size_t tile = (size_t)(R >> 5) * Kb_dst + (Kc >> 6);
+        dt[tile * 64 + ((Kc >> 5) & 1) * 32 + (R & 31)] = d;
+    }
+}
+
+// Row-major F16 copy of a window of a Q8_0 tiled operand: dst[r][c] = half(d * q) of tiled element
+// (row_off + r, k_off + c), or (row_off + c, k_off + r) when transposed.  fmt as in WeightOp.
+__global__ void untile_q8(const uint8_t *__restrict__ qt, const half_t *__restrict__ dt, int fmt, int Kb,
+                          int row_off, int k_off, int transpose, int rows, int cols, half_t *__restrict__ dst)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)rows * cols) return;
+    const int r = (int)(idx / cols), c = (int)(idx % cols);
+    const int R = transpose ? row_off + c : row_off + r, Kc = transpose ? k_off + r : k_off + c;
+    const size_t tile = (size_t)(R >> 5) * Kb + (Kc >> 6);
+    const int cc = Kc & 63, j = (cc & 31) >> 3, lane = (cc >> 5) * 32 + (R & 31);
+    const int8_t q = (int8_t)qt[((tile * 2 + (j >> 1)) * 64 + lane) * 16 + (j & 1) * 8 + (cc & 7)];
+    const half_t d = fmt == 1 ? dt[tile * 64 + lane] : dt[tile * 64 + cc];
+    dst[idx] = (half_t)__fmul_rn(h2f(d), (float)q);
+}
+
 struct ProfRec { hipEvent_t a, b; double wbytes; };
 int g_prof_on = 0;
 std::vector<ProfRec> g_prof;
-int g_force_nb = 0, g_force_S = 0, g_force_nw = 0;
+int g_force_nb = 0, g_force_S = 0;
 
 }  // namespace
 
@@ -94,18 +136,19 @@ namespace lmhip {
 // (activation bytes through L1/L2 = weight bytes), about three workgroups per CU, chunks of at
 // least 4 and at most 40 K steps (long chunks gain nothing and short ones spread the
 // activation reads over more L2 lines); beyond that, splitting K only adds plane traffic.
-GemmPlan plan_gemm(int M, int N, int K)
+GemmPlan plan_gemm(int M, int N, int K, int nbq)
 {
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), m_tiles = (M + 63) / 64;
     const int cus = num_cus() > 0 ? num_cus() : 256;
     GemmPlan p{};
     p.nb = g_force_nb ? g_force_nb : (Nb >= 2 ? 2 : 1);
-    p.nw = g_force_nw ? g_force_nw : 4;
+    if (nbq & 1) p.nb = 1;                                 // a workgroup must not straddle the Q8_0 / F16 boundary
+    p.nw = 4;
     p.n_tiles = (Nb + p.nb - 1) / p.nb;
     p.m_tiles = m_tiles;
     const int base = p.n_tiles * m_tiles;
     // about twelve waves per CU in flight, whatever the workgroup size
-    int S = g_force_S ? g_force_S : (12 * cus / p.nw + base - 1) / base;
+    int S = g_force_S ? g_force_S : (3 * cus + base - 1) / base;
     if (S < 1) S = 1;
     int steps = (Kb + S - 1) / S;
     if (!g_force_S) {
@@ -121,16 +164,20 @@ GemmPlan plan_gemm(int M, int N, int K)
     return p;
 }
 
-void launch_gemm(const half_t *A, const float *a_inv_scale, const half_t *W,
+void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
                  float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p)
 {
     if (M <= 0 || N <= 0 || K <= 0) return;
-    if (ldp < N || p.S < 1 || p.steps < 1 || (p.nb != 1 && p.nb != 2) || (p.nw != 4 && p.nw != 8 && p.nw != 16)) {
-        fprintf(stderr, "[fast_hip] gemm: bad launch M=%d N=%d K=%d ldp=%d plan(nb=%d S=%d steps=%d)\n",
-                M, N, K, ldp, p.nb, p.S, p.steps);
+    const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
+    bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2) && p.nw == 4 && W.fmt >= 0 && W.fmt <= 2;
+    if (W.fmt == 0) ok = ok && W.w16;
+    if (W.fmt == 1) ok = ok && W.q && W.d && W.nbq >= 0 && W.nbq <= Nb && (W.nbq == Nb || (W.w16 && (W.nbq % p.nb) == 0));
+    if (W.fmt == 2) ok = ok && W.q && W.d && W.kbq >= 0 && W.kbq <= Kb && (W.kbq == Kb || W.w16);
+    if (!ok) {
+        fprintf(stderr, "[fast_hip] gemm: bad launch M=%d N=%d K=%d ldp=%d fmt=%d nbq=%d kbq=%d plan(nb=%d S=%d steps=%d)\n",
+                M, N, K, ldp, W.fmt, W.nbq, W.kbq, p.nb, p.S, p.steps);
         abort();
     }
-    const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
     dim3 grid(p.n_tiles, p.S, p.m_tiles), block(p.nw * 64);
     const size_t lds = (size_t)(p.nw / 2) * (2 * p.nb * 16) * 64 * sizeof(float);
     // When profiling, the events ride on the dispatch itself (hipExtLaunchKernelGGL), so their
@@ -140,30 +187,35 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const half_t *W,
     if (g_prof_on) {
         HIP_CHECK(hipEventCreate(&rec.a));
         HIP_CHECK(hipEventCreate(&rec.b));
-        rec.wbytes = 2.0 * (double)N * (double)K * p.m_tiles;
+        rec.wbytes = weight_stream_bytes(W, N, K);
         ev_a = rec.a; ev_b = rec.b;
     }
-    const half8 *A8 = reinterpret_cast<const half8 *>(A), *W8 = reinterpret_cast<const half8 *>(W);
-    // every instantiation may use more than the default 64 KB of dynamic LDS
-#define GEMM_LAUNCH(NBV, NWV, ROT, SC) do { \
-        static bool attr_set = false; \
-        if (!attr_set) { \
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tiled_f16<NBV, NWV, ROT, SC>), \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (NWV / 2) * (2 * NBV * 16) * 64 * 4)); \
-            attr_set = true; \
-        } \
-        hipExtLaunchKernelGGL((gemm_tiled_f16<NBV, NWV, ROT, SC>), grid, block, lds, stream(), ev_a, ev_b, 0, \
-                              A8, a_inv_scale, W8, P, ldp, plane_stride, M, N, Mb, Nb, Kb, p.steps); } while (0)
-#define GEMM_PICK_SC(NBV, NWV, ROT) do { if (a_inv_scale) GEMM_LAUNCH(NBV, NWV, ROT, 1); else GEMM_LAUNCH(NBV, NWV, ROT, 0); } while (0)
-#define GEMM_PICK_ROT(NBV, NWV) do { if (p.rotate) GEMM_PICK_SC(NBV, NWV, 1); else GEMM_PICK_SC(NBV, NWV, 0); } while (0)
-#define GEMM_PICK_NW(NBV) do { if (p.nw == 4) GEMM_PICK_ROT(NBV, 4); else if (p.nw == 8) GEMM_PICK_ROT(NBV, 8); else GEMM_PICK_ROT(NBV, 16); } while (0)
-    if (p.nb == 2) GEMM_PICK_NW(2); else GEMM_PICK_NW(1);
-#undef GEMM_PICK_NW
+    GemmKArgs g{};
+    g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
+    g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
+    g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
+#define GEMM_LAUNCH(NBV, ROT, SC, WFV) \
+        hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g)
+#define GEMM_PICK_SC(NBV, ROT, WFV) do { if (a_inv_scale) GEMM_LAUNCH(NBV, ROT, 1, WFV); else GEMM_LAUNCH(NBV, ROT, 0, WFV); } while (0)
+#define GEMM_PICK_ROT(NBV, WFV) do { if (p.rotate) GEMM_PICK_SC(NBV, 1, WFV); else GEMM_PICK_SC(NBV, 0, WFV); } while (0)
+#define GEMM_PICK_NB(WFV) do { if (p.nb == 2) GEMM_PICK_ROT(2, WFV); else GEMM_PICK_ROT(1, WFV); } while (0)
+    if (W.fmt == 0) GEMM_PICK_NB(0); else if (W.fmt == 1) GEMM_PICK_NB(1); else GEMM_PICK_NB(2);
+#undef GEMM_PICK_NB
 #undef GEMM_PICK_ROT
 #undef GEMM_PICK_SC
 #undef GEMM_LAUNCH
     HIP_CHECK(hipGetLastError());
     if (g_prof_on) g_prof.push_back(rec);
+}
+
+// Bytes of weight data one launch has to stream for an [N, K] operand: 2 per F16 weight, 34 per 32 Q8_0 weights.
+double weight_stream_bytes(const WeightOp &W, int N, int K)
+{
+    const double nk = (double)N * K;
+    if (W.fmt == 0) return 2.0 * nk;
+    if (W.fmt == 1) { const double nq = (double)(W.nbq * 32 < N ? W.nbq * 32 : N); return nq * K * 34.0 / 32.0 + (N - nq) * K * 2.0; }
+    const double kq = (double)(W.kbq * 64 < K ? W.kbq * 64 : K);
+    return (double)N * kq * 34.0 / 32.0 + (double)N * (K - kq) * 2.0;
 }
 
 void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_scale, int M, int K)
@@ -186,6 +238,30 @@ void launch_tile_f16(const half_t *src, int rows, int cols, half_t *dst_tiled, i
     if (rows <= 0 || cols <= 0) return;
     hipLaunchKernelGGL(tile_f16, dim3((cols + 63) / 64, (rows + 63) / 64), dim3(256), 0, stream(),
                        src, rows, cols, dst_tiled, Kb_dst, row_off, k_off, transpose);
+    HIP_CHECK(hipGetLastError());
+}
+
+void launch_tile_q8(const uint8_t *blocks, int rows, int cols, uint8_t *q_tiles, half_t *d_tiles, int Kb_dst,
+                    int row_off, int k_off, int transpose)
+{
+    if (rows <= 0 || cols < 32) return;
+    if ((cols & 31) || (row_off & 31) || (!transpose && (k_off & 31))) {
+        fprintf(stderr, "[fast_hip] tile_q8: offsets and width must be multiples of 32\n");
+        abort();
+    }
+    const size_t n = (size_t)rows * (cols / 32);
+    hipLaunchKernelGGL(tile_q8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(),
+                       blocks, rows, cols / 32, q_tiles, d_tiles, Kb_dst, row_off, k_off, transpose);
+    HIP_CHECK(hipGetLastError());
+}
+
+void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, int Kb, int row_off, int k_off, int transpose,
+                      int rows, int cols, half_t *dst)
+{
+    const size_t n = (size_t)rows * cols;
+    if (!n) return;
+    hipLaunchKernelGGL(untile_q8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(),
+                       q_tiles, d_tiles, fmt, Kb, row_off, k_off, transpose, rows, cols, dst);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -294,37 +370,48 @@ int hip_gemm_profile_read(double *total_ms, double *total_weight_bytes)
 }
 
 // Times `iters` launches of the GEMM alone on synthetic tiled operands of the given shape
-// (HIP events on the library's stream).  nb / nw / S = 0 let the planner choose; otherwise they
-// force the tile height, the waves per workgroup and the K split.  Returns the average milliseconds per launch.
-double hip_gemm_time_shape(int M, int N, int K, int nb, int nw, int S, int iters, int *used_nb, int *used_S)
+// (HIP events on the library's stream).  nb / S = 0 let the planner choose; otherwise they force the
+// tile height and the K split.  wf = weight format (0 F16, 1 Q8_0 row scales, 2 Q8_0 column scales).
+// Returns the average milliseconds per launch.
+double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S)
 {
-    g_force_nb = nb; g_force_S = S; g_force_nw = nw;
+    g_force_nb = nb; g_force_S = S;
     GemmPlan p = plan_gemm(M, N, K);
-    g_force_nb = 0; g_force_S = 0; g_force_nw = 0;
+    g_force_nb = 0; g_force_S = 0;
     if (used_nb) *used_nb = p.nb;
     if (used_S) *used_S = p.S;
-    void *A = nullptr, *W = nullptr, *P = nullptr, *inv = nullptr;
-    const size_t ab = tiled_elems(M, K) * 2, wb = tiled_elems(N, K) * 2, pb = (size_t)p.S * M * N * 4;
+    void *A = nullptr, *W = nullptr, *D = nullptr, *P = nullptr, *inv = nullptr;
+    const size_t tiles = (size_t)tiled_rb(N) * tiled_kb(K);
+    const size_t ab = tiled_elems(M, K) * 2, wb = wf ? tiles * 2048 : tiles * 4096, db = tiles * 128, pb = (size_t)p.S * M * N * 4;
     // rotate through enough distinct weight images that no launch finds its weights in a cache
     const int nbuf = (int)((size_t)1200 * 1024 * 1024 / wb) + 1;
-    HIP_CHECK(hipMalloc(&A, ab)); HIP_CHECK(hipMalloc(&W, wb * nbuf)); HIP_CHECK(hipMalloc(&P, pb)); HIP_CHECK(hipMalloc(&inv, (size_t)M * 4));
+    HIP_CHECK(hipMalloc(&A, ab)); HIP_CHECK(hipMalloc(&W, wb * nbuf)); HIP_CHECK(hipMalloc(&D, db * nbuf));
+    HIP_CHECK(hipMalloc(&P, pb)); HIP_CHECK(hipMalloc(&inv, (size_t)M * 4));
     HIP_CHECK(hipMemsetAsync(A, 0x11, ab, stream())); HIP_CHECK(hipMemsetAsync(W, 0x11, wb * nbuf, stream()));
+    HIP_CHECK(hipMemsetAsync(D, 0x11, db * nbuf, stream()));
     HIP_CHECK(hipMemsetAsync(inv, 0, (size_t)M * 4, stream()));
     hipEvent_t e0, e1;
     HIP_CHECK(hipEventCreate(&e0)); HIP_CHECK(hipEventCreate(&e1));
     const int saved = g_prof_on;
     g_prof_on = 0;
-    for (int i = 0; i < 3; i++) launch_gemm((half_t *)A, nullptr, (half_t *)W, (float *)P, N, (size_t)M * N, M, N, K, p);
+    auto op = [&](int i) {
+        WeightOp w{};
+        w.fmt = wf;
+        if (wf == 0) w.w16 = (half_t *)((char *)W + (size_t)(i % nbuf) * wb);
+        else { w.q = (uint8_t *)W + (size_t)(i % nbuf) * wb; w.d = (half_t *)((char *)D + (size_t)(i % nbuf) * db);
+               w.nbq = tiled_rb(N); w.kbq = tiled_kb(K); }
+        return w;
+    };
+    for (int i = 0; i < 3; i++) launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
     HIP_CHECK(hipEventRecord(e0, stream()));
-    for (int i = 0; i < iters; i++)
-        launch_gemm((half_t *)A, nullptr, (half_t *)((char *)W + (size_t)(i % nbuf) * wb), (float *)P, N, (size_t)M * N, M, N, K, p);
+    for (int i = 0; i < iters; i++) launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
     HIP_CHECK(hipEventRecord(e1, stream()));
     HIP_CHECK(hipStreamSynchronize(stream()));
     g_prof_on = saved;
     float ms = 0;
     HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
     hipEventDestroy(e0); hipEventDestroy(e1);
-    hipFree(A); hipFree(W); hipFree(P); hipFree(inv);
+    hipFree(A); hipFree(W); hipFree(D); hipFree(P); hipFree(inv);
     return (double)ms / iters;
 }
 

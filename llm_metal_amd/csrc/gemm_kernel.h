@@ -1,8 +1,73 @@
 // The weight-streaming GEMM kernel (device code only; included by gemm.hip).
 #pragma once
 #include "devutil.h"
+#include "gemm.h"
 
 namespace lmhip {
+
+struct GemmKArgs {
+    const half8 *A; const float *a_inv_scale;
+    WeightOp W;
+    float *P; int ldp; size_t plane_stride;
+    int M, N, Mb, Nb, Kb, steps_per_chunk;
+};
+
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+// Eight int8 (two dwords, little endian) -> eight exact fp16 integers.  x ^ 0x80 is q + 128 as an
+// unsigned byte; 0x6400 | byte is the fp16 number 1024 + byte; subtracting 1152 leaves q.
+__device__ __forceinline__ half8 q8_unpack8(uint32_t lo, uint32_t hi)
+{
+    lo ^= 0x80808080u; hi ^= 0x80808080u;
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    u4 bits;
+    bits[0] = __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u);
+    bits[1] = __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u);
+    bits[2] = __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u);
+    bits[3] = __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u);
+    half8 v = __builtin_bit_cast(half8, bits);
+    const half_t off = (half_t)1152.0f;
+    return v - off;
+}
+
+// Weight registers of one 64-wide K step for row block `nb`: w[j] feeds the j-th MFMA of the step.
+// FMT 0: F16 tiles, `kb_stride` K blocks per row block, K block `kt`.
+__device__ __forceinline__ void load_w_f16(half8 (&w)[4], const half_t *W16, int nb, int kb_stride, int kt, int lane)
+{
+    const half8 *p = reinterpret_cast<const half8 *>(W16) + ((size_t)nb * kb_stride + kt) * 256 + lane;
+#pragma unroll
+    for (int j = 0; j < 4; j++) w[j] = __builtin_nontemporal_load(&p[j * 64]);     // streamed once
+}
+
+// FMT 1: Q8_0, one scale per (row, 32 columns): the 32 weights of a lane share one scale.
+// The products d * q are rounded to fp16 once, which is what a stored F16 image of the
+// dequantised weight would hold.
+__device__ __forceinline__ void load_w_q8_rows(half8 (&w)[4], const WeightOp &W, int nb, int kb_stride, int kt, int lane)
+{
+    const size_t tile = (size_t)nb * kb_stride + kt;
+    const uint4v *q = reinterpret_cast<const uint4v *>(W.q) + tile * 128 + lane;
+    const uint4v r0 = __builtin_nontemporal_load(&q[0]), r1 = __builtin_nontemporal_load(&q[64]);
+    const half_t d = __builtin_nontemporal_load(&W.d[tile * 64 + lane]);
+    w[0] = q8_unpack8(r0[0], r0[1]) * d;
+    w[1] = q8_unpack8(r0[2], r0[3]) * d;
+    w[2] = q8_unpack8(r1[0], r1[1]) * d;
+    w[3] = q8_unpack8(r1[2], r1[3]) * d;
+}
+
+// FMT 2: Q8_0 of the transposed matrix: one scale per (column, 32 rows), so a tile (32 rows) has 64
+// column scales and a lane multiplies its weight (j, e) by the scale of column (lane / 32) * 32 + 8 j + e.
+__device__ __forceinline__ void load_w_q8_cols(half8 (&w)[4], const WeightOp &W, int nb, int kb_stride, int kt, int lane)
+{
+    const size_t tile = (size_t)nb * kb_stride + kt;
+    const uint4v *q = reinterpret_cast<const uint4v *>(W.q) + tile * 128 + lane;
+    const uint4v r0 = __builtin_nontemporal_load(&q[0]), r1 = __builtin_nontemporal_load(&q[64]);
+    const half8 *sc = reinterpret_cast<const half8 *>(W.d + tile * 64 + (lane >> 5) * 32);
+    const half8 s0 = sc[0], s1 = sc[1], s2 = sc[2], s3 = sc[3];
+    w[0] = q8_unpack8(r0[0], r0[1]) * s0;
+    w[1] = q8_unpack8(r0[2], r0[3]) * s1;
+    w[2] = q8_unpack8(r1[0], r1[1]) * s2;
+    w[3] = q8_unpack8(r1[2], r1[3]) * s3;
+}
 
 // grid: x = ceil(Nb / NB) weight-row tiles, y = S (K chunks), z = ceil(M / 64); block = NW waves of 64.
 // Kb = number of 64-wide K steps of the (padded) reduction; Nb, Mb = 32-row blocks of W and A.
@@ -17,25 +82,27 @@ namespace lmhip {
 // NW (4, 8 or 16 waves) trades partial planes for workgroup size: the waves of a workgroup split its K chunk
 // and add their accumulators through LDS, so a larger workgroup covers a longer chunk and the launch writes
 // fewer planes for the same number of waves in flight.
-template <int NB, int NW, int ROTATE, int SCALE>
-__global__ __launch_bounds__(NW * 64, 2) void gemm_tiled_f16(
-    const half8 *__restrict__ A, const float *__restrict__ a_inv_scale, const half8 *__restrict__ W,
-    float *__restrict__ P, int ldp, size_t plane_stride,
-    int M, int N, int Mb, int Nb, int Kb, int steps_per_chunk)
+// WF: weight format (WeightOp::fmt).  1: row blocks below W.nbq are Q8_0 tiles, the rest F16 tiles
+// (the trainable LoRA rows of the fused QKV weight); the planner keeps W.nbq a multiple of NB, so a
+// workgroup is of one kind.  2: K steps below W.kbq are Q8_0 tiles with column scales, the rest F16.
+template <int NB, int NW, int ROTATE, int SCALE, int WF>
+__global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 {
     extern __shared__ float red[];                       // [NW/2][2*NB*16 regs][64 lanes]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb0 = blockIdx.x * NB, mb0 = blockIdx.z * 2;
-    const int kb_beg = blockIdx.y * steps_per_chunk;
-    const int nsteps = min(Kb, kb_beg + steps_per_chunk) - kb_beg;
+    const int Kb = g.Kb, Nb = g.Nb, M = g.M, N = g.N;
+    const int kb_beg = blockIdx.y * g.steps_per_chunk;
+    const int nsteps = min(Kb, kb_beg + g.steps_per_chunk) - kb_beg;
 
-    const half8 *wp[NB];
+    int nbi[NB];                                          // row block of each weight tile (clamped: the extra rows are never stored)
     const half8 *ap[2];
 #pragma unroll
-    for (int b = 0; b < NB; b++) wp[b] = W + (size_t)min(nb0 + b, Nb - 1) * Kb * 256 + lane;
+    for (int b = 0; b < NB; b++) nbi[b] = min(nb0 + b, Nb - 1);
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++) ap[mb] = A + (size_t)min(mb0 + mb, Mb - 1) * Kb * 256 + lane;
+    for (int mb = 0; mb < 2; mb++) ap[mb] = g.A + (size_t)min(mb0 + mb, g.Mb - 1) * Kb * 256 + lane;
+    const bool q8_rows = WF == 1 && nb0 < g.W.nbq;
 
     // row factors of the 2 x 16 rows this lane stores, fetched before the K loop so that the
     // epilogue of the last wave does not wait for them
@@ -46,7 +113,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled_f16(
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                rsc[mb][v] = a_inv_scale[min(m, M - 1)];
+                rsc[mb][v] = g.a_inv_scale[min(m, M - 1)];
             }
     }
 
@@ -63,15 +130,23 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled_f16(
     for (int i = wave; i < nsteps; i += NW) {
         int kk = i + rot;
         if (kk >= nsteps) kk -= nsteps;
-        const size_t o = (size_t)(kb_beg + kk) * 256;    // 4 x 64 half8 per K step
+        const int kt = kb_beg + kk;
         half8 a[2][4], w[NB][4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-#pragma unroll
-            for (int b = 0; b < NB; b++) w[b][j] = __builtin_nontemporal_load(&wp[b][o + j * 64]);   // streamed once
-#pragma unroll
-            for (int mb = 0; mb < 2; mb++) a[mb][j] = ap[mb][o + j * 64];
+        for (int b = 0; b < NB; b++) {
+            if (WF == 0) load_w_f16(w[b], g.W.w16, nbi[b], Kb, kt, lane);
+            else if (WF == 1) {
+                if (q8_rows) load_w_q8_rows(w[b], g.W, nbi[b], Kb, kt, lane);
+                else load_w_f16(w[b], g.W.w16, nbi[b] - g.W.nbq, Kb, kt, lane);
+            } else {
+                if (kt < g.W.kbq) load_w_q8_cols(w[b], g.W, nbi[b], g.W.kbq, kt, lane);
+                else load_w_f16(w[b], g.W.w16, nbi[b], Kb - g.W.kbq, kt - g.W.kbq, lane);
+            }
         }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++) a[mb][j] = ap[mb][(size_t)kt * 256 + j * 64];
 #pragma unroll
         for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -108,7 +183,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled_f16(
         if (half > 1) __syncthreads();
     }
     if (wave != 0) return;
-    float *Pp = P + (size_t)blockIdx.y * plane_stride;
+    float *Pp = g.P + (size_t)blockIdx.y * g.plane_stride;
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
 #pragma unroll
@@ -121,7 +196,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled_f16(
                 const int n = (nb0 + b) * 32 + r;
                 if (m < M && n < N) {
                     if (SCALE) sres *= rsc[mb][v];
-                    Pp[(size_t)m * ldp + n] = sres;
+                    Pp[(size_t)m * g.ldp + n] = sres;
                 }
             }
 }

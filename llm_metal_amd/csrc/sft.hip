@@ -35,7 +35,11 @@ struct SFTState {
     // frozen weights, F16 in the GEMM's tiled layout, one arena per matrix kind with a fixed layer stride;
     // the ...T arenas hold the transposed matrices for the dX products
     MetalBuf *wqkv, *wqkvT, *wo, *woT, *wgu, *wguT, *wd, *wdT, *wlm, *wlmT;
-    MetalBuf *q8_blocks;                 // Q8_0 mode: the quantised bytes of every matrix, in upload order
+    // Q8_0-native mode: the frozen matrices stay quantised in HBM (int8 tiles + fp16 scales, both orientations,
+    // 1.0625 bytes per weight and image) and the GEMM dequantises on the fly; wqkv / wqkvT then hold only the F16
+    // tiles of the LoRA A rows.  Layer strides are in tiles (32 x 64 weights).
+    int q8_native;
+    struct Q8Arena { MetalBuf *q, *d, *qT, *dT; size_t st, stT; } zqkv, zo, zgu, zd, zlm;
     MetalBuf *g_in, *g_post_attn, *g_pre_ff, *g_post_ff, *g_q, *g_k, *g_final;
     MetalBuf *emb;                       // fp32 [V, D]
     std::vector<LayerW> layer_views;     // WMat/MetalBuf windows handed out by sft_get_layers-style accessors
@@ -112,6 +116,46 @@ void put_matrix(SFTState *s, const float *src, int rows, int cols, const Dest &a
     metal_buf_free(stage);
 }
 
+struct QDest { MetalBuf *q, *d; size_t tile_off; int Kb; int row_off, k_off, transpose; };
+
+// Q8_0-native upload: quantise (bit-exact GGML blocks) and scatter the blocks into the GEMM's int8 tiles,
+// `a` with row scales, `b` (the transposed image) with column scales.
+void put_matrix_q8(const float *src, int rows, int cols, const QDest &a, const QDest &b)
+{
+    const size_t n = (size_t)rows * cols;
+    MetalBuf *stage = metal_buf_from_data(src, n * sizeof(float));
+    MetalBuf *q8 = metal_buf_create((size_t)rows * (cols / 32) * 34);
+    hip_enqueue_q8_quantize(stage, q8, rows, cols);
+    for (const QDest *d : {&a, &b})
+        launch_tile_q8(at<uint8_t>(q8), rows, cols, at<uint8_t>(d->q, d->tile_off * 2048), at<half_t>(d->d, d->tile_off * 64),
+                       d->Kb, d->row_off, d->k_off, d->transpose);
+    metal_buf_free(q8);                                   // synchronises the stream first
+    metal_buf_free(stage);
+}
+
+enum { W_QKV = 0, W_O, W_GU, W_D, W_LM };
+
+// The weight operand of one GEMM: matrix kind of layer L, as stored (T = false) or transposed.
+WeightOp wop(SFTState *s, int kind, int L, bool T)
+{
+    MetalBuf *w16[5][2] = {{s->wqkv, s->wqkvT}, {s->wo, s->woT}, {s->wgu, s->wguT}, {s->wd, s->wdT}, {s->wlm, s->wlmT}};
+    const size_t st16[5][2] = {{s->st_qkv, s->st_qkvT}, {s->st_o, s->st_oT}, {s->st_gu, s->st_guT}, {s->st_d, s->st_dT}, {0, 0}};
+    if (!s->q8_native) return weight_f16(at<half_t>(w16[kind][T], (size_t)L * st16[kind][T]));
+    SFTState::Q8Arena *z[5] = {&s->zqkv, &s->zo, &s->zgu, &s->zd, &s->zlm};
+    const int qcols = s->qd + 2 * s->kd;                  // quantised part of the fused QKV matrix
+    const int Nfwd[5] = {qcols, s->D, 2 * s->IS, s->D, s->V}, Kfwd[5] = {s->D, s->qd, s->D, s->IS, s->D};
+    WeightOp w{};
+    w.fmt = T ? 2 : 1;
+    const size_t off = (size_t)L * (T ? z[kind]->stT : z[kind]->st);
+    w.q = at<uint8_t>(T ? z[kind]->qT : z[kind]->q, off * 2048);
+    w.d = at<half_t>(T ? z[kind]->dT : z[kind]->d, off * 64);
+    w.nbq = tiled_rb(Nfwd[kind]);                         // forward image: every row block up to the LoRA rows
+    w.kbq = T ? tiled_kb(Nfwd[kind]) : 0;                 // transposed image: the K steps that hold quantised columns
+    (void)Kfwd;
+    if (kind == W_QKV && s->R > 0) w.w16 = at<half_t>(T ? s->wqkvT : s->wqkv, (size_t)L * (T ? s->st_qkvT : s->st_qkv));
+    return w;
+}
+
 size_t max_planes_elems(SFTState *s)
 {
     struct Sh { int N, K; };
@@ -119,7 +163,7 @@ size_t max_planes_elems(SFTState *s)
                          {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->nq_ext}};
     size_t mx = 0;
     for (const Sh &sh : shapes) {
-        GemmPlan p = plan_gemm(s->BN, sh.N, sh.K);
+        GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0);
         const size_t e = (size_t)p.S * s->BN * sh.N;
         if (e > mx) mx = e;
     }
@@ -127,9 +171,9 @@ size_t max_planes_elems(SFTState *s)
 }
 
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
-Planes gemm(SFTState *s, const half_t *A, const float *inv, const half_t *W, int N, int K, float *out = nullptr)
+Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr)
 {
-    GemmPlan p = plan_gemm(s->BN, N, K);
+    GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
     float *P = out ? out : at<float>(s->planes);
     const size_t stride = (size_t)s->BN * N;
     if (!out && (size_t)p.S * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
@@ -169,7 +213,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         launch_norm_rows(n1, BN);
 
         // [q | k | v | tq | tv] = ln1 [Wq; Wk; Wv; A_q; A_v]^T                 [:638-656]
-        Planes pq = gemm(s, ln1, ln1inv, at<half_t>(s->wqkv, L * s->st_qkv), s->nq_ext, D);
+        Planes pq = gemm(s, ln1, ln1inv, wop(s, W_QKV, L, false), s->nq_ext, D);
         QkvPostArgs qa{};
         qa.qkv = pq;
         qa.Bq = at<float>(s->lora, L * s->lsz + (size_t)R * D);
@@ -186,18 +230,12 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         half_t *attn16 = s->full_param ? at<half_t>(s->attn16, L * s->st_attn) : a16;
         float *probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
         const float attn_scale = 1.0f / sqrtf((float)s->hd);
-        if (attn_fused_fwd_supported(qa)) {
-            AttnFusedFwdArgs fa{};
-            fa.q = qa; fa.batch = s->B; fa.scale = attn_scale; fa.probs = probs; fa.out16 = attn16;
-            launch_attn_fused_fwd(fa);
-        } else {
-            launch_qkv_post(qa, BN);
-            AttnFwdArgs aa{};
-            aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
-            aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
-            aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16;
-            launch_attn_fwd(aa);
-        }
+        launch_qkv_post(qa, BN);
+        AttnFwdArgs aa{};
+        aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
+        aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
+        aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16;
+        launch_attn_fwd(aa);
         // full-parameter mode keeps the FFN GEMM operands of every layer as well
         half_t *ln2 = s->full_param ? at<half_t>(s->ln2_16, L * s->st_ln1) : a16;
         float *ln2inv = s->full_param ? at<float>(s->ln2_inv, (size_t)L * BN) : ainv;
@@ -205,7 +243,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         float *actinv = s->full_param ? at<float>(s->act_inv, (size_t)L * BN) : ainv;
 
         // o = attn Wo^T; x_mid = x_in + o (Qwen3) | x_in + RN(o; g_post_attn) (Gemma3); ln2 = RN(x_mid; g_ffn_in)   [:696-711]
-        Planes po = gemm(s, attn16, at<float>(s->ones), at<half_t>(s->wo, L * s->st_o), D, qd);
+        Planes po = gemm(s, attn16, at<float>(s->ones), wop(s, W_O, L, false), D, qd);
         NormRowsArgs n2{};
         n2.x_prev = x_in; n2.branch = po;
         if (gemma) { n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); n2.branch_raw_out = at<float>(s->o_raw, (size_t)L * xsz); }
@@ -215,7 +253,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         launch_norm_rows(n2, BN);
 
         // [gate | up] = ln2 [Wg; Wu]^T; act = silu|gelu(gate) * up              [:715-725]
-        Planes pg = gemm(s, ln2, ln2inv, at<half_t>(s->wgu, L * s->st_gu), 2 * IS, D);
+        Planes pg = gemm(s, ln2, ln2inv, wop(s, W_GU, L, false), 2 * IS, D);
         GluArgs ga{};
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
         ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
@@ -223,7 +261,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         launch_glu_fwd(ga, BN);
 
         // ff = act Wd^T, added by the next row kernel                          [:730-740]
-        pending = gemm(s, act16, actinv, at<half_t>(s->wd, L * s->st_d), D, IS);
+        pending = gemm(s, act16, actinv, wop(s, W_D, L, false), D, IS);
     }
 
     // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
@@ -240,9 +278,9 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
     launch_norm_rows(nf, BN);
     GemmPlan pl = plan_gemm(BN, s->V, D);
     if (pl.S == 1) {
-        gemm(s, lnf, lnfinv, at<half_t>(s->wlm), s->V, D, at<float>(s->logits));
+        gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D, at<float>(s->logits));
     } else {
-        Planes p = gemm(s, lnf, lnfinv, at<half_t>(s->wlm), s->V, D);
+        Planes p = gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D);
         launch_reduce_planes(p.p, p.S, p.stride, p.ld, p.row_scale, at<float>(s->logits), BN, s->V);
     }
 }
@@ -278,7 +316,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
     int cur = 0;                                          // dx ping-pong
 
     // dx = RNB(x_final, dlogits Wlm; g_final)                                [:777-790]
-    Planes p = gemm(s, at<half_t>(s->dl16), at<float>(s->dl_inv), at<half_t>(s->wlmT), D, s->V);
+    Planes p = gemm(s, at<half_t>(s->dl16), at<float>(s->dl_inv), wop(s, W_LM, 0, true), D, s->V);
     if (mode != BWD_LORA)                                                     // [:778-786]
         weight_grad(s, mode, lr, at<half_t>(s->dl16), at<float>(s->dl_inv), s->V, at<half_t>(s->lnf16), at<float>(s->lnf_inv), D,
                     s->wlm, s->wlmT, s->glm, 0, 0);
@@ -291,7 +329,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
 
     for (int L = NL - 1; L >= 0; L--) {
         // FFN: d act = d Wd; (dgate, dup); dln2 = dgate Wg + dup Wu; dx += RNB(x_mid, dln2)   [:798-874]
-        Planes pd = gemm(s, a16, ainv, at<half_t>(s->wdT, L * s->st_dT), IS, D);
+        Planes pd = gemm(s, a16, ainv, wop(s, W_D, L, true), IS, D);
         if (mode != BWD_LORA)                                                 // [:804-811, 842-849]
             weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->act16, L * s->st_act), at<float>(s->act_inv, (size_t)L * BN), IS,
                         s->wd, s->wdT, s->gd, L * s->st_d, L * s->st_dT);
@@ -300,7 +338,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         gb.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); gb.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
         gb.out16 = a16; gb.inv_scale = ainv;
         launch_glu_bwd(gb, BN);
-        Planes pgu = gemm(s, a16, ainv, at<half_t>(s->wguT, L * s->st_guT), D, 2 * IS);
+        Planes pgu = gemm(s, a16, ainv, wop(s, W_GU, L, true), D, 2 * IS);
         if (mode != BWD_LORA)                                                 // gate and up as one matrix [:817-833, 853-869]
             weight_grad(s, mode, lr, a16, ainv, 2 * IS, at<half_t>(s->ln2_16, L * s->st_ln1), at<float>(s->ln2_inv, (size_t)L * BN), D,
                         s->wgu, s->wguT, s->ggu, L * s->st_gu, L * s->st_guT);
@@ -314,7 +352,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         cur ^= 1;
 
         // attention: dO = d Wo; dq, dk, dv                                    [:877-911]
-        Planes pdo = gemm(s, a16, ainv, at<half_t>(s->woT, L * s->st_oT), qd, D);
+        Planes pdo = gemm(s, a16, ainv, wop(s, W_O, L, true), qd, D);
         if (mode != BWD_LORA)                                                 // [:883-901]
             weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->attn16, L * s->st_attn), at<float>(s->ones), qd,
                         s->wo, s->woT, s->go, L * s->st_o, L * s->st_oT);
@@ -360,7 +398,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
                         s->wqkv, s->wqkvT, s->gqkv, L * s->st_qkv, L * s->st_qkvT);
 
         // dln1 = [dq|dk|dv|dh] [Wq;Wk;Wv;A_q;A_v]; dx += RNB(x_in, dln1; g_in); clamp     [:956-980]
-        Planes pl = gemm(s, a16, ainv, at<half_t>(s->wqkvT, L * s->st_qkvT), D, s->nq_ext);
+        Planes pl = gemm(s, a16, ainv, wop(s, W_QKV, L, true), D, s->nq_ext);
         NormBwdArgs n1{};
         n1.dy = pl; n1.x_saved = at<float>(s->xs, (size_t)(2 * L) * xsz); n1.g = at<float>(s->g_in, (size_t)L * D);
         n1.eps = s->eps; n1.D = D; n1.dx_prev = at<float>(s->dx[cur]); n1.dx_out = at<float>(s->dx[cur ^ 1]); n1.clamp = 1e6f;
@@ -392,6 +430,8 @@ void enqueue_update(SFTState *s)
     a.wqkv = at<half_t>(s->wqkv); a.wqkv_layer_stride = s->st_qkv;
     a.wqkvT = at<half_t>(s->wqkvT); a.wqkvT_layer_stride = s->st_qkvT;
     a.NL = s->NL; a.D = s->D; a.qd = s->qd; a.kd = s->kd; a.R = s->R; a.layer_size = s->lsz;
+    a.a_row0 = s->q8_native ? 0 : s->qd + 2 * s->kd;
+    a.kbT = s->q8_native ? tiled_kb(2 * s->R) : tiled_kb(s->nq_ext);
     a.grad_norm_out = at<float>(s->grad_norm);
     launch_adamw(a);
 }
@@ -400,7 +440,8 @@ void refresh_shadow(SFTState *s)
 {
     if (!s->R) return;
     launch_lora_shadow(at<float>(s->lora), s->lora_n, at<half_t>(s->wqkv), s->st_qkv,
-                       at<half_t>(s->wqkvT), s->st_qkvT, s->D, s->qd, s->kd, s->R, s->lsz);
+                       at<half_t>(s->wqkvT), s->st_qkvT, s->D, s->qd, s->kd, s->R, s->lsz,
+                       s->q8_native ? 0 : s->qd + 2 * s->kd, s->q8_native ? tiled_kb(2 * s->R) : tiled_kb(s->nq_ext));
 }
 
 MetalBuf *host_buf(size_t bytes, void **cpu)
@@ -446,32 +487,69 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
         return nullptr;
     }
 
-    // ---- frozen weights: tiled F16 arenas plus transposed images for the dX products ----
-    s->st_qkv = tiled_elems(s->nq_ext, D); s->st_qkvT = tiled_elems(D, s->nq_ext);
-    s->st_o = tiled_elems(D, qd);          s->st_oT = tiled_elems(qd, D);
-    s->st_gu = tiled_elems(2 * IS, D);     s->st_guT = tiled_elems(D, 2 * IS);
-    s->st_d = tiled_elems(D, IS);          s->st_dT = tiled_elems(IS, D);
+    // ---- frozen weights: tiled arenas plus transposed images for the dX products ----
+    // Q8_0 weights stay quantised when the fused QKV matrix splits into quantised and LoRA parts on tile
+    // boundaries; otherwise (and in full-parameter mode, which rewrites the weights) they are stored as the
+    // F16 image of their dequantised values.
+    s->q8_native = !weight_format && !s->full_param && (qd % 32) == 0 && (kd % 32) == 0 && ((qd + 2 * kd) % 64) == 0;
+    const int kbD = tiled_kb(D), kbQ = tiled_kb(qd), kbI = tiled_kb(IS), kb2I = tiled_kb(2 * IS), kbX = tiled_kb(s->nq_ext);
     s->st_ln1 = tiled_elems(BN, D);
-    s->wqkv = hbuf(NL * s->st_qkv); s->wqkvT = hbuf(NL * s->st_qkvT);
-    s->wo = hbuf(NL * s->st_o);     s->woT = hbuf(NL * s->st_oT);
-    s->wgu = hbuf(NL * s->st_gu);   s->wguT = hbuf(NL * s->st_guT);
-    s->wd = hbuf(NL * s->st_d);     s->wdT = hbuf(NL * s->st_dT);
-    s->wlm = hbuf(tiled_elems(V, D)); s->wlmT = hbuf(tiled_elems(D, V));
-    for (MetalBuf *b : {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT})
-        HIP_CHECK(hipMemsetAsync(dptr(b), 0, b->size, stream()));        // row and K padding must read as zero
+    if (!s->q8_native) {
+        s->st_qkv = tiled_elems(s->nq_ext, D); s->st_qkvT = tiled_elems(D, s->nq_ext);
+        s->st_o = tiled_elems(D, qd);          s->st_oT = tiled_elems(qd, D);
+        s->st_gu = tiled_elems(2 * IS, D);     s->st_guT = tiled_elems(D, 2 * IS);
+        s->st_d = tiled_elems(D, IS);          s->st_dT = tiled_elems(IS, D);
+        s->wqkv = hbuf(NL * s->st_qkv); s->wqkvT = hbuf(NL * s->st_qkvT);
+        s->wo = hbuf(NL * s->st_o);     s->woT = hbuf(NL * s->st_oT);
+        s->wgu = hbuf(NL * s->st_gu);   s->wguT = hbuf(NL * s->st_guT);
+        s->wd = hbuf(NL * s->st_d);     s->wdT = hbuf(NL * s->st_dT);
+        s->wlm = hbuf(tiled_elems(V, D)); s->wlmT = hbuf(tiled_elems(D, V));
+    } else {
+        const int qc = qd + 2 * kd;
+        auto arena = [&](SFTState::Q8Arena &z, int Nw, int Kw, int layers, int kq_T) {
+            z.st = (size_t)tiled_rb(Nw) * tiled_kb(Kw);       // forward image [Nw, Kw]
+            z.stT = (size_t)tiled_rb(Kw) * kq_T;              // transposed image [Kw, Nw]: kq_T quantised K steps
+            z.q = metal_buf_create(layers * z.st * 2048);   z.d = hbuf(layers * z.st * 64);
+            z.qT = metal_buf_create(layers * z.stT * 2048); z.dT = hbuf(layers * z.stT * 64);
+        };
+        arena(s->zqkv, qc, D, NL, qc / 64);
+        arena(s->zo, D, qd, NL, kbD);
+        arena(s->zgu, 2 * IS, D, NL, kb2I);
+        arena(s->zd, D, IS, NL, kbD);
+        arena(s->zlm, V, D, 1, tiled_kb(V));
+        // F16 tiles of the LoRA A rows: [2R, D] next to the forward image, [D, 2R] next to the transposed one
+        s->st_qkv = R ? tiled_elems(2 * R, D) : 0; s->st_qkvT = R ? tiled_elems(D, 2 * R) : 0;
+        s->wqkv = hbuf(R ? NL * s->st_qkv : 1); s->wqkvT = hbuf(R ? NL * s->st_qkvT : 1);
+    }
+    for (MetalBuf *b : {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT,
+                        s->zqkv.q, s->zqkv.d, s->zqkv.qT, s->zqkv.dT, s->zo.q, s->zo.d, s->zo.qT, s->zo.dT,
+                        s->zgu.q, s->zgu.d, s->zgu.qT, s->zgu.dT, s->zd.q, s->zd.d, s->zd.qT, s->zd.dT,
+                        s->zlm.q, s->zlm.d, s->zlm.qT, s->zlm.dT})
+        if (b) HIP_CHECK(hipMemsetAsync(dptr(b), 0, b->size, stream()));     // row and K padding must read as zero
     s->g_in = fbuf((size_t)NL * D); s->g_post_attn = fbuf((size_t)NL * D);
     s->g_pre_ff = fbuf((size_t)NL * D); s->g_post_ff = fbuf((size_t)NL * D);
     s->g_q = fbuf((size_t)NL * s->hd); s->g_k = fbuf((size_t)NL * s->hd);
-    const int kbD = tiled_kb(D), kbQ = tiled_kb(qd), kbI = tiled_kb(IS), kb2I = tiled_kb(2 * IS), kbX = tiled_kb(s->nq_ext);
     for (int L = 0; L < NL; L++) {
         const LayerWeightRef *r = &m->layers[L];
-        put_matrix(s, r->q_proj.data, qd, D, {s->wqkv, L * s->st_qkv, kbD, 0, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, 0, 1});
-        put_matrix(s, r->k_proj.data, kd, D, {s->wqkv, L * s->st_qkv, kbD, qd, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, qd, 1});
-        put_matrix(s, r->v_proj.data, kd, D, {s->wqkv, L * s->st_qkv, kbD, qd + kd, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, qd + kd, 1});
-        put_matrix(s, r->o_proj.data, D, qd, {s->wo, L * s->st_o, kbQ, 0, 0, 0}, {s->woT, L * s->st_oT, kbD, 0, 0, 1});
-        put_matrix(s, r->gate_proj.data, IS, D, {s->wgu, L * s->st_gu, kbD, 0, 0, 0}, {s->wguT, L * s->st_guT, kb2I, 0, 0, 1});
-        put_matrix(s, r->up_proj.data, IS, D, {s->wgu, L * s->st_gu, kbD, IS, 0, 0}, {s->wguT, L * s->st_guT, kb2I, 0, IS, 1});
-        put_matrix(s, r->down_proj.data, D, IS, {s->wd, L * s->st_d, kbI, 0, 0, 0}, {s->wdT, L * s->st_dT, kbD, 0, 0, 1});
+        if (!s->q8_native) {
+            put_matrix(s, r->q_proj.data, qd, D, {s->wqkv, L * s->st_qkv, kbD, 0, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, 0, 1});
+            put_matrix(s, r->k_proj.data, kd, D, {s->wqkv, L * s->st_qkv, kbD, qd, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, qd, 1});
+            put_matrix(s, r->v_proj.data, kd, D, {s->wqkv, L * s->st_qkv, kbD, qd + kd, 0, 0}, {s->wqkvT, L * s->st_qkvT, kbX, 0, qd + kd, 1});
+            put_matrix(s, r->o_proj.data, D, qd, {s->wo, L * s->st_o, kbQ, 0, 0, 0}, {s->woT, L * s->st_oT, kbD, 0, 0, 1});
+            put_matrix(s, r->gate_proj.data, IS, D, {s->wgu, L * s->st_gu, kbD, 0, 0, 0}, {s->wguT, L * s->st_guT, kb2I, 0, 0, 1});
+            put_matrix(s, r->up_proj.data, IS, D, {s->wgu, L * s->st_gu, kbD, IS, 0, 0}, {s->wguT, L * s->st_guT, kb2I, 0, IS, 1});
+            put_matrix(s, r->down_proj.data, D, IS, {s->wd, L * s->st_d, kbI, 0, 0, 0}, {s->wdT, L * s->st_dT, kbD, 0, 0, 1});
+        } else {
+            const int kqT = (qd + 2 * kd) / 64;
+            SFTState::Q8Arena &zq = s->zqkv, &zo = s->zo, &zg = s->zgu, &zd = s->zd;
+            put_matrix_q8(r->q_proj.data, qd, D, {zq.q, zq.d, L * zq.st, kbD, 0, 0, 0}, {zq.qT, zq.dT, L * zq.stT, kqT, 0, 0, 1});
+            put_matrix_q8(r->k_proj.data, kd, D, {zq.q, zq.d, L * zq.st, kbD, qd, 0, 0}, {zq.qT, zq.dT, L * zq.stT, kqT, 0, qd, 1});
+            put_matrix_q8(r->v_proj.data, kd, D, {zq.q, zq.d, L * zq.st, kbD, qd + kd, 0, 0}, {zq.qT, zq.dT, L * zq.stT, kqT, 0, qd + kd, 1});
+            put_matrix_q8(r->o_proj.data, D, qd, {zo.q, zo.d, L * zo.st, kbQ, 0, 0, 0}, {zo.qT, zo.dT, L * zo.stT, kbD, 0, 0, 1});
+            put_matrix_q8(r->gate_proj.data, IS, D, {zg.q, zg.d, L * zg.st, kbD, 0, 0, 0}, {zg.qT, zg.dT, L * zg.stT, kb2I, 0, 0, 1});
+            put_matrix_q8(r->up_proj.data, IS, D, {zg.q, zg.d, L * zg.st, kbD, IS, 0, 0}, {zg.qT, zg.dT, L * zg.stT, kb2I, 0, IS, 1});
+            put_matrix_q8(r->down_proj.data, D, IS, {zd.q, zd.d, L * zd.st, kbI, 0, 0, 0}, {zd.qT, zd.dT, L * zd.stT, kbD, 0, 0, 1});
+        }
         metal_buf_write(s->g_in, (size_t)L * D * 4, r->input_norm_g, (size_t)D * 4);
         metal_buf_write(s->g_post_attn, (size_t)L * D * 4, r->post_attn_norm_g, (size_t)D * 4);
         if (r->pre_ff_norm_g) metal_buf_write(s->g_pre_ff, (size_t)L * D * 4, r->pre_ff_norm_g, (size_t)D * 4);
@@ -479,10 +557,10 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
         metal_buf_write(s->g_q, (size_t)L * s->hd * 4, r->q_norm_g, (size_t)s->hd * 4);
         metal_buf_write(s->g_k, (size_t)L * s->hd * 4, r->k_norm_g, (size_t)s->hd * 4);
     }
-    put_matrix(s, m->lm_head, V, D, {s->wlm, 0, kbD, 0, 0, 0}, {s->wlmT, 0, tiled_kb(V), 0, 0, 1});
+    if (!s->q8_native) put_matrix(s, m->lm_head, V, D, {s->wlm, 0, kbD, 0, 0, 0}, {s->wlmT, 0, tiled_kb(V), 0, 0, 1});
+    else put_matrix_q8(m->lm_head, V, D, {s->zlm.q, s->zlm.d, 0, kbD, 0, 0, 0}, {s->zlm.qT, s->zlm.dT, 0, tiled_kb(V), 0, 0, 1});
     s->g_final = metal_buf_from_data(m->final_norm_g, (size_t)D * 4);
     s->emb = metal_buf_from_data(m->token_emb, (size_t)V * D * 4);
-    s->q8_blocks = nullptr;
 
     // ---- RoPE tables: one per distinct theta (Gemma3 has two) ----
     {
@@ -598,7 +676,8 @@ void sft_state_free(SFTState *s)
     metal_flush();
     for (MetalBuf *b : s->lora_views) metal_buf_free(b);
     for (MetalBuf *b : s->grad_views) metal_buf_free(b);
-    MetalBuf *all[] = {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT, s->q8_blocks,
+    MetalBuf *all[] = {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT, s->zqkv.q, s->zqkv.d, s->zqkv.qT, s->zqkv.dT, s->zo.q, s->zo.d, s->zo.qT, s->zo.dT,
+                       s->zgu.q, s->zgu.d, s->zgu.qT, s->zgu.dT, s->zd.q, s->zd.d, s->zd.qT, s->zd.dT, s->zlm.q, s->zlm.d, s->zlm.qT, s->zlm.dT,
                        s->rope_tabs, s->g_in, s->g_post_attn, s->g_pre_ff, s->g_post_ff, s->g_q, s->g_k, s->g_final, s->emb,
                        s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
@@ -712,7 +791,12 @@ void sft_copy_matrix_f16(SFTState *s, int layer, int which, int source, uint16_t
     if (layer < 0 || layer >= s->NL || (source == 2 && !sel.G)) return;
     const size_t n = (size_t)sel.rows * sel.N;
     MetalBuf *tmp = hbuf(n);
-    if (source == 1)
+    if (s->q8_native) {                                   // dequantised values of the quantised tiles
+        const int kind = which <= 2 ? W_QKV : (which == 3 ? W_O : (which <= 5 ? W_GU : (which == 6 ? W_D : W_LM)));
+        const WeightOp w = wop(s, kind, layer, source == 1);
+        if (source == 1) launch_untile_q8(w.q, w.d, 2, w.kbq, 0, sel.row_off, 1, sel.rows, sel.N, at<half_t>(tmp));
+        else launch_untile_q8(w.q, w.d, 1, tiled_kb(sel.N), sel.row_off, 0, 0, sel.rows, sel.N, at<half_t>(tmp));
+    } else if (source == 1)
         launch_untile_f16(at<half_t>(sel.WT, layer * sel.stT), tiled_kb(sel.M), 0, sel.row_off, 1, sel.rows, sel.N, at<half_t>(tmp));
     else
         launch_untile_f16(at<half_t>(source == 2 ? sel.G : sel.W, layer * sel.st), tiled_kb(sel.N), sel.row_off, 0, 0, sel.rows, sel.N, at<half_t>(tmp));
@@ -857,12 +941,18 @@ LayerW *sft_get_layers(SFTState *s)
         }
     }
     for (int L = 0; L < NL; L++) {
-        struct Src { MetalBuf *W; size_t st; int N, row_off; };
-        const Src src[7] = {{s->wqkv, s->st_qkv, D, 0}, {s->wqkv, s->st_qkv, D, qd}, {s->wqkv, s->st_qkv, D, qd + kd},
-                            {s->wo, s->st_o, qd, 0}, {s->wgu, s->st_gu, D, 0}, {s->wgu, s->st_gu, D, IS}, {s->wd, s->st_d, IS, 0}};
-        for (int w = 0; w < 7; w++)
-            launch_untile_f16(at<half_t>(src[w].W, L * src[w].st), tiled_kb(src[w].N), src[w].row_off, 0, 0, rows[w], cols[w],
-                              at<half_t>(s->wmats_out[(size_t)L * 7 + w].mbuf));
+        struct Src { MetalBuf *W; size_t st; int N, row_off, kind; };
+        const Src src[7] = {{s->wqkv, s->st_qkv, D, 0, W_QKV}, {s->wqkv, s->st_qkv, D, qd, W_QKV}, {s->wqkv, s->st_qkv, D, qd + kd, W_QKV},
+                            {s->wo, s->st_o, qd, 0, W_O}, {s->wgu, s->st_gu, D, 0, W_GU}, {s->wgu, s->st_gu, D, IS, W_GU}, {s->wd, s->st_d, IS, 0, W_D}};
+        for (int w = 0; w < 7; w++) {
+            half_t *out = at<half_t>(s->wmats_out[(size_t)L * 7 + w].mbuf);
+            if (s->q8_native) {
+                const WeightOp op = wop(s, src[w].kind, L, false);
+                launch_untile_q8(op.q, op.d, 1, tiled_kb(src[w].N), src[w].row_off, 0, 0, rows[w], cols[w], out);
+            } else {
+                launch_untile_f16(at<half_t>(src[w].W, L * src[w].st), tiled_kb(src[w].N), src[w].row_off, 0, 0, rows[w], cols[w], out);
+            }
+        }
     }
     return s->layers_out.data();
 }
@@ -871,7 +961,8 @@ WMat *sft_get_lm_head(SFTState *s)
 {
     WMat &m = s->lm_head_out;
     if (!m.mbuf) { m.rows = s->V; m.cols = s->D; m.nb = s->D / 32; m.mbuf = hbuf((size_t)s->V * s->D); }
-    launch_untile_f16(at<half_t>(s->wlm), tiled_kb(s->D), 0, 0, 0, s->V, s->D, at<half_t>(m.mbuf));
+    if (s->q8_native) { const WeightOp op = wop(s, W_LM, 0, false); launch_untile_q8(op.q, op.d, 1, tiled_kb(s->D), 0, 0, 0, s->V, s->D, at<half_t>(m.mbuf)); }
+    else launch_untile_f16(at<half_t>(s->wlm), tiled_kb(s->D), 0, 0, 0, s->V, s->D, at<half_t>(m.mbuf));
     return &m;
 }
 

@@ -30,6 +30,12 @@ CASES = [
     C1.with_(name="hd128", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),       # config 3's head shape
     C1.with_(name="ragged_seq40", NL=2, batch=2, seq=40, R=4, alpha=8.0),                    # rows past the sequence in a 64-row block
     C1.with_(name="seq17_mqa", NL=1, Hq=4, Hkv=1, seq=17, V=1024),                           # one KV head, odd length
+    # Q8_0 kept quantised in HBM: widths that are multiples of 32 but not of 64 (half-filled last K tile), an odd
+    # number of vocabulary row blocks, Gemma3 order; and a head layout whose fused QKV matrix does not split on
+    # tile boundaries, which falls back to the F16 image of the dequantised values
+    C1.with_(name="q8_odd_blocks", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format="q8_0"),
+    TINY_GEMMA3.with_(name="gemma_q8", weight_format="q8_0"),
+    C1.with_(name="q8_fallback", NL=2, D=128, Hq=3, Hkv=1, hd=32, IS=256, V=1024, seq=24, weight_format="q8_0"),
 ]
 
 
@@ -73,6 +79,24 @@ def test_train_steps_match_oracle(cfg):
         assert (d_ref != 0).mean() > 0.99
         assert rel(d_gpu, d_ref) < 0.1
         assert (np.sign(d_gpu) == np.sign(d_ref)).mean() > 0.97
+
+
+def test_q8_tiles_hold_the_dequantised_values_in_both_images():
+    """Q8_0 weights stay quantised on the device (int8 tiles with row scales, transposed twin with column
+    scales).  Read back through the dequantising accessor, both images must equal half(d * q) of the
+    reference's blocks (src/nn/wmat.c:19-44) bit for bit."""
+    cfg = C1.with_(name="q8_images", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=16, weight_format="q8_0")
+    model = make_model(cfg, seed=21)
+    used = oracle.weights_as_used(model, "q8")
+    with SFTState(cfg, model) as st:
+        for L in range(cfg.NL):
+            for k in ("wq", "wk", "wv", "wo", "wg", "wu", "wd"):
+                want = oracle.f32_to_f16_bits(used[k][L])
+                assert np.array_equal(st.matrix_f16(L, k, 0), want), (L, k, "forward image")
+                assert np.array_equal(st.matrix_f16(L, k, 1), want), (L, k, "transposed image")
+        want = oracle.f32_to_f16_bits(used["lm_head"])
+        assert np.array_equal(st.matrix_f16(0, "lm_head", 0), want)
+        assert np.array_equal(st.matrix_f16(0, "lm_head", 1), want)
 
 
 def test_zero_b_gives_zero_da_and_training_reduces_loss():
