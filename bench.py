@@ -141,7 +141,7 @@ def main():
     gbs = wb.value / (tms.value * 1e-3) / 1e9 if tms.value > 0 else 0.0
     roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "gemm_tiled_f16", "launches_per_step": n // prof_steps,
+                "kernel": "gemm_tiled", "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                 "weight_bytes_per_step": wb.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}

@@ -65,8 +65,10 @@ C2 = SFTConfig("c2_gemma3_1b", GEMMA3, NL=26, D=1152, Hq=4, Hkv=1, hd=256, IS=69
 C3 = SFTConfig("c3_qwen3_4b_f16", QWEN3, NL=36, D=2560, Hq=32, Hkv=8, hd=128, IS=9728, V=151936)
 C4 = C3.with_(name="c4_qwen3_4b_q8", batch=4, seq=512, weight_format="q8_0")
 C5 = C2.with_(name="c5_gemma3_1b_grpo", batch=1, seq=160, R=0)
+# config 3's step on Q8_0 weights: the dequant-fused weight-streaming GEMM at M = 64
+C3Q = C3.with_(name="c3_qwen3_4b_q8_seq64", weight_format="q8_0")
 
 # small Gemma3-shaped case for parity tests (4-norm ordering, GeGLU, tied head, mixed thetas)
 TINY_GEMMA3 = SFTConfig("tiny_gemma3", GEMMA3, NL=7, D=128, Hq=4, Hkv=1, hd=32, IS=384, V=2048, tied=True, seq=32)
 
-CONFIGS = {c.name: c for c in (C1, C2, C3, C4, C5, TINY_GEMMA3)}
+CONFIGS = {c.name: c for c in (C1, C2, C3, C4, C5, C3Q, TINY_GEMMA3)}

@@ -62,6 +62,11 @@ struct AttnBwdArgs {
     float *dq, *dk, *dv;          // [rows][Hq*hd], [rows][Hkv*hd] x2 (post-RoPE domain)
 };
 void launch_attn_bwd(const AttnBwdArgs &a);
+// The same two operations on the fp32 matrix cores (attn_mfma.hip): head_dim a multiple of 32 and a
+// 32-row block of scores within the LDS budget; the wave-per-query kernels above remain the general path.
+bool attn_mfma_supported(int hd, int seq);
+void launch_attn_fwd_mfma(const AttnFwdArgs &a);
+void launch_attn_bwd_mfma(const AttnBwdArgs &a);
 
 struct QkvBwdArgs {
     const float *dq, *dk, *dv;    // post-RoPE-domain gradients

@@ -235,7 +235,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
         aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16;
-        launch_attn_fwd(aa);
+        if (attn_mfma_supported(s->hd, s->N)) launch_attn_fwd_mfma(aa); else launch_attn_fwd(aa);
         // full-parameter mode keeps the FFN GEMM operands of every layer as well
         half_t *ln2 = s->full_param ? at<half_t>(s->ln2_16, L * s->st_ln1) : a16;
         float *ln2inv = s->full_param ? at<float>(s->ln2_inv, (size_t)L * BN) : ainv;
@@ -365,7 +365,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         ab.scale = 1.0f / sqrtf((float)s->hd);
         ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore);
         ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv);
-        launch_attn_bwd(ab);
+        if (attn_mfma_supported(s->hd, s->N)) launch_attn_bwd_mfma(ab); else launch_attn_bwd(ab);
 
         // inverse RoPE, QK-norm backward, dh; LoRA gradients                  [:912-966]
         QkvBwdArgs qb{};
