@@ -129,6 +129,7 @@ void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
  * enable and adds up their durations (ms) and weight bytes. */
 void hip_gemm_profile_enable(int on);
 int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
+int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double *total_flops);
 /* Microbenchmark of the GEMM alone at one shape (M rows, N x K weight) on synthetic operands,
  * rotating through > 1 GB of distinct weight images.  nb / S = 0: planner's choice, else forced
  * tile height (1, 2) and K split.  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),

@@ -63,8 +63,15 @@ inline void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const h
 {
     launch_gemm(A_tiled, a_inv_scale, weight_f16(W_tiled), P, ldp, plane_stride, M, N, K, p);
 }
+// non-zero while per-launch GEMM events are being recorded (hip_gemm_profile_enable)
+int gemm_profiling();
+// when profiling: registers one launch (weight bytes, flops) and hands out the two events to attach to its dispatch
+bool gemm_prof_begin(double wbytes, double flops, hipEvent_t *a, hipEvent_t *b);
 // bytes of weight data one launch streams for an [N, K] operand (2 per F16 weight, 34 per 32 Q8_0 weights)
 double weight_stream_bytes(const WeightOp &W, int N, int K);
+// C[m][n] (row stride ldc) = a_inv_scale[m] * sum_k A[m][k] W[n][k] in one launch of 128 x 128 output blocks staged
+// through LDS (gemm_big.hip): the path for M of several hundred rows and more, where the product is MFMA bound.
+void launch_gemm_big(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K);
 // Q8_0 blocks in the reference's row-major layout ([rows][cols/32] blocks of 34 bytes) -> kernel tiles.
 // Element (r, c) goes to tiled (row_off + r, k_off + c) with row scales (fmt 1), or, transposed, to
 // (row_off + c, k_off + r) with column scales (fmt 2).  Kb_dst = K blocks per row block of the destination.

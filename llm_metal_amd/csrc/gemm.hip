@@ -123,7 +123,7 @@ __global__ void untile_q8(const uint8_t *__restrict__ qt, const half_t *__restri
     dst[idx] = (half_t)__fmul_rn(h2f(d), (float)q);
 }
 
-struct ProfRec { hipEvent_t a, b; double wbytes; };
+struct ProfRec { hipEvent_t a, b; double wbytes, flops; };
 int g_prof_on = 0;
 std::vector<ProfRec> g_prof;
 int g_force_nb = 0, g_force_S = 0;
@@ -188,14 +188,16 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         HIP_CHECK(hipEventCreate(&rec.a));
         HIP_CHECK(hipEventCreate(&rec.b));
         rec.wbytes = weight_stream_bytes(W, N, K);
+        rec.flops = 2.0 * M * N * K;
         ev_a = rec.a; ev_b = rec.b;
     }
     GemmKArgs g{};
     g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
     g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
     g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
-#define GEMM_LAUNCH(NBV, ROT, SC, WFV) \
-        hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g)
+#define GEMM_LAUNCH(NBV, ROT, SC, WFV) do { \
+        if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
+        else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), g); } while (0)
 #define GEMM_PICK_SC(NBV, ROT, WFV) do { if (a_inv_scale) GEMM_LAUNCH(NBV, ROT, 1, WFV); else GEMM_LAUNCH(NBV, ROT, 0, WFV); } while (0)
 #define GEMM_PICK_ROT(NBV, WFV) do { if (p.rotate) GEMM_PICK_SC(NBV, 1, WFV); else GEMM_PICK_SC(NBV, 0, WFV); } while (0)
 #define GEMM_PICK_NB(WFV) do { if (p.nb == 2) GEMM_PICK_ROT(2, WFV); else GEMM_PICK_ROT(1, WFV); } while (0)
@@ -263,6 +265,20 @@ void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, in
     hipLaunchKernelGGL(untile_q8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(),
                        q_tiles, d_tiles, fmt, Kb, row_off, k_off, transpose, rows, cols, dst);
     HIP_CHECK(hipGetLastError());
+}
+
+int gemm_profiling() { return g_prof_on; }
+
+bool gemm_prof_begin(double wbytes, double flops, hipEvent_t *a, hipEvent_t *b)
+{
+    if (!g_prof_on) return false;
+    ProfRec rec{};
+    HIP_CHECK(hipEventCreate(&rec.a));
+    HIP_CHECK(hipEventCreate(&rec.b));
+    rec.wbytes = wbytes; rec.flops = flops;
+    g_prof.push_back(rec);
+    *a = rec.a; *b = rec.b;
+    return true;
 }
 
 }  // namespace lmhip
@@ -356,16 +372,23 @@ void hip_gemm_profile_enable(int on)
 
 int hip_gemm_profile_read(double *total_ms, double *total_weight_bytes)
 {
+    return hip_gemm_profile_read2(total_ms, total_weight_bytes, nullptr);
+}
+
+int hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double *total_flops)
+{
     HIP_CHECK(hipStreamSynchronize(stream()));
-    double ms = 0, wb = 0;
+    double ms = 0, wb = 0, fl = 0;
     for (auto &r : g_prof) {
         float t = 0;
         HIP_CHECK(hipEventElapsedTime(&t, r.a, r.b));
         ms += t;
         wb += r.wbytes;
+        fl += r.flops;
     }
     if (total_ms) *total_ms = ms;
     if (total_weight_bytes) *total_weight_bytes = wb;
+    if (total_flops) *total_flops = fl;
     return (int)g_prof.size();
 }
 

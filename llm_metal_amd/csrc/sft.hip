@@ -156,6 +156,9 @@ WeightOp wop(SFTState *s, int kind, int L, bool T)
     return w;
 }
 
+// From this many rows on the products go through the LDS-tiled large-M kernel (one launch, final output).
+inline bool big_m(const SFTState *s) { return s->BN >= 256; }
+
 size_t max_planes_elems(SFTState *s)
 {
     struct Sh { int N, K; };
@@ -163,6 +166,7 @@ size_t max_planes_elems(SFTState *s)
                          {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->nq_ext}};
     size_t mx = 0;
     for (const Sh &sh : shapes) {
+        if (big_m(s)) { if ((size_t)s->BN * sh.N > mx) mx = (size_t)s->BN * sh.N; continue; }
         GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0);
         const size_t e = (size_t)p.S * s->BN * sh.N;
         if (e > mx) mx = e;
@@ -173,6 +177,12 @@ size_t max_planes_elems(SFTState *s)
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr)
 {
+    if (big_m(s)) {
+        float *C = out ? out : at<float>(s->planes);
+        if (!out && (size_t)s->BN * N > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
+        launch_gemm_big(A, inv, W, C, N, s->BN, N, K);
+        return Planes{C, 1, (size_t)s->BN * N, N, nullptr};
+    }
     GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
     float *P = out ? out : at<float>(s->planes);
     const size_t stride = (size_t)s->BN * N;
@@ -277,7 +287,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
     nf.ln16 = lnf; nf.inv_scale = lnfinv; nf.D = D; nf.eps = s->eps;
     launch_norm_rows(nf, BN);
     GemmPlan pl = plan_gemm(BN, s->V, D);
-    if (pl.S == 1) {
+    if (pl.S == 1 || big_m(s)) {
         gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D, at<float>(s->logits));
     } else {
         Planes p = gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D);
@@ -695,11 +705,8 @@ void sft_state_free(SFTState *s)
     fast_metal_shutdown();
 }
 
-void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr)
+static void enqueue_step_kernels(SFTState *s, float lr)
 {
-    memcpy(s->tokens_cpu, input_tokens, (size_t)s->BN * 4);
-    memcpy(s->targets_cpu, target_tokens, (size_t)s->BN * 4);
-    if (s->R) { s->step_count++; write_hyper(s, lr, s->step_count); }
     forward_impl(s, true);
     CeArgs ce{};
     ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
@@ -708,6 +715,14 @@ void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uin
     if (s->full_param) backward_impl(s, s->gqkv ? BWD_ACCUM : BWD_SGD, lr);     // src/nn/fast_sft.c:1136-1140 with :778-786
     else backward_impl(s);
     enqueue_update(s);
+}
+
+void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr)
+{
+    memcpy(s->tokens_cpu, input_tokens, (size_t)s->BN * 4);
+    memcpy(s->targets_cpu, target_tokens, (size_t)s->BN * 4);
+    if (s->R) { s->step_count++; write_hyper(s, lr, s->step_count); }
+    enqueue_step_kernels(s, lr);
 }
 
 float sft_finish_train_step(SFTState *s)

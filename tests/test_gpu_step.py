@@ -36,6 +36,11 @@ CASES = [
     C1.with_(name="q8_odd_blocks", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_q8", weight_format="q8_0"),
     C1.with_(name="q8_fallback", NL=2, D=128, Hq=3, Hkv=1, hd=32, IS=256, V=1024, seq=24, weight_format="q8_0"),
+    # 256 rows and more: every product goes through the LDS-tiled large-M GEMM (F16 tiles; Q8_0 unpacked into LDS
+    # with row and column scales; row counts that are not multiples of the 128-row block)
+    C1.with_(name="big_m_f16", batch=4, seq=64),
+    C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
+    TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
 ]
 
 
