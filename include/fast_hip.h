@@ -127,6 +127,8 @@ void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
  * GEMM is bracketed by HIP events on the library's stream.  hip_gemm_profile_read
  * (after metal_flush) returns the number of launches recorded since the last
  * enable and adds up their durations (ms) and weight bytes. */
+/* 0: choose the GEMM kernel by the measured rule; 1: always the LDS-tiled large-M kernel; -1: never. */
+void hip_gemm_force_large_m(int policy);
 void hip_gemm_profile_enable(int on);
 int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
 int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double *total_flops);

@@ -72,6 +72,8 @@ double weight_stream_bytes(const WeightOp &W, int N, int K);
 // C[m][n] (row stride ldc) = a_inv_scale[m] * sum_k A[m][k] W[n][k] in one launch of 128 x 128 output blocks staged
 // through LDS (gemm_big.hip): the path for M of several hundred rows and more, where the product is MFMA bound.
 void launch_gemm_big(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K);
+// true when the large-M kernel is the faster one for this product
+bool use_big_gemm(int M, int N, int K, int fmt);
 // Q8_0 blocks in the reference's row-major layout ([rows][cols/32] blocks of 34 bytes) -> kernel tiles.
 // Element (r, c) goes to tiled (row_off + r, k_off + c) with row scales (fmt 1), or, transposed, to
 // (row_off + c, k_off + r) with column scales (fmt 2).  Kb_dst = K blocks per row block of the destination.

@@ -269,6 +269,19 @@ void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, in
 
 int gemm_profiling() { return g_prof_on; }
 
+// Which kernel multiplies an [M, K] activation block with an [N, K] weight.  Measured on MI355X (Qwen3-4B shapes):
+// the 128 x 256 LDS-tiled kernel wins for F16 weights once there is at least one block per CU (2048 rows: 490-650
+// against 300 TFLOP/s); with Q8_0 weights the weight-streaming kernel, whose waves overlap each other's unpacking
+// and MFMAs, stays ahead at every M (400-470 against 340-460 TFLOP/s).
+int g_big_policy = 0;                                     // 0 measured rule, 1 always, -1 never
+bool use_big_gemm(int M, int N, int K, int fmt)
+{
+    (void)K;
+    if (g_big_policy) return g_big_policy > 0;
+    const long blocks = (long)((M + 127) / 128) * ((N + 255) / 256);
+    return fmt == 0 && M >= 512 && blocks >= 224;
+}
+
 bool gemm_prof_begin(double wbytes, double flops, hipEvent_t *a, hipEvent_t *b)
 {
     if (!g_prof_on) return false;
@@ -362,6 +375,8 @@ void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, i
     mark_written(C);
 }
 
+void hip_gemm_force_large_m(int policy) { g_big_policy = policy; }
+
 void hip_gemm_profile_enable(int on)
 {
     HIP_CHECK(hipStreamSynchronize(stream()));
@@ -398,7 +413,7 @@ int hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double 
 // Returns the average milliseconds per launch.
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S)
 {
-    g_force_nb = nb; g_force_S = S;
+    g_force_nb = nb == 128 ? 0 : nb; g_force_S = S;
     GemmPlan p = plan_gemm(M, N, K);
     g_force_nb = 0; g_force_S = 0;
     if (used_nb) *used_nb = p.nb;
@@ -425,9 +440,14 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters
                w.nbq = tiled_rb(N); w.kbq = tiled_kb(K); }
         return w;
     };
-    for (int i = 0; i < 3; i++) launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
+    const bool big = nb == 128;                            // nb = 128 selects the large-M kernel (one launch, 128-row blocks)
+    auto run = [&](int i) {
+        if (big) launch_gemm_big((half_t *)A, (float *)inv, op(i), (float *)P, N, M, N, K);
+        else launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
+    };
+    for (int i = 0; i < 3; i++) run(i);
     HIP_CHECK(hipEventRecord(e0, stream()));
-    for (int i = 0; i < iters; i++) launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
+    for (int i = 0; i < iters; i++) run(i);
     HIP_CHECK(hipEventRecord(e1, stream()));
     HIP_CHECK(hipStreamSynchronize(stream()));
     g_prof_on = saved;

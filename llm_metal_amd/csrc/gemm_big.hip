@@ -19,81 +19,162 @@
 namespace lmhip {
 namespace {
 
-struct Stage {                       // what one thread holds of the next K step: one row block of A, one of W
+constexpr int WPW = 2;               // weight row blocks each wave fetches per K step: the block is 128 x (WPW * 128)
+constexpr int PF = 3;                // K steps whose operands are in flight in registers ahead of the one being multiplied
+
+// What one thread holds of a K step that is still on its way to LDS: one row block of A and WPW of W, as loaded
+// (Q8_0 stays packed until it is written to LDS, so nothing waits on a fresh load).
+struct Stage {
     half8 a[4];
-    half8 w[4];
+    half8 w16[WPW][4];               // F16 tile, or the column scales of a transposed Q8_0 tile
+    uint4v q[WPW][2];                // Q8_0 int8
+    half_t d[WPW];                   // Q8_0 row scale of this lane's weights
 };
 
+// kind of weight tile (uniform per wave): 0 F16, 1 Q8_0 row scales, 2 Q8_0 column scales
 template <int WF>
-__device__ __forceinline__ void fetch(Stage &s, const GemmKArgs &g, int mb, int nb, bool w_q8_rows, int kt, int lane)
+__device__ __forceinline__ int tile_kind(const GemmKArgs &g, int nb, int kt)
+{
+    if (WF == 0) return 0;
+    if (WF == 1) return nb < g.W.nbq ? 1 : 0;
+    return kt < g.W.kbq ? 2 : 0;
+}
+
+template <int WF>
+__device__ __forceinline__ void fetch(Stage &s, const GemmKArgs &g, int mb, const int (&nb)[WPW], int kt, int lane)
 {
     const half8 *ap = g.A + ((size_t)mb * g.Kb + kt) * 256 + lane;
 #pragma unroll
     for (int j = 0; j < 4; j++) s.a[j] = ap[j * 64];
-    if (WF == 0) load_w_f16(s.w, g.W.w16, nb, g.Kb, kt, lane);
-    else if (WF == 1) {
-        if (w_q8_rows) load_w_q8_rows(s.w, g.W, nb, g.Kb, kt, lane);
-        else load_w_f16(s.w, g.W.w16, nb - g.W.nbq, g.Kb, kt, lane);
-    } else {
-        if (kt < g.W.kbq) load_w_q8_cols(s.w, g.W, nb, g.W.kbq, kt, lane);
-        else load_w_f16(s.w, g.W.w16, nb, g.Kb - g.W.kbq, kt - g.W.kbq, lane);
+#pragma unroll
+    for (int u = 0; u < WPW; u++) {
+        const int kind = tile_kind<WF>(g, nb[u], kt);
+        if (kind == 0) {
+            if (WF == 0) load_w_f16(s.w16[u], g.W.w16, nb[u], g.Kb, kt, lane);
+            else if (WF == 1) load_w_f16(s.w16[u], g.W.w16, nb[u] - g.W.nbq, g.Kb, kt, lane);
+            else load_w_f16(s.w16[u], g.W.w16, nb[u], g.Kb - g.W.kbq, kt - g.W.kbq, lane);
+        } else {
+            const size_t tile = (size_t)nb[u] * (kind == 1 ? g.Kb : g.W.kbq) + kt;
+            const uint4v *q = reinterpret_cast<const uint4v *>(g.W.q) + tile * 128 + lane;
+            s.q[u][0] = __builtin_nontemporal_load(&q[0]);
+            s.q[u][1] = __builtin_nontemporal_load(&q[64]);
+            if (kind == 1) s.d[u] = g.W.d[tile * 64 + lane];
+            else {
+                const half8 *sc = reinterpret_cast<const half8 *>(g.W.d + tile * 64 + (lane >> 5) * 32);
+#pragma unroll
+                for (int j = 0; j < 4; j++) s.w16[u][j] = sc[j];
+            }
+        }
     }
 }
 
-// grid: x = ceil(N / 128), y = ceil(M / 128); block 256; LDS 2 x (4 + 4) row blocks x 4 KB = 64 KB
+// fp16 weight registers of a fetched tile (Q8_0: int8 * scale, rounded once to fp16)
 template <int WF>
-__global__ __launch_bounds__(256, 2) void gemm_big(GemmKArgs g)
+__device__ __forceinline__ void unpack(half8 (&w)[4], const Stage &s, int u, int kind)
 {
-    extern __shared__ half8 tiles[];                      // [buf][A blocks 0-3 | W blocks 0-3][j][lane]
+    if (kind == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = s.w16[u][j];
+        return;
+    }
+    const half8 q0 = q8_unpack8(s.q[u][0][0], s.q[u][0][1]), q1 = q8_unpack8(s.q[u][0][2], s.q[u][0][3]);
+    const half8 q2 = q8_unpack8(s.q[u][1][0], s.q[u][1][1]), q3 = q8_unpack8(s.q[u][1][2], s.q[u][1][3]);
+    if (kind == 1) { const half8 d = bcast8(s.d[u]); w[0] = q0 * d; w[1] = q1 * d; w[2] = q2 * d; w[3] = q3 * d; }
+    else { w[0] = q0 * s.w16[u][0]; w[1] = q1 * s.w16[u][1]; w[2] = q2 * s.w16[u][2]; w[3] = q3 * s.w16[u][3]; }
+}
+
+// 1-D grid, block 256; LDS 2 x (4 + 4 WPW) row blocks x 4 KB.
+// Wave (wm, wn) owns rows [64 wm, +64) and columns [64 WPW wn, +64 WPW) of the block.
+//
+// Which block a workgroup takes is chosen for the eight L2 caches: the hardware deals consecutive workgroup ids
+// to the XCDs in turn, so id % 8 is the XCD.  Each XCD gets every eighth column of blocks, and the 32 workgroups
+// that are resident on it together form an 8 x 4 patch (8 row blocks x 4 column blocks).  They walk K in step, so
+// an activation slice fetched into that L2 serves 4 workgroups and a weight slice 8, instead of one each.
+template <int WF>
+__global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
+{
+    extern __shared__ half8 tiles[];                      // [buf][A blocks 0-3 | W blocks 0 .. 4 WPW - 1][j][lane]
+    constexpr int NBLK = 4 + 4 * WPW, BUF = NBLK * 256, NW = 2 * WPW;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int nb0 = blockIdx.x * 4, mb0 = blockIdx.y * 4;
-    const int wm = wave >> 1, wn = wave & 1;              // this wave's 64 x 64 quadrant of the block
+    const int MT = (g.M + 127) >> 7, NT = (g.N + 128 * WPW - 1) / (128 * WPW);
+    const int m_patches = (MT + 7) >> 3;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3, patch = seq >> 5, in_patch = seq & 31;
+    const int mt = (patch % m_patches) * 8 + (in_patch & 7);
+    const int nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
+    if (mt >= MT || nt >= NT) return;                     // padding of the patch grid; the whole workgroup leaves
+    const int nb0 = nt * 4 * WPW, mb0 = mt * 4;
+    const int wm = wave >> 1, wn = wave & 1;
     // the row blocks this wave fetches (clamped: rows past the end are computed and never stored)
-    const int mb_ld = min(mb0 + wave, g.Mb - 1), nb_ld = min(nb0 + wave, g.Nb - 1);
-    const bool q8r = WF == 1 && nb_ld < g.W.nbq;
+    const int mb_ld = min(mb0 + wave, g.Mb - 1);
+    int nb_ld[WPW];
+#pragma unroll
+    for (int u = 0; u < WPW; u++) nb_ld[u] = min(nb0 + wave * WPW + u, g.Nb - 1);
 
-    float16v acc[2][2];
+    float16v acc[2][NW];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NW; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    Stage st;
-    fetch<WF>(st, g, mb_ld, nb_ld, q8r, 0, lane);
-    {
-        half8 *buf = tiles;
+    Stage st[PF];                                         // step s travels in st[s % PF]
+    auto park = [&](const Stage &s, int kt, half8 *buf) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) { buf[(wave * 4 + j) * 64 + lane] = st.a[j]; buf[((4 + wave) * 4 + j) * 64 + lane] = st.w[j]; }
-    }
-    __syncthreads();
-    for (int kt = 0; kt < g.Kb; kt++) {
-        const half8 *cur = tiles + (size_t)(kt & 1) * 2048;
-        half8 *nxt = tiles + (size_t)((kt + 1) & 1) * 2048;
-        const bool more = kt + 1 < g.Kb;
-        if (more) fetch<WF>(st, g, mb_ld, nb_ld, q8r, kt + 1, lane);
-        half8 a[2][4], w[2][4];
+        for (int j = 0; j < 4; j++) buf[(wave * 4 + j) * 64 + lane] = s.a[j];
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int u = 0; u < WPW; u++) {
+            half8 w[4];
+            unpack<WF>(w, s, u, tile_kind<WF>(g, nb_ld[u], kt));
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                a[i][j] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
-                w[i][j] = cur[((4 + 2 * wn + i) * 4 + j) * 64 + lane];
-            }
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int k = 0; k < 2; k++)
-                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i][j], w[k][j], acc[i][k], 0, 0, 0);
-        if (more) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) { nxt[(wave * 4 + j) * 64 + lane] = st.a[j]; nxt[((4 + wave) * 4 + j) * 64 + lane] = st.w[j]; }
+            for (int j = 0; j < 4; j++) buf[((4 + wave * WPW + u) * 4 + j) * 64 + lane] = w[j];
         }
-        __syncthreads();
+    };
+#pragma unroll
+    for (int p = 0; p < PF; p++) if (p < g.Kb) fetch<WF>(st[p], g, mb_ld, nb_ld, p, lane);
+    park(st[0], 0, tiles);
+    __syncthreads();
+    for (int kt0 = 0; kt0 < g.Kb; kt0 += PF) {
+#pragma unroll
+        for (int u = 0; u < PF; u++) {
+            const int kt = kt0 + u;
+            if (kt < g.Kb) {
+                const half8 *cur = tiles + (size_t)(kt & 1) * BUF;
+                // the slot of step kt is free (it was written to LDS in the previous round): refill it with step kt + PF
+                if (kt + PF < g.Kb) fetch<WF>(st[u], g, mb_ld, nb_ld, kt + PF, lane);
+                // fp16 image of the next step's weight blocks: plain VALU work with no dependence on this step's
+                // MFMAs, placed in the same block of code so that the two interleave (on the last step it
+                // unpacks stale registers and the result is dropped)
+                const Stage &sn = st[(u + 1) % PF];
+                half8 wnext[WPW][4];
+#pragma unroll
+                for (int x = 0; x < WPW; x++) unpack<WF>(wnext[x], sn, x, tile_kind<WF>(g, nb_ld[x], min(kt + 1, g.Kb - 1)));
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    half8 a[2], w[NW];
+#pragma unroll
+                    for (int i = 0; i < 2; i++) a[i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
+#pragma unroll
+                    for (int k = 0; k < NW; k++) w[k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
+#pragma unroll
+                    for (int i = 0; i < 2; i++)
+#pragma unroll
+                        for (int k = 0; k < NW; k++)
+                            acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
+                }
+                if (kt + 1 < g.Kb) {
+                    half8 *nxt = tiles + (size_t)((kt + 1) & 1) * BUF;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        nxt[(wave * 4 + j) * 64 + lane] = sn.a[j];
+#pragma unroll
+                        for (int x = 0; x < WPW; x++) nxt[((4 + wave * WPW + x) * 4 + j) * 64 + lane] = wnext[x][j];
+                    }
+                }
+                __syncthreads();
+            }
+        }
     }
 
 #pragma unroll
@@ -105,8 +186,8 @@ __global__ __launch_bounds__(256, 2) void gemm_big(GemmKArgs g)
             if (m >= g.M) continue;
             const float sc = g.a_inv_scale ? g.a_inv_scale[m] : 1.0f;
 #pragma unroll
-            for (int k = 0; k < 2; k++) {
-                const int n = (nb0 + 2 * wn + k) * 32 + r;
+            for (int k = 0; k < NW; k++) {
+                const int n = (nb0 + NW * wn + k) * 32 + r;
                 if (n < g.N) g.P[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
             }
         }
@@ -127,8 +208,10 @@ void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &
     g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
     g.P = C; g.ldp = ldc; g.plane_stride = 0;
     g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = Kb;
-    const dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
-    const size_t lds = 2 * 2048 * sizeof(half8);
+    const int MT = (M + 127) / 128, NT = (N + 128 * WPW - 1) / (128 * WPW);
+    const int m_patches = (MT + 7) / 8, n_patches = ((NT + 7) / 8 + 3) / 4;
+    const dim3 grid(8 * 32 * m_patches * n_patches), block(256);
+    const size_t lds = (size_t)2 * (4 + 4 * WPW) * 256 * sizeof(half8);
     static bool attr_set = false;
     if (!attr_set) {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_big<0>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

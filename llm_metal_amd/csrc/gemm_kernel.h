@@ -30,6 +30,14 @@ __device__ __forceinline__ half8 q8_unpack8(uint32_t lo, uint32_t hi)
     return v - off;
 }
 
+__device__ __forceinline__ half8 bcast8(half_t d)
+{
+    half8 v;
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = d;
+    return v;
+}
+
 // Weight registers of one 64-wide K step for row block `nb`: w[j] feeds the j-th MFMA of the step.
 // FMT 0: F16 tiles, `kb_stride` K blocks per row block, K block `kt`.
 __device__ __forceinline__ void load_w_f16(half8 (&w)[4], const half_t *W16, int nb, int kb_stride, int kt, int lane)
@@ -47,7 +55,7 @@ __device__ __forceinline__ void load_w_q8_rows(half8 (&w)[4], const WeightOp &W,
     const size_t tile = (size_t)nb * kb_stride + kt;
     const uint4v *q = reinterpret_cast<const uint4v *>(W.q) + tile * 128 + lane;
     const uint4v r0 = __builtin_nontemporal_load(&q[0]), r1 = __builtin_nontemporal_load(&q[64]);
-    const half_t d = __builtin_nontemporal_load(&W.d[tile * 64 + lane]);
+    const half8 d = bcast8(__builtin_nontemporal_load(&W.d[tile * 64 + lane]));
     w[0] = q8_unpack8(r0[0], r0[1]) * d;
     w[1] = q8_unpack8(r0[2], r0[3]) * d;
     w[2] = q8_unpack8(r1[0], r1[1]) * d;

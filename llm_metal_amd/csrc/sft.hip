@@ -156,9 +156,6 @@ WeightOp wop(SFTState *s, int kind, int L, bool T)
     return w;
 }
 
-// From this many rows on the products go through the LDS-tiled large-M kernel (one launch, final output).
-inline bool big_m(const SFTState *s) { return s->BN >= 256; }
-
 size_t max_planes_elems(SFTState *s)
 {
     struct Sh { int N, K; };
@@ -166,7 +163,6 @@ size_t max_planes_elems(SFTState *s)
                          {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->nq_ext}};
     size_t mx = 0;
     for (const Sh &sh : shapes) {
-        if (big_m(s)) { if ((size_t)s->BN * sh.N > mx) mx = (size_t)s->BN * sh.N; continue; }
         GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0);
         const size_t e = (size_t)p.S * s->BN * sh.N;
         if (e > mx) mx = e;
@@ -177,7 +173,7 @@ size_t max_planes_elems(SFTState *s)
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr)
 {
-    if (big_m(s)) {
+    if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch, final output
         float *C = out ? out : at<float>(s->planes);
         if (!out && (size_t)s->BN * N > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
         launch_gemm_big(A, inv, W, C, N, s->BN, N, K);
@@ -287,7 +283,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
     nf.ln16 = lnf; nf.inv_scale = lnfinv; nf.D = D; nf.eps = s->eps;
     launch_norm_rows(nf, BN);
     GemmPlan pl = plan_gemm(BN, s->V, D);
-    if (pl.S == 1 || big_m(s)) {
+    if (pl.S == 1 || use_big_gemm(BN, s->V, D, s->q8_native ? 1 : 0)) {
         gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D, at<float>(s->logits));
     } else {
         Planes p = gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D);
