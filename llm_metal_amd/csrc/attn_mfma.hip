@@ -33,87 +33,117 @@ __device__ __forceinline__ float16v zero16()
 // they are added when the tile is complete.
 struct Acc2 { float16v a, b; };
 
-// One 32 x 32 product tile A[32, HD] (LDS, row stride lda) * Bm[32 rows, HD]^T, with the 32 B rows read straight from
-// memory.  The reduction index is split between the lane halves (lanes 0-31 take columns [0, HD/2), lanes 32-63
-// the rest), so a lane reads one contiguous half row of its B row in chunks of CH floats.  Every load is
-// unconditional and issued one chunk ahead of its MFMAs: `first` arrives holding chunk 0 and leaves holding chunk 0
-// of `next_half_row` (the tile this wave multiplies next; any valid row when there is none).
-template <int HD> struct BCfg { static constexpr int HALF = HD / 2, CH = HALF < 32 ? HALF : 32, NCH = HALF / CH; };
-template <int HD> struct BChunk { float4 v[BCfg<HD>::CH / 4]; };
+// One 32 x 32 product tile A[32, HD] (LDS, row stride lda) * Bm[32 rows, HD]^T.  The reduction index is split
+// between the lane halves (lanes 0-31 take columns [0, HD/2), lanes 32-63 the rest), so a lane needs one
+// half row of its B row: a BTile, HD/2 floats per lane, read straight from memory a whole tile
+// (64 MFMAs at HD = 128, about 2 us) ahead of its use.  The A values come from LDS, 32 floats at a time, one
+// such chunk ahead.
+template <int HD> struct BTile { float4 v[HD / 8]; };
 
+// The values come from a copy of the head's matrix laid out as BT[HD/4][ldt][4] (group of four columns, key, column
+// in the group; ldt = attn_ldt(seq)): a lane still reads 16 bytes at a time, but the 32 lanes of a half wave read
+// 512 contiguous bytes, where the rows themselves (4 KB apart) would cost one cache line per lane and instruction
+// and keep the memory pipeline busy for as long as the MFMAs run.
 template <int HD>
-__device__ __forceinline__ void b_chunk_load(BChunk<HD> &c, const float *b_half_row, int c0)
+__device__ __forceinline__ void b_tile_load(BTile<HD> &t, const float *bt_lane, int ldt)
 {
 #pragma unroll
-    for (int t = 0; t < BCfg<HD>::CH / 4; t++) c.v[t] = ld4(b_half_row + c0 + 4 * t);
+    for (int i = 0; i < HD / 8; i++) t.v[i] = ld4(bt_lane + (size_t)i * ldt * 4);
 }
 
 template <int HD>
-__device__ __forceinline__ float16v tile_abt(const float *As, int lda, const float *b_half_row, int lane,
-                                             BChunk<HD> &first, const float *next_half_row)
+__device__ __forceinline__ float16v tile_abt(const float *As, int lda, int lane, const BTile<HD> &bt)
 {
-    constexpr int CH = BCfg<HD>::CH, NCH = BCfg<HD>::NCH;
-    const float *a = As + (lane & 31) * lda + (lane >> 5) * BCfg<HD>::HALF;
+    constexpr int HALF = HD / 2, CH = HALF < 32 ? HALF : 32, NCH = HALF / CH;
+    const float *a = As + (lane & 31) * lda + (lane >> 5) * HALF;
     Acc2 acc{zero16(), zero16()};
-    BChunk<HD> buf[2];
-    buf[0] = first;
+    float4 abuf[2][CH / 4];
+#pragma unroll
+    for (int t = 0; t < CH / 4; t++) abuf[0][t] = *reinterpret_cast<const float4 *>(a + 4 * t);     // LDS, 16-byte aligned
 #pragma unroll
     for (int ci = 0; ci < NCH; ci++) {
-        if (ci + 1 < NCH) b_chunk_load<HD>(buf[(ci + 1) & 1], b_half_row, (ci + 1) * CH);
-        else b_chunk_load<HD>(buf[(ci + 1) & 1], next_half_row, 0);
-        const BChunk<HD> &c = buf[ci & 1];
+        if (ci + 1 < NCH) {
+#pragma unroll
+            for (int t = 0; t < CH / 4; t++) abuf[(ci + 1) & 1][t] = *reinterpret_cast<const float4 *>(a + (ci + 1) * CH + 4 * t);
+        }
 #pragma unroll
         for (int t = 0; t < CH / 4; t++) {
-            acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ci * CH + 4 * t + 0], c.v[t].x, acc.a, 0, 0, 0);
-            acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ci * CH + 4 * t + 1], c.v[t].y, acc.b, 0, 0, 0);
-            acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ci * CH + 4 * t + 2], c.v[t].z, acc.a, 0, 0, 0);
-            acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ci * CH + 4 * t + 3], c.v[t].w, acc.b, 0, 0, 0);
+            const float4 x = abuf[ci & 1][t], c = bt.v[ci * (CH / 4) + t];
+            acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, c.x, acc.a, 0, 0, 0);
+            acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, c.y, acc.b, 0, 0, 0);
+            acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, c.z, acc.a, 0, 0, 0);
+            acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, c.w, acc.b, 0, 0, 0);
         }
     }
-    first = buf[NCH & 1];
     return acc.a + acc.b;
 }
 
 // One 32 x 32 product tile X[32, nk] (LDS, row stride ldx) * C[nk rows, 32 columns], C row-major with row stride ldc;
-// rows beyond n_valid are read as row n_valid - 1 (their X column is zero).  Chunks of 32 rows of C (16 loads) are
-// requested one chunk ahead, unconditionally (past the end the last chunk is read again); `first` holds chunk 0.
+// rows beyond n_valid are read as row n_valid - 1 (their X column is zero).  Inside a chunk of 32 keys lanes 0-31
+// take keys 0-15 and lanes 32-63 keys 16-31, so a lane reads 16 consecutive X values (four 16-byte LDS reads) and
+// 16 rows of C.  Both are requested one chunk ahead, unconditionally (past the end the last chunk is read again);
+// `first` holds chunk 0 of C.
 struct CChunk { float v[16]; };
+struct XChunk { float4 v[4]; };
 
 __device__ __forceinline__ void c_chunk_load(CChunk &c, const float *ccol_lane, size_t ldc, int k0, int hh, int n_valid)
 {
 #pragma unroll
-    for (int t = 0; t < 16; t++) c.v[t] = ccol_lane[(size_t)min(k0 + 2 * t + hh, n_valid - 1) * ldc];
+    for (int t = 0; t < 16; t++) c.v[t] = ccol_lane[(size_t)min(k0 + 16 * hh + t, n_valid - 1) * ldc];
 }
 
-__device__ __forceinline__ void c_chunk_mfma(Acc2 &acc, const float *x, const CChunk &c)
+__device__ __forceinline__ void x_chunk_load(XChunk &c, const float *x_row_half, int k0)
 {
 #pragma unroll
-    for (int t = 0; t < 16; t += 2) {
-        acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x[2 * t], c.v[t], acc.a, 0, 0, 0);
-        acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x[2 * t + 2], c.v[t + 1], acc.b, 0, 0, 0);
+    for (int t = 0; t < 4; t++) c.v[t] = *reinterpret_cast<const float4 *>(x_row_half + k0 + 4 * t);
+}
+
+__device__ __forceinline__ void c_chunk_mfma(Acc2 &acc, const XChunk &x, const CChunk &c)
+{
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].x, c.v[4 * t + 0], acc.a, 0, 0, 0);
+        acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].y, c.v[4 * t + 1], acc.b, 0, 0, 0);
+        acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].z, c.v[4 * t + 2], acc.a, 0, 0, 0);
+        acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].w, c.v[4 * t + 3], acc.b, 0, 0, 0);
     }
 }
 
+// The C chunks travel in a ring of four (chunk q in slot q % 4), requested three chunks (about 1.4 us of MFMAs)
+// ahead; on entry slots 0-2 hold chunks 0-2, which the caller may have requested long before.
+struct CRing { CChunk c[4]; };
+
+__device__ __forceinline__ void c_ring_start(CRing &r, const float *ccol_lane, size_t ldc, int nk, int hh, int n_valid)
+{
+#pragma unroll
+    for (int q = 0; q < 3; q++) c_chunk_load(r.c[q], ccol_lane, ldc, min(32 * q, nk - 32), hh, n_valid);
+}
+
 __device__ __forceinline__ float16v tile_xc(const float *Xs, int ldx, int nk, const float *ccol_lane, size_t ldc, int n_valid, int lane,
-                                            CChunk &first)
+                                            CRing &ring)
 {
     const int hh = lane >> 5;
-    const float *x = Xs + (lane & 31) * ldx + hh;
+    const float *x = Xs + (lane & 31) * ldx + 16 * hh;
     Acc2 acc{zero16(), zero16()};
-    CChunk other;
-    for (int k0 = 0; k0 < nk; k0 += 64) {                 // nk is a multiple of 32
-        c_chunk_load(other, ccol_lane, ldc, min(k0 + 32, nk - 32), hh, n_valid);
-        c_chunk_mfma(acc, x + k0, first);
-        c_chunk_load(first, ccol_lane, ldc, min(k0 + 64, nk - 32), hh, n_valid);
-        if (k0 + 32 < nk) c_chunk_mfma(acc, x + k0 + 32, other);
+    XChunk xr[2];
+    x_chunk_load(xr[0], x, 0);
+    for (int k0 = 0; k0 < nk; k0 += 128) {                // nk is a multiple of 32
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int kc = k0 + 32 * u;
+            c_chunk_load(ring.c[(u + 3) & 3], ccol_lane, ldc, min(kc + 96, nk - 32), hh, n_valid);
+            x_chunk_load(xr[(u + 1) & 1], x, min(kc + 32, nk - 32));
+            if (kc < nk) c_chunk_mfma(acc, xr[u & 1], ring.c[u]);
+        }
     }
     return acc.a + acc.b;
 }
 
 struct AttnTileArgs {
-    // forward: A = q, B = k, C = v;  dQ: A = dO (planes), B = v, C = k
+    // forward: A = q, B = k, C = v;  dQ: A = dO (planes), B = v, C = k.  B is given transposed per head:
+    // BT[batch][Hkv][hd/4][attn_ldt(seq)][4]
     const float *A; Planes Apl;
-    const float *B, *C;
+    const float *BT, *C;
     int Hq, Hkv, hd, seq, batch; float scale;
     float *probs;                 // forward: written; dQ: read          [batch][Hq][seq][seq]
     float *dscore;                // dQ: written
@@ -122,67 +152,75 @@ struct AttnTileArgs {
     half_t *out16;                // forward: tiled [rows, Hq*hd]
 };
 
-// Row step for four rows at a time: a wave holds NE elements per lane of each row (keys lane, lane + 64, ...), so
-// the LDS reads of a row are in flight together and the four rows' wave reductions interleave.  The finished rows
-// go back to LDS for phase 3 and, whole (zeros right of the diagonal), to memory.
-template <int BWD, int NE>
-__device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int nk, int N, int i0, int b, int h, int wave, int lane)
+// Row step: eight threads per row, thread `part` owns the keys 32 m + 4 part + (0..3) for m < M32 and keeps them in
+// registers, so every LDS and memory access is a 16-byte one (eight threads cover 128 contiguous bytes) and the
+// row reductions need three shuffles.  The finished rows go back to LDS for phase 3 and, whole (zeros right of the
+// diagonal, out to column N), to memory.
+template <int BWD, int M32>
+__device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int nk, int N, int i0, int b, int h, int tid)
 {
-    for (int r4 = 0; r4 < 8; r4 += 4) {
-        float v[4][NE], p[4][NE];
-        float red[4];
+    const int rr = tid >> 3, part = tid & 7, i = i0 + rr;
+    const bool row_ok = i < N;
+    float *xr = Xs + rr * ldx + 4 * part;
+    const size_t goff = (((size_t)b * a.Hq + h) * N + min(i, N - 1)) * N + 4 * part;
+    float4 v[M32], p[BWD ? M32 : 1];
+    float red = BWD ? 0.f : -1e30f;
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int rr = wave * 8 + r4 + q, i = i0 + rr;
-            const float *prow = a.probs + (((size_t)b * a.Hq + h) * N + min(i, N - 1)) * N;
-            red[q] = BWD ? 0.f : -1e30f;
-#pragma unroll
-            for (int e = 0; e < NE; e++) {
-                const int j = lane + 64 * e;
-                const bool ok = j <= i && j < nk && i < N;
-                v[q][e] = Xs[rr * ldx + min(j, nk - 1)];
-                if (BWD) { p[q][e] = ok ? prow[j] : 0.f; red[q] += p[q][e] * v[q][e]; }
-                else { v[q][e] = ok ? v[q][e] * a.scale : -1e30f; red[q] = fmaxf(red[q], v[q][e]); }
+    for (int m = 0; m < M32; m++) {
+        const int j = 32 * m + 4 * part;
+        v[m] = (j < nk) ? *reinterpret_cast<const float4 *>(xr + 32 * m) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float *e = &v[m].x;
+        if (BWD) {
+            // probabilities are zero right of the diagonal; whole 16-byte groups exist when N % 4 == 0, else go by element
+            float4 pv = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row_ok && j <= i) {
+                if ((N & 3) == 0) pv = *reinterpret_cast<const float4 *>(a.probs + goff + 32 * m);
+                else { float *q = &pv.x; for (int c = 0; c < 4; c++) if (j + c < N) q[c] = a.probs[goff + 32 * m + c]; }
             }
+            p[m] = pv;
+            red += pv.x * e[0] + pv.y * e[1] + pv.z * e[2] + pv.w * e[3];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++) { e[c] = (j + c <= i && j + c < nk) ? e[c] * a.scale : -1e30f; red = fmaxf(red, e[c]); }
         }
+    }
+    if (BWD) { red += __shfl_xor(red, 1, WAVE); red += __shfl_xor(red, 2, WAVE); red += __shfl_xor(red, 4, WAVE); }
+    else { red = fmaxf(red, __shfl_xor(red, 1, WAVE)); red = fmaxf(red, __shfl_xor(red, 2, WAVE)); red = fmaxf(red, __shfl_xor(red, 4, WAVE)); }
+    float inv = 1.0f;
+    if (!BWD) {
+        float sum = 0.f;
 #pragma unroll
-        for (int q = 0; q < 4; q++) red[q] = BWD ? wave_sum(red[q]) : wave_max(red[q]);
-        if (!BWD) {
-            float sum[4];
+        for (int m = 0; m < M32; m++) {
+            const int j = 32 * m + 4 * part;
+            float *e = &v[m].x;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                sum[q] = 0.f;
-#pragma unroll
-                for (int e = 0; e < NE; e++) {
-                    const int j = lane + 64 * e;
-                    v[q][e] = (j <= i0 + wave * 8 + r4 + q && j < nk) ? expf(v[q][e] - red[q]) : 0.f;
-                    sum[q] += v[q][e];
-                }
-            }
-#pragma unroll
-            for (int q = 0; q < 4; q++) red[q] = 1.0f / wave_sum(sum[q]);
+            for (int c = 0; c < 4; c++) { e[c] = (j + c <= i && j + c < nk) ? expf(e[c] - red) : 0.f; sum += e[c]; }
         }
+        sum += __shfl_xor(sum, 1, WAVE); sum += __shfl_xor(sum, 2, WAVE); sum += __shfl_xor(sum, 4, WAVE);
+        inv = 1.0f / sum;
+    }
+    float *gdst = (BWD ? a.dscore : a.probs) + goff;
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int rr = wave * 8 + r4 + q, i = i0 + rr;
-            float *grow = (BWD ? a.dscore : a.probs) + (((size_t)b * a.Hq + h) * N + min(i, N - 1)) * N;
-#pragma unroll
-            for (int e = 0; e < NE; e++) {
-                const int j = lane + 64 * e;
-                const float o = BWD ? p[q][e] * (v[q][e] - red[q]) * a.scale : v[q][e] * red[q];
-                if (j < nk) Xs[rr * ldx + j] = o;
-                if (j < N && i < N) grow[j] = (j < nk) ? o : 0.f;
-            }
+    for (int m = 0; m < M32; m++) {
+        const int j = 32 * m + 4 * part;
+        float4 o;
+        if (BWD) o = make_float4(p[m].x * (v[m].x - red) * a.scale, p[m].y * (v[m].y - red) * a.scale,
+                                 p[m].z * (v[m].z - red) * a.scale, p[m].w * (v[m].w - red) * a.scale);
+        else o = make_float4(v[m].x * inv, v[m].y * inv, v[m].z * inv, v[m].w * inv);
+        if (j < nk) *reinterpret_cast<float4 *>(xr + 32 * m) = o;
+        if (row_ok && j < N) {
+            if ((N & 3) == 0) *reinterpret_cast<float4 *>(gdst + 32 * m) = o;
+            else { const float *q = &o.x; for (int c = 0; c < 4; c++) if (j + c < N) gdst[32 * m + c] = q[c]; }
         }
     }
 }
 
-// grid (query blocks of 32, Hq, batch), block 256; LDS: As[32][HD+1], Xs[32][ldx]
+// grid (query blocks of 32, Hq, batch), block 256; LDS: As[32][HD+4], Xs[32][ldx]
 template <int BWD, int HD>
 __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
 {
     extern __shared__ float lds[];
-    constexpr int lda = HD + 1, half = HD / 2;
+    constexpr int lda = HD + 4, half = HD / 2;            // rows 16-byte aligned; 132 floats apart: conflict-free 16-byte reads
     const int N = a.seq;
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l31 = lane & 31, hh = lane >> 5;
@@ -190,56 +228,64 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     const size_t r0 = (size_t)b * N;
     const int i0 = qb * 32;
     const int nk = min(i0 + 32, (N + 31) & ~31);          // keys this block can see, rounded up to 32
-    const int ldx = ((N + 63) & ~63) + 1;
+    const int ldx = ((N + 31) & ~31) + 4;
     float *As = lds, *Xs = As + 32 * lda;
 
     // ---- the first B tile and the first C chunk of this wave do not depend on anything computed here:
     //      request them before the A rows are staged (waves without a tile of their own read tile 0)
-    auto b_row = [&](int jb) { return a.B + (r0 + min(jb * 32 + l31, N - 1)) * kd + hk * HD + hh * half; };
+    // this lane's column of the transposed B matrix: key jb * 32 + l31, rows hh * half ...
+    const int ldt = attn_ldt(N);
+    auto b_row = [&](int jb) { return a.BT + ((((size_t)b * a.Hkv + hk) * (HD / 4) + hh * (half / 4)) * ldt + min(jb * 32 + l31, N - 1)) * 4; };
     const int nkb = nk >> 5;
-    BChunk<HD> bfirst;
-    b_chunk_load<HD>(bfirst, b_row(wave < nkb ? wave : 0), 0);
-    CChunk cfirst;
+    BTile<HD> bt0, bt1;
+    b_tile_load<HD>(bt0, b_row(wave < nkb ? wave : 0), ldt);
+    CRing cring;
     const float *c_lane0 = a.C + r0 * kd + hk * HD + l31;
-    c_chunk_load(cfirst, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, 0, hh, N);
+    c_ring_start(cring, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, nk, hh, N);
 
-    // ---- A rows into LDS (rows past the sequence as zeros)
-    for (int idx = tid; idx < 32 * (HD >> 2); idx += 256) {
-        const int rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i0 + rr < N) {
-            if (BWD) {
-                v = planes_at4(a.Apl, r0 + i0 + rr, h * HD + 4 * c4);
-                st4(a.A_out + (r0 + i0 + rr) * qd + h * HD + 4 * c4, v);
-            } else {
-                v = ld4(a.A + (r0 + i0 + rr) * qd + h * HD + 4 * c4);
-            }
+    // ---- A rows into LDS (rows past the sequence as zeros); the loads of all HD / 32 rounds are issued together
+    {
+        float4 av[HD / 32];
+#pragma unroll
+        for (int u = 0; u < HD / 32; u++) {
+            const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
+            av[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (i0 + rr < N) av[u] = BWD ? planes_at4(a.Apl, r0 + i0 + rr, h * HD + 4 * c4) : ld4(a.A + (r0 + i0 + rr) * qd + h * HD + 4 * c4);
         }
-        float *d = As + rr * lda + 4 * c4;
-        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+#pragma unroll
+        for (int u = 0; u < HD / 32; u++) {
+            const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
+            if (BWD && i0 + rr < N) st4(a.A_out + (r0 + i0 + rr) * qd + h * HD + 4 * c4, av[u]);
+            *reinterpret_cast<float4 *>(As + rr * lda + 4 * c4) = av[u];
+        }
     }
     __syncthreads();
 
-    // ---- phase 1: X = A B^T, one 32-key block per wave and round
-    for (int jb = wave; jb < nkb; jb += 4) {
-        const float16v acc = tile_abt<HD>(As, lda, b_row(jb), lane, bfirst, b_row(jb + 4 < nkb ? jb + 4 : jb));
+    // ---- phase 1: X = A B^T, one 32-key block per wave and round; the B rows of the block after it are on their way
+    auto put_x = [&](const float16v &acc, int jb) {
 #pragma unroll
         for (int v = 0; v < 16; v++) Xs[(8 * (v >> 2) + 4 * hh + (v & 3)) * ldx + jb * 32 + l31] = acc[v];
+    };
+    for (int jb = wave; jb < nkb; jb += 8) {
+        b_tile_load<HD>(bt1, b_row(jb + 4 < nkb ? jb + 4 : jb), ldt);
+        put_x(tile_abt<HD>(As, lda, lane, bt0), jb);
+        b_tile_load<HD>(bt0, b_row(jb + 8 < nkb ? jb + 8 : jb), ldt);
+        if (jb + 4 < nkb) put_x(tile_abt<HD>(As, lda, lane, bt1), jb + 4);
     }
     __syncthreads();
 
     // ---- row step
-    if (N <= 64) row_step<BWD, 1>(a, Xs, ldx, nk, N, i0, b, h, wave, lane);          // whole rows of N entries are written
-    else if (N <= 256) row_step<BWD, 4>(a, Xs, ldx, nk, N, i0, b, h, wave, lane);
-    else if (N <= 512) row_step<BWD, 8>(a, Xs, ldx, nk, N, i0, b, h, wave, lane);
-    else row_step<BWD, 16>(a, Xs, ldx, nk, N, i0, b, h, wave, lane);
+    if (N <= 64) row_step<BWD, 2>(a, Xs, ldx, nk, N, i0, b, h, tid);                 // whole rows of N entries are written
+    else if (N <= 256) row_step<BWD, 8>(a, Xs, ldx, nk, N, i0, b, h, tid);
+    else if (N <= 512) row_step<BWD, 16>(a, Xs, ldx, nk, N, i0, b, h, tid);
+    else row_step<BWD, 32>(a, Xs, ldx, nk, N, i0, b, h, tid);
     __syncthreads();
 
     // ---- phase 3: Y = X C, one 32-column block of the head per wave and round
     const int Kb = tiled_kb(qd);
     for (int dt = wave; dt * 32 < HD; dt += 4) {
-        if (dt != wave) c_chunk_load(cfirst, c_lane0 + dt * 32, (size_t)kd, 0, hh, N);
-        const float16v acc = tile_xc(Xs, ldx, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cfirst);
+        if (dt != wave) c_ring_start(cring, c_lane0 + dt * 32, (size_t)kd, nk, hh, N);
+        const float16v acc = tile_xc(Xs, ldx, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
         const int d = dt * 32 + l31;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
@@ -320,12 +366,14 @@ __global__ __launch_bounds__(256) void k_attn_dkv_tile(AttnDkvArgs a)
     }
 }
 
+size_t tile_lds_bytes(int hd, int seq) { return (size_t)32 * (hd + 4 + ((seq + 31) & ~31) + 4) * sizeof(float); }
+
 template <int BWD, int HD>
 void launch_tile_hd(const AttnTileArgs &a)
 {
     static bool attr_set = false;
     if (!attr_set) { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_attn_tile<BWD, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); attr_set = true; }
-    const size_t lds = (size_t)32 * (HD + 1 + ((a.seq + 63) & ~63) + 1) * sizeof(float);
+    const size_t lds = tile_lds_bytes(HD, a.seq);
     LAUNCH((k_attn_tile<BWD, HD>), dim3((a.seq + 31) / 32, a.Hq, a.batch), dim3(256), lds, a);
 }
 
@@ -340,7 +388,7 @@ void launch_tile(const AttnTileArgs &a)
     }
 }
 
-size_t tile_lds_bytes(int hd, int seq) { return (size_t)32 * (hd + 1 + ((seq + 63) & ~63) + 1) * sizeof(float); }
+
 
 }  // namespace
 
@@ -351,9 +399,9 @@ bool attn_mfma_supported(int hd, int seq)
 
 void launch_attn_fwd_mfma(const AttnFwdArgs &f)
 {
-    if (!attn_mfma_supported(f.hd, f.seq)) { fprintf(stderr, "[fast_hip] attn_fwd_mfma: unsupported shape\n"); abort(); }
+    if (!attn_mfma_supported(f.hd, f.seq) || !f.kT) { fprintf(stderr, "[fast_hip] attn_fwd_mfma: unsupported shape\n"); abort(); }
     AttnTileArgs a{};
-    a.A = f.q; a.B = f.k; a.C = f.v;
+    a.A = f.q; a.BT = f.kT; a.C = f.v;
     a.Hq = f.Hq; a.Hkv = f.Hkv; a.hd = f.hd; a.seq = f.seq; a.batch = f.batch; a.scale = f.scale;
     a.probs = f.probs; a.out16 = f.out16;
     launch_tile<0>(a);
@@ -361,9 +409,9 @@ void launch_attn_fwd_mfma(const AttnFwdArgs &f)
 
 void launch_attn_bwd_mfma(const AttnBwdArgs &g)
 {
-    if (!attn_mfma_supported(g.hd, g.seq)) { fprintf(stderr, "[fast_hip] attn_bwd_mfma: unsupported shape\n"); abort(); }
+    if (!attn_mfma_supported(g.hd, g.seq) || !g.vT) { fprintf(stderr, "[fast_hip] attn_bwd_mfma: unsupported shape\n"); abort(); }
     AttnTileArgs a{};
-    a.Apl = g.dO; a.B = g.v; a.C = g.k;
+    a.Apl = g.dO; a.BT = g.vT; a.C = g.k;
     a.Hq = g.Hq; a.Hkv = g.Hkv; a.hd = g.hd; a.seq = g.seq; a.batch = g.batch; a.scale = g.scale;
     a.probs = const_cast<float *>(g.probs); a.dscore = g.dscore; a.A_out = g.dO_red; a.out32 = g.dq;
     launch_tile<1>(a);

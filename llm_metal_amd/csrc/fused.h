@@ -32,6 +32,11 @@ struct NormRowsArgs {
 };
 void launch_norm_rows(const NormRowsArgs &a, int rows);
 
+// The matrix-core attention reads K and V once more from copies laid out [batch][Hkv][hd/4][attn_ldt(seq)][4]:
+// element (pos, d) of a head at ((d / 4) * ldt + pos) * 4 + d % 4.
+__host__ __device__ inline int attn_ldt(int seq) { return seq + 32; }
+__host__ __device__ inline size_t attn_t_index(int d, int pos, int ldt) { return ((size_t)(d >> 2) * ldt + pos) * 4 + (d & 3); }
+
 struct QkvPostArgs {
     Planes qkv;                   // [rows][q | k | v | tq(R) | tv(R)]
     const float *Bq, *Bv;         // LoRA B, [Hq*hd][R], [Hkv*hd][R]
@@ -41,6 +46,7 @@ struct QkvPostArgs {
     int Hq, Hkv, hd, seq;
     float *q_pre, *k_pre, *q_fin, *k_fin, *v_out;   // [rows][H*hd]
     float *tq, *tv;               // [rows][R]
+    float *kT, *vT;               // optional: the same k_fin / v_out per head and transposed, [batch][Hkv][hd/4][attn_ldt(seq)][4]
     int rows;
 };
 void launch_qkv_post(const QkvPostArgs &a, int rows);
@@ -52,12 +58,14 @@ struct AttnFwdArgs {
     const float *q, *k, *v; int Hq, Hkv, hd, seq, batch; float scale;
     float *probs;                 // [batch][Hq][seq][seq]
     half_t *out16;                // tiled [rows, Hq*hd], unit scale
+    const float *kT;              // k transposed per head [batch][Hkv][hd/4][attn_ldt(seq)][4] (matrix-core path only)
 };
 void launch_attn_fwd(const AttnFwdArgs &a);
 
 struct AttnBwdArgs {
     Planes dO;                    // [rows][Hq*hd]
     const float *probs, *q, *k, *v; int Hq, Hkv, hd, seq, batch; float scale;
+    const float *vT;              // v transposed per head [batch][Hkv][hd/4][attn_ldt(seq)][4] (matrix-core path only)
     float *dO_red, *dscore;       // scratch: [rows][Hq*hd], [batch][Hq][seq][seq]
     float *dq, *dk, *dv;          // [rows][Hq*hd], [rows][Hkv*hd] x2 (post-RoPE domain)
 };

@@ -196,7 +196,14 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
 #pragma unroll
         for (int p = 0; p < MAXP; p++) {
             const int d = lane + 64 * p;
-            if (d < half) { a.v_out[row * kd + h * hd + d] = x0[p]; a.v_out[row * kd + h * hd + d + half] = x1[p]; }
+            if (d < half) {
+                a.v_out[row * kd + h * hd + d] = x0[p]; a.v_out[row * kd + h * hd + d + half] = x1[p];
+                if (a.vT) {
+                    const int ldt = attn_ldt(a.seq), ps = (int)(row % a.seq);
+                    float *t = a.vT + ((row / a.seq * a.Hkv + h) * hd) * (size_t)ldt;
+                    t[attn_t_index(d, ps, ldt)] = x0[p]; t[attn_t_index(d + half, ps, ldt)] = x1[p];
+                }
+            }
         }
         return;
     }
@@ -215,8 +222,14 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
         pre[o + half] = x1[p];
         const float n0 = x0[p] * inv * g[d], n1 = x1[p] * inv * g[d + half];
         const float2 cs = a.rope[(size_t)pos * half + d];
-        fin[o] = n0 * cs.x - n1 * cs.y;
-        fin[o + half] = n0 * cs.y + n1 * cs.x;
+        const float f0 = n0 * cs.x - n1 * cs.y, f1 = n0 * cs.y + n1 * cs.x;
+        fin[o] = f0;
+        fin[o + half] = f1;
+        if (kind == 1 && a.kT) {
+            const int ldt = attn_ldt(a.seq);
+            float *t = a.kT + ((row / a.seq * a.Hkv + h) * hd) * (size_t)ldt;
+            t[attn_t_index(d, pos, ldt)] = f0; t[attn_t_index(d + half, pos, ldt)] = f1;
+        }
     }
 }
 

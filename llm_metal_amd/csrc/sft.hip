@@ -59,6 +59,7 @@ struct SFTState {
     MetalBuf *xs;                        // [2*NL + 1][BN*D]: x_in[L] = 2L, x_mid[L] = 2L+1, x_final = 2NL
     MetalBuf *ln1_16, *ln1_inv;          // [NL][BN*D] f16, [NL][BN]
     MetalBuf *q_pre, *k_pre, *q_fin, *k_fin, *v_sav, *probs, *gate_pre, *up_val, *tq, *tv, *o_raw, *ff_raw;
+    MetalBuf *kT, *vT;                   // k_fin / v_sav once more, per head and transposed, for the matrix-core attention
     // transients
     MetalBuf *a16, *a16_inv;             // largest fp16 operand (BN x max K) and its row factors
     MetalBuf *ones;                      // [BN] of 1.0f
@@ -232,6 +233,8 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         qa.q_fin = at<float>(s->q_fin, (size_t)L * BN * qd); qa.k_fin = at<float>(s->k_fin, (size_t)L * BN * kd);
         qa.v_out = at<float>(s->v_sav, (size_t)L * BN * kd);
         qa.tq = at<float>(s->tq, (size_t)L * BN * (R ? R : 1)); qa.tv = at<float>(s->tv, (size_t)L * BN * (R ? R : 1));
+        const size_t st_kt = (size_t)s->B * kd * attn_ldt(s->N);
+        if (s->kT) { qa.kT = at<float>(s->kT, (size_t)L * st_kt); qa.vT = at<float>(s->vT, (size_t)L * st_kt); }
         // causal GQA attention                                               [:678-689]
         half_t *attn16 = s->full_param ? at<half_t>(s->attn16, L * s->st_attn) : a16;
         float *probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
@@ -240,7 +243,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         AttnFwdArgs aa{};
         aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
-        aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16;
+        aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16; aa.kT = qa.kT;
         if (attn_mfma_supported(s->hd, s->N)) launch_attn_fwd_mfma(aa); else launch_attn_fwd(aa);
         // full-parameter mode keeps the FFN GEMM operands of every layer as well
         half_t *ln2 = s->full_param ? at<half_t>(s->ln2_16, L * s->st_ln1) : a16;
@@ -369,6 +372,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         ab.v = at<float>(s->v_sav, (size_t)L * BN * kd);
         ab.Hq = s->Hq; ab.Hkv = s->Hkv; ab.hd = s->hd; ab.seq = s->N; ab.batch = s->B;
         ab.scale = 1.0f / sqrtf((float)s->hd);
+        ab.vT = s->vT ? at<float>(s->vT, (size_t)L * s->B * kd * attn_ldt(s->N)) : nullptr;
         ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore);
         ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv);
         if (attn_mfma_supported(s->hd, s->N)) launch_attn_bwd_mfma(ab); else launch_attn_bwd(ab);
@@ -634,6 +638,9 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->q_pre = fbuf((size_t)NL * BN * qd); s->k_pre = fbuf((size_t)NL * BN * kd);
     s->q_fin = fbuf((size_t)NL * BN * qd); s->k_fin = fbuf((size_t)NL * BN * kd); s->v_sav = fbuf((size_t)NL * BN * kd);
     s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
+    if (attn_mfma_supported(s->hd, s->N)) {
+        s->kT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N)); s->vT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N));
+    }
     s->gate_pre = fbuf((size_t)NL * BN * IS); s->up_val = fbuf((size_t)NL * BN * IS);
     s->tq = fbuf((size_t)NL * BN * (R ? R : 1)); s->tv = fbuf((size_t)NL * BN * (R ? R : 1));
     const bool gemma = s->model_type == MODEL_GEMMA3;
@@ -688,7 +695,7 @@ void sft_state_free(SFTState *s)
                        s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
-                       s->gate_pre, s->up_val, s->tq, s->tv, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->ones, s->planes,
+                       s->gate_pre, s->up_val, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->ones, s->planes,
                        s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
                        s->dq, s->dk, s->dv, s->dq_f, s->dh,
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
