@@ -88,12 +88,15 @@ struct QkvBwdArgs {
 };
 void launch_qkv_bwd(const QkvBwdArgs &a, int rows);
 
+// All pointers address layer 0; layer L of a launch over `layers` layers lies L * (the matching stride) further on.
 struct LoraGradArgs {
     const float *dq_f, *dv_f, *tq, *tv, *dh;
     const half_t *ln16; const float *ln_inv_scale;  // tiled [rows, D]
     int rows, D, qd, kd, R; float sc;
-    float *grad;                  // this layer's arena: dA_q | dB_q | dA_v | dB_v
+    float *grad;                  // arena: dA_q | dB_q | dA_v | dB_v per layer
     float *sq_slots;              // one partial sum of squares per workgroup
+    int layers;
+    size_t st_dq, st_dv, st_t, st_dh, st_ln16, st_lninv, st_grad, st_slots;   // layer strides in elements
 };
 int  lora_grad_blocks(int D, int qd, int kd, int R);
 void launch_lora_grads(const LoraGradArgs &a);
@@ -118,9 +121,11 @@ void launch_norm_bwd_rows(const NormBwdArgs &a, int rows);
 struct CeArgs {
     const float *logits; int V; const uint32_t *targets; float *losses;
     half_t *dl16; float *inv_scale; int rows_total;     // tiled [rows, V]
+    float2 *partials;             // scratch [rows][CE_CHUNKS] (running maximum, sum of exponentials) of the row chunks
     // policy-gradient variant (grpo != 0): targets are the sampled actions; losses is not written
     int grpo; const float *old_lp, *advs; float *new_lp; float clip_eps, dl_scale;
 };
+constexpr int CE_CHUNKS = 16;
 void launch_ce_rows(const CeArgs &a, int rows);
 
 struct AdamArgs {

@@ -488,6 +488,11 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
 __global__ __launch_bounds__(TB) void k_lora_grads(LoraGradArgs a)
 {
     __shared__ float sm[16];
+    {                                                     // blockIdx.y = layer
+        const size_t L = blockIdx.y;
+        a.dq_f += L * a.st_dq; a.dv_f += L * a.st_dv; a.tq += L * a.st_t; a.tv += L * a.st_t; a.dh += L * a.st_dh;
+        a.ln16 += L * a.st_ln16; a.ln_inv_scale += L * a.st_lninv; a.grad += L * a.st_grad; a.sq_slots += L * a.st_slots;
+    }
     const size_t idx = (size_t)blockIdx.x * TB + threadIdx.x;
     const size_t nA = (size_t)a.R * a.D, nBq = (size_t)a.qd * a.R, nBv = (size_t)a.kd * a.R;
     float gval = 0.f;
@@ -695,41 +700,73 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 // src/nn/fast_sft.c:754-760.  The gradient is written once, as the lm_head dX GEMM's
 // fp16 operand: (softmax - onehot) * 1024 with row factor (1/BN) / 1024.  With a.grpo the row
 // factor carries the policy-gradient weight instead (src/nn/fast_grpo.c:437-452).
-__global__ __launch_bounds__(1024) void k_ce_rows(CeArgs a)
+// A row of logits (150 k to 260 k floats) is cut into CE_CHUNKS pieces so that rows x CE_CHUNKS workgroups
+// share the work: the first launch leaves every piece's maximum and sum of exponentials, the second combines
+// them into the row's log-sum-exp and writes its piece of the gradient.
+__device__ __forceinline__ void ce_chunk_range(int V, int chunk, int &c_beg, int &c_end)
+{
+    const int groups = tiled_kb(V) * 8;                   // 8-column groups of the tiled fp16 row, K padding included
+    const int per = (groups + CE_CHUNKS - 1) / CE_CHUNKS;
+    c_beg = min(chunk * per, groups);
+    c_end = min(c_beg + per, groups);
+}
+
+__global__ __launch_bounds__(256) void k_ce_partial(CeArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
-    const int V = a.V;
+    const size_t r = blockIdx.y;
+    const int chunk = blockIdx.x, V = a.V;
     const float *lg = a.logits + r * V;
-    const uint32_t tgt = a.targets[r];
-    const int nv = V >> 2;                                // V % 4 == 0 is checked by the launcher
+    int c_beg, c_end;
+    ce_chunk_range(V, chunk, c_beg, c_end);
+    const int e_beg = min(c_beg * 8, V), e_end = min(c_end * 8, V);     // V % 4 == 0 is checked by the launcher
     float mx = -1e30f;
-    for (int v = threadIdx.x; v < nv; v += blockDim.x) { const float4 x = ld4(lg + 4 * v); mx = fmaxf(mx, fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w))); }
+    for (int i = e_beg + 4 * threadIdx.x; i < e_end; i += 4 * 256) { const float4 x = ld4(lg + i); mx = fmaxf(mx, fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w))); }
     mx = block_max(mx, sm);
     float sum = 0.f;
-    for (int v = threadIdx.x; v < nv; v += blockDim.x) {
-        const float4 x = ld4(lg + 4 * v);
+    for (int i = e_beg + 4 * threadIdx.x; i < e_end; i += 4 * 256) {
+        const float4 x = ld4(lg + i);
         sum += expf(x.x - mx) + expf(x.y - mx) + expf(x.z - mx) + expf(x.w - mx);
     }
     sum = block_sum(sum, sm);
+    if (threadIdx.x == 0) a.partials[r * CE_CHUNKS + chunk] = make_float2(mx, sum);
+}
+
+__global__ __launch_bounds__(256) void k_ce_rows(CeArgs a)
+{
+    const size_t r = blockIdx.y;
+    const int chunk = blockIdx.x, V = a.V;
+    const float *lg = a.logits + r * V;
+    const uint32_t tgt = a.targets[r];
+    float mx = -1e30f;
+    float2 part[CE_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CE_CHUNKS; c++) { part[c] = a.partials[r * CE_CHUNKS + c]; mx = fmaxf(mx, part[c].x); }
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CE_CHUNKS; c++) sum += part[c].y * expf(part[c].x - mx);      // empty pieces: 0 * exp(-1e30 - mx) = 0
     const float lse = logf(sum) + mx;
-    // coefficient of (softmax - onehot): 1/BN for the cross-entropy; w * ratio * dl_scale for the
-    // PPO-clip policy gradient (grpo_policy_grad, shaders/q8_kernels.metal:741-760)
-    float coef = 1.0f / (float)a.rows_total;
-    if (a.grpo) {
-        const float new_lp = lg[tgt] - lse;
-        const float ratio = expf(new_lp - a.old_lp[r]);
-        const float clipped = fminf(fmaxf(ratio, 1.0f - a.clip_eps), 1.0f + a.clip_eps);
-        const float adv = a.advs[r];
-        const float w = (adv >= 0.f) ? ((ratio <= clipped) ? -adv : 0.f) : ((ratio >= clipped) ? -adv : 0.f);
-        coef = w * ratio * a.dl_scale;
-        if (threadIdx.x == 0) a.new_lp[r] = new_lp;
-    } else if (threadIdx.x == 0) {
-        a.losses[r] = lse - lg[tgt];
+    if (chunk == 0 && threadIdx.x == 0) {
+        // coefficient of (softmax - onehot): 1/BN for the cross-entropy; w * ratio * dl_scale for the
+        // PPO-clip policy gradient (grpo_policy_grad, shaders/q8_kernels.metal:741-760)
+        float coef = 1.0f / (float)a.rows_total;
+        if (a.grpo) {
+            const float new_lp = lg[tgt] - lse;
+            const float ratio = expf(new_lp - a.old_lp[r]);
+            const float clipped = fminf(fmaxf(ratio, 1.0f - a.clip_eps), 1.0f + a.clip_eps);
+            const float adv = a.advs[r];
+            const float w = (adv >= 0.f) ? ((ratio <= clipped) ? -adv : 0.f) : ((ratio >= clipped) ? -adv : 0.f);
+            coef = w * ratio * a.dl_scale;
+            a.new_lp[r] = new_lp;
+        } else {
+            a.losses[r] = lse - lg[tgt];
+        }
+        a.inv_scale[r] = coef * (1.0f / 1024.0f);
     }
-    if (threadIdx.x == 0) a.inv_scale[r] = coef * (1.0f / 1024.0f);
+    int c_beg, c_end;
+    ce_chunk_range(V, chunk, c_beg, c_end);
     const int Kb = tiled_kb(V);
-    for (int c = threadIdx.x; c < Kb * 8; c += blockDim.x) {
+    for (int c = c_beg + threadIdx.x; c < c_end; c += 256) {
         half8 hv;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -872,7 +909,7 @@ int lora_grad_blocks(int D, int qd, int kd, int R)
 
 void launch_lora_grads(const LoraGradArgs &a)
 {
-    LAUNCH(k_lora_grads, dim3(lora_grad_blocks(a.D, a.qd, a.kd, a.R)), dim3(TB), 0, a);
+    LAUNCH(k_lora_grads, dim3(lora_grad_blocks(a.D, a.qd, a.kd, a.R), a.layers > 0 ? a.layers : 1), dim3(TB), 0, a);
 }
 
 void launch_glu_fwd(const GluArgs &a, int rows)
@@ -895,7 +932,9 @@ void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
 void launch_ce_rows(const CeArgs &a, int rows)
 {
     require(a.V % 4 == 0, "ce_rows: vocabulary size must be a multiple of 4");
-    LAUNCH(k_ce_rows, dim3(rows), dim3(a.V >= 4096 ? 1024 : 256), 0, a);
+    require(a.partials != nullptr, "ce_rows: partials scratch missing");
+    LAUNCH(k_ce_partial, dim3(CE_CHUNKS, rows), dim3(256), 0, a);
+    LAUNCH(k_ce_rows, dim3(CE_CHUNKS, rows), dim3(256), 0, a);
 }
 
 void launch_adamw(const AdamArgs &a)

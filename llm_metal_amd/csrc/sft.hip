@@ -65,7 +65,9 @@ struct SFTState {
     MetalBuf *ones;                      // [BN] of 1.0f
     MetalBuf *planes;
     MetalBuf *logits, *dlogits, *dl16, *dl_inv;
-    MetalBuf *dx[2], *dO_red, *dscore, *dq, *dk, *dv, *dq_f, *dh;
+    MetalBuf *dx[2], *dO_red, *dscore, *dq, *dk, *dv, *dq_f, *dh;   // LoRA mode: dv, dq_f, dh are kept per layer until the
+                                                                   // adapter gradients of all layers are formed in one launch
+    MetalBuf *ce_part;
     size_t planes_cap;
 
     // full-parameter mode (lora_rank == 0): the GEMM operands of the forward are kept per layer, because
@@ -374,7 +376,8 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         ab.scale = 1.0f / sqrtf((float)s->hd);
         ab.vT = s->vT ? at<float>(s->vT, (size_t)L * s->B * kd * attn_ldt(s->N)) : nullptr;
         ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore);
-        ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv);
+        const size_t keepL = R ? (size_t)L : 0;                 // LoRA mode keeps dv, dq_f and dh of every layer
+        ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv, keepL * BN * kd);
         if (attn_mfma_supported(s->hd, s->N)) launch_attn_bwd_mfma(ab); else launch_attn_bwd(ab);
 
         // inverse RoPE, QK-norm backward, dh; LoRA gradients                  [:912-966]
@@ -387,20 +390,9 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         qb.Bv = at<float>(s->lora, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
         qb.R = R; qb.sc = s->lora_scaling;
         qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
-        qb.dq_f = at<float>(s->dq_f); qb.dv_f = nullptr; qb.dh = at<float>(s->dh);
+        qb.dq_f = at<float>(s->dq_f, keepL * BN * qd); qb.dv_f = nullptr; qb.dh = at<float>(s->dh, keepL * BN * (R ? 2 * R : 1));
         qb.out16 = a16; qb.inv_scale = ainv;
         launch_qkv_bwd(qb, BN);
-        if (R > 0) {
-            LoraGradArgs lg{};
-            lg.dq_f = qb.dq_f; lg.dv_f = ab.dv; lg.tq = at<float>(s->tq, (size_t)L * BN * R); lg.tv = at<float>(s->tv, (size_t)L * BN * R);
-            lg.dh = qb.dh;
-            lg.ln16 = at<half_t>(s->ln1_16, (size_t)L * s->st_ln1); lg.ln_inv_scale = at<float>(s->ln1_inv, (size_t)L * BN);
-            lg.rows = BN; lg.D = D; lg.qd = qd; lg.kd = kd; lg.R = R; lg.sc = s->lora_scaling;
-            lg.grad = at<float>(s->lora_grad, L * s->lsz);
-            lg.sq_slots = at<float>(s->sq_slots, (size_t)L * s->slots_per_layer);
-            launch_lora_grads(lg);
-        }
-
         // full-parameter: W_q, W_k, W_v are updated BEFORE the dX product, which then multiplies with the
         // new weights in SGD mode, as the reference does                       [:922-946]
         if (mode != BWD_LORA)
@@ -418,6 +410,19 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         }
         launch_norm_bwd_rows(n1, BN);
         cur ^= 1;
+    }
+
+    // LoRA gradients of all layers in one launch: dB = sc * dY^T t, dA = dh^T ln1     [:948-952, 962-966]
+    if (R > 0) {
+        LoraGradArgs lg{};
+        lg.dq_f = at<float>(s->dq_f); lg.dv_f = at<float>(s->dv); lg.tq = at<float>(s->tq); lg.tv = at<float>(s->tv); lg.dh = at<float>(s->dh);
+        lg.ln16 = at<half_t>(s->ln1_16); lg.ln_inv_scale = at<float>(s->ln1_inv);
+        lg.rows = BN; lg.D = D; lg.qd = qd; lg.kd = kd; lg.R = R; lg.sc = s->lora_scaling;
+        lg.grad = at<float>(s->lora_grad); lg.sq_slots = at<float>(s->sq_slots);
+        lg.layers = NL;
+        lg.st_dq = (size_t)BN * qd; lg.st_dv = (size_t)BN * kd; lg.st_t = (size_t)BN * R; lg.st_dh = (size_t)BN * 2 * R;
+        lg.st_ln16 = s->st_ln1; lg.st_lninv = BN; lg.st_grad = s->lsz; lg.st_slots = s->slots_per_layer;
+        launch_lora_grads(lg);
     }
 }
 
@@ -658,8 +663,10 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->dl16 = hbuf(tiled_elems(BN, V)); s->dl_inv = fbuf(BN);
     s->dx[0] = fbuf(xsz); s->dx[1] = fbuf(xsz);
     s->dO_red = fbuf((size_t)BN * qd); s->dscore = fbuf((size_t)s->B * s->Hq * s->N * s->N);
-    s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf((size_t)BN * kd);
-    s->dq_f = fbuf((size_t)BN * qd); s->dh = fbuf((size_t)BN * (R ? 2 * R : 1));
+    const size_t keep = R ? NL : 1;
+    s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf(keep * BN * kd);
+    s->dq_f = fbuf(keep * BN * qd); s->dh = fbuf(keep * BN * (R ? 2 * R : 1));
+    s->ce_part = metal_buf_create((size_t)BN * CE_CHUNKS * sizeof(float2));
 
     // ---- full-parameter mode: kept GEMM operands and the transposed pair of one weight gradient ----
     s->st_act = tiled_elems(BN, IS); s->st_attn = tiled_elems(BN, qd);
@@ -697,7 +704,7 @@ void sft_state_free(SFTState *s)
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
                        s->gate_pre, s->up_val, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->ones, s->planes,
                        s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
-                       s->dq, s->dk, s->dv, s->dq_f, s->dh,
+                       s->dq, s->dk, s->dv, s->dq_f, s->dh, s->ce_part,
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
                        s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
                        s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf};
@@ -714,6 +721,7 @@ static void enqueue_step_kernels(SFTState *s, float lr)
     CeArgs ce{};
     ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
     ce.dl16 = at<half_t>(s->dl16); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
+    ce.partials = at<float2>(s->ce_part);
     launch_ce_rows(ce, s->BN);
     if (s->full_param) backward_impl(s, s->gqkv ? BWD_ACCUM : BWD_SGD, lr);     // src/nn/fast_sft.c:1136-1140 with :778-786
     else backward_impl(s);
@@ -1034,6 +1042,7 @@ void grpo_apply_completions(SFTState *s, const GRPOCompletions *c, float lr, flo
         CeArgs ce{};
         ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
         ce.dl16 = at<half_t>(s->dl16); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
+        ce.partials = at<float2>(s->ce_part);
         ce.grpo = 1; ce.old_lp = at<float>(s->grpo_old_lp); ce.advs = at<float>(s->grpo_advs); ce.new_lp = at<float>(s->grpo_new_lp);
         ce.clip_eps = c->clip_eps; ce.dl_scale = 1.0f / (float)G;                 // [:445-452]
         launch_ce_rows(ce, s->BN);
