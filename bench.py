@@ -23,6 +23,19 @@ from llm_metal_amd.configs import CONFIGS  # noqa: E402
 from llm_metal_amd.synth import make_batch, make_model  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFS = 2500.0          # dense fp16 MFMA
+
+
+def measured_traffic(cfg_name):
+    """HBM bytes per GEMM launch from the committed hardware-counter summary of this workload (two rocprofv3
+    --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by a copy kernel of known size), or None when there is none."""
+    path = os.path.join(ROOT, "profiles", "c3_gemm_hbm_traffic_pmc.txt")
+    if cfg_name != "c3_qwen3_4b_f16" or not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_gemm_launch_c3"):
+            return float(line.split("=")[1])
+    return None
 
 
 def cpu_baseline(cfg, budget_s=20.0):
@@ -30,8 +43,8 @@ def cpu_baseline(cfg, budget_s=20.0):
     sample of the same workload: the full step on a model with fewer layers and a truncated
     vocabulary, scaled to the full configuration by the GEMM flop ratio."""
     from oracle import oracle
-    nl = 1
-    v = min(cfg.V, 8192)
+    nl = min(cfg.NL, 3)
+    v = min(cfg.V, 16384)
     small = cfg.with_(name=cfg.name + "_sample", NL=nl, V=v, tied=False)
     model = make_model(small, seed=0)
     used = oracle.weights_as_used(model)
@@ -135,16 +148,24 @@ def main():
     for i in range(prof_steps):
         step(i)
     import ctypes as C
-    tms, wb = C.c_double(0), C.c_double(0)
-    n = L.hip_gemm_profile_read(C.byref(tms), C.byref(wb))
+    tms, wb, fl = C.c_double(0), C.c_double(0), C.c_double(0)
+    n = L.hip_gemm_profile_read2(C.byref(tms), C.byref(wb), C.byref(fl))
     L.hip_gemm_profile_enable(0)
     gbs = wb.value / (tms.value * 1e-3) / 1e9 if tms.value > 0 else 0.0
-    roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+    tfs = fl.value / (tms.value * 1e-3) / 1e12 if tms.value > 0 else 0.0
+    # the GEMMs stream every weight once per pass; from a few hundred rows on their flops, not the bytes, bound them
+    # (ridge of the MI355X: 2.5 PFLOP/s / 8 TB/s = 312 flop per byte = 156 rows of F16 weights, 83 rows of Q8_0)
+    compute_bound = fl.value / max(wb.value, 1.0) > MFMA_PEAK_TFS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    roofline = {"bound": "mfma" if compute_bound else "hbm",
+                "achieved": round(tfs if compute_bound else gbs, 1),
+                "peak": MFMA_PEAK_TFS if compute_bound else HBM_PEAK_GBS,
+                "unit": "TFLOP/s" if compute_bound else "GB/s",
+                "frac": round(tfs / MFMA_PEAK_TFS if compute_bound else gbs / HBM_PEAK_GBS, 4), "traffic": None,
                 "kernel": "gemm_tiled", "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
-                "weight_bytes_per_step": wb.value / prof_steps,
+                "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}
+    roofline["traffic"] = measured_traffic(cfg.name)
     st.free()
 
     metric = ("SFT train tokens/s, Qwen3-4B LoRA r16 seq64; % of HBM-BW / MFMA peak" if cfg.name == "c3_qwen3_4b_f16" else
