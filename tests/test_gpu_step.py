@@ -36,6 +36,9 @@ CASES = [
     C1.with_(name="q8_odd_blocks", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_q8", weight_format="q8_0"),
     C1.with_(name="q8_fallback", NL=2, D=128, Hq=3, Hkv=1, hd=32, IS=256, V=1024, seq=24, weight_format="q8_0"),
+    # long sequences: 16 key blocks per query block (config 4's 512), and a ragged length beyond 256
+    C1.with_(name="seq512", NL=1, seq=512, V=1024),
+    C1.with_(name="seq300_hd128", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300),
     # every product through the LDS-tiled large-M GEMM (F16 tiles; Q8_0 unpacked into LDS with row and column
     # scales; row counts that are not multiples of the 128-row block)
     C1.with_(name="big_m_f16", batch=4, seq=64),
