@@ -123,18 +123,17 @@ void hip_enqueue_q8_dequant(MetalBuf *src, MetalBuf *dst, int rows, int cols);
 /* dst F16 [rows, cols] = half(float(scale) * code): the values the dequant-fused GEMM multiplies with */
 void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
 
-/* Timing aid for benchmarks: when enabled, every launch of the weight-streaming
- * GEMM is bracketed by HIP events on the library's stream.  hip_gemm_profile_read
- * (after metal_flush) returns the number of launches recorded since the last
- * enable and adds up their durations (ms) and weight bytes. */
 /* 0: choose the GEMM kernel by the measured rule; 1: always the LDS-tiled large-M kernel; -1: never. */
 void hip_gemm_force_large_m(int policy);
+/* Timing aid for benchmarks: when enabled, every GEMM launch is bracketed by HIP events on the
+ * library's stream.  hip_gemm_profile_read (after metal_flush) returns the number of launches recorded
+ * since the last enable and adds up their durations (ms) and weight bytes; _read2 also their flops. */
 void hip_gemm_profile_enable(int on);
 int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
 int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double *total_flops);
 /* Microbenchmark of the GEMM alone at one shape (M rows, N x K weight) on synthetic operands,
  * rotating through > 1 GB of distinct weight images.  nb / S = 0: planner's choice, else forced
- * tile height (1, 2) and K split.  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
+ * tile height (1, 2; 128 = the large-M kernel) and K split.  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
  * 2 Q8_0 with column scales (transposed image).  Returns average ms per launch. */
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S);
 
