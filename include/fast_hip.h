@@ -67,6 +67,35 @@ void metal_enqueue_silu_mul(MetalBuf *gate, MetalBuf *up, int n);
 void metal_enqueue_gelu_mul(MetalBuf *gate, MetalBuf *up, int n);
 void metal_enqueue_residual_add(MetalBuf *x, MetalBuf *y, int n);
 
+/* ---- inference enqueues (src/nn/fast_metal.h:19-80): one decode step, all activations fp32 ---- */
+/* y[rows] = W x, W = rows x nb Q8_0 blocks of 34 bytes (src/nn/fast_metal.h:20-21).  The first call on a weight
+ * builds an aligned image of it (all codes, then all scales: its size again in HBM), kept until the buffer is written. */
+void metal_enqueue_q8_matvec(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int nb);
+/* y[rows] = W x, W F16 [rows, cols] (src/nn/fast_metal.h:24-25) */
+void metal_enqueue_f16_matvec(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols);
+/* Y[B, rows] = X[B, cols] W^T (src/nn/fast_metal.h:28-29); any B (the reference's kernel holds at most 32) */
+void metal_enqueue_f16_batch_matvec(MetalBuf *W, MetalBuf *X, MetalBuf *Y, int rows, int cols, int B);
+/* out = gamma * x / sqrt(mean(x^2) + eps) for one vector (src/nn/fast_metal.h:33-34); out may alias x */
+void metal_enqueue_rms_norm(MetalBuf *x, MetalBuf *gamma, MetalBuf *out, int dim, float eps);
+/* in-place RMSNorm of each of n_heads vectors of head_dim with a shared gamma (src/nn/fast_metal.h:39-40) */
+void metal_enqueue_per_head_rms_norm(MetalBuf *vec, MetalBuf *gamma, int n_heads, int head_dim, float eps);
+/* half-split rotary embedding of q [Hq*hd] and k [Hkv*hd] at position pos (src/nn/fast_metal.h:43-44) */
+void metal_enqueue_rope(MetalBuf *q, MetalBuf *k, int Hq, int Hkv, int hd, int pos, float theta);
+/* caches [Hkv, max_seq, hd]: row pos of every head := k, v (src/nn/fast_metal.h:47-49) */
+void metal_enqueue_kv_cache_store(MetalBuf *k, MetalBuf *v, MetalBuf *k_cache, MetalBuf *v_cache,
+                                  int Hkv, int max_seq, int hd, int pos);
+/* out[h] = softmax(q[h] K[h / group_ratio, 0..n_attend)^T / sqrt(hd)) V (src/nn/fast_metal.h:52-54); hd <= 256,
+ * group_ratio <= 16; the reference holds the scores of at most 4096 keys, this one any n_attend <= max_seq */
+void metal_enqueue_attention(MetalBuf *Q, MetalBuf *Kc, MetalBuf *Vc, MetalBuf *attn_out, int n_attend, int hd,
+                             int max_seq, int Hq, int group_ratio);
+/* the same four with byte offsets into the per-item buffers (src/nn/fast_metal.h:66-80); offsets are multiples of 4 */
+void metal_enqueue_per_head_rms_norm_off(MetalBuf *vec, size_t vec_off, MetalBuf *gamma, int n_heads, int head_dim, float eps);
+void metal_enqueue_rope_off(MetalBuf *q, size_t q_off, MetalBuf *k, size_t k_off, int Hq, int Hkv, int hd, int pos, float theta);
+void metal_enqueue_kv_cache_store_off(MetalBuf *k, size_t k_off, MetalBuf *v, size_t v_off, MetalBuf *k_cache,
+                                      MetalBuf *v_cache, int Hkv, int max_seq, int hd, int pos);
+void metal_enqueue_attention_off(MetalBuf *Q, size_t q_off, MetalBuf *Kc, MetalBuf *Vc, MetalBuf *attn_out, size_t out_off,
+                                 int n_attend, int hd, int max_seq, int Hq, int group_ratio);
+
 /* ---- training enqueues (src/nn/fast_metal.h:88-188) ----
  * Argument ORDER follows the reference's implementation and call sites
  * (src/nn/fast_metal.m:562-594, src/nn/fast_sft.c:638): the first buffer is the

@@ -14,9 +14,9 @@ struct MetalBuf {
     int     owns;         // 0 for views
     MetalBuf *parent;     // views: the buffer whose allocation this window lies in
     size_t  parent_off;
-    // lazily built tiled images of an F16 weight held in this buffer ([0] as is, [1] transposed),
-    // used by metal_enqueue_f16_matmul / _nt
-    struct Tiled { void *dev; int rows, cols; uint64_t version; } tiled[2];
+    // lazily built images of a weight held in this buffer: [0], [1] tiled F16 (as is, transposed) for
+    // metal_enqueue_f16_matmul / _nt; [2] Q8_0 split into codes and scales for metal_enqueue_q8_matvec
+    struct Tiled { void *dev; int rows, cols; uint64_t version; } tiled[3];
     uint64_t version;     // bumped by every enqueue that writes this buffer
 };
 

@@ -1,0 +1,574 @@
+// The inference enqueues of the reference's dispatch ABI (src/nn/fast_metal.h:19-80) as HIP kernels with the
+// reference's buffer layouts: the matrix-vector products of a decode step (F16 rows, Q8_0 blocks, a batch of up to 32
+// vectors), the single-vector RMSNorm / per-head RMSNorm / RoPE / KV-cache store, and attention of one query per head
+// over the cache.  All activations fp32.
+//
+// The products are pure weight streaming (2 flop per weight), so the kernels are shaped for HBM: one wave per weight
+// row (four rows per wave when there are enough rows), 16-byte (F16) or 8-byte (Q8_0) loads per lane with several in
+// flight, the vector(s) held in LDS once per workgroup, fp32 accumulation.  Q8_0 blocks are 34 bytes and therefore
+// never aligned; the weight is re-laid once into a split image (all int8 codes, row-major, then all fp16 scales), kept
+// with the buffer until something writes it, and the product streams that image.
+#include "backend.h"
+#include "devutil.h"
+
+using namespace lmhip;
+
+namespace {
+
+constexpr int TB = 256;
+#define LAUNCH(kern, grid, block, lds, ...) do { \
+    hipLaunchKernelGGL(kern, grid, block, lds, stream(), __VA_ARGS__); HIP_CHECK(hipGetLastError()); } while (0)
+
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+__global__ __launch_bounds__(TB) void k_zero(float *p, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * TB + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+// a product over an empty reduction
+void zero_result(MetalBuf *y, size_t n)
+{
+    LAUNCH(k_zero, dim3((unsigned)((n + TB - 1) / TB)), dim3(TB), 0, dptr_as<float>(y), n);
+    mark_written(y);
+}
+
+// ---------------------------------------------------------------- Q8_0 split image
+
+// blocks [n_blocks] of {fp16 d; int8 q[32]} -> q [n_blocks * 32], d [n_blocks]; thread per code
+__global__ __launch_bounds__(TB) void k_q8_split(const uint8_t *__restrict__ blocks, int8_t *__restrict__ q,
+                                                 uint16_t *__restrict__ d, size_t n_blocks)
+{
+    const size_t idx = (size_t)blockIdx.x * TB + threadIdx.x;
+    if (idx >= n_blocks * 32) return;
+    const size_t b = idx >> 5;
+    const int j = (int)(idx & 31);
+    const uint8_t *blk = blocks + b * 34;
+    q[idx] = (int8_t)blk[2 + j];
+    if (j == 0) d[b] = (uint16_t)(blk[0] | (blk[1] << 8));
+}
+
+inline size_t q8_scale_offset(size_t n_blocks) { return (n_blocks * 32 + 255) & ~(size_t)255; }
+
+// Split image of a Q8_0 weight held in W (rows x nb blocks).  Cached with the buffer (slot 2 of its
+// derived images) while the buffer is device-resident and unwritten; otherwise rebuilt in scratch.
+const int8_t *q8_split_of(MetalBuf *W, int rows, int nb, const half_t **scales)
+{
+    const size_t n_blocks = (size_t)rows * nb, soff = q8_scale_offset(n_blocks), bytes = soff + n_blocks * 2;
+    const bool cacheable = W->owns && !W->host && !W->parent;
+    uint8_t *img;
+    bool build = true;
+    if (!cacheable) {
+        img = (uint8_t *)scratch(SCR_MISC, bytes);
+    } else {
+        MetalBuf::Tiled &c = W->tiled[2];
+        if (c.dev && (c.rows != rows || c.cols != nb)) {
+            HIP_CHECK(hipStreamSynchronize(stream()));
+            HIP_CHECK(hipFree(c.dev));
+            c.dev = nullptr;
+        }
+        if (!c.dev) HIP_CHECK(hipMalloc(&c.dev, bytes));
+        else if (c.version == W->version) build = false;
+        c.rows = rows; c.cols = nb; c.version = W->version;
+        img = (uint8_t *)c.dev;
+    }
+    if (build)
+        LAUNCH(k_q8_split, dim3((unsigned)((n_blocks * 32 + TB - 1) / TB)), dim3(TB), 0, dptr_as<uint8_t>(W), (int8_t *)img,
+               (uint16_t *)(img + soff), n_blocks);
+    *scales = (const half_t *)(img + soff);
+    return (const int8_t *)img;
+}
+
+// ---------------------------------------------------------------- matrix-vector products
+
+// Y[b, row] = sum_c W[row, c] X[b, c] for b < B <= NBT.  FMT 0: W F16 row-major.  FMT 1: W int8 codes row-major with
+// one fp16 scale per 32 columns.  Requires cols % 8 == 0 and 16-byte aligned W and X.
+// Workgroup = 4 waves; wave w owns rows (4 blockIdx.x + w) R .. + R - 1; a lane owns 8 consecutive columns of every
+// 512-column step and U steps are loaded before any is used.  The vectors are staged through LDS in chunks of kc
+// columns (kc % 512 == 0).  Q8_0: codes are biased to unsigned (q + 128, one v_cvt_f32_ubyte each) and the bias is
+// taken out with the lane's sum of x, once per step for all rows.
+template <int FMT, int R, int U, int NBT>
+__global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, const half_t *__restrict__ scales,
+                                               const float *__restrict__ X, float *__restrict__ Y, int rows, int cols,
+                                               int B, int kc)
+{
+    extern __shared__ float xs[];                               // [NBT][kc]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = (blockIdx.x * 4 + wave) * R;
+    size_t roff[R];                                             // element offset of each row (clamped: extra rows are not stored)
+#pragma unroll
+    for (int r = 0; r < R; r++) roff[r] = (size_t)min(row0 + r, rows - 1) * cols;
+    float acc[R][NBT];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int b = 0; b < NBT; b++) acc[r][b] = 0.f;
+
+    for (int c0 = 0; c0 < cols; c0 += kc) {
+        const int n = min(kc, cols - c0);                       // multiple of 8
+        __syncthreads();
+        for (int b = 0; b < NBT; b++) {
+            const float *xrow = X + (size_t)min(b, B - 1) * cols + c0;
+            for (int i = tid * 4; i < n; i += TB * 4)
+                *reinterpret_cast<float4v *>(&xs[b * kc + i]) = *reinterpret_cast<const float4v *>(&xrow[i]);
+        }
+        __syncthreads();
+        for (int c = lane * 8; c < n; c += 512 * U) {
+            half8  w16[R][U];
+            uint2v w8[R][U];
+            float  dsc[R][U];
+            int    cu[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) cu[u] = min(c + 512 * u, n - 8);        // clamped: loads stay unconditional
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const size_t e = roff[r] + c0 + cu[u];
+                    if (FMT == 0) w16[r][u] = __builtin_nontemporal_load(reinterpret_cast<const half8 *>((const half_t *)Wp + e));
+                    else {
+                        w8[r][u] = __builtin_nontemporal_load(reinterpret_cast<const uint2v *>((const int8_t *)Wp + e));
+                        dsc[r][u] = (float)scales[e >> 5];
+                    }
+                }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float live = (c + 512 * u < n) ? 1.f : 0.f;
+                float xv[NBT][8], xsum[NBT];
+#pragma unroll
+                for (int b = 0; b < NBT; b++) {
+                    const float4v x0 = *reinterpret_cast<const float4v *>(&xs[b * kc + cu[u]]);
+                    const float4v x1 = *reinterpret_cast<const float4v *>(&xs[b * kc + cu[u] + 4]);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { xv[b][e] = x0[e] * live; xv[b][4 + e] = x1[e] * live; }
+                    if (FMT == 1) {
+                        float s = 0.f;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) s += xv[b][e];
+                        xsum[b] = 128.f * s;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    if (FMT == 0) {
+#pragma unroll
+                        for (int b = 0; b < NBT; b++)
+#pragma unroll
+                            for (int e = 0; e < 8; e++) acc[r][b] = fmaf((float)w16[r][u][e], xv[b][e], acc[r][b]);
+                    } else {
+                        const uint32_t lo = w8[r][u][0] ^ 0x80808080u, hi = w8[r][u][1] ^ 0x80808080u;
+                        float uf[8];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            uf[e] = (float)((lo >> (8 * e)) & 255u);
+                            uf[4 + e] = (float)((hi >> (8 * e)) & 255u);
+                        }
+#pragma unroll
+                        for (int b = 0; b < NBT; b++) {
+                            float p = -xsum[b];
+#pragma unroll
+                            for (int e = 0; e < 8; e++) p = fmaf(uf[e], xv[b][e], p);
+                            acc[r][b] = fmaf(dsc[r][u], p, acc[r][b]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int b = 0; b < NBT; b++) {
+            const float s = wave_sum(acc[r][b]);
+            if (lane == 0 && row0 + r < rows && b < B) Y[(size_t)b * rows + row0 + r] = s;
+        }
+}
+
+// Any cols / alignment: one wave per row, lanes stride single elements.
+__global__ __launch_bounds__(TB) void k_matvec_any(const half_t *__restrict__ W, const float *__restrict__ X,
+                                                   float *__restrict__ Y, int rows, int cols, int B)
+{
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const half_t *w = W + (size_t)row * cols;
+    for (int b = 0; b < B; b++) {
+        const float *x = X + (size_t)b * cols;
+        float s = 0.f;
+        for (int i = lane; i < cols; i += 64) s = fmaf((float)w[i], x[i], s);
+        s = wave_sum(s);
+        if (lane == 0) Y[(size_t)b * rows + row] = s;
+    }
+}
+
+template <int FMT, int NBT>
+void launch_matvec(const void *W, const half_t *scales, const float *X, float *Y, int rows, int cols, int B)
+{
+    // LDS budget 48 KB per workgroup (three workgroups per CU stay resident)
+    int kc = (48 * 1024 / 4 / NBT) / 512 * 512;
+    kc = min(kc, (cols + 511) / 512 * 512);
+    const size_t lds = (size_t)NBT * kc * 4;
+    constexpr int U1 = NBT == 1 ? 4 : (NBT <= 4 ? 2 : 1);        // one row per wave: loads in flight come from column steps
+    constexpr int U4 = NBT == 1 ? 2 : 1;
+    if (rows >= 4096)
+        LAUNCH((k_matvec<FMT, 4, U4, NBT>), dim3((rows + 15) / 16), dim3(TB), lds, W, scales, X, Y, rows, cols, B, kc);
+    else
+        LAUNCH((k_matvec<FMT, 1, U1, NBT>), dim3((rows + 3) / 4), dim3(TB), lds, W, scales, X, Y, rows, cols, B, kc);
+}
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+void f16_matvec_any_batch(const half_t *W, const float *X, float *Y, int rows, int cols, int B)
+{
+    if (cols % 8 || !aligned16(W) || !aligned16(X)) {
+        LAUNCH(k_matvec_any, dim3((rows + 3) / 4), dim3(TB), 0, W, X, Y, rows, cols, B);
+        return;
+    }
+    // batches beyond 8 vectors stream the weight once per group of 8 (the later passes mostly hit the caches)
+    for (int b0 = 0; b0 < B; b0 += 8) {
+        const int nb = min(8, B - b0);
+        const float *x = X + (size_t)b0 * cols;
+        float *y = Y + (size_t)b0 * rows;
+        if (nb == 1) launch_matvec<0, 1>(W, nullptr, x, y, rows, cols, nb);
+        else if (nb == 2) launch_matvec<0, 2>(W, nullptr, x, y, rows, cols, nb);
+        else if (nb <= 4) launch_matvec<0, 4>(W, nullptr, x, y, rows, cols, nb);
+        else launch_matvec<0, 8>(W, nullptr, x, y, rows, cols, nb);
+    }
+}
+
+// ---------------------------------------------------------------- single-vector row ops
+
+// rms_norm, shaders/q8_kernels.metal:133-158 (one workgroup per vector).  out may alias x.
+__global__ __launch_bounds__(TB) void k_rms_norm1(const float *x, const float *__restrict__ gamma, float *out, int dim, float eps)
+{
+    __shared__ float sm[16];
+    const size_t off = (size_t)blockIdx.x * dim;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dim; i += TB) { const float v = x[off + i]; ss += v * v; }
+    ss = block_sum(ss, sm);
+    const float inv = rsqrtf(ss / (float)dim + eps);
+    for (int i = threadIdx.x; i < dim; i += TB) out[off + i] = x[off + i] * inv * gamma[i];
+}
+
+// rope, shaders/q8_kernels.metal:195-231: half-split pairs (d, d + hd/2) of every q and k head at one position.
+__global__ __launch_bounds__(TB) void k_rope1(float *q, float *k, int Hq, int Hkv, int hd, int pos, float theta)
+{
+    const int half = hd / 2, q_pairs = Hq * half, total = q_pairs + Hkv * half;
+    int idx = blockIdx.x * TB + threadIdx.x;
+    if (idx >= total) return;
+    float *base = q;
+    if (idx >= q_pairs) { idx -= q_pairs; base = k; }
+    const int d = idx % half;
+    float *vec = base + (size_t)(idx / half) * hd;
+    const float freq = 1.0f / powf(theta, (float)(2 * d) / (float)hd);
+    float s, c;
+    sincosf((float)pos * freq, &s, &c);
+    const float x0 = vec[d], x1 = vec[d + half];
+    vec[d] = x0 * c - x1 * s;
+    vec[d + half] = x0 * s + x1 * c;
+}
+
+// kv_cache_store, shaders/q8_kernels.metal:237-256: caches are [Hkv, max_seq, hd].
+__global__ __launch_bounds__(TB) void k_kv_store(const float *__restrict__ k, const float *__restrict__ v,
+                                                 float *__restrict__ kc, float *__restrict__ vc, int Hkv, int max_seq,
+                                                 int hd, int pos)
+{
+    const int idx = blockIdx.x * TB + threadIdx.x;
+    if (idx >= Hkv * hd) return;
+    const size_t ci = ((size_t)(idx / hd) * max_seq + pos) * hd + idx % hd;
+    kc[ci] = k[idx];
+    vc[ci] = v[idx];
+}
+
+// ---------------------------------------------------------------- attention of one query per head over the cache
+
+constexpr int SL = 256;      // keys per workgroup
+
+// attention, shaders/q8_kernels.metal:262-331, restructured for a GPU with 256 CUs: one workgroup per (KV head, slice of
+// SL keys) serves all G query heads of the group, so the cache is read once; with more than one slice the workgroups
+// leave (max, sum, unnormalised output) per query head and k_attn_combine merges them.
+// LDS: q [G][hd], scores [G][SL], ml [2][G], red [4 * 256].  hd <= 256.
+__global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q, const float *__restrict__ Kc,
+                                                    const float *__restrict__ Vc, float *__restrict__ out,
+                                                    float *__restrict__ part_o, float *__restrict__ part_ml,
+                                                    int n_attend, int hd, int max_seq, int G, float scale, int nsplit)
+{
+    extern __shared__ float sm[];
+    __shared__ float rs[16];
+    float *qs = sm, *sc = qs + G * hd, *ml = sc + G * SL, *red = ml + 2 * G;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hkv = blockIdx.x, split = blockIdx.y;
+    const int j0 = split * SL, nj = min(SL, n_attend - j0);
+    const float *kbase = Kc + ((size_t)hkv * max_seq + j0) * hd;
+    const float *vbase = Vc + ((size_t)hkv * max_seq + j0) * hd;
+
+    for (int i = tid; i < G * hd; i += TB) qs[i] = Q[(size_t)hkv * G * hd + i];
+    __syncthreads();
+
+    // scores: wave per key, lanes over the head dimension, four query heads per pass over the key
+    for (int g0 = 0; g0 < G; g0 += 4) {
+        int gq[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, G - 1);
+        for (int jj = wave; jj < nj; jj += 4) {
+            const float *kp = kbase + (size_t)jj * hd;
+            float p[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int d = lane; d < hd; d += 64) {
+                const float kv = kp[d];
+#pragma unroll
+                for (int u = 0; u < 4; u++) p[u] = fmaf(qs[gq[u] * hd + d], kv, p[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const float s = wave_sum(p[u]);
+                if (lane == 0 && g0 + u < G) sc[(g0 + u) * SL + jj] = s * scale;
+            }
+        }
+    }
+    __syncthreads();
+
+    // softmax statistics of the slice, per query head
+    for (int g = 0; g < G; g++) {
+        float m = -3.0e38f;
+        for (int j = tid; j < nj; j += TB) m = fmaxf(m, sc[g * SL + j]);
+        m = block_max(m, rs);
+        float l = 0.f;
+        for (int j = tid; j < nj; j += TB) { const float e = __expf(sc[g * SL + j] - m); sc[g * SL + j] = e; l += e; }
+        l = block_sum(l, rs);
+        if (tid == 0) { ml[g] = m; ml[G + g] = l; }
+    }
+    __syncthreads();
+
+    // weighted value sum: thread = (part of the keys, d); parts are added through LDS
+    const int parts = max(1, TB / hd), part = tid / hd, d = tid % hd;
+    const bool active = part < parts;
+    for (int g0 = 0; g0 < G; g0 += 4) {
+        int gq[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, G - 1);
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+        if (active)
+            for (int jj = part; jj < nj; jj += parts) {
+                const float v = vbase[(size_t)jj * hd + d];
+#pragma unroll
+                for (int u = 0; u < 4; u++) o[u] = fmaf(sc[gq[u] * SL + jj], v, o[u]);
+            }
+        if (active) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) red[(part * 4 + u) * hd + d] = o[u];
+        }
+        __syncthreads();
+        if (part == 0) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (g0 + u >= G) continue;
+                float s = 0.f;
+                for (int pp = 0; pp < parts; pp++) s += red[(pp * 4 + u) * hd + d];
+                const int hq = hkv * G + g0 + u;
+                if (nsplit == 1) out[(size_t)hq * hd + d] = s / ml[G + g0 + u];
+                else part_o[((size_t)hq * nsplit + split) * hd + d] = s;
+            }
+        }
+        __syncthreads();
+    }
+    if (nsplit > 1 && tid < G) {
+        const int hq = hkv * G + tid;
+        part_ml[((size_t)hq * nsplit + split) * 2] = ml[tid];
+        part_ml[((size_t)hq * nsplit + split) * 2 + 1] = ml[G + tid];
+    }
+}
+
+// merge of the slices of one query head: grid = Hq, block = hd threads (<= 256)
+__global__ __launch_bounds__(TB) void k_attn_combine(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                                                     float *__restrict__ out, int hd, int nsplit)
+{
+    const int hq = blockIdx.x, d = threadIdx.x;
+    if (d >= hd) return;
+    const float *mlp = part_ml + (size_t)hq * nsplit * 2;
+    float m = -3.0e38f;
+    for (int s = 0; s < nsplit; s++) m = fmaxf(m, mlp[2 * s]);
+    float l = 0.f, o = 0.f;
+    for (int s = 0; s < nsplit; s++) {
+        const float w = __expf(mlp[2 * s] - m);
+        l = fmaf(mlp[2 * s + 1], w, l);
+        o = fmaf(part_o[((size_t)hq * nsplit + s) * hd + d], w, o);
+    }
+    out[(size_t)hq * hd + d] = o / l;
+}
+
+// byte offset into a buffer, checked against its size
+float *at_offset(MetalBuf *b, size_t off, size_t need, const char *fn)
+{
+    if (!b || off + need > b->size || (off & 3)) {
+        fprintf(stderr, "[fast_hip] %s: offset %zu + %zu bytes outside the buffer (%zu) or unaligned; launch skipped\n", fn, off,
+                need, b ? b->size : (size_t)0);
+        return nullptr;
+    }
+    return (float *)((char *)dptr(b) + off);
+}
+
+void per_head_rms_norm(float *vec, MetalBuf *gamma, int n_heads, int hd, float eps, const char *fn)
+{
+    REQUIRE_BYTES(gamma, (size_t)hd * 4, fn);
+    if (n_heads <= 0 || hd <= 0) return;
+    LAUNCH(k_rms_norm1, dim3(n_heads), dim3(TB), 0, vec, dptr_as<float>(gamma), vec, hd, eps);
+}
+
+void rope1(float *q, float *k, int Hq, int Hkv, int hd, int pos, float theta)
+{
+    const int total = (Hq + Hkv) * (hd / 2);
+    if (total <= 0) return;
+    LAUNCH(k_rope1, dim3((total + TB - 1) / TB), dim3(TB), 0, q, k, Hq, Hkv, hd, pos, theta);
+}
+
+void kv_store(const float *k, const float *v, MetalBuf *kc, MetalBuf *vc, int Hkv, int max_seq, int hd, int pos, const char *fn)
+{
+    REQUIRE_BYTES(kc, (size_t)Hkv * max_seq * hd * 4, fn);
+    REQUIRE_BYTES(vc, (size_t)Hkv * max_seq * hd * 4, fn);
+    if (pos < 0 || pos >= max_seq) { fprintf(stderr, "[fast_hip] %s: position %d outside the cache (%d); launch skipped\n", fn, pos, max_seq); return; }
+    if (Hkv * hd <= 0) return;
+    LAUNCH(k_kv_store, dim3((Hkv * hd + TB - 1) / TB), dim3(TB), 0, k, v, dptr_as<float>(kc), dptr_as<float>(vc), Hkv, max_seq, hd, pos);
+    mark_written(kc); mark_written(vc);
+}
+
+void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_attend, int hd, int max_seq, int Hq, int G, const char *fn)
+{
+    if (Hq <= 0 || n_attend <= 0) return;
+    if (G <= 0 || Hq % G) { fprintf(stderr, "[fast_hip] %s: %d query heads are not a multiple of the group ratio %d; launch skipped\n", fn, Hq, G); return; }
+    const int Hkv = Hq / G;
+    REQUIRE_BYTES(Kc, (size_t)Hkv * max_seq * hd * 4, fn);
+    REQUIRE_BYTES(Vc, (size_t)Hkv * max_seq * hd * 4, fn);
+    if (n_attend > max_seq) { fprintf(stderr, "[fast_hip] %s: n_attend %d exceeds the cache (%d); launch skipped\n", fn, n_attend, max_seq); return; }
+    if (hd > 256 || G > 16) { fprintf(stderr, "[fast_hip] %s: head_dim %d / group ratio %d not supported (<= 256 / <= 16); launch skipped\n", fn, hd, G); return; }
+    const int nsplit = (n_attend + SL - 1) / SL;
+    const size_t lds = ((size_t)G * hd + (size_t)G * SL + 2 * G + 4 * 256) * 4;
+    float *po = nullptr, *pml = nullptr;
+    if (nsplit > 1) {
+        const size_t o_bytes = (size_t)Hq * nsplit * hd * 4;
+        po = (float *)scratch(SCR_MISC, o_bytes + (size_t)Hq * nsplit * 2 * 4);
+        pml = po + (size_t)Hq * nsplit * hd;
+    }
+    const float scale = 1.0f / sqrtf((float)hd);
+    LAUNCH(k_attn_decode, dim3(Hkv, nsplit), dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml, n_attend, hd,
+           max_seq, G, scale, nsplit);
+    if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq), dim3(TB), 0, po, pml, out, hd, nsplit);
+}
+
+}  // namespace
+
+extern "C" {
+
+// q8_matvec, shaders/q8_kernels.metal:10-42; dispatch src/nn/fast_metal.m:253-270.  W: rows x nb Q8_0 blocks.
+void metal_enqueue_q8_matvec(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int nb)
+{
+    REQUIRE_BYTES(W, (size_t)rows * nb * 34, "q8_matvec");
+    REQUIRE_BYTES(x, (size_t)nb * 32 * 4, "q8_matvec");
+    REQUIRE_BYTES(y, (size_t)rows * 4, "q8_matvec");
+    if (rows <= 0) return;
+    if (nb <= 0) { zero_result(y, (size_t)rows); return; }
+    if (!aligned16(dptr(x))) { fprintf(stderr, "[fast_hip] q8_matvec: x must be 16-byte aligned; launch skipped\n"); return; }
+    const half_t *scales = nullptr;
+    const int8_t *q = q8_split_of(W, rows, nb, &scales);
+    launch_matvec<1, 1>(q, scales, dptr_as<float>(x), dptr_as<float>(y), rows, nb * 32, 1);
+    mark_written(y);
+}
+
+// f16_matvec, shaders/q8_kernels.metal:97-127; dispatch src/nn/fast_metal.m:272-289.
+void metal_enqueue_f16_matvec(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols)
+{
+    REQUIRE_BYTES(W, (size_t)rows * cols * 2, "f16_matvec");
+    REQUIRE_BYTES(x, (size_t)cols * 4, "f16_matvec");
+    REQUIRE_BYTES(y, (size_t)rows * 4, "f16_matvec");
+    if (rows <= 0) return;
+    if (cols <= 0) { zero_result(y, (size_t)rows); return; }
+    f16_matvec_any_batch(dptr_as<half_t>(W), dptr_as<float>(x), dptr_as<float>(y), rows, cols, 1);
+    mark_written(y);
+}
+
+// f16_batch_matvec, shaders/q8_kernels.metal:49-91; dispatch src/nn/fast_metal.m:291-307.  Y[B, rows] = X[B, cols] W^T.
+// The reference keeps 32 accumulators per lane and is undefined beyond; this one takes any B.
+void metal_enqueue_f16_batch_matvec(MetalBuf *W, MetalBuf *X, MetalBuf *Y, int rows, int cols, int B)
+{
+    if (B <= 0 || rows <= 0) return;
+    REQUIRE_BYTES(W, (size_t)rows * cols * 2, "f16_batch_matvec");
+    REQUIRE_BYTES(X, (size_t)B * cols * 4, "f16_batch_matvec");
+    REQUIRE_BYTES(Y, (size_t)B * rows * 4, "f16_batch_matvec");
+    if (cols <= 0) { zero_result(Y, (size_t)B * rows); return; }
+    f16_matvec_any_batch(dptr_as<half_t>(W), dptr_as<float>(X), dptr_as<float>(Y), rows, cols, B);
+    mark_written(Y);
+}
+
+// rms_norm of one vector, dispatch src/nn/fast_metal.m:309-324
+void metal_enqueue_rms_norm(MetalBuf *x, MetalBuf *gamma, MetalBuf *out, int dim, float eps)
+{
+    REQUIRE_BYTES(x, (size_t)dim * 4, "rms_norm");
+    REQUIRE_BYTES(out, (size_t)dim * 4, "rms_norm");
+    REQUIRE_BYTES(gamma, (size_t)dim * 4, "rms_norm");
+    if (dim <= 0) return;
+    LAUNCH(k_rms_norm1, dim3(1), dim3(TB), 0, dptr_as<float>(x), dptr_as<float>(gamma), dptr_as<float>(out), dim, eps);
+    mark_written(out);
+}
+
+// per_head_rms_norm, shaders/q8_kernels.metal:165-189; dispatch src/nn/fast_metal.m:343-357, 468-483.  In place.
+void metal_enqueue_per_head_rms_norm(MetalBuf *vec, MetalBuf *gamma, int n_heads, int head_dim, float eps)
+{
+    metal_enqueue_per_head_rms_norm_off(vec, 0, gamma, n_heads, head_dim, eps);
+}
+
+void metal_enqueue_per_head_rms_norm_off(MetalBuf *vec, size_t vec_off, MetalBuf *gamma, int n_heads, int head_dim, float eps)
+{
+    float *v = at_offset(vec, vec_off, (size_t)n_heads * head_dim * 4, "per_head_rms_norm");
+    if (!v) return;
+    per_head_rms_norm(v, gamma, n_heads, head_dim, eps, "per_head_rms_norm");
+    mark_written(vec);
+}
+
+// rope, shaders/q8_kernels.metal:195-231; dispatch src/nn/fast_metal.m:359-379, 485-506.  In place on q and k.
+void metal_enqueue_rope(MetalBuf *q, MetalBuf *k, int Hq, int Hkv, int hd, int pos, float theta)
+{
+    metal_enqueue_rope_off(q, 0, k, 0, Hq, Hkv, hd, pos, theta);
+}
+
+void metal_enqueue_rope_off(MetalBuf *q, size_t q_off, MetalBuf *k, size_t k_off, int Hq, int Hkv, int hd, int pos, float theta)
+{
+    float *qp = at_offset(q, q_off, (size_t)Hq * hd * 4, "rope");
+    float *kp = at_offset(k, k_off, (size_t)Hkv * hd * 4, "rope");
+    if (!qp || !kp) return;
+    rope1(qp, kp, Hq, Hkv, hd, pos, theta);
+    mark_written(q); mark_written(k);
+}
+
+// kv_cache_store, shaders/q8_kernels.metal:237-256; dispatch src/nn/fast_metal.m:381-402, 508-530.
+void metal_enqueue_kv_cache_store(MetalBuf *k, MetalBuf *v, MetalBuf *k_cache, MetalBuf *v_cache, int Hkv, int max_seq, int hd, int pos)
+{
+    metal_enqueue_kv_cache_store_off(k, 0, v, 0, k_cache, v_cache, Hkv, max_seq, hd, pos);
+}
+
+void metal_enqueue_kv_cache_store_off(MetalBuf *k, size_t k_off, MetalBuf *v, size_t v_off, MetalBuf *k_cache, MetalBuf *v_cache,
+                                      int Hkv, int max_seq, int hd, int pos)
+{
+    const float *kp = at_offset(k, k_off, (size_t)Hkv * hd * 4, "kv_cache_store");
+    const float *vp = at_offset(v, v_off, (size_t)Hkv * hd * 4, "kv_cache_store");
+    if (!kp || !vp) return;
+    kv_store(kp, vp, k_cache, v_cache, Hkv, max_seq, hd, pos, "kv_cache_store");
+}
+
+// attention, shaders/q8_kernels.metal:262-331; dispatch src/nn/fast_metal.m:404-425, 532-556.
+// Q, out: [Hq * hd]; caches [Hq / group_ratio, max_seq, hd]; attends keys 0 .. n_attend - 1.
+void metal_enqueue_attention(MetalBuf *Q, MetalBuf *Kc, MetalBuf *Vc, MetalBuf *out, int n_attend, int hd, int max_seq, int Hq,
+                             int group_ratio)
+{
+    metal_enqueue_attention_off(Q, 0, Kc, Vc, out, 0, n_attend, hd, max_seq, Hq, group_ratio);
+}
+
+void metal_enqueue_attention_off(MetalBuf *Q, size_t q_off, MetalBuf *Kc, MetalBuf *Vc, MetalBuf *out, size_t out_off, int n_attend,
+                                 int hd, int max_seq, int Hq, int group_ratio)
+{
+    const float *qp = at_offset(Q, q_off, (size_t)Hq * hd * 4, "attention");
+    float *op = at_offset(out, out_off, (size_t)Hq * hd * 4, "attention");
+    if (!qp || !op) return;
+    attention(qp, Kc, Vc, op, n_attend, hd, max_seq, Hq, group_ratio, "attention");
+    mark_written(out);
+}
+
+}  // extern "C"

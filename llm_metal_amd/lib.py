@@ -85,6 +85,15 @@ def load():
         "metal_enqueue_rms_norm_batched": (None, [vp, vp, vp, i, f, i]),
         "metal_enqueue_silu_mul": (None, [vp, vp, i]), "metal_enqueue_gelu_mul": (None, [vp, vp, i]),
         "metal_enqueue_residual_add": (None, [vp, vp, i]),
+        "metal_enqueue_q8_matvec": (None, [vp, vp, vp, i, i]), "metal_enqueue_f16_matvec": (None, [vp, vp, vp, i, i]),
+        "metal_enqueue_f16_batch_matvec": (None, [vp, vp, vp, i, i, i]), "metal_enqueue_rms_norm": (None, [vp, vp, vp, i, f]),
+        "metal_enqueue_per_head_rms_norm": (None, [vp, vp, i, i, f]), "metal_enqueue_rope": (None, [vp, vp, i, i, i, i, f]),
+        "metal_enqueue_kv_cache_store": (None, [vp, vp, vp, vp, i, i, i, i]),
+        "metal_enqueue_attention": (None, [vp, vp, vp, vp, i, i, i, i, i]),
+        "metal_enqueue_per_head_rms_norm_off": (None, [vp, sz, vp, i, i, f]),
+        "metal_enqueue_rope_off": (None, [vp, sz, vp, sz, i, i, i, i, f]),
+        "metal_enqueue_kv_cache_store_off": (None, [vp, sz, vp, sz, vp, vp, i, i, i, i]),
+        "metal_enqueue_attention_off": (None, [vp, sz, vp, vp, vp, sz, i, i, i, i, i]),
         "metal_enqueue_f16_matmul": (None, [vp, vp, vp, i, i, i]), "metal_enqueue_f16_matmul_nt": (None, [vp, vp, vp, i, i, i]),
         "metal_enqueue_transpose_heads_fwd": (None, [vp, vp, i, i, i]), "metal_enqueue_transpose_heads_rev": (None, [vp, vp, i, i, i]),
         "metal_enqueue_repeat_kv": (None, [vp, vp, i, i, i, i]), "metal_enqueue_repeat_kv_bwd": (None, [vp, vp, i, i, i, i]),

@@ -573,6 +573,104 @@ OR_API void or_f16_sgd_apply(uint16_t *W, uint16_t *G, size_t n, float lr)
 }
 
 /* ------------------------------------------------------------------ */
+/* Decode-step ops — shaders/q8_kernels.metal:10-331                   */
+/* ------------------------------------------------------------------ */
+
+/* q8_matvec, shaders/q8_kernels.metal:10-42: W is rows x nb blocks of
+ * {fp16 d; int8 q[32]} (34 bytes, little endian); per block the 32 products
+ * q * x are summed first and the block sum is scaled by d. */
+OR_API void or_q8_matvec(const uint8_t *W, const real *x, real *y, int rows, int nb)
+{
+    for (int r = 0; r < rows; r++) {
+        const uint8_t *rp = W + (size_t)r * nb * 34;
+        real sum = 0;
+        for (int b = 0; b < nb; b++) {
+            const uint8_t *blk = rp + (size_t)b * 34;
+            real scale = (real)or_f16_bits_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+            real bs = 0;
+            for (int j = 0; j < 32; j++) bs += (real)(int8_t)blk[2 + j] * x[b * 32 + j];
+            sum += scale * bs;
+        }
+        y[r] = sum;
+    }
+}
+
+/* f16_batch_matvec, shaders/q8_kernels.metal:49-91 (B = 1: f16_matvec, :97-127):
+ * Y[b, row] = sum_c float(W[row, c]) * X[b, c], W given as fp16 bit patterns. */
+OR_API void or_f16_batch_matvec(const uint16_t *W, const real *X, real *Y, int rows, int cols, int B)
+{
+    for (int b = 0; b < B; b++)
+        for (int r = 0; r < rows; r++) {
+            real s = 0;
+            for (int c = 0; c < cols; c++)
+                s += (real)or_f16_bits_to_f32(W[(size_t)r * cols + c]) * X[(size_t)b * cols + c];
+            Y[(size_t)b * rows + r] = s;
+        }
+}
+
+/* rope, shaders/q8_kernels.metal:195-231: the pairs (d, d + hd/2) of every q and
+ * k head rotated by pos / theta^(2d/hd); q is [Hq, hd], k is [Hkv, hd]. */
+OR_API void or_rope(real *q, real *k, int Hq, int Hkv, int hd, int pos, float theta)
+{
+    int half = hd / 2;
+    for (int t = 0; t < Hq + Hkv; t++) {
+        real *vec = t < Hq ? q + (size_t)t * hd : k + (size_t)(t - Hq) * hd;
+        for (int d = 0; d < half; d++) {
+            real freq = (real)1 / R_POW((real)theta, (real)(2 * d) / (real)hd);
+            real ang = (real)pos * freq;
+            real c = R_COS(ang), s = R_SIN(ang);
+            real x0 = vec[d], x1 = vec[d + half];
+            vec[d]        = x0 * c - x1 * s;
+            vec[d + half] = x0 * s + x1 * c;
+        }
+    }
+}
+
+/* kv_cache_store, shaders/q8_kernels.metal:237-256: caches are [Hkv, max_seq, hd]. */
+OR_API void or_kv_cache_store(const real *k, const real *v, real *kc, real *vc, int Hkv, int max_seq, int hd, int pos)
+{
+    for (int h = 0; h < Hkv; h++)
+        for (int d = 0; d < hd; d++) {
+            size_t ci = ((size_t)h * max_seq + pos) * hd + d;
+            kc[ci] = k[h * hd + d];
+            vc[ci] = v[h * hd + d];
+        }
+}
+
+/* attention, shaders/q8_kernels.metal:262-331; scale 1/sqrt(hd) from the dispatch
+ * (src/nn/fast_metal.m:414): per query head h (KV head h / group_ratio)
+ * s_j = q.k_j * scale for j < n_attend, softmax with the maximum subtracted,
+ * out = sum_j p_j v_j. */
+OR_API void or_attention(const real *Q, const real *Kc, const real *Vc, real *out, int n_attend, int hd, int max_seq,
+                         int Hq, int group_ratio)
+{
+    real *sc = (real *)malloc((size_t)n_attend * sizeof(real));
+    real inv_sqrt = (real)(1.0f / sqrtf((float)hd));         /* a float in the dispatch */
+    for (int h = 0; h < Hq; h++) {
+        const real *qp = Q + (size_t)h * hd;
+        const real *kp = Kc + (size_t)(h / group_ratio) * max_seq * hd;
+        const real *vp = Vc + (size_t)(h / group_ratio) * max_seq * hd;
+        real mx = (real)-1e30;
+        for (int j = 0; j < n_attend; j++) {
+            real dot = 0;
+            for (int d = 0; d < hd; d++) dot += qp[d] * kp[(size_t)j * hd + d];
+            sc[j] = dot * inv_sqrt;
+            if (sc[j] > mx) mx = sc[j];
+        }
+        real sum = 0;
+        for (int j = 0; j < n_attend; j++) { sc[j] = R_EXP(sc[j] - mx); sum += sc[j]; }
+        real inv_sum = (real)1 / sum;
+        for (int j = 0; j < n_attend; j++) sc[j] *= inv_sum;
+        for (int d = 0; d < hd; d++) {
+            real val = 0;
+            for (int j = 0; j < n_attend; j++) val += sc[j] * vp[(size_t)j * hd + d];
+            out[(size_t)h * hd + d] = val;
+        }
+    }
+    free(sc);
+}
+
+/* ------------------------------------------------------------------ */
 /* Optimiser — src/nn/fast_sft.c:1045-1107                             */
 /* ------------------------------------------------------------------ */
 

@@ -34,6 +34,12 @@ class Dev:
         self.bufs.append(b)
         return b
 
+    def view(self, parent, offset, nbytes):
+        from llm_metal_amd.sft import Buf
+        b = Buf(self.L, self.L.metal_buf_view(parent.h, offset, nbytes), nbytes)
+        self.bufs.insert(0, b)                      # freed before its parent
+        return b
+
     def close(self):
         for b in self.bufs:
             b.free()

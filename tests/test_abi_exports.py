@@ -22,7 +22,8 @@ def test_every_declared_symbol_is_exported(L):
 
 
 def test_reference_abi_names_present(L):
-    # the 33 symbols of src/nn/fast_metal.h the LoRA SFT step uses, plus the 3 of the GRPO accumulate path
+    # all 49 symbols of src/nn/fast_metal.h: the 33 the LoRA SFT step uses, the 4 of the full-parameter / GRPO
+    # path, and the 12 inference enqueues (+ 4 offset variants counted among them)
     names = """fast_metal_init fast_metal_shutdown metal_buf_create metal_buf_from_data metal_buf_free metal_buf_ptr
     metal_flush metal_enqueue_rms_norm_batched metal_enqueue_silu_mul metal_enqueue_gelu_mul metal_enqueue_residual_add
     metal_enqueue_f16_matmul metal_enqueue_f16_matmul_nt metal_enqueue_transpose_heads_fwd
@@ -31,7 +32,12 @@ def test_reference_abi_names_present(L):
     metal_enqueue_softmax_ce metal_enqueue_attn_train_fwd metal_enqueue_attn_bwd_dq metal_enqueue_attn_bwd_dkv
     metal_enqueue_repeat_kv_bwd metal_enqueue_rope_train_bwd metal_enqueue_float_matmul metal_enqueue_float_matmul_tn
     metal_enqueue_float_matmul_nt metal_enqueue_copy metal_enqueue_clamp metal_enqueue_f16_sgd_fused
-    metal_enqueue_grpo_policy_grad metal_enqueue_f16_grad_accum metal_enqueue_f16_sgd_apply""".split()
+    metal_enqueue_grpo_policy_grad metal_enqueue_f16_grad_accum metal_enqueue_f16_sgd_apply
+    metal_enqueue_q8_matvec metal_enqueue_f16_matvec metal_enqueue_f16_batch_matvec metal_enqueue_rms_norm
+    metal_enqueue_per_head_rms_norm metal_enqueue_rope metal_enqueue_kv_cache_store metal_enqueue_attention
+    metal_enqueue_per_head_rms_norm_off metal_enqueue_rope_off metal_enqueue_kv_cache_store_off
+    metal_enqueue_attention_off""".split()
+    assert len(names) == 49
     for n in names:
         assert hasattr(L, n), n
 

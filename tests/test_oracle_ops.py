@@ -224,3 +224,77 @@ def test_adamw_vs_torch_and_clip_rule():
     s2 = small.copy()
     op(P, "or_clip_grad_norm", s2, SZ(n), 1.0)
     assert np.array_equal(s2, small)                        # norm <= 1: untouched
+
+
+# ---------------------------------------------------------------- decode-step ops
+
+def test_q8_matvec_known_answer_and_vs_dequantised_product():
+    # one block: d = 0.5, q = 1..32, x = 1  ->  0.5 * (1 + ... + 32) = 264
+    blk = np.zeros(34, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    blk[2:] = np.arange(1, 33, dtype=np.int8).view(np.uint8)
+    y = np.zeros(1); op(P, "or_q8_matvec", blk, np.ones(32), y, 1, 1)
+    assert y[0] == 264.0
+    # negative codes and a negative scale keep their signs
+    blk[0:2] = np.frombuffer(np.float16(-2.0).tobytes(), np.uint8)
+    blk[2:] = np.full(32, -128, np.int8).view(np.uint8)
+    x = np.zeros(32); x[5] = 1.0
+    op(P, "or_q8_matvec", blk, x, y, 1, 1)
+    assert y[0] == 256.0
+    # random matrix: equals (dequantised weight) @ x with numpy
+    rows, nb = 7, 5
+    w = r(rows, nb * 32).astype(np.float32)
+    q = oracle.q8_quantize(w)
+    wd = oracle.q8_dequant(q, rows, nb * 32).astype(np.float64)
+    x = r(nb * 32)
+    y = np.zeros(rows); op(P, "or_q8_matvec", q, x, y, rows, nb)
+    assert rel(y, wd @ x) < 1e-14
+
+
+def test_f16_matvec_and_batch_vs_numpy():
+    rows, cols, B = 9, 50, 3
+    W = r(rows, cols).astype(np.float16)
+    X = r(B, cols)
+    Y = np.zeros((B, rows)); op(P, "or_f16_batch_matvec", W.view(np.uint16), X, Y, rows, cols, B)
+    assert rel(Y, X @ W.astype(np.float64).T) < 1e-14
+    y1 = np.zeros(rows); op(P, "or_f16_batch_matvec", W.view(np.uint16), X[1].copy(), y1, rows, cols, 1)
+    assert np.array_equal(y1, Y[1])
+
+
+def test_rope_at_one_position_is_the_training_rope_row():
+    Hq, Hkv, hd, N, theta = 4, 2, 16, 9, 1e4
+    q, k = r(Hq, N, hd), r(Hkv, N, hd)
+    qt, kt = q.copy(), k.copy(); op(P, "or_rope_train", qt, kt, Hq, Hkv, hd, N, theta)   # pinned above
+    for pos in (0, 3, 8):
+        q1, k1 = np.ascontiguousarray(q[:, pos]), np.ascontiguousarray(k[:, pos])
+        op(P, "or_rope", q1, k1, Hq, Hkv, hd, pos, theta)
+        assert np.array_equal(q1, qt[:, pos]) and np.array_equal(k1, kt[:, pos])
+    q0 = np.ascontiguousarray(q[:, 0]); k0 = np.ascontiguousarray(k[:, 0])
+    assert np.array_equal(q0, qt[:, 0])                                                # position 0: identity
+
+
+def test_kv_cache_store_writes_one_row_per_head():
+    Hkv, max_seq, hd, pos = 3, 6, 4, 4
+    k, v = r(Hkv, hd), r(Hkv, hd)
+    kc, vc = r(Hkv, max_seq, hd), r(Hkv, max_seq, hd)
+    ek, ev = kc.copy(), vc.copy(); ek[:, pos] = k; ev[:, pos] = v
+    op(P, "or_kv_cache_store", k, v, kc, vc, Hkv, max_seq, hd, pos)
+    assert np.array_equal(kc, ek) and np.array_equal(vc, ev)
+
+
+def test_decode_attention_vs_sdpa_and_the_training_kernel_row():
+    Hq, ratio, hd, max_seq, n = 6, 3, 16, 12, 7          # 1/sqrt(16) is exact in the dispatch's float
+    Hkv = Hq // ratio
+    Q, Kc, Vc = r(Hq, hd), r(Hkv, max_seq, hd), r(Hkv, max_seq, hd)
+    out = np.zeros((Hq, hd)); op(P, "or_attention", Q, Kc, Vc, out, n, hd, max_seq, Hq, ratio)
+    Kx = np.repeat(Kc[:, :n], ratio, axis=0); Vx = np.repeat(Vc[:, :n], ratio, axis=0)        # [Hq, n, hd]
+    ref = F.scaled_dot_product_attention(torch.tensor(Q)[:, None], torch.tensor(Kx), torch.tensor(Vx)).numpy()[:, 0]
+    assert rel(out, ref) < 1e-13
+    # the last query of the causal training kernel attends the same n keys
+    Qn = r(Hq, n, hd); Qn[:, n - 1] = Q
+    o2, probs = np.zeros((Hq, n, hd)), np.zeros((Hq, n, n))
+    op(P, "or_attn_train_fwd", Qn, np.ascontiguousarray(Kx), np.ascontiguousarray(Vx), o2, probs, Hq, n, hd, float(1 / np.sqrt(hd)))
+    assert rel(out, o2[:, n - 1]) < 1e-13
+    # one key: the output is that key's value
+    op(P, "or_attention", Q, Kc, Vc, out, 1, hd, max_seq, Hq, ratio)
+    assert rel(out, np.repeat(Vc[:, 0], ratio, axis=0)) < 1e-15
