@@ -166,6 +166,10 @@ int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double
  * 2 Q8_0 with column scales (transposed image).  Returns average ms per launch. */
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S);
 
+/* The same for the matrix-vector kernels of the decode step: rows x cols weight, fmt 0 F16 or 1 Q8_0 (split image),
+ * B = 1; cols a multiple of 32.  Returns average ms per launch, -1 for bad arguments. */
+double hip_matvec_time_shape(int rows, int cols, int fmt, int B, int iters);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,9 @@ void launch_tile_q8(const uint8_t *blocks, int rows, int cols, uint8_t *q_tiles,
 // out (tiled [M, K]) = fp16(X[m][k] * s_m), zero in the K padding; inv_scale[m] = 1/s_m
 void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_scale, int M, int K);
 // C[m][n] = row_scale[m] * sum_s P[s][m][n] (row_scale may be null)
+// C[M, N] fp32 = A[M, K] fp32 * W^T on the matrix cores with A kept to 22 bits: every row goes in twice, as its fp16
+// image and as the fp16 image of the rounding residual.  W: row-major F16 [N, K] buffer (its tiled image is cached).
+void gemm_f32a_exact(const float *A, struct ::MetalBuf *W, float *C, int M, int N, int K);
 void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, const float *row_scale, float *C, int M, int N);
 // dst (tiled, Kb_dst K blocks) <- src row-major F16 [rows, cols]:
 //   element (r, c) goes to tiled(row_off + r, k_off + c), or tiled(row_off + c, k_off + r) when transposed

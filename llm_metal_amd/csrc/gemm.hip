@@ -46,6 +46,49 @@ __global__ __launch_bounds__(256) void rows_to_f16_scaled(
     if (threadIdx.x == 0) inv_scale[row] = 1.0f / s;
 }
 
+// The same, keeping 22 bits of every element: row m of the tiled operand holds the fp16 image of x, row M + m the
+// fp16 image of what that rounding lost (x - fp16(x s) / s is exact in fp32), each with its own power-of-two scale.
+__global__ __launch_bounds__(256) void rows_to_f16_split(
+    const float *__restrict__ X, int ldx, half_t *__restrict__ out, float *__restrict__ inv_scale, int M, int K, int Kb)
+{
+    __shared__ float sm[16];
+    const int row = blockIdx.x;
+    const float *x = X + (size_t)row * ldx;
+    float amax = 0.f;
+    for (int i = threadIdx.x; i < K; i += blockDim.x) amax = fmaxf(amax, fabsf(x[i]));
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax), inv = 1.0f / s;
+    float lmax = 0.f;
+    for (int i = threadIdx.x; i < Kb * 64; i += blockDim.x) {
+        const half_t h = (i < K) ? f2h(x[i] * s) : (half_t)0;
+        out[lmhip::tiled_index(row, i, Kb)] = h;
+        if (i < K) lmax = fmaxf(lmax, fabsf(x[i] - h2f(h) * inv));
+    }
+    lmax = block_max(lmax, sm);
+    const float s2 = row_scale_for(lmax);
+    for (int i = threadIdx.x; i < Kb * 64; i += blockDim.x) {
+        half_t l = (half_t)0;
+        if (i < K) { const half_t h = f2h(x[i] * s); l = f2h((x[i] - h2f(h) * inv) * s2); }
+        out[lmhip::tiled_index(M + row, i, Kb)] = l;
+    }
+    if (threadIdx.x == 0) { inv_scale[row] = inv; inv_scale[M + row] = 1.0f / s2; }
+}
+
+// C[m, n] = sum over planes of row m and of row M + m, each times its row factor
+__global__ void reduce_planes_split(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
+                                    const float *__restrict__ row_scale, float *__restrict__ C, int M, int N)
+{
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)M * N) return;
+    const int m = (int)(idx / N), n = (int)(idx % N);
+    float hi = 0.f, lo = 0.f;
+    for (int p = 0; p < S; p++) {
+        hi += P[p * plane_stride + (size_t)m * ldp + n];
+        lo += P[p * plane_stride + (size_t)(M + m) * ldp + n];
+    }
+    C[idx] = fmaf(lo, row_scale[M + m], hi * row_scale[m]);
+}
+
 __global__ void reduce_planes(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
                               const float *__restrict__ row_scale, float *__restrict__ C, int M, int N)
 {
@@ -348,6 +391,27 @@ void gemm_f32a(const float *A, const half_t *Wt, float *C, int M, int Nout, int 
 }
 
 }  // namespace
+
+namespace lmhip {
+
+// C[M, N] fp32 = A[M, K] fp32 * W^T, W an F16 [N, K] weight buffer, with A split into value and residual rows
+void gemm_f32a_exact(const float *A, MetalBuf *W, float *C, int M, int N, int K)
+{
+    const half_t *Wt = tiled_copy_of(W, N, K, 0);
+    const int M2 = 2 * M;
+    half_t *a16 = (half_t *)scratch(SCR_A16, tiled_elems(M2, K) * sizeof(half_t));
+    float *inv = (float *)scratch(SCR_SCALE, (size_t)M2 * sizeof(float));
+    hipLaunchKernelGGL(rows_to_f16_split, dim3(M), dim3(256), 0, stream(), A, K, a16, inv, M, K, tiled_kb(K));
+    GemmPlan p = plan_gemm(M2, N, K);
+    const size_t plane = (size_t)M2 * N;
+    float *P = (float *)scratch(SCR_PARTIAL, plane * p.S * sizeof(float));
+    launch_gemm(a16, nullptr, Wt, P, N, plane, M2, N, K, p);
+    const size_t n = (size_t)M * N;
+    hipLaunchKernelGGL(reduce_planes_split, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(), P, p.S, plane, N, inv, C, M, N);
+    HIP_CHECK(hipGetLastError());
+}
+
+}  // namespace lmhip
 
 extern "C" {
 

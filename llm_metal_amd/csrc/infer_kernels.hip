@@ -10,6 +10,7 @@
 // with the buffer until something writes it, and the product streams that image.
 #include "backend.h"
 #include "devutil.h"
+#include "gemm.h"
 
 using namespace lmhip;
 
@@ -82,107 +83,106 @@ const int8_t *q8_split_of(MetalBuf *W, int rows, int nb, const half_t **scales)
 
 // ---------------------------------------------------------------- matrix-vector products
 
-// Y[b, row] = sum_c W[row, c] X[b, c] for b < B <= NBT.  FMT 0: W F16 row-major.  FMT 1: W int8 codes row-major with
-// one fp16 scale per 32 columns.  Requires cols % 8 == 0 and 16-byte aligned W and X.
+// y[row] = sum_c W[row, c] x[c].  FMT 0: W F16 row-major.  FMT 1: W int8 codes row-major with one fp16 scale per
+// 32 columns.  Requires cols % 8 == 0 and 16-byte aligned W and x.
 // Workgroup = 4 waves; wave w owns rows (4 blockIdx.x + w) R .. + R - 1; a lane owns 8 consecutive columns of every
-// 512-column step and U steps are loaded before any is used.  The vectors are staged through LDS in chunks of kc
-// columns (kc % 512 == 0).  Q8_0: codes are biased to unsigned (q + 128, one v_cvt_f32_ubyte each) and the bias is
-// taken out with the lane's sum of x, once per step for all rows.
-template <int FMT, int R, int U, int NBT>
+// 512-column step.  The weights of U steps (all R rows) are one register stage; the next stage is loaded before the
+// current one is used, and the first before x is staged into LDS (XLDS; without it, for rows longer than the LDS
+// budget, every lane reads its x values from global memory with the weights).  Q8_0: codes are biased to unsigned
+// (q + 128, one v_cvt_f32_ubyte each) and the bias is taken out with the lane's sum of x, once per step for all rows.
+template <int FMT, int R, int U, int XLDS>
 __global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, const half_t *__restrict__ scales,
-                                               const float *__restrict__ X, float *__restrict__ Y, int rows, int cols,
-                                               int B, int kc)
+                                               const float *__restrict__ x, float *__restrict__ y, int rows, int cols)
 {
-    extern __shared__ float xs[];                               // [NBT][kc]
+    extern __shared__ float xs[];                               // [cols] when XLDS
+    struct Stage {
+        half8   w16[FMT == 0 ? R : 1][U];
+        uint2v  w8[FMT == 1 ? R : 1][U];
+        float   dsc[FMT == 1 ? R : 1][U];
+        float4v x0[XLDS ? 1 : U], x1[XLDS ? 1 : U];
+    };
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = (blockIdx.x * 4 + wave) * R;
     size_t roff[R];                                             // element offset of each row (clamped: extra rows are not stored)
 #pragma unroll
     for (int r = 0; r < R; r++) roff[r] = (size_t)min(row0 + r, rows - 1) * cols;
-    float acc[R][NBT];
+    float acc[R];
 #pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < NBT; b++) acc[r][b] = 0.f;
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
 
-    for (int c0 = 0; c0 < cols; c0 += kc) {
-        const int n = min(kc, cols - c0);                       // multiple of 8
-        __syncthreads();
-        for (int b = 0; b < NBT; b++) {
-            const float *xrow = X + (size_t)min(b, B - 1) * cols + c0;
-            for (int i = tid * 4; i < n; i += TB * 4)
-                *reinterpret_cast<float4v *>(&xs[b * kc + i]) = *reinterpret_cast<const float4v *>(&xrow[i]);
+    auto load = [&](Stage &g, int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int cu = min(c + 512 * u, cols - 8);          // clamped: loads stay unconditional
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const size_t e = roff[r] + cu;
+                if (FMT == 0) g.w16[r][u] = __builtin_nontemporal_load(reinterpret_cast<const half8 *>((const half_t *)Wp + e));
+                else {
+                    g.w8[r][u] = __builtin_nontemporal_load(reinterpret_cast<const uint2v *>((const int8_t *)Wp + e));
+                    g.dsc[r][u] = (float)scales[e >> 5];
+                }
+            }
+            if (!XLDS) {
+                g.x0[u] = *reinterpret_cast<const float4v *>(&x[cu]);
+                g.x1[u] = *reinterpret_cast<const float4v *>(&x[cu + 4]);
+            }
         }
-        __syncthreads();
-        for (int c = lane * 8; c < n; c += 512 * U) {
-            half8  w16[R][U];
-            uint2v w8[R][U];
-            float  dsc[R][U];
-            int    cu[U];
+    };
+    auto use = [&](const Stage &g, int c) __attribute__((always_inline)) {
 #pragma unroll
-            for (int u = 0; u < U; u++) cu[u] = min(c + 512 * u, n - 8);        // clamped: loads stay unconditional
+        for (int u = 0; u < U; u++) {
+            const int cu = min(c + 512 * u, cols - 8);
+            const float live = (c + 512 * u < cols) ? 1.f : 0.f;
+            float4v x0, x1;
+            if (XLDS) { x0 = *reinterpret_cast<const float4v *>(&xs[cu]); x1 = *reinterpret_cast<const float4v *>(&xs[cu + 4]); }
+            else { x0 = g.x0[u]; x1 = g.x1[u]; }
+            float xv[8];
 #pragma unroll
-            for (int u = 0; u < U; u++)
+            for (int e = 0; e < 4; e++) { xv[e] = x0[e] * live; xv[4 + e] = x1[e] * live; }
+            float xsum = 0.f;
+            if (FMT == 1) {
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    const size_t e = roff[r] + c0 + cu[u];
-                    if (FMT == 0) w16[r][u] = __builtin_nontemporal_load(reinterpret_cast<const half8 *>((const half_t *)Wp + e));
-                    else {
-                        w8[r][u] = __builtin_nontemporal_load(reinterpret_cast<const uint2v *>((const int8_t *)Wp + e));
-                        dsc[r][u] = (float)scales[e >> 5];
+                for (int e = 0; e < 8; e++) xsum += xv[e];
+                xsum *= 128.f;
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (FMT == 0) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[r] = fmaf((float)g.w16[r][u][e], xv[e], acc[r]);
+                } else {
+                    const uint32_t lo = g.w8[r][u][0] ^ 0x80808080u, hi = g.w8[r][u][1] ^ 0x80808080u;
+                    float p = -xsum;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        p = fmaf((float)((lo >> (8 * e)) & 255u), xv[e], p);
+                        p = fmaf((float)((hi >> (8 * e)) & 255u), xv[4 + e], p);
                     }
-                }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const float live = (c + 512 * u < n) ? 1.f : 0.f;
-                float xv[NBT][8], xsum[NBT];
-#pragma unroll
-                for (int b = 0; b < NBT; b++) {
-                    const float4v x0 = *reinterpret_cast<const float4v *>(&xs[b * kc + cu[u]]);
-                    const float4v x1 = *reinterpret_cast<const float4v *>(&xs[b * kc + cu[u] + 4]);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) { xv[b][e] = x0[e] * live; xv[b][4 + e] = x1[e] * live; }
-                    if (FMT == 1) {
-                        float s = 0.f;
-#pragma unroll
-                        for (int e = 0; e < 8; e++) s += xv[b][e];
-                        xsum[b] = 128.f * s;
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    if (FMT == 0) {
-#pragma unroll
-                        for (int b = 0; b < NBT; b++)
-#pragma unroll
-                            for (int e = 0; e < 8; e++) acc[r][b] = fmaf((float)w16[r][u][e], xv[b][e], acc[r][b]);
-                    } else {
-                        const uint32_t lo = w8[r][u][0] ^ 0x80808080u, hi = w8[r][u][1] ^ 0x80808080u;
-                        float uf[8];
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            uf[e] = (float)((lo >> (8 * e)) & 255u);
-                            uf[4 + e] = (float)((hi >> (8 * e)) & 255u);
-                        }
-#pragma unroll
-                        for (int b = 0; b < NBT; b++) {
-                            float p = -xsum[b];
-#pragma unroll
-                            for (int e = 0; e < 8; e++) p = fmaf(uf[e], xv[b][e], p);
-                            acc[r][b] = fmaf(dsc[r][u], p, acc[r][b]);
-                        }
-                    }
+                    acc[r] = fmaf(g.dsc[r][u], p, acc[r]);
                 }
             }
         }
+    };
+
+    Stage cur;
+    load(cur, lane * 8);
+    if (XLDS) {
+        for (int i = tid * 4; i < cols; i += TB * 4)
+            *reinterpret_cast<float4v *>(&xs[i]) = *reinterpret_cast<const float4v *>(&x[i]);
+        __syncthreads();
+    }
+    for (int c = lane * 8; c < cols; c += 512 * U) {
+        Stage nxt;
+        load(nxt, c + 512 * U);
+        use(cur, c);
+        cur = nxt;
     }
 #pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int b = 0; b < NBT; b++) {
-            const float s = wave_sum(acc[r][b]);
-            if (lane == 0 && row0 + r < rows && b < B) Y[(size_t)b * rows + row0 + r] = s;
-        }
+    for (int r = 0; r < R; r++) {
+        const float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < rows) y[row0 + r] = s;
+    }
 }
 
 // Any cols / alignment: one wave per row, lanes stride single elements.
@@ -201,40 +201,24 @@ __global__ __launch_bounds__(TB) void k_matvec_any(const half_t *__restrict__ W,
     }
 }
 
-template <int FMT, int NBT>
-void launch_matvec(const void *W, const half_t *scales, const float *X, float *Y, int rows, int cols, int B)
+// Rows per wave grow with the matrix so that mid-sized weights (a few thousand rows) still put 16 waves on every CU.
+template <int FMT>
+void launch_matvec(const void *W, const half_t *scales, const float *x, float *y, int rows, int cols)
 {
-    // LDS budget 48 KB per workgroup (three workgroups per CU stay resident)
-    int kc = (48 * 1024 / 4 / NBT) / 512 * 512;
-    kc = min(kc, (cols + 511) / 512 * 512);
-    const size_t lds = (size_t)NBT * kc * 4;
-    constexpr int U1 = NBT == 1 ? 4 : (NBT <= 4 ? 2 : 1);        // one row per wave: loads in flight come from column steps
-    constexpr int U4 = NBT == 1 ? 2 : 1;
-    if (rows >= 4096)
-        LAUNCH((k_matvec<FMT, 4, U4, NBT>), dim3((rows + 15) / 16), dim3(TB), lds, W, scales, X, Y, rows, cols, B, kc);
+    // x goes through LDS only where a workgroup covers 16 rows: with fewer, refilling it costs more than it saves
+    const size_t lds = (size_t)cols * 4;
+    if (rows >= 32768 && lds <= 40 * 1024)
+        LAUNCH((k_matvec<FMT, 4, 2, 1>), dim3((rows + 15) / 16), dim3(TB), lds, W, scales, x, y, rows, cols);
+    else if (rows >= 32768)
+        LAUNCH((k_matvec<FMT, 4, 2, 0>), dim3((rows + 15) / 16), dim3(TB), 0, W, scales, x, y, rows, cols);
+    else if (rows >= 8192)
+        LAUNCH((k_matvec<FMT, 2, 2, 0>), dim3((rows + 7) / 8), dim3(TB), 0, W, scales, x, y, rows, cols);
     else
-        LAUNCH((k_matvec<FMT, 1, U1, NBT>), dim3((rows + 3) / 4), dim3(TB), lds, W, scales, X, Y, rows, cols, B, kc);
+        LAUNCH((k_matvec<FMT, 1, 4, 0>), dim3((rows + 3) / 4), dim3(TB), 0, W, scales, x, y, rows, cols);
+#undef MATVEC_PICK
 }
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
-
-void f16_matvec_any_batch(const half_t *W, const float *X, float *Y, int rows, int cols, int B)
-{
-    if (cols % 8 || !aligned16(W) || !aligned16(X)) {
-        LAUNCH(k_matvec_any, dim3((rows + 3) / 4), dim3(TB), 0, W, X, Y, rows, cols, B);
-        return;
-    }
-    // batches beyond 8 vectors stream the weight once per group of 8 (the later passes mostly hit the caches)
-    for (int b0 = 0; b0 < B; b0 += 8) {
-        const int nb = min(8, B - b0);
-        const float *x = X + (size_t)b0 * cols;
-        float *y = Y + (size_t)b0 * rows;
-        if (nb == 1) launch_matvec<0, 1>(W, nullptr, x, y, rows, cols, nb);
-        else if (nb == 2) launch_matvec<0, 2>(W, nullptr, x, y, rows, cols, nb);
-        else if (nb <= 4) launch_matvec<0, 4>(W, nullptr, x, y, rows, cols, nb);
-        else launch_matvec<0, 8>(W, nullptr, x, y, rows, cols, nb);
-    }
-}
 
 // ---------------------------------------------------------------- single-vector row ops
 
@@ -469,7 +453,7 @@ void metal_enqueue_q8_matvec(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, in
     if (!aligned16(dptr(x))) { fprintf(stderr, "[fast_hip] q8_matvec: x must be 16-byte aligned; launch skipped\n"); return; }
     const half_t *scales = nullptr;
     const int8_t *q = q8_split_of(W, rows, nb, &scales);
-    launch_matvec<1, 1>(q, scales, dptr_as<float>(x), dptr_as<float>(y), rows, nb * 32, 1);
+    launch_matvec<1>(q, scales, dptr_as<float>(x), dptr_as<float>(y), rows, nb * 32);
     mark_written(y);
 }
 
@@ -481,12 +465,16 @@ void metal_enqueue_f16_matvec(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, i
     REQUIRE_BYTES(y, (size_t)rows * 4, "f16_matvec");
     if (rows <= 0) return;
     if (cols <= 0) { zero_result(y, (size_t)rows); return; }
-    f16_matvec_any_batch(dptr_as<half_t>(W), dptr_as<float>(x), dptr_as<float>(y), rows, cols, 1);
+    if (cols % 8 || !aligned16(dptr(W)) || !aligned16(dptr(x)))
+        LAUNCH(k_matvec_any, dim3((rows + 3) / 4), dim3(TB), 0, dptr_as<half_t>(W), dptr_as<float>(x), dptr_as<float>(y), rows, cols, 1);
+    else launch_matvec<0>(dptr(W), nullptr, dptr_as<float>(x), dptr_as<float>(y), rows, cols);
     mark_written(y);
 }
 
 // f16_batch_matvec, shaders/q8_kernels.metal:49-91; dispatch src/nn/fast_metal.m:291-307.  Y[B, rows] = X[B, cols] W^T.
-// The reference keeps 32 accumulators per lane and is undefined beyond; this one takes any B.
+// The reference keeps 32 accumulators per lane and is undefined beyond; this one takes any B.  From two vectors on the
+// product runs on the matrix cores over the tiled image of W, each fp32 vector split into two fp16 rows (value and
+// rounding residual, each with its own power-of-two scale), which keeps 22 bits of every x.
 void metal_enqueue_f16_batch_matvec(MetalBuf *W, MetalBuf *X, MetalBuf *Y, int rows, int cols, int B)
 {
     if (B <= 0 || rows <= 0) return;
@@ -494,7 +482,8 @@ void metal_enqueue_f16_batch_matvec(MetalBuf *W, MetalBuf *X, MetalBuf *Y, int r
     REQUIRE_BYTES(X, (size_t)B * cols * 4, "f16_batch_matvec");
     REQUIRE_BYTES(Y, (size_t)B * rows * 4, "f16_batch_matvec");
     if (cols <= 0) { zero_result(Y, (size_t)B * rows); return; }
-    f16_matvec_any_batch(dptr_as<half_t>(W), dptr_as<float>(X), dptr_as<float>(Y), rows, cols, B);
+    if (B == 1) { metal_enqueue_f16_matvec(W, X, Y, rows, cols); return; }
+    gemm_f32a_exact(dptr_as<float>(X), W, dptr_as<float>(Y), B, rows, cols);
     mark_written(Y);
 }
 
@@ -569,6 +558,40 @@ void metal_enqueue_attention_off(MetalBuf *Q, size_t q_off, MetalBuf *Kc, MetalB
     if (!qp || !op) return;
     attention(qp, Kc, Vc, op, n_attend, hd, max_seq, Hq, group_ratio, "attention");
     mark_written(out);
+}
+
+// Microbenchmark of the matrix-vector kernels alone: average ms per launch over `iters` launches that rotate through
+// more than 1 GB of distinct weights, so that no launch finds its weights in a cache.  fmt 0: F16 rows (B vectors,
+// fmt 1: the split Q8_0 image.  B must be 1 (batches run on the GEMM, see hip_gemm_time_shape).
+double hip_matvec_time_shape(int rows, int cols, int fmt, int B, int iters)
+{
+    if (rows <= 0 || cols <= 0 || cols % 32 || B != 1 || iters <= 0) return -1.0;
+    const size_t wb = ((fmt == 1 ? q8_scale_offset((size_t)rows * (cols / 32)) + (size_t)rows * (cols / 32) * 2
+                                 : (size_t)rows * cols * 2) + 255) & ~(size_t)255;
+    const int nbuf = (int)((size_t)1200 * 1024 * 1024 / wb) + 1;
+    void *W = nullptr, *X = nullptr, *Y = nullptr;
+    HIP_CHECK(hipMalloc(&W, wb * nbuf)); HIP_CHECK(hipMalloc(&X, (size_t)B * cols * 4)); HIP_CHECK(hipMalloc(&Y, (size_t)B * rows * 4));
+    HIP_CHECK(hipMemsetAsync(W, 0x11, wb * nbuf, stream()));
+    HIP_CHECK(hipMemsetAsync(X, 0, (size_t)B * cols * 4, stream()));
+    auto run = [&](int i) {
+        const char *w = (const char *)W + (size_t)(i % nbuf) * wb;
+        if (fmt == 1)
+            launch_matvec<1>(w, (const half_t *)(w + q8_scale_offset((size_t)rows * (cols / 32))), (const float *)X, (float *)Y,
+                             rows, cols);
+        else launch_matvec<0>(w, nullptr, (const float *)X, (float *)Y, rows, cols);
+    };
+    hipEvent_t e0, e1;
+    HIP_CHECK(hipEventCreate(&e0)); HIP_CHECK(hipEventCreate(&e1));
+    for (int i = 0; i < 3; i++) run(i);
+    HIP_CHECK(hipEventRecord(e0, stream()));
+    for (int i = 0; i < iters; i++) run(i + 3);
+    HIP_CHECK(hipEventRecord(e1, stream()));
+    HIP_CHECK(hipStreamSynchronize(stream()));
+    float ms = 0;
+    HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    hipEventDestroy(e0); hipEventDestroy(e1);
+    hipFree(W); hipFree(X); hipFree(Y);
+    return (double)ms / iters;
 }
 
 }  // extern "C"

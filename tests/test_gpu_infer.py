@@ -33,8 +33,10 @@ def rnd(rng, *shape, scale=1.0):
     return (rng.standard_normal(shape) * scale).astype(F)
 
 
-# rows >= 4096 takes the four-rows-per-wave kernel; cols % 8 != 0 the element-wise one
-@pytest.mark.parametrize("rows,cols", [(4096, 2560), (1024, 2560), (4100, 1152), (37, 9728), (7, 100), (33, 24), (5000, 8)])
+# rows per wave grow at 8192 and 32768 rows; from 32768 rows on x is staged in LDS unless longer than 10240; cols % 8 != 0 takes the
+# element-wise kernel
+@pytest.mark.parametrize("rows,cols", [(4096, 2560), (1024, 2560), (8200, 1152), (33000, 256), (37, 9728), (21, 12800),
+                                       (33000, 10248), (7, 100), (33, 24), (5000, 8)])
 def test_f16_matvec(dev, rows, cols):
     say("f16_matvec", rows, cols)
     rng = np.random.default_rng(rows + cols)
@@ -61,7 +63,7 @@ def test_f16_batch_matvec(dev, rows, cols, B):
     assert maxrel(yb.read(F, (B, rows)), ref) < 2e-5
 
 
-@pytest.mark.parametrize("rows,nb", [(4096, 80), (1000, 36), (5, 1), (4099, 17), (151, 304)])
+@pytest.mark.parametrize("rows,nb", [(4096, 80), (1000, 36), (5, 1), (8195, 17), (33001, 4), (151, 304), (70, 416)])
 def test_q8_matvec_and_its_cached_image(dev, rows, nb):
     say("q8_matvec", rows, nb)
     rng = np.random.default_rng(rows + nb)
