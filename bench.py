@@ -64,6 +64,79 @@ def cpu_baseline(cfg, budget_s=20.0):
                       f"({dt:.1f} s measured), scaled by the frozen-parameter ratio {scale:.1f}"}
 
 
+def decode_cpu_baseline(cfg):
+    """The CPU oracle's decode chain (scalar, 1 thread) for one token at position 16 on a model with fewer layers
+    and a truncated vocabulary, scaled to the full configuration by the frozen-parameter ratio."""
+    from oracle import oracle
+    from oracle.oracle import op
+    nl, v = min(cfg.NL, 8), min(cfg.V, 32768)
+    small = cfg.with_(name=cfg.name + "_sample", NL=nl, V=v, tied=False)
+    model = make_model(small, seed=0)
+    from llm_metal_amd.synth import MATS
+    mats = [model[k][L] for L in range(nl) for k in MATS] + [model["lm_head"]]
+    W = [np.ascontiguousarray(m.astype(np.float16)).view(np.uint16) for m in mats]
+    x = np.ones(max(small.D, small.IS, small.Hq * small.hd), np.float32)
+    y = np.zeros(max(small.V, small.IS), np.float32)
+    t0 = time.perf_counter()
+    for w in W:                                            # the products are all but a per-mille of a decode step's work
+        op("f32", "or_f16_batch_matvec", w, x, y, w.shape[0], w.shape[1], 1)
+    dt = time.perf_counter() - t0
+    scale = cfg.frozen_params / small.frozen_params
+    return {"value": 1.0 / (dt * scale), "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"oracle matrix-vector products of one token on {nl} of {cfg.NL} layers + {v} of {cfg.V} vocab rows "
+                      f"({dt:.2f} s measured), scaled by the frozen-parameter ratio {scale:.1f}"}
+
+
+def decode_bench(args, cfg, L):
+    """Greedy generation, one token per step; the matrix-vector kernel is the dominant kernel and every one of its
+    launches is timed with HIP events on the library's stream in a second pass."""
+    import ctypes as C
+    from llm_metal_amd.sft import InferenceState
+    f16 = cfg.weight_format == "f16"
+    t0 = time.perf_counter()
+    model = make_model(cfg, seed=0)
+    t_gen = time.perf_counter() - t0
+    max_seq = args.prompt_len + args.warmup + 2 * args.steps + 8
+    inf = InferenceState(cfg, model, max_seq=max_seq, use_fp16=f16)
+    t_init = time.perf_counter() - t0 - t_gen
+    del model
+    rng = np.random.default_rng(3)
+    tok = 1
+    for t in rng.integers(0, cfg.V, args.prompt_len):
+        tok = inf.forward_token_argmax(int(t))
+    for _ in range(args.warmup):
+        tok = inf.forward_token_argmax(tok)
+    L.metal_flush()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        tok = inf.forward_token_argmax(tok)
+    L.metal_flush()
+    dt = time.perf_counter() - t1
+    prof_steps = max(1, min(5, args.steps))
+    L.hip_gemm_profile_enable(1)
+    for _ in range(prof_steps):
+        tok = inf.forward_token_argmax(tok)
+    tms, wb, fl = C.c_double(0), C.c_double(0), C.c_double(0)
+    n = L.hip_gemm_profile_read2(C.byref(tms), C.byref(wb), C.byref(fl))
+    L.hip_gemm_profile_enable(0)
+    inf.free()
+    gbs = wb.value / (tms.value * 1e-3) / 1e9 if tms.value > 0 else 0.0
+    out = {"metric": "greedy decode tokens/s, batch 1", "value": round(args.steps / dt, 1), "unit": "tokens/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt / args.steps * 1e3, 3), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f16 weights x f32 activations, f32 accumulate" if f16 else
+           "q8_0 weights x f32 activations, f32 accumulate", "data": "synthetic",
+           "config": {"workload": cfg.name + "_decode", "layers": cfg.NL, "frozen_params": cfg.frozen_params,
+                      "weight_format": cfg.weight_format, "prompt_len": args.prompt_len},
+           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_matvec",
+                        "launches_per_step": n // prof_steps, "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
+                        "weight_bytes_per_step": wb.value / prof_steps, "matvec_ms_per_step": round(tms.value / prof_steps, 3)},
+           "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = decode_cpu_baseline(cfg)
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -71,6 +144,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c3_qwen3_4b_f16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--decode", action="store_true",
+                    help="time greedy token-by-token generation (include/inference_hip.h) on the configuration's model "
+                         "instead of the training step: a step is one token")
+    ap.add_argument("--prompt-len", type=int, default=16)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the library's plain copy kernel (1 GiB in, 1 GiB out, 5 launches): "
                          "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
@@ -99,6 +176,9 @@ def main():
         print(json.dumps({"copy_calibration": {"kernel": "k_copy", "bytes_read_per_launch": 4 * n,
                                                "bytes_written_per_launch": 4 * n, "launches": 5}}))
         return
+
+    if args.decode:
+        return decode_bench(args, cfg, L)
 
     t0 = time.perf_counter()
     model = make_model(cfg, seed=0, lora_b_std=0.0)          # timing runs: B = 0 as the reference initialises it

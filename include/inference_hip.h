@@ -1,0 +1,65 @@
+/*
+ * inference_hip.h — pipeline-level C ABI of the HIP backend for token-by-token generation: the replacement for the
+ * reference's src/nn/fast_inference.h.  One decode step is the sequence of src/nn/fast_inference.c:376-467 (embedding
+ * row, per layer RMSNorm -> Q/K/V products (+ LoRA on Q and V) -> per-head RMSNorm -> RoPE -> KV-cache store ->
+ * attention over the cache -> O product -> residual -> RMSNorm -> gated FFN -> residual, final RMSNorm, LM head),
+ * enqueued on the library's stream through the inference enqueues of fast_hip.h.  Weights are the reference's WMat
+ * containers (F16 rows or Q8_0 blocks).
+ *
+ * The reference takes its Qwen3Model / Gemma3Model structs; this library takes the same plain description of the
+ * model that the SFT state takes (SFTModelRef, sft_hip.h), which a caller fills from those structs as the
+ * reference's build_refs does (src/nn/fast_sft.c:171-225).
+ */
+#ifndef INFERENCE_HIP_H
+#define INFERENCE_HIP_H
+
+#include "sft_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct InferenceState InferenceState;
+
+/* inference_state_create / inference_state_create_gemma3 (src/nn/fast_inference.h:17-20; impl
+ * src/nn/fast_inference.c:262-316): converts and uploads every matrix (use_fp16 != 0: F16, else Q8_0), allocates the
+ * KV caches [n_kv_heads, max_seq_len, head_dim] per layer.  max_seq_len is not clamped to 4096 (the reference's
+ * attention kernel holds 4096 scores; this one has no such limit).  NULL when no GPU is present. */
+InferenceState *inference_state_create_from_ref(const SFTModelRef *model, int max_seq_len, int use_fp16);
+
+/* src/nn/fast_inference.h:49 (impl src/nn/fast_inference.c:527-610): shares the SFT state's weights (row-major F16
+ * copies handed out by sft_get_layers / sft_get_lm_head), embedding table, final norm and LoRA adapters; the SFT
+ * state must outlive it.  After a full-parameter update call inference_state_refresh_from_sft. */
+InferenceState *inference_state_create_from_sft(SFTState *sft, int max_seq_len);
+/* re-reads the weights of the SFT state this state was created from (no counterpart in the reference, whose shared
+ * buffers are the training weights themselves) */
+void inference_state_refresh_from_sft(InferenceState *state);
+
+void inference_state_free(InferenceState *state);                    /* src/nn/fast_inference.h:21 */
+
+/* src/nn/fast_inference.h:26-28 (impl :612-675): greedy decoding.  Prefills the prompt token by token, then emits
+ * argmax tokens until an EOS token has been emitted, max_gen_len tokens are out or the cache is full.  Returns the
+ * number of tokens written (the EOS token included, as in the reference). */
+int inference_generate(InferenceState *state, const uint32_t *prompt_tokens, int prompt_len,
+                       uint32_t *output_tokens, int max_gen_len);
+
+ModelType inference_state_model_type(InferenceState *state);         /* src/nn/fast_inference.h:31 */
+int  inference_state_vocab_size(InferenceState *state);              /* src/nn/fast_inference.h:34 */
+void inference_state_reset(InferenceState *state);                   /* src/nn/fast_inference.h:37: position := 0 */
+/* src/nn/fast_inference.h:41: one step at the current position, which it advances; returns the logits [vocab] in
+ * host memory, valid until the next call.  NULL when the cache is full. */
+const float *inference_forward_token(InferenceState *state, int token);
+/* the same without the copy of the logits to the host: returns their argmax (computed on the GPU) */
+int  inference_forward_token_argmax(InferenceState *state, int token);
+
+void inference_state_set_lora(InferenceState *state, SFTState *sft); /* src/nn/fast_inference.h:46 */
+/* src/nn/fast_inference.h:52 reads eos_token_id from <model_path>/generation_config.json or config.json; here the
+ * caller passes the ids (at most 4); the defaults are the reference's (Qwen3: 151645, 151643; Gemma3: 1, 106). */
+void inference_state_set_eos(InferenceState *state, const int *eos_tokens, int n_eos);
+void inference_state_load_eos(InferenceState *state, const char *model_path);
+int  inference_state_position(InferenceState *state);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFERENCE_HIP_H */

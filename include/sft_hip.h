@@ -121,6 +121,9 @@ const float *sft_get_rope_thetas(SFTState *state);
 int sft_is_full_param(SFTState *state);          /* 1 when the state was created with lora_rank 0 (sft_state_create_full) */
 const float *sft_get_token_emb(SFTState *state);  /* the caller's fp32 table, borrowed: it must outlive the state */
 MetalBuf *sft_get_final_norm_g(SFTState *state);
+/* the device copy of the embedding table, fp32 [vocab, d_model], unscaled (no counterpart in the reference, whose
+ * shared-memory table is the host pointer above); borrowed by inference_state_create_from_sft */
+MetalBuf *sft_get_token_emb_buf(SFTState *state);
 /* Weight sharing accessors (src/nn/fast_sft.h:98-101).  The state keeps its matrices in the GEMM's own
  * operand layout, so these hand out row-major F16 COPIES, refreshed on every call. */
 LayerW *sft_get_layers(SFTState *state);

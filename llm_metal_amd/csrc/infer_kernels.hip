@@ -11,6 +11,7 @@
 #include "backend.h"
 #include "devutil.h"
 #include "gemm.h"
+#include <hip/hip_ext.h>
 
 using namespace lmhip;
 
@@ -207,15 +208,19 @@ void launch_matvec(const void *W, const half_t *scales, const float *x, float *y
 {
     // x goes through LDS only where a workgroup covers 16 rows: with fewer, refilling it costs more than it saves
     const size_t lds = (size_t)cols * 4;
-    if (rows >= 32768 && lds <= 40 * 1024)
-        LAUNCH((k_matvec<FMT, 4, 2, 1>), dim3((rows + 15) / 16), dim3(TB), lds, W, scales, x, y, rows, cols);
-    else if (rows >= 32768)
-        LAUNCH((k_matvec<FMT, 4, 2, 0>), dim3((rows + 15) / 16), dim3(TB), 0, W, scales, x, y, rows, cols);
-    else if (rows >= 8192)
-        LAUNCH((k_matvec<FMT, 2, 2, 0>), dim3((rows + 7) / 8), dim3(TB), 0, W, scales, x, y, rows, cols);
-    else
-        LAUNCH((k_matvec<FMT, 1, 4, 0>), dim3((rows + 3) / 4), dim3(TB), 0, W, scales, x, y, rows, cols);
-#undef MATVEC_PICK
+    // with the GEMM profile enabled (hip_gemm_profile_enable) every launch is bracketed by events and counted there
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+    const bool prof = gemm_prof_begin((double)rows * cols * (FMT == 0 ? 2.0 : 34.0 / 32.0), 2.0 * rows * cols, &ev_a, &ev_b);
+#define MATVEC_LAUNCH(R_, U_, XL_, RPW_, L_) do { \
+    const dim3 grid((rows + RPW_ - 1) / RPW_); \
+    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, R_, U_, XL_>), grid, dim3(TB), L_, stream(), ev_a, ev_b, 0, W, scales, x, y, rows, cols); \
+    else hipLaunchKernelGGL((k_matvec<FMT, R_, U_, XL_>), grid, dim3(TB), L_, stream(), W, scales, x, y, rows, cols); \
+    HIP_CHECK(hipGetLastError()); } while (0)
+    if (rows >= 32768 && lds <= 40 * 1024) MATVEC_LAUNCH(4, 2, 1, 16, lds);
+    else if (rows >= 32768) MATVEC_LAUNCH(4, 2, 0, 16, 0);
+    else if (rows >= 8192) MATVEC_LAUNCH(2, 2, 0, 8, 0);
+    else MATVEC_LAUNCH(1, 4, 0, 4, 0);
+#undef MATVEC_LAUNCH
 }
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }

@@ -917,6 +917,7 @@ const float *sft_get_rope_thetas(SFTState *s) { return s->rope_thetas.data(); }
 int sft_is_full_param(SFTState *s) { return s->full_param; }
 const float *sft_get_token_emb(SFTState *s) { return s->token_emb_host; }
 MetalBuf *sft_get_final_norm_g(SFTState *s) { return s->g_final; }
+MetalBuf *sft_get_token_emb_buf(SFTState *s) { return s->emb; }
 
 size_t sft_lora_numel(SFTState *s) { return s->lora_n; }
 void sft_copy_lora(SFTState *s, float *dst) { if (s->lora_n) metal_buf_read(s->lora, 0, dst, s->lora_n * 4); }

@@ -136,7 +136,15 @@ def load():
         "sft_get_rope_thetas": (vp, [vp]), "sft_is_full_param": (i, [vp]), "sft_save_lora": (None, [vp, C.c_char_p]),
         "sft_lora_numel": (sz, [vp]), "sft_copy_lora": (None, [vp, vp]), "sft_copy_lora_grads": (None, [vp, vp]),
         "sft_set_lora": (None, [vp, vp]), "sft_get_last_grad_norm": (f, [vp]),
-        "sft_get_token_emb": (vp, [vp]), "sft_get_final_norm_g": (vp, [vp]),
+        "sft_get_token_emb": (vp, [vp]), "sft_get_token_emb_buf": (vp, [vp]),
+        "inference_state_create_from_ref": (vp, [C.POINTER(SFTModelRef), i, i]),
+        "inference_state_create_from_sft": (vp, [vp, i]), "inference_state_refresh_from_sft": (None, [vp]),
+        "inference_state_free": (None, [vp]), "inference_generate": (i, [vp, vp, i, vp, i]),
+        "inference_state_model_type": (i, [vp]), "inference_state_vocab_size": (i, [vp]),
+        "inference_state_reset": (None, [vp]), "inference_forward_token": (C.POINTER(C.c_float), [vp, i]),
+        "inference_forward_token_argmax": (i, [vp, i]), "inference_state_set_lora": (None, [vp, vp]),
+        "inference_state_set_eos": (None, [vp, vp, i]), "inference_state_load_eos": (None, [vp, C.c_char_p]),
+        "inference_state_position": (i, [vp]), "sft_get_final_norm_g": (vp, [vp]),
         "sft_get_layers": (C.POINTER(LayerW), [vp]), "sft_get_lm_head": (C.POINTER(WMat), [vp]),
         "sft_backward_sgd": (None, [vp, f]), "sft_alloc_grad_accum": (None, [vp]), "sft_backward_accum": (None, [vp]),
         "sft_apply_grad_sgd": (None, [vp, f]), "sft_save_full_checkpoint": (None, [vp, C.c_char_p]),

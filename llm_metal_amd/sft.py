@@ -89,27 +89,35 @@ def _layer_refs(c: SFTConfig, model, keep):
     return refs
 
 
+def model_ref(c: SFTConfig, model, lora_init=True):
+    """SFTModelRef over the numpy arrays of a synthetic model; returns (ref, arrays the ref points into, embedding
+    table).  The arrays must live until the create call returns; the SFT state also borrows the embedding table for
+    its lifetime (sft_get_token_emb hands it out)."""
+    keep = []
+    refs = _layer_refs(c, model, keep)
+    thetas = np.asarray(c.rope_thetas(), dtype=np.float32)
+    emb = np.ascontiguousarray(model["token_emb"], dtype=np.float32)
+    head = emb if model["lm_head"] is model["token_emb"] else np.ascontiguousarray(model["lm_head"], dtype=np.float32)
+    gf = np.ascontiguousarray(model["g_final"], dtype=np.float32)
+    lora = np.ascontiguousarray(model["lora"], dtype=np.float32) if (lora_init and c.R) else None
+    m = _lib.SFTModelRef(c.model_type, c.NL, c.D, c.Hq, c.Hkv, c.hd, c.IS, c.V, thetas.ctypes.data, refs,
+                         emb.ctypes.data, head.ctypes.data, gf.ctypes.data,
+                         lora.ctypes.data if lora is not None else None)
+    keep += [refs, thetas, emb, head, gf, lora]
+    return m, keep, emb
+
+
 class SFTState:
     """sft_state_create_from_ref ... sft_state_free."""
 
     def __init__(self, c: SFTConfig, model, lora_init=True):
         self.L = _lib.load()
         self.c = c
-        keep = []
-        refs = _layer_refs(c, model, keep)
-        thetas = np.asarray(c.rope_thetas(), dtype=np.float32)
-        emb = np.ascontiguousarray(model["token_emb"], dtype=np.float32)
-        head = emb if model["lm_head"] is model["token_emb"] else np.ascontiguousarray(model["lm_head"], dtype=np.float32)
-        gf = np.ascontiguousarray(model["g_final"], dtype=np.float32)
-        lora = np.ascontiguousarray(model["lora"], dtype=np.float32) if (lora_init and c.R) else None
-        m = _lib.SFTModelRef(c.model_type, c.NL, c.D, c.Hq, c.Hkv, c.hd, c.IS, c.V, thetas.ctypes.data, refs,
-                             emb.ctypes.data, head.ctypes.data, gf.ctypes.data,
-                             lora.ctypes.data if lora is not None else None)
+        m, keep, self._emb = model_ref(c, model, lora_init)
         self.h = self.L.sft_state_create_from_ref(C.byref(m), c.batch, c.seq, c.R, c.alpha,
                                                   1 if c.weight_format == "f16" else 0)
         if not self.h:
             raise RuntimeError("sft_state_create_from_ref failed (no gfx950 device or unsupported dims)")
-        self._emb = emb                                    # sft_get_token_emb hands out this (borrowed) table
 
     def train_step(self, tok, tgt, lr):
         tok = np.ascontiguousarray(tok, dtype=np.uint32)
@@ -217,6 +225,67 @@ class SFTState:
     def free(self):
         if self.h:
             self.L.sft_state_free(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.free()
+
+
+class InferenceState:
+    """inference_state_create_from_ref / _from_sft ... inference_state_free (include/inference_hip.h)."""
+
+    def __init__(self, c: SFTConfig = None, model=None, max_seq=256, use_fp16=True, sft: "SFTState" = None):
+        self.L = _lib.load()
+        if sft is not None:
+            self.c, self._keep = sft.c, [sft]
+            self.h = self.L.inference_state_create_from_sft(sft.h, max_seq)
+        else:
+            self.c = c
+            m, keep, _ = model_ref(c, model, lora_init=False)
+            self._keep = []
+            self.h = self.L.inference_state_create_from_ref(C.byref(m), max_seq, 1 if use_fp16 else 0)
+            del keep
+        if not self.h:
+            raise RuntimeError("inference state creation failed (no gfx950 device or unsupported dims)")
+        self.V = self.L.inference_state_vocab_size(self.h)
+
+    def reset(self):
+        self.L.inference_state_reset(self.h)
+
+    def forward_token(self, token):
+        p = self.L.inference_forward_token(self.h, int(token))
+        if not p:
+            raise RuntimeError("inference_forward_token refused the token (outside the vocabulary or cache full)")
+        return np.ctypeslib.as_array(p, shape=(self.V,)).copy()
+
+    def forward_token_argmax(self, token):
+        return int(self.L.inference_forward_token_argmax(self.h, int(token)))
+
+    def generate(self, prompt, max_gen_len):
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.zeros(max_gen_len, dtype=np.uint32)
+        n = self.L.inference_generate(self.h, _vp(prompt), len(prompt), _vp(out), max_gen_len)
+        return out[:n]
+
+    def set_eos(self, ids):
+        a = np.ascontiguousarray(ids, dtype=np.int32)
+        self.L.inference_state_set_eos(self.h, _vp(a), len(a))
+
+    def load_eos(self, path):
+        self.L.inference_state_load_eos(self.h, str(path).encode())
+
+    def refresh_from_sft(self):
+        self.L.inference_state_refresh_from_sft(self.h)
+
+    def position(self):
+        return int(self.L.inference_state_position(self.h))
+
+    def free(self):
+        if self.h:
+            self.L.inference_state_free(self.h)
             self.h = None
 
     def __enter__(self):
