@@ -294,24 +294,39 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
     for (int i = tid; i < G * hd; i += TB) qs[i] = Q[(size_t)hkv * G * hd + i];
     __syncthreads();
 
-    // scores: wave per key, lanes over the head dimension, four query heads per pass over the key
+    // scores: a wave takes four keys at a time (their loads are in flight together), lanes over the head dimension,
+    // four query heads per pass over the keys
     for (int g0 = 0; g0 < G; g0 += 4) {
         int gq[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, G - 1);
-        for (int jj = wave; jj < nj; jj += 4) {
-            const float *kp = kbase + (size_t)jj * hd;
-            float p[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int jj = wave * 4; jj < nj; jj += 16) {
+            const float *kp[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) kp[t] = kbase + (size_t)min(jj + t, nj - 1) * hd;
+            float p[4][4];
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int u = 0; u < 4; u++) p[t][u] = 0.f;
             for (int d = lane; d < hd; d += 64) {
-                const float kv = kp[d];
+                float kv[4], qv[4];
 #pragma unroll
-                for (int u = 0; u < 4; u++) p[u] = fmaf(qs[gq[u] * hd + d], kv, p[u]);
+                for (int t = 0; t < 4; t++) kv[t] = kp[t][d];
+#pragma unroll
+                for (int u = 0; u < 4; u++) qv[u] = qs[gq[u] * hd + d];
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int u = 0; u < 4; u++) p[t][u] = fmaf(qv[u], kv[t], p[t][u]);
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const float s = wave_sum(p[u]);
-                if (lane == 0 && g0 + u < G) sc[(g0 + u) * SL + jj] = s * scale;
-            }
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const float s = wave_sum(p[t][u]);
+                    if (lane == 0 && g0 + u < G && jj + t < nj) sc[(g0 + u) * SL + jj + t] = s * scale;
+                }
         }
     }
     __syncthreads();
@@ -337,10 +352,17 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
         for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, G - 1);
         float o[4] = {0.f, 0.f, 0.f, 0.f};
         if (active)
-            for (int jj = part; jj < nj; jj += parts) {
-                const float v = vbase[(size_t)jj * hd + d];
+            for (int jj = part; jj < nj; jj += 4 * parts) {                    // four independent loads per trip
+                float v[4];
+                int jt[4];
 #pragma unroll
-                for (int u = 0; u < 4; u++) o[u] = fmaf(sc[gq[u] * SL + jj], v, o[u]);
+                for (int t = 0; t < 4; t++) { jt[t] = jj + t * parts; v[t] = vbase[(size_t)min(jt[t], nj - 1) * hd + d]; }
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    if (jt[t] >= nj) v[t] = 0.f;
+#pragma unroll
+                    for (int u = 0; u < 4; u++) o[u] = fmaf(sc[gq[u] * SL + min(jt[t], nj - 1)], v[t], o[u]);
+                }
             }
         if (active) {
 #pragma unroll

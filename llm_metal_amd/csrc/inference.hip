@@ -2,6 +2,11 @@
 // src/nn/fast_inference.c (state, forward_token, generate, sharing with the SFT state) for the HIP backend.
 // Every step is enqueued on the library's one stream; the host waits once per token, for the logits or for
 // the argmax computed on the GPU.
+//
+// One decode step computes what src/nn/fast_inference.c:376-467 computes, in 9 launches per layer instead of 17
+// (10 instead of 23 with adapters): Q|K|V and gate|up are one matrix each (row concatenation, built when the state is
+// created), the residual add travels with the RMSNorm that follows it, and one kernel does LoRA up-projection,
+// per-head RMSNorm, RoPE and the KV-cache store for all heads.
 #include "backend.h"
 #include "devutil.h"
 #include "../../include/inference_hip.h"
@@ -24,11 +29,13 @@ struct InferenceState {
     float emb_scale, eps;
     int eos[4], n_eos;
     std::vector<float> thetas;
-    MetalBuf *x, *x2, *ln, *q, *k, *v, *att, *gate, *up, *ff, *logits, *best;
+    MetalBuf *x, *branch, *ln, *qkv, *att, *gu, *gate_v, *up_v, *logits, *best;   // gate_v / up_v: the halves of gu
     float *logits_host;
     int *best_host;
     std::vector<MetalBuf *> kc, vc;
-    LayerW *layers;
+    // per layer: fused [Wq; Wk; Wv] and [Wgate; Wup] (owned), Wo and Wdown and the norm gammas (owned, or the SFT state's)
+    struct Layer { WMat qkv, gu; WMat *o, *down; MetalBuf *g_in, *g_post_attn, *g_pre_ff, *g_post_ff, *g_q, *g_k; };
+    std::vector<Layer> layers;
     WMat *lm_head;
     MetalBuf *g_final, *emb;
     int owns_weights;
@@ -37,7 +44,7 @@ struct InferenceState {
     std::vector<Lora> lora;
     int R;
     float scaling;
-    MetalBuf *lora_tmp, *lora_out;
+    MetalBuf *lora_t;                    // [2R]: A_q ln | A_v ln
 };
 
 namespace {
@@ -51,90 +58,201 @@ __global__ __launch_bounds__(TB) void k_embed_row(const float *__restrict__ emb,
     if (i < D) x[i] = emb[(size_t)token * D + i] * scale;
 }
 
-// index of the first maximum of v[0..n) (src/nn/fast_inference.c:469-476), one workgroup of 1024 threads
-__global__ __launch_bounds__(1024) void k_argmax(const float *__restrict__ v, int n, int *__restrict__ out)
+// index of the first maximum of v[0..n) (src/nn/fast_inference.c:469-476) in two launches: AM_WGS workgroups leave
+// (value, index) of their slice, one workgroup picks among them
+constexpr int AM_WGS = 128;
+
+__device__ __forceinline__ void am_pick(float &best, int &idx, float ob, int oi)
 {
-    __shared__ float bv[16];
-    __shared__ int bi[16];
-    float best = -INFINITY;
-    int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const float a = v[i];
-        if (a > best || (a == best && i < idx)) { best = a; idx = i; }
-    }
+    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+}
+
+__device__ __forceinline__ void am_block(float &best, int &idx, float *bv, int *bi)
+{
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float ob = __shfl_xor(best, o, 64);
-        const int oi = __shfl_xor(idx, o, 64);
-        if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
-    }
+    for (int o = 32; o > 0; o >>= 1) am_pick(best, idx, __shfl_xor(best, o, 64), __shfl_xor(idx, o, 64));
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     if (lane == 0) { bv[w] = best; bi[w] = idx; }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int i = 1; i < 16; i++)
-            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) { best = bv[i]; idx = bi[i]; }
-        *out = idx == 0x7fffffff ? 0 : idx;
+    if (threadIdx.x == 0)
+        for (int i = 1; i < (int)(blockDim.x >> 6); i++) am_pick(best, idx, bv[i], bi[i]);
+}
+
+__global__ __launch_bounds__(TB) void k_argmax_part(const float *__restrict__ v, int n, float *__restrict__ pv, int *__restrict__ pi)
+{
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = blockIdx.x * TB + threadIdx.x; i < n; i += AM_WGS * TB) am_pick(best, idx, v[i], i);
+    am_block(best, idx, bv, bi);
+    if (threadIdx.x == 0) { pv[blockIdx.x] = best; pi[blockIdx.x] = idx; }
+}
+
+__global__ __launch_bounds__(AM_WGS) void k_argmax_final(const float *__restrict__ pv, const int *__restrict__ pi, int *__restrict__ out)
+{
+    __shared__ float bv[AM_WGS / 64];
+    __shared__ int bi[AM_WGS / 64];
+    float best = pv[threadIdx.x];
+    int idx = pi[threadIdx.x];
+    am_block(best, idx, bv, bi);
+    if (threadIdx.x == 0) *out = idx == 0x7fffffff ? 0 : idx;
+}
+
+// x += b (b = branch, or RMSNorm(branch; g_branch) where Gemma3 norms the branch output first); ln = RMSNorm(x; g).
+// branch == NULL: only the norm.  One workgroup of 1024 threads: the vector is a few thousand floats.
+__global__ __launch_bounds__(1024) void k_add_norm(float *__restrict__ x, const float *__restrict__ branch,
+                                                   const float *__restrict__ g_branch, const float *__restrict__ g,
+                                                   float *__restrict__ ln, int D, float eps)
+{
+    __shared__ float sm[16];
+    float inv_b = 1.f;
+    if (branch && g_branch) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < D; i += 1024) { const float v = branch[i]; ss += v * v; }
+        inv_b = rsqrtf(block_sum(ss, sm) / (float)D + eps);
+    }
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < D; i += 1024) {
+        float v = x[i];
+        if (branch) { v += g_branch ? branch[i] * inv_b * g_branch[i] : branch[i]; x[i] = v; }
+        ss += v * v;
+    }
+    const float inv = rsqrtf(block_sum(ss, sm) / (float)D + eps);
+    for (int i = threadIdx.x; i < D; i += 1024) ln[i] = x[i] * inv * g[i];       // own elements only: no barrier needed
+}
+
+// t[r] = A_q[r] . ln for r < R, t[R + r] = A_v[r] . ln: one wave per adapter row
+__global__ __launch_bounds__(64) void k_lora_down(const float *__restrict__ ln, const float *__restrict__ Aq,
+                                                  const float *__restrict__ Av, float *__restrict__ t, int R, int D)
+{
+    const int r = blockIdx.x;
+    const float *a = r < R ? Aq + (size_t)r * D : Av + (size_t)(r - R) * D;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < D; i += 64) s = fmaf(a[i], ln[i], s);
+    s = wave_sum(s);
+    if (threadIdx.x == 0) t[r] = s;
+}
+
+struct QkPostArgs {
+    float *qkv;                          // [Hq*hd | Hkv*hd | Hkv*hd]; q is finished in place
+    const float *g_q, *g_k;              // per-head norm gammas or NULL
+    float *kc, *vc;                      // caches [Hkv, max_seq, hd]
+    const float *t, *Bq, *Bv;            // adapters: t [2R], B_q [Hq*hd, R], B_v [Hkv*hd, R]; R == 0: none
+    int Hq, Hkv, hd, max_seq, pos, R;
+    float theta, eps, sc;
+};
+
+// One wave per head (q heads, then k heads, then v heads); lane i owns the rotary pair (i, i + hd/2), hd <= 256.
+// q: += sc B_q t_q, per-head RMSNorm, RoPE, in place.  k: RMSNorm, RoPE, into the cache row `pos`.  v: += sc B_v t_v,
+// into the cache.  (src/nn/fast_inference.c:402-427; kernels shaders/q8_kernels.metal:165-256)
+__global__ __launch_bounds__(64) void k_qk_post(QkPostArgs a)
+{
+    const int h = blockIdx.x, lane = threadIdx.x, half = a.hd / 2;
+    const bool is_q = h < a.Hq, is_k = !is_q && h < a.Hq + a.Hkv;
+    const int hk = is_q ? 0 : (is_k ? h - a.Hq : h - a.Hq - a.Hkv);
+    float *vec = a.qkv + (size_t)h * a.hd;
+    float x0[2] = {0.f, 0.f}, x1[2] = {0.f, 0.f};                    // pairs lane and lane + 64
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int i = lane + 64 * u;
+        if (i < half) {
+            x0[u] = vec[i]; x1[u] = vec[i + half];
+            if (a.R && !is_k) {
+                const float *B = is_q ? a.Bq + (size_t)h * a.hd * a.R : a.Bv + (size_t)hk * a.hd * a.R;
+                const float *t = is_q ? a.t : a.t + a.R;
+                float d0 = 0.f, d1 = 0.f;
+                for (int r = 0; r < a.R; r++) { d0 = fmaf(B[(size_t)i * a.R + r], t[r], d0); d1 = fmaf(B[(size_t)(i + half) * a.R + r], t[r], d1); }
+                x0[u] = fmaf(a.sc, d0, x0[u]); x1[u] = fmaf(a.sc, d1, x1[u]);
+            }
+            ss += x0[u] * x0[u] + x1[u] * x1[u];
+        }
+    }
+    if (is_q || is_k) {
+        const float *g = is_q ? a.g_q : a.g_k;
+        if (g) {
+            const float inv = rsqrtf(wave_sum(ss) / (float)a.hd + a.eps);
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int i = lane + 64 * u;
+                if (i < half) { x0[u] *= inv * g[i]; x1[u] *= inv * g[i + half]; }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int i = lane + 64 * u;
+            if (i < half) {
+                const float freq = 1.0f / powf(a.theta, (float)(2 * i) / (float)a.hd);
+                float sn, cs;
+                sincosf((float)a.pos * freq, &sn, &cs);
+                const float r0 = x0[u] * cs - x1[u] * sn, r1 = x0[u] * sn + x1[u] * cs;
+                x0[u] = r0; x1[u] = r1;
+            }
+        }
+    }
+    float *dst = is_q ? vec : (is_k ? a.kc : a.vc) + ((size_t)hk * a.max_seq + a.pos) * a.hd;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int i = lane + 64 * u;
+        if (i < half) { dst[i] = x0[u]; dst[i + half] = x1[u]; }
     }
 }
 
 MetalBuf *fbuf(size_t n) { return metal_buf_create(n * sizeof(float)); }
 
-void matvec(InferenceState *s, WMat *w, MetalBuf *x, MetalBuf *y)
+void matvec(InferenceState *s, const WMat *w, MetalBuf *x, MetalBuf *y)
 {
     if (s->use_fp16) metal_enqueue_f16_matvec(w->mbuf, x, y, w->rows, w->cols);
     else metal_enqueue_q8_matvec(w->mbuf, x, y, w->rows, w->nb);
 }
 
+void add_norm(InferenceState *s, MetalBuf *branch, MetalBuf *g_branch, MetalBuf *g)
+{
+    hipLaunchKernelGGL(k_add_norm, dim3(1), dim3(1024), 0, stream(), dptr_as<float>(s->x), branch ? dptr_as<float>(branch) : nullptr,
+                       g_branch ? dptr_as<float>(g_branch) : nullptr, dptr_as<float>(g), dptr_as<float>(s->ln), s->D, s->eps);
+}
+
 // src/nn/fast_inference.c:376-467
 void forward_token(InferenceState *s, int token, int pos)
 {
-    const int D = s->D, Hq = s->Hq, Hkv = s->Hkv, hd = s->hd, qd = Hq * hd, kd = Hkv * hd;
+    const int D = s->D, Hq = s->Hq, Hkv = s->Hkv, hd = s->hd;
     const bool gemma = s->model_type == MODEL_GEMMA3;
     hipLaunchKernelGGL(k_embed_row, dim3((D + TB - 1) / TB), dim3(TB), 0, stream(), dptr_as<float>(s->emb), token, s->emb_scale,
                        dptr_as<float>(s->x), D);
+    MetalBuf *pending = nullptr, *pending_g = nullptr;           // FFN branch of the previous layer, added by the next norm kernel
     for (int L = 0; L < s->NL; L++) {
-        LayerW *lw = &s->layers[L];
-        metal_enqueue_rms_norm(s->x, lw->input_norm_g, s->ln, D, s->eps);
-        matvec(s, lw->q_proj, s->ln, s->q);
-        matvec(s, lw->k_proj, s->ln, s->k);
-        matvec(s, lw->v_proj, s->ln, s->v);
+        const InferenceState::Layer &lw = s->layers[L];
+        add_norm(s, pending, pending_g, lw.g_in);
+        matvec(s, &lw.qkv, s->ln, s->qkv);
+        QkPostArgs a{};
+        a.qkv = dptr_as<float>(s->qkv);
+        a.g_q = lw.g_q ? dptr_as<float>(lw.g_q) : nullptr; a.g_k = lw.g_k ? dptr_as<float>(lw.g_k) : nullptr;
+        a.kc = dptr_as<float>(s->kc[L]); a.vc = dptr_as<float>(s->vc[L]);
+        a.Hq = Hq; a.Hkv = Hkv; a.hd = hd; a.max_seq = s->max_seq; a.pos = pos;
+        a.theta = s->thetas[L]; a.eps = s->eps;
         if (!s->lora.empty()) {
             const InferenceState::Lora &lr = s->lora[L];
-            metal_enqueue_float_matmul(s->ln, lr.Aq, s->lora_tmp, 1, s->R, D);
-            metal_enqueue_float_matmul(s->lora_tmp, lr.Bq, s->lora_out, 1, qd, s->R);
-            metal_enqueue_add_scaled(s->q, s->lora_out, s->scaling, qd);
-            metal_enqueue_float_matmul(s->ln, lr.Av, s->lora_tmp, 1, s->R, D);
-            metal_enqueue_float_matmul(s->lora_tmp, lr.Bv, s->lora_out, 1, kd, s->R);
-            metal_enqueue_add_scaled(s->v, s->lora_out, s->scaling, kd);
+            hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R), dim3(64), 0, stream(), dptr_as<float>(s->ln), dptr_as<float>(lr.Aq),
+                               dptr_as<float>(lr.Av), dptr_as<float>(s->lora_t), s->R, D);
+            a.t = dptr_as<float>(s->lora_t); a.Bq = dptr_as<float>(lr.Bq); a.Bv = dptr_as<float>(lr.Bv);
+            a.R = s->R; a.sc = s->scaling;
         }
-        if (lw->q_norm_g) metal_enqueue_per_head_rms_norm(s->q, lw->q_norm_g, Hq, hd, s->eps);
-        if (lw->k_norm_g) metal_enqueue_per_head_rms_norm(s->k, lw->k_norm_g, Hkv, hd, s->eps);
-        metal_enqueue_rope(s->q, s->k, Hq, Hkv, hd, pos, s->thetas[L]);
-        metal_enqueue_kv_cache_store(s->k, s->v, s->kc[L], s->vc[L], Hkv, s->max_seq, hd, pos);
-        metal_enqueue_attention(s->q, s->kc[L], s->vc[L], s->att, pos + 1, hd, s->max_seq, Hq, Hq / Hkv);
-        matvec(s, lw->o_proj, s->att, s->x2);
-        if (lw->post_attn_norm_g && lw->pre_ff_norm_g) {         // Gemma3: norm of the branch before the residual add
-            metal_enqueue_rms_norm(s->x2, lw->post_attn_norm_g, s->ln, D, s->eps);
-            metal_enqueue_residual_add(s->x, s->ln, D);
-        } else {
-            metal_enqueue_residual_add(s->x, s->x2, D);
-        }
-        MetalBuf *ff_norm = lw->pre_ff_norm_g ? lw->pre_ff_norm_g : lw->post_attn_norm_g;
-        metal_enqueue_rms_norm(s->x, ff_norm, s->ln, D, s->eps);
-        matvec(s, lw->gate_proj, s->ln, s->gate);
-        matvec(s, lw->up_proj, s->ln, s->up);
-        if (gemma) metal_enqueue_gelu_mul(s->gate, s->up, s->IS);
-        else metal_enqueue_silu_mul(s->gate, s->up, s->IS);
-        matvec(s, lw->down_proj, s->gate, s->ff);
-        if (lw->post_ff_norm_g) {
-            metal_enqueue_rms_norm(s->ff, lw->post_ff_norm_g, s->x2, D, s->eps);
-            metal_enqueue_residual_add(s->x, s->x2, D);
-        } else {
-            metal_enqueue_residual_add(s->x, s->ff, D);
-        }
+        hipLaunchKernelGGL(k_qk_post, dim3(Hq + 2 * Hkv), dim3(64), 0, stream(), a);
+        mark_written(s->kc[L]); mark_written(s->vc[L]);
+        metal_enqueue_attention_off(s->qkv, 0, s->kc[L], s->vc[L], s->att, 0, pos + 1, hd, s->max_seq, Hq, Hq / Hkv);
+        matvec(s, lw.o, s->att, s->branch);
+        // x += o (Gemma3: RMSNorm(o; g_post_attn)); ln = RMSNorm(x; g_pre_ff | g_post_attn)
+        add_norm(s, s->branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
+        matvec(s, &lw.gu, s->ln, s->gu);
+        if (gemma) metal_enqueue_gelu_mul(s->gate_v, s->up_v, s->IS);
+        else metal_enqueue_silu_mul(s->gate_v, s->up_v, s->IS);
+        matvec(s, lw.down, s->gate_v, s->branch);
+        pending = s->branch;
+        pending_g = gemma ? lw.g_post_ff : nullptr;
     }
-    metal_enqueue_rms_norm(s->x, s->g_final, s->ln, D, s->eps);
+    add_norm(s, pending, pending_g, s->g_final);
+    HIP_CHECK(hipGetLastError());
     matvec(s, s->lm_head, s->ln, s->logits);
 }
 
@@ -147,7 +265,10 @@ const float *logits_to_host(InferenceState *s)
 
 int argmax_to_host(InferenceState *s)
 {
-    hipLaunchKernelGGL(k_argmax, dim3(1), dim3(1024), 0, stream(), dptr_as<float>(s->logits), s->V, dptr_as<int>(s->best));
+    float *pv = dptr_as<float>(s->best) + 4;
+    int *pi = dptr_as<int>(s->best) + 4 + AM_WGS;
+    hipLaunchKernelGGL(k_argmax_part, dim3(AM_WGS), dim3(TB), 0, stream(), dptr_as<float>(s->logits), s->V, pv, pi);
+    hipLaunchKernelGGL(k_argmax_final, dim3(1), dim3(AM_WGS), 0, stream(), pv, pi, dptr_as<int>(s->best));
     HIP_CHECK(hipMemcpyAsync(s->best_host, dptr(s->best), sizeof(int), hipMemcpyDeviceToHost, stream()));
     HIP_CHECK(hipStreamSynchronize(stream()));
     return *s->best_host;
@@ -164,8 +285,8 @@ InferenceState *new_state(ModelType mt, int D, int Hq, int Hkv, int hd, int IS, 
                           const float *thetas)
 {
     if (fast_metal_init() != 0) { fprintf(stderr, "[FastGen] no GPU: fast_metal_init failed\n"); return nullptr; }
-    if (Hkv <= 0 || Hq % Hkv || hd > 256 || Hq / Hkv > 16 || max_seq <= 0) {
-        fprintf(stderr, "[FastGen] unsupported shape: %d / %d heads of %d (head_dim <= 256, group ratio <= 16)\n", Hq, Hkv, hd);
+    if (Hkv <= 0 || Hq % Hkv || hd > 256 || (hd & 1) || Hq / Hkv > 16 || max_seq <= 0 || (IS & 3)) {
+        fprintf(stderr, "[FastGen] unsupported shape: %d / %d heads of %d (head_dim even and <= 256, group ratio <= 16, FFN width a multiple of 4)\n", Hq, Hkv, hd);
         fast_metal_shutdown();
         return nullptr;
     }
@@ -177,17 +298,19 @@ InferenceState *new_state(ModelType mt, int D, int Hq, int Hkv, int hd, int IS, 
     s->thetas.assign(thetas, thetas + NL);
     default_eos(s);
     const int qd = Hq * hd, kd = Hkv * hd;
-    s->x = fbuf(D); s->x2 = fbuf(D); s->ln = fbuf(D);
-    s->q = fbuf(qd); s->k = fbuf(kd); s->v = fbuf(kd); s->att = fbuf(qd);
-    s->gate = fbuf(IS); s->up = fbuf(IS); s->ff = fbuf(D);
-    s->logits = fbuf(V); s->best = metal_buf_create(sizeof(int));
+    s->x = fbuf(D); s->branch = fbuf(D); s->ln = fbuf(D);
+    s->qkv = fbuf(qd + 2 * kd); s->att = fbuf(qd);
+    s->gu = fbuf(2 * (size_t)IS);
+    s->gate_v = metal_buf_view(s->gu, 0, (size_t)IS * 4); s->up_v = metal_buf_view(s->gu, (size_t)IS * 4, (size_t)IS * 4);
+    s->logits = fbuf(V); s->best = metal_buf_create((4 + 2 * AM_WGS) * sizeof(int));   // result, then the per-workgroup (value, index) pairs
     HIP_CHECK(hipHostMalloc((void **)&s->logits_host, (size_t)V * 4, hipHostMallocDefault));
     HIP_CHECK(hipHostMalloc((void **)&s->best_host, sizeof(int), hipHostMallocDefault));
     const size_t cache_bytes = (size_t)Hkv * max_seq * hd * sizeof(float);
     for (int L = 0; L < NL; L++) { s->kc.push_back(metal_buf_create(cache_bytes)); s->vc.push_back(metal_buf_create(cache_bytes)); }
-    s->R = 0; s->scaling = 0.f; s->lora_tmp = s->lora_out = nullptr;
+    s->R = 0; s->scaling = 0.f; s->lora_t = nullptr;
     s->sft = nullptr; s->owns_weights = 0;
-    s->layers = nullptr; s->lm_head = nullptr; s->g_final = s->emb = nullptr;
+    s->layers.resize(NL);
+    s->lm_head = nullptr; s->g_final = s->emb = nullptr;
     return s;
 }
 
@@ -226,7 +349,35 @@ InferenceState *inference_state_create_from_ref(const SFTModelRef *m, int max_se
     InferenceState *s = new_state(m->model_type, m->d_model, m->n_q_heads, m->n_kv_heads, m->head_dim, m->intermediate_size,
                                   m->vocab_size, m->n_layers, max_seq_len, use_fp16, m->rope_thetas);
     if (!s) return nullptr;
-    s->layers = layers_convert_upload(m->layers, m->n_layers, use_fp16);
+    // [Wq; Wk; Wv] and [Wgate; Wup] are converted as one matrix each: F16 rounding and Q8_0 blocks are per row, so
+    // the rows of the fused matrix are bit for bit those of wmat_create_f16 / wmat_create_q8 on the parts
+    std::vector<float> cat;
+    auto fused = [&](std::initializer_list<const WeightRef *> parts) {
+        int rows = 0;
+        const int cols = (*parts.begin())->cols;
+        for (const WeightRef *w : parts) rows += w->rows;
+        cat.resize((size_t)rows * cols);
+        size_t o = 0;
+        for (const WeightRef *w : parts) { memcpy(cat.data() + o, w->data, (size_t)w->rows * cols * sizeof(float)); o += (size_t)w->rows * cols; }
+        WMat *t = wmat_convert(cat.data(), rows, cols, use_fp16);
+        WMat out = *t;
+        free(t);                                                          // the handle only; the buffer lives on in `out`
+        return out;
+    };
+    for (int L = 0; L < m->n_layers; L++) {
+        const LayerWeightRef *r = &m->layers[L];
+        InferenceState::Layer &lw = s->layers[L];
+        lw.qkv = fused({&r->q_proj, &r->k_proj, &r->v_proj});
+        lw.gu = fused({&r->gate_proj, &r->up_proj});
+        lw.o = wmat_convert(r->o_proj.data, r->o_proj.rows, r->o_proj.cols, use_fp16);
+        lw.down = wmat_convert(r->down_proj.data, r->down_proj.rows, r->down_proj.cols, use_fp16);
+        lw.g_in = norm_upload(r->input_norm_g, r->d_model);
+        lw.g_post_attn = norm_upload(r->post_attn_norm_g, r->d_model);
+        lw.g_pre_ff = r->pre_ff_norm_g ? norm_upload(r->pre_ff_norm_g, r->d_model) : nullptr;
+        lw.g_post_ff = r->post_ff_norm_g ? norm_upload(r->post_ff_norm_g, r->d_model) : nullptr;
+        lw.g_q = r->q_norm_g ? norm_upload(r->q_norm_g, r->head_dim) : nullptr;
+        lw.g_k = r->k_norm_g ? norm_upload(r->k_norm_g, r->head_dim) : nullptr;
+    }
     s->lm_head = wmat_convert(m->lm_head, m->vocab_size, m->d_model, use_fp16);
     s->g_final = norm_upload(m->final_norm_g, m->d_model);
     s->emb = metal_buf_from_data(m->token_emb, (size_t)m->vocab_size * m->d_model * sizeof(float));
@@ -251,7 +402,28 @@ InferenceState *inference_state_create_from_sft(SFTState *sft, int max_seq_len)
 void inference_state_refresh_from_sft(InferenceState *s)
 {
     if (!s || !s->sft) return;
-    s->layers = sft_get_layers(s->sft);
+    LayerW *src = sft_get_layers(s->sft);                                 // row-major F16 copies, refreshed by the call
+    const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS;
+    for (int L = 0; L < s->NL; L++) {
+        InferenceState::Layer &lw = s->layers[L];
+        if (!lw.qkv.mbuf) {
+            lw.qkv = WMat{metal_buf_create((size_t)(qd + 2 * kd) * D * 2), qd + 2 * kd, D, D / 32};
+            lw.gu = WMat{metal_buf_create((size_t)2 * IS * D * 2), 2 * IS, D, D / 32};
+        }
+        struct Part { WMat *w; MetalBuf *dst; size_t row0; };
+        const Part parts[5] = {{src[L].q_proj, lw.qkv.mbuf, 0}, {src[L].k_proj, lw.qkv.mbuf, (size_t)qd},
+                               {src[L].v_proj, lw.qkv.mbuf, (size_t)(qd + kd)}, {src[L].gate_proj, lw.gu.mbuf, 0},
+                               {src[L].up_proj, lw.gu.mbuf, (size_t)IS}};
+        for (const Part &p : parts) {
+            HIP_CHECK(hipMemcpyAsync((char *)dptr(p.dst) + p.row0 * D * 2, dptr(p.w->mbuf), (size_t)p.w->rows * D * 2,
+                                     hipMemcpyDeviceToDevice, stream()));
+            mark_written(p.dst);
+        }
+        lw.o = src[L].o_proj; lw.down = src[L].down_proj;
+        lw.g_in = src[L].input_norm_g; lw.g_post_attn = src[L].post_attn_norm_g;
+        lw.g_pre_ff = src[L].pre_ff_norm_g; lw.g_post_ff = src[L].post_ff_norm_g;
+        lw.g_q = src[L].q_norm_g; lw.g_k = src[L].k_norm_g;
+    }
     s->lm_head = sft_get_lm_head(s->sft);
 }
 
@@ -259,11 +431,7 @@ void inference_state_set_lora(InferenceState *s, SFTState *sft)
 {
     const int R = sft_get_lora_rank(sft);
     if (R == 0) return;                                                   // full-parameter state: no adapters
-    const int qd = s->Hq * s->hd, kd = s->Hkv * s->hd;
-    if (s->lora.empty()) {
-        s->lora_tmp = fbuf(R);
-        s->lora_out = fbuf(qd > kd ? qd : kd);
-    }
+    if (!s->lora_t) s->lora_t = fbuf(2 * (size_t)R);
     s->lora.resize(s->NL);
     for (int L = 0; L < s->NL; L++)
         s->lora[L] = InferenceState::Lora{sft_get_lora_weight_buf(sft, L, 0), sft_get_lora_weight_buf(sft, L, 1),
@@ -276,14 +444,21 @@ void inference_state_free(InferenceState *s)
 {
     if (!s) return;
     metal_flush();
-    for (MetalBuf *b : {s->x, s->x2, s->ln, s->q, s->k, s->v, s->att, s->gate, s->up, s->ff, s->logits, s->best, s->lora_tmp, s->lora_out})
+    for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t})
         metal_buf_free(b);
     for (MetalBuf *b : s->kc) metal_buf_free(b);
     for (MetalBuf *b : s->vc) metal_buf_free(b);
     hipHostFree(s->logits_host);
     hipHostFree(s->best_host);
+    for (InferenceState::Layer &lw : s->layers) {
+        metal_buf_free(lw.qkv.mbuf);
+        metal_buf_free(lw.gu.mbuf);
+        if (s->owns_weights) {
+            wmat_free(lw.o); wmat_free(lw.down);
+            for (MetalBuf *b : {lw.g_in, lw.g_post_attn, lw.g_pre_ff, lw.g_post_ff, lw.g_q, lw.g_k}) metal_buf_free(b);
+        }
+    }
     if (s->owns_weights) {
-        layers_free(s->layers, s->NL);
         wmat_free(s->lm_head);
         metal_buf_free(s->g_final);
         metal_buf_free(s->emb);
