@@ -273,33 +273,35 @@ __global__ __launch_bounds__(TB) void k_kv_store(const float *__restrict__ k, co
 
 constexpr int SL = 256;      // keys per workgroup
 
-// attention, shaders/q8_kernels.metal:262-331, restructured for a GPU with 256 CUs: one workgroup per (KV head, slice of
-// SL keys) serves all G query heads of the group, so the cache is read once; with more than one slice the workgroups
-// leave (max, sum, unnormalised output) per query head and k_attn_combine merges them.
-// LDS: q [G][hd], scores [G][SL], ml [2][G], red [4 * 256].  hd <= 256.
+// attention, shaders/q8_kernels.metal:262-331, restructured for a GPU with 256 CUs: a workgroup serves `gpw` query
+// heads that share a KV head (all G of the group when the context is long, so that the cache is read once; one when
+// it is short and the launch is bound by latency, not bytes) over a slice of SL keys; with more than one slice the
+// workgroups leave (max, sum, unnormalised output) per query head and k_attn_combine merges them.
+// VEC: floats of V per thread in the weighted sum (4 when hd % 4 == 0).
+// LDS: q [gpw][hd], scores [gpw][SL], ml [2][gpw], red [4 * 1024].  hd <= 256.
+template <int VEC>
 __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q, const float *__restrict__ Kc,
                                                     const float *__restrict__ Vc, float *__restrict__ out,
                                                     float *__restrict__ part_o, float *__restrict__ part_ml,
-                                                    int n_attend, int hd, int max_seq, int G, float scale, int nsplit)
+                                                    int n_attend, int hd, int max_seq, int G, int gpw, float scale, int nsplit)
 {
     extern __shared__ float sm[];
-    __shared__ float rs[16];
-    float *qs = sm, *sc = qs + G * hd, *ml = sc + G * SL, *red = ml + 2 * G;
+    float *qs = sm, *sc = qs + gpw * hd, *ml = sc + gpw * SL, *red = ml + 2 * gpw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hkv = blockIdx.x, split = blockIdx.y;
+    const int hq0 = blockIdx.x * gpw, hkv = hq0 / G, split = blockIdx.y;
     const int j0 = split * SL, nj = min(SL, n_attend - j0);
     const float *kbase = Kc + ((size_t)hkv * max_seq + j0) * hd;
     const float *vbase = Vc + ((size_t)hkv * max_seq + j0) * hd;
 
-    for (int i = tid; i < G * hd; i += TB) qs[i] = Q[(size_t)hkv * G * hd + i];
+    for (int i = tid; i < gpw * hd; i += TB) qs[i] = Q[(size_t)hq0 * hd + i];
     __syncthreads();
 
     // scores: a wave takes four keys at a time (their loads are in flight together), lanes over the head dimension,
     // four query heads per pass over the keys
-    for (int g0 = 0; g0 < G; g0 += 4) {
+    for (int g0 = 0; g0 < gpw; g0 += 4) {
         int gq[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, G - 1);
+        for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, gpw - 1);
         for (int jj = wave * 4; jj < nj; jj += 16) {
             const float *kp[4];
 #pragma unroll
@@ -321,71 +323,93 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
                     for (int u = 0; u < 4; u++) p[t][u] = fmaf(qv[u], kv[t], p[t][u]);
             }
 #pragma unroll
-            for (int t = 0; t < 4; t++)
+            for (int u = 0; u < 4; u++) {
+                if (g0 + u >= gpw) break;                                   // uniform
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
+                for (int t = 0; t < 4; t++) {
                     const float s = wave_sum(p[t][u]);
-                    if (lane == 0 && g0 + u < G && jj + t < nj) sc[(g0 + u) * SL + jj + t] = s * scale;
+                    if (lane == 0 && jj + t < nj) sc[(g0 + u) * SL + jj + t] = s * scale;
                 }
+            }
         }
     }
     __syncthreads();
 
-    // softmax statistics of the slice, per query head
-    for (int g = 0; g < G; g++) {
+    // softmax statistics of the slice: one wave per query head, no barriers
+    for (int g = wave; g < gpw; g += 4) {
         float m = -3.0e38f;
-        for (int j = tid; j < nj; j += TB) m = fmaxf(m, sc[g * SL + j]);
-        m = block_max(m, rs);
+        for (int j = lane; j < nj; j += 64) m = fmaxf(m, sc[g * SL + j]);
+        m = wave_max(m);
         float l = 0.f;
-        for (int j = tid; j < nj; j += TB) { const float e = __expf(sc[g * SL + j] - m); sc[g * SL + j] = e; l += e; }
-        l = block_sum(l, rs);
-        if (tid == 0) { ml[g] = m; ml[G + g] = l; }
+        for (int j = lane; j < nj; j += 64) { const float e = __expf(sc[g * SL + j] - m); sc[g * SL + j] = e; l += e; }
+        l = wave_sum(l);
+        if (lane == 0) { ml[g] = m; ml[gpw + g] = l; }
     }
     __syncthreads();
 
-    // weighted value sum: thread = (part of the keys, d); parts are added through LDS
-    const int parts = max(1, TB / hd), part = tid / hd, d = tid % hd;
+    // weighted value sum: thread = (part of the keys, VEC consecutive d); parts are added through LDS
+    const int dpt = hd / VEC;                                               // threads along d
+    const int parts = max(1, TB / dpt), part = tid / dpt, d = (tid % dpt) * VEC;
     const bool active = part < parts;
-    for (int g0 = 0; g0 < G; g0 += 4) {
+    typedef float vecf __attribute__((ext_vector_type(VEC)));
+    for (int g0 = 0; g0 < gpw; g0 += 4) {
         int gq[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, G - 1);
-        float o[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < 4; u++) gq[u] = min(g0 + u, gpw - 1);
+        float o[4][VEC];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int e = 0; e < VEC; e++) o[u][e] = 0.f;
         if (active)
             for (int jj = part; jj < nj; jj += 4 * parts) {                    // four independent loads per trip
-                float v[4];
+                float v[4][VEC];
                 int jt[4];
 #pragma unroll
-                for (int t = 0; t < 4; t++) { jt[t] = jj + t * parts; v[t] = vbase[(size_t)min(jt[t], nj - 1) * hd + d]; }
-#pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    if (jt[t] >= nj) v[t] = 0.f;
+                    jt[t] = min(jj + t * parts, nj - 1);
+                    const float live = (jj + t * parts < nj) ? 1.f : 0.f;
+                    if (VEC == 1) v[t][0] = vbase[(size_t)jt[t] * hd + d] * live;
+                    else {
+                        const vecf vv = *reinterpret_cast<const vecf *>(&vbase[(size_t)jt[t] * hd + d]);
 #pragma unroll
-                    for (int u = 0; u < 4; u++) o[u] = fmaf(sc[gq[u] * SL + min(jt[t], nj - 1)], v[t], o[u]);
+                        for (int e = 0; e < VEC; e++) v[t][e] = vv[e] * live;
+                    }
                 }
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const float w = sc[gq[u] * SL + jt[t]];
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) o[u][e] = fmaf(w, v[t][e], o[u][e]);
+                    }
             }
         if (active) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) red[(part * 4 + u) * hd + d] = o[u];
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) red[(part * 4 + u) * hd + d + e] = o[u][e];
         }
         __syncthreads();
-        if (part == 0) {
+        // thread t < hd finishes element t of every head of this pass
+        if (tid < hd) {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                if (g0 + u >= G) continue;
+                if (g0 + u >= gpw) continue;
                 float s = 0.f;
-                for (int pp = 0; pp < parts; pp++) s += red[(pp * 4 + u) * hd + d];
-                const int hq = hkv * G + g0 + u;
-                if (nsplit == 1) out[(size_t)hq * hd + d] = s / ml[G + g0 + u];
-                else part_o[((size_t)hq * nsplit + split) * hd + d] = s;
+                for (int pp = 0; pp < parts; pp++) s += red[(pp * 4 + u) * hd + tid];
+                const int hq = hq0 + g0 + u;
+                if (nsplit == 1) out[(size_t)hq * hd + tid] = s / ml[gpw + g0 + u];
+                else part_o[((size_t)hq * nsplit + split) * hd + tid] = s;
             }
         }
         __syncthreads();
     }
-    if (nsplit > 1 && tid < G) {
-        const int hq = hkv * G + tid;
+    if (nsplit > 1 && tid < gpw) {
+        const int hq = hq0 + tid;
         part_ml[((size_t)hq * nsplit + split) * 2] = ml[tid];
-        part_ml[((size_t)hq * nsplit + split) * 2 + 1] = ml[G + tid];
+        part_ml[((size_t)hq * nsplit + split) * 2 + 1] = ml[gpw + tid];
     }
 }
 
@@ -452,7 +476,9 @@ void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_att
     if (n_attend > max_seq) { fprintf(stderr, "[fast_hip] %s: n_attend %d exceeds the cache (%d); launch skipped\n", fn, n_attend, max_seq); return; }
     if (hd > 256 || G > 16) { fprintf(stderr, "[fast_hip] %s: head_dim %d / group ratio %d not supported (<= 256 / <= 16); launch skipped\n", fn, hd, G); return; }
     const int nsplit = (n_attend + SL - 1) / SL;
-    const size_t lds = ((size_t)G * hd + (size_t)G * SL + 2 * G + 4 * 256) * 4;
+    // short contexts are bound by latency: one query head per workgroup; long ones by cache bytes: the whole group
+    const int gpw = n_attend <= 128 ? 1 : G;
+    const size_t lds = ((size_t)gpw * hd + (size_t)gpw * SL + 2 * gpw + 4 * 1024) * 4;
     float *po = nullptr, *pml = nullptr;
     if (nsplit > 1) {
         const size_t o_bytes = (size_t)Hq * nsplit * hd * 4;
@@ -460,8 +486,13 @@ void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_att
         pml = po + (size_t)Hq * nsplit * hd;
     }
     const float scale = 1.0f / sqrtf((float)hd);
-    LAUNCH(k_attn_decode, dim3(Hkv, nsplit), dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml, n_attend, hd,
-           max_seq, G, scale, nsplit);
+    const bool vec4 = hd % 4 == 0 && (((uintptr_t)dptr(Vc)) & 15) == 0;
+    if (vec4)
+        LAUNCH(k_attn_decode<4>, dim3(Hq / gpw, nsplit), dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml,
+               n_attend, hd, max_seq, G, gpw, scale, nsplit);
+    else
+        LAUNCH(k_attn_decode<1>, dim3(Hq / gpw, nsplit), dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml,
+               n_attend, hd, max_seq, G, gpw, scale, nsplit);
     if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq), dim3(TB), 0, po, pml, out, hd, nsplit);
 }
 

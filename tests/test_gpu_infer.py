@@ -144,8 +144,9 @@ def test_rope_and_kv_cache_store(dev, Hq, Hkv, hd, theta):
         assert np.array_equal(kcb2.read(F, ek.shape), e2) and np.array_equal(vcb2.read(F, ev.shape), ev)
 
 
-# n_attend > 256 splits the keys over several workgroups per KV head
-@pytest.mark.parametrize("Hq,ratio,hd,max_seq,n", [(32, 4, 128, 512, 1), (32, 4, 128, 512, 200), (4, 4, 256, 1024, 700),
+# up to 128 keys one query head per workgroup, beyond that the whole group; n_attend > 256 splits the keys over
+# several workgroups
+@pytest.mark.parametrize("Hq,ratio,hd,max_seq,n", [(32, 4, 128, 512, 1), (32, 4, 128, 512, 100), (32, 4, 128, 512, 200), (4, 4, 256, 1024, 700), (6, 2, 30, 200, 77),
                                                    (6, 3, 32, 300, 300), (2, 1, 64, 64, 64), (8, 8, 128, 2100, 2100),
                                                    (5, 5, 48, 260, 257)])
 def test_attention_over_the_cache(dev, Hq, ratio, hd, max_seq, n):
