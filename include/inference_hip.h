@@ -27,6 +27,12 @@ typedef struct InferenceState InferenceState;
  * attention kernel holds 4096 scores; this one has no such limit).  NULL when no GPU is present. */
 InferenceState *inference_state_create_from_ref(const SFTModelRef *model, int max_seq_len, int use_fp16);
 
+/* The same from a checkpoint file (loader_hip.h: safetensors file / shard directory or GGUF): the reference's
+ * qwen3_load_safetensors / qwen3_load_gguf / gemma3_load_safetensors followed by inference_state_create, without the
+ * fp32 copy of the model in host memory: tensor bytes are uploaded as stored and converted on the GPU, and F16 / Q8_0
+ * tensors that already have the wanted format are used bit for bit (no dequantise -> requantise). */
+InferenceState *inference_state_create_from_file(const char *path, ModelType model_type, int max_seq_len, int use_fp16);
+
 /* src/nn/fast_inference.h:49 (impl src/nn/fast_inference.c:527-610): shares the SFT state's weights (row-major F16
  * copies handed out by sft_get_layers / sft_get_lm_head), embedding table, final norm and LoRA adapters; the SFT
  * state must outlive it.  After a full-parameter update call inference_state_refresh_from_sft. */

@@ -10,6 +10,7 @@
 #include "backend.h"
 #include "devutil.h"
 #include "../../include/inference_hip.h"
+#include "../../include/loader_hip.h"
 
 #include <fstream>
 #include <math.h>
@@ -382,6 +383,91 @@ InferenceState *inference_state_create_from_ref(const SFTModelRef *m, int max_se
     s->g_final = norm_upload(m->final_norm_g, m->d_model);
     s->emb = metal_buf_from_data(m->token_emb, (size_t)m->vocab_size * m->d_model * sizeof(float));
     s->owns_weights = 1;
+    return s;
+}
+
+// Straight from the file to HBM: every matrix is uploaded as stored and converted on the GPU (F16 and Q8_0 tensors that
+// already have the wanted format are used bit for bit); Q|K|V and gate|up are joined by device copies of whole rows.
+InferenceState *inference_state_create_from_file(const char *path, ModelType model_type, int max_seq_len, int use_fp16)
+{
+    ModelFile *f = model_file_open(path);
+    if (!f) return nullptr;
+    const bool gg = model_file_is_gguf(f);
+    if (gg && model_type == MODEL_GEMMA3) { fprintf(stderr, "[FastGen] Gemma3 is read from safetensors only\n"); model_file_close(f); return nullptr; }
+    auto lname = [&](int L, const char *hf, const char *g) {
+        char buf[256];
+        if (gg) snprintf(buf, sizeof buf, "blk.%d.%s.weight", L, g); else snprintf(buf, sizeof buf, "model.layers.%d.%s.weight", L, hf);
+        return std::string(buf);
+    };
+    const char *emb_name = gg ? "token_embd.weight" : "model.embed_tokens.weight";
+    int V = 0, D = 0, NL = 0, qd = 0, kd = 0, IS = 0, hd = 0, one = 0, c = 0;
+    bool ok = model_file_matrix_shape(f, emb_name, &V, &D) != 0;
+    while (ok && model_file_find(f, lname(NL, "self_attn.q_proj", "attn_q").c_str(), nullptr, nullptr, nullptr)) NL++;
+    ok = ok && NL > 0 && model_file_matrix_shape(f, lname(0, "self_attn.q_proj", "attn_q").c_str(), &qd, &c) && c == D &&
+         model_file_matrix_shape(f, lname(0, "self_attn.k_proj", "attn_k").c_str(), &kd, &c) && c == D &&
+         model_file_matrix_shape(f, lname(0, "mlp.gate_proj", "ffn_gate").c_str(), &IS, &c) && c == D &&
+         model_file_matrix_shape(f, lname(0, "self_attn.q_norm", "attn_q_norm").c_str(), &one, &hd) && hd > 0 && qd % hd == 0 && kd % hd == 0;
+    if (!ok) { fprintf(stderr, "[FastGen] %s: embedding or layer 0 tensors missing or inconsistent\n", path); model_file_close(f); return nullptr; }
+    const bool gemma = model_type == MODEL_GEMMA3;
+    std::vector<float> thetas(NL);
+    for (int L = 0; L < NL; L++) thetas[L] = gemma ? ((L % 6) != 0 ? 1e4f : 1e6f) : 1e6f;   // src/nn/fast_sft.c:308-313
+    InferenceState *s = new_state(model_type, D, qd / hd, kd / hd, hd, IS, V, NL, max_seq_len, use_fp16, thetas.data());
+    if (!s) { model_file_close(f); return nullptr; }
+    s->owns_weights = 1;
+    auto gamma = [&](const std::string &name, int dim) -> MetalBuf * {
+        size_t n = 0;
+        float *g = model_file_load_f32(f, name.c_str(), &n);
+        if (!g || (int)n != dim) { free(g); ok = false; return nullptr; }
+        if (gemma) for (size_t i = 0; i < n; i++) g[i] += 1.0f;                            // src/nn/gemma3.c:259-278
+        MetalBuf *b = norm_upload(g, dim);
+        free(g);
+        return b;
+    };
+    auto matrix = [&](const std::string &name, int rows, int cols) -> WMat * {
+        WMat *w = model_file_load_wmat(f, name.c_str(), use_fp16);
+        if (!w || w->rows != rows || w->cols != cols) { fprintf(stderr, "[FastGen] %s: expected %d x %d\n", name.c_str(), rows, cols); wmat_free(w); ok = false; return nullptr; }
+        return w;
+    };
+    auto fuse = [&](std::initializer_list<WMat *> parts, int cols) {
+        int rows = 0;
+        for (WMat *w : parts) { if (!w) return WMat{nullptr, 0, 0, 0}; rows += w->rows; }
+        const size_t row_bytes = use_fp16 ? (size_t)cols * 2 : (size_t)(cols / 32) * 34;
+        WMat out{metal_buf_create((size_t)rows * row_bytes), rows, cols, use_fp16 ? 0 : cols / 32};
+        size_t o = 0;
+        for (WMat *w : parts) {
+            HIP_CHECK(hipMemcpyAsync((char *)dptr(out.mbuf) + o, dptr(w->mbuf), (size_t)w->rows * row_bytes, hipMemcpyDeviceToDevice, stream()));
+            o += (size_t)w->rows * row_bytes;
+        }
+        mark_written(out.mbuf);
+        for (WMat *w : parts) wmat_free(w);                                                // synchronises the stream first
+        return out;
+    };
+    for (int L = 0; L < NL && ok; L++) {
+        InferenceState::Layer &lw = s->layers[L];
+        lw.g_in = gamma(lname(L, "input_layernorm", "attn_norm"), D);
+        lw.qkv = fuse({matrix(lname(L, "self_attn.q_proj", "attn_q"), qd, D), matrix(lname(L, "self_attn.k_proj", "attn_k"), kd, D),
+                       matrix(lname(L, "self_attn.v_proj", "attn_v"), kd, D)}, D);
+        lw.g_q = gamma(lname(L, "self_attn.q_norm", "attn_q_norm"), hd);
+        lw.g_k = gamma(lname(L, "self_attn.k_norm", "attn_k_norm"), hd);
+        lw.o = matrix(lname(L, "self_attn.o_proj", "attn_output"), D, qd);
+        lw.g_post_attn = gamma(lname(L, "post_attention_layernorm", "ffn_norm"), D);
+        if (gemma) lw.g_pre_ff = gamma(lname(L, "pre_feedforward_layernorm", ""), D);
+        lw.gu = fuse({matrix(lname(L, "mlp.gate_proj", "ffn_gate"), IS, D), matrix(lname(L, "mlp.up_proj", "ffn_up"), IS, D)}, D);
+        lw.down = matrix(lname(L, "mlp.down_proj", "ffn_down"), D, IS);
+        if (gemma) lw.g_post_ff = gamma(lname(L, "post_feedforward_layernorm", ""), D);
+    }
+    if (ok) {
+        s->g_final = gamma(gg ? "output_norm.weight" : "model.norm.weight", D);
+        const char *head = gg ? "output.weight" : "lm_head.weight";
+        const bool tied = gemma || !model_file_find(f, head, nullptr, nullptr, nullptr);   // src/nn/qwen3.c:264-270, 363-367
+        s->lm_head = matrix(tied ? emb_name : head, V, D);
+        size_t n = 0;
+        float *emb = model_file_load_f32(f, emb_name, &n);
+        if (emb && n == (size_t)V * D) s->emb = metal_buf_from_data(emb, n * sizeof(float)); else ok = false;
+        free(emb);
+    }
+    model_file_close(f);
+    if (!ok) { fprintf(stderr, "[FastGen] %s: a tensor is missing or mis-shaped\n", path); inference_state_free(s); return nullptr; }
     return s;
 }
 

@@ -144,7 +144,16 @@ def load():
         "inference_state_reset": (None, [vp]), "inference_forward_token": (C.POINTER(C.c_float), [vp, i]),
         "inference_forward_token_argmax": (i, [vp, i]), "inference_state_set_lora": (None, [vp, vp]),
         "inference_state_set_eos": (None, [vp, vp, i]), "inference_state_load_eos": (None, [vp, C.c_char_p]),
-        "inference_state_position": (i, [vp]), "sft_get_final_norm_g": (vp, [vp]),
+        "inference_state_position": (i, [vp]),
+        "inference_state_create_from_file": (vp, [C.c_char_p, i, i, i]),
+        "model_file_open": (vp, [C.c_char_p]), "model_file_close": (None, [vp]), "model_file_is_gguf": (i, [vp]),
+        "model_file_count": (i, [vp]), "model_file_name": (C.c_char_p, [vp, i]),
+        "model_file_find": (i, [vp, C.c_char_p, C.POINTER(i), C.POINTER(i), C.POINTER(C.c_uint64)]),
+        "model_file_matrix_shape": (i, [vp, C.c_char_p, C.POINTER(i), C.POINTER(i)]),
+        "model_file_data": (vp, [vp, C.c_char_p, C.POINTER(sz)]),
+        "model_file_load_f32": (vp, [vp, C.c_char_p, C.POINTER(sz)]),
+        "model_file_load_wmat": (C.POINTER(WMat), [vp, C.c_char_p, i]),
+        "model_ref_load": (C.POINTER(SFTModelRef), [C.c_char_p, i]), "model_ref_free": (None, [C.POINTER(SFTModelRef)]), "sft_get_final_norm_g": (vp, [vp]),
         "sft_get_layers": (C.POINTER(LayerW), [vp]), "sft_get_lm_head": (C.POINTER(WMat), [vp]),
         "sft_backward_sgd": (None, [vp, f]), "sft_alloc_grad_accum": (None, [vp]), "sft_backward_accum": (None, [vp]),
         "sft_apply_grad_sgd": (None, [vp, f]), "sft_save_full_checkpoint": (None, [vp, C.c_char_p]),

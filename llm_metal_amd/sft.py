@@ -237,9 +237,13 @@ class SFTState:
 class InferenceState:
     """inference_state_create_from_ref / _from_sft ... inference_state_free (include/inference_hip.h)."""
 
-    def __init__(self, c: SFTConfig = None, model=None, max_seq=256, use_fp16=True, sft: "SFTState" = None):
+    def __init__(self, c: SFTConfig = None, model=None, max_seq=256, use_fp16=True, sft: "SFTState" = None, path=None,
+                 model_type=0):
         self.L = _lib.load()
-        if sft is not None:
+        if path is not None:                               # inference_state_create_from_file
+            self.c, self._keep = c, []
+            self.h = self.L.inference_state_create_from_file(str(path).encode(), model_type, max_seq, 1 if use_fp16 else 0)
+        elif sft is not None:
             self.c, self._keep = sft.c, [sft]
             self.h = self.L.inference_state_create_from_sft(sft.h, max_seq)
         else:

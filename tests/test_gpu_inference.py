@@ -109,3 +109,117 @@ def test_state_sharing_weights_and_adapters_with_sft(cfg):
             got2 = np.stack([inf.forward_token(t) for t in toks])
             assert maxrel(got2, ref2) < 2e-4
             assert maxrel(got2, got) > 1e-4
+
+
+# ---------------------------------------------------------------- checkpoint files (include/loader_hip.h)
+
+def _as_used(model, conv):
+    m = dict(model)
+    for k in ("wq", "wk", "wv", "wo", "wg", "wu", "wd"):
+        m[k] = [conv(w) for w in model[k]]
+    return m
+
+
+def test_weights_from_files_are_bit_exact_in_every_format_pair(tmp_path):
+    import ctypes as C
+    from llm_metal_amd.sft import Backend, Buf
+    from oracle import oracle
+    from tests import model_files as mf
+    rng = np.random.default_rng(21)
+    w = (rng.standard_normal((48, 96)) * 0.05).astype(F)
+    wb = mf.bf16_round(w)
+    mf.write_safetensors(tmp_path / "t.safetensors", {"f32": (w, "F32"), "f16": (w, "F16"), "bf16": (wb, "BF16")})
+    mf.write_gguf(tmp_path / "t.gguf", {"q8": (w, mf.GGML_Q8_0), "f16": (w, mf.GGML_F16), "f32": (w, mf.GGML_F32)})
+    h16 = w.astype(np.float16)
+    blocks = oracle.q8_quantize(w)
+    deq = oracle.q8_dequant(blocks, 48, 96)
+    want = {("f32", 1): h16.tobytes(), ("f16", 1): h16.tobytes(), ("bf16", 1): wb.astype(np.float16).tobytes(),
+            ("f32", 0): blocks.tobytes(), ("f16", 0): oracle.q8_quantize(h16.astype(F)).tobytes(),
+            ("bf16", 0): oracle.q8_quantize(wb).tobytes(), ("q8", 0): blocks.tobytes(), ("q8", 1): deq.astype(np.float16).tobytes()}
+    with Backend() as be:
+        for fname, names in (("t.safetensors", ("f32", "f16", "bf16")), ("t.gguf", ("q8", "f16", "f32"))):
+            fh = be.L.model_file_open(str(tmp_path / fname).encode())
+            assert fh
+            for name in names:
+                for use_fp16 in (1, 0):
+                    wm = be.L.model_file_load_wmat(fh, name.encode(), use_fp16)
+                    assert wm and (wm.contents.rows, wm.contents.cols) == (48, 96)
+                    nbytes = 48 * 96 * 2 if use_fp16 else 48 * 3 * 34
+                    got = Buf(be.L, wm.contents.mbuf, nbytes, owned=False).read(np.uint8).tobytes()
+                    assert got == want[(name, use_fp16)], (fname, name, use_fp16)
+                    be.L.wmat_free(wm)
+            be.L.model_file_close(fh)
+
+
+@pytest.mark.parametrize("case", ["qwen_bf16_to_f16", "qwen_gguf_q8_as_is", "qwen_gguf_q8_to_f16", "gemma_f16_to_q8"])
+def test_generation_state_straight_from_a_checkpoint_file(case, tmp_path):
+    from oracle import oracle
+    from tests import model_files as mf
+    say("inference from file", case)
+    gemma = case.startswith("gemma")
+    c = TINY_GEMMA if gemma else C1.with_(seq=6, tied=case != "qwen_bf16_to_f16")
+    model = make_model(c, seed=13, gamma_jitter=0.1)
+    if gemma:
+        for k in ("g_in", "g_post_attn", "g_pre_ff", "g_post_ff", "g_q", "g_k"):
+            model[k] = [((g - F(1)).astype(F) + F(1)).astype(F) for g in model[k]]
+        model["g_final"] = ((model["g_final"] - F(1)).astype(F) + F(1)).astype(F)
+    tied = model["lm_head"] is model["token_emb"]
+    if case == "qwen_bf16_to_f16":
+        model = _as_used(model, mf.bf16_round)
+        model["token_emb"], model["lm_head"] = mf.bf16_round(model["token_emb"]), mf.bf16_round(model["lm_head"])
+        t = mf.model_tensors(c, model)
+        path = tmp_path / "m.safetensors"
+        mf.write_safetensors(path, {n: (a, "BF16" if a.ndim == 2 else "F32") for n, a in t.items()})
+        used, fmt, fp16 = model, "f16", True
+    elif case.startswith("qwen_gguf"):
+        emb16 = model["token_emb"].astype(np.float16).astype(F)                # the file stores the table as F16
+        model["token_emb"] = model["lm_head"] = emb16
+        t = mf.model_tensors(c, model, gguf=True)
+        path = tmp_path / "m.gguf"
+        mf.write_gguf(path, {n: (a, mf.GGML_F32 if a.ndim == 1 else mf.GGML_F16 if n == "token_embd.weight" else mf.GGML_Q8_0)
+                             for n, a in t.items()}, kv=mf.SAMPLE_KV)
+        if case == "qwen_gguf_q8_as_is":
+            used, fmt, fp16 = model, "q8_0", False                             # the oracle quantises the same fp32 values
+        else:
+            used = _as_used(model, lambda w: oracle.q8_dequant(oracle.q8_quantize(w), *w.shape))
+            used["token_emb"] = used["lm_head"] = emb16
+            fmt, fp16 = "f16", True
+    else:
+        model = _as_used(model, lambda w: w.astype(np.float16).astype(F))
+        model["token_emb"] = model["lm_head"] = model["token_emb"].astype(np.float16).astype(F)
+        t = mf.model_tensors(c, model)
+        path = tmp_path / "g.safetensors"
+        mf.write_safetensors(path, {n: (a, "F16" if a.ndim == 2 else "F32") for n, a in t.items()})
+        used, fmt, fp16 = model, "q8_0", False
+    assert tied == (used["lm_head"] is used["token_emb"])
+    tok, _ = make_batch(c, seed=14)
+    toks = [int(x) for x in tok]
+    ref = oracle_decode(c, used, fmt, toks, max_seq=16, precision="f32")
+    with InferenceState(c, path=path, model_type=c.model_type, max_seq=16, use_fp16=fp16) as inf:
+        assert inf.V == c.V
+        got = np.stack([inf.forward_token(x) for x in toks])
+        assert maxrel(got, ref) < 2e-4
+
+
+def test_sft_state_from_a_loaded_model_description(tmp_path):
+    import ctypes as C
+    from llm_metal_amd import lib as _lib
+    from tests import model_files as mf
+    c = C1.with_(seq=16)
+    model = make_model(c, seed=15, gamma_jitter=0.1)
+    t = mf.model_tensors(c, model)
+    mf.write_safetensors(tmp_path / "m.safetensors", {n: (a, "F32") for n, a in t.items()})
+    tok, tgt = make_batch(c, seed=16)
+    with SFTState(c, model) as a:
+        la = a.train_step(tok, tgt, 1e-3)
+    L = _lib.load()
+    ref = L.model_ref_load(str(tmp_path / "m.safetensors").encode(), 0)
+    assert ref
+    lora = np.ascontiguousarray(model["lora"], F)
+    ref.contents.lora_init = lora.ctypes.data
+    h = L.sft_state_create_from_ref(ref, c.batch, c.seq, c.R, c.alpha, 1)
+    assert h
+    lb = float(L.sft_train_step(h, np.ascontiguousarray(tok, np.uint32).ctypes.data, np.ascontiguousarray(tgt, np.uint32).ctypes.data, 1e-3))
+    L.sft_state_free(h)
+    L.model_ref_free(ref)
+    assert la == lb                                                            # the same weights, the same arithmetic
