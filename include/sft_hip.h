@@ -154,6 +154,9 @@ typedef struct {
 void grpo_apply_completions(SFTState *state, const GRPOCompletions *c, float lr, float *new_logprobs);
 /* "LORA" adapter file, src/nn/fast_sft.c:1255-1285 */
 void sft_save_lora(SFTState *state, const char *path);
+/* the reverse (qwen3_load_lora, src/nn/qwen3.c:558-602, applied to the state): 0, or -1 with a message when the file is
+ * unreadable, has another magic, layer count or rank, or is truncated (the state is then unchanged) */
+int sft_load_lora(SFTState *state, const char *path);
 
 /* Extensions: bulk copies that leave the adapters in HBM (flat layout as lora_init). */
 size_t sft_lora_numel(SFTState *state);

@@ -1080,4 +1080,27 @@ void sft_save_lora(SFTState *s, const char *path)
     fclose(f);
 }
 
+// qwen3_load_lora (src/nn/qwen3.c:558-602) for the SFT state: the file sft_save_lora writes (magic "LORA", layers,
+// rank, then A_q | B_q | A_v | B_v of every layer, fp32) becomes the state's adapters; optimiser moments are kept.
+int sft_load_lora(SFTState *s, const char *path)
+{
+    FILE *f = fopen(path, "rb");
+    if (!f) { fprintf(stderr, "[FastSFT] Cannot open %s for reading\n", path); return -1; }
+    uint32_t magic = 0;
+    int32_t nl = 0, rank = 0;
+    const bool head = fread(&magic, 4, 1, f) == 1 && fread(&nl, 4, 1, f) == 1 && fread(&rank, 4, 1, f) == 1;
+    if (!head || magic != 0x4C4F5241u) { fprintf(stderr, "[FastSFT] Invalid LoRA file magic\n"); fclose(f); return -1; }
+    if (nl != s->NL || rank != s->R) {
+        fprintf(stderr, "[FastSFT] LoRA config mismatch: file(layers=%d,rank=%d) vs state(layers=%d,rank=%d)\n", nl, rank, s->NL, s->R);
+        fclose(f);
+        return -1;
+    }
+    std::vector<float> w(s->lora_n);
+    const size_t got = fread(w.data(), 4, w.size(), f);
+    fclose(f);
+    if (got != w.size()) { fprintf(stderr, "[FastSFT] LoRA file %s is truncated\n", path); return -1; }
+    sft_set_lora(s, w.data());
+    return 0;
+}
+
 }  // extern "C"

@@ -133,7 +133,7 @@ def load():
         "sft_set_lora_grad": (None, [vp, i, vp, i]), "sft_get_lora_weight_buf": (vp, [vp, i, i]),
         "sft_get_lora_scaling": (f, [vp]), "sft_get_model_type": (i, [vp]), "sft_get_n_q_heads": (i, [vp]),
         "sft_get_n_kv_heads": (i, [vp]), "sft_get_head_dim": (i, [vp]), "sft_get_intermediate_size": (i, [vp]),
-        "sft_get_rope_thetas": (vp, [vp]), "sft_is_full_param": (i, [vp]), "sft_save_lora": (None, [vp, C.c_char_p]),
+        "sft_get_rope_thetas": (vp, [vp]), "sft_is_full_param": (i, [vp]), "sft_save_lora": (None, [vp, C.c_char_p]), "sft_load_lora": (i, [vp, C.c_char_p]),
         "sft_lora_numel": (sz, [vp]), "sft_copy_lora": (None, [vp, vp]), "sft_copy_lora_grads": (None, [vp, vp]),
         "sft_set_lora": (None, [vp, vp]), "sft_get_last_grad_norm": (f, [vp]),
         "sft_get_token_emb": (vp, [vp]), "sft_get_token_emb_buf": (vp, [vp]),
@@ -153,6 +153,9 @@ def load():
         "model_file_data": (vp, [vp, C.c_char_p, C.POINTER(sz)]),
         "model_file_load_f32": (vp, [vp, C.c_char_p, C.POINTER(sz)]),
         "model_file_load_wmat": (C.POINTER(WMat), [vp, C.c_char_p, i]),
+        "token_loader_open": (vp, [C.c_char_p, i, i]), "token_loader_free": (None, [vp]),
+        "token_loader_next": (i, [vp, vp, vp]), "token_loader_reset": (None, [vp]), "token_loader_shuffle": (None, [vp]),
+        "token_loader_n_batches": (sz, [vp]), "token_loader_n_tokens": (sz, [vp]), "token_loader_position": (sz, [vp]),
         "model_ref_load": (C.POINTER(SFTModelRef), [C.c_char_p, i]), "model_ref_free": (None, [C.POINTER(SFTModelRef)]), "sft_get_final_norm_g": (vp, [vp]),
         "sft_get_layers": (C.POINTER(LayerW), [vp]), "sft_get_lm_head": (C.POINTER(WMat), [vp]),
         "sft_backward_sgd": (None, [vp, f]), "sft_alloc_grad_accum": (None, [vp]), "sft_backward_accum": (None, [vp]),

@@ -177,3 +177,69 @@ def test_save_lora_file_format():
         assert (magic, nl, rank) == (0x4C4F5241, cfg.NL, cfg.R)
         body = np.frombuffer(raw[12:], dtype=np.float32)
         assert np.array_equal(body, model["lora"])
+
+
+def test_load_lora_restores_the_adapters_and_refuses_foreign_files(capfd):
+    cfg = C1
+    model = make_model(cfg, seed=10)
+    tok, tgt = make_batch(cfg, seed=11)
+    tmp = tempfile.mkdtemp()
+    path = os.path.join(tmp, "a.lora")
+    with SFTState(cfg, model) as st:
+        st.train_step(tok, tgt, 1e-2)
+        trained = st.lora()
+        st.L.sft_save_lora(st.h, path.encode())
+    other = make_model(cfg, seed=12)                       # other adapters, same frozen weights
+    other.update({k: model[k] for k in model if k != "lora"})
+    with SFTState(cfg, other) as st:
+        assert not np.array_equal(st.lora(), trained)
+        assert st.L.sft_load_lora(st.h, path.encode()) == 0
+        assert np.array_equal(st.lora(), trained)
+        loss_a = st.train_step(tok, tgt, 0.0)
+        # refused: absent, wrong magic, other rank, truncated; the adapters stay
+        raw = open(path, "rb").read()
+        cases = {"magic": b"XXXX" + raw[4:], "rank": raw[:8] + struct.pack("<i", 8) + raw[12:], "cut": raw[:-8]}
+        assert st.L.sft_load_lora(st.h, os.path.join(tmp, "absent").encode()) == -1
+        for name, data in cases.items():
+            p = os.path.join(tmp, name)
+            open(p, "wb").write(data)
+            assert st.L.sft_load_lora(st.h, p.encode()) == -1, name
+        assert np.array_equal(st.lora(), trained)
+    with SFTState(cfg, model) as st:                        # the state the file came from, one step later
+        st.train_step(tok, tgt, 1e-2)
+        loss_b = st.train_step(tok, tgt, 0.0)
+    assert abs(loss_a - loss_b) < 1e-6
+    assert "mismatch" in capfd.readouterr().err
+
+
+def test_run_sft_driver_matches_the_library_driven_from_python(tmp_path):
+    """The C++ `--mode sft` driver: checkpoint file + adapter file + token file in, log lines and adapter file out."""
+    import subprocess
+    import sys
+    from tests import model_files as mf
+    cfg = C1.with_(seq=16)
+    model = make_model(cfg, seed=31, gamma_jitter=0.1)
+    mdir = tmp_path / "model"
+    mdir.mkdir()
+    mf.write_safetensors(mdir / "model.safetensors", {n: (a, "F32") for n, a in mf.model_tensors(cfg, model).items()})
+    (mdir / "config.json").write_text('{"model_type": "qwen3", "eos_token_id": 3}')
+    rng = np.random.default_rng(32)
+    ids = rng.integers(0, cfg.V, 16 * 3 + 1).astype(np.int32)
+    ids.tofile(tmp_path / "train.bin")
+    adapter = tmp_path / "adapter.bin"
+    losses = []
+    with SFTState(cfg, model) as st:
+        st.L.sft_save_lora(st.h, str(adapter).encode())
+        for k in range(3):
+            losses.append(st.train_step(ids[16 * k:16 * k + 16].astype(np.uint32), ids[16 * k + 1:16 * k + 17].astype(np.uint32), 1e-3))
+        want = st.lora()
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "llm_metal_amd", "run_sft_hip")
+    print("run_sft_hip", flush=True, file=sys.stderr)
+    out = subprocess.run([exe, "--mode", "sft", "--model", str(mdir), "--train", str(tmp_path / "train.bin"), "--seq", "16",
+                          "--steps", "3", "--lr", "1e-3", "--lora-adapter", str(adapter)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert "=== Qwen3 Fast LoRA SFT ===" in out.stdout and "Detected model_type: qwen3" in out.stdout
+    got = [float(line.split("|")[1].split()[1]) for line in out.stdout.splitlines() if line.startswith("step")]
+    assert len(got) == 3 and np.allclose(got, losses, atol=6e-5)                 # printed with four decimals
+    raw = open(adapter, "rb").read()
+    assert np.array_equal(np.frombuffer(raw[12:], np.float32), want)             # the same three updates
