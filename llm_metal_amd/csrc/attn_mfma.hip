@@ -1,5 +1,8 @@
-// Causal GQA attention, forward and backward, on the fp32 matrix cores
-// (v_mfma_f32_32x32x2_f32: operands are not rounded).  Same arithmetic as
+// Causal GQA attention, forward and backward, on the matrix cores.  Every fp32 operand enters as two bf16 values,
+// x = hi + lo (hi the upper 16 bits of x, lo those of x - hi), and a product is three v_mfma_f32_32x32x16_bf16:
+// hi*hi + lo*hi + hi*lo, accumulated in fp32.  That keeps 16 mantissa bits and the whole fp32 exponent range of
+// every operand (gradients of 1e-7 do not underflow as they would in fp16) at a fifth of the matrix-core time of
+// the fp32 instruction (v_mfma_f32_32x32x2_f32, 64 cycles for 2 reduction steps).  Same arithmetic as
 // attn_train_fwd / attn_bwd_dq / attn_bwd_dkv / repeat_kv_bwd of
 // shaders/q8_kernels.metal:769-992, on [rows][H*hd] activations with the KV head
 // picked as h / ratio; the probabilities are saved for the backward as the
@@ -33,58 +36,91 @@ __device__ __forceinline__ float16v zero16()
 // they are added when the tile is complete.
 struct Acc2 { float16v a, b; };
 
-// One 32 x 32 product tile A[32, HD] (LDS, row stride lda) * Bm[32 rows, HD]^T.  The reduction index is split
-// between the lane halves (lanes 0-31 take columns [0, HD/2), lanes 32-63 the rest), so a lane needs one
-// half row of its B row: a BTile, HD/2 floats per lane, read straight from memory a whole tile
-// (64 MFMAs at HD = 128, about 2 us) ahead of its use.  The A values come from LDS, 32 floats at a time, one
-// such chunk ahead.
-template <int HD> struct BTile { float4 v[HD / 8]; };
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// upper halves of two floats in one dword: (lo16 = bf16 of a, hi16 = bf16 of b), truncating
+__device__ __forceinline__ uint32_t pack_hi(float a, float b) { return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u); }
+// what the truncation to bf16 leaves behind (exact in fp32)
+__device__ __forceinline__ float rest(float a) { return a - __uint_as_float(__float_as_uint(a) & 0xffff0000u); }
+
+// eight consecutive reduction values of a lane as matrix-core operands
+struct HL { bf16x8 hi, lo; };
+__device__ __forceinline__ HL split8(const float (&x)[8])
+{
+    u32x4 h, l;
+#pragma unroll
+    for (int i = 0; i < 4; i++) { h[i] = pack_hi(x[2 * i], x[2 * i + 1]); l[i] = pack_hi(rest(x[2 * i]), rest(x[2 * i + 1])); }
+    return HL{__builtin_bit_cast(bf16x8, h), __builtin_bit_cast(bf16x8, l)};
+}
+__device__ __forceinline__ HL split8(const float4 &p, const float4 &q)
+{
+    const float x[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+    return split8(x);
+}
+// acc += a b over 16 reduction steps (first operand: rows of the result, second: its columns)
+__device__ __forceinline__ void mfma3(float16v &acc, const HL &a, const HL &b)
+{
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.hi, b.hi, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.lo, b.hi, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.hi, b.lo, acc, 0, 0, 0);
+}
+
+// A 32 x 32 product tile A[32, HD] * Bm[32 rows, HD]^T is formed CB columns of the head at a time (CB = HD up to 128;
+// two passes at HD = 256, which keeps the B operands of a pass within 64 registers).  Within a pass the reduction
+// index is split between the lane halves (lanes 0-31 take the first CB/2 columns, lanes 32-63 the rest), so a lane
+// needs CB/2 floats of its B row: a BTile, read straight from memory a whole pass ahead of its use and split into
+// bf16 pairs here.  The A rows sit in LDS already split (Ahi / Alo, bf16, row stride lda halves): 16 bytes of each
+// per instruction.
+template <int CB> struct BTile { float4 v[CB / 8]; };
 
 // The values come from a copy of the head's matrix laid out as BT[HD/4][ldt][4] (group of four columns, key, column
 // in the group; ldt = attn_ldt(seq)): a lane still reads 16 bytes at a time, but the 32 lanes of a half wave read
-// 512 contiguous bytes, where the rows themselves (4 KB apart) would cost one cache line per lane and instruction
-// and keep the memory pipeline busy for as long as the MFMAs run.
-template <int HD>
-__device__ __forceinline__ void b_tile_load(BTile<HD> &t, const float *bt_lane, int ldt)
+// 512 contiguous bytes, where the rows themselves (4 KB apart) would cost one cache line per lane and instruction.
+template <int CB>
+__device__ __forceinline__ void b_tile_load(BTile<CB> &t, const float *bt_lane, int ldt)
 {
 #pragma unroll
-    for (int i = 0; i < HD / 8; i++) t.v[i] = ld4(bt_lane + (size_t)i * ldt * 4);
+    for (int i = 0; i < CB / 8; i++) t.v[i] = ld4(bt_lane + (size_t)i * ldt * 4);
 }
 
-template <int HD>
-__device__ __forceinline__ float16v tile_abt(const float *As, int lda, int lane, const BTile<HD> &bt)
+// acc += A[:, col0 .. col0 + CB) * B-pass^T
+template <int CB>
+__device__ __forceinline__ void tile_abt(Acc2 &acc, const __bf16 *Ahi, const __bf16 *Alo, int lda, int col0, int lane, const BTile<CB> &bt)
 {
-    constexpr int HALF = HD / 2, CH = HALF < 32 ? HALF : 32, NCH = HALF / CH;
-    const float *a = As + (lane & 31) * lda + (lane >> 5) * HALF;
-    Acc2 acc{zero16(), zero16()};
-    float4 abuf[2][CH / 4];
+    constexpr int HALF = CB / 2, NT = HALF / 8;              // instruction triples per pass
+    constexpr int CT = NT < 4 ? NT : 4, NC = NT / CT;        // A operands are fetched CT triples at a time, one group ahead
+    const size_t off = (size_t)(lane & 31) * lda + col0 + (lane >> 5) * HALF;
+    HL a[2][CT];
+    auto fetch = [&](int buf, int c) __attribute__((always_inline)) {
 #pragma unroll
-    for (int t = 0; t < CH / 4; t++) abuf[0][t] = *reinterpret_cast<const float4 *>(a + 4 * t);     // LDS, 16-byte aligned
-#pragma unroll
-    for (int ci = 0; ci < NCH; ci++) {
-        if (ci + 1 < NCH) {
-#pragma unroll
-            for (int t = 0; t < CH / 4; t++) abuf[(ci + 1) & 1][t] = *reinterpret_cast<const float4 *>(a + (ci + 1) * CH + 4 * t);
+        for (int t = 0; t < CT; t++) {                       // LDS, 16-byte aligned
+            a[buf][t].hi = *reinterpret_cast<const bf16x8 *>(Ahi + off + 8 * (c * CT + t));
+            a[buf][t].lo = *reinterpret_cast<const bf16x8 *>(Alo + off + 8 * (c * CT + t));
         }
+    };
+    fetch(0, 0);
 #pragma unroll
-        for (int t = 0; t < CH / 4; t++) {
-            const float4 x = abuf[ci & 1][t], c = bt.v[ci * (CH / 4) + t];
-            acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, c.x, acc.a, 0, 0, 0);
-            acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, c.y, acc.b, 0, 0, 0);
-            acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, c.z, acc.a, 0, 0, 0);
-            acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, c.w, acc.b, 0, 0, 0);
+    for (int c = 0; c < NC; c++) {
+        if (c + 1 < NC) fetch((c + 1) & 1, c + 1);
+#pragma unroll
+        for (int t = 0; t < CT; t++) {
+            const int tt = c * CT + t;
+            const HL b = split8(bt.v[2 * tt], bt.v[2 * tt + 1]);
+            mfma3((t & 1) ? acc.b : acc.a, a[c & 1][t], b);
         }
     }
-    return acc.a + acc.b;
 }
 
-// One 32 x 32 product tile X[32, nk] (LDS, row stride ldx) * C[nk rows, 32 columns], C row-major with row stride ldc;
-// rows beyond n_valid are read as row n_valid - 1 (their X column is zero).  Inside a chunk of 32 keys lanes 0-31
-// take keys 0-15 and lanes 32-63 keys 16-31, so a lane reads 16 consecutive X values (four 16-byte LDS reads) and
-// 16 rows of C.  Both are requested one chunk ahead, unconditionally (past the end the last chunk is read again);
-// `first` holds chunk 0 of C.
+// One 32 x 32 product tile X[32, nk] * C[nk rows, 32 columns], C row-major with row stride ldc; rows beyond n_valid
+// are read as row n_valid - 1 (their X column is zero).  X sits in LDS split into bf16 pairs: row r holds the upper
+// parts of its nk values at Xh + r * ldxh (halves), the lower parts xlo halves further on.  Inside a chunk of 32 keys
+// lanes 0-31 take keys 0-15 and lanes 32-63 keys 16-31 (instruction u of the chunk reduces over keys 16 hh + 8 u +
+// 0..7), so a lane reads 16 consecutive X values (two 16-byte LDS reads for each part) and 16 rows of C.  Both are
+// requested ahead, unconditionally (past the end the last chunk is read again); `first` holds chunk 0 of C.
 struct CChunk { float v[16]; };
-struct XChunk { float4 v[4]; };
+struct XChunk { bf16x8 hi[2], lo[2]; };
 
 __device__ __forceinline__ void c_chunk_load(CChunk &c, const float *ccol_lane, size_t ldc, int k0, int hh, int n_valid)
 {
@@ -92,25 +128,26 @@ __device__ __forceinline__ void c_chunk_load(CChunk &c, const float *ccol_lane, 
     for (int t = 0; t < 16; t++) c.v[t] = ccol_lane[(size_t)min(k0 + 16 * hh + t, n_valid - 1) * ldc];
 }
 
-__device__ __forceinline__ void x_chunk_load(XChunk &c, const float *x_row_half, int k0)
+__device__ __forceinline__ void x_chunk_load(XChunk &c, const __bf16 *x_row_half, int xlo, int k0)
 {
 #pragma unroll
-    for (int t = 0; t < 4; t++) c.v[t] = *reinterpret_cast<const float4 *>(x_row_half + k0 + 4 * t);
+    for (int u = 0; u < 2; u++) {
+        c.hi[u] = *reinterpret_cast<const bf16x8 *>(x_row_half + k0 + 8 * u);
+        c.lo[u] = *reinterpret_cast<const bf16x8 *>(x_row_half + xlo + k0 + 8 * u);
+    }
 }
 
 __device__ __forceinline__ void c_chunk_mfma(Acc2 &acc, const XChunk &x, const CChunk &c)
 {
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-        acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].x, c.v[4 * t + 0], acc.a, 0, 0, 0);
-        acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].y, c.v[4 * t + 1], acc.b, 0, 0, 0);
-        acc.a = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].z, c.v[4 * t + 2], acc.a, 0, 0, 0);
-        acc.b = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t].w, c.v[4 * t + 3], acc.b, 0, 0, 0);
+    for (int u = 0; u < 2; u++) {
+        const float cv[8] = {c.v[8 * u], c.v[8 * u + 1], c.v[8 * u + 2], c.v[8 * u + 3], c.v[8 * u + 4], c.v[8 * u + 5], c.v[8 * u + 6], c.v[8 * u + 7]};
+        mfma3(u ? acc.b : acc.a, HL{x.hi[u], x.lo[u]}, split8(cv));
     }
 }
 
-// The C chunks travel in a ring of four (chunk q in slot q % 4), requested three chunks (about 1.4 us of MFMAs)
-// ahead; on entry slots 0-2 hold chunks 0-2, which the caller may have requested long before.
+// The C chunks travel in a ring of four (chunk q in slot q % 4), requested three chunks ahead; on entry slots 0-2 hold
+// chunks 0-2, which the caller may have requested long before.
 struct CRing { CChunk c[4]; };
 
 __device__ __forceinline__ void c_ring_start(CRing &r, const float *ccol_lane, size_t ldc, int nk, int hh, int n_valid)
@@ -119,20 +156,20 @@ __device__ __forceinline__ void c_ring_start(CRing &r, const float *ccol_lane, s
     for (int q = 0; q < 3; q++) c_chunk_load(r.c[q], ccol_lane, ldc, min(32 * q, nk - 32), hh, n_valid);
 }
 
-__device__ __forceinline__ float16v tile_xc(const float *Xs, int ldx, int nk, const float *ccol_lane, size_t ldc, int n_valid, int lane,
-                                            CRing &ring)
+__device__ __forceinline__ float16v tile_xc(const __bf16 *Xh, int ldxh, int xlo, int nk, const float *ccol_lane, size_t ldc, int n_valid,
+                                            int lane, CRing &ring)
 {
     const int hh = lane >> 5;
-    const float *x = Xs + (lane & 31) * ldx + 16 * hh;
+    const __bf16 *x = Xh + (size_t)(lane & 31) * ldxh + 16 * hh;
     Acc2 acc{zero16(), zero16()};
     XChunk xr[2];
-    x_chunk_load(xr[0], x, 0);
+    x_chunk_load(xr[0], x, xlo, 0);
     for (int k0 = 0; k0 < nk; k0 += 128) {                // nk is a multiple of 32
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int kc = k0 + 32 * u;
             c_chunk_load(ring.c[(u + 3) & 3], ccol_lane, ldc, min(kc + 96, nk - 32), hh, n_valid);
-            x_chunk_load(xr[(u + 1) & 1], x, min(kc + 32, nk - 32));
+            x_chunk_load(xr[(u + 1) & 1], x, xlo, min(kc + 32, nk - 32));
             if (kc < nk) c_chunk_mfma(acc, xr[u & 1], ring.c[u]);
         }
     }
@@ -154,10 +191,12 @@ struct AttnTileArgs {
 
 // Row step: eight threads per row, thread `part` owns the keys 32 m + 4 part + (0..3) for m < M32 and keeps them in
 // registers, so every LDS and memory access is a 16-byte one (eight threads cover 128 contiguous bytes) and the
-// row reductions need three shuffles.  The finished rows go back to LDS for phase 3 and, whole (zeros right of the
-// diagonal, out to column N), to memory.
+// row reductions need three shuffles.  The finished rows go to memory whole (fp32, zeros right of the diagonal, out to
+// column N) and back to LDS for phase 3 as bf16 pairs, in place: the upper parts of keys 0.. at the start of the
+// row, the lower parts xlo halves further on.  A row belongs to eight lanes of one wave, which have read all of it
+// before they write.
 template <int BWD, int M32>
-__device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int nk, int N, int i0, int b, int h, int tid)
+__device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int xlo, int nk, int N, int i0, int b, int h, int tid)
 {
     const int rr = tid >> 3, part = tid & 7, i = i0 + rr;
     const bool row_ok = i < N;
@@ -207,7 +246,11 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
         if (BWD) o = make_float4(p[m].x * (v[m].x - red) * a.scale, p[m].y * (v[m].y - red) * a.scale,
                                  p[m].z * (v[m].z - red) * a.scale, p[m].w * (v[m].w - red) * a.scale);
         else o = make_float4(v[m].x * inv, v[m].y * inv, v[m].z * inv, v[m].w * inv);
-        if (j < nk) *reinterpret_cast<float4 *>(xr + 32 * m) = o;
+        if (j < nk) {
+            __bf16 *xh = reinterpret_cast<__bf16 *>(Xs + rr * ldx) + j;
+            *reinterpret_cast<u32x2 *>(xh) = u32x2{pack_hi(o.x, o.y), pack_hi(o.z, o.w)};
+            *reinterpret_cast<u32x2 *>(xh + xlo) = u32x2{pack_hi(rest(o.x), rest(o.y)), pack_hi(rest(o.z), rest(o.w))};
+        }
         if (row_ok && j < N) {
             if ((N & 3) == 0) *reinterpret_cast<float4 *>(gdst + 32 * m) = o;
             else { const float *q = &o.x; for (int c = 0; c < 4; c++) if (j + c < N) gdst[32 * m + c] = q[c]; }
@@ -215,12 +258,12 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
     }
 }
 
-// grid (query blocks of 32, Hq, batch), block 256; LDS: As[32][HD+4], Xs[32][ldx]
+// grid (query blocks of 32, Hq, batch), block 256; LDS: Ahi, Alo [32][HD+8] bf16, Xs[32][ldx] fp32 / bf16 pairs
 template <int BWD, int HD>
 __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
 {
     extern __shared__ float lds[];
-    constexpr int lda = HD + 4, half = HD / 2;            // rows 16-byte aligned; 132 floats apart: conflict-free 16-byte reads
+    constexpr int lda = HD + 8, half = HD / 2;            // halves; rows 16-byte aligned and 4 banks apart: conflict-free 16-byte reads
     const int N = a.seq;
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l31 = lane & 31, hh = lane >> 5;
@@ -228,17 +271,25 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     const size_t r0 = (size_t)b * N;
     const int i0 = qb * 32;
     const int nk = min(i0 + 32, (N + 31) & ~31);          // keys this block can see, rounded up to 32
-    const int ldx = ((N + 31) & ~31) + 4;
-    float *As = lds, *Xs = As + 32 * lda;
+    const int N32 = (N + 31) & ~31, ldx = N32 + 4;
+    __bf16 *Ahi = reinterpret_cast<__bf16 *>(lds), *Alo = Ahi + 32 * lda;
+    float *Xs = lds + 32 * lda;                           // behind the two bf16 images of A
 
-    // ---- the first B tile and the first C chunk of this wave do not depend on anything computed here:
+    // ---- the first B pass and the first C chunk of this wave do not depend on anything computed here:
     //      request them before the A rows are staged (waves without a tile of their own read tile 0)
-    // this lane's column of the transposed B matrix: key jb * 32 + l31, rows hh * half ...
+    // Work items of a wave in phase 1: (key block jb = wave + 4 (q / NCB), column pass c = q % NCB), q = 0 .. nitems - 1.
+    // This lane's part of the transposed B matrix for an item: key jb * 32 + l31, columns c * CB + hh * CB/2 ...
+    constexpr int CB = HD > 128 ? 128 : HD, NCB = HD / CB;
     const int ldt = attn_ldt(N);
-    auto b_row = [&](int jb) { return a.BT + ((((size_t)b * a.Hkv + hk) * (HD / 4) + hh * (half / 4)) * ldt + min(jb * 32 + l31, N - 1)) * 4; };
     const int nkb = nk >> 5;
-    BTile<HD> bt0, bt1;
-    b_tile_load<HD>(bt0, b_row(wave < nkb ? wave : 0), ldt);
+    const int nitems = wave < nkb ? ((nkb - wave + 3) >> 2) * NCB : 0;
+    auto b_item = [&](int q) {
+        const int qq = nitems ? min(q, nitems - 1) : 0;
+        const int jb = nitems ? wave + 4 * (qq / NCB) : 0, c = qq % NCB;
+        return a.BT + ((((size_t)b * a.Hkv + hk) * (HD / 4) + c * (CB / 4) + hh * (CB / 8)) * ldt + min(jb * 32 + l31, N - 1)) * 4;
+    };
+    BTile<CB> bt0, bt1;
+    b_tile_load<CB>(bt0, b_item(0), ldt);
     CRing cring;
     const float *c_lane0 = a.C + r0 * kd + hk * HD + l31;
     c_ring_start(cring, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, nk, hh, N);
@@ -256,36 +307,46 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
         for (int u = 0; u < HD / 32; u++) {
             const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
             if (BWD && i0 + rr < N) st4(a.A_out + (r0 + i0 + rr) * qd + h * HD + 4 * c4, av[u]);
-            *reinterpret_cast<float4 *>(As + rr * lda + 4 * c4) = av[u];
+            *reinterpret_cast<u32x2 *>(Ahi + rr * lda + 4 * c4) = u32x2{pack_hi(av[u].x, av[u].y), pack_hi(av[u].z, av[u].w)};
+            *reinterpret_cast<u32x2 *>(Alo + rr * lda + 4 * c4) = u32x2{pack_hi(rest(av[u].x), rest(av[u].y)), pack_hi(rest(av[u].z), rest(av[u].w))};
         }
     }
     __syncthreads();
 
-    // ---- phase 1: X = A B^T, one 32-key block per wave and round; the B rows of the block after it are on their way
+    // ---- phase 1: X = A B^T, one 32-key block per wave and round; the B values of the next item are on their way
     auto put_x = [&](const float16v &acc, int jb) {
 #pragma unroll
         for (int v = 0; v < 16; v++) Xs[(8 * (v >> 2) + 4 * hh + (v & 3)) * ldx + jb * 32 + l31] = acc[v];
     };
-    for (int jb = wave; jb < nkb; jb += 8) {
-        b_tile_load<HD>(bt1, b_row(jb + 4 < nkb ? jb + 4 : jb), ldt);
-        put_x(tile_abt<HD>(As, lda, lane, bt0), jb);
-        b_tile_load<HD>(bt0, b_row(jb + 8 < nkb ? jb + 8 : jb), ldt);
-        if (jb + 4 < nkb) put_x(tile_abt<HD>(As, lda, lane, bt1), jb + 4);
+    {
+        Acc2 acc{zero16(), zero16()};
+        auto run = [&](int q, const BTile<CB> &bt) __attribute__((always_inline)) {
+            const int jb = wave + 4 * (q / NCB), c = q % NCB;
+            if (c == 0) { acc.a = zero16(); acc.b = zero16(); }
+            tile_abt<CB>(acc, Ahi, Alo, lda, c * CB, lane, bt);
+            if (c == NCB - 1) put_x(acc.a + acc.b, jb);
+        };
+        for (int q = 0; q < nitems; q += 2) {
+            b_tile_load<CB>(bt1, b_item(q + 1), ldt);
+            run(q, bt0);
+            b_tile_load<CB>(bt0, b_item(q + 2), ldt);
+            if (q + 1 < nitems) run(q + 1, bt1);
+        }
     }
     __syncthreads();
 
     // ---- row step
-    if (N <= 64) row_step<BWD, 2>(a, Xs, ldx, nk, N, i0, b, h, tid);                 // whole rows of N entries are written
-    else if (N <= 256) row_step<BWD, 8>(a, Xs, ldx, nk, N, i0, b, h, tid);
-    else if (N <= 512) row_step<BWD, 16>(a, Xs, ldx, nk, N, i0, b, h, tid);
-    else row_step<BWD, 32>(a, Xs, ldx, nk, N, i0, b, h, tid);
+    if (N <= 64) row_step<BWD, 2>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);                 // whole rows of N entries are written
+    else if (N <= 256) row_step<BWD, 8>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);
+    else if (N <= 512) row_step<BWD, 16>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);
+    else row_step<BWD, 32>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);
     __syncthreads();
 
     // ---- phase 3: Y = X C, one 32-column block of the head per wave and round
     const int Kb = tiled_kb(qd);
     for (int dt = wave; dt * 32 < HD; dt += 4) {
         if (dt != wave) c_ring_start(cring, c_lane0 + dt * 32, (size_t)kd, nk, hh, N);
-        const float16v acc = tile_xc(Xs, ldx, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
+        const float16v acc = tile_xc(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
         const int d = dt * 32 + l31;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
@@ -330,24 +391,25 @@ __global__ __launch_bounds__(256) void k_attn_dkv_tile(AttnDkvArgs a)
         const float *S = a.dscore + ((size_t)b * a.Hq + hq) * N * N + j;
         const float *Q = a.q + r0 * qd + hq * hd + dt * 32 + l31;
         const float *O = a.dO + r0 * qd + hq * hd + dt * 32 + l31;
+        // lane half hh takes the query rows ib * 32 + 2 s + hh, s = 0..15; instruction u reduces over s = 8 u + 0..7
+        float pv[16], sv[16], qv[16], ov[16];
 #pragma unroll
-        for (int k0 = 0; k0 < 32; k0 += 8) {
-            float pv[4], sv[4], qv[4], ov[4];
+        for (int t = 0; t < 16; t++) {
+            const int i = ib * 32 + 2 * t + hh;
+            const int ic = min(i, N - 1);
+            const bool ok = i < N;
+            pv[t] = ok ? P[(size_t)ic * N] : 0.f;
+            sv[t] = ok ? S[(size_t)ic * N] : 0.f;
+            qv[t] = Q[(size_t)ic * qd];
+            ov[t] = O[(size_t)ic * qd];
+        }
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const int i = ib * 32 + k0 + 2 * t + hh;
-                const int ic = min(i, N - 1);
-                const bool ok = i < N;
-                pv[t] = ok ? P[(size_t)ic * N] : 0.f;
-                sv[t] = ok ? S[(size_t)ic * N] : 0.f;
-                qv[t] = Q[(size_t)ic * qd];
-                ov[t] = O[(size_t)ic * qd];
-            }
+        for (int u = 0; u < 2; u++) {
+            float x[4][8];
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                accV = __builtin_amdgcn_mfma_f32_32x32x2f32(pv[t], ov[t], accV, 0, 0, 0);
-                accK = __builtin_amdgcn_mfma_f32_32x32x2f32(sv[t], qv[t], accK, 0, 0, 0);
-            }
+            for (int e = 0; e < 8; e++) { x[0][e] = pv[8 * u + e]; x[1][e] = ov[8 * u + e]; x[2][e] = sv[8 * u + e]; x[3][e] = qv[8 * u + e]; }
+            mfma3(accV, split8(x[0]), split8(x[1]));
+            mfma3(accK, split8(x[2]), split8(x[3]));
         }
     }
     if (wave > 0) {
@@ -366,7 +428,7 @@ __global__ __launch_bounds__(256) void k_attn_dkv_tile(AttnDkvArgs a)
     }
 }
 
-size_t tile_lds_bytes(int hd, int seq) { return (size_t)32 * (hd + 4 + ((seq + 31) & ~31) + 4) * sizeof(float); }
+size_t tile_lds_bytes(int hd, int seq) { return (size_t)32 * (hd + 8 + ((seq + 31) & ~31) + 4) * sizeof(float); }
 
 template <int BWD, int HD>
 void launch_tile_hd(const AttnTileArgs &a)
