@@ -29,7 +29,7 @@ void die(const char *what, hipError_t e, const char *file, int line);
 
 // Grow-only device scratch, one arena per purpose; contents are only valid
 // within the enqueue that asked for them.
-enum ScratchSlot { SCR_A16 = 0, SCR_SCALE, SCR_PARTIAL, SCR_MISC, SCR_COUNT };
+enum ScratchSlot { SCR_A16 = 0, SCR_SCALE, SCR_PARTIAL, SCR_MISC, SCR_WF16, SCR_COUNT };   // SCR_WF16: F16 image of a Q8_0 weight
 void *scratch(ScratchSlot slot, size_t bytes);
 
 // Device address of a buffer; views resolve through their parent so that they

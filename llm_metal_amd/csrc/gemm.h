@@ -71,6 +71,8 @@ bool gemm_prof_begin(double wbytes, double flops, hipEvent_t *a, hipEvent_t *b);
 double weight_stream_bytes(const WeightOp &W, int N, int K);
 // C[m][n] (row stride ldc) = a_inv_scale[m] * sum_k A[m][k] W[n][k] in one launch of 128 x 128 output blocks staged
 // through LDS (gemm_big.hip): the path for M of several hundred rows and more, where the product is MFMA bound.
+// W as plain F16 tiles: itself when F16, else dequantised once into a scratch image that the next call overwrites
+WeightOp f16_image_of(const WeightOp &W, int N, int K);
 void launch_gemm_big(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K);
 // true when the large-M kernel is the faster one for this product
 bool use_big_gemm(int M, int N, int K, int fmt);

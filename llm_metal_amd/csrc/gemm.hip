@@ -100,6 +100,27 @@ __global__ void reduce_planes(const float *__restrict__ P, int S, size_t plane_s
     C[idx] = row_scale ? s * row_scale[m] : s;
 }
 
+// F16 tile image of a Q8_0 (or mixed Q8_0 / F16) weight operand: one wave per 32 x 64 tile loads the tile the way
+// the streaming GEMM does (codes unpacked and scaled in registers, F16 tiles as they are) and stores the four operand
+// vectors of every lane at the tile's place in a plain F16 operand, out[(nb * Kb + kt) * 256 + j * 64 + lane].
+__global__ __launch_bounds__(256) void q8_operand_to_f16(lmhip::WeightOp W, int Nb, int Kb, half8 *__restrict__ out)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t tile = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tile >= (size_t)Nb * Kb) return;
+    const int nb = (int)(tile / Kb), kt = (int)(tile % Kb);
+    half8 w[4];
+    if (W.fmt == 1) {
+        if (nb < W.nbq) lmhip::load_w_q8_rows(w, W, nb, Kb, kt, lane);
+        else lmhip::load_w_f16(w, W.w16, nb - W.nbq, Kb, kt, lane);
+    } else {
+        if (kt < W.kbq) lmhip::load_w_q8_cols(w, W, nb, W.kbq, kt, lane);
+        else lmhip::load_w_f16(w, W.w16, nb, Kb - W.kbq, kt - W.kbq, lane);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) out[tile * 256 + j * 64 + lane] = w[j];
+}
+
 // Row-major F16 [rows, cols] -> tiled layout, optionally transposed; 64x64 element tiles via LDS
 // so that both the reads (along cols) and the writes (16-byte groups along the destination K) coalesce.
 __global__ __launch_bounds__(256) void tile_f16(const half_t *__restrict__ src, int rows, int cols,
@@ -313,16 +334,33 @@ void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, in
 int gemm_profiling() { return g_prof_on; }
 
 // Which kernel multiplies an [M, K] activation block with an [N, K] weight.  Measured on MI355X (Qwen3-4B shapes):
-// the 128 x 256 LDS-tiled kernel wins for F16 weights once there is at least one block per CU (2048 rows: 490-650
-// against 300 TFLOP/s); with Q8_0 weights the weight-streaming kernel, whose waves overlap each other's unpacking
-// and MFMAs, stays ahead at every M (400-470 against 340-460 TFLOP/s).
+// the 128 x 256 LDS-tiled kernel wins for F16 weights once there is about one block per CU (2048 rows: 490-650
+// against 300 TFLOP/s for the weight-streaming kernel).  With Q8_0 weights the streaming kernel, whose waves overlap
+// each other's unpacking and MFMAs, is ahead of the large-M kernel unpacking tiles into LDS itself (400-470 against
+// 340-460 TFLOP/s), but from 1024 rows on it pays to dequantise the operand once into an F16 image (3 bytes of extra
+// HBM traffic per weight) and run the large-M kernel on that instead of unpacking every tile again for each 64 rows
+// of activations: 4 x 512 rows, 112.9 ms per step against 123 ms (streaming) and 125 ms (Q8_0 inside the large-M kernel).
 int g_big_policy = 0;                                     // 0 measured rule, 1 always, -1 never
 bool use_big_gemm(int M, int N, int K, int fmt)
 {
     (void)K;
     if (g_big_policy) return g_big_policy > 0;
     const long blocks = (long)((M + 127) / 128) * ((N + 255) / 256);
+    if (M >= 1024) return blocks >= 160;                  // either format (Q8_0 through its F16 image)
     return fmt == 0 && M >= 512 && blocks >= 224;
+}
+
+// The operand as plain F16 tiles: W itself when it is F16, else an image in the library's scratch arena (valid until
+// the next call).
+WeightOp f16_image_of(const WeightOp &W, int N, int K)
+{
+    if (W.fmt == 0) return W;
+    const int Nb = tiled_rb(N), Kb = tiled_kb(K);
+    const size_t tiles = (size_t)Nb * Kb;
+    half8 *img = (half8 *)scratch(SCR_WF16, tiles * 256 * sizeof(half8));
+    hipLaunchKernelGGL(q8_operand_to_f16, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, stream(), W, Nb, Kb, img);
+    HIP_CHECK(hipGetLastError());
+    return weight_f16(reinterpret_cast<const half_t *>(img));
 }
 
 bool gemm_prof_begin(double wbytes, double flops, hipEvent_t *a, hipEvent_t *b)

@@ -179,7 +179,7 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
     if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch, final output
         float *C = out ? out : at<float>(s->planes);
         if (!out && (size_t)s->BN * N > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
-        launch_gemm_big(A, inv, W, C, N, s->BN, N, K);
+        launch_gemm_big(A, inv, f16_image_of(W, N, K), C, N, s->BN, N, K);
         return Planes{C, 1, (size_t)s->BN * N, N, nullptr};
     }
     GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
