@@ -112,19 +112,6 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
     for (int mb = 0; mb < 2; mb++) ap[mb] = g.A + (size_t)min(mb0 + mb, g.Mb - 1) * Kb * 256 + lane;
     const bool q8_rows = WF == 1 && nb0 < g.W.nbq;
 
-    // row factors of the 2 x 16 rows this lane stores, fetched before the K loop so that the
-    // epilogue of the last wave does not wait for them
-    float rsc[2][16];
-    if (SCALE) {
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                rsc[mb][v] = g.a_inv_scale[min(m, M - 1)];
-            }
-    }
-
     float16v acc[2][NB];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++)
@@ -191,9 +178,16 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
         if (half > 1) __syncthreads();
     }
     if (wave != 0) return;
+    // the row factors of the 16 rows of a block are fetched here, block by block, where the K loop's registers are free
+    // (holding all 32 through the loop costs a wave of occupancy per SIMD)
     float *Pp = g.P + (size_t)blockIdx.y * g.plane_stride;
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++)
+    for (int mb = 0; mb < 2; mb++) {
+        float rsc[16];
+        if (SCALE) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) rsc[v] = g.a_inv_scale[min((mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), M - 1)];
+        }
 #pragma unroll
         for (int b = 0; b < NB; b++)
 #pragma unroll
@@ -203,10 +197,11 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
                 const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
                 const int n = (nb0 + b) * 32 + r;
                 if (m < M && n < N) {
-                    if (SCALE) sres *= rsc[mb][v];
+                    if (SCALE) sres *= rsc[v];
                     Pp[(size_t)m * g.ldp + n] = sres;
                 }
             }
+    }
 }
 
 }  // namespace lmhip
