@@ -391,52 +391,99 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     const int n = qd + 2 * kd + 2 * R;
     float *dhp = buf + n;
     const int pos = (int)(row % a.seq);
-    for (int slot = wave; slot < a.Hq + a.Hkv; slot += RB / 64) {
-        const int isk = slot >= a.Hq, h = isk ? slot - a.Hq : slot;
-        const int W = isk ? kd : qd;
-        const float *gin = (isk ? a.dk : a.dq) + row * W + h * hd;
-        const float *xp = (isk ? a.k_pre : a.q_pre) + row * W + h * hd;
-        const float *g = isk ? a.g_k : a.g_q;
-        float y0[MAXP], y1[MAXP], p0[MAXP], p1[MAXP];
-        float ss = 0.f, dot = 0.f;
+    // A wave takes the (q or k) heads wave, wave + 16, wave + 32, ... three at a time: the loads of all three are
+    // issued before the first reduction, so their latency is paid once per trip instead of once per head.
+    constexpr int SU = 3;
+    const int nslots = a.Hq + a.Hkv;
+    for (int s0 = wave; s0 < nslots; s0 += (RB / 64) * SU) {
+        float g0[SU][MAXP], g1[SU][MAXP], p0[SU][MAXP], p1[SU][MAXP], w0[SU][MAXP], w1[SU][MAXP];
+        float2 cs[MAXP];
 #pragma unroll
         for (int p = 0; p < MAXP; p++) {
             const int d = lane + 64 * p;
-            y0[p] = y1[p] = p0[p] = p1[p] = 0.f;
-            if (d < half) {
-                const float g0 = gin[d], g1 = gin[d + half];
-                const float2 cs = a.rope[(size_t)pos * half + d];
-                y0[p] = g0 * cs.x + g1 * cs.y;
-                y1[p] = -g0 * cs.y + g1 * cs.x;
-                p0[p] = xp[d];
-                p1[p] = xp[d + half];
-                ss += p0[p] * p0[p] + p1[p] * p1[p];
-                dot += y0[p] * g[d] * p0[p] + y1[p] * g[d + half] * p1[p];
+            cs[p] = d < half ? a.rope[(size_t)pos * half + d] : make_float2(1.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < SU; u++) {
+            const int slot = min(s0 + (RB / 64) * u, nslots - 1);      // clamped: the extra work is not stored
+            const int isk = slot >= a.Hq, h = isk ? slot - a.Hq : slot;
+            const int W = isk ? kd : qd;
+            const float *gin = (isk ? a.dk : a.dq) + row * W + h * hd;
+            const float *xp = (isk ? a.k_pre : a.q_pre) + row * W + h * hd;
+            const float *g = isk ? a.g_k : a.g_q;
+#pragma unroll
+            for (int p = 0; p < MAXP; p++) {
+                const int d = lane + 64 * p;
+                g0[u][p] = g1[u][p] = p0[u][p] = p1[u][p] = w0[u][p] = w1[u][p] = 0.f;
+                if (d < half) {
+                    g0[u][p] = gin[d]; g1[u][p] = gin[d + half];
+                    p0[u][p] = xp[d]; p1[u][p] = xp[d + half];
+                    w0[u][p] = g[d]; w1[u][p] = g[d + half];
+                }
             }
         }
-        ss = wave_sum(ss);
-        dot = wave_sum(dot);
-        const float inv = rsqrtf(ss / (float)hd + a.eps);
-        const float coeff = dot * inv * inv / (float)hd;
 #pragma unroll
-        for (int p = 0; p < MAXP; p++) {
-            const int d = lane + 64 * p;
-            if (d >= half) continue;
-            const float d0 = (g[d] * y0[p] - coeff * p0[p]) * inv;
-            const float d1 = (g[d + half] * y1[p] - coeff * p1[p]) * inv;
-            const int c0 = (isk ? qd : 0) + h * hd + d;
-            buf[c0] = d0;
-            buf[c0 + half] = d1;
-            if (!isk) { a.dq_f[row * qd + h * hd + d] = d0; a.dq_f[row * qd + h * hd + d + half] = d1; }
+        for (int u = 0; u < SU; u++) {
+            const int slot = s0 + (RB / 64) * u;
+            float y0[MAXP], y1[MAXP];
+            float ss = 0.f, dot = 0.f;
+#pragma unroll
+            for (int p = 0; p < MAXP; p++) {
+                y0[p] = g0[u][p] * cs[p].x + g1[u][p] * cs[p].y;
+                y1[p] = -g0[u][p] * cs[p].y + g1[u][p] * cs[p].x;
+                ss += p0[u][p] * p0[u][p] + p1[u][p] * p1[u][p];
+                dot += y0[p] * w0[u][p] * p0[u][p] + y1[p] * w1[u][p] * p1[u][p];
+            }
+            ss = wave_sum(ss);
+            dot = wave_sum(dot);
+            if (slot >= nslots) continue;                              // uniform per wave
+            const int isk = slot >= a.Hq, h = isk ? slot - a.Hq : slot;
+            const float inv = rsqrtf(ss / (float)hd + a.eps);
+            const float coeff = dot * inv * inv / (float)hd;
+#pragma unroll
+            for (int p = 0; p < MAXP; p++) {
+                const int d = lane + 64 * p;
+                if (d >= half) continue;
+                const float d0 = (w0[u][p] * y0[p] - coeff * p0[u][p]) * inv;
+                const float d1 = (w1[u][p] * y1[p] - coeff * p1[u][p]) * inv;
+                const int c0 = (isk ? qd : 0) + h * hd + d;
+                buf[c0] = d0;
+                buf[c0 + half] = d1;
+                if (!isk) { a.dq_f[row * qd + h * hd + d] = d0; a.dq_f[row * qd + h * hd + d + half] = d1; }
+            }
         }
     }
     for (int c = threadIdx.x; c < kd; c += RB) buf[qd + kd + c] = a.dv[row * kd + c];
     __syncthreads();
-    // dh[r] = sc * sum_c d[c] * B[c][r]: a thread walks whole rows of B (R contiguous floats)
+    // dh[r] = sc * sum_c d[c] * B[c][r].  Rank 16 (the common case): four threads share a row of B (16 floats, one
+    // float4 each) and 256 such groups split the columns, so a thread keeps 4 + 4 sums and a wave reduces over its 16
+    // groups in four shuffle steps; other ranks: a thread walks whole rows of B.
     if (R > 0) {
         float acc[32];
 #pragma unroll
         for (int r = 0; r < 32; r++) acc[r] = 0.f;
+        if (R == 16) {
+            const int sub = threadIdx.x & 3;
+            float aq[4] = {0.f, 0.f, 0.f, 0.f}, av[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int c = threadIdx.x >> 2; c < qd + kd; c += RB / 4) {
+                const int isv = c >= qd;
+                const float x = buf[isv ? c + kd : c];
+                const float4 w = ld4((isv ? a.Bv + (size_t)(c - qd) * 16 : a.Bq + (size_t)c * 16) + 4 * sub);
+                if (isv) { av[0] += x * w.x; av[1] += x * w.y; av[2] += x * w.z; av[3] += x * w.w; }
+                else { aq[0] += x * w.x; aq[1] += x * w.y; aq[2] += x * w.z; aq[3] += x * w.w; }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+#pragma unroll
+                for (int o = 4; o < 64; o <<= 1) { aq[e] += __shfl_xor(aq[e], o, WAVE); av[e] += __shfl_xor(av[e], o, WAVE); }
+            }
+            if (lane < 4) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) { dhp[wave * 32 + 4 * lane + e] = aq[e]; dhp[wave * 32 + 16 + 4 * lane + e] = av[e]; }
+            }
+        } else {
+#pragma unroll 4
         for (int c = threadIdx.x; c < qd + kd; c += RB) {
             const int isv = c >= qd;
             const float x = buf[isv ? c + kd : c];
@@ -461,6 +508,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         if (lane == 0) {
 #pragma unroll
             for (int r = 0; r < 32; r++) dhp[wave * 32 + r] = acc[r];
+        }
         }
         __syncthreads();
         if (threadIdx.x < 2 * R) {
