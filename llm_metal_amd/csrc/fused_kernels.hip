@@ -168,11 +168,24 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
             x0[p] = planes_at(a.qkv, row, col0 + d);
             x1[p] = planes_at(a.qkv, row, col0 + d + half);
         }
-        if (lora) {                                           // uniform branch: shuffles stay convergent
+        if (lora && 64 * p < half) {                          // uniform branch: the broadcasts stay convergent
             float acc0 = 0.f, acc1 = 0.f;
             const float *b0 = B + (size_t)(h * hd + (d < half ? d : 0)) * a.R;
             const float *b1 = b0 + (size_t)half * a.R;
-            if ((a.R & 3) == 0) {                              // whole rows of B as independent 16-byte loads
+            if (a.R == 16) {                                   // t through scalar registers, whole rows of B as 16-byte loads
+                float4 w0[4], w1[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) { w0[i] = w1[i] = make_float4(0.f, 0.f, 0.f, 0.f); if (d < half) { w0[i] = ld4(b0 + 4 * i); w1[i] = ld4(b1 + 4 * i); } }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float t0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tval), 4 * i));
+                    const float t1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tval), 4 * i + 1));
+                    const float t2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tval), 4 * i + 2));
+                    const float t3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tval), 4 * i + 3));
+                    acc0 += t0 * w0[i].x; acc0 += t1 * w0[i].y; acc0 += t2 * w0[i].z; acc0 += t3 * w0[i].w;
+                    acc1 += t0 * w1[i].x; acc1 += t1 * w1[i].y; acc1 += t2 * w1[i].z; acc1 += t3 * w1[i].w;
+                }
+            } else if ((a.R & 3) == 0) {
                 for (int r4 = 0; r4 < a.R; r4 += 4) {
                     float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w1 = w0;
                     if (d < half) { w0 = ld4(b0 + r4); w1 = ld4(b1 + r4); }
