@@ -263,7 +263,7 @@ template <int BWD, int HD>
 __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
 {
     extern __shared__ float lds[];
-    constexpr int lda = HD + 8, half = HD / 2;            // halves; rows 16-byte aligned and 4 banks apart: conflict-free 16-byte reads
+    constexpr int lda = HD + 8;                            // halves; rows 16-byte aligned and 4 banks apart: conflict-free 16-byte reads
     const int N = a.seq;
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l31 = lane & 31, hh = lane >> 5;
@@ -297,11 +297,21 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     // ---- A rows into LDS (rows past the sequence as zeros); the loads of all HD / 32 rounds are issued together
     {
         float4 av[HD / 32];
+        if (BWD) {
+            size_t rows[HD / 32]; int cols[HD / 32]; bool ok[HD / 32];
 #pragma unroll
-        for (int u = 0; u < HD / 32; u++) {
-            const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
-            av[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (i0 + rr < N) av[u] = BWD ? planes_at4(a.Apl, r0 + i0 + rr, h * HD + 4 * c4) : ld4(a.A + (r0 + i0 + rr) * qd + h * HD + 4 * c4);
+            for (int u = 0; u < HD / 32; u++) {
+                const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
+                ok[u] = i0 + rr < N; rows[u] = r0 + (ok[u] ? i0 + rr : 0); cols[u] = h * HD + 4 * c4;
+            }
+            planes_at4_multi<HD / 32, (HD <= 128 ? 5 : 3)>(a.Apl, rows, cols, ok, av);
+        } else {
+#pragma unroll
+            for (int u = 0; u < HD / 32; u++) {
+                const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
+                av[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (i0 + rr < N) av[u] = ld4(a.A + (r0 + i0 + rr) * qd + h * HD + 4 * c4);
+            }
         }
 #pragma unroll
         for (int u = 0; u < HD / 32; u++) {

@@ -42,6 +42,19 @@ __device__ __forceinline__ float block_sum(float v, float *smem)
     return r;
 }
 
+// Two sums for one pair of barriers; `smem` must hold 32 floats.  Each sum is formed in the order block_sum forms it.
+__device__ __forceinline__ void block_sum2(float &a, float &b, float *smem)
+{
+    a = wave_sum(a); b = wave_sum(b);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    if (lane == 0) { smem[w] = a; smem[16 + w] = b; }
+    __syncthreads();
+    float ra = 0.f, rb = 0.f;
+    for (int i = 0; i < nw; i++) { ra += smem[i]; rb += smem[16 + i]; }
+    __syncthreads();
+    a = ra; b = rb;
+}
+
 __device__ __forceinline__ float block_max(float v, float *smem)
 {
     v = wave_max(v);

@@ -18,6 +18,7 @@ namespace {
 constexpr int TB = 256;
 constexpr int RB = 1024;                                  // threads of a row workgroup
 constexpr int MAXV = 3;                                   // float4 per thread: rows up to 12288 wide
+constexpr int MAXV_ROW = MAXV;                            // (the name the row kernels with their own MAXV parameter use)
 
 // four consecutive elements (k % 4 == 0) of row `row` of a tiled fp16 operand
 __device__ __forceinline__ void st_tiled4(half_t *out, size_t row, int k, int Kb, float4 v, float s)
@@ -48,6 +49,8 @@ __device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t
 // x = (gathered embedding | x_prev) [+ branch | + RN(branch; g_branch)];  ln = RN(x; g_norm).
 // rms_norm: shaders/q8_kernels.metal:133-158; residual_add :369-375; the Gemma3
 // ordering (norm the branch, then add) is src/nn/fast_sft.c:698-705, 732-736.
+// MAXV: float4 per thread (1 for rows up to 4096 wide, which leaves registers for 20 planes of the branch in flight).
+template <int MAXV>
 __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
@@ -56,15 +59,18 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
     float4 x[MAXV], b[MAXV];
     const bool padded = a.emb && a.n_valid > 0 && (int)r >= a.n_valid;      // zero rows past the sequence
     const float *base = a.emb ? a.emb + (size_t)(padded ? 0u : a.tokens[r]) * D : a.x_prev + r * D;
+    size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         const int v = threadIdx.x + t * RB;
         x[t] = b[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (v < nv) {
-            if (!padded) x[t] = ld4(base + 4 * v);
-            if (a.emb && a.emb_scale != 1.0f) { x[t].x *= a.emb_scale; x[t].y *= a.emb_scale; x[t].z *= a.emb_scale; x[t].w *= a.emb_scale; }
-            if (a.branch.S > 0) b[t] = planes_at4(a.branch, r, 4 * v);
-        }
+        rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
+        if (v < nv && !padded) x[t] = ld4(base + 4 * v);
+    }
+    if (a.branch.S > 0) planes_at4_multi<MAXV, (MAXV == 1 ? 20 : 6)>(a.branch, rows, cols, ok, b);
+    if (a.emb && a.emb_scale != 1.0f) {
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) { x[t].x *= a.emb_scale; x[t].y *= a.emb_scale; x[t].z *= a.emb_scale; x[t].w *= a.emb_scale; }
     }
     if (a.branch.S > 0) {
         float inv = 1.0f;
@@ -154,20 +160,28 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
     const bool lora = a.R > 0 && kind != 1;
     const float *B = kind == 0 ? a.Bq : a.Bv;
 
-    float tval = 0.f;
-    if (lora && lane < a.R) tval = planes_at(a.qkv, row, t0 + lane);
+    // everything this lane reads from the planes in one go: positions p (first half of the head), MAXP + p (second
+    // half) and 2 MAXP (the lane's entry of x A^T)
+    float x0[MAXP], x1[MAXP], tval;
+    {
+        int cols[2 * MAXP + 1]; bool ok[2 * MAXP + 1]; float got[2 * MAXP + 1];
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) {
+            const int d = lane + 64 * p;
+            cols[p] = col0 + d; cols[MAXP + p] = col0 + d + half; ok[p] = ok[MAXP + p] = d < half;
+        }
+        cols[2 * MAXP] = t0 + lane; ok[2 * MAXP] = lora && lane < a.R;
+        planes_at_multi<2 * MAXP + 1, 5>(a.qkv, row, cols, ok, got);
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) { x0[p] = got[p]; x1[p] = got[MAXP + p]; }
+        tval = got[2 * MAXP];
+    }
     if (lora && h == 0 && lane < a.R) (kind == 0 ? a.tq : a.tv)[row * a.R + lane] = tval;
 
-    float x0[MAXP], x1[MAXP];
     float ss = 0.f;
 #pragma unroll
     for (int p = 0; p < MAXP; p++) {
         const int d = lane + 64 * p;
-        x0[p] = x1[p] = 0.f;
-        if (d < half) {
-            x0[p] = planes_at(a.qkv, row, col0 + d);
-            x1[p] = planes_at(a.qkv, row, col0 + d + half);
-        }
         if (lora && 64 * p < half) {                          // uniform branch: the broadcasts stay convergent
             float acc0 = 0.f, acc1 = 0.f;
             const float *b0 = B + (size_t)(h * hd + (d < half ? d : 0)) * a.R;
@@ -608,12 +622,23 @@ __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
     const int IS = a.IS, nv = IS >> 2;
     float4 act[MAXV];
     float amax = 0.f;
+    // the gate and up values of all the thread's columns in one go: positions t (gate) and MAXV + t (up)
+    float4 gu[2 * MAXV];
+    {
+        size_t rows[2 * MAXV]; int cols[2 * MAXV]; bool ok[2 * MAXV];
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const int v = threadIdx.x + t * RB;
+            rows[t] = rows[MAXV + t] = r; cols[t] = 4 * v; cols[MAXV + t] = IS + 4 * v; ok[t] = ok[MAXV + t] = v < nv;
+        }
+        planes_at4_multi<2 * MAXV, 3>(a.in, rows, cols, ok, gu);
+    }
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         const int v = threadIdx.x + t * RB;
         act[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (v < nv) {
-            const float4 g = planes_at4(a.in, r, 4 * v), u = planes_at4(a.in, r, IS + 4 * v);
+            const float4 g = gu[t], u = gu[MAXV + t];
             st4(a.gate_pre + r * IS + 4 * v, g);
             st4(a.up_val + r * IS + 4 * v, u);
             act[t] = make_float4(act_fwd(g.x, a.gelu) * u.x, act_fwd(g.y, a.gelu) * u.y,
@@ -651,12 +676,24 @@ __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
     const int IS = a.IS, nv = IS >> 2;
     float4 dg[MAXV], du[MAXV];
     float amax = 0.f;
+    float4 dys[MAXV], gs[MAXV], us[MAXV];
+    {
+        size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const int v = threadIdx.x + t * RB;
+            rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
+            gs[t] = us[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (v < nv) { gs[t] = ld4(a.gate_pre + r * IS + 4 * v); us[t] = ld4(a.up_val + r * IS + 4 * v); }
+        }
+        planes_at4_multi<MAXV, 5>(a.in, rows, cols, ok, dys);
+    }
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         const int v = threadIdx.x + t * RB;
         dg[t] = du[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (v < nv) {
-            const float4 dy = planes_at4(a.in, r, 4 * v), g = ld4(a.gate_pre + r * IS + 4 * v), u = ld4(a.up_val + r * IS + 4 * v);
+            const float4 dy = dys[t], g = gs[t], u = us[t];
             act_bwd(dy.x, g.x, u.x, a.gelu, dg[t].x, du[t].x);
             act_bwd(dy.y, g.y, u.y, a.gelu, dg[t].y, du[t].y);
             act_bwd(dy.z, g.z, u.z, a.gelu, dg[t].z, du[t].z);
@@ -682,27 +719,29 @@ __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
 // src/nn/fast_sft.c:870-874, 975-980).  The operand of the next dX GEMM is dx_out
 // itself (Qwen3) or RNB(branch_raw, dx_out; g_branch) (Gemma3's post-norms,
 // src/nn/fast_sft.c:798-802, 877-881).
+template <int MAXV>
 __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
-    __shared__ float sm[16];
+    __shared__ float sm[32];
     const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 dy[MAXV], x[MAXV], g[MAXV];
     float ss = 0.f, dot = 0.f;
+    size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         const int v = threadIdx.x + t * RB;
-        dy[t] = x[t] = g[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (v < nv) {
-            dy[t] = planes_at4(a.dy, r, 4 * v);
-            x[t] = ld4(a.x_saved + r * D + 4 * v);
-            g[t] = ld4(a.g + 4 * v);
-            ss += sumsq4(x[t]);
-            dot += dy[t].x * g[t].x * x[t].x + dy[t].y * g[t].y * x[t].y + dy[t].z * g[t].z * x[t].z + dy[t].w * g[t].w * x[t].w;
-        }
+        x[t] = g[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
+        if (v < nv) { x[t] = ld4(a.x_saved + r * D + 4 * v); g[t] = ld4(a.g + 4 * v); }
     }
-    ss = block_sum(ss, sm);
-    dot = block_sum(dot, sm);
+    planes_at4_multi<MAXV, (MAXV == 1 ? 20 : 4)>(a.dy, rows, cols, ok, dy);
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) {
+        ss += sumsq4(x[t]);
+        dot += dy[t].x * g[t].x * x[t].x + dy[t].y * g[t].y * x[t].y + dy[t].z * g[t].z * x[t].z + dy[t].w * g[t].w * x[t].w;
+    }
+    block_sum2(ss, dot, sm);
     const float inv = rsqrtf(ss / (float)D + a.eps);
     const float coeff = dot * inv * inv / (float)D;
     float4 dx[MAXV];
@@ -733,8 +772,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
             ssb += sumsq4(x[t]);
             dotb += dx[t].x * g[t].x * x[t].x + dx[t].y * g[t].y * x[t].y + dx[t].z * g[t].z * x[t].z + dx[t].w * g[t].w * x[t].w;
         }
-        ssb = block_sum(ssb, sm);
-        dotb = block_sum(dotb, sm);
+        block_sum2(ssb, dotb, sm);
         const float invb = rsqrtf(ssb / (float)D + a.eps);
         const float cb = dotb * invb * invb / (float)D;
 #pragma unroll
@@ -922,7 +960,8 @@ void launch_norm_rows(const NormRowsArgs &a, int rows)
 {
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV, "norm_rows: hidden size must be a multiple of 4, <= 12288");
     require(a.branch.S == 0 || a.branch.ld % 4 == 0, "norm_rows: plane row length must be a multiple of 4");
-    LAUNCH(k_norm_rows, dim3(rows), dim3(RB), 0, a);
+    if (a.D <= 4 * RB) LAUNCH(k_norm_rows<1>, dim3(rows), dim3(RB), 0, a);
+    else LAUNCH(k_norm_rows<MAXV_ROW>, dim3(rows), dim3(RB), 0, a);
 }
 
 void launch_rope_table(float2 *tab, int seq, int hd, float theta)
@@ -987,7 +1026,8 @@ void launch_glu_bwd(const GluArgs &a, int rows)
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
 {
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV && a.dy.ld % 4 == 0, "norm_bwd_rows: hidden size must be a multiple of 4, <= 12288");
-    LAUNCH(k_norm_bwd_rows, dim3(rows), dim3(RB), 0, a);
+    if (a.D <= 4 * RB) LAUNCH(k_norm_bwd_rows<1>, dim3(rows), dim3(RB), 0, a);
+    else LAUNCH(k_norm_bwd_rows<MAXV_ROW>, dim3(rows), dim3(RB), 0, a);
 }
 
 void launch_ce_rows(const CeArgs &a, int rows)

@@ -31,6 +31,60 @@ __device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int co
     return s;
 }
 
+// The same for T positions of one thread at once: the loads of NB planes at all T positions are issued together, so the
+// thread pays ceil(S / NB) memory round trips for all of them, where one call of planes_at4 per position pays at least
+// one each (its loop over the planes has a run-time bound, which keeps the compiler from overlapping two calls).
+// Position t is read only when ok[t]; the sums are formed in plane order, exactly as planes_at4 forms them.
+template <int T, int NB>
+__device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (&row)[T], const int (&col)[T], const bool (&ok)[T], float4 (&s)[T])
+{
+    const float *p[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) { p[t] = P.p + row[t] * P.ld + col[t]; s[t] = make_float4(0.f, 0.f, 0.f, 0.f); }
+    for (int i0 = 0; i0 < P.S; i0 += NB) {
+        float4 v[T][NB];
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+#pragma unroll
+            for (int t = 0; t < T; t++)
+                v[t][i] = (ok[t] && i0 + i < P.S) ? *reinterpret_cast<const float4 *>(p[t] + (size_t)(i0 + i) * P.stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int t = 0; t < T; t++)
+#pragma unroll
+            for (int i = 0; i < NB; i++) { s[t].x += v[t][i].x; s[t].y += v[t][i].y; s[t].z += v[t][i].z; s[t].w += v[t][i].w; }
+    }
+    if (P.row_scale) {
+#pragma unroll
+        for (int t = 0; t < T; t++)
+            if (ok[t]) { const float f = P.row_scale[row[t]]; s[t].x *= f; s[t].y *= f; s[t].z *= f; s[t].w *= f; }
+    }
+}
+
+// Single values instead of groups of four.
+template <int T, int NB>
+__device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, const int (&col)[T], const bool (&ok)[T], float (&s)[T])
+{
+    const float *p[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) { p[t] = P.p + row * P.ld + col[t]; s[t] = 0.f; }
+    for (int i0 = 0; i0 < P.S; i0 += NB) {
+        float v[T][NB];
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+#pragma unroll
+            for (int t = 0; t < T; t++) v[t][i] = (ok[t] && i0 + i < P.S) ? p[t][(size_t)(i0 + i) * P.stride] : 0.f;
+#pragma unroll
+        for (int t = 0; t < T; t++)
+#pragma unroll
+            for (int i = 0; i < NB; i++) s[t] += v[t][i];
+    }
+    if (P.row_scale) {
+        const float f = P.row_scale[row];
+#pragma unroll
+        for (int t = 0; t < T; t++) s[t] *= f;
+    }
+}
+
 __device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 __device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
 __device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
