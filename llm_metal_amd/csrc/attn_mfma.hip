@@ -481,7 +481,7 @@ void launch_attn_fwd_mfma(const AttnFwdArgs &f)
 
 void launch_attn_bwd_mfma(const AttnBwdArgs &g)
 {
-    if (!attn_mfma_supported(g.hd, g.seq) || !g.vT) { fprintf(stderr, "[fast_hip] attn_bwd_mfma: unsupported shape\n"); abort(); }
+    if (!attn_mfma_supported(g.hd, g.seq) || !g.vT || g.dO.scale_groups) { fprintf(stderr, "[fast_hip] attn_bwd_mfma: unsupported shape\n"); abort(); }
     AttnTileArgs a{};
     a.Apl = g.dO; a.BT = g.vT; a.C = g.k;
     a.Hq = g.Hq; a.Hkv = g.Hkv; a.hd = g.hd; a.seq = g.seq; a.batch = g.batch; a.scale = g.scale;

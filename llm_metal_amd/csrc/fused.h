@@ -16,7 +16,15 @@ struct Planes {
     size_t stride;
     int ld;
     const float *row_scale;   // value(row, col) is multiplied by row_scale[row] when non-null
+    // scale_groups != 0: the operand rows were scaled in that many groups of columns, each the K range of 2^group_shift
+    // planes, and plane s is multiplied by row_scale[row * scale_groups + (s >> group_shift)] before it is added
+    int group_shift, scale_groups;
 };
+
+// How a row kernel splits the columns of an fp16 operand row [*, K] among workgroups, each with a power-of-two scale of
+// its own: `cols` columns per group (a whole number of K chunks of the GEMM that consumes the operand), `groups` of
+// them; cols == 0: one workgroup and one scale per row.
+struct ScaleGroups { int cols, groups, shift; };
 
 struct NormRowsArgs {
     // source of the residual stream row: token gather (emb != null) or x_prev
@@ -106,6 +114,7 @@ struct GluArgs {
     int IS, gelu;
     float *gate_pre, *up_val;     // fwd: written; bwd: read
     half_t *out16; float *inv_scale;                // tiled; fwd: act [rows, IS]; bwd: [rows, dgate | dup]
+    ScaleGroups sg;               // sg.cols != 0: inv_scale is [rows][sg.groups]
 };
 void launch_glu_fwd(const GluArgs &a, int rows);
 void launch_glu_bwd(const GluArgs &a, int rows);

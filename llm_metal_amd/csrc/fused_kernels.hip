@@ -50,7 +50,8 @@ __device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t
 // rms_norm: shaders/q8_kernels.metal:133-158; residual_add :369-375; the Gemma3
 // ordering (norm the branch, then add) is src/nn/fast_sft.c:698-705, 732-736.
 // MAXV: float4 per thread (1 for rows up to 4096 wide, which leaves registers for 20 planes of the branch in flight).
-template <int MAXV>
+// GROUPED: the branch planes carry a factor per group of planes.
+template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv && !padded) x[t] = ld4(base + 4 * v);
     }
-    if (a.branch.S > 0) planes_at4_multi<MAXV, (MAXV == 1 ? 20 : 6)>(a.branch, rows, cols, ok, b);
+    if (a.branch.S > 0) planes_at4_multi<MAXV, (MAXV == 1 ? 20 : 6), GROUPED>(a.branch, rows, cols, ok, b);
     if (a.emb && a.emb_scale != 1.0f) {
 #pragma unroll
         for (int t = 0; t < MAXV; t++) { x[t].x *= a.emb_scale; x[t].y *= a.emb_scale; x[t].z *= a.emb_scale; x[t].w *= a.emb_scale; }
@@ -655,6 +656,49 @@ __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
 
+// The same with the columns of a row split among workgroups (grid (rows, groups), block 256): group c covers the
+// columns [c * sg.cols, (c + 1) * sg.cols) and scales them by a factor of its own, inv_scale[row * groups + c].  The
+// GEMM that reads the operand cuts K into chunks that do not straddle groups, so every plane of its result belongs to
+// one factor.  64 rows then occupy the whole GPU instead of 64 CUs.
+constexpr int GC = 256, MAXC = 2;                         // threads of a column-group workgroup; float4 per thread
+__global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
+{
+    __shared__ float sm[16];
+    const size_t r = blockIdx.x;
+    const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(IS, c0 + a.sg.cols) - c0, nv = width >> 2;
+    float4 act[MAXC], gu[2 * MAXC];
+    float amax = 0.f;
+    {
+        size_t rows[2 * MAXC]; int cols[2 * MAXC]; bool ok[2 * MAXC];
+#pragma unroll
+        for (int t = 0; t < MAXC; t++) {
+            const int v = threadIdx.x + t * GC;
+            rows[t] = rows[MAXC + t] = r; cols[t] = c0 + 4 * v; cols[MAXC + t] = IS + c0 + 4 * v; ok[t] = ok[MAXC + t] = v < nv;
+        }
+        planes_at4_multi<2 * MAXC, 3>(a.in, rows, cols, ok, gu);
+    }
+#pragma unroll
+    for (int t = 0; t < MAXC; t++) {
+        const int v = threadIdx.x + t * GC;
+        act[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) {
+            const float4 g = gu[t], u = gu[MAXC + t];
+            st4(a.gate_pre + r * IS + c0 + 4 * v, g);
+            st4(a.up_val + r * IS + c0 + 4 * v, u);
+            act[t] = make_float4(act_fwd(g.x, a.gelu) * u.x, act_fwd(g.y, a.gelu) * u.y,
+                                 act_fwd(g.z, a.gelu) * u.z, act_fwd(g.w, a.gelu) * u.w);
+            amax = fmaxf(amax, amax4(act[t]));
+        }
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    const int Kb = tiled_kb(IS);
+#pragma unroll
+    for (int t = 0; t < MAXC; t++) { const int v = threadIdx.x + t * GC; if (v < nv) st_tiled4(a.out16, r, c0 + 4 * v, Kb, act[t], s); }
+    if (c0 + width == IS) zero_tiled_pad(a.out16, r, IS, Kb);
+    if (threadIdx.x == 0) a.inv_scale[r * gridDim.y + blockIdx.y] = 1.0f / s;
+}
+
 __device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, float &dg, float &du)
 {
     if (gelu) {                                           // gelu_mul_backward, shaders/q8_kernels.metal:561-580
@@ -719,7 +763,7 @@ __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
 // src/nn/fast_sft.c:870-874, 975-980).  The operand of the next dX GEMM is dx_out
 // itself (Qwen3) or RNB(branch_raw, dx_out; g_branch) (Gemma3's post-norms,
 // src/nn/fast_sft.c:798-802, 877-881).
-template <int MAXV>
+template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
     __shared__ float sm[32];
@@ -735,7 +779,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv) { x[t] = ld4(a.x_saved + r * D + 4 * v); g[t] = ld4(a.g + 4 * v); }
     }
-    planes_at4_multi<MAXV, (MAXV == 1 ? 20 : 4)>(a.dy, rows, cols, ok, dy);
+    planes_at4_multi<MAXV, (MAXV == 1 ? 20 : 4), GROUPED>(a.dy, rows, cols, ok, dy);
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         ss += sumsq4(x[t]);
@@ -960,8 +1004,9 @@ void launch_norm_rows(const NormRowsArgs &a, int rows)
 {
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV, "norm_rows: hidden size must be a multiple of 4, <= 12288");
     require(a.branch.S == 0 || a.branch.ld % 4 == 0, "norm_rows: plane row length must be a multiple of 4");
-    if (a.D <= 4 * RB) LAUNCH(k_norm_rows<1>, dim3(rows), dim3(RB), 0, a);
-    else LAUNCH(k_norm_rows<MAXV_ROW>, dim3(rows), dim3(RB), 0, a);
+    const bool grouped = a.branch.S > 0 && a.branch.scale_groups != 0;
+    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_rows<1, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_rows<1, false>), dim3(rows), dim3(RB), 0, a); }
+    else { if (grouped) LAUNCH((k_norm_rows<MAXV_ROW, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_rows<MAXV_ROW, false>), dim3(rows), dim3(RB), 0, a); }
 }
 
 void launch_rope_table(float2 *tab, int seq, int hd, float theta)
@@ -973,6 +1018,7 @@ void launch_rope_table(float2 *tab, int seq, int hd, float theta)
 void launch_qkv_post(const QkvPostArgs &a, int rows)
 {
     require(a.hd % 2 == 0 && a.hd <= 2 * 64 * MAXP && a.R <= 64 && a.Hq % a.Hkv == 0, "qkv_post: head_dim <= 512, rank <= 64");
+    require(!a.qkv.scale_groups, "qkv_post: input planes with grouped row factors are not supported");
     const size_t tasks = (size_t)rows * (a.Hq + 2 * a.Hkv);
     QkvPostArgs b = a;
     b.rows = rows;
@@ -1015,19 +1061,28 @@ void launch_lora_grads(const LoraGradArgs &a)
 void launch_glu_fwd(const GluArgs &a, int rows)
 {
     require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_fwd: FFN width must be a multiple of 4, <= 12288");
+    require(!a.in.scale_groups, "glu_fwd: input planes with grouped row factors are not supported");
+    if (a.sg.cols) {
+        require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC * MAXC && (long)a.sg.cols * a.sg.groups >= a.IS && (long)a.sg.cols * (a.sg.groups - 1) < a.IS,
+                "glu_fwd: column groups do not fit the row");
+        LAUNCH(k_glu_fwd_cols, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        return;
+    }
     LAUNCH(k_glu_fwd, dim3(rows), dim3(RB), 0, a);
 }
 void launch_glu_bwd(const GluArgs &a, int rows)
 {
     require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_bwd: FFN width must be a multiple of 4, <= 12288");
+    require(!a.in.scale_groups, "glu_bwd: input planes with grouped row factors are not supported");
     LAUNCH(k_glu_bwd, dim3(rows), dim3(RB), 0, a);
 }
 
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
 {
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV && a.dy.ld % 4 == 0, "norm_bwd_rows: hidden size must be a multiple of 4, <= 12288");
-    if (a.D <= 4 * RB) LAUNCH(k_norm_bwd_rows<1>, dim3(rows), dim3(RB), 0, a);
-    else LAUNCH(k_norm_bwd_rows<MAXV_ROW>, dim3(rows), dim3(RB), 0, a);
+    const bool grouped = a.dy.scale_groups != 0;
+    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_bwd_rows<1, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_bwd_rows<1, false>), dim3(rows), dim3(RB), 0, a); }
+    else { if (grouped) LAUNCH((k_norm_bwd_rows<MAXV_ROW, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_bwd_rows<MAXV_ROW, false>), dim3(rows), dim3(RB), 0, a); }
 }
 
 void launch_ce_rows(const CeArgs &a, int rows)

@@ -9,6 +9,10 @@ __device__ __forceinline__ float planes_at(const Planes &P, size_t row, int col)
 {
     float s = 0.f;
     const float *p = P.p + row * P.ld + col;
+    if (P.scale_groups) {
+        for (int i = 0; i < P.S; i++) s += p[(size_t)i * P.stride] * P.row_scale[row * P.scale_groups + (i >> P.group_shift)];
+        return s;
+    }
     for (int i = 0; i < P.S; i++) s += p[(size_t)i * P.stride];
     return P.row_scale ? s * P.row_scale[row] : s;
 }
@@ -19,6 +23,14 @@ __device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int co
 {
     const float *p = P.p + row * P.ld + col;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (P.scale_groups) {
+        for (int i = 0; i < P.S; i++) {
+            const float4 v = *reinterpret_cast<const float4 *>(p + (size_t)i * P.stride);
+            const float f = P.row_scale[row * P.scale_groups + (i >> P.group_shift)];
+            s.x += v.x * f; s.y += v.y * f; s.z += v.z * f; s.w += v.w * f;
+        }
+        return s;
+    }
     for (int i0 = 0; i0 < P.S; i0 += 8) {
         float4 v[8];
 #pragma unroll
@@ -35,39 +47,61 @@ __device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int co
 // thread pays ceil(S / NB) memory round trips for all of them, where one call of planes_at4 per position pays at least
 // one each (its loop over the planes has a run-time bound, which keeps the compiler from overlapping two calls).
 // Position t is read only when ok[t]; the sums are formed in plane order, exactly as planes_at4 forms them.
-template <int T, int NB>
+// GROUPED: the planes carry a factor per group of planes (Planes::scale_groups != 0); all T positions must then lie in
+// row[0], and row[0] must be the same for the whole wave.
+template <int T, int NB, bool GROUPED = false>
 __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (&row)[T], const int (&col)[T], const bool (&ok)[T], float4 (&s)[T])
 {
     const float *p[T];
 #pragma unroll
     for (int t = 0; t < T; t++) { p[t] = P.p + row[t] * P.ld + col[t]; s[t] = make_float4(0.f, 0.f, 0.f, 0.f); }
-    for (int i0 = 0; i0 < P.S; i0 += NB) {
+    // (a loop, not unrolled: these kernels run their code once, and what they gain from straight-line batches they lose
+    // again fetching the longer code)
+    auto batch = [&](int i0) __attribute__((always_inline)) {
         float4 v[T][NB];
 #pragma unroll
         for (int i = 0; i < NB; i++)
 #pragma unroll
             for (int t = 0; t < T; t++)
                 v[t][i] = (ok[t] && i0 + i < P.S) ? *reinterpret_cast<const float4 *>(p[t] + (size_t)(i0 + i) * P.stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (GROUPED) {                                    // a factor per plane, fetched with the planes
+            // lane i of every wave fetches the factor of plane i0 + i (one load, in flight with the planes); the
+            // values then reach all lanes through scalar registers
+            static_assert(NB <= 64, "one lane per plane of a batch");
+            const int li = threadIdx.x & 63;
+            const float fl = (li < NB && i0 + li < P.S) ? P.row_scale[row[0] * P.scale_groups + ((i0 + li) >> P.group_shift)] : 0.f;
+            float f[NB];
+#pragma unroll
+            for (int i = 0; i < NB; i++) f[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fl), i));
+#pragma unroll
+            for (int t = 0; t < T; t++)
+#pragma unroll
+                for (int i = 0; i < NB; i++) {
+                    s[t].x += v[t][i].x * f[i]; s[t].y += v[t][i].y * f[i]; s[t].z += v[t][i].z * f[i]; s[t].w += v[t][i].w * f[i];
+                }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < T; t++)
 #pragma unroll
             for (int i = 0; i < NB; i++) { s[t].x += v[t][i].x; s[t].y += v[t][i].y; s[t].z += v[t][i].z; s[t].w += v[t][i].w; }
-    }
-    if (P.row_scale) {
+    };
+    for (int i0 = 0; i0 < P.S; i0 += NB) batch(i0);
+    if (!GROUPED && P.row_scale) {
 #pragma unroll
         for (int t = 0; t < T; t++)
             if (ok[t]) { const float f = P.row_scale[row[t]]; s[t].x *= f; s[t].y *= f; s[t].z *= f; s[t].w *= f; }
     }
 }
 
-// Single values instead of groups of four.
+// Single values instead of groups of four (planes without grouped factors only).
 template <int T, int NB>
 __device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, const int (&col)[T], const bool (&ok)[T], float (&s)[T])
 {
     const float *p[T];
 #pragma unroll
     for (int t = 0; t < T; t++) { p[t] = P.p + row * P.ld + col[t]; s[t] = 0.f; }
-    for (int i0 = 0; i0 < P.S; i0 += NB) {
+    auto batch = [&](int i0) __attribute__((always_inline)) {
         float v[T][NB];
 #pragma unroll
         for (int i = 0; i < NB; i++)
@@ -77,7 +111,8 @@ __device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, con
         for (int t = 0; t < T; t++)
 #pragma unroll
             for (int i = 0; i < NB; i++) s[t] += v[t][i];
-    }
+    };
+    for (int i0 = 0; i0 < P.S; i0 += NB) batch(i0);
     if (P.row_scale) {
         const float f = P.row_scale[row];
 #pragma unroll

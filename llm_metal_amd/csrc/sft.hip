@@ -173,8 +173,28 @@ size_t max_planes_elems(SFTState *s)
     return mx;
 }
 
+constexpr int MAX_SCALE_GROUPS = 64;                      // a16_inv holds this many factors per row
+
+// Column groups for the row kernel that writes the operand [BN, K] of the product with W [N, K]: as many groups as it
+// takes to put about two workgroups on every CU, each a power-of-two number of the GEMM's K chunks and at most 2048
+// columns wide.  None (cols = 0) when the product does not leave planes (large M, S == 1) or the rows alone fill the GPU.
+ScaleGroups scale_groups_for(SFTState *s, const WeightOp &W, int N, int K)
+{
+    ScaleGroups none{0, 1, 0};
+    if (s->full_param || use_big_gemm(s->BN, N, K, W.fmt)) return none;      // weight gradients take one factor per row
+    const GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
+    const int plane_cols = p.steps * 64, cus = num_cus() > 0 ? num_cus() : 256;
+    const int want = (2 * cus + s->BN - 1) / s->BN;
+    if (p.S <= 1 || want <= 1 || plane_cols > 2048) return none;
+    int shift = 0;
+    while ((plane_cols << (shift + 1)) <= 2048 && ((p.S + (2 << shift) - 1) >> (shift + 1)) >= want) shift++;
+    ScaleGroups g{plane_cols << shift, (p.S + (1 << shift) - 1) >> shift, shift};
+    return g.groups <= MAX_SCALE_GROUPS ? g : none;
+}
+
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
-Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr)
+Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr,
+            const ScaleGroups *sg = nullptr)
 {
     if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch, final output
         float *C = out ? out : at<float>(s->planes);
@@ -189,6 +209,12 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
     if (out && p.S != 1) { fprintf(stderr, "[fast_sft] direct GEMM output needs S == 1\n"); abort(); }
     // a direct (final) output gets its row factors in the GEMM epilogue; planes leave them to the consumer
     launch_gemm(A, out ? inv : nullptr, W, P, N, stride, s->BN, N, K, p);
+    if (sg && sg->cols) {
+        if (out || sg->cols != (p.steps * 64) << sg->shift || sg->groups != (p.S + (1 << sg->shift) - 1) >> sg->shift) {
+            fprintf(stderr, "[fast_sft] column groups of the operand do not match the K chunks of the product\n"); abort();
+        }
+        return Planes{P, p.S, stride, N, inv, sg->shift, sg->groups};
+    }
     return Planes{P, p.S, stride, N, out ? nullptr : inv};
 }
 
@@ -269,10 +295,11 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
         ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
         ga.out16 = act16; ga.inv_scale = actinv;
+        ga.sg = scale_groups_for(s, wop(s, W_D, L, false), D, IS);
         launch_glu_fwd(ga, BN);
 
         // ff = act Wd^T, added by the next row kernel                          [:730-740]
-        pending = gemm(s, act16, actinv, wop(s, W_D, L, false), D, IS);
+        pending = gemm(s, act16, actinv, wop(s, W_D, L, false), D, IS, nullptr, &ga.sg);
     }
 
     // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
@@ -654,7 +681,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     if (qd > maxk) maxk = qd;
     if (2 * IS > maxk) maxk = 2 * IS;
     if (s->nq_ext > maxk) maxk = s->nq_ext;
-    s->a16 = hbuf(tiled_elems(BN, maxk)); s->a16_inv = fbuf(BN);
+    s->a16 = hbuf(tiled_elems(BN, maxk)); s->a16_inv = fbuf((size_t)BN * MAX_SCALE_GROUPS);
     s->ones = fbuf(BN);
     launch_fill_f32(at<float>(s->ones), 1.0f, BN);
     s->planes_cap = max_planes_elems(s);
