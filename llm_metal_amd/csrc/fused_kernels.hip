@@ -28,6 +28,17 @@ __device__ __forceinline__ void st_tiled4(half_t *out, size_t row, int k, int Kb
 }
 
 // zero the K padding [n, Kb*64) of a tiled row
+// Row of this workgroup (grid.x = rows).  Workgroups go to the eight XCDs round-robin by their linear id, and eight
+// consecutive rows of a tiled fp16 operand share every 128-byte line of it: rows 8k .. 8k+7 are given to one XCD, so the
+// pieces of a line meet in one L2 instead of reaching memory as eight partial writes.
+__device__ __forceinline__ size_t xcd_row()
+{
+    const unsigned id = blockIdx.x;
+    if (gridDim.x & 63) return id;
+    const unsigned x = id & 7, y = id >> 3;              // XCD, position within the XCD
+    return (size_t)(y >> 3) * 64 + x * 8 + (y & 7);
+}
+
 __device__ __forceinline__ void zero_tiled_pad(half_t *out, size_t row, int n, int Kb)
 {
     for (int i = n + threadIdx.x; i < Kb * 64; i += blockDim.x) out[tiled_index((int)row, i, Kb)] = (half_t)0;
@@ -55,7 +66,7 @@ template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_row();
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
     const bool padded = a.emb && a.n_valid > 0 && (int)r >= a.n_valid;      // zero rows past the sequence
@@ -414,7 +425,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [16 waves][32] partials
     __shared__ float sm[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const size_t row = blockIdx.x;
+    const size_t row = xcd_row();
     const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd, R = a.R;
     const int n = qd + 2 * kd + 2 * R;
     float *dhp = buf + n;
@@ -619,7 +630,7 @@ __device__ __forceinline__ float act_fwd(float g, int gelu)
 __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_row();
     const int IS = a.IS, nv = IS >> 2;
     float4 act[MAXV];
     float amax = 0.f;
@@ -661,10 +672,11 @@ __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
 // GEMM that reads the operand cuts K into chunks that do not straddle groups, so every plane of its result belongs to
 // one factor.  64 rows then occupy the whole GPU instead of 64 CUs.
 constexpr int GC = 256, MAXC = 2;                         // threads of a column-group workgroup; float4 per thread
+template <int GELU>                                       // compile-time: the kernel's code stays one straight run
 __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_row();
     const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(IS, c0 + a.sg.cols) - c0, nv = width >> 2;
     float4 act[MAXC], gu[2 * MAXC];
     float amax = 0.f;
@@ -685,8 +697,8 @@ __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
             const float4 g = gu[t], u = gu[MAXC + t];
             st4(a.gate_pre + r * IS + c0 + 4 * v, g);
             st4(a.up_val + r * IS + c0 + 4 * v, u);
-            act[t] = make_float4(act_fwd(g.x, a.gelu) * u.x, act_fwd(g.y, a.gelu) * u.y,
-                                 act_fwd(g.z, a.gelu) * u.z, act_fwd(g.w, a.gelu) * u.w);
+            act[t] = make_float4(act_fwd(g.x, GELU) * u.x, act_fwd(g.y, GELU) * u.y,
+                                 act_fwd(g.z, GELU) * u.z, act_fwd(g.w, GELU) * u.w);
             amax = fmaxf(amax, amax4(act[t]));
         }
     }
@@ -716,7 +728,7 @@ __device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, fl
 __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_row();
     const int IS = a.IS, nv = IS >> 2;
     float4 dg[MAXV], du[MAXV];
     float amax = 0.f;
@@ -757,6 +769,52 @@ __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
 
+// The same with the columns of the output row [dgate | dup] split among workgroups (grid (rows, groups), block GC), as
+// in k_glu_fwd_cols.  A group may lie in either half or straddle the middle, so a thread computes the half its output
+// column belongs to; the inputs of a column are then read twice in all, by different workgroups.
+template <int GELU>
+__global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
+{
+    __shared__ float sm[16];
+    const size_t r = xcd_row();
+    const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(2 * IS, c0 + a.sg.cols) - c0, nv = width >> 2;
+    float4 o[MAXC], dys[MAXC], gs[MAXC], us[MAXC];
+    float amax = 0.f;
+    {
+        size_t rows[MAXC]; int cols[MAXC]; bool ok[MAXC];
+#pragma unroll
+        for (int t = 0; t < MAXC; t++) {
+            const int v = threadIdx.x + t * GC, j = c0 + 4 * v;
+            rows[t] = r; cols[t] = j < IS ? j : j - IS; ok[t] = v < nv;
+            gs[t] = us[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (v < nv) { gs[t] = ld4(a.gate_pre + r * IS + cols[t]); us[t] = ld4(a.up_val + r * IS + cols[t]); }
+        }
+        planes_at4_multi<MAXC, 5>(a.in, rows, cols, ok, dys);
+    }
+#pragma unroll
+    for (int t = 0; t < MAXC; t++) {
+        const int v = threadIdx.x + t * GC, j = c0 + 4 * v;
+        o[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) {
+            float4 dg, du;
+            act_bwd(dys[t].x, gs[t].x, us[t].x, GELU, dg.x, du.x);
+            act_bwd(dys[t].y, gs[t].y, us[t].y, GELU, dg.y, du.y);
+            act_bwd(dys[t].z, gs[t].z, us[t].z, GELU, dg.z, du.z);
+            act_bwd(dys[t].w, gs[t].w, us[t].w, GELU, dg.w, du.w);
+            const bool first = j < IS;
+            o[t] = make_float4(first ? dg.x : du.x, first ? dg.y : du.y, first ? dg.z : du.z, first ? dg.w : du.w);
+            amax = fmaxf(amax, amax4(o[t]));
+        }
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax);
+    const int Kb = tiled_kb(2 * IS);
+#pragma unroll
+    for (int t = 0; t < MAXC; t++) { const int v = threadIdx.x + t * GC; if (v < nv) st_tiled4(a.out16, r, c0 + 4 * v, Kb, o[t], s); }
+    if (c0 + width == 2 * IS) zero_tiled_pad(a.out16, r, 2 * IS, Kb);
+    if (threadIdx.x == 0) a.inv_scale[r * gridDim.y + blockIdx.y] = 1.0f / s;
+}
+
 // ------------------------------------------------------------------ backward rows
 // dx_out = dx_prev + RNB(x_saved, sum(dy planes); g), clamped (rms_norm_train_backward,
 // shaders/q8_kernels.metal:584-625; residual_add; clamp_tensor :1155-1161;
@@ -767,7 +825,7 @@ template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
     __shared__ float sm[32];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_row();
     const int D = a.D, nv = D >> 2;
     float4 dy[MAXV], x[MAXV], g[MAXV];
     float ss = 0.f, dot = 0.f;
@@ -1065,7 +1123,8 @@ void launch_glu_fwd(const GluArgs &a, int rows)
     if (a.sg.cols) {
         require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC * MAXC && (long)a.sg.cols * a.sg.groups >= a.IS && (long)a.sg.cols * (a.sg.groups - 1) < a.IS,
                 "glu_fwd: column groups do not fit the row");
-        LAUNCH(k_glu_fwd_cols, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        if (a.gelu) LAUNCH(k_glu_fwd_cols<1>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        else LAUNCH(k_glu_fwd_cols<0>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
         return;
     }
     LAUNCH(k_glu_fwd, dim3(rows), dim3(RB), 0, a);
@@ -1074,6 +1133,13 @@ void launch_glu_bwd(const GluArgs &a, int rows)
 {
     require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_bwd: FFN width must be a multiple of 4, <= 12288");
     require(!a.in.scale_groups, "glu_bwd: input planes with grouped row factors are not supported");
+    if (a.sg.cols) {
+        require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC * MAXC && (long)a.sg.cols * a.sg.groups >= 2 * a.IS && (long)a.sg.cols * (a.sg.groups - 1) < 2 * a.IS,
+                "glu_bwd: column groups do not fit the row");
+        if (a.gelu) LAUNCH(k_glu_bwd_cols<1>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        else LAUNCH(k_glu_bwd_cols<0>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        return;
+    }
     LAUNCH(k_glu_bwd, dim3(rows), dim3(RB), 0, a);
 }
 

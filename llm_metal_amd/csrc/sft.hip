@@ -62,6 +62,8 @@ struct SFTState {
     MetalBuf *kT, *vT;                   // k_fin / v_sav once more, per head and transposed, for the matrix-core attention
     // transients
     MetalBuf *a16, *a16_inv;             // largest fp16 operand (BN x max K) and its row factors
+    MetalBuf *group_inv;                 // row factors per column group [BN][MAX_SCALE_GROUPS]: never the buffer the
+                                         // kernel that writes them reads its own input factors from
     MetalBuf *ones;                      // [BN] of 1.0f
     MetalBuf *planes;
     MetalBuf *logits, *dlogits, *dl16, *dl_inv;
@@ -173,7 +175,7 @@ size_t max_planes_elems(SFTState *s)
     return mx;
 }
 
-constexpr int MAX_SCALE_GROUPS = 64;                      // a16_inv holds this many factors per row
+constexpr int MAX_SCALE_GROUPS = 64;                      // group_inv holds this many factors per row
 
 // Column groups for the row kernel that writes the operand [BN, K] of the product with W [N, K]: as many groups as it
 // takes to put about two workgroups on every CU, each a power-of-two number of the GEMM's K chunks and at most 2048
@@ -294,12 +296,12 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         GluArgs ga{};
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
         ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
-        ga.out16 = act16; ga.inv_scale = actinv;
         ga.sg = scale_groups_for(s, wop(s, W_D, L, false), D, IS);
+        ga.out16 = act16; ga.inv_scale = ga.sg.cols ? at<float>(s->group_inv) : actinv;
         launch_glu_fwd(ga, BN);
 
         // ff = act Wd^T, added by the next row kernel                          [:730-740]
-        pending = gemm(s, act16, actinv, wop(s, W_D, L, false), D, IS, nullptr, &ga.sg);
+        pending = gemm(s, act16, ga.inv_scale, wop(s, W_D, L, false), D, IS, nullptr, &ga.sg);
     }
 
     // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
@@ -374,9 +376,10 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         GluArgs gb{};
         gb.in = pd; gb.IS = IS; gb.gelu = gemma;
         gb.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); gb.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
-        gb.out16 = a16; gb.inv_scale = ainv;
+        if (mode == BWD_LORA) gb.sg = scale_groups_for(s, wop(s, W_GU, L, true), D, 2 * IS);
+        gb.out16 = a16; gb.inv_scale = gb.sg.cols ? at<float>(s->group_inv) : ainv;
         launch_glu_bwd(gb, BN);
-        Planes pgu = gemm(s, a16, ainv, wop(s, W_GU, L, true), D, 2 * IS);
+        Planes pgu = gemm(s, a16, gb.inv_scale, wop(s, W_GU, L, true), D, 2 * IS, nullptr, &gb.sg);
         if (mode != BWD_LORA)                                                 // gate and up as one matrix [:817-833, 853-869]
             weight_grad(s, mode, lr, a16, ainv, 2 * IS, at<half_t>(s->ln2_16, L * s->st_ln1), at<float>(s->ln2_inv, (size_t)L * BN), D,
                         s->wgu, s->wguT, s->ggu, L * s->st_gu, L * s->st_guT);
@@ -681,7 +684,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     if (qd > maxk) maxk = qd;
     if (2 * IS > maxk) maxk = 2 * IS;
     if (s->nq_ext > maxk) maxk = s->nq_ext;
-    s->a16 = hbuf(tiled_elems(BN, maxk)); s->a16_inv = fbuf((size_t)BN * MAX_SCALE_GROUPS);
+    s->a16 = hbuf(tiled_elems(BN, maxk)); s->a16_inv = fbuf(BN); s->group_inv = fbuf((size_t)BN * MAX_SCALE_GROUPS);
     s->ones = fbuf(BN);
     launch_fill_f32(at<float>(s->ones), 1.0f, BN);
     s->planes_cap = max_planes_elems(s);
@@ -729,7 +732,7 @@ void sft_state_free(SFTState *s)
                        s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
-                       s->gate_pre, s->up_val, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->ones, s->planes,
+                       s->gate_pre, s->up_val, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->group_inv, s->ones, s->planes,
                        s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
                        s->dq, s->dk, s->dv, s->dq_f, s->dh, s->ce_part,
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
