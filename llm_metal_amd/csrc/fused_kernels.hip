@@ -28,17 +28,6 @@ __device__ __forceinline__ void st_tiled4(half_t *out, size_t row, int k, int Kb
 }
 
 // zero the K padding [n, Kb*64) of a tiled row
-// Row of this workgroup (grid.x = rows).  Workgroups go to the eight XCDs round-robin by their linear id, and eight
-// consecutive rows of a tiled fp16 operand share every 128-byte line of it: rows 8k .. 8k+7 are given to one XCD, so the
-// pieces of a line meet in one L2 instead of reaching memory as eight partial writes.
-__device__ __forceinline__ size_t xcd_row()
-{
-    const unsigned id = blockIdx.x;
-    if (gridDim.x & 63) return id;
-    const unsigned x = id & 7, y = id >> 3;              // XCD, position within the XCD
-    return (size_t)(y >> 3) * 64 + x * 8 + (y & 7);
-}
-
 __device__ __forceinline__ void zero_tiled_pad(half_t *out, size_t row, int n, int Kb)
 {
     for (int i = n + threadIdx.x; i < Kb * 64; i += blockDim.x) out[tiled_index((int)row, i, Kb)] = (half_t)0;
@@ -66,7 +55,7 @@ template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = xcd_row();
+    const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
     const bool padded = a.emb && a.n_valid > 0 && (int)r >= a.n_valid;      // zero rows past the sequence
@@ -425,7 +414,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [16 waves][32] partials
     __shared__ float sm[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const size_t row = xcd_row();
+    const size_t row = blockIdx.x;
     const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd, R = a.R;
     const int n = qd + 2 * kd + 2 * R;
     float *dhp = buf + n;
@@ -630,7 +619,7 @@ __device__ __forceinline__ float act_fwd(float g, int gelu)
 __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = xcd_row();
+    const size_t r = blockIdx.x;
     const int IS = a.IS, nv = IS >> 2;
     float4 act[MAXV];
     float amax = 0.f;
@@ -676,7 +665,7 @@ template <int GELU>                                       // compile-time: the k
 __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = xcd_row();
+    const size_t r = blockIdx.x;
     const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(IS, c0 + a.sg.cols) - c0, nv = width >> 2;
     float4 act[MAXC], gu[2 * MAXC];
     float amax = 0.f;
@@ -728,7 +717,7 @@ __device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, fl
 __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = xcd_row();
+    const size_t r = blockIdx.x;
     const int IS = a.IS, nv = IS >> 2;
     float4 dg[MAXV], du[MAXV];
     float amax = 0.f;
@@ -776,7 +765,7 @@ template <int GELU>
 __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = xcd_row();
+    const size_t r = blockIdx.x;
     const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(2 * IS, c0 + a.sg.cols) - c0, nv = width >> 2;
     float4 o[MAXC], dys[MAXC], gs[MAXC], us[MAXC];
     float amax = 0.f;
@@ -825,7 +814,7 @@ template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
     __shared__ float sm[32];
-    const size_t r = xcd_row();
+    const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 dy[MAXV], x[MAXV], g[MAXV];
     float ss = 0.f, dot = 0.f;
