@@ -150,10 +150,25 @@ __device__ __forceinline__ void c_chunk_mfma(Acc2 &acc, const XChunk &x, const C
 // chunks 0-2, which the caller may have requested long before.
 struct CRing { CChunk c[4]; };
 
+template <int M32>
 __device__ __forceinline__ void c_ring_start(CRing &r, const float *ccol_lane, size_t ldc, int nk, int hh, int n_valid)
 {
 #pragma unroll
-    for (int q = 0; q < 3; q++) c_chunk_load(r.c[q], ccol_lane, ldc, min(32 * q, nk - 32), hh, n_valid);
+    for (int q = 0; q < (M32 == 2 ? 2 : 3); q++) c_chunk_load(r.c[q], ccol_lane, ldc, min(32 * q, nk - 32), hh, n_valid);
+}
+
+// The product for sequences of at most 64 keys: both chunks of C are in the ring already.
+__device__ __forceinline__ float16v tile_xc_2(const __bf16 *Xh, int ldxh, int xlo, int nk, int lane, const CRing &ring)
+{
+    const int hh = lane >> 5;
+    const __bf16 *x = Xh + (size_t)(lane & 31) * ldxh + 16 * hh;
+    Acc2 acc{zero16(), zero16()};
+    XChunk xr[2];
+    x_chunk_load(xr[0], x, xlo, 0);
+    x_chunk_load(xr[1], x, xlo, nk - 32);
+    c_chunk_mfma(acc, xr[0], ring.c[0]);
+    if (nk > 32) c_chunk_mfma(acc, xr[1], ring.c[1]);
+    return acc.a + acc.b;
 }
 
 __device__ __forceinline__ float16v tile_xc(const __bf16 *Xh, int ldxh, int xlo, int nk, const float *ccol_lane, size_t ldc, int n_valid,
@@ -259,7 +274,9 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
 }
 
 // grid (query blocks of 32, Hq, batch), block 256; LDS: Ahi, Alo [32][HD+8] bf16, Xs[32][ldx] fp32 / bf16 pairs
-template <int BWD, int HD>
+// M32: 32-key blocks a row can hold (2, 8, 16 or 32: sequences up to 64, 256, 512, 1024); a template parameter so
+// that the kernel's code is one straight run (the kernel runs once per workgroup, and what it skips it still fetches).
+template <int BWD, int HD, int M32>
 __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
 {
     extern __shared__ float lds[];
@@ -292,7 +309,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     b_tile_load<CB>(bt0, b_item(0), ldt);
     CRing cring;
     const float *c_lane0 = a.C + r0 * kd + hk * HD + l31;
-    c_ring_start(cring, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, nk, hh, N);
+    c_ring_start<M32>(cring, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, nk, hh, N);
 
     // ---- A rows into LDS (rows past the sequence as zeros); the loads of all HD / 32 rounds are issued together
     {
@@ -336,27 +353,30 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
             tile_abt<CB>(acc, Ahi, Alo, lda, c * CB, lane, bt);
             if (c == NCB - 1) put_x(acc.a + acc.b, jb);
         };
-        for (int q = 0; q < nitems; q += 2) {
-            b_tile_load<CB>(bt1, b_item(q + 1), ldt);
-            run(q, bt0);
-            b_tile_load<CB>(bt0, b_item(q + 2), ldt);
-            if (q + 1 < nitems) run(q + 1, bt1);
+        if constexpr (((M32 + 3) / 4) * NCB == 1) {       // at most one item per wave: no second tile on its way
+            if (nitems) run(0, bt0);
+        } else {
+            for (int q = 0; q < nitems; q += 2) {
+                b_tile_load<CB>(bt1, b_item(q + 1), ldt);
+                run(q, bt0);
+                b_tile_load<CB>(bt0, b_item(q + 2), ldt);
+                if (q + 1 < nitems) run(q + 1, bt1);
+            }
         }
     }
     __syncthreads();
 
     // ---- row step
-    if (N <= 64) row_step<BWD, 2>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);                 // whole rows of N entries are written
-    else if (N <= 256) row_step<BWD, 8>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);
-    else if (N <= 512) row_step<BWD, 16>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);
-    else row_step<BWD, 32>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);
+    row_step<BWD, M32>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);             // whole rows of N entries are written
     __syncthreads();
 
     // ---- phase 3: Y = X C, one 32-column block of the head per wave and round
     const int Kb = tiled_kb(qd);
     for (int dt = wave; dt * 32 < HD; dt += 4) {
-        if (dt != wave) c_ring_start(cring, c_lane0 + dt * 32, (size_t)kd, nk, hh, N);
-        const float16v acc = tile_xc(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
+        if (dt != wave) c_ring_start<M32>(cring, c_lane0 + dt * 32, (size_t)kd, nk, hh, N);
+        float16v acc;
+        if constexpr (M32 == 2) acc = tile_xc_2(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, lane, cring);
+        else acc = tile_xc(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
         const int d = dt * 32 + l31;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
@@ -440,13 +460,22 @@ __global__ __launch_bounds__(256) void k_attn_dkv_tile(AttnDkvArgs a)
 
 size_t tile_lds_bytes(int hd, int seq) { return (size_t)32 * (hd + 8 + ((seq + 31) & ~31) + 4) * sizeof(float); }
 
+template <int BWD, int HD, int M32>
+void launch_tile_m(const AttnTileArgs &a)
+{
+    static bool attr_set = false;
+    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_attn_tile<BWD, HD, M32>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); attr_set = true; }
+    const size_t lds = tile_lds_bytes(HD, a.seq);
+    LAUNCH((k_attn_tile<BWD, HD, M32>), dim3((a.seq + 31) / 32, a.Hq, a.batch), dim3(256), lds, a);
+}
+
 template <int BWD, int HD>
 void launch_tile_hd(const AttnTileArgs &a)
 {
-    static bool attr_set = false;
-    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_attn_tile<BWD, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); attr_set = true; }
-    const size_t lds = tile_lds_bytes(HD, a.seq);
-    LAUNCH((k_attn_tile<BWD, HD>), dim3((a.seq + 31) / 32, a.Hq, a.batch), dim3(256), lds, a);
+    if (a.seq <= 64) launch_tile_m<BWD, HD, 2>(a);
+    else if (a.seq <= 256) launch_tile_m<BWD, HD, 8>(a);
+    else if (a.seq <= 512) launch_tile_m<BWD, HD, 16>(a);
+    else launch_tile_m<BWD, HD, 32>(a);
 }
 
 template <int BWD>
