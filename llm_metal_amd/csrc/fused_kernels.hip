@@ -145,6 +145,9 @@ __global__ void k_rope_table(float2 *tab, int seq, int half, int hd, float theta
 // [rows][H*hd] layout, so the reference's three head transposes, repeat_kv and
 // five buffer copies disappear.  A lane owns the pairs (d, d + hd/2).
 constexpr int MAXP = 4;                                   // pairs per lane: hd <= 512
+// NP: pairs per lane compiled in (1 serves head_dim <= 128); RK: the LoRA rank compiled in (16), 0 for none, -1 for any.
+// The kernel runs once per wave, so what is compiled out is code it does not have to fetch.
+template <int NP, int RK>
 __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -158,36 +161,36 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
     const int h = kind == 0 ? slot : (kind == 1 ? slot - a.Hq : slot - a.Hq - a.Hkv);
     const int col0 = kind == 0 ? h * hd : (kind == 1 ? qd + h * hd : qd + kd + h * hd);
     const int t0 = qd + 2 * kd + (kind == 2 ? a.R : 0);
-    const bool lora = a.R > 0 && kind != 1;
+    const bool lora = RK != 0 && a.R > 0 && kind != 1;
     const float *B = kind == 0 ? a.Bq : a.Bv;
 
-    // everything this lane reads from the planes in one go: positions p (first half of the head), MAXP + p (second
-    // half) and 2 MAXP (the lane's entry of x A^T)
-    float x0[MAXP], x1[MAXP], tval;
+    // everything this lane reads from the planes in one go: positions p (first half of the head), NP + p (second
+    // half) and 2 NP (the lane's entry of x A^T)
+    float x0[NP], x1[NP], tval;
     {
-        int cols[2 * MAXP + 1]; bool ok[2 * MAXP + 1]; float got[2 * MAXP + 1];
+        int cols[2 * NP + 1]; bool ok[2 * NP + 1]; float got[2 * NP + 1];
 #pragma unroll
-        for (int p = 0; p < MAXP; p++) {
+        for (int p = 0; p < NP; p++) {
             const int d = lane + 64 * p;
-            cols[p] = col0 + d; cols[MAXP + p] = col0 + d + half; ok[p] = ok[MAXP + p] = d < half;
+            cols[p] = col0 + d; cols[NP + p] = col0 + d + half; ok[p] = ok[NP + p] = d < half;
         }
-        cols[2 * MAXP] = t0 + lane; ok[2 * MAXP] = lora && lane < a.R;
-        planes_at_multi<2 * MAXP + 1, 5>(a.qkv, row, cols, ok, got);
+        cols[2 * NP] = t0 + lane; ok[2 * NP] = lora && lane < a.R;
+        planes_at_multi<2 * NP + 1, 5>(a.qkv, row, cols, ok, got);
 #pragma unroll
-        for (int p = 0; p < MAXP; p++) { x0[p] = got[p]; x1[p] = got[MAXP + p]; }
-        tval = got[2 * MAXP];
+        for (int p = 0; p < NP; p++) { x0[p] = got[p]; x1[p] = got[NP + p]; }
+        tval = got[2 * NP];
     }
     if (lora && h == 0 && lane < a.R) (kind == 0 ? a.tq : a.tv)[row * a.R + lane] = tval;
 
     float ss = 0.f;
 #pragma unroll
-    for (int p = 0; p < MAXP; p++) {
+    for (int p = 0; p < NP; p++) {
         const int d = lane + 64 * p;
         if (lora && 64 * p < half) {                          // uniform branch: the broadcasts stay convergent
             float acc0 = 0.f, acc1 = 0.f;
             const float *b0 = B + (size_t)(h * hd + (d < half ? d : 0)) * a.R;
             const float *b1 = b0 + (size_t)half * a.R;
-            if (a.R == 16) {                                   // t through scalar registers, whole rows of B as 16-byte loads
+            if constexpr (RK == 16) {                          // t through scalar registers, whole rows of B as 16-byte loads
                 float4 w0[4], w1[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) { w0[i] = w1[i] = make_float4(0.f, 0.f, 0.f, 0.f); if (d < half) { w0[i] = ld4(b0 + 4 * i); w1[i] = ld4(b1 + 4 * i); } }
@@ -200,6 +203,7 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
                     acc0 += t0 * w0[i].x; acc0 += t1 * w0[i].y; acc0 += t2 * w0[i].z; acc0 += t3 * w0[i].w;
                     acc1 += t0 * w1[i].x; acc1 += t1 * w1[i].y; acc1 += t2 * w1[i].z; acc1 += t3 * w1[i].w;
                 }
+            } else if constexpr (RK == 0) {
             } else if ((a.R & 3) == 0) {
                 for (int r4 = 0; r4 < a.R; r4 += 4) {
                     float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w1 = w0;
@@ -222,7 +226,7 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
     }
     if (kind == 2) {
 #pragma unroll
-        for (int p = 0; p < MAXP; p++) {
+        for (int p = 0; p < NP; p++) {
             const int d = lane + 64 * p;
             if (d < half) {
                 a.v_out[row * kd + h * hd + d] = x0[p]; a.v_out[row * kd + h * hd + d + half] = x1[p];
@@ -242,7 +246,7 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
     const int W = kind == 0 ? qd : kd;
     const int pos = (int)(row % a.seq);
 #pragma unroll
-    for (int p = 0; p < MAXP; p++) {
+    for (int p = 0; p < NP; p++) {
         const int d = lane + 64 * p;
         if (d >= half) continue;
         const size_t o = row * W + h * hd + d;
@@ -409,6 +413,8 @@ __global__ __launch_bounds__(TB) void k_attn_bwd_dkv(AttnBwdArgs a)
 // row [dq | dk | dv | dh_q | dh_v] as one scaled fp16 operand so that a single GEMM
 // against [Wq; Wk; Wv; A_q; A_v]^T yields dq Wq + dk Wk + dv Wv + dh_q A_q + dh_v A_v
 // (src/nn/fast_sft.c:953-971).
+// NP, RK: pairs per lane and LoRA rank compiled in, as in k_qkv_post.
+template <int NP, int RK>
 __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
 {
     extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [16 waves][32] partials
@@ -424,10 +430,10 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     constexpr int SU = 3;
     const int nslots = a.Hq + a.Hkv;
     for (int s0 = wave; s0 < nslots; s0 += (RB / 64) * SU) {
-        float g0[SU][MAXP], g1[SU][MAXP], p0[SU][MAXP], p1[SU][MAXP], w0[SU][MAXP], w1[SU][MAXP];
-        float2 cs[MAXP];
+        float g0[SU][NP], g1[SU][NP], p0[SU][NP], p1[SU][NP], w0[SU][NP], w1[SU][NP];
+        float2 cs[NP];
 #pragma unroll
-        for (int p = 0; p < MAXP; p++) {
+        for (int p = 0; p < NP; p++) {
             const int d = lane + 64 * p;
             cs[p] = d < half ? a.rope[(size_t)pos * half + d] : make_float2(1.f, 0.f);
         }
@@ -440,7 +446,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
             const float *xp = (isk ? a.k_pre : a.q_pre) + row * W + h * hd;
             const float *g = isk ? a.g_k : a.g_q;
 #pragma unroll
-            for (int p = 0; p < MAXP; p++) {
+            for (int p = 0; p < NP; p++) {
                 const int d = lane + 64 * p;
                 g0[u][p] = g1[u][p] = p0[u][p] = p1[u][p] = w0[u][p] = w1[u][p] = 0.f;
                 if (d < half) {
@@ -453,10 +459,10 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
 #pragma unroll
         for (int u = 0; u < SU; u++) {
             const int slot = s0 + (RB / 64) * u;
-            float y0[MAXP], y1[MAXP];
+            float y0[NP], y1[NP];
             float ss = 0.f, dot = 0.f;
 #pragma unroll
-            for (int p = 0; p < MAXP; p++) {
+            for (int p = 0; p < NP; p++) {
                 y0[p] = g0[u][p] * cs[p].x + g1[u][p] * cs[p].y;
                 y1[p] = -g0[u][p] * cs[p].y + g1[u][p] * cs[p].x;
                 ss += p0[u][p] * p0[u][p] + p1[u][p] * p1[u][p];
@@ -469,7 +475,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
             const float inv = rsqrtf(ss / (float)hd + a.eps);
             const float coeff = dot * inv * inv / (float)hd;
 #pragma unroll
-            for (int p = 0; p < MAXP; p++) {
+            for (int p = 0; p < NP; p++) {
                 const int d = lane + 64 * p;
                 if (d >= half) continue;
                 const float d0 = (w0[u][p] * y0[p] - coeff * p0[u][p]) * inv;
@@ -486,11 +492,8 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     // dh[r] = sc * sum_c d[c] * B[c][r].  Rank 16 (the common case): four threads share a row of B (16 floats, one
     // float4 each) and 256 such groups split the columns, so a thread keeps 4 + 4 sums and a wave reduces over its 16
     // groups in four shuffle steps; other ranks: a thread walks whole rows of B.
-    if (R > 0) {
-        float acc[32];
-#pragma unroll
-        for (int r = 0; r < 32; r++) acc[r] = 0.f;
-        if (R == 16) {
+    if (RK != 0 && R > 0) {
+        if constexpr (RK == 16) {
             const int sub = threadIdx.x & 3;
             float aq[4] = {0.f, 0.f, 0.f, 0.f}, av[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
@@ -511,6 +514,9 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
                 for (int e = 0; e < 4; e++) { dhp[wave * 32 + 4 * lane + e] = aq[e]; dhp[wave * 32 + 16 + 4 * lane + e] = av[e]; }
             }
         } else {
+        float acc[32];
+#pragma unroll
+        for (int r = 0; r < 32; r++) acc[r] = 0.f;
 #pragma unroll 4
         for (int c = threadIdx.x; c < qd + kd; c += RB) {
             const int isv = c >= qd;
@@ -1069,7 +1075,16 @@ void launch_qkv_post(const QkvPostArgs &a, int rows)
     const size_t tasks = (size_t)rows * (a.Hq + 2 * a.Hkv);
     QkvPostArgs b = a;
     b.rows = rows;
-    LAUNCH(k_qkv_post, dim3((unsigned)((tasks + 3) / 4)), dim3(TB), 0, b);
+    const dim3 grid((unsigned)((tasks + 3) / 4));
+    if (a.hd <= 128) {
+        if (a.R == 16) LAUNCH((k_qkv_post<1, 16>), grid, dim3(TB), 0, b);
+        else if (a.R == 0) LAUNCH((k_qkv_post<1, 0>), grid, dim3(TB), 0, b);
+        else LAUNCH((k_qkv_post<1, -1>), grid, dim3(TB), 0, b);
+    } else {
+        if (a.R == 16) LAUNCH((k_qkv_post<MAXP, 16>), grid, dim3(TB), 0, b);
+        else if (a.R == 0) LAUNCH((k_qkv_post<MAXP, 0>), grid, dim3(TB), 0, b);
+        else LAUNCH((k_qkv_post<MAXP, -1>), grid, dim3(TB), 0, b);
+    }
 }
 
 void launch_attn_fwd(const AttnFwdArgs &a)
@@ -1091,7 +1106,15 @@ void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
 {
     const size_t n = (size_t)(a.Hq + 2 * a.Hkv) * a.hd + 2 * a.R + 16 * 32;
     require(a.hd <= 2 * 64 * MAXP && n * 4 <= 64 * 1024 && a.R <= 16, "qkv_bwd: row of dq|dk|dv must fit 64 KB of LDS, rank <= 16");
-    LAUNCH(k_qkv_bwd_rows, dim3(rows), dim3(RB), n * 4, a);
+    if (a.hd <= 128) {
+        if (a.R == 16) LAUNCH((k_qkv_bwd_rows<1, 16>), dim3(rows), dim3(RB), n * 4, a);
+        else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<1, 0>), dim3(rows), dim3(RB), n * 4, a);
+        else LAUNCH((k_qkv_bwd_rows<1, -1>), dim3(rows), dim3(RB), n * 4, a);
+    } else {
+        if (a.R == 16) LAUNCH((k_qkv_bwd_rows<MAXP, 16>), dim3(rows), dim3(RB), n * 4, a);
+        else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<MAXP, 0>), dim3(rows), dim3(RB), n * 4, a);
+        else LAUNCH((k_qkv_bwd_rows<MAXP, -1>), dim3(rows), dim3(RB), n * 4, a);
+    }
 }
 
 int lora_grad_blocks(int D, int qd, int kd, int R)
