@@ -496,13 +496,19 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         if constexpr (RK == 16) {
             const int sub = threadIdx.x & 3;
             float aq[4] = {0.f, 0.f, 0.f, 0.f}, av[4] = {0.f, 0.f, 0.f, 0.f};
+            // two plain loops (q columns, then v columns), so that the loads of B of eight trips can be in flight at once:
+            // every workgroup reads all of B, and what bounds it is how much of that one CU keeps in flight
+#pragma unroll 8
+            for (int c = threadIdx.x >> 2; c < qd; c += RB / 4) {
+                const float x = buf[c];
+                const float4 w = ld4(a.Bq + (size_t)c * 16 + 4 * sub);
+                aq[0] += x * w.x; aq[1] += x * w.y; aq[2] += x * w.z; aq[3] += x * w.w;
+            }
 #pragma unroll 4
-            for (int c = threadIdx.x >> 2; c < qd + kd; c += RB / 4) {
-                const int isv = c >= qd;
-                const float x = buf[isv ? c + kd : c];
-                const float4 w = ld4((isv ? a.Bv + (size_t)(c - qd) * 16 : a.Bq + (size_t)c * 16) + 4 * sub);
-                if (isv) { av[0] += x * w.x; av[1] += x * w.y; av[2] += x * w.z; av[3] += x * w.w; }
-                else { aq[0] += x * w.x; aq[1] += x * w.y; aq[2] += x * w.z; aq[3] += x * w.w; }
+            for (int c = threadIdx.x >> 2; c < kd; c += RB / 4) {
+                const float x = buf[qd + kd + c];
+                const float4 w = ld4(a.Bv + (size_t)c * 16 + 4 * sub);
+                av[0] += x * w.x; av[1] += x * w.y; av[2] += x * w.z; av[3] += x * w.w;
             }
 #pragma unroll
             for (int e = 0; e < 4; e++) {
