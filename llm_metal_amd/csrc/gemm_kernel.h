@@ -87,16 +87,15 @@ __device__ __forceinline__ void load_w_q8_cols(half8 (&w)[4], const WeightOp &W,
 // it all workgroups of a chunk ask L2 for the same activation lines at the same moment.
 // SCALE: multiply row m of the result by a_inv_scale[m] here (used when the output is final, S == 1);
 // otherwise the consumer of the partial planes applies the row factors.
-// NW (4, 8 or 16 waves) trades partial planes for workgroup size: the waves of a workgroup split its K chunk
-// and add their accumulators through LDS, so a larger workgroup covers a longer chunk and the launch writes
-// fewer planes for the same number of waves in flight.
+// NW = 4: the waves of a workgroup split its K chunk and add their accumulators through LDS; each then stores a quarter
+// of the tile.
 // WF: weight format (WeightOp::fmt).  1: row blocks below W.nbq are Q8_0 tiles, the rest F16 tiles
 // (the trainable LoRA rows of the fused QKV weight); the planner keeps W.nbq a multiple of NB, so a
 // workgroup is of one kind.  2: K steps below W.kbq are Q8_0 tiles with column scales, the rest F16.
 template <int NB, int NW, int ROTATE, int SCALE, int WF>
 __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 {
-    extern __shared__ float red[];                       // [NW/2][2*NB*16 regs][64 lanes]
+    extern __shared__ float red[];                       // [NW][NB*16 regs][64 lanes]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb0 = blockIdx.x * NB, mb0 = blockIdx.z * 2;
@@ -151,57 +150,53 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
                     acc[mb][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mb][j], w[b][j], acc[mb][b], 0, 0, 0);
     }
 
-    // add the waves' accumulators in log2(NW) rounds through LDS (lane fastest => conflict-free):
-    // in every round the upper half of the remaining waves parks its registers and the lower half adds them
-    constexpr int REGS = 2 * NB * 16;
+    // Add the four waves' accumulators through LDS so that every wave ends up with the finished sums of a quarter of
+    // the tile and stores that quarter: the registers are numbered i = (mb * NB + b) * 16 + v; in round one the waves
+    // w and w ^ 2 exchange halves (waves 0, 1 keep the lower half), in round two the waves w and w ^ 1 exchange quarters
+    // of the half they kept.  Wave w finishes the registers [w * Q, (w + 1) * Q).
+    static_assert(NW == 4, "the exchange below is written for four waves");
+    constexpr int REGS = 2 * NB * 16, H = REGS / 2, Q = REGS / 4;
+#define ACC_AT(i) acc[(i) / (NB * 16)][((i) / 16) % NB][(i) % 16]
+    {
+        float *mine = red + (size_t)wave * H * 64;
+        const float *theirs = red + (size_t)(wave ^ 2) * H * 64;
+        if (wave < 2) {
 #pragma unroll
-    for (int half = NW / 2; half >= 1; half >>= 1) {
-        if (wave >= half && wave < 2 * half) {
-            float *slot = red + (size_t)(wave - half) * REGS * 64;
+            for (int k = 0; k < H; k++) mine[k * 64 + lane] = ACC_AT(H + k);
+        } else {
 #pragma unroll
-            for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                for (int b = 0; b < NB; b++)
-#pragma unroll
-                    for (int v = 0; v < 16; v++) slot[((mb * NB + b) * 16 + v) * 64 + lane] = acc[mb][b][v];
+            for (int k = 0; k < H; k++) mine[k * 64 + lane] = ACC_AT(k);
         }
         __syncthreads();
-        if (wave < half) {
-            const float *slot = red + (size_t)wave * REGS * 64;
+        if (wave < 2) {
 #pragma unroll
-            for (int mb = 0; mb < 2; mb++)
+            for (int k = 0; k < H; k++) ACC_AT(k) += theirs[k * 64 + lane];
+        } else {
 #pragma unroll
-                for (int b = 0; b < NB; b++)
-#pragma unroll
-                    for (int v = 0; v < 16; v++) acc[mb][b][v] += slot[((mb * NB + b) * 16 + v) * 64 + lane];
+            for (int k = 0; k < H; k++) ACC_AT(H + k) += theirs[k * 64 + lane];
         }
-        if (half > 1) __syncthreads();
+        __syncthreads();                                  // all have read before the slots are written again
     }
-    if (wave != 0) return;
-    // the row factors of the 16 rows of a block are fetched here, block by block, where the K loop's registers are free
-    // (holding all 32 through the loop costs a wave of occupancy per SIMD)
     float *Pp = g.P + (size_t)blockIdx.y * g.plane_stride;
-#pragma unroll
-    for (int mb = 0; mb < 2; mb++) {
-        float rsc[16];
-        if (SCALE) {
-#pragma unroll
-            for (int v = 0; v < 16; v++) rsc[v] = g.a_inv_scale[min((mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), M - 1)];
-        }
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                float sres = acc[mb][b][v];
-                // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4
-                const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                const int n = (nb0 + b) * 32 + r;
-                if (m < M && n < N) {
-                    if (SCALE) sres *= rsc[v];
-                    Pp[(size_t)m * g.ldp + n] = sres;
-                }
-            }
-    }
+    float *mine = red + (size_t)wave * Q * 64;
+    const float *theirs = red + (size_t)(wave ^ 1) * Q * 64;
+#define QUARTER_GIVE(W) if (wave == (W)) { _Pragma("unroll") for (int k = 0; k < Q; k++) mine[k * 64 + lane] = ACC_AT(((W) ^ 1) * Q + k); }
+    QUARTER_GIVE(0) QUARTER_GIVE(1) QUARTER_GIVE(2) QUARTER_GIVE(3)
+#undef QUARTER_GIVE
+    __syncthreads();
+    // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4.  SCALE: the row factors
+    // are fetched here, where the K loop's registers are free (holding them through the loop costs a wave of occupancy).
+#define QUARTER_STORE(W) if (wave == (W)) { \
+        _Pragma("unroll") for (int k = 0; k < Q; k++) { \
+            constexpr int i0 = (W) * Q; \
+            const int i = i0 + k, mb = i / (NB * 16), b = (i / 16) % NB, v = i % 16; \
+            const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), n = (nb0 + b) * 32 + r; \
+            float sres = ACC_AT(i0 + k) + theirs[k * 64 + lane]; \
+            if (m < M && n < N) { if (SCALE) sres *= g.a_inv_scale[m]; Pp[(size_t)m * g.ldp + n] = sres; } \
+        } }
+    QUARTER_STORE(0) QUARTER_STORE(1) QUARTER_STORE(2) QUARTER_STORE(3)
+#undef QUARTER_STORE
+#undef ACC_AT
 }
 
 }  // namespace lmhip
