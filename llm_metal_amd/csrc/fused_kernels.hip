@@ -615,6 +615,86 @@ __global__ __launch_bounds__(TB) void k_lora_grads(LoraGradArgs a)
     if (threadIdx.x == 0) a.sq_slots[blockIdx.x] = sq;
 }
 
+// The same for rank R (16), laid out for coalesced reads: a thread owns one column of dY and forms the R entries of
+// its row of dB (or one column d of the input and the 2R entries dA_q[:, d], dA_v[:, d]), looping over the rows with the
+// R (2R) factors of a row coming from LDS.  Every sum runs over the rows in the same order as above, so the results are
+// the same; only the partial sums of squares are grouped differently.  grid.x = lora_grad_blocks(), block 256.
+template <int R>
+__global__ __launch_bounds__(256) void k_lora_grads_rank(LoraGradArgs a)
+{
+    __shared__ float ts[64 * 2 * R];
+    __shared__ float sm[16];
+    {                                                     // blockIdx.y = layer
+        const size_t L = blockIdx.y;
+        a.dq_f += L * a.st_dq; a.dv_f += L * a.st_dv; a.tq += L * a.st_t; a.tv += L * a.st_t; a.dh += L * a.st_dh;
+        a.ln16 += L * a.st_ln16; a.ln_inv_scale += L * a.st_lninv; a.grad += L * a.st_grad; a.sq_slots += L * a.st_slots;
+    }
+    const int nbq = (a.qd + 255) / 256, nbv = (a.kd + 255) / 256;
+    const int bx = blockIdx.x, tid = threadIdx.x;
+    const size_t nA = (size_t)R * a.D, nBq = (size_t)a.qd * R;
+    float sq = 0.f;
+    if (bx < nbq + nbv) {                                 // dB_q, dB_v
+        const bool isv = bx >= nbq;
+        const int c = (isv ? bx - nbq : bx) * 256 + tid, W = isv ? a.kd : a.qd;
+        const float *dy = isv ? a.dv_f : a.dq_f, *t = isv ? a.tv : a.tq;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = 0.f;
+        for (int i0 = 0; i0 < a.rows; i0 += 64) {
+            const int nr = min(64, a.rows - i0);
+            __syncthreads();
+            for (int e = tid; e < nr * R; e += 256) ts[e] = t[(size_t)i0 * R + e];
+            __syncthreads();
+            if (c < W) {
+#pragma unroll 8
+                for (int i = 0; i < nr; i++) {
+                    const float y = dy[(size_t)(i0 + i) * W + c];
+#pragma unroll
+                    for (int r = 0; r < R; r++) acc[r] += y * ts[i * R + r];
+                }
+            }
+        }
+        if (c < W) {
+            float *out = a.grad + (isv ? 2 * nA + nBq : nA) + (size_t)c * R;
+#pragma unroll
+            for (int r = 0; r < R; r += 4) {
+                const float4 gv = make_float4(acc[r] * a.sc, acc[r + 1] * a.sc, acc[r + 2] * a.sc, acc[r + 3] * a.sc);
+                st4(out + r, gv);
+                sq += sumsq4(gv);
+            }
+        }
+    } else {                                              // dA_q, dA_v
+        const int d = (bx - nbq - nbv) * 256 + tid, Kb = tiled_kb(a.D);
+        float aq[R], av[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) aq[r] = av[r] = 0.f;
+        for (int i0 = 0; i0 < a.rows; i0 += 64) {
+            const int nr = min(64, a.rows - i0);
+            __syncthreads();
+            for (int e = tid; e < nr * 2 * R; e += 256) ts[e] = a.dh[(size_t)i0 * 2 * R + e];
+            __syncthreads();
+            if (d < a.D) {
+#pragma unroll 4
+                for (int i = 0; i < nr; i++) {
+                    const float x = h2f(a.ln16[tiled_index(i0 + i, d, Kb)]) * a.ln_inv_scale[i0 + i];
+#pragma unroll
+                    for (int r = 0; r < R; r++) { aq[r] += ts[i * 2 * R + r] * x; av[r] += ts[i * 2 * R + R + r] * x; }
+                }
+            }
+        }
+        if (d < a.D) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                a.grad[(size_t)r * a.D + d] = aq[r];
+                a.grad[nA + nBq + (size_t)r * a.D + d] = av[r];
+                sq += aq[r] * aq[r] + av[r] * av[r];
+            }
+        }
+    }
+    sq = block_sum(sq, sm);
+    if (tid == 0) a.sq_slots[bx] = sq;
+}
+
 // ------------------------------------------------------------------ gated FFN rows
 __device__ __forceinline__ float gelu_inner(float g)
 {
@@ -1125,13 +1205,16 @@ void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
 
 int lora_grad_blocks(int D, int qd, int kd, int R)
 {
+    if (R == 16) return (qd + 255) / 256 + (kd + 255) / 256 + (D + 255) / 256;      // k_lora_grads_rank
     const size_t n = (size_t)2 * R * D + (size_t)qd * R + (size_t)kd * R;
     return (int)((n + TB - 1) / TB);
 }
 
 void launch_lora_grads(const LoraGradArgs &a)
 {
-    LAUNCH(k_lora_grads, dim3(lora_grad_blocks(a.D, a.qd, a.kd, a.R), a.layers > 0 ? a.layers : 1), dim3(TB), 0, a);
+    const dim3 grid(lora_grad_blocks(a.D, a.qd, a.kd, a.R), a.layers > 0 ? a.layers : 1);
+    if (a.R == 16) LAUNCH(k_lora_grads_rank<16>, grid, dim3(256), 0, a);
+    else LAUNCH(k_lora_grads, grid, dim3(TB), 0, a);
 }
 
 void launch_glu_fwd(const GluArgs &a, int rows)
