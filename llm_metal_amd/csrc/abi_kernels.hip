@@ -292,12 +292,6 @@ __global__ __launch_bounds__(64) void k_attn_bwd_dkv(const float *__restrict__ d
 
 // ---------------------------------------------------------------- elementwise
 
-__device__ __forceinline__ float gelu_inner(float g)
-{
-    float in = 0.7978845608f * (g + 0.044715f * g * g * g);
-    return fminf(fmaxf(in, -15.0f), 15.0f);
-}
-
 __global__ void k_silu_mul(float *gate, const float *__restrict__ up, size_t n)
 {
     const size_t i = (size_t)blockIdx.x * TB + threadIdx.x;

@@ -39,6 +39,9 @@ template <typename T> inline T *dptr_as(const MetalBuf *b) { return (T *)dptr(b)
 
 inline void mark_written(MetalBuf *b) { if (b) { b->version++; if (b->parent) b->parent->version++; } }
 
+// infer_kernels.hip: y[i] = act(gate_i . x) * (up_i . x) for W = [gate; up] of 2 * rows rows (F16, or Q8_0 blocks when q8)
+void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q8, int gelu);
+
 }  // namespace lmhip
 
 #define LMHIP_API extern "C" __attribute__((visibility("default")))

@@ -80,5 +80,13 @@ __device__ __forceinline__ float row_scale_for(float amax)
     return ldexpf(1.0f, p);
 }
 
+// Argument of the tanh in the GELU approximation, clamped as the reference clamps it (gelu_mul,
+// shaders/q8_kernels.metal:349-362).
+__device__ __forceinline__ float gelu_inner(float g)
+{
+    const float in = 0.7978845608f * (g + 0.044715f * g * g * g);
+    return fminf(fmaxf(in, -15.0f), 15.0f);
+}
+
 __device__ __forceinline__ half_t f2h(float x) { return (half_t)x; }      // v_cvt_f16_f32: round to nearest even
 __device__ __forceinline__ float  h2f(half_t x) { return (float)x; }

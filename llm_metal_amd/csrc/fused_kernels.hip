@@ -696,11 +696,6 @@ __global__ __launch_bounds__(256) void k_lora_grads_rank(LoraGradArgs a)
 }
 
 // ------------------------------------------------------------------ gated FFN rows
-__device__ __forceinline__ float gelu_inner(float g)
-{
-    const float in = 0.7978845608f * (g + 0.044715f * g * g * g);
-    return fminf(fmaxf(in, -15.0f), 15.0f);
-}
 __device__ __forceinline__ float act_fwd(float g, int gelu)
 {
     return gelu ? 0.5f * g * (1.0f + tanhf(gelu_inner(g))) : g / (1.0f + expf(-g));

@@ -91,10 +91,13 @@ const int8_t *q8_split_of(MetalBuf *W, int rows, int nb, const half_t **scales)
 // current one is used, and the first before x is staged into LDS (XLDS; without it, for rows longer than the LDS
 // budget, every lane reads its x values from global memory with the weights).  Q8_0: codes are biased to unsigned
 // (q + 128, one v_cvt_f32_ubyte each) and the bias is taken out with the lane's sum of x, once per step for all rows.
-template <int FMT, int R, int U, int XLDS>
+// GLU (1 SiLU, 2 GELU; R = 2): the matrix is [gate; up] with `rows` rows each; a wave takes gate row i and up row i and
+// writes act(gate . x) * (up . x), the gated product the FFN forms next, in place of the two sums.
+template <int FMT, int R, int U, int XLDS, int GLU = 0>
 __global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, const half_t *__restrict__ scales,
                                                const float *__restrict__ x, float *__restrict__ y, int rows, int cols)
 {
+    static_assert(GLU == 0 || R == 2, "the gated variant pairs two rows");
     extern __shared__ float xs[];                               // [cols] when XLDS
     struct Stage {
         half8   w16[FMT == 0 ? R : 1][U];
@@ -103,10 +106,10 @@ __global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, cons
         float4v x0[XLDS ? 1 : U], x1[XLDS ? 1 : U];
     };
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row0 = (blockIdx.x * 4 + wave) * R;
+    const int row0 = (blockIdx.x * 4 + wave) * (GLU ? 1 : R);
     size_t roff[R];                                             // element offset of each row (clamped: extra rows are not stored)
 #pragma unroll
-    for (int r = 0; r < R; r++) roff[r] = (size_t)min(row0 + r, rows - 1) * cols;
+    for (int r = 0; r < R; r++) roff[r] = GLU ? ((size_t)r * rows + min(row0, rows - 1)) * cols : (size_t)min(row0 + r, rows - 1) * cols;
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
@@ -179,6 +182,12 @@ __global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, cons
         use(cur, c);
         cur = nxt;
     }
+    if (GLU) {
+        const float g = wave_sum(acc[0]), u = wave_sum(acc[R - 1]);
+        if (lane == 0 && row0 < rows)                           // the expressions of silu_mul / gelu_mul
+            y[row0] = (GLU == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + tanhf(gelu_inner(g)))) * u;
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const float s = wave_sum(acc[r]);
@@ -221,6 +230,21 @@ void launch_matvec(const void *W, const half_t *scales, const float *x, float *y
     else if (rows >= 8192) MATVEC_LAUNCH(2, 2, 0, 8, 0);
     else MATVEC_LAUNCH(1, 4, 0, 4, 0);
 #undef MATVEC_LAUNCH
+}
+
+// [gate; up] x with the gate applied (see k_matvec): y[i] = act(gate_i . x) * (up_i . x), i < rows.
+template <int FMT>
+void launch_matvec_glu(const void *W, const half_t *scales, const float *x, float *y, int rows, int cols, int gelu)
+{
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+    const bool prof = gemm_prof_begin(2.0 * rows * cols * (FMT == 0 ? 2.0 : 34.0 / 32.0), 4.0 * rows * cols, &ev_a, &ev_b);
+    const dim3 grid((rows + 3) / 4);
+#define GLU_LAUNCH(G_) do { \
+    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, 2, 2, 0, G_>), grid, dim3(TB), 0, stream(), ev_a, ev_b, 0, W, scales, x, y, rows, cols); \
+    else hipLaunchKernelGGL((k_matvec<FMT, 2, 2, 0, G_>), grid, dim3(TB), 0, stream(), W, scales, x, y, rows, cols); \
+    HIP_CHECK(hipGetLastError()); } while (0)
+    if (gelu) GLU_LAUNCH(2); else GLU_LAUNCH(1);
+#undef GLU_LAUNCH
 }
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -653,3 +677,29 @@ double hip_matvec_time_shape(int rows, int cols, int fmt, int B, int iters)
 }
 
 }  // extern "C"
+
+namespace lmhip {
+
+// The gate|up product of the FFN with the gate applied in its epilogue: W = [gate; up] ([2 * rows, cols], F16 rows or
+// Q8_0 blocks), y[i] = act(gate_i . x) * (up_i . x).  What metal_enqueue_*_matvec followed by metal_enqueue_silu_mul /
+// gelu_mul computes (src/nn/fast_inference.c:441-452), in one launch and without the [2 * rows] intermediate.
+void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q8, int gelu)
+{
+    if (rows <= 0 || cols <= 0 || (cols & 31) || !aligned16(dptr(W)) || !aligned16(dptr(x))) {
+        fprintf(stderr, "[fast_hip] matvec_glu: unsupported shape %d x %d\n", rows, cols); abort();
+    }
+    REQUIRE_BYTES(x, (size_t)cols * 4, "matvec_glu");
+    REQUIRE_BYTES(y, (size_t)rows * 4, "matvec_glu");
+    if (q8) {
+        REQUIRE_BYTES(W, (size_t)2 * rows * (cols / 32) * 34, "matvec_glu");
+        const half_t *scales = nullptr;
+        const int8_t *q = q8_split_of(W, 2 * rows, cols / 32, &scales);
+        launch_matvec_glu<1>(q, scales, dptr_as<float>(x), dptr_as<float>(y), rows, cols, gelu);
+    } else {
+        REQUIRE_BYTES(W, (size_t)2 * rows * cols * 2, "matvec_glu");
+        launch_matvec_glu<0>(dptr(W), nullptr, dptr_as<float>(x), dptr_as<float>(y), rows, cols, gelu);
+    }
+    mark_written(y);
+}
+
+}  // namespace lmhip

@@ -245,9 +245,8 @@ void forward_token(InferenceState *s, int token, int pos)
         matvec(s, lw.o, s->att, s->branch);
         // x += o (Gemma3: RMSNorm(o; g_post_attn)); ln = RMSNorm(x; g_pre_ff | g_post_attn)
         add_norm(s, s->branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
-        matvec(s, &lw.gu, s->ln, s->gu);
-        if (gemma) metal_enqueue_gelu_mul(s->gate_v, s->up_v, s->IS);
-        else metal_enqueue_silu_mul(s->gate_v, s->up_v, s->IS);
+        // act = silu | gelu (gate) * up, formed in the epilogue of the [gate; up] product
+        matvec_glu(lw.gu.mbuf, s->ln, s->gate_v, s->IS, D, s->use_fp16 ? 0 : 1, gemma ? 1 : 0);
         matvec(s, lw.down, s->gate_v, s->branch);
         pending = s->branch;
         pending_g = gemma ? lw.g_post_ff : nullptr;
