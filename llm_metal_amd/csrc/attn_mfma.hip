@@ -202,6 +202,7 @@ struct AttnTileArgs {
     float *A_out;                 // dQ: plane-summed dO rows [rows][Hq*hd]
     float *out32;                 // dQ: dq [rows][Hq*hd]
     half_t *out16;                // forward: tiled [rows, Hq*hd]
+    WeightPrefetch pf;            // weights of the product that follows: fetched by the grid slices z >= batch
 };
 
 // Row step: eight threads per row, thread `part` owns the keys 32 m + 4 part + (0..3) for m < M32 and keeps them in
@@ -282,6 +283,11 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     extern __shared__ float lds[];
     constexpr int lda = HD + 8;                            // halves; rows 16-byte aligned and 4 banks apart: conflict-free 16-byte reads
     const int N = a.seq;
+    if ((int)blockIdx.z >= a.batch) {
+        const int per_z = gridDim.x * gridDim.y;
+        prefetch_weight_tiles<256>(a.pf, (blockIdx.z - a.batch) * per_z + blockIdx.y * gridDim.x + blockIdx.x, a.batch * per_z);
+        return;
+    }
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l31 = lane & 31, hh = lane >> 5;
     const int qd = a.Hq * HD, kd = a.Hkv * HD, hk = h / (a.Hq / a.Hkv);
@@ -466,7 +472,9 @@ void launch_tile_m(const AttnTileArgs &a)
     static bool attr_set = false;
     if (!attr_set) { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_attn_tile<BWD, HD, M32>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); attr_set = true; }
     const size_t lds = tile_lds_bytes(HD, a.seq);
-    LAUNCH((k_attn_tile<BWD, HD, M32>), dim3((a.seq + 31) / 32, a.Hq, a.batch), dim3(256), lds, a);
+    const int per_z = ((a.seq + 31) / 32) * a.Hq;
+    const int extra = a.pf.base ? a.pf.wgs / per_z : 0;   // the planner made pf.wgs a multiple of per_z
+    LAUNCH((k_attn_tile<BWD, HD, M32>), dim3((a.seq + 31) / 32, a.Hq, a.batch + extra), dim3(256), lds, a);
 }
 
 template <int BWD, int HD>
@@ -505,6 +513,7 @@ void launch_attn_fwd_mfma(const AttnFwdArgs &f)
     a.A = f.q; a.BT = f.kT; a.C = f.v;
     a.Hq = f.Hq; a.Hkv = f.Hkv; a.hd = f.hd; a.seq = f.seq; a.batch = f.batch; a.scale = f.scale;
     a.probs = f.probs; a.out16 = f.out16;
+    a.pf = f.pf;
     launch_tile<0>(a);
 }
 

@@ -26,6 +26,19 @@ struct Planes {
 // them; cols == 0: one workgroup and one scale per row.
 struct ScaleGroups { int cols, groups, shift; };
 
+// Weight tiles of the product that follows a row kernel, for the workgroups the row kernel starts beyond its rows: they
+// read, into the L2 of their XCD, the tiles that the product's workgroups on the same XCD ask for first (workgroups of a
+// launch go to the XCDs round-robin by linear index).  F16 tiles only; wgs == 0: nothing to fetch.
+struct WeightPrefetch {
+    const char *base;             // tiled F16 weight image
+    int Kb, Nb;                   // K steps and 32-row blocks of the image
+    int nb, steps, S, n_tiles;    // the product's plan: blocks per workgroup, K steps per chunk, chunks, row tiles
+    int rotate;
+    int wgs;                      // prefetching workgroups (a multiple of 8)
+    int per_wg;                   // product workgroups each of them covers
+    int depth;                    // K steps fetched per product workgroup (its waves' first steps)
+};
+
 struct NormRowsArgs {
     // source of the residual stream row: token gather (emb != null) or x_prev
     const float *emb; const uint32_t *tokens; float emb_scale;
@@ -37,6 +50,7 @@ struct NormRowsArgs {
     const float *g_norm;          // null: no normalised output wanted
     half_t *ln16; float *inv_scale;   // tiled [rows, D]
     int D; float eps;
+    WeightPrefetch pf; int rows_launched;             // rows_launched: set by the launcher
 };
 void launch_norm_rows(const NormRowsArgs &a, int rows);
 
@@ -67,6 +81,7 @@ struct AttnFwdArgs {
     float *probs;                 // [batch][Hq][seq][seq]
     half_t *out16;                // tiled [rows, Hq*hd], unit scale
     const float *kT;              // k transposed per head [batch][Hkv][hd/4][attn_ldt(seq)][4] (matrix-core path only)
+    WeightPrefetch pf;            // matrix-core path: weights of the product that follows
 };
 void launch_attn_fwd(const AttnFwdArgs &a);
 
@@ -93,6 +108,7 @@ struct QkvBwdArgs {
     float *dq_f, *dv_f;           // pre-norm-domain dq [rows][Hq*hd], dv copy [rows][Hkv*hd] (for dB)
     float *dh;                    // [rows][2R] = sc * dq B_q | sc * dv B_v
     half_t *out16; float *inv_scale;                // tiled [rows, dq | dk | dv | dh_q | dh_v]
+    WeightPrefetch pf; int rows_launched;           // weights of the product that follows; rows_launched: set by the launcher
 };
 void launch_qkv_bwd(const QkvBwdArgs &a, int rows);
 
@@ -124,6 +140,7 @@ struct NormBwdArgs {
     const float *dx_prev; float *dx_out; float clamp;   // clamp <= 0: none
     const float *branch_raw, *g_branch;                 // Gemma3: next GEMM input is RNB(branch_raw, dx_out)
     half_t *d16; float *inv_scale;                      // tiled [rows, D]; may be null on the last kernel of the backward
+    WeightPrefetch pf; int rows_launched;
 };
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows);
 

@@ -55,6 +55,10 @@ template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
+    if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
+        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched, a.rows_launched);
+        return;
+    }
     const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
@@ -420,6 +424,10 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [16 waves][32] partials
     __shared__ float sm[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
+        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched, a.rows_launched);
+        return;
+    }
     const size_t row = blockIdx.x;
     const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd, R = a.R;
     const int n = qd + 2 * kd + 2 * R;
@@ -784,7 +792,7 @@ __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
 #pragma unroll
     for (int t = 0; t < MAXC; t++) { const int v = threadIdx.x + t * GC; if (v < nv) st_tiled4(a.out16, r, c0 + 4 * v, Kb, act[t], s); }
     if (c0 + width == IS) zero_tiled_pad(a.out16, r, IS, Kb);
-    if (threadIdx.x == 0) a.inv_scale[r * gridDim.y + blockIdx.y] = 1.0f / s;
+    if (threadIdx.x == 0) a.inv_scale[r * a.sg.groups + blockIdx.y] = 1.0f / s;
 }
 
 __device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, float &dg, float &du)
@@ -888,7 +896,7 @@ __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
 #pragma unroll
     for (int t = 0; t < MAXC; t++) { const int v = threadIdx.x + t * GC; if (v < nv) st_tiled4(a.out16, r, c0 + 4 * v, Kb, o[t], s); }
     if (c0 + width == 2 * IS) zero_tiled_pad(a.out16, r, 2 * IS, Kb);
-    if (threadIdx.x == 0) a.inv_scale[r * gridDim.y + blockIdx.y] = 1.0f / s;
+    if (threadIdx.x == 0) a.inv_scale[r * a.sg.groups + blockIdx.y] = 1.0f / s;
 }
 
 // ------------------------------------------------------------------ backward rows
@@ -901,6 +909,10 @@ template <int MAXV, bool GROUPED>
 __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
     __shared__ float sm[32];
+    if (blockIdx.x >= a.rows_launched) {
+        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched, a.rows_launched);
+        return;
+    }
     const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 dy[MAXV], x[MAXV], g[MAXV];
@@ -1139,8 +1151,11 @@ void launch_norm_rows(const NormRowsArgs &a, int rows)
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV, "norm_rows: hidden size must be a multiple of 4, <= 12288");
     require(a.branch.S == 0 || a.branch.ld % 4 == 0, "norm_rows: plane row length must be a multiple of 4");
     const bool grouped = a.branch.S > 0 && a.branch.scale_groups != 0;
-    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_rows<1, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_rows<1, false>), dim3(rows), dim3(RB), 0, a); }
-    else { if (grouped) LAUNCH((k_norm_rows<MAXV_ROW, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_rows<MAXV_ROW, false>), dim3(rows), dim3(RB), 0, a); }
+    NormRowsArgs b = a;
+    b.rows_launched = rows;
+    const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
+    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_rows<1, false>), grid, dim3(RB), 0, b); }
+    else { if (grouped) LAUNCH((k_norm_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
 }
 
 void launch_rope_table(float2 *tab, int seq, int hd, float theta)
@@ -1187,14 +1202,17 @@ void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
 {
     const size_t n = (size_t)(a.Hq + 2 * a.Hkv) * a.hd + 2 * a.R + 16 * 32;
     require(a.hd <= 2 * 64 * MAXP && n * 4 <= 64 * 1024 && a.R <= 16, "qkv_bwd: row of dq|dk|dv must fit 64 KB of LDS, rank <= 16");
+    QkvBwdArgs b = a;
+    b.rows_launched = rows;
+    const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
     if (a.hd <= 128) {
-        if (a.R == 16) LAUNCH((k_qkv_bwd_rows<1, 16>), dim3(rows), dim3(RB), n * 4, a);
-        else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<1, 0>), dim3(rows), dim3(RB), n * 4, a);
-        else LAUNCH((k_qkv_bwd_rows<1, -1>), dim3(rows), dim3(RB), n * 4, a);
+        if (a.R == 16) LAUNCH((k_qkv_bwd_rows<1, 16>), grid, dim3(RB), n * 4, b);
+        else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<1, 0>), grid, dim3(RB), n * 4, b);
+        else LAUNCH((k_qkv_bwd_rows<1, -1>), grid, dim3(RB), n * 4, b);
     } else {
-        if (a.R == 16) LAUNCH((k_qkv_bwd_rows<MAXP, 16>), dim3(rows), dim3(RB), n * 4, a);
-        else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<MAXP, 0>), dim3(rows), dim3(RB), n * 4, a);
-        else LAUNCH((k_qkv_bwd_rows<MAXP, -1>), dim3(rows), dim3(RB), n * 4, a);
+        if (a.R == 16) LAUNCH((k_qkv_bwd_rows<MAXP, 16>), grid, dim3(RB), n * 4, b);
+        else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<MAXP, 0>), grid, dim3(RB), n * 4, b);
+        else LAUNCH((k_qkv_bwd_rows<MAXP, -1>), grid, dim3(RB), n * 4, b);
     }
 }
 
@@ -1243,8 +1261,11 @@ void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
 {
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV && a.dy.ld % 4 == 0, "norm_bwd_rows: hidden size must be a multiple of 4, <= 12288");
     const bool grouped = a.dy.scale_groups != 0;
-    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_bwd_rows<1, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_bwd_rows<1, false>), dim3(rows), dim3(RB), 0, a); }
-    else { if (grouped) LAUNCH((k_norm_bwd_rows<MAXV_ROW, true>), dim3(rows), dim3(RB), 0, a); else LAUNCH((k_norm_bwd_rows<MAXV_ROW, false>), dim3(rows), dim3(RB), 0, a); }
+    NormBwdArgs b = a;
+    b.rows_launched = rows;
+    const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
+    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_bwd_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_bwd_rows<1, false>), grid, dim3(RB), 0, b); }
+    else { if (grouped) LAUNCH((k_norm_bwd_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_bwd_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
 }
 
 void launch_ce_rows(const CeArgs &a, int rows)

@@ -120,6 +120,43 @@ __device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, con
     }
 }
 
+// Workgroup `pw` of pf.wgs prefetching workgroups of THREADS threads (`first_id` = linear index of prefetching
+// workgroup 0 in the launch).  A 4 KB tile is one 16-byte load for each of 256 threads, so the workgroup takes
+// THREADS / 256 tiles at a time; the loads of a thread are issued eight at a time before the first is waited for.
+template <int THREADS>
+__device__ __forceinline__ void prefetch_weight_tiles(const WeightPrefetch &pf, int pw, int first_id)
+{
+    constexpr int TPR = THREADS / 256;                   // tiles per round
+    const int xcd = (first_id + pw) & 7, slot = pw >> 3, slots = pf.wgs >> 3;
+    const int total = pf.n_tiles * pf.S, q = threadIdx.x >> 8, t16 = (threadIdx.x & 255) * 16;
+    const int per_g = (pf.depth * pf.nb + TPR - 1) / TPR;  // loads of a thread per workgroup of the product
+    unsigned sink = 0u;
+    for (int j0 = 0; j0 < pf.per_wg * per_g; j0 += 8) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            v[u] = make_uint4(0u, 0u, 0u, 0u);
+            const int j = (j0 + u) / per_g, e = (j0 + u) % per_g;
+            const int g = xcd + 8 * (slot + slots * j);  // a workgroup of the product that will run on this XCD
+            const int ts = e * TPR + q, w = ts / pf.nb, b = ts % pf.nb;
+            if (j0 + u < pf.per_wg * per_g && g < total && w < pf.depth) {
+                const int x = g % pf.n_tiles, y = g / pf.n_tiles;
+                const int kb_beg = y * pf.steps, nsteps = min(pf.Kb, kb_beg + pf.steps) - kb_beg;
+                const int rot = pf.rotate ? (int)((x * 7u + y * 3u) % (unsigned)nsteps) : 0;
+                int kk = w + rot;
+                if (kk >= nsteps) kk -= nsteps;
+                if (w < nsteps) {
+                    const size_t tile = (size_t)min(x * pf.nb + b, pf.Nb - 1) * pf.Kb + kb_beg + kk;
+                    v[u] = *reinterpret_cast<const uint4 *>(pf.base + tile * 4096 + t16);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) sink ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    asm volatile("" :: "v"(sink));                        // the loads have a use, and nothing is stored
+}
+
 __device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 __device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
 __device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }

@@ -194,6 +194,31 @@ ScaleGroups scale_groups_for(SFTState *s, const WeightOp &W, int N, int K)
     return g.groups <= MAX_SCALE_GROUPS ? g : none;
 }
 
+// What the workgroups a row kernel starts beyond its own fetch into L2 for the product with W [N, K] that follows it.
+// `threads`: block size of that kernel; `unit`: its prefetching workgroups come in multiples of this many (1 for a
+// one-dimensional grid, else the size of a grid slice).  About 16 MB, the first K steps of as many of the product's
+// workgroups as that covers: what fits beside the row kernel's own work in time and in the L2s.
+WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int threads, int unit = 1)
+{
+    // measured on config 3 (MI355X): 16 MB by 160 workgroups of 1024 threads shortens the product by 3 us and lengthens
+    // the row kernel by 1.5; less fetches too little, more (or fewer, longer-running workgroups) holds the row kernel up
+    constexpr int mb = 16, depth = 4, wgs1024 = 160;
+    WeightPrefetch pf{};
+    if (s->full_param || W.fmt != 0 || !W.w16 || use_big_gemm(s->BN, N, K, W.fmt)) return pf;
+    const GemmPlan p = plan_gemm(s->BN, N, K, 0);
+    if (p.m_tiles != 1 || unit <= 0) return pf;
+    int wgs = wgs1024 * (1024 / threads);
+    wgs = (wgs + unit - 1) / unit * unit;
+    if (wgs & 7) return pf;
+    pf.base = reinterpret_cast<const char *>(W.w16);
+    pf.Kb = tiled_kb(K); pf.Nb = tiled_rb(N);
+    pf.nb = p.nb; pf.steps = p.steps; pf.S = p.S; pf.n_tiles = p.n_tiles; pf.rotate = p.rotate;
+    pf.wgs = wgs; pf.depth = depth;
+    const long covered = std::min<long>((long)mb * 1024 * 1024 / ((long)p.nb * depth * 4096), (long)p.n_tiles * p.S);
+    pf.per_wg = (int)((covered + wgs - 1) / wgs);
+    return pf;
+}
+
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr,
             const ScaleGroups *sg = nullptr)
@@ -247,6 +272,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         n1.x_out = x_in;
         n1.g_norm = at<float>(s->g_in, (size_t)L * D);
         n1.ln16 = ln1; n1.inv_scale = ln1inv; n1.D = D; n1.eps = s->eps;
+        n1.pf = prefetch_for(s, wop(s, W_QKV, L, false), s->nq_ext, D, 1024);
         launch_norm_rows(n1, BN);
 
         // [q | k | v | tq | tv] = ln1 [Wq; Wk; Wv; A_q; A_v]^T                 [:638-656]
@@ -274,7 +300,10 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
         aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16; aa.kT = qa.kT;
-        if (attn_mfma_supported(s->hd, s->N)) launch_attn_fwd_mfma(aa); else launch_attn_fwd(aa);
+        if (attn_mfma_supported(s->hd, s->N)) {
+            aa.pf = prefetch_for(s, wop(s, W_O, L, false), D, qd, 256, ((s->N + 31) / 32) * s->Hq);
+            launch_attn_fwd_mfma(aa);
+        } else launch_attn_fwd(aa);
         // full-parameter mode keeps the FFN GEMM operands of every layer as well
         half_t *ln2 = s->full_param ? at<half_t>(s->ln2_16, L * s->st_ln1) : a16;
         float *ln2inv = s->full_param ? at<float>(s->ln2_inv, (size_t)L * BN) : ainv;
@@ -289,6 +318,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         n2.x_out = x_mid;
         n2.g_norm = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
         n2.ln16 = ln2; n2.inv_scale = ln2inv; n2.D = D; n2.eps = s->eps;
+        n2.pf = prefetch_for(s, wop(s, W_GU, L, false), 2 * IS, D, 1024);
         launch_norm_rows(n2, BN);
 
         // [gate | up] = ln2 [Wg; Wu]^T; act = silu|gelu(gate) * up              [:715-725]
@@ -315,6 +345,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
     half_t *lnf = s->full_param ? at<half_t>(s->lnf16) : a16;
     float *lnfinv = s->full_param ? at<float>(s->lnf_inv) : ainv;
     nf.ln16 = lnf; nf.inv_scale = lnfinv; nf.D = D; nf.eps = s->eps;
+    nf.pf = prefetch_for(s, wop(s, W_LM, 0, false), s->V, D, 1024);
     launch_norm_rows(nf, BN);
     GemmPlan pl = plan_gemm(BN, s->V, D);
     if (pl.S == 1 || use_big_gemm(BN, s->V, D, s->q8_native ? 1 : 0)) {
@@ -365,6 +396,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
     nb.eps = s->eps; nb.D = D; nb.dx_prev = nullptr; nb.dx_out = at<float>(s->dx[cur]); nb.clamp = 0.f;
     if (gemma) { nb.branch_raw = at<float>(s->ff_raw, (size_t)(NL - 1) * xsz); nb.g_branch = at<float>(s->g_post_ff, (size_t)(NL - 1) * D); }
     nb.d16 = a16; nb.inv_scale = ainv;
+    if (mode == BWD_LORA) nb.pf = prefetch_for(s, wop(s, W_D, NL - 1, true), IS, D, 1024);
     launch_norm_bwd_rows(nb, BN);
 
     for (int L = NL - 1; L >= 0; L--) {
@@ -389,6 +421,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         n2.eps = s->eps; n2.D = D; n2.dx_prev = at<float>(s->dx[cur]); n2.dx_out = at<float>(s->dx[cur ^ 1]); n2.clamp = 0.f;
         if (gemma) { n2.branch_raw = at<float>(s->o_raw, (size_t)L * xsz); n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); }
         n2.d16 = a16; n2.inv_scale = ainv;
+        if (mode == BWD_LORA) n2.pf = prefetch_for(s, wop(s, W_O, L, true), qd, D, 1024);
         launch_norm_bwd_rows(n2, BN);
         cur ^= 1;
 
@@ -422,6 +455,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
         qb.dq_f = at<float>(s->dq_f, keepL * BN * qd); qb.dv_f = nullptr; qb.dh = at<float>(s->dh, keepL * BN * (R ? 2 * R : 1));
         qb.out16 = a16; qb.inv_scale = ainv;
+        if (mode == BWD_LORA) qb.pf = prefetch_for(s, wop(s, W_QKV, L, true), D, s->nq_ext, 1024);
         launch_qkv_bwd(qb, BN);
         // full-parameter: W_q, W_k, W_v are updated BEFORE the dX product, which then multiplies with the
         // new weights in SGD mode, as the reference does                       [:922-946]
@@ -438,6 +472,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
             if (gemma) { n1.branch_raw = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); n1.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); }
             n1.d16 = a16; n1.inv_scale = ainv;
         }
+        if (mode == BWD_LORA && L > 0) n1.pf = prefetch_for(s, wop(s, W_D, L - 1, true), IS, D, 1024);
         launch_norm_bwd_rows(n1, BN);
         cur ^= 1;
     }
