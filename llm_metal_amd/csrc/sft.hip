@@ -194,10 +194,10 @@ ScaleGroups scale_groups_for(SFTState *s, const WeightOp &W, int N, int K)
     return g.groups <= MAX_SCALE_GROUPS ? g : none;
 }
 
-// What the workgroups a row kernel starts beyond its own fetch into L2 for the product with W [N, K] that follows it.
+// What the workgroups a row kernel starts beyond its own request ahead for the product with W [N, K] that follows it.
 // `threads`: block size of that kernel; `unit`: its prefetching workgroups come in multiples of this many (1 for a
 // one-dimensional grid, else the size of a grid slice).  About 16 MB, the first K steps of as many of the product's
-// workgroups as that covers: what fits beside the row kernel's own work in time and in the L2s.
+// workgroups as that covers: what fits beside the row kernel's own work in time.
 WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int threads, int unit = 1)
 {
     // measured on config 3 (MI355X): 16 MB by 160 workgroups of 1024 threads shortens the product by 3 us and lengthens
