@@ -285,7 +285,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     const int N = a.seq;
     if ((int)blockIdx.z >= a.batch) {
         const int per_z = gridDim.x * gridDim.y;
-        prefetch_weight_tiles<256>(a.pf, (blockIdx.z - a.batch) * per_z + blockIdx.y * gridDim.x + blockIdx.x, a.batch * per_z);
+        prefetch_weight_tiles<256>(a.pf, (blockIdx.z - a.batch) * per_z + blockIdx.y * gridDim.x + blockIdx.x);
         return;
     }
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;

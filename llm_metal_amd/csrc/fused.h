@@ -27,17 +27,17 @@ struct Planes {
 struct ScaleGroups { int cols, groups, shift; };
 
 // Weight tiles of the product that follows a row kernel, for the workgroups the row kernel starts beyond its rows: they
-// request, while most CUs have nothing to do, the tiles that the product's workgroups ask for first.  Hardware counters
-// show that the product fetches them again from beyond L2 (no line survives a kernel boundary there), but it then finds
-// them in the memory-side cache, and its first K steps stop waiting for HBM.  The tiles are visited in the order of the
-// product's workgroups on the prefetching workgroup's own XCD (workgroups of a launch go to the XCDs round-robin by
-// linear index).  F16 tiles only; base == null: nothing to fetch.
+// request, while most CUs have nothing to do, the tiles that the product's workgroups ask for first (its workgroup g
+// starts with the K steps rot(g) .. rot(g) + 3 of its chunk).  Hardware counters show that the product fetches them
+// again from beyond L2 (no line survives a kernel boundary there), but it then finds them in the memory-side cache, and
+// its first K steps stop waiting for HBM.  Which XCD asks makes no difference.  F16 tiles only; base == null: nothing
+// to fetch.
 struct WeightPrefetch {
     const char *base;             // tiled F16 weight image
     int Kb, Nb;                   // K steps and 32-row blocks of the image
     int nb, steps, S, n_tiles;    // the product's plan: blocks per workgroup, K steps per chunk, chunks, row tiles
     int rotate;
-    int wgs;                      // prefetching workgroups (a multiple of 8)
+    int wgs;                      // prefetching workgroups
     int per_wg;                   // product workgroups each of them covers
     int depth;                    // K steps fetched per product workgroup (its waves' first steps)
 };

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
     if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
-        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched, a.rows_launched);
+        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t r = blockIdx.x;
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     __shared__ float sm[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
-        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched, a.rows_launched);
+        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t row = blockIdx.x;
@@ -910,7 +910,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
 {
     __shared__ float sm[32];
     if (blockIdx.x >= a.rows_launched) {
-        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched, a.rows_launched);
+        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t r = blockIdx.x;

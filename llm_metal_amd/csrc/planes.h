@@ -120,14 +120,13 @@ __device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, con
     }
 }
 
-// Workgroup `pw` of pf.wgs prefetching workgroups of THREADS threads (`first_id` = linear index of prefetching
-// workgroup 0 in the launch).  A 4 KB tile is one 16-byte load for each of 256 threads, so the workgroup takes
-// THREADS / 256 tiles at a time; the loads of a thread are issued eight at a time before the first is waited for.
+// Workgroup `pw` of pf.wgs prefetching workgroups of THREADS threads.  A 4 KB tile is one 16-byte load for each of 256
+// threads, so the workgroup takes THREADS / 256 tiles at a time; the loads of a thread are issued eight at a time before
+// the first is waited for.
 template <int THREADS>
-__device__ __forceinline__ void prefetch_weight_tiles(const WeightPrefetch &pf, int pw, int first_id)
+__device__ __forceinline__ void prefetch_weight_tiles(const WeightPrefetch &pf, int pw)
 {
     constexpr int TPR = THREADS / 256;                   // tiles per round
-    const int xcd = (first_id + pw) & 7, slot = pw >> 3, slots = pf.wgs >> 3;
     const int total = pf.n_tiles * pf.S, q = threadIdx.x >> 8, t16 = (threadIdx.x & 255) * 16;
     const int per_g = (pf.depth * pf.nb + TPR - 1) / TPR;  // loads of a thread per workgroup of the product
     unsigned sink = 0u;
@@ -137,7 +136,7 @@ __device__ __forceinline__ void prefetch_weight_tiles(const WeightPrefetch &pf, 
         for (int u = 0; u < 8; u++) {
             v[u] = make_uint4(0u, 0u, 0u, 0u);
             const int j = (j0 + u) / per_g, e = (j0 + u) % per_g;
-            const int g = xcd + 8 * (slot + slots * j);  // a workgroup of the product that will run on this XCD
+            const int g = pw + pf.wgs * j;               // a workgroup of the product
             const int ts = e * TPR + q, w = ts / pf.nb, b = ts % pf.nb;
             if (j0 + u < pf.per_wg * per_g && g < total && w < pf.depth) {
                 const int x = g % pf.n_tiles, y = g / pf.n_tiles;

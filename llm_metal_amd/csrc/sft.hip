@@ -209,7 +209,6 @@ WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int th
     if (p.m_tiles != 1 || unit <= 0) return pf;
     int wgs = wgs1024 * (1024 / threads);
     wgs = (wgs + unit - 1) / unit * unit;
-    if (wgs & 7) return pf;
     pf.base = reinterpret_cast<const char *>(W.w16);
     pf.Kb = tiled_kb(K); pf.Nb = tiled_rb(N);
     pf.nb = p.nb; pf.steps = p.steps; pf.S = p.S; pf.n_tiles = p.n_tiles; pf.rotate = p.rotate;
