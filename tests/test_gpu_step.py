@@ -44,6 +44,10 @@ CASES = [
     C1.with_(name="big_m_f16", batch=4, seq=64),
     C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
+    # a wide FFN: the GLU kernels split each row into column groups of two (forward) and four (backward) K chunks with
+    # a factor each, and 2 * IS is not a whole number of backward groups, so one group straddles the dgate | dup boundary
+    C1.with_(name="wide_ffn_groups", NL=1, IS=4224, V=1024, seq=64),
+    TINY_GEMMA3.with_(name="gemma_wide_ffn", NL=2, IS=2112, seq=64),
 ]
 
 
