@@ -39,6 +39,20 @@ template <typename T> inline T *dptr_as(const MetalBuf *b) { return (T *)dptr(b)
 
 inline void mark_written(MetalBuf *b) { if (b) { b->version++; if (b->parent) b->parent->version++; } }
 
+// What the generation pipeline does to the Q|K|V product before the attention (src/nn/fast_inference.c:402-427): LoRA
+// terms on q and v, per-head RMSNorm and RoPE on q and k, k and v into row `pos` of the caches.
+struct HeadPost {
+    const float *qkv;                    // [Hq*hd | Hkv*hd | Hkv*hd], left as it is
+    const float *g_q, *g_k;              // per-head norm gammas or NULL
+    float *kc, *vc;                      // caches [Hkv, max_seq, hd]
+    const float *t, *Bq, *Bv;            // adapters: t [2R], B_q [Hq*hd, R], B_v [Hkv*hd, R]; R == 0: none
+    int Hq, Hkv, R, pos;
+    const float2 *rope;                  // (cos, sin) of the hd/2 rotary pairs at position pos
+    float eps, sc;
+};
+// infer_kernels.hip: that and the attention over the cache rows 0 .. pos in one launch (out [Hq*hd])
+void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq);
+
 // infer_kernels.hip: y[i] = act(gate_i . x) * (up_i . x) for W = [gate; up] of 2 * rows rows (F16, or Q8_0 blocks when q8)
 void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q8, int gelu);
 

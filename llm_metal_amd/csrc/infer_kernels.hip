@@ -303,11 +303,67 @@ constexpr int SL = 256;      // keys per workgroup
 // workgroups leave (max, sum, unnormalised output) per query head and k_attn_combine merges them.
 // VEC: floats of V per thread in the weighted sum (4 when hd % 4 == 0).
 // LDS: q [gpw][hd], scores [gpw][SL], ml [2][gpw], red [4 * 1024].  hd <= 256.
-template <int VEC>
-__global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q, const float *__restrict__ Kc,
-                                                    const float *__restrict__ Vc, float *__restrict__ out,
-                                                    float *__restrict__ part_o, float *__restrict__ part_ml,
-                                                    int n_attend, int hd, int max_seq, int G, int gpw, float scale, int nsplit)
+// FUSED: Q is the raw q part of the Q|K|V product; the workgroup finishes its query heads itself (into LDS only) and, when
+// its slice holds the newest key, writes that key's and value's cache rows before it reads the cache (every workgroup
+// that needs them writes the same values, so no workgroup waits for another).
+
+// One head of the Q|K|V product finished by one wave (lane i owns the rotary pairs i and i + 64 of up to 256 values):
+// kind 0 q (LoRA, norm, RoPE), 1 k (norm, RoPE), 2 v (LoRA).  per_head_rms_norm, rope, add_scaled of
+// shaders/q8_kernels.metal:165-231, 378-384.
+__device__ __forceinline__ void finish_head(const HeadPost &a, int kind, int h, int hd, int lane, float *dst)
+{
+    const int half = hd / 2;
+    const float *vec = a.qkv + (size_t)(kind == 0 ? h : (kind == 1 ? a.Hq + h : a.Hq + a.Hkv + h)) * hd;
+    float x0[2] = {0.f, 0.f}, x1[2] = {0.f, 0.f};
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int i = lane + 64 * u;
+        if (i < half) {
+            x0[u] = vec[i]; x1[u] = vec[i + half];
+            if (a.R && kind != 1) {
+                const float *B = (kind == 0 ? a.Bq : a.Bv) + (size_t)h * hd * a.R;
+                const float *t = kind == 0 ? a.t : a.t + a.R;
+                float d0 = 0.f, d1 = 0.f;
+                for (int r = 0; r < a.R; r++) { d0 = fmaf(B[(size_t)i * a.R + r], t[r], d0); d1 = fmaf(B[(size_t)(i + half) * a.R + r], t[r], d1); }
+                x0[u] = fmaf(a.sc, d0, x0[u]); x1[u] = fmaf(a.sc, d1, x1[u]);
+            }
+            ss += x0[u] * x0[u] + x1[u] * x1[u];
+        }
+    }
+    if (kind != 2) {
+        const float *g = kind == 0 ? a.g_q : a.g_k;
+        if (g) {
+            const float inv = rsqrtf(wave_sum(ss) / (float)hd + a.eps);
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int i = lane + 64 * u;
+                if (i < half) { x0[u] *= inv * g[i]; x1[u] *= inv * g[i + half]; }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int i = lane + 64 * u;
+            if (i < half) {
+                const float2 c = a.rope[i];
+                const float cs = c.x, sn = c.y;
+                const float r0 = x0[u] * cs - x1[u] * sn, r1 = x0[u] * sn + x1[u] * cs;
+                x0[u] = r0; x1[u] = r1;
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int i = lane + 64 * u;
+        if (i < half) { dst[i] = x0[u]; dst[i + half] = x1[u]; }
+    }
+}
+
+template <int VEC, bool FUSED>
+__global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q, const float *Kc, const float *Vc,
+                                                    float *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                                                    int n_attend, int hd, int max_seq, int G, int gpw, float scale, int nsplit,
+                                                    HeadPost hp)
 {
     extern __shared__ float sm[];
     float *qs = sm, *sc = qs + gpw * hd, *ml = sc + gpw * SL, *red = ml + 2 * gpw;
@@ -317,8 +373,17 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
     const float *kbase = Kc + ((size_t)hkv * max_seq + j0) * hd;
     const float *vbase = Vc + ((size_t)hkv * max_seq + j0) * hd;
 
-    for (int i = tid; i < gpw * hd; i += TB) qs[i] = Q[(size_t)hq0 * hd + i];
-    __syncthreads();
+    if (FUSED) {
+        for (int g = wave; g < gpw; g += 4) finish_head(hp, 0, hq0 + g, hd, lane, qs + g * hd);
+        if (j0 <= hp.pos && hp.pos < j0 + SL) {           // the waves after those that had a query head (or all in turn)
+            const size_t row = ((size_t)hkv * max_seq + hp.pos) * hd;
+            if (wave == (gpw & 3)) finish_head(hp, 1, hkv, hd, lane, hp.kc + row);
+            if (wave == ((gpw + 1) & 3)) finish_head(hp, 2, hkv, hd, lane, hp.vc + row);
+        }
+    } else {
+        for (int i = tid; i < gpw * hd; i += TB) qs[i] = Q[(size_t)hq0 * hd + i];
+    }
+    __syncthreads();                                      // also orders the cache rows written above before the reads below
 
     // scores: a wave takes four keys at a time (their loads are in flight together), lanes over the head dimension,
     // four query heads per pass over the keys
@@ -490,7 +555,8 @@ void kv_store(const float *k, const float *v, MetalBuf *kc, MetalBuf *vc, int Hk
     mark_written(kc); mark_written(vc);
 }
 
-void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_attend, int hd, int max_seq, int Hq, int G, const char *fn)
+void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_attend, int hd, int max_seq, int Hq, int G, const char *fn,
+               const HeadPost *hp = nullptr)
 {
     if (Hq <= 0 || n_attend <= 0) return;
     if (G <= 0 || Hq % G) { fprintf(stderr, "[fast_hip] %s: %d query heads are not a multiple of the group ratio %d; launch skipped\n", fn, Hq, G); return; }
@@ -511,12 +577,13 @@ void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_att
     }
     const float scale = 1.0f / sqrtf((float)hd);
     const bool vec4 = hd % 4 == 0 && (((uintptr_t)dptr(Vc)) & 15) == 0;
-    if (vec4)
-        LAUNCH(k_attn_decode<4>, dim3(Hq / gpw, nsplit), dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml,
-               n_attend, hd, max_seq, G, gpw, scale, nsplit);
-    else
-        LAUNCH(k_attn_decode<1>, dim3(Hq / gpw, nsplit), dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml,
-               n_attend, hd, max_seq, G, gpw, scale, nsplit);
+    const dim3 grid(Hq / gpw, nsplit);
+    const HeadPost none{};
+#define ATTN_LAUNCH(V_, F_) LAUNCH((k_attn_decode<V_, F_>), grid, dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml, \
+                                   n_attend, hd, max_seq, G, gpw, scale, nsplit, F_ ? *hp : none)
+    if (hp) { if (vec4) ATTN_LAUNCH(4, true); else ATTN_LAUNCH(1, true); }
+    else { if (vec4) ATTN_LAUNCH(4, false); else ATTN_LAUNCH(1, false); }
+#undef ATTN_LAUNCH
     if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq), dim3(TB), 0, po, pml, out, hd, nsplit);
 }
 
@@ -700,6 +767,16 @@ void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q
         launch_matvec_glu<0>(dptr(W), nullptr, dptr_as<float>(x), dptr_as<float>(y), rows, cols, gelu);
     }
     mark_written(y);
+}
+
+
+void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq)
+{
+    if (hp.Hkv <= 0 || hp.Hq % hp.Hkv || (hd & 1) || hp.pos < 0 || hp.pos >= max_seq) {
+        fprintf(stderr, "[fast_hip] attention_decode_fused: unsupported shape\n"); abort();
+    }
+    attention(hp.qkv, Kc, Vc, out, hp.pos + 1, hd, max_seq, hp.Hq, hp.Hq / hp.Hkv, "attention_decode_fused", &hp);
+    mark_written(Kc); mark_written(Vc);
 }
 
 }  // namespace lmhip

@@ -9,6 +9,7 @@
 // per-head RMSNorm, RoPE and the KV-cache store for all heads.
 #include "backend.h"
 #include "devutil.h"
+#include "fused.h"
 #include "../../include/inference_hip.h"
 #include "../../include/loader_hip.h"
 
@@ -30,6 +31,8 @@ struct InferenceState {
     float emb_scale, eps;
     int eos[4], n_eos;
     std::vector<float> thetas;
+    MetalBuf *rope_tabs;                 // (cos, sin) [distinct thetas][max_seq][hd/2], as rope forms them
+    std::vector<int> theta_slot;         // table of each layer
     MetalBuf *x, *branch, *ln, *qkv, *att, *gu, *gate_v, *up_v, *logits, *best;   // gate_v / up_v: the halves of gu
     float *logits_host;
     int *best_host;
@@ -135,71 +138,6 @@ __global__ __launch_bounds__(64) void k_lora_down(const float *__restrict__ ln, 
     if (threadIdx.x == 0) t[r] = s;
 }
 
-struct QkPostArgs {
-    float *qkv;                          // [Hq*hd | Hkv*hd | Hkv*hd]; q is finished in place
-    const float *g_q, *g_k;              // per-head norm gammas or NULL
-    float *kc, *vc;                      // caches [Hkv, max_seq, hd]
-    const float *t, *Bq, *Bv;            // adapters: t [2R], B_q [Hq*hd, R], B_v [Hkv*hd, R]; R == 0: none
-    int Hq, Hkv, hd, max_seq, pos, R;
-    float theta, eps, sc;
-};
-
-// One wave per head (q heads, then k heads, then v heads); lane i owns the rotary pair (i, i + hd/2), hd <= 256.
-// q: += sc B_q t_q, per-head RMSNorm, RoPE, in place.  k: RMSNorm, RoPE, into the cache row `pos`.  v: += sc B_v t_v,
-// into the cache.  (src/nn/fast_inference.c:402-427; kernels shaders/q8_kernels.metal:165-256)
-__global__ __launch_bounds__(64) void k_qk_post(QkPostArgs a)
-{
-    const int h = blockIdx.x, lane = threadIdx.x, half = a.hd / 2;
-    const bool is_q = h < a.Hq, is_k = !is_q && h < a.Hq + a.Hkv;
-    const int hk = is_q ? 0 : (is_k ? h - a.Hq : h - a.Hq - a.Hkv);
-    float *vec = a.qkv + (size_t)h * a.hd;
-    float x0[2] = {0.f, 0.f}, x1[2] = {0.f, 0.f};                    // pairs lane and lane + 64
-    float ss = 0.f;
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        const int i = lane + 64 * u;
-        if (i < half) {
-            x0[u] = vec[i]; x1[u] = vec[i + half];
-            if (a.R && !is_k) {
-                const float *B = is_q ? a.Bq + (size_t)h * a.hd * a.R : a.Bv + (size_t)hk * a.hd * a.R;
-                const float *t = is_q ? a.t : a.t + a.R;
-                float d0 = 0.f, d1 = 0.f;
-                for (int r = 0; r < a.R; r++) { d0 = fmaf(B[(size_t)i * a.R + r], t[r], d0); d1 = fmaf(B[(size_t)(i + half) * a.R + r], t[r], d1); }
-                x0[u] = fmaf(a.sc, d0, x0[u]); x1[u] = fmaf(a.sc, d1, x1[u]);
-            }
-            ss += x0[u] * x0[u] + x1[u] * x1[u];
-        }
-    }
-    if (is_q || is_k) {
-        const float *g = is_q ? a.g_q : a.g_k;
-        if (g) {
-            const float inv = rsqrtf(wave_sum(ss) / (float)a.hd + a.eps);
-#pragma unroll
-            for (int u = 0; u < 2; u++) {
-                const int i = lane + 64 * u;
-                if (i < half) { x0[u] *= inv * g[i]; x1[u] *= inv * g[i + half]; }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const int i = lane + 64 * u;
-            if (i < half) {
-                const float freq = 1.0f / powf(a.theta, (float)(2 * i) / (float)a.hd);
-                float sn, cs;
-                sincosf((float)a.pos * freq, &sn, &cs);
-                const float r0 = x0[u] * cs - x1[u] * sn, r1 = x0[u] * sn + x1[u] * cs;
-                x0[u] = r0; x1[u] = r1;
-            }
-        }
-    }
-    float *dst = is_q ? vec : (is_k ? a.kc : a.vc) + ((size_t)hk * a.max_seq + a.pos) * a.hd;
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        const int i = lane + 64 * u;
-        if (i < half) { dst[i] = x0[u]; dst[i + half] = x1[u]; }
-    }
-}
-
 MetalBuf *fbuf(size_t n) { return metal_buf_create(n * sizeof(float)); }
 
 void matvec(InferenceState *s, const WMat *w, MetalBuf *x, MetalBuf *y)
@@ -226,12 +164,14 @@ void forward_token(InferenceState *s, int token, int pos)
         const InferenceState::Layer &lw = s->layers[L];
         add_norm(s, pending, pending_g, lw.g_in);
         matvec(s, &lw.qkv, s->ln, s->qkv);
-        QkPostArgs a{};
+        // LoRA on q and v, per-head RMSNorm and RoPE on q and k, k and v into the caches, and the attention over the
+        // cache: one launch (infer_kernels.hip: k_attn_decode<.., FUSED>)
+        HeadPost a{};
         a.qkv = dptr_as<float>(s->qkv);
         a.g_q = lw.g_q ? dptr_as<float>(lw.g_q) : nullptr; a.g_k = lw.g_k ? dptr_as<float>(lw.g_k) : nullptr;
         a.kc = dptr_as<float>(s->kc[L]); a.vc = dptr_as<float>(s->vc[L]);
-        a.Hq = Hq; a.Hkv = Hkv; a.hd = hd; a.max_seq = s->max_seq; a.pos = pos;
-        a.theta = s->thetas[L]; a.eps = s->eps;
+        a.Hq = Hq; a.Hkv = Hkv; a.pos = pos;
+        a.rope = dptr_as<float2>(s->rope_tabs) + ((size_t)s->theta_slot[L] * s->max_seq + pos) * (hd / 2); a.eps = s->eps;
         if (!s->lora.empty()) {
             const InferenceState::Lora &lr = s->lora[L];
             hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R), dim3(64), 0, stream(), dptr_as<float>(s->ln), dptr_as<float>(lr.Aq),
@@ -239,9 +179,8 @@ void forward_token(InferenceState *s, int token, int pos)
             a.t = dptr_as<float>(s->lora_t); a.Bq = dptr_as<float>(lr.Bq); a.Bv = dptr_as<float>(lr.Bv);
             a.R = s->R; a.sc = s->scaling;
         }
-        hipLaunchKernelGGL(k_qk_post, dim3(Hq + 2 * Hkv), dim3(64), 0, stream(), a);
-        mark_written(s->kc[L]); mark_written(s->vc[L]);
-        metal_enqueue_attention_off(s->qkv, 0, s->kc[L], s->vc[L], s->att, 0, pos + 1, hd, s->max_seq, Hq, Hq / Hkv);
+        attention_decode_fused(a, s->kc[L], s->vc[L], dptr_as<float>(s->att), hd, s->max_seq);
+        mark_written(s->att);
         matvec(s, lw.o, s->att, s->branch);
         // x += o (Gemma3: RMSNorm(o; g_post_attn)); ln = RMSNorm(x; g_pre_ff | g_post_attn)
         add_norm(s, s->branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
@@ -296,6 +235,18 @@ InferenceState *new_state(ModelType mt, int D, int Hq, int Hkv, int hd, int IS, 
     s->emb_scale = mt == MODEL_GEMMA3 ? sqrtf((float)D) : 1.0f;
     s->eps = 1e-6f;                                                       // src/nn/fast_inference.c:383
     s->thetas.assign(thetas, thetas + NL);
+    {                                                                     // one table per distinct RoPE base
+        std::vector<float> distinct;
+        for (int L = 0; L < NL; L++) {
+            size_t k = 0;
+            while (k < distinct.size() && distinct[k] != thetas[L]) k++;
+            if (k == distinct.size()) distinct.push_back(thetas[L]);
+            s->theta_slot.push_back((int)k);
+        }
+        const size_t per = (size_t)max_seq * (hd / 2);
+        s->rope_tabs = metal_buf_create(distinct.size() * per * sizeof(float2));
+        for (size_t k = 0; k < distinct.size(); k++) launch_rope_table(dptr_as<float2>(s->rope_tabs) + k * per, max_seq, hd, distinct[k]);
+    }
     default_eos(s);
     const int qd = Hq * hd, kd = Hkv * hd;
     s->x = fbuf(D); s->branch = fbuf(D); s->ln = fbuf(D);
@@ -529,7 +480,7 @@ void inference_state_free(InferenceState *s)
 {
     if (!s) return;
     metal_flush();
-    for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t})
+    for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t, s->rope_tabs})
         metal_buf_free(b);
     for (MetalBuf *b : s->kc) metal_buf_free(b);
     for (MetalBuf *b : s->vc) metal_buf_free(b);
