@@ -361,6 +361,12 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
         };
         if constexpr (((M32 + 3) / 4) * NCB == 1) {       // at most one item per wave: no second tile on its way
             if (nitems) run(0, bt0);
+        } else if constexpr (((M32 + 3) / 4) * NCB == 2) { // at most two items (two column passes, or two key blocks)
+            if (nitems) {
+                if (nitems > 1) b_tile_load<CB>(bt1, b_item(1), ldt);
+                run(0, bt0);
+                if (nitems > 1) run(1, bt1);
+            }
         } else {
             for (int q = 0; q < nitems; q += 2) {
                 b_tile_load<CB>(bt1, b_item(q + 1), ldt);
