@@ -211,14 +211,41 @@ struct AttnTileArgs {
 // column N) and back to LDS for phase 3 as bf16 pairs, in place: the upper parts of keys 0.. at the start of the
 // row, the lower parts xlo halves further on.  A row belongs to eight lanes of one wave, which have read all of it
 // before they write.
+// The saved probabilities this thread needs in the dQ row step (zero right of the diagonal; whole 16-byte groups exist
+// when N % 4 == 0, else they go by element).  They depend on nothing computed in the kernel, so short rows (M32 <= 8)
+// are requested at the start of the kernel and arrive while the scores are formed.
+template <int M32>
+__device__ __forceinline__ void load_probs(float4 (&p)[M32], const AttnTileArgs &a, int N, int i0, int b, int h, int tid)
+{
+    const int rr = tid >> 3, part = tid & 7, i = i0 + rr;
+    const size_t goff = (((size_t)b * a.Hq + h) * N + min(i, N - 1)) * N + 4 * part;
+#pragma unroll
+    for (int m = 0; m < M32; m++) {
+        const int j = 32 * m + 4 * part;
+        float4 pv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < N && j <= i) {
+            if ((N & 3) == 0) pv = *reinterpret_cast<const float4 *>(a.probs + goff + 32 * m);
+            else { float *q = &pv.x; for (int c = 0; c < 4; c++) if (j + c < N) q[c] = a.probs[goff + 32 * m + c]; }
+        }
+        p[m] = pv;
+    }
+}
+
 template <int BWD, int M32>
-__device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int xlo, int nk, int N, int i0, int b, int h, int tid)
+__device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int xlo, int nk, int N, int i0, int b, int h, int tid,
+                                         const float4 (&p_early)[BWD ? M32 : 1])
 {
     const int rr = tid >> 3, part = tid & 7, i = i0 + rr;
     const bool row_ok = i < N;
     float *xr = Xs + rr * ldx + 4 * part;
     const size_t goff = (((size_t)b * a.Hq + h) * N + min(i, N - 1)) * N + 4 * part;
     float4 v[M32], p[BWD ? M32 : 1];
+    if constexpr (BWD) {
+        if constexpr (M32 <= 8) {
+#pragma unroll
+            for (int m = 0; m < M32; m++) p[m] = p_early[m];
+        } else load_probs<M32>(p, a, N, i0, b, h, tid);
+    }
     float red = BWD ? 0.f : -1e30f;
 #pragma unroll
     for (int m = 0; m < M32; m++) {
@@ -226,13 +253,7 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
         v[m] = (j < nk) ? *reinterpret_cast<const float4 *>(xr + 32 * m) : make_float4(0.f, 0.f, 0.f, 0.f);
         float *e = &v[m].x;
         if (BWD) {
-            // probabilities are zero right of the diagonal; whole 16-byte groups exist when N % 4 == 0, else go by element
-            float4 pv = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (row_ok && j <= i) {
-                if ((N & 3) == 0) pv = *reinterpret_cast<const float4 *>(a.probs + goff + 32 * m);
-                else { float *q = &pv.x; for (int c = 0; c < 4; c++) if (j + c < N) q[c] = a.probs[goff + 32 * m + c]; }
-            }
-            p[m] = pv;
+            const float4 pv = p[m];
             red += pv.x * e[0] + pv.y * e[1] + pv.z * e[2] + pv.w * e[3];
         } else {
 #pragma unroll
@@ -313,6 +334,8 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     };
     BTile<CB> bt0, bt1;
     b_tile_load<CB>(bt0, b_item(0), ldt);
+    float4 p_early[BWD ? M32 : 1];
+    if constexpr (BWD && M32 <= 8) load_probs<M32>(p_early, a, N, i0, b, h, tid);
     CRing cring;
     const float *c_lane0 = a.C + r0 * kd + hk * HD + l31;
     c_ring_start<M32>(cring, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, nk, hh, N);
@@ -379,7 +402,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     __syncthreads();
 
     // ---- row step
-    row_step<BWD, M32>(a, Xs, ldx, N32, nk, N, i0, b, h, tid);             // whole rows of N entries are written
+    row_step<BWD, M32>(a, Xs, ldx, N32, nk, N, i0, b, h, tid, p_early);    // whole rows of N entries are written
     __syncthreads();
 
     // ---- phase 3: Y = X C, one 32-column block of the head per wave and round
