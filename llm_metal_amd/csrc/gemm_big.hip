@@ -131,51 +131,55 @@ __global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
             for (int j = 0; j < 4; j++) buf[((4 + wave * WPW + u) * 4 + j) * 64 + lane] = w[j];
         }
     };
+    // Every fetch is issued unconditionally (past the end it asks for the last step again): with a fetch under a
+    // condition the compiler cannot count how many younger loads are in flight when a stage is parked, and waits for
+    // all of them -- the prefetch then hides nothing.
+    const int last = g.Kb - 1;
 #pragma unroll
-    for (int p = 0; p < PF; p++) if (p < g.Kb) fetch<WF>(st[p], g, mb_ld, nb_ld, p, lane);
+    for (int p = 0; p < PF; p++) fetch<WF>(st[p], g, mb_ld, nb_ld, min(p, last), lane);
     park(st[0], 0, tiles);
     __syncthreads();
-    for (int kt0 = 0; kt0 < g.Kb; kt0 += PF) {
+    // one K step: multiply step kt out of LDS buffer kt & 1 while step kt + 1 is unpacked and parked in the other one
+    // and step kt + PF is requested into the slot that step kt left (u = kt % PF, a compile-time constant at every call)
+    auto step = [&](int kt, int u) __attribute__((always_inline)) {
+        const half8 *cur = tiles + (size_t)(kt & 1) * BUF;
+        fetch<WF>(st[u], g, mb_ld, nb_ld, min(kt + PF, last), lane);
+        // fp16 image of the next step's weight blocks: plain VALU work with no dependence on this step's MFMAs, placed in
+        // the same block of code so that the two interleave (on the last step it unpacks a repeated step and the result
+        // lands in the buffer nobody reads any more)
+        const Stage &sn = st[(u + 1) % PF];
+        half8 wnext[WPW][4];
 #pragma unroll
-        for (int u = 0; u < PF; u++) {
-            const int kt = kt0 + u;
-            if (kt < g.Kb) {
-                const half8 *cur = tiles + (size_t)(kt & 1) * BUF;
-                // the slot of step kt is free (it was written to LDS in the previous round): refill it with step kt + PF
-                if (kt + PF < g.Kb) fetch<WF>(st[u], g, mb_ld, nb_ld, kt + PF, lane);
-                // fp16 image of the next step's weight blocks: plain VALU work with no dependence on this step's
-                // MFMAs, placed in the same block of code so that the two interleave (on the last step it
-                // unpacks stale registers and the result is dropped)
-                const Stage &sn = st[(u + 1) % PF];
-                half8 wnext[WPW][4];
+        for (int x = 0; x < WPW; x++) unpack<WF>(wnext[x], sn, x, tile_kind<WF>(g, nb_ld[x], min(kt + 1, last)));
 #pragma unroll
-                for (int x = 0; x < WPW; x++) unpack<WF>(wnext[x], sn, x, tile_kind<WF>(g, nb_ld[x], min(kt + 1, g.Kb - 1)));
+        for (int j = 0; j < 4; j++) {
+            half8 a[2], w[NW];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    half8 a[2], w[NW];
+            for (int i = 0; i < 2; i++) a[i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
 #pragma unroll
-                    for (int i = 0; i < 2; i++) a[i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
+            for (int k = 0; k < NW; k++) w[k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
 #pragma unroll
-                    for (int k = 0; k < NW; k++) w[k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-                    for (int i = 0; i < 2; i++)
-#pragma unroll
-                        for (int k = 0; k < NW; k++)
-                            acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
-                }
-                if (kt + 1 < g.Kb) {
-                    half8 *nxt = tiles + (size_t)((kt + 1) & 1) * BUF;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        nxt[(wave * 4 + j) * 64 + lane] = sn.a[j];
-#pragma unroll
-                        for (int x = 0; x < WPW; x++) nxt[((4 + wave * WPW + x) * 4 + j) * 64 + lane] = wnext[x][j];
-                    }
-                }
-                __syncthreads();
-            }
+                for (int k = 0; k < NW; k++)
+                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
         }
+        half8 *nxt = tiles + (size_t)((kt + 1) & 1) * BUF;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            nxt[(wave * 4 + j) * 64 + lane] = sn.a[j];
+#pragma unroll
+            for (int x = 0; x < WPW; x++) nxt[((4 + wave * WPW + x) * 4 + j) * 64 + lane] = wnext[x][j];
+        }
+        __syncthreads();
+    };
+    const int full = g.Kb / PF * PF;
+    for (int kt0 = 0; kt0 < full; kt0 += PF) {
+#pragma unroll
+        for (int u = 0; u < PF; u++) step(kt0 + u, u);
     }
+#pragma unroll
+    for (int u = 0; u < PF - 1; u++) if (full + u < g.Kb) step(full + u, u);
 
 #pragma unroll
     for (int i = 0; i < 2; i++)
