@@ -28,7 +28,8 @@ struct Stage {
     half8 a[4];
     half8 w16[WPW][4];               // F16 tile, or the column scales of a transposed Q8_0 tile
     uint4v q[WPW][2];                // Q8_0 int8
-    half_t d[WPW];                   // Q8_0 row scale of this lane's weights
+    uint32_t d[WPW];                 // Q8_0 row scale of this lane's weights: the fp16 bits in a register of their own (two halves
+                                     // packed into one register would make the pack wait for the load that was just issued)
 };
 
 // kind of weight tile (uniform per wave): 0 F16, 1 Q8_0 row scales, 2 Q8_0 column scales
@@ -58,7 +59,7 @@ __device__ __forceinline__ void fetch(Stage &s, const GemmKArgs &g, int mb, cons
             const uint4v *q = reinterpret_cast<const uint4v *>(g.W.q) + tile * 128 + lane;
             s.q[u][0] = __builtin_nontemporal_load(&q[0]);
             s.q[u][1] = __builtin_nontemporal_load(&q[64]);
-            if (kind == 1) s.d[u] = g.W.d[tile * 64 + lane];
+            if (kind == 1) s.d[u] = reinterpret_cast<const uint16_t *>(g.W.d)[tile * 64 + lane];
             else {
                 const half8 *sc = reinterpret_cast<const half8 *>(g.W.d + tile * 64 + (lane >> 5) * 32);
 #pragma unroll
@@ -79,7 +80,7 @@ __device__ __forceinline__ void unpack(half8 (&w)[4], const Stage &s, int u, int
     }
     const half8 q0 = q8_unpack8(s.q[u][0][0], s.q[u][0][1]), q1 = q8_unpack8(s.q[u][0][2], s.q[u][0][3]);
     const half8 q2 = q8_unpack8(s.q[u][1][0], s.q[u][1][1]), q3 = q8_unpack8(s.q[u][1][2], s.q[u][1][3]);
-    if (kind == 1) { const half8 d = bcast8(s.d[u]); w[0] = q0 * d; w[1] = q1 * d; w[2] = q2 * d; w[3] = q3 * d; }
+    if (kind == 1) { const half8 d = bcast8(__builtin_bit_cast(half_t, (uint16_t)s.d[u])); w[0] = q0 * d; w[1] = q1 * d; w[2] = q2 * d; w[3] = q3 * d; }
     else { w[0] = q0 * s.w16[u][0]; w[1] = q1 * s.w16[u][1]; w[2] = q2 * s.w16[u][2]; w[3] = q3 * s.w16[u][3]; }
 }
 
@@ -151,18 +152,23 @@ __global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
         half8 wnext[WPW][4];
 #pragma unroll
         for (int x = 0; x < WPW; x++) unpack<WF>(wnext[x], sn, x, tile_kind<WF>(g, nb_ld[x], min(kt + 1, last)));
+        // operands of K slice j + 1 are read from LDS before the MFMAs of slice j are issued, so the reads run under them
+        half8 a[2][2], w[2][NW];
+        auto read = [&](int j) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) a[j & 1][i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
+#pragma unroll
+            for (int k = 0; k < NW; k++) w[j & 1][k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
+        };
+        read(0);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            half8 a[2], w[NW];
-#pragma unroll
-            for (int i = 0; i < 2; i++) a[i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
-#pragma unroll
-            for (int k = 0; k < NW; k++) w[k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
+            if (j + 1 < 4) read(j + 1);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
                 for (int k = 0; k < NW; k++)
-                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
+                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 1][i], w[j & 1][k], acc[i][k], 0, 0, 0);
         }
         half8 *nxt = tiles + (size_t)((kt + 1) & 1) * BUF;
 #pragma unroll
@@ -170,6 +176,18 @@ __global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
             nxt[(wave * 4 + j) * 64 + lane] = sn.a[j];
 #pragma unroll
             for (int x = 0; x < WPW; x++) nxt[((4 + wave * WPW + x) * 4 + j) * 64 + lane] = wnext[x][j];
+        }
+        // Issue order of the step, one memory instruction in the shadow of each MFMA (a wave is the only one on its SIMD,
+        // so whatever is not issued between two MFMAs is paid for on top of them): the 6 LDS reads of slice 0, then per
+        // MFMA of slices 0-2 one LDS read of the next slice, the 12 global loads under slices 0-1, the 12 LDS writes
+        // under slices 2-3.  Left to itself the scheduler sinks every read to just before its use.
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 24 && (i & 7) < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (i >= 20) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         __syncthreads();
     };
