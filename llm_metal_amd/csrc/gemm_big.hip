@@ -199,11 +199,37 @@ __global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
 #pragma unroll
     for (int u = 0; u < PF - 1; u++) if (full + u < g.Kb) step(full + u, u);
 
+    // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4
+    if (mb0 * 32 + 128 <= g.M && (nb0 + 4 * WPW) * 32 <= g.N) {
+        // Block inside the matrix: no bounds tests, so the row factors are all requested at once and the stores follow
+        // each other without a wait (a store under a condition makes the compiler drain the queue before every one).
+        float sc[2][16];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) sc[i][v] = 1.0f;
+        if (g.a_inv_scale) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    sc[i][v] = g.a_inv_scale[(mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3)];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = (mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                float *row = g.P + (size_t)m * g.ldp + (nb0 + NW * wn) * 32 + r;
+#pragma unroll
+                for (int k = 0; k < NW; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4
             const int m = (mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
             if (m >= g.M) continue;
             const float sc = g.a_inv_scale ? g.a_inv_scale[m] : 1.0f;
