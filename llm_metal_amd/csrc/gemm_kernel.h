@@ -187,12 +187,22 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
     // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4.  SCALE: the row factors
     // are fetched here, where the K loop's registers are free (holding them through the loop costs a wave of occupancy).
 #define QUARTER_STORE(W) if (wave == (W)) { \
+        constexpr int i0 = (W) * Q; \
+        float sc[Q]; \
+        if (SCALE) { \
+            /* all factors requested before the first store (row clamped): a load under the store's condition would make \
+               every store wait for the one before it */ \
+            _Pragma("unroll") for (int k = 0; k < Q; k++) { \
+                const int i = i0 + k, mb = i / (NB * 16), v = i % 16; \
+                sc[k] = g.a_inv_scale[min((mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), M - 1)]; \
+            } \
+        } \
         _Pragma("unroll") for (int k = 0; k < Q; k++) { \
-            constexpr int i0 = (W) * Q; \
             const int i = i0 + k, mb = i / (NB * 16), b = (i / 16) % NB, v = i % 16; \
             const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), n = (nb0 + b) * 32 + r; \
             float sres = ACC_AT(i0 + k) + theirs[k * 64 + lane]; \
-            if (m < M && n < N) { if (SCALE) sres *= g.a_inv_scale[m]; Pp[(size_t)m * g.ldp + n] = sres; } \
+            if (SCALE) sres *= sc[k]; \
+            if (m < M && n < N) Pp[(size_t)m * g.ldp + n] = sres; \
         } }
     QUARTER_STORE(0) QUARTER_STORE(1) QUARTER_STORE(2) QUARTER_STORE(3)
 #undef QUARTER_STORE
