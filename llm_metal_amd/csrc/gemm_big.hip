@@ -4,12 +4,13 @@
 // (gemm.h: tiled fp16 activations with per-row power-of-two factors; F16 or Q8_0 weight tiles), same
 // arithmetic (v_mfma_f32_32x32x16_f16, fp32 accumulation), one launch, no K split.
 //
-// A workgroup of four waves owns a 128 x 128 block of C and walks K in steps of 64.  Per step every wave
-// fetches one 32-row block of the activation tile and one of the weight tile from L2/HBM in the MFMA
+// A workgroup of four waves owns a 128 x 256 block of C and walks K in steps of 64.  Per step every wave
+// fetches one 32-row block of the activation tile and two of the weight tile from L2/HBM in the MFMA
 // register layout, Q8_0 blocks are unpacked to fp16 there (int8 * fp16 scale, once per tile instead of once
 // per consumer), and both go to LDS in the same [j][lane][8 halves] order, so a wave reads any row block back
-// with conflict-free 16-byte loads.  LDS is double buffered: the global loads of step k+1 are issued before the
-// MFMAs of step k and written to the other buffer after them; one barrier per step.
+// with conflict-free 16-byte loads.  LDS is double buffered and the operands travel three steps ahead in registers:
+// during the MFMAs of step k the loads of step k+3 are issued and step k+1 is written to the other buffer; one
+// barrier per step.
 #include "backend.h"
 #include "devutil.h"
 #include "gemm.h"
