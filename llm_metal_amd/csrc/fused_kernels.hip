@@ -18,6 +18,7 @@ namespace {
 constexpr int TB = 256;
 constexpr int RB = 1024;                                  // threads of a row workgroup
 constexpr int MAXV = 3;                                   // float4 per thread: rows up to 12288 wide
+constexpr int MANY_ROWS = 512;                            // rows from which a row kernel takes 256 threads per row instead of 1024
 constexpr int MAXV_ROW = MAXV;                            // (the name the row kernels with their own MAXV parameter use)
 
 // four consecutive elements (k % 4 == 0) of row `row` of a tiled fp16 operand
@@ -51,12 +52,14 @@ __device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t
 // ordering (norm the branch, then add) is src/nn/fast_sft.c:698-705, 732-736.
 // MAXV: float4 per thread (1 for rows up to 4096 wide, which leaves registers for 20 planes of the branch in flight).
 // GROUPED: the branch planes carry a factor per group of planes.
-template <int MAXV, bool GROUPED>
-__global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
+// NT: threads per row.  1024 when a step has few rows (one row's loads all in flight at once); 256 from a few hundred
+// rows on, where eight resident workgroups per CU hide each other's reductions and barriers.
+template <int MAXV, bool GROUPED, int NT = RB>
+__global__ __launch_bounds__(NT) void k_norm_rows(NormRowsArgs a)
 {
     __shared__ float sm[16];
     if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
-        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
+        prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t r = blockIdx.x;
@@ -67,7 +70,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
     size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
-        const int v = threadIdx.x + t * RB;
+        const int v = threadIdx.x + t * NT;
         x[t] = b[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv && !padded) x[t] = ld4(base + 4 * v);
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
         }
 #pragma unroll
         for (int t = 0; t < MAXV; t++) {
-            const int v = threadIdx.x + t * RB;
+            const int v = threadIdx.x + t * NT;
             if (v >= nv) continue;
             if (a.g_branch) {
                 if (a.branch_raw_out) st4(a.branch_raw_out + r * D + 4 * v, b[t]);
@@ -102,7 +105,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
     }
     if (a.x_out) {
 #pragma unroll
-        for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st4(a.x_out + r * D + 4 * v, x[t]); }
+        for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) st4(a.x_out + r * D + 4 * v, x[t]); }
     }
     if (!a.g_norm) return;
     float ss = 0.f;
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
     float amax = 0.f;
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
-        const int v = threadIdx.x + t * RB;
+        const int v = threadIdx.x + t * NT;
         if (v >= nv) continue;
         const float4 g = ld4(a.g_norm + 4 * v);
         x[t].x = x[t].x * inv * g.x; x[t].y = x[t].y * inv * g.y; x[t].z = x[t].z * inv * g.z; x[t].w = x[t].w * inv * g.w;
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(RB) void k_norm_rows(NormRowsArgs a)
     const float s = row_scale_for(amax);
     const int Kb = tiled_kb(D);
 #pragma unroll
-    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st_tiled4(a.ln16, r, 4 * v, Kb, x[t], s); }
+    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) st_tiled4(a.ln16, r, 4 * v, Kb, x[t], s); }
     zero_tiled_pad(a.ln16, r, D, Kb);
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
@@ -905,12 +908,12 @@ __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
 // src/nn/fast_sft.c:870-874, 975-980).  The operand of the next dX GEMM is dx_out
 // itself (Qwen3) or RNB(branch_raw, dx_out; g_branch) (Gemma3's post-norms,
 // src/nn/fast_sft.c:798-802, 877-881).
-template <int MAXV, bool GROUPED>
-__global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
+template <int MAXV, bool GROUPED, int NT = RB>
+__global__ __launch_bounds__(NT) void k_norm_bwd_rows(NormBwdArgs a)
 {
     __shared__ float sm[32];
     if (blockIdx.x >= a.rows_launched) {
-        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
+        prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t r = blockIdx.x;
@@ -920,7 +923,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
     size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
-        const int v = threadIdx.x + t * RB;
+        const int v = threadIdx.x + t * NT;
         x[t] = g[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv) { x[t] = ld4(a.x_saved + r * D + 4 * v); g[t] = ld4(a.g + 4 * v); }
@@ -937,7 +940,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
     float4 dx[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
-        const int v = threadIdx.x + t * RB;
+        const int v = threadIdx.x + t * NT;
         dx[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (v >= nv) continue;
         dx[t] = make_float4((g[t].x * dy[t].x - coeff * x[t].x) * inv, (g[t].y * dy[t].y - coeff * x[t].y) * inv,
@@ -955,7 +958,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
         float ssb = 0.f, dotb = 0.f;
 #pragma unroll
         for (int t = 0; t < MAXV; t++) {
-            const int v = threadIdx.x + t * RB;
+            const int v = threadIdx.x + t * NT;
             if (v >= nv) continue;
             x[t] = ld4(a.branch_raw + r * D + 4 * v);
             g[t] = ld4(a.g_branch + 4 * v);
@@ -967,7 +970,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
         const float cb = dotb * invb * invb / (float)D;
 #pragma unroll
         for (int t = 0; t < MAXV; t++) {
-            const int v = threadIdx.x + t * RB;
+            const int v = threadIdx.x + t * NT;
             if (v >= nv) continue;
             dx[t] = make_float4((g[t].x * dx[t].x - cb * x[t].x) * invb, (g[t].y * dx[t].y - cb * x[t].y) * invb,
                                 (g[t].z * dx[t].z - cb * x[t].z) * invb, (g[t].w * dx[t].w - cb * x[t].w) * invb);
@@ -979,7 +982,7 @@ __global__ __launch_bounds__(RB) void k_norm_bwd_rows(NormBwdArgs a)
     const float s = row_scale_for(amax);
     const int Kb = tiled_kb(D);
 #pragma unroll
-    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * RB; if (v < nv) st_tiled4(a.d16, r, 4 * v, Kb, dx[t], s); }
+    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) st_tiled4(a.d16, r, 4 * v, Kb, dx[t], s); }
     zero_tiled_pad(a.d16, r, D, Kb);
     if (threadIdx.x == 0) a.inv_scale[r] = 1.0f / s;
 }
@@ -1154,6 +1157,7 @@ void launch_norm_rows(const NormRowsArgs &a, int rows)
     NormRowsArgs b = a;
     b.rows_launched = rows;
     const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
+    if (rows >= MANY_ROWS && !grouped && !a.pf.base && a.D <= 4 * TB * MAXV_ROW) { LAUNCH((k_norm_rows<MAXV_ROW, false, TB>), grid, dim3(TB), 0, b); return; }
     if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_rows<1, false>), grid, dim3(RB), 0, b); }
     else { if (grouped) LAUNCH((k_norm_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
 }
@@ -1264,6 +1268,7 @@ void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
     NormBwdArgs b = a;
     b.rows_launched = rows;
     const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
+    if (rows >= MANY_ROWS && !grouped && !a.pf.base && a.D <= 4 * TB * MAXV_ROW) { LAUNCH((k_norm_bwd_rows<MAXV_ROW, false, TB>), grid, dim3(TB), 0, b); return; }
     if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_bwd_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_bwd_rows<1, false>), grid, dim3(RB), 0, b); }
     else { if (grouped) LAUNCH((k_norm_bwd_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_bwd_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
 }

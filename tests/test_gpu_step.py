@@ -48,6 +48,8 @@ CASES = [
     # a factor each, and 2 * IS is not a whole number of backward groups, so one group straddles the dgate | dup boundary
     C1.with_(name="wide_ffn_groups", NL=1, IS=4224, V=1024, seq=64),
     TINY_GEMMA3.with_(name="gemma_wide_ffn", NL=2, IS=2112, seq=64),
+    # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
+    TINY_GEMMA3.with_(name="gemma_many_rows", NL=2, batch=4, seq=128),
 ]
 
 
