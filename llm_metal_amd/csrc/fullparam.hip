@@ -131,6 +131,47 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
                 for (int nh = 0; nh < 2; nh++)
                     acc[mt][nh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[nh][j], y[mt][j], acc[mt][nh], 0, 0, 0);
     }
+    if ((mb0 + 2) * 32 <= M_out && nk * 64 + 64 <= N_in) {
+        // Block inside the matrix: everything the read-modify-write needs is requested at once, then computed, then
+        // stored.  With the bounds tests of the general path below between them, each of the wave's sixteen
+        // load-update-store groups waits for the one before it.
+        float sy[2];
+        float4 xi[2][4];
+        half4 g[2][2][4];
+        half4 *gp[2][2][4];
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) sy[mt] = y_inv[(mb0 + mt) * 32 + l31];
+#pragma unroll
+        for (int nh = 0; nh < 2; nh++)
+#pragma unroll
+            for (int j4 = 0; j4 < 4; j4++) xi[nh][j4] = *reinterpret_cast<const float4 *>(x_inv + nk * 64 + nh * 32 + 8 * j4 + 4 * h);
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+            for (int nh = 0; nh < 2; nh++)
+#pragma unroll
+                for (int j4 = 0; j4 < 4; j4++) {
+                    gp[mt][nh][j4] = reinterpret_cast<half4 *>(
+                        target + ((((size_t)(mb0 + mt) * KbG + nk) * 4 + j4) * 64 + nh * 32 + l31) * 8 + 4 * h);
+                    g[mt][nh][j4] = *gp[mt][nh][j4];
+                }
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+            for (int nh = 0; nh < 2; nh++)
+#pragma unroll
+                for (int j4 = 0; j4 < 4; j4++) {
+                    const float xs[4] = {xi[nh][j4].x, xi[nh][j4].y, xi[nh][j4].z, xi[nh][j4].w};
+                    half4 o = g[mt][nh][j4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float a = acc[mt][nh][4 * j4 + i] * sy[mt] * xs[i];
+                        o[i] = SGD ? f2h(h2f(o[i]) - lr * a) : f2h(h2f(o[i]) + a);
+                    }
+                    *gp[mt][nh][j4] = o;
+                }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < 2; mt++) {
         const int m = (mb0 + mt) * 32 + l31;
