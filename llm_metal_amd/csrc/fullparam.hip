@@ -44,17 +44,30 @@ __global__ __launch_bounds__(256) void k_transpose_scaled(const half8 *__restric
     if (tid < 64) amax[tid] = 0.f;
     __syncthreads();
     {
+        // Requests in batches of four token blocks, none under a condition (indices clamped, the factor of a token that
+        // does not exist is 0): loads under a bounds test are waited for one at a time.  Per-thread maxima first, then
+        // one LDS atomic per feature.
         const int j = tid >> 6, lp = tid & 63, f0 = (lp >> 5) * 32 + 8 * j;
-        for (int tb = 0; tb < TbIn; tb++) {
-            const int token = tb * 32 + (lp & 31);
-            const half8 h = in[((size_t)tb * KbIn + fb) * 256 + tid];
-            const float s = token < T ? in_inv[token] : 0.f;
+        float lm[8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float v = fabsf(h2f(h[e]) * s);
-                if (v > 0.f) atomicMax(reinterpret_cast<unsigned *>(&amax[f0 + e]), __float_as_uint(v));
+        for (int e = 0; e < 8; e++) lm[e] = 0.f;
+        for (int tb0 = 0; tb0 < TbIn; tb0 += 4) {
+            half8 hb[4]; float sb[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int tb = tb0 + u, token = tb * 32 + (lp & 31);
+                hb[u] = in[((size_t)min(tb, TbIn - 1) * KbIn + fb) * 256 + tid];
+                sb[u] = in_inv[min(token, T - 1)];
+                if (token >= T) sb[u] = 0.f;
             }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) lm[e] = fmaxf(lm[e], fabsf(h2f(hb[u][e]) * sb[u]));
         }
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (lm[e] > 0.f) atomicMax(reinterpret_cast<unsigned *>(&amax[f0 + e]), __float_as_uint(lm[e]));
     }
     __syncthreads();
     if (tid < 64) {
@@ -64,28 +77,42 @@ __global__ __launch_bounds__(256) void k_transpose_scaled(const half8 *__restric
         out_inv[f] = f < F ? 1.0f / s : 0.f;
     }
     __syncthreads();
-    for (int tb2 = 0; tb2 < KbOut; tb2++) {
-        for (int q = tid; q < 512; q += 256) {
-            const int th = q >> 8, qq = q & 255, tile = tb2 * 2 + th;
-            const int j = qq >> 6, lp = qq & 63, tl = th * 32 + (lp & 31), f0 = (lp >> 5) * 32 + 8 * j;
-            const int token = tb2 * 64 + tl;
-            half8 h = {0, 0, 0, 0, 0, 0, 0, 0};
-            float s = 0.f;
-            if (tile < TbIn && token < T) { h = in[((size_t)tile * KbIn + fb) * 256 + qq]; s = in_inv[token]; }
+    // thread tid handles the quarter-tile slots q = tid (token half 0) and q = tid + 256 (token half 1) of every K step
+    const int j = tid >> 6, lp = tid & 63, f0 = (lp >> 5) * 32 + 8 * j;
+    auto request = [&](int tb2, half8 (&h)[2], float (&sc)[2]) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) t[tl][f0 + e] = f2h(h2f(h[e]) * s * scl[f0 + e]);
+        for (int th = 0; th < 2; th++) {
+            const int tile = tb2 * 2 + th, token = tb2 * 64 + th * 32 + (lp & 31);
+            h[th] = in[((size_t)min(tile, TbIn - 1) * KbIn + fb) * 256 + tid];
+            sc[th] = in_inv[min(token, T - 1)];
+            if (tile >= TbIn || token >= T) { sc[th] = 0.f; h[th] = half8{0, 0, 0, 0, 0, 0, 0, 0}; }
+        }
+    };
+    half8 h[2], hn[2];
+    float sc[2], scn[2];
+    request(0, h, sc);
+    for (int tb2 = 0; tb2 < KbOut; tb2++) {
+#pragma unroll
+        for (int th = 0; th < 2; th++) {
+            const int tl = th * 32 + (lp & 31);
+#pragma unroll
+            for (int e = 0; e < 8; e++) t[tl][f0 + e] = f2h(h2f(h[th][e]) * sc[th] * scl[f0 + e]);
         }
         __syncthreads();
-        for (int q = tid; q < 512; q += 256) {
-            const int th = q >> 8, qq = q & 255, rowtile = fb * 2 + th;
+        request(min(tb2 + 1, KbOut - 1), hn, scn);            // the next step's tiles travel while this one is written out
+#pragma unroll
+        for (int th = 0; th < 2; th++) {
+            const int rowtile = fb * 2 + th;
             if (rowtile >= FbOut) continue;
-            const int j = qq >> 6, lp = qq & 63, fl = th * 32 + (lp & 31), k0 = (lp >> 5) * 32 + 8 * j;
+            const int fl = th * 32 + (lp & 31), k0 = (lp >> 5) * 32 + 8 * j;
             half8 o;
 #pragma unroll
             for (int e = 0; e < 8; e++) o[e] = t[k0 + e][fl];
-            out[((size_t)rowtile * KbOut + tb2) * 256 + qq] = o;
+            out[((size_t)rowtile * KbOut + tb2) * 256 + tid] = o;
         }
         __syncthreads();
+#pragma unroll
+        for (int th = 0; th < 2; th++) { h[th] = hn[th]; sc[th] = scn[th]; }
     }
 }
 
