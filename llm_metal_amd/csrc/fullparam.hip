@@ -34,12 +34,12 @@ namespace {
 // out: tiled [F, T] fp16, value(f, t) = out[f][t] * out_inv[f]; zero in the K (token) padding and in
 //      rows >= F; out_inv has room for a multiple of 64 entries and gets 0 beyond F.
 // One workgroup per block of 64 features; two sweeps over the tokens (row maxima, then the data).
-__global__ __launch_bounds__(256) void k_transpose_scaled(const half8 *__restrict__ in, const float *__restrict__ in_inv,
-                                                           int T, int F, half8 *__restrict__ out, float *__restrict__ out_inv)
+__device__ __forceinline__ void transpose_scaled_block(const half8 *__restrict__ in, const float *__restrict__ in_inv,
+                                                       int T, int F, half8 *__restrict__ out, float *__restrict__ out_inv, int fb)
 {
     __shared__ float amax[64], scl[64];
     __shared__ half_t t[64][72];
-    const int tid = threadIdx.x, fb = blockIdx.x;
+    const int tid = threadIdx.x;
     const int KbIn = tiled_kb(F), TbIn = tiled_rb(T), KbOut = tiled_kb(T), FbOut = tiled_rb(F);
     if (tid < 64) amax[tid] = 0.f;
     __syncthreads();
@@ -114,6 +114,21 @@ __global__ __launch_bounds__(256) void k_transpose_scaled(const half8 *__restric
 #pragma unroll
         for (int th = 0; th < 2; th++) { h[th] = hn[th]; sc[th] = scn[th]; }
     }
+}
+
+__global__ __launch_bounds__(256) void k_transpose_scaled(const half8 *__restrict__ in, const float *__restrict__ in_inv,
+                                                           int T, int F, half8 *__restrict__ out, float *__restrict__ out_inv)
+{
+    transpose_scaled_block(in, in_inv, T, F, out, out_inv, blockIdx.x);
+}
+
+// Both operands of one weight gradient in one launch: the first nb0 workgroups transpose job 0, the rest job 1.
+struct TransposeJob { const half8 *in; const float *in_inv; int F; half8 *out; float *out_inv; };
+__global__ __launch_bounds__(256) void k_transpose_scaled_pair(TransposeJob j0, TransposeJob j1, int T, int nb0)
+{
+    const bool first = (int)blockIdx.x < nb0;             // uniform per workgroup
+    const TransposeJob &j = first ? j0 : j1;
+    transpose_scaled_block(j.in, j.in_inv, T, j.F, j.out, j.out_inv, first ? blockIdx.x : blockIdx.x - nb0);
 }
 
 // Target[m][n] (tiled [M_out, N_in] F16) <- half(float(Target) + alpha * sum_t Y[t][m] X[t][n])
@@ -283,6 +298,16 @@ void launch_transpose_scaled(const half_t *in_tiled, const float *in_inv, int T,
     if (T <= 0 || F <= 0) return;
     LAUNCH(k_transpose_scaled, dim3(tiled_kb(F)), dim3(256), 0, reinterpret_cast<const half8 *>(in_tiled), in_inv, T, F,
            reinterpret_cast<half8 *>(out_tiled), out_inv);
+}
+
+void launch_transpose_scaled_pair(const half_t *in0, const float *in0_inv, int F0, half_t *out0, float *out0_inv,
+                                  const half_t *in1, const float *in1_inv, int F1, half_t *out1, float *out1_inv, int T)
+{
+    if (T <= 0 || F0 <= 0 || F1 <= 0) { fprintf(stderr, "[fast_hip] transpose_scaled_pair: empty operand\n"); abort(); }
+    const TransposeJob j0{reinterpret_cast<const half8 *>(in0), in0_inv, F0, reinterpret_cast<half8 *>(out0), out0_inv};
+    const TransposeJob j1{reinterpret_cast<const half8 *>(in1), in1_inv, F1, reinterpret_cast<half8 *>(out1), out1_inv};
+    const int nb0 = tiled_kb(F0);
+    LAUNCH(k_transpose_scaled_pair, dim3(nb0 + tiled_kb(F1)), dim3(256), 0, j0, j1, T, nb0);
 }
 
 void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,

@@ -180,6 +180,9 @@ void launch_fill_f32(float *p, float v, size_t n);
 // ---- full-parameter mode (fullparam.hip) ----
 // out (tiled [F, T]) and out_inv[F] <- transposed in (tiled [T, F]) with in_inv[T]; out_inv needs tiled_kb(F)*64 floats
 void launch_transpose_scaled(const half_t *in_tiled, const float *in_inv, int T, int F, half_t *out_tiled, float *out_inv);
+// two operands [T, F0] and [T, F1] in one launch
+void launch_transpose_scaled_pair(const half_t *in0, const float *in0_inv, int F0, half_t *out0, float *out0_inv,
+                                  const half_t *in1, const float *in1_inv, int F1, half_t *out1, float *out1_inv, int T);
 // target (tiled [M_out, N_in] F16) <- half(target + alpha * Y^T X), XT/YT = transposed operands over T tokens;
 // sgd: alpha = -lr (f16_sgd_fused), else alpha = 1 (f16_grad_accum)
 void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,

@@ -362,8 +362,8 @@ void weight_grad(SFTState *s, int mode, float lr, const half_t *dY16, const floa
                  MetalBuf *W, MetalBuf *WT, MetalBuf *G, size_t w_off, size_t wt_off)
 {
     if (mode == BWD_ACCUM && !G) { fprintf(stderr, "[fast_sft] gradient accumulators are not allocated\n"); abort(); }
-    launch_transpose_scaled(dY16, dy_inv, s->BN, M_out, at<half_t>(s->yT), at<float>(s->yT_inv));
-    launch_transpose_scaled(X16, x_inv, s->BN, N_in, at<half_t>(s->xT), at<float>(s->xT_inv));
+    launch_transpose_scaled_pair(dY16, dy_inv, M_out, at<half_t>(s->yT), at<float>(s->yT_inv),
+                                 X16, x_inv, N_in, at<half_t>(s->xT), at<float>(s->xT_inv), s->BN);
     if (mode == BWD_ACCUM) {
         launch_wgrad(at<half_t>(s->xT), at<float>(s->xT_inv), at<half_t>(s->yT), at<float>(s->yT_inv),
                      at<half_t>(G, w_off), M_out, N_in, s->BN, 0, 0.f);
