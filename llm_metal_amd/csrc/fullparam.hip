@@ -158,25 +158,27 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
         for (int b = 0; b < 2; b++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
-    for (int kt = 0; kt < Kt; kt++) {
-        const size_t o = (size_t)kt * 256;
-        half8 x[2][4], y[2][4];
+    auto contract_tokens = [&]() {
+        for (int kt = 0; kt < Kt; kt++) {
+            const size_t o = (size_t)kt * 256;
+            half8 x[2][4], y[2][4];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+            for (int j = 0; j < 4; j++)
 #pragma unroll
-            for (int i = 0; i < 2; i++) { x[i][j] = xp[i][o + j * 64]; y[i][j] = yp[i][o + j * 64]; }
+                for (int i = 0; i < 2; i++) { x[i][j] = xp[i][o + j * 64]; y[i][j] = yp[i][o + j * 64]; }
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+            for (int j = 0; j < 4; j++)
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++)
+                for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-                for (int nh = 0; nh < 2; nh++)
-                    acc[mt][nh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[nh][j], y[mt][j], acc[mt][nh], 0, 0, 0);
-    }
+                    for (int nh = 0; nh < 2; nh++)
+                        acc[mt][nh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[nh][j], y[mt][j], acc[mt][nh], 0, 0, 0);
+        }
+    };
     if ((mb0 + 2) * 32 <= M_out && nk * 64 + 64 <= N_in) {
-        // Block inside the matrix: everything the read-modify-write needs is requested at once, then computed, then
-        // stored.  With the bounds tests of the general path below between them, each of the wave's sixteen
-        // load-update-store groups waits for the one before it.
+        // Block inside the matrix: everything the read-modify-write needs is requested at once, before the contraction
+        // (whose loads it then travels with), then computed, then stored.  With the bounds tests of the general path
+        // below between them, each of the wave's sixteen load-update-store groups waits for the one before it.
         float sy[2];
         float4 xi[2][4];
         half4 g[2][2][4];
@@ -197,6 +199,7 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
                         target + ((((size_t)(mb0 + mt) * KbG + nk) * 4 + j4) * 64 + nh * 32 + l31) * 8 + 4 * h);
                     g[mt][nh][j4] = *gp[mt][nh][j4];
                 }
+        contract_tokens();
 #pragma unroll
         for (int mt = 0; mt < 2; mt++)
 #pragma unroll
@@ -214,6 +217,7 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
                 }
         return;
     }
+    contract_tokens();
 #pragma unroll
     for (int mt = 0; mt < 2; mt++) {
         const int m = (mb0 + mt) * 32 + l31;
