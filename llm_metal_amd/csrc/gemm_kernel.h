@@ -186,9 +186,12 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
     __syncthreads();
     // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4.  SCALE: the row factors
     // are fetched here, where the K loop's registers are free (holding them through the loop costs a wave of occupancy).
+    // A tile inside the matrix stores without bounds tests: under a test per element the compiler puts each LDS read into
+    // the branch of its store, and the sixteen read-wait-store groups run one after the other.
+    const bool inside = (mb0 + 2) * 32 <= M && (nb0 + NB) * 32 <= N;
 #define QUARTER_STORE(W) if (wave == (W)) { \
         constexpr int i0 = (W) * Q; \
-        float sc[Q]; \
+        float sc[Q], sres[Q]; \
         if (SCALE) { \
             /* all factors requested before the first store (row clamped): a load under the store's condition would make \
                every store wait for the one before it */ \
@@ -198,11 +201,21 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
             } \
         } \
         _Pragma("unroll") for (int k = 0; k < Q; k++) { \
-            const int i = i0 + k, mb = i / (NB * 16), b = (i / 16) % NB, v = i % 16; \
-            const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), n = (nb0 + b) * 32 + r; \
-            float sres = ACC_AT(i0 + k) + theirs[k * 64 + lane]; \
-            if (SCALE) sres *= sc[k]; \
-            if (m < M && n < N) Pp[(size_t)m * g.ldp + n] = sres; \
+            sres[k] = ACC_AT(i0 + k) + theirs[k * 64 + lane]; \
+            if (SCALE) sres[k] *= sc[k]; \
+        } \
+        if (inside) { \
+            _Pragma("unroll") for (int k = 0; k < Q; k++) { \
+                const int i = i0 + k, mb = i / (NB * 16), b = (i / 16) % NB, v = i % 16; \
+                const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), n = (nb0 + b) * 32 + r; \
+                Pp[(size_t)m * g.ldp + n] = sres[k]; \
+            } \
+        } else { \
+            _Pragma("unroll") for (int k = 0; k < Q; k++) { \
+                const int i = i0 + k, mb = i / (NB * 16), b = (i / 16) % NB, v = i % 16; \
+                const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), n = (nb0 + b) * 32 + r; \
+                if (m < M && n < N) Pp[(size_t)m * g.ldp + n] = sres[k]; \
+            } \
         } }
     QUARTER_STORE(0) QUARTER_STORE(1) QUARTER_STORE(2) QUARTER_STORE(3)
 #undef QUARTER_STORE
