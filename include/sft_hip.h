@@ -9,8 +9,9 @@
  *  - State is built from the reference's own model-independent description
  *    (LayerWeightRef, src/nn/wmat.h:39-56) wrapped in SFTModelRef, not from
  *    Qwen3Model / Gemma3Model: those structs belong to the reference's CPU
- *    tensor runtime.  The two-line adapters that fill an SFTModelRef from them
- *    are shown in INTEGRATION.md.
+ *    tensor runtime.  An adapter that fills an SFTModelRef from either is a loop
+ *    over the layers that fills one LayerWeightRef (seven matrices, six norm
+ *    vectors) per layer.
  *  - `batch` sequences per step (the reference has batch 1): RoPE positions and
  *    causal attention restart at every sequence.
  *  - Embedding gather, loss scaling, global-norm clipping and AdamW run on the

@@ -336,8 +336,9 @@ OR_API void or_rope_train_bwd(real *q, real *k, int Hq, int Hkv, int hd, int N, 
 /* attn_train_fwd, shaders/q8_kernels.metal:769-851: per (head, query i):
  * s_j = q_i.k_j * scale for j <= i, softmax over j <= i, probs row saved
  * (zeros for j > i), out_i = sum_j p_j v_j.  The row reduction is the exact
- * sum (the reference's tree reduction is only exact for power-of-two group
- * sizes; see DESIGN notes in the repository root). */
+ * sum (the reference's tree reduction leaves lanes out when the group size is
+ * not a power of two; for power-of-two sizes both give the same sum up to
+ * fp32 rounding order). */
 OR_API void or_attn_train_fwd(const real *Q, const real *K, const real *V, real *out, real *probs,
                               int H, int N, int D, float scale)
 {
