@@ -243,6 +243,7 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         abort();
     }
     dim3 grid(p.n_tiles, p.S, p.m_tiles), block(p.nw * 64);
+    if (p.m_tiles > 1) grid = dim3((unsigned)(((size_t)p.n_tiles * p.S + 7) / 8 * 8 * p.m_tiles), 1, 1);   // see gemm_tiled
     const size_t lds = (size_t)(p.nw / 2) * (2 * p.nb * 16) * 64 * sizeof(float);
     // When profiling, the events ride on the dispatch itself (hipExtLaunchKernelGGL), so their
     // difference is the kernel's own execution time without the gaps a separate record adds.
@@ -259,6 +260,7 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
     g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
     g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
     g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
+    g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = p.m_tiles;
 #define GEMM_LAUNCH(NBV, ROT, SC, WFV) do { \
         if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
         else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), g); } while (0)

@@ -10,6 +10,7 @@ struct GemmKArgs {
     WeightOp W;
     float *P; int ldp; size_t plane_stride;
     int M, N, Mb, Nb, Kb, steps_per_chunk;
+    int n_tiles, S, m_tiles;                             // set (m_tiles > 1) when the grid is the 1-D one described at gemm_tiled
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -98,9 +99,20 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
     extern __shared__ float red[];                       // [NW][NB*16 regs][64 lanes]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int nb0 = blockIdx.x * NB, mb0 = blockIdx.z * 2;
+    // Block coordinates: (weight-row tile, K chunk, 64-row tile of the activations).  With one row tile they are the grid's.
+    // With several, the workgroups that share a weight tile must meet in one L2 or the weights are streamed from memory
+    // once per row tile: the grid is then 1-D, the hardware deals consecutive ids to the eight XCDs in turn, and the ids
+    // (8 * (m_tiles * u + z) + xcd), z = 0 .. m_tiles - 1, take the row tiles of weight tile 8 * u + xcd.
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    if (g.m_tiles > 1) {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        const int t = (slot / g.m_tiles) * 8 + xcd;
+        if (t >= g.n_tiles * g.S) return;                 // padding of the last group of eight; the whole workgroup leaves
+        bz = slot % g.m_tiles; bx = t % g.n_tiles; by = t / g.n_tiles;
+    }
+    const int nb0 = bx * NB, mb0 = bz * 2;
     const int Kb = g.Kb, Nb = g.Nb, M = g.M, N = g.N;
-    const int kb_beg = blockIdx.y * g.steps_per_chunk;
+    const int kb_beg = by * g.steps_per_chunk;
     const int nsteps = min(Kb, kb_beg + g.steps_per_chunk) - kb_beg;
 
     int nbi[NB];                                          // row block of each weight tile (clamped: the extra rows are never stored)
@@ -120,7 +132,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
             for (int v = 0; v < 16; v++) acc[mb][b][v] = 0.f;
 
     // wave w takes the K steps w, w+NW, w+2NW, ... of this workgroup's chunk (rotated)
-    const int rot = ROTATE ? (int)((blockIdx.x * 7u + blockIdx.y * 3u) % (unsigned)nsteps) : 0;
+    const int rot = ROTATE ? (int)(((unsigned)bx * 7u + (unsigned)by * 3u) % (unsigned)nsteps) : 0;
     for (int i = wave; i < nsteps; i += NW) {
         int kk = i + rot;
         if (kk >= nsteps) kk -= nsteps;
@@ -177,7 +189,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
         }
         __syncthreads();                                  // all have read before the slots are written again
     }
-    float *Pp = g.P + (size_t)blockIdx.y * g.plane_stride;
+    float *Pp = g.P + (size_t)by * g.plane_stride;
     float *mine = red + (size_t)wave * Q * 64;
     const float *theirs = red + (size_t)(wave ^ 1) * Q * 64;
 #define QUARTER_GIVE(W) if (wave == (W)) { _Pragma("unroll") for (int k = 0; k < Q; k++) mine[k * 64 + lane] = ACC_AT(((W) ^ 1) * Q + k); }
