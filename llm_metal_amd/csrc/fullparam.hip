@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l31 = lane & 31, h = lane >> 5;
     const int KbG = tiled_kb(N_in), MbG = tiled_rb(M_out), NbX = tiled_rb(N_in);
     const int nk = blockIdx.x * 4 + wave, mb0 = blockIdx.y * 2;
-    if (nk >= KbG) return;
+    const bool active = nk < KbG;                         // a wave past the last column block still fetches its share of Y
     const half8 *xp[2], *yp[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -158,14 +158,26 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
         for (int b = 0; b < 2; b++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+    // The four waves of a workgroup multiply the same two row blocks of Y^T: each fetches a quarter of them (block
+    // wave & 1, MFMA slices 2 (wave >> 1) and + 1) and they exchange through LDS, double buffered, one barrier per step.
+    __shared__ half8 ysh[2][2][4][64];
     auto contract_tokens = [&]() {
+        const int yi = wave & 1, yj = (wave >> 1) * 2;
         for (int kt = 0; kt < Kt; kt++) {
             const size_t o = (size_t)kt * 256;
             half8 x[2][4], y[2][4];
+            const half8 ya = yp[yi][o + yj * 64], yb = yp[yi][o + (yj + 1) * 64];
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int i = 0; i < 2; i++) { x[i][j] = xp[i][o + j * 64]; y[i][j] = yp[i][o + j * 64]; }
+                for (int i = 0; i < 2; i++) x[i][j] = xp[i][o + j * 64];
+            ysh[kt & 1][yi][yj][lane] = ya;
+            ysh[kt & 1][yi][yj + 1][lane] = yb;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int i = 0; i < 2; i++) y[i][j] = ysh[kt & 1][i][j][lane];
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -175,7 +187,7 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
                         acc[mt][nh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[nh][j], y[mt][j], acc[mt][nh], 0, 0, 0);
         }
     };
-    if ((mb0 + 2) * 32 <= M_out && nk * 64 + 64 <= N_in) {
+    if (active && (mb0 + 2) * 32 <= M_out && nk * 64 + 64 <= N_in) {
         // Block inside the matrix: everything the read-modify-write needs is requested at once, before the contraction
         // (whose loads it then travels with), then computed, then stored.  With the bounds tests of the general path
         // below between them, each of the wave's sixteen load-update-store groups waits for the one before it.
@@ -218,6 +230,7 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
         return;
     }
     contract_tokens();
+    if (!active) return;
 #pragma unroll
     for (int mt = 0; mt < 2; mt++) {
         const int m = (mb0 + mt) * 32 + l31;
