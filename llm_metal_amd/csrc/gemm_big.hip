@@ -242,6 +242,139 @@ __global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
         }
 }
 
+
+// F16 weight tiles need no unpacking, so their steps go from L2/HBM straight into LDS (global_load_lds_dwordx4: a
+// wave-uniform LDS base in M0, lane i's 16 bytes land at base + 16 i -- the [j][lane] order of the tiles) and never
+// pass through registers or ds_write.  Three LDS buffers (distinct objects, so that the compiler knows that a read of
+// one does not have to wait for a load into another): step kt is multiplied out of buffer kt % 3 while the loads of
+// steps kt + 1 and kt + 2 are in flight.  One barrier per step; the wait before it is written by hand (vmcnt <= 12: the
+// twelve loads of the step after may still be out), because a fence would wait for all of them.
+constexpr int DMA_LOADS = 4 + 4 * WPW;                    // per wave and step
+static_assert(DMA_LOADS == 12, "the hand-written wait below counts twelve loads per step");
+
+__global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
+{
+    constexpr int NBLK = 4 + 4 * WPW, BUF = NBLK * 256, NW = 2 * WPW;
+    __shared__ half8 lb0[BUF], lb1[BUF], lb2[BUF];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int MT = (g.M + 127) >> 7, NT = (g.N + 128 * WPW - 1) / (128 * WPW);
+    const int m_patches = (MT + 7) >> 3;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3, patch = seq >> 5, in_patch = seq & 31;
+    const int mt = (patch % m_patches) * 8 + (in_patch & 7);
+    const int nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
+    if (mt >= MT || nt >= NT) return;
+    const int nb0 = nt * 4 * WPW, mb0 = mt * 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const half8 *asrc = g.A + (size_t)min(mb0 + wave, g.Mb - 1) * g.Kb * 256 + lane;
+    const half8 *wsrc[WPW];
+#pragma unroll
+    for (int u = 0; u < WPW; u++)
+        wsrc[u] = reinterpret_cast<const half8 *>(g.W.w16) + (size_t)min(nb0 + wave * WPW + u, g.Nb - 1) * g.Kb * 256 + lane;
+
+    float16v acc[2][NW];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < NW; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    typedef __attribute__((address_space(3))) void lds_void;
+    auto request = [&](half8 (&buf)[BUF], int kt) __attribute__((always_inline)) {
+        const size_t o = (size_t)kt * 256;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            __builtin_amdgcn_global_load_lds(asrc + o + j * 64, (lds_void *)(buf + (wave * 4 + j) * 64), 16, 0, 0);
+#pragma unroll
+        for (int u = 0; u < WPW; u++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                __builtin_amdgcn_global_load_lds(wsrc[u] + o + j * 64, (lds_void *)(buf + ((4 + wave * WPW + u) * 4 + j) * 64), 16, 0, 0);
+    };
+    const int last = g.Kb - 1;
+    // one K step: `cur` holds step kt; `free_buf` held step kt - 1 and takes step kt + 2
+    auto step = [&](int kt, half8 (&cur)[BUF], half8 (&free_buf)[BUF]) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+        request(free_buf, min(kt + 2, last));
+        half8 a[2][2], w[2][NW];
+        auto read = [&](int j) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) a[j & 1][i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
+#pragma unroll
+            for (int k = 0; k < NW; k++) w[j & 1][k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
+        };
+        read(0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (j + 1 < 4) read(j + 1);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int k = 0; k < NW; k++)
+                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 1][i], w[j & 1][k], acc[i][k], 0, 0, 0);
+        }
+        // issue order: the 6 LDS reads of slice 0, then under each MFMA one LDS read of the next slice and one of the
+        // twelve requests
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 24 && (i & 7) < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+    };
+    request(lb0, 0);
+    request(lb1, min(1, last));
+    const int full = g.Kb / 3 * 3;
+    for (int kt0 = 0; kt0 < full; kt0 += 3) {
+        step(kt0, lb0, lb2);
+        step(kt0 + 1, lb1, lb0);
+        step(kt0 + 2, lb2, lb1);
+    }
+    if (full < g.Kb) step(full, lb0, lb2);
+    if (full + 1 < g.Kb) step(full + 1, lb1, lb0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the repeated requests of the last steps land before the LDS is given back
+
+    if (mb0 * 32 + 128 <= g.M && (nb0 + 4 * WPW) * 32 <= g.N) {
+        float sc[2][16];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) sc[i][v] = 1.0f;
+        if (g.a_inv_scale) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    sc[i][v] = g.a_inv_scale[(mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3)];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = (mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                float *row = g.P + (size_t)m * g.ldp + (nb0 + NW * wn) * 32 + r;
+#pragma unroll
+                for (int k = 0; k < NW; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = (mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (m >= g.M) continue;
+            const float sc = g.a_inv_scale ? g.a_inv_scale[m] : 1.0f;
+#pragma unroll
+            for (int k = 0; k < NW; k++) {
+                const int n = (nb0 + NW * wn + k) * 32 + r;
+                if (n < g.N) g.P[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
+            }
+        }
+}
+
 }  // namespace
 
 void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K)
@@ -270,11 +403,11 @@ void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &
     }
     hipEvent_t ev_a = nullptr, ev_b = nullptr;
     if (gemm_prof_begin(weight_stream_bytes(W, N, K), 2.0 * M * N * K, &ev_a, &ev_b)) {
-        if (W.fmt == 0) hipExtLaunchKernelGGL(gemm_big<0>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
+        if (W.fmt == 0) hipExtLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), ev_a, ev_b, 0, g);
         else if (W.fmt == 1) hipExtLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
         else hipExtLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
     } else {
-        if (W.fmt == 0) hipLaunchKernelGGL(gemm_big<0>, grid, block, lds, stream(), g);
+        if (W.fmt == 0) hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), g);
         else if (W.fmt == 1) hipLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), g);
         else hipLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), g);
     }
