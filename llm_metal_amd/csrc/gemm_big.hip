@@ -10,7 +10,8 @@
 // per consumer), and both go to LDS in the same [j][lane][8 halves] order, so a wave reads any row block back
 // with conflict-free 16-byte loads.  LDS is double buffered and the operands travel three steps ahead in registers:
 // during the MFMAs of step k the loads of step k+3 are issued and step k+1 is written to the other buffer; one
-// barrier per step.
+// barrier per step.  That is the kernel for Q8_0 tiles (gemm_big<1>, <2>); F16 tiles take gemm_big_f16 below, whose
+// operands reach LDS without passing through registers.
 #include "backend.h"
 #include "devutil.h"
 #include "gemm.h"
@@ -396,7 +397,6 @@ void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &
     const size_t lds = (size_t)2 * (4 + 4 * WPW) * 256 * sizeof(half8);
     static bool attr_set = false;
     if (!attr_set) {
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_big<0>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_big<1>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_big<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_set = true;
