@@ -262,8 +262,13 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
     g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
     g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = p.m_tiles;
 #define GEMM_LAUNCH(NBV, ROT, SC, WFV) do { \
-        if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
-        else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), g); } while (0)
+        if (p.m_tiles > 1) { \
+            if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV, 1>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
+            else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV, 1>), grid, block, lds, stream(), g); \
+        } else { \
+            if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
+            else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), g); \
+        } } while (0)
 #define GEMM_PICK_SC(NBV, ROT, WFV) do { if (a_inv_scale) GEMM_LAUNCH(NBV, ROT, 1, WFV); else GEMM_LAUNCH(NBV, ROT, 0, WFV); } while (0)
 #define GEMM_PICK_ROT(NBV, WFV) do { if (p.rotate) GEMM_PICK_SC(NBV, 1, WFV); else GEMM_PICK_SC(NBV, 0, WFV); } while (0)
 #define GEMM_PICK_NB(WFV) do { if (p.nb == 2) GEMM_PICK_ROT(2, WFV); else GEMM_PICK_ROT(1, WFV); } while (0)

@@ -93,7 +93,7 @@ __device__ __forceinline__ void load_w_q8_cols(half8 (&w)[4], const WeightOp &W,
 // WF: weight format (WeightOp::fmt).  1: row blocks below W.nbq are Q8_0 tiles, the rest F16 tiles
 // (the trainable LoRA rows of the fused QKV weight); the planner keeps W.nbq a multiple of NB, so a
 // workgroup is of one kind.  2: K steps below W.kbq are Q8_0 tiles with column scales, the rest F16.
-template <int NB, int NW, int ROTATE, int SCALE, int WF>
+template <int NB, int NW, int ROTATE, int SCALE, int WF, int MTILES = 0>
 __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 {
     extern __shared__ float red[];                       // [NW][NB*16 regs][64 lanes]
@@ -102,9 +102,9 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
     // Block coordinates: (weight-row tile, K chunk, 64-row tile of the activations).  With one row tile they are the grid's.
     // With several, the workgroups that share a weight tile must meet in one L2 or the weights are streamed from memory
     // once per row tile: the grid is then 1-D, the hardware deals consecutive ids to the eight XCDs in turn, and the ids
-    // (8 * (m_tiles * u + z) + xcd), z = 0 .. m_tiles - 1, take the row tiles of weight tile 8 * u + xcd.
+    // (8 * (m_tiles * u + z) + xcd), z = 0 .. m_tiles - 1, take the row tiles of weight tile 8 * u + xcd (MTILES = 1).
     int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
-    if (g.m_tiles > 1) {
+    if (MTILES) {                                         // compile-time: the one-tile kernels do not carry this code
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
         const int t = (slot / g.m_tiles) * 8 + xcd;
         if (t >= g.n_tiles * g.S) return;                 // padding of the last group of eight; the whole workgroup leaves
