@@ -17,9 +17,9 @@
  *     (rms_norm, rms_norm_backward, silu/gelu_mul_backward with dgate == dout).
  * Differences forced by a discrete GPU are listed at metal_buf_ptr.
  *
- * Not exported yet: the 16 inference-only enqueues (q8_matvec, f16_matvec,
- * f16_batch_matvec, rms_norm (single), per_head_rms_norm, rope,
- * kv_cache_store, attention and the _off variants; src/nn/fast_metal.h:20-80).
+ * All 49 symbols of src/nn/fast_metal.h are exported: init / shutdown, the
+ * buffer functions, flush, the 26 training enqueues and the 16 inference
+ * enqueues (:20-80, declared further down).
  */
 #ifndef FAST_HIP_H
 #define FAST_HIP_H
@@ -152,7 +152,9 @@ void hip_enqueue_q8_dequant(MetalBuf *src, MetalBuf *dst, int rows, int cols);
 /* dst F16 [rows, cols] = half(float(scale) * code): the values the dequant-fused GEMM multiplies with */
 void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
 
-/* 0: choose the GEMM kernel by the measured rule; 1: always the LDS-tiled large-M kernel; -1: never. */
+/* 0: choose the GEMM kernel by the measured rule; 1: always the LDS-tiled large-M kernel (Q8_0 operands through an
+ * F16 image made once per product); 2: always the large-M kernel with Q8_0 tiles kept quantised and unpacked into LDS
+ * by the kernel itself; -1: never (always the weight-streaming kernel). */
 void hip_gemm_force_large_m(int policy);
 /* Timing aid for benchmarks: when enabled, every GEMM launch is bracketed by HIP events on the
  * library's stream.  hip_gemm_profile_read (after metal_flush) returns the number of launches recorded

@@ -9,13 +9,26 @@
  *  - State is built from the reference's own model-independent description
  *    (LayerWeightRef, src/nn/wmat.h:39-56) wrapped in SFTModelRef, not from
  *    Qwen3Model / Gemma3Model: those structs belong to the reference's CPU
- *    tensor runtime.  An adapter that fills an SFTModelRef from either is a loop
- *    over the layers that fills one LayerWeightRef (seven matrices, six norm
- *    vectors) per layer.
+ *    tensor runtime.  The constructors and the adapter sync with the
+ *    reference's signatures (src/nn/fast_sft.h:14-23, 54-55) are declared and
+ *    implemented, over the functions below, in llm_metal_amd/compat/
+ *    fast_sft_compat.{h,c}, which are compiled inside the reference tree.
  *  - `batch` sequences per step (the reference has batch 1): RoPE positions and
  *    causal attention restart at every sequence.
  *  - Embedding gather, loss scaling, global-norm clipping and AdamW run on the
  *    device; the host touches only tokens, targets and the per-row losses.
+ *
+ * Limits (a constructor prints the reason and returns NULL, a product that does
+ * not fit aborts with a message):
+ *  - d_model, FFN width, vocabulary and head_dim multiples of 4; n_q_heads a
+ *    multiple of n_kv_heads; Q8_0 additionally needs d_model, FFN width and
+ *    n_q_heads * head_dim to be multiples of 32;
+ *  - LoRA rank even and at most 16 (0 selects full-parameter mode);
+ *  - d_model and FFN width at most 12 288 (one workgroup keeps a row in
+ *    registers); (n_q_heads + 2 n_kv_heads) * head_dim + 2 rank at most 15 872
+ *    (a row of dq | dk | dv | dh is staged in 64 KB of LDS); head_dim at most 512;
+ *    seq_len at most 4096.  head_dim 32, 64, 128 or 256 with seq_len <= 1024
+ *    takes the matrix-core attention, other shapes a slower kernel.
  */
 #ifndef SFT_HIP_H
 #define SFT_HIP_H
@@ -26,7 +39,10 @@
 extern "C" {
 #endif
 
-/* ---- src/nn/wmat.h:10-78 ---- */
+/* ---- src/nn/wmat.h:10-78, under that header's own include guard: whichever of the two comes first in a
+ *      translation unit of the reference declares these types and functions ---- */
+#ifndef WMAT_H
+#define WMAT_H
 typedef enum { MODEL_QWEN3, MODEL_GEMMA3 } ModelType;
 
 typedef struct WMat {
@@ -64,6 +80,7 @@ LayerW *layers_convert_upload(const LayerWeightRef *refs, int n_layers, int use_
 void  layers_free(LayerW *layers, int n_layers);
 WMat *wmat_convert(const float *data, int rows, int cols, int use_fp16);
 MetalBuf *norm_upload(const float *gamma, int dim);
+#endif /* WMAT_H */
 
 /* ---- model description (replaces the Qwen3Model / Gemma3Model arguments of
  *      sft_state_create*, src/nn/fast_sft.c:171-396) ---- */
@@ -165,7 +182,12 @@ void sft_copy_lora(SFTState *state, float *dst);
 void sft_copy_lora_grads(SFTState *state, float *dst);
 void sft_set_lora(SFTState *state, const float *src);
 float sft_get_last_grad_norm(SFTState *state);
-/* Enqueue forward + loss + backward + update without waiting (sft_train_step = this + flush + mean). */
+/* Enqueue forward + loss + backward + update without waiting (sft_train_step = this + flush + mean).
+ * One step is in flight at a time: the kernels read tokens, targets and optimiser parameters from pinned buffers of
+ * the state, so a second enqueue before sft_finish_train_step first waits for the outstanding step.
+ * Token and target ids are checked against the vocabulary on the host; with an id outside it nothing is launched, a
+ * message goes to stderr and sft_finish_train_step / sft_train_step return NaN (grpo_apply_completions returns
+ * without touching the state). */
 void sft_enqueue_train_step(SFTState *state, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr);
 float sft_finish_train_step(SFTState *state);
 

@@ -347,7 +347,7 @@ int gemm_profiling() { return g_prof_on; }
 // 340-460 TFLOP/s), but from 1024 rows on it pays to dequantise the operand once into an F16 image (3 bytes of extra
 // HBM traffic per weight) and run the large-M kernel on that instead of unpacking every tile again for each 64 rows
 // of activations: 4 x 512 rows, 112.9 ms per step against 123 ms (streaming) and 125 ms (Q8_0 inside the large-M kernel).
-int g_big_policy = 0;                                     // 0 measured rule, 1 always, -1 never
+int g_big_policy = 0;                                     // 0 measured rule, 1 always, -1 never, 2 always and Q8_0 tiles stay quantised
 bool use_big_gemm(int M, int N, int K, int fmt)
 {
     (void)K;
@@ -361,7 +361,7 @@ bool use_big_gemm(int M, int N, int K, int fmt)
 // the next call).
 WeightOp f16_image_of(const WeightOp &W, int N, int K)
 {
-    if (W.fmt == 0) return W;
+    if (W.fmt == 0 || g_big_policy == 2) return W;        // policy 2: the large-M kernel unpacks the Q8_0 tiles into LDS itself
     const int Nb = tiled_rb(N), Kb = tiled_kb(K);
     const size_t tiles = (size_t)Nb * Kb;
     half8 *img = (half8 *)scratch(SCR_WF16, tiles * 256 * sizeof(half8));

@@ -296,7 +296,10 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
     const int last = g.Kb - 1;
     // one K step: `cur` holds step kt; `free_buf` held step kt - 1 and takes step kt + 2
     auto step = [&](int kt, half8 (&cur)[BUF], half8 (&free_buf)[BUF]) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+        // lgkmcnt(0): every LDS read this wave issued for step kt - 1 has returned before the barrier lets other waves
+        // overwrite that buffer (the MFMAs that consume them are not memory operations and may be scheduled past this
+        // statement, so their own waits do not order the reuse)
+        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
         request(free_buf, min(kt + 2, last));
         half8 a[2][2], w[2][NW];
         auto read = [&](int j) {

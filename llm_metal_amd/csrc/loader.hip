@@ -32,8 +32,26 @@ struct TensorInfo {
     int dtype = -1, ndim = 0, shard = 0;
     uint64_t shape[4] = {0, 0, 0, 0};
     uint64_t begin = 0, nbytes = 0;   // relative to the shard's data_off
-    uint64_t elements() const { uint64_t n = 1; for (int d = 0; d < ndim; d++) n *= shape[d]; return n; }
+    // Product of the dimensions; UINT64_MAX when it would pass 2^48 (no tensor of a model file is that large, and
+    // nothing downstream can then overflow when it multiplies by an element size).
+    uint64_t elements() const
+    {
+        constexpr uint64_t cap = (uint64_t)1 << 48;
+        uint64_t n = 1;
+        for (int d = 0; d < ndim; d++) {
+            if (shape[d] != 0 && n > cap / shape[d]) return UINT64_MAX;
+            n *= shape[d];
+        }
+        return n;
+    }
 };
+
+// true when [begin, begin + nbytes) lies inside the data section of a mapping of `size` bytes that starts at data_off
+// (written so that no sum can wrap)
+bool range_inside(uint64_t data_off, uint64_t begin, uint64_t nbytes, uint64_t size)
+{
+    return data_off <= size && begin <= size - data_off && nbytes <= size - data_off - begin;
+}
 
 }  // namespace
 
@@ -154,6 +172,7 @@ bool parse_safetensors_header(const char *text, size_t len, int shard, std::vect
             } while (j.eat(','));
             if (!j.eat('}')) return false;
         }
+        if (off[1] < off[0]) return false;                 // reversed data_offsets
         t.begin = off[0];
         t.nbytes = off[1] - off[0];
         out.push_back(t);
@@ -179,7 +198,8 @@ bool open_safetensors_shard(const std::string &path, ModelFile *f)
     }
     for (size_t i = before; i < f->tensors.size(); i++) {
         const TensorInfo &t = f->tensors[i];
-        if (m.data_off + t.begin + t.nbytes > m.size || (t.dtype >= 0 && t.nbytes != bytes_of(t.dtype, t.elements()))) {
+        const uint64_t ne = t.elements();
+        if (ne == UINT64_MAX || !range_inside(m.data_off, t.begin, t.nbytes, m.size) || (t.dtype >= 0 && t.nbytes != bytes_of(t.dtype, ne))) {
             fprintf(stderr, "[Loader] %s: tensor %s has offsets outside the file or not matching its shape\n", path.c_str(), t.name.c_str());
             f->tensors.resize(before);
             munmap(m.p, m.size);
@@ -197,8 +217,8 @@ struct Reader {
     size_t off, size;
     bool ok = true;
     template <typename T> T get() { T v{}; if (off + sizeof(T) > size) { ok = false; return v; } memcpy(&v, p + off, sizeof(T)); off += sizeof(T); return v; }
-    std::string str() { const uint64_t n = get<uint64_t>(); if (!ok || off + n > size) { ok = false; return ""; } std::string s((const char *)p + off, n); off += n; return s; }
-    void skip(size_t n) { if (off + n > size) ok = false; else off += n; }
+    std::string str() { const uint64_t n = get<uint64_t>(); if (!ok || n > size - off) { ok = false; return ""; } std::string s((const char *)p + off, n); off += n; return s; }
+    void skip(uint64_t n) { if (n > size - off) ok = false; else off += n; }   // off <= size always, so the difference cannot wrap
 };
 
 // GGUF metadata value types (src/data/gguf.h:13-25): sizes of the scalar ones, 8 = string, 9 = array
@@ -209,7 +229,7 @@ void skip_gguf_value(Reader &r, uint32_t type, uint32_t *u32_out = nullptr)
     if (type == 9) {
         const uint32_t et = r.get<uint32_t>();
         const uint64_t n = r.get<uint64_t>();
-        if (et < 13 && scalar[et]) { r.skip((size_t)n * scalar[et]); return; }
+        if (et < 13 && scalar[et]) { if (n > r.size) r.ok = false; else r.skip(n * (uint64_t)scalar[et]); return; }
         for (uint64_t i = 0; i < n && r.ok; i++) skip_gguf_value(r, et);
         return;
     }
@@ -246,13 +266,14 @@ bool open_gguf(const std::string &path, ModelFile *f)
         const uint32_t type = r.get<uint32_t>();
         t.dtype = (type == MF_F32 || type == MF_F16 || type == MF_Q8_0) ? (int)type : -1;
         t.begin = r.get<uint64_t>();
+        if (t.elements() == UINT64_MAX) { r.ok = false; break; }      // dimensions whose product overflows
         t.nbytes = bytes_of(t.dtype, t.elements());
         f->tensors.push_back(t);
     }
     if (!r.ok || alignment == 0) { fprintf(stderr, "[Loader] %s: truncated or malformed GGUF header\n", path.c_str()); f->tensors.clear(); munmap(m.p, m.size); return false; }
     m.data_off = (r.off + alignment - 1) / alignment * alignment;
     for (const TensorInfo &t : f->tensors)
-        if (m.data_off + t.begin + t.nbytes > m.size) {
+        if (!range_inside(m.data_off, t.begin, t.nbytes, m.size)) {
             fprintf(stderr, "[Loader] %s: tensor %s lies outside the file\n", path.c_str(), t.name.c_str());
             f->tensors.clear(); munmap(m.p, m.size);
             return false;

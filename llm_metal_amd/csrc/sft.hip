@@ -83,6 +83,7 @@ struct SFTState {
     MetalBuf *grpo_old_lp, *grpo_advs, *grpo_new_lp;   // host-visible [BN] inputs/outputs of the policy gradient
     float *grpo_old_lp_cpu, *grpo_advs_cpu, *grpo_new_lp_cpu;
     MetalBuf *lora_acc;                  // LoRA gradients summed over the completions of a GRPO group
+    int step_in_flight, step_rejected;   // sft_enqueue_train_step without its sft_finish_train_step yet; ids refused
     std::vector<LayerW> layers_out;      // row-major F16 copies handed out by sft_get_layers
     std::vector<WMat> wmats_out;
     std::vector<MetalBuf *> views_out;
@@ -792,8 +793,26 @@ static void enqueue_step_kernels(SFTState *s, float lr)
     enqueue_update(s);
 }
 
+// The kernels gather embedding rows by token id and read logits[target] without a test of their own, so ids are
+// checked here, on the host, before anything is launched (an int32 id < 0 from a token file arrives as a huge uint32).
+static bool ids_in_vocab(const SFTState *s, const uint32_t *ids, size_t n, const char *what)
+{
+    for (size_t i = 0; i < n; i++)
+        if (ids[i] >= (uint32_t)s->V) {
+            fprintf(stderr, "[FastSFT] %s id %u at position %zu is outside the vocabulary (%d): nothing launched\n", what, ids[i], i, s->V);
+            return false;
+        }
+    return true;
+}
+
 void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uint32_t *target_tokens, float lr)
 {
+    // One step in flight: the pinned token / target / optimiser-parameter buffers are read by the kernels of the
+    // step that was enqueued last, so a second enqueue first waits for that step.
+    if (s->step_in_flight) metal_flush();
+    s->step_rejected = !ids_in_vocab(s, input_tokens, (size_t)s->BN, "token") || !ids_in_vocab(s, target_tokens, (size_t)s->BN, "target");
+    s->step_in_flight = 1;
+    if (s->step_rejected) return;
     memcpy(s->tokens_cpu, input_tokens, (size_t)s->BN * 4);
     memcpy(s->targets_cpu, target_tokens, (size_t)s->BN * 4);
     if (s->R) { s->step_count++; write_hyper(s, lr, s->step_count); }
@@ -803,6 +822,8 @@ void sft_enqueue_train_step(SFTState *s, const uint32_t *input_tokens, const uin
 float sft_finish_train_step(SFTState *s)
 {
     metal_flush();
+    s->step_in_flight = 0;
+    if (s->step_rejected) { s->step_rejected = 0; return NAN; }
     float tot = 0.f;
     for (int i = 0; i < s->BN; i++) tot += s->losses_cpu[i];
     return tot / (float)s->BN;
@@ -1069,6 +1090,10 @@ void grpo_apply_completions(SFTState *s, const GRPOCompletions *c, float lr, flo
     if (s->B != 1) { fprintf(stderr, "[FastGRPO] the state must be built with batch 1\n"); return; }
     const int G = c->group_size, seq_len = s->BN;
     if (G <= 0) return;
+    if (s->step_in_flight) { metal_flush(); s->step_in_flight = 0; }
+    if (!ids_in_vocab(s, c->prompt, (size_t)(c->prompt_len > 0 ? c->prompt_len : 0), "prompt token")) return;
+    for (int i = 0; i < G; i++)
+        if (!ids_in_vocab(s, c->gen_tokens[i], (size_t)(c->gen_lengths[i] > 0 ? c->gen_lengths[i] : 0), "completion token")) return;
     const bool accurate = s->full_param && c->accurate;
     if (accurate) sft_alloc_grad_accum(s);
     if (!s->grpo_old_lp) {

@@ -39,11 +39,15 @@ CASES = [
     # long sequences: 16 key blocks per query block (config 4's 512), and a ragged length beyond 256
     C1.with_(name="seq512", NL=1, seq=512, V=1024),
     C1.with_(name="seq300_hd128", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300),
-    # every product through the LDS-tiled large-M GEMM (F16 tiles; Q8_0 unpacked into LDS with row and column
-    # scales; row counts that are not multiples of the 128-row block)
+    # every product through the LDS-tiled large-M GEMM: F16 tiles; Q8_0 operands dequantised once per product into an
+    # F16 image (what the measured rule does from 1024 rows on); and, in the "_lds" cases, Q8_0 tiles kept quantised and
+    # unpacked into LDS by the kernel itself, with row scales (forward image) and column scales (transposed image).
+    # Row counts that are not multiples of the 128-row block.
     C1.with_(name="big_m_f16", batch=4, seq=64),
     C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
+    C1.with_(name="big_m_q8_lds", NL=1, batch=2, seq=160, weight_format="q8_0"),
+    TINY_GEMMA3.with_(name="gemma_big_m_q8_lds", NL=2, batch=3, seq=100, weight_format="q8_0"),
     # a wide FFN: the GLU kernels split each row into column groups of two (forward) and four (backward) K chunks with
     # a factor each, and 2 * IS is not a whole number of backward groups, so one group straddles the dgate | dup boundary
     C1.with_(name="wide_ffn_groups", NL=1, IS=4224, V=1024, seq=64),
@@ -75,7 +79,7 @@ def test_train_steps_match_oracle(cfg):
     from llm_metal_amd import lib
     # the "big_m" cases pin every product to the LDS-tiled large-M kernel (by itself it is only chosen for
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
-    lib.load().hip_gemm_force_large_m(1 if "big_m" in cfg.name else 0)
+    lib.load().hip_gemm_force_large_m(2 if cfg.name.endswith("_lds") else 1 if "big_m" in cfg.name else 0)
     with SFTState(cfg, model) as st:
         for i, (tok, tgt) in enumerate(batches):
             loss = st.train_step(tok, tgt, lr)
@@ -249,3 +253,30 @@ def test_run_sft_driver_matches_the_library_driven_from_python(tmp_path):
     assert len(got) == 3 and np.allclose(got, losses, atol=6e-5)                 # printed with four decimals
     raw = open(adapter, "rb").read()
     assert np.array_equal(np.frombuffer(raw[12:], np.float32), want)             # the same three updates
+
+
+def test_ids_outside_the_vocabulary_launch_nothing_and_two_enqueues_do_not_race(capfd):
+    """An id >= V (a negative int32 from a token file arrives as a huge uint32) would be an out-of-bounds gather on the
+    device: the step is refused on the host, returns NaN and leaves adapters and step count alone.  A second enqueue
+    before the first step was finished waits for it, so both steps see their own tokens."""
+    cfg = C1
+    model = make_model(cfg, seed=21)
+    tok, tgt = make_batch(cfg, seed=30)
+    tok2, tgt2 = make_batch(cfg, seed=31)
+    with SFTState(cfg, model) as st:
+        bad = tok.copy()
+        bad[5] = cfg.V
+        assert np.isnan(st.train_step(bad, tgt, 1e-4))
+        bad_t = tgt.copy()
+        bad_t[0] = np.uint32(np.int32(-1))
+        assert np.isnan(st.train_step(tok, bad_t, 1e-4))
+        assert st.step_count() == 0 and np.array_equal(st.lora(), model["lora"])
+        assert "outside the vocabulary" in capfd.readouterr().err
+        st.enqueue_train_step(tok, tgt, 1e-4)
+        st.enqueue_train_step(tok2, tgt2, 1e-4)            # waits for the first step before reusing its input buffers
+        loss2 = st.finish_train_step()
+        after2 = st.lora()
+    with SFTState(cfg, model) as st:
+        st.train_step(tok, tgt, 1e-4)
+        assert st.train_step(tok2, tgt2, 1e-4) == loss2
+        assert np.array_equal(st.lora(), after2)

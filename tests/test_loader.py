@@ -137,6 +137,56 @@ def test_unreadable_files_are_refused(L, tmp_path, capfd):
     assert "[Loader]" in capfd.readouterr().err
 
 
+def _safetensors_raw(path, header: str, data: bytes):
+    h = header.encode()
+    path.write_bytes(struct.pack("<Q", len(h)) + h + data)
+
+
+def test_crafted_offsets_and_shapes_are_refused(L, tmp_path, capfd):
+    """Headers whose sums would wrap 64 bits, reversed offsets and dimension products that overflow must be refused at
+    open time: later reads trust the shape."""
+    data = b"\0" * 64
+    big = (1 << 64) - 8
+    cases = {
+        "reversed": '{"t":{"dtype":"F32","shape":[2,2],"data_offsets":[16,0]}}',
+        "wrapping_begin": '{"t":{"dtype":"F32","shape":[2,2],"data_offsets":[%d,%d]}}' % (big, big + 4),
+        "huge_end": '{"t":{"dtype":"F32","shape":[2,2],"data_offsets":[0,%d]}}' % big,
+        "overflowing_shape": '{"t":{"dtype":"F32","shape":[4294967296,4294967296],"data_offsets":[0,0]}}',
+        "shape_mismatch": '{"t":{"dtype":"F32","shape":[4,5],"data_offsets":[0,16]}}',
+    }
+    for name, hdr in cases.items():
+        f = tmp_path / f"{name}.safetensors"
+        _safetensors_raw(f, hdr, data)
+        assert not L.model_file_open(str(f).encode()), name
+    ok = tmp_path / "ok.safetensors"
+    _safetensors_raw(ok, '{"t":{"dtype":"F32","shape":[2,2],"data_offsets":[0,16]}}', data)
+    h = L.model_file_open(str(ok).encode())
+    assert h
+    L.model_file_close(h)
+
+    def gguf(dims, typ, off, n_data=64):
+        info = mf._gg_str("t") + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims) + struct.pack("<IQ", typ, off)
+        head = struct.pack("<IIQQ", 0x46554747, 3, 1, 0) + info
+        head += b"\0" * (-len(head) % 32)
+        return head + b"\0" * n_data
+    bad = {
+        "dims_overflow_to_zero": gguf([1 << 32, 1 << 32], mf.GGML_F32, 0),          # product 2^64 wraps to 0 bytes
+        "dims_overflow_q8": gguf([1 << 40, 1 << 30], mf.GGML_Q8_0, 0),
+        "wrapping_offset": gguf([4, 4], mf.GGML_F32, (1 << 64) - 32),
+        "array_count_overflow": struct.pack("<IIQQ", 0x46554747, 3, 0, 1) + mf._gg_str("k") + struct.pack("<IIQ", 9, 10, (1 << 62) + 1) + b"\0" * 64,
+    }
+    for name, raw in bad.items():
+        f = tmp_path / f"{name}.gguf"
+        f.write_bytes(raw)
+        assert not L.model_file_open(str(f).encode()), name
+    f = tmp_path / "fine.gguf"
+    f.write_bytes(gguf([4, 4], mf.GGML_F32, 0))
+    h = L.model_file_open(str(f).encode())
+    assert h
+    L.model_file_close(h)
+    assert "[Loader]" in capfd.readouterr().err
+
+
 TINY_GEMMA = SFTConfig("tiny_gemma3", GEMMA3, NL=7, D=128, Hq=4, Hkv=1, hd=32, IS=256, V=512, seq=5, tied=True)
 
 
