@@ -54,6 +54,9 @@ void     *metal_buf_ptr(MetalBuf *b);
 void   metal_buf_read(MetalBuf *b, size_t offset, void *dst, size_t n);
 void   metal_buf_write(MetalBuf *b, size_t offset, const void *src, size_t n);
 size_t metal_buf_size(MetalBuf *b);
+/* Extension: the address kernels use for the buffer (device memory, or the device view of pinned host memory once
+ * metal_buf_ptr was called).  For callers that pass plain device pointers to hip_attention_noalloc. */
+void *hip_buf_device_ptr(MetalBuf *b);
 /* Non-owning window [offset, offset+size) of another buffer. */
 MetalBuf *metal_buf_view(MetalBuf *parent, size_t offset, size_t size);
 
@@ -167,6 +170,16 @@ int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double
  * tile height (1, 2; 128 = the large-M kernel) and K split.  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
  * 2 Q8_0 with column scales (transposed image).  Returns average ms per launch. */
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S);
+
+/* metal_enqueue_attention once more, ALLOCATING NOTHING.  No counterpart in the reference: it is for callers that cannot
+ * call hipMalloc -- code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  Plain device
+ * pointers: Q, out [Hq * hd] fp32; caches [Hq / group_ratio, max_seq, hd] fp32; keys 0 .. n_attend - 1 are attended.
+ * Same kernels on the library's stream, results identical to metal_enqueue_attention.  The slice results that contexts
+ * beyond 256 keys need go to a fixed 2 MiB array that each device holds until the process ends, which bounds the call:
+ * Hq <= 64, hd <= 256, group_ratio <= 16, n_attend <= 8192; anything larger returns -1 with a message and launches
+ * nothing (0 otherwise).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU race. */
+int hip_attention_noalloc(const float *Q, const float *Kc, const float *Vc, float *out, int n_attend, int hd, int max_seq,
+                          int Hq, int group_ratio);
 
 /* The same for the matrix-vector kernels of the decode step: rows x cols weight, fmt 0 F16 or 1 Q8_0 (split image),
  * B = 1; cols a multiple of 32.  Returns average ms per launch, -1 for bad arguments. */

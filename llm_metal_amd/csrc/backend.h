@@ -31,6 +31,8 @@ void die(const char *what, hipError_t e, const char *file, int line);
 // within the enqueue that asked for them.
 enum ScratchSlot { SCR_A16 = 0, SCR_SCALE, SCR_PARTIAL, SCR_MISC, SCR_WF16, SCR_COUNT };   // SCR_WF16: F16 image of a Q8_0 weight
 void *scratch(ScratchSlot slot, size_t bytes);
+// infer_kernels.hip: resolves, for the current device, the fixed array behind hip_attention_noalloc (0 / -1)
+int noalloc_setup();
 
 // Device address of a buffer; views resolve through their parent so that they
 // follow it when metal_buf_ptr migrates the allocation to host memory.

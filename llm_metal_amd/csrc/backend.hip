@@ -69,6 +69,7 @@ int fast_metal_init(void)
         return -1;
     }
     g_refcount = 1;
+    lmhip::noalloc_setup();                            // a failure is reported there and again by the entry point that needs it
     return 0;
 }
 
@@ -129,6 +130,8 @@ void metal_buf_free(MetalBuf *b)
 }
 
 size_t metal_buf_size(MetalBuf *b) { return b ? b->size : 0; }
+
+void *hip_buf_device_ptr(MetalBuf *b) { return b ? lmhip::dptr(b) : nullptr; }
 
 void *metal_buf_ptr(MetalBuf *b)
 {

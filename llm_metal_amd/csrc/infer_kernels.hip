@@ -555,6 +555,36 @@ void kv_store(const float *k, const float *v, MetalBuf *kc, MetalBuf *vc, int Hk
     mark_written(kc); mark_written(vc);
 }
 
+// floats of slice results the attention over n_attend keys leaves for its merge kernel: per (query head, slice) hd sums and
+// (max, sum of exponentials); none for a single slice
+size_t attention_partial_floats(int Hq, int hd, int n_attend)
+{
+    const int nsplit = (n_attend + SL - 1) / SL;
+    return nsplit > 1 ? (size_t)Hq * nsplit * (hd + 2) : 0;
+}
+
+// The launches of one attention over device pointers whose shapes the caller has checked.  `partials` holds
+// attention_partial_floats(...) floats (unused when that is 0).
+void attention_launch(const float *Q, const float *Kc, const float *Vc, float *out, float *partials, int n_attend, int hd, int max_seq,
+                      int Hq, int G, const HeadPost *hp)
+{
+    const int nsplit = (n_attend + SL - 1) / SL;
+    // short contexts are bound by latency: one query head per workgroup; long ones by cache bytes: the whole group
+    const int gpw = n_attend <= 128 ? 1 : G;
+    const size_t lds = ((size_t)gpw * hd + (size_t)gpw * SL + 2 * gpw + 4 * 1024) * 4;
+    float *po = nsplit > 1 ? partials : nullptr, *pml = nsplit > 1 ? partials + (size_t)Hq * nsplit * hd : nullptr;
+    const float scale = 1.0f / sqrtf((float)hd);
+    const bool vec4 = hd % 4 == 0 && (((uintptr_t)Vc) & 15) == 0;
+    const dim3 grid(Hq / gpw, nsplit);
+    const HeadPost none{};
+#define ATTN_LAUNCH(V_, F_) LAUNCH((k_attn_decode<V_, F_>), grid, dim3(TB), lds, Q, Kc, Vc, out, po, pml, \
+                                   n_attend, hd, max_seq, G, gpw, scale, nsplit, F_ ? *hp : none)
+    if (hp) { if (vec4) ATTN_LAUNCH(4, true); else ATTN_LAUNCH(1, true); }
+    else { if (vec4) ATTN_LAUNCH(4, false); else ATTN_LAUNCH(1, false); }
+#undef ATTN_LAUNCH
+    if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq), dim3(TB), 0, po, pml, out, hd, nsplit);
+}
+
 void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_attend, int hd, int max_seq, int Hq, int G, const char *fn,
                const HeadPost *hp = nullptr)
 {
@@ -565,29 +595,47 @@ void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_att
     REQUIRE_BYTES(Vc, (size_t)Hkv * max_seq * hd * 4, fn);
     if (n_attend > max_seq) { fprintf(stderr, "[fast_hip] %s: n_attend %d exceeds the cache (%d); launch skipped\n", fn, n_attend, max_seq); return; }
     if (hd > 256 || G > 16) { fprintf(stderr, "[fast_hip] %s: head_dim %d / group ratio %d not supported (<= 256 / <= 16); launch skipped\n", fn, hd, G); return; }
-    const int nsplit = (n_attend + SL - 1) / SL;
-    // short contexts are bound by latency: one query head per workgroup; long ones by cache bytes: the whole group
-    const int gpw = n_attend <= 128 ? 1 : G;
-    const size_t lds = ((size_t)gpw * hd + (size_t)gpw * SL + 2 * gpw + 4 * 1024) * 4;
-    float *po = nullptr, *pml = nullptr;
-    if (nsplit > 1) {
-        const size_t o_bytes = (size_t)Hq * nsplit * hd * 4;
-        po = (float *)scratch(SCR_MISC, o_bytes + (size_t)Hq * nsplit * 2 * 4);
-        pml = po + (size_t)Hq * nsplit * hd;
-    }
-    const float scale = 1.0f / sqrtf((float)hd);
-    const bool vec4 = hd % 4 == 0 && (((uintptr_t)dptr(Vc)) & 15) == 0;
-    const dim3 grid(Hq / gpw, nsplit);
-    const HeadPost none{};
-#define ATTN_LAUNCH(V_, F_) LAUNCH((k_attn_decode<V_, F_>), grid, dim3(TB), lds, Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, po, pml, \
-                                   n_attend, hd, max_seq, G, gpw, scale, nsplit, F_ ? *hp : none)
-    if (hp) { if (vec4) ATTN_LAUNCH(4, true); else ATTN_LAUNCH(1, true); }
-    else { if (vec4) ATTN_LAUNCH(4, false); else ATTN_LAUNCH(1, false); }
-#undef ATTN_LAUNCH
-    if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq), dim3(TB), 0, po, pml, out, hd, nsplit);
+    const size_t pf = attention_partial_floats(Hq, hd, n_attend);
+    float *partials = pf ? (float *)scratch(SCR_MISC, pf * sizeof(float)) : nullptr;
+    attention_launch(Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, partials, n_attend, hd, max_seq, Hq, G, hp);
 }
 
+// ---- the attention once more for callers that cannot allocate ------------------------------------------------
+// Slice results go to a fixed array in the code object's own data segment instead of the grow-only arena.  Each
+// device the library runs on holds its own copy of the array at its own address until the process ends.  In host
+// code the array's NAME is a stand-in, not a device address: only the pointer hipGetSymbolAddress returns for the
+// current device may be handed to a kernel.
+constexpr int NA_MAX_HQ = 64, NA_MAX_HD = 256, NA_MAX_KEYS = 8192, NA_MAX_DEVICES = 16;
+constexpr size_t NA_FLOATS = (size_t)NA_MAX_HQ * (NA_MAX_KEYS / SL) * (NA_MAX_HD + 2);      // 2.0 MiB
+static __device__ __align__(256) float attn_partials_static[NA_FLOATS];
+float *g_na_ptr[NA_MAX_DEVICES];                           // per device; null until noalloc_setup ran with that device current
+
 }  // namespace
+
+namespace lmhip {
+
+// Resolves the fixed partials array on the current device (once per device).  Called from fast_metal_init and, for a
+// device that became current later, from the first no-allocation call on it.  0, or -1 with a message.
+int noalloc_setup()
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= NA_MAX_DEVICES) {
+        fprintf(stderr, "[fast_hip] noalloc_setup: no current device below %d (%s)\n", NA_MAX_DEVICES, hipGetErrorString(e));
+        return -1;
+    }
+    if (g_na_ptr[dev]) return 0;
+    float *p = nullptr;
+    e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(attn_partials_static));
+    if (e != hipSuccess || !p) {
+        fprintf(stderr, "[fast_hip] noalloc_setup: hipGetSymbolAddress failed on device %d (%s)\n", dev, hipGetErrorString(e));
+        return -1;
+    }
+    g_na_ptr[dev] = p;
+    return 0;
+}
+
+}  // namespace lmhip
 
 extern "C" {
 
@@ -707,6 +755,33 @@ void metal_enqueue_attention_off(MetalBuf *Q, size_t q_off, MetalBuf *Kc, MetalB
     if (!qp || !op) return;
     attention(qp, Kc, Vc, op, n_attend, hd, max_seq, Hq, group_ratio, "attention");
     mark_written(out);
+}
+
+// metal_enqueue_attention over plain device pointers, allocating nothing.  Q, out: [Hq * hd] fp32; caches
+// [Hq / group_ratio, max_seq, hd] fp32; attends keys 0 .. n_attend - 1.  Same kernels and the same results as
+// metal_enqueue_attention; the slice results of contexts beyond 256 keys go to the fixed per-device array above, which
+// every call on a device shares and which keeps the last call's contents (every element a call reads it has written
+// first, so nothing needs clearing).  Returns 0, or -1 with a message when a limit is exceeded (nothing launched).
+int hip_attention_noalloc(const float *Q, const float *Kc, const float *Vc, float *out, int n_attend, int hd, int max_seq,
+                          int Hq, int group_ratio)
+{
+    if (!initialized()) { fprintf(stderr, "[fast_hip] attention_noalloc before fast_metal_init\n"); return -1; }
+    if (!Q || !Kc || !Vc || !out || Hq <= 0 || hd <= 0 || n_attend <= 0 || group_ratio <= 0 || Hq % group_ratio || n_attend > max_seq) {
+        fprintf(stderr, "[fast_hip] attention_noalloc: bad arguments (Hq %d, group ratio %d, head_dim %d, n_attend %d, max_seq %d)\n",
+                Hq, group_ratio, hd, n_attend, max_seq);
+        return -1;
+    }
+    if (Hq > NA_MAX_HQ || hd > NA_MAX_HD || group_ratio > 16 || n_attend > NA_MAX_KEYS) {
+        fprintf(stderr, "[fast_hip] attention_noalloc: at most %d query heads, head_dim %d, group ratio 16 and %d keys (got %d, %d, %d, %d)\n",
+                NA_MAX_HQ, NA_MAX_HD, NA_MAX_KEYS, Hq, hd, group_ratio, n_attend);
+        return -1;
+    }
+    if (attention_partial_floats(Hq, hd, n_attend) > NA_FLOATS) return -1;      // cannot happen within the limits above
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NA_MAX_DEVICES) return -1;
+    if (!g_na_ptr[dev] && noalloc_setup() != 0) return -1;
+    attention_launch(Q, Kc, Vc, out, g_na_ptr[dev], n_attend, hd, max_seq, Hq, group_ratio, nullptr);
+    return 0;
 }
 
 // Microbenchmark of the matrix-vector kernels alone: average ms per launch over `iters` launches that rotate through

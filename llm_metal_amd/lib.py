@@ -81,7 +81,8 @@ def load():
         "fast_metal_init": (i, []), "fast_metal_shutdown": (None, []), "metal_flush": (None, []),
         "metal_buf_create": (vp, [sz]), "metal_buf_from_data": (vp, [vp, sz]), "metal_buf_free": (None, [vp]),
         "metal_buf_ptr": (vp, [vp]), "metal_buf_read": (None, [vp, sz, vp, sz]), "metal_buf_write": (None, [vp, sz, vp, sz]),
-        "metal_buf_size": (sz, [vp]), "metal_buf_view": (vp, [vp, sz, sz]),
+        "metal_buf_size": (sz, [vp]), "metal_buf_view": (vp, [vp, sz, sz]), "hip_buf_device_ptr": (vp, [vp]),
+        "hip_attention_noalloc": (i, [vp, vp, vp, vp, i, i, i, i, i]),
         "metal_enqueue_rms_norm_batched": (None, [vp, vp, vp, i, f, i]),
         "metal_enqueue_silu_mul": (None, [vp, vp, i]), "metal_enqueue_gelu_mul": (None, [vp, vp, i]),
         "metal_enqueue_residual_add": (None, [vp, vp, i]),
