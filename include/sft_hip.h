@@ -130,6 +130,12 @@ float *sft_get_lora_grad_ptr(SFTState *state, int idx, int *out_size);
 void sft_set_lora_grad(SFTState *state, int idx, const float *data, int size);
 MetalBuf *sft_get_lora_weight_buf(SFTState *state, int layer, int sub);
 float sft_get_lora_scaling(SFTState *state);
+/* Extension: sliding-window attention.  window > 0: on the local layers query i attends keys i - window + 1 .. i
+ * (forward and, through the saved probabilities, backward); 0 (the state's default) = every earlier key on every
+ * layer, which is what the reference computes: it stores Gemma3's window (src/nn/gemma3.c:20, 99) and never reads it.
+ * layer_is_local: [n_layers] flags, or NULL for Gemma3's pattern (src/nn/gemma3.c:49-57: all layers but L % 6 == 0;
+ * every layer of a Qwen3 model). */
+void sft_set_sliding_window(SFTState *state, int window, const int *layer_is_local);
 ModelType sft_get_model_type(SFTState *state);
 int sft_get_n_q_heads(SFTState *state);
 int sft_get_n_kv_heads(SFTState *state);

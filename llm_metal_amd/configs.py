@@ -28,6 +28,7 @@ class SFTConfig:
     local_rope_theta: float = 1e4   # Gemma3 local layers (src/nn/fast_sft.c:310-313)
     tied: bool = False       # lm_head shares the embedding table
     weight_format: str = "f16"      # "f16" | "q8_0"
+    window: int = 0          # sliding-window attention on the local layers (0 = off: the reference never applies it)
 
     @property
     def BN(self):
@@ -46,6 +47,10 @@ class SFTConfig:
         if self.model_type == GEMMA3:
             return [self.rope_theta if (L % 6) == 0 else self.local_rope_theta for L in range(self.NL)]
         return [self.rope_theta] * self.NL
+
+    def local_layers(self):
+        """Layers the sliding window applies to: Gemma3's pattern (src/nn/gemma3.c:49-57), every layer otherwise."""
+        return [(L % 6) != 0 if self.model_type == GEMMA3 else True for L in range(self.NL)]
 
     @property
     def lora_layer_size(self):

@@ -203,6 +203,7 @@ struct AttnTileArgs {
     float *out32;                 // dQ: dq [rows][Hq*hd]
     half_t *out16;                // forward: tiled [rows, Hq*hd]
     WeightPrefetch pf;            // weights of the product that follows: fetched by the grid slices z >= batch
+    int window;                   // forward: > 0 masks keys older than i - window + 1 (the saved zeros carry it into the backward)
 };
 
 // Row step: eight threads per row, thread `part` owns the keys 32 m + 4 part + (0..3) for m < M32 and keeps them in
@@ -247,6 +248,7 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
         } else load_probs<M32>(p, a, N, i0, b, h, tid);
     }
     float red = BWD ? 0.f : -1e30f;
+    const int lo = (!BWD && a.window > 0 && i >= a.window) ? i - a.window + 1 : 0;      // first key row i sees
 #pragma unroll
     for (int m = 0; m < M32; m++) {
         const int j = 32 * m + 4 * part;
@@ -257,7 +259,7 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
             red += pv.x * e[0] + pv.y * e[1] + pv.z * e[2] + pv.w * e[3];
         } else {
 #pragma unroll
-            for (int c = 0; c < 4; c++) { e[c] = (j + c <= i && j + c < nk) ? e[c] * a.scale : -1e30f; red = fmaxf(red, e[c]); }
+            for (int c = 0; c < 4; c++) { e[c] = (j + c <= i && j + c < nk && j + c >= lo) ? e[c] * a.scale : -1e30f; red = fmaxf(red, e[c]); }
         }
     }
     if (BWD) { red += __shfl_xor(red, 1, WAVE); red += __shfl_xor(red, 2, WAVE); red += __shfl_xor(red, 4, WAVE); }
@@ -270,7 +272,7 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
             const int j = 32 * m + 4 * part;
             float *e = &v[m].x;
 #pragma unroll
-            for (int c = 0; c < 4; c++) { e[c] = (j + c <= i && j + c < nk) ? expf(e[c] - red) : 0.f; sum += e[c]; }
+            for (int c = 0; c < 4; c++) { e[c] = (j + c <= i && j + c < nk && j + c >= lo) ? expf(e[c] - red) : 0.f; sum += e[c]; }
         }
         sum += __shfl_xor(sum, 1, WAVE); sum += __shfl_xor(sum, 2, WAVE); sum += __shfl_xor(sum, 4, WAVE);
         inv = 1.0f / sum;
@@ -542,7 +544,7 @@ void launch_attn_fwd_mfma(const AttnFwdArgs &f)
     a.A = f.q; a.BT = f.kT; a.C = f.v;
     a.Hq = f.Hq; a.Hkv = f.Hkv; a.hd = f.hd; a.seq = f.seq; a.batch = f.batch; a.scale = f.scale;
     a.probs = f.probs; a.out16 = f.out16;
-    a.pf = f.pf;
+    a.pf = f.pf; a.window = f.window;
     launch_tile<0>(a);
 }
 

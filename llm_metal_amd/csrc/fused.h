@@ -85,6 +85,7 @@ struct AttnFwdArgs {
     half_t *out16;                // tiled [rows, Hq*hd], unit scale
     const float *kT;              // k transposed per head [batch][Hkv][hd/4][attn_ldt(seq)][4] (matrix-core path only)
     WeightPrefetch pf;            // matrix-core path: weights of the product that follows
+    int window;                   // > 0: query i sees keys i - window + 1 .. i only (sliding window); 0: all keys up to i
 };
 void launch_attn_fwd(const AttnFwdArgs &a);
 

@@ -287,8 +287,9 @@ __global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
     const float *q = a.q + (r0 + i) * qd + h * hd;
     for (int d = lane; d < hd; d += 64) qs[d] = q[d];
     __syncthreads();
+    const int lo = (a.window > 0 && i >= a.window) ? i - a.window + 1 : 0;      // first key the query sees
     float mx = -1e30f;
-    for (int j = lane; j <= i; j += 64) {
+    for (int j = lo + lane; j <= i; j += 64) {
         const float4 *kr = reinterpret_cast<const float4 *>(a.k + (r0 + j) * kd + hk * hd);
         float dot = 0.f;
 #pragma unroll 8
@@ -302,12 +303,12 @@ __global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
     }
     mx = wave_max(mx);
     float sum = 0.f;
-    for (int j = lane; j <= i; j += 64) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
+    for (int j = lo + lane; j <= i; j += 64) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
     sum = wave_sum(sum);
     const float inv = 1.0f / sum;
     float *pr = a.probs + (((size_t)b * a.Hq + h) * N + i) * N;
     for (int j = lane; j < N; j += 64) {
-        const float p = (j <= i) ? sc[j] * inv : 0.f;
+        const float p = (j >= lo && j <= i) ? sc[j] * inv : 0.f;
         sc[j] = p;
         pr[j] = p;
     }
@@ -316,7 +317,7 @@ __global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
     for (int d = lane; d < hd; d += 64) {
         float acc = 0.f;
 #pragma unroll 8
-        for (int j = 0; j <= i; j++) acc += sc[j] * a.v[(r0 + j) * kd + hk * hd + d];
+        for (int j = lo; j <= i; j++) acc += sc[j] * a.v[(r0 + j) * kd + hk * hd + d];
         a.out16[tiled_index((int)(r0 + i), h * hd + d, Kb)] = f2h(acc);
     }
     if (h == a.Hq - 1)                                    // zero the K padding of this row once

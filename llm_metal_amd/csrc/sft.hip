@@ -29,6 +29,8 @@ struct SFTState {
     ModelType model_type;
     int step_count, weight_format;
     std::vector<float> rope_thetas;
+    int window;                          // sliding-window attention (sft_set_sliding_window): 0 = off, the reference's behaviour
+    std::vector<int> layer_local;        // layers the window applies to
     MetalBuf *rope_tabs;                 // one (cos, sin) table [seq][hd/2] per distinct theta
     std::vector<int> rope_slot;          // layer -> table index
 
@@ -300,6 +302,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
         aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16; aa.kT = qa.kT;
+        aa.window = (s->window > 0 && s->layer_local[L]) ? s->window : 0;
         if (attn_mfma_supported(s->hd, s->N)) {
             aa.pf = prefetch_for(s, wop(s, W_O, L, false), D, qd, 256, ((s->N + 31) / 32) * s->Hq);
             launch_attn_fwd_mfma(aa);
@@ -558,6 +561,8 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->full_param = lora_rank == 0;                        // sft_state_create_full, src/nn/fast_sft.c:402-410
     s->token_emb_host = m->token_emb;
     s->rope_thetas.assign(m->rope_thetas, m->rope_thetas + s->NL);
+    s->window = 0;
+    s->layer_local.assign(s->NL, 0);
     const int D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R, NL = s->NL, BN = s->BN, V = s->V;
     if ((s->hd & 3) || (s->Hq % s->Hkv) || (D & 3) || (IS & 3) || (V & 3) || (lora_rank & 1) || lora_rank > 16 || (!weight_format && ((D & 31) || (IS & 31) || (qd & 31)))) {
         fprintf(stderr, "[FastSFT] unsupported dims: d_model, FFN width, vocab, head_dim must be multiples of 4, Hq of Hkv, rank even and <= 16 "
@@ -993,6 +998,17 @@ MetalBuf *sft_get_lora_weight_buf(SFTState *s, int layer, int sub)
     return i < s->lora_views.size() ? s->lora_views[i] : nullptr;
 }
 float sft_get_lora_scaling(SFTState *s) { return s->lora_scaling; }
+
+// Sliding-window attention on the local layers.  The reference stores Gemma3's window (src/nn/gemma3.c:20, 99) and
+// never applies it: its attention kernels see every earlier key on every layer (shaders/q8_kernels.metal:769-855), which
+// is what a state does until this is called.  layer_is_local: [n_layers] flags, or NULL for the pattern the reference
+// marks (src/nn/gemma3.c:49-57: every layer but those with L % 6 == 0 on Gemma3; every layer on Qwen3).
+void sft_set_sliding_window(SFTState *s, int window, const int *layer_is_local)
+{
+    s->window = window > 0 ? window : 0;
+    for (int L = 0; L < s->NL; L++)
+        s->layer_local[L] = layer_is_local ? (layer_is_local[L] != 0) : (s->model_type == MODEL_GEMMA3 ? (L % 6) != 0 : 1);
+}
 ModelType sft_get_model_type(SFTState *s) { return s->model_type; }
 int sft_get_n_q_heads(SFTState *s) { return s->Hq; }
 int sft_get_n_kv_heads(SFTState *s) { return s->Hkv; }

@@ -132,7 +132,7 @@ def load():
         "sft_get_emb_scale": (f, [vp]), "sft_get_step_count": (i, [vp]), "sft_set_step_count": (None, [vp, i]),
         "sft_get_n_lora_grad_bufs": (i, [vp]), "sft_get_lora_grad_ptr": (vp, [vp, i, C.POINTER(i)]),
         "sft_set_lora_grad": (None, [vp, i, vp, i]), "sft_get_lora_weight_buf": (vp, [vp, i, i]),
-        "sft_get_lora_scaling": (f, [vp]), "sft_get_model_type": (i, [vp]), "sft_get_n_q_heads": (i, [vp]),
+        "sft_get_lora_scaling": (f, [vp]), "sft_set_sliding_window": (None, [vp, i, vp]), "sft_get_model_type": (i, [vp]), "sft_get_n_q_heads": (i, [vp]),
         "sft_get_n_kv_heads": (i, [vp]), "sft_get_head_dim": (i, [vp]), "sft_get_intermediate_size": (i, [vp]),
         "sft_get_rope_thetas": (vp, [vp]), "sft_is_full_param": (i, [vp]), "sft_save_lora": (None, [vp, C.c_char_p]), "sft_load_lora": (i, [vp, C.c_char_p]),
         "sft_lora_numel": (sz, [vp]), "sft_copy_lora": (None, [vp, vp]), "sft_copy_lora_grads": (None, [vp, vp]),

@@ -118,6 +118,8 @@ class SFTState:
                                                   1 if c.weight_format == "f16" else 0)
         if not self.h:
             raise RuntimeError("sft_state_create_from_ref failed (no gfx950 device or unsupported dims)")
+        if c.window:
+            self.L.sft_set_sliding_window(self.h, c.window, None)
 
     def train_step(self, tok, tgt, lr):
         tok = np.ascontiguousarray(tok, dtype=np.uint32)

@@ -25,7 +25,7 @@ class OrCfg(C.Structure):
     _fields_ = [("model_type", C.c_int), ("NL", C.c_int), ("D", C.c_int), ("Hq", C.c_int),
                 ("Hkv", C.c_int), ("hd", C.c_int), ("IS", C.c_int), ("V", C.c_int),
                 ("batch", C.c_int), ("seq", C.c_int), ("R", C.c_int),
-                ("lora_scaling", C.c_float), ("eps", C.c_float), ("emb_scale", C.c_float)]
+                ("lora_scaling", C.c_float), ("eps", C.c_float), ("emb_scale", C.c_float), ("window", C.c_int)]
 
 
 _PP = C.POINTER(C.POINTER(C.c_float))
@@ -130,7 +130,7 @@ def weights_as_used(model, fmt="f16"):
 
 def _cfg(c):
     return OrCfg(c.model_type, c.NL, c.D, c.Hq, c.Hkv, c.hd, c.IS, c.V, c.batch, c.seq, c.R,
-                 c.lora_scaling if c.R else 0.0, c.eps, c.emb_scale)
+                 c.lora_scaling if c.R else 0.0, c.eps, c.emb_scale, getattr(c, "window", 0))
 
 
 class _Packed:

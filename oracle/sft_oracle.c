@@ -339,15 +339,29 @@ OR_API void or_rope_train_bwd(real *q, real *k, int Hq, int Hkv, int hd, int N, 
  * sum (the reference's tree reduction leaves lanes out when the group size is
  * not a power of two; for power-of-two sizes both give the same sum up to
  * fp32 rounding order). */
+OR_API void or_attn_train_fwd_window(const real *Q, const real *K, const real *V, real *out, real *probs,
+                                     int H, int N, int D, float scale, int window);
+
 OR_API void or_attn_train_fwd(const real *Q, const real *K, const real *V, real *out, real *probs,
                               int H, int N, int D, float scale)
+{
+    or_attn_train_fwd_window(Q, K, V, out, probs, H, N, D, scale, 0);
+}
+
+/* The same with a sliding window: query i sees keys max(0, i - window + 1) .. i; window <= 0: every key up to i, which
+ * is all the reference's kernel does (it has no window argument; Gemma3's sliding_window is stored by
+ * src/nn/gemma3.c:20,99 and never read).  The saved probabilities are zero outside the window, so the backward
+ * kernels, which weigh every key by them, need no window of their own. */
+OR_API void or_attn_train_fwd_window(const real *Q, const real *K, const real *V, real *out, real *probs,
+                                     int H, int N, int D, float scale, int window)
 {
     real *s = (real *)malloc(sizeof(real) * N);
     for (int h = 0; h < H; h++)
         for (int i = 0; i < N; i++) {
             const real *q = Q + ((size_t)h * N + i) * D;
             real mx = (real)-1e30;
-            for (int j = 0; j <= i; j++) {
+            const int lo = (window > 0 && i >= window) ? i - window + 1 : 0;
+            for (int j = lo; j <= i; j++) {
                 const real *k = K + ((size_t)h * N + j) * D;
                 real dot = 0;
                 for (int d = 0; d < D; d++) dot += q[d] * k[d];
@@ -355,13 +369,13 @@ OR_API void or_attn_train_fwd(const real *Q, const real *K, const real *V, real 
                 if (s[j] > mx) mx = s[j];
             }
             real sum = 0;
-            for (int j = 0; j <= i; j++) { s[j] = R_EXP(s[j] - mx); sum += s[j]; }
+            for (int j = lo; j <= i; j++) { s[j] = R_EXP(s[j] - mx); sum += s[j]; }
             real inv = (real)1 / sum;
             real *pr = probs + ((size_t)h * N + i) * N;
-            for (int j = 0; j < N; j++) pr[j] = (j <= i) ? s[j] * inv : (real)0;
+            for (int j = 0; j < N; j++) pr[j] = (j >= lo && j <= i) ? s[j] * inv : (real)0;
             real *o = out + ((size_t)h * N + i) * D;
             for (int d = 0; d < D; d++) o[d] = 0;
-            for (int j = 0; j <= i; j++) {
+            for (int j = lo; j <= i; j++) {
                 const real *v = V + ((size_t)h * N + j) * D;
                 for (int d = 0; d < D; d++) o[d] += pr[j] * v[d];
             }
@@ -718,6 +732,7 @@ typedef struct {
     float lora_scaling;      /* alpha / R */
     float eps;               /* RMSNorm epsilon, 1e-6 (src/nn/fast_sft.c:190) */
     float emb_scale;         /* 1 for Qwen3, sqrtf(D) for Gemma3 (src/nn/fast_sft.c:302) */
+    int window;              /* sliding-window attention on the local layers; 0 = none, the reference's behaviour */
 } OrCfg;
 
 typedef struct {
@@ -840,8 +855,10 @@ static void forward(OrRun *r, const OrWeights *w, const real *lora, real *x)
             memcpy(s->q_fin + ro * qd, qt, sizeof(real) * N * qd);
             or_repeat_kv(kt, s->k_exp + ro * qd, Hkv, N, hd, ratio);
             or_repeat_kv(vt, s->v_exp + ro * qd, Hkv, N, hd, ratio);
-            or_attn_train_fwd(qt, s->k_exp + ro * qd, s->v_exp + ro * qd, ao,
-                              s->probs + (size_t)b * Hq * N * N, Hq, N, hd, attn_scale);
+            /* local layers: Gemma3's pattern (src/nn/gemma3.c:49-57), every layer of other models */
+            const int local = c->window > 0 && (c->model_type == 1 ? (L % 6) != 0 : 1);
+            or_attn_train_fwd_window(qt, s->k_exp + ro * qd, s->v_exp + ro * qd, ao,
+                                     s->probs + (size_t)b * Hq * N * N, Hq, N, hd, attn_scale, local ? c->window : 0);
             or_transpose_heads_rev(ao, af + ro * qd, N, Hq, hd);
         }
 

@@ -52,6 +52,12 @@ CASES = [
     # a factor each, and 2 * IS is not a whole number of backward groups, so one group straddles the dgate | dup boundary
     C1.with_(name="wide_ffn_groups", NL=1, IS=4224, V=1024, seq=64),
     TINY_GEMMA3.with_(name="gemma_wide_ffn", NL=2, IS=2112, seq=64),
+    # sliding-window attention (off by default, as in the reference): windows shorter than the sequence on the matrix-core
+    # kernels (Qwen3: every layer; Gemma3: local layers only, global ones untouched) and on the wave-per-query kernels
+    C1.with_(name="window24", window=24),
+    TINY_GEMMA3.with_(name="gemma_window8", window=8),
+    C1.with_(name="window_seq300", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
+    C1.with_(name="window7_small_heads", NL=1, D=64, Hq=4, Hkv=2, hd=16, IS=96, V=512, seq=40, window=7),
     # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
     TINY_GEMMA3.with_(name="gemma_many_rows", NL=2, batch=4, seq=128),
 ]

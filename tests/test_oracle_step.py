@@ -25,7 +25,13 @@ def _rel(a, b):
     return float(np.linalg.norm(np.asarray(a, dtype=np.float64) - b) / (np.linalg.norm(b) + 1e-300))
 
 
-@pytest.mark.parametrize("cfg", [SMALL_Q, SMALL_G], ids=lambda c: c.name)
+# sliding-window attention (an option the reference stores and never applies): the torch model masks with
+# F.scaled_dot_product_attention(attn_mask=...), windows shorter than the sequence, local and global Gemma3 layers
+WINDOW_Q = SMALL_Q.with_(name="small_q_window5", window=5)
+WINDOW_G = SMALL_G.with_(name="small_g_window4", window=4)
+
+
+@pytest.mark.parametrize("cfg", [SMALL_Q, SMALL_G, WINDOW_Q, WINDOW_G], ids=lambda c: c.name)
 def test_f64_step_matches_torch_autograd_and_adamw(cfg):
     model = make_model(cfg, seed=3, gamma_jitter=0.1)
     used = oracle.weights_as_used(model)
@@ -133,3 +139,20 @@ def test_c1_f32_step_runs_in_seconds():
     out = oracle.sft_train_step(C1, used, lora, m, v, 0, tok, tgt, 1e-4)
     assert abs(out["loss"] - np.log(C1.V)) < 0.2      # random init: loss ~ ln V
     assert out["step"] == 1 and np.isfinite(out["grad"]).all()
+
+
+def test_window_changes_the_result_and_a_long_window_does_not():
+    """The option is live (a short window moves loss and gradients) and a window that covers the whole sequence is the
+    unwindowed step bit for bit."""
+    cfg = SMALL_Q
+    model = make_model(cfg, seed=8, gamma_jitter=0.1)
+    used = oracle.weights_as_used(model)
+    tok, tgt = make_batch(cfg, seed=9)
+
+    def run(c):
+        lora = model["lora"].copy()
+        z = np.zeros_like(lora)
+        return oracle.sft_train_step(c, used, lora, z, z.copy(), 0, tok, tgt, 1e-3, do_update=False)
+    base, wide, short = run(cfg), run(cfg.with_(window=cfg.seq)), run(cfg.with_(window=3))
+    assert base["loss"] == wide["loss"] and np.array_equal(base["grad"], wide["grad"])
+    assert abs(short["loss"] - base["loss"]) > 1e-6 and _rel(short["grad"], base["grad"]) > 1e-3

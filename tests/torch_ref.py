@@ -80,7 +80,12 @@ def forward_loss(c, used, lora_flat, tok, tgt, x_embed=None, params=None, qkv_lr
         v = v.reshape(B, N, Hkv, hd).transpose(1, 2)
         q = rope_hf(F.rms_norm(q, (hd,), g("g_q"), c.eps), thetas[L])
         k = rope_hf(F.rms_norm(k, (hd,), g("g_k"), c.eps), thetas[L])
-        o = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        if getattr(c, "window", 0) and c.local_layers()[L]:
+            # sliding window as a boolean mask for the library routine: query i attends keys i - window + 1 .. i
+            i, j = torch.arange(N)[:, None], torch.arange(N)[None, :]
+            o = F.scaled_dot_product_attention(q, k, v, attn_mask=(j <= i) & (i - j < c.window), enable_gqa=True)
+        else:
+            o = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
         o = o.transpose(1, 2).reshape(B, N, Hq * hd) @ g("wo").T
         if c.model_type == GEMMA3:
             x = x + F.rms_norm(o, (D,), g("g_post_attn"), c.eps)
