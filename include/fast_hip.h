@@ -159,6 +159,10 @@ void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
  * F16 image made once per product); 2: always the large-M kernel with Q8_0 tiles kept quantised and unpacked into LDS
  * by the kernel itself; -1: never (always the weight-streaming kernel). */
 void hip_gemm_force_large_m(int policy);
+/* K chunks of the large-M kernel on F16 tiles (each chunk writes a plane, the consumer adds them): 1 = by the measured
+ * rule (three chunks when the 128 x 256 output blocks leave a third of the CUs idle and K >= 4096), 0 = never, n > 1 =
+ * always n. */
+void hip_gemm_large_m_split(int mode);
 /* Timing aid for benchmarks: when enabled, every GEMM launch is bracketed by HIP events on the
  * library's stream.  hip_gemm_profile_read (after metal_flush) returns the number of launches recorded
  * since the last enable and adds up their durations (ms) and weight bytes; _read2 also their flops. */
@@ -167,7 +171,7 @@ int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
 int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double *total_flops);
 /* Microbenchmark of the GEMM alone at one shape (M rows, N x K weight) on synthetic operands,
  * rotating through > 1 GB of distinct weight images.  nb / S = 0: planner's choice, else forced
- * tile height (1, 2; 128 = the large-M kernel) and K split.  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
+ * tile height (1, 2; 128 = the large-M kernel) and K split (for the large-M kernel: K chunks, F16 tiles only).  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
  * 2 Q8_0 with column scales (transposed image).  Returns average ms per launch. */
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S);
 

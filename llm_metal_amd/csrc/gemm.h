@@ -73,7 +73,13 @@ double weight_stream_bytes(const WeightOp &W, int N, int K);
 // through LDS (gemm_big.hip): the path for M of several hundred rows and more, where the product is MFMA bound.
 // W as plain F16 tiles: itself when F16, else dequantised once into a scratch image that the next call overwrites
 WeightOp f16_image_of(const WeightOp &W, int N, int K);
-void launch_gemm_big(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K);
+// chunks > 1 (F16 tiles only): the K steps are cut into that many chunks, chunk c writing the plane at C + c * plane_stride;
+// big_gemm_chunks: what the measured rule picks for a product
+int big_gemm_chunks(int M, int N, int K, int fmt);
+void set_big_gemm_split(int mode);     // 1 measured rule, 0 never, n > 1 always n chunks
+// Returns the number of planes written (fewer than `chunks` when K has too few steps for that many).
+int launch_gemm_big(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K,
+                    int chunks = 1, size_t plane_stride = 0);
 // true when the large-M kernel is the faster one for this product
 bool use_big_gemm(int M, int N, int K, int fmt);
 // Q8_0 blocks in the reference's row-major layout ([rows][cols/32] blocks of 34 bytes) -> kernel tiles.

@@ -485,6 +485,7 @@ void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, i
 }
 
 void hip_gemm_force_large_m(int policy) { g_big_policy = policy; }
+void hip_gemm_large_m_split(int mode) { set_big_gemm_split(mode); }
 
 void hip_gemm_profile_enable(int on)
 {
@@ -529,7 +530,8 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters
     if (used_S) *used_S = p.S;
     void *A = nullptr, *W = nullptr, *D = nullptr, *P = nullptr, *inv = nullptr;
     const size_t tiles = (size_t)tiled_rb(N) * tiled_kb(K);
-    const size_t ab = tiled_elems(M, K) * 2, wb = wf ? tiles * 2048 : tiles * 4096, db = tiles * 128, pb = (size_t)p.S * M * N * 4;
+    const size_t ab = tiled_elems(M, K) * 2, wb = wf ? tiles * 2048 : tiles * 4096, db = tiles * 128;
+    const size_t pb = (size_t)(nb == 128 ? (S > 0 ? S : 1) : p.S) * M * N * 4;
     // rotate through enough distinct weight images that no launch finds its weights in a cache
     const int nbuf = (int)((size_t)1200 * 1024 * 1024 / wb) + 1;
     HIP_CHECK(hipMalloc(&A, ab)); HIP_CHECK(hipMalloc(&W, wb * nbuf)); HIP_CHECK(hipMalloc(&D, db * nbuf));
@@ -551,7 +553,7 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters
     };
     const bool big = nb == 128;                            // nb = 128 selects the large-M kernel (one launch, 128-row blocks)
     auto run = [&](int i) {
-        if (big) launch_gemm_big((half_t *)A, (float *)inv, op(i), (float *)P, N, M, N, K);
+        if (big) launch_gemm_big((half_t *)A, (float *)inv, op(i), (float *)P, N, M, N, K, S > 0 ? S : 1, (size_t)M * N);
         else launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
     };
     for (int i = 0; i < 3; i++) run(i);

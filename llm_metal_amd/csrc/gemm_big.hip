@@ -21,6 +21,7 @@
 namespace lmhip {
 namespace {
 
+int g_big_split = 1;                  // 1: K chunks by the measured rule (big_gemm_chunks), 0: never, n > 1: always n
 constexpr int WPW = 2;               // weight row blocks each wave fetches per K step: the block is 128 x (WPW * 128)
 constexpr int PF = 3;                // K steps whose operands are in flight in registers ahead of the one being multiplied
 
@@ -261,17 +262,28 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
     const int r = lane & 31, h = lane >> 5;
     const int MT = (g.M + 127) >> 7, NT = (g.N + 128 * WPW - 1) / (128 * WPW);
     const int m_patches = (MT + 7) >> 3;
-    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3, patch = seq >> 5, in_patch = seq & 31;
-    const int mt = (patch % m_patches) * 8 + (in_patch & 7);
-    const int nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
-    if (mt >= MT || nt >= NT) return;
+    int mt, nt, chunk = 0;
+    if (g.S > 1) {
+        // K chunks: the grid is S * MT * NT workgroups, id = (chunk * NT + nt) * MT + mt.  The hardware deals ids to the
+        // XCDs in turn, so (MT a multiple of 8) an XCD takes the row blocks mt = xcd (mod 8) of every column block and
+        // chunk: equal shares, and an activation row block is fetched into one L2 only.
+        const int t = blockIdx.x % (MT * NT);
+        chunk = blockIdx.x / (MT * NT); mt = t % MT; nt = t / MT;
+    } else {
+        const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3, patch = seq >> 5, in_patch = seq & 31;
+        mt = (patch % m_patches) * 8 + (in_patch & 7);
+        nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
+        if (mt >= MT || nt >= NT) return;
+    }
     const int nb0 = nt * 4 * WPW, mb0 = mt * 4;
     const int wm = wave >> 1, wn = wave & 1;
-    const half8 *asrc = g.A + (size_t)min(mb0 + wave, g.Mb - 1) * g.Kb * 256 + lane;
+    const int k_beg = chunk * g.steps_per_chunk, nsteps = min(g.Kb, k_beg + g.steps_per_chunk) - k_beg;
+    const half8 *asrc = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
     const half8 *wsrc[WPW];
 #pragma unroll
     for (int u = 0; u < WPW; u++)
-        wsrc[u] = reinterpret_cast<const half8 *>(g.W.w16) + (size_t)min(nb0 + wave * WPW + u, g.Nb - 1) * g.Kb * 256 + lane;
+        wsrc[u] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + wave * WPW + u, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
+    float *const Cp = g.P + (size_t)chunk * g.plane_stride;
 
     float16v acc[2][NW];
 #pragma unroll
@@ -293,7 +305,7 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
             for (int j = 0; j < 4; j++)
                 __builtin_amdgcn_global_load_lds(wsrc[u] + o + j * 64, (lds_void *)(buf + ((4 + wave * WPW + u) * 4 + j) * 64), 16, 0, 0);
     };
-    const int last = g.Kb - 1;
+    const int last = nsteps - 1;
     // one K step: `cur` holds step kt; `free_buf` held step kt - 1 and takes step kt + 2
     auto step = [&](int kt, half8 (&cur)[BUF], half8 (&free_buf)[BUF]) __attribute__((always_inline)) {
         // lgkmcnt(0): every LDS read this wave issued for step kt - 1 has returned before the barrier lets other waves
@@ -330,14 +342,14 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
     };
     request(lb0, 0);
     request(lb1, min(1, last));
-    const int full = g.Kb / 3 * 3;
+    const int full = nsteps / 3 * 3;
     for (int kt0 = 0; kt0 < full; kt0 += 3) {
         step(kt0, lb0, lb2);
         step(kt0 + 1, lb1, lb0);
         step(kt0 + 2, lb2, lb1);
     }
-    if (full < g.Kb) step(full, lb0, lb2);
-    if (full + 1 < g.Kb) step(full + 1, lb1, lb0);
+    if (full < nsteps) step(full, lb0, lb2);
+    if (full + 1 < nsteps) step(full + 1, lb1, lb0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the repeated requests of the last steps land before the LDS is given back
 
     if (mb0 * 32 + 128 <= g.M && (nb0 + 4 * WPW) * 32 <= g.N) {
@@ -358,7 +370,7 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = (mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                float *row = g.P + (size_t)m * g.ldp + (nb0 + NW * wn) * 32 + r;
+                float *row = Cp + (size_t)m * g.ldp + (nb0 + NW * wn) * 32 + r;
 #pragma unroll
                 for (int k = 0; k < NW; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
             }
@@ -374,16 +386,31 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
 #pragma unroll
             for (int k = 0; k < NW; k++) {
                 const int n = (nb0 + NW * wn + k) * 32 + r;
-                if (n < g.N) g.P[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
+                if (n < g.N) Cp[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
             }
         }
 }
 
 }  // namespace
 
-void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K)
+// How many K chunks the large-M kernel should cut a product with F16 tiles into: three when its 128 x 256 output blocks
+// would leave a third of the CUs or more without work and K is at least 4096, else one.  Measured on MI355X at 2048
+// rows: the products with 2560 output columns (160 blocks for 256 CUs) go from 66 / 140 / 281 / 93 us to 54 / 103 /
+// 199 / 73 us (K = 4096 / 9728 / 19456 / 6176) with three chunks dealt evenly to the XCDs; two chunks change nothing
+// (320 blocks are two rounds again) and every product with K = 2560 loses (13 K steps per workgroup).
+int big_gemm_chunks(int M, int N, int K, int fmt)
 {
-    if (M <= 0 || N <= 0 || K <= 0) return;
+    if (fmt != 0 || g_big_split == 0) return 1;
+    if (g_big_split > 1) return g_big_split;
+    const long blocks = (long)((M + 127) / 128) * ((N + 128 * WPW - 1) / (128 * WPW));
+    const int cus = num_cus() > 0 ? num_cus() : 256;
+    return (blocks * 3 <= cus * 2 && K >= 4096) ? 3 : 1;
+}
+
+int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K,
+                    int chunks, size_t plane_stride)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
     bool ok = ldc >= N && W.fmt >= 0 && W.fmt <= 2;
     if (W.fmt == 0) ok = ok && W.w16;
@@ -392,11 +419,14 @@ void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &
     if (!ok) { fprintf(stderr, "[fast_hip] gemm_big: bad launch M=%d N=%d K=%d ldc=%d fmt=%d\n", M, N, K, ldc, W.fmt); abort(); }
     GemmKArgs g{};
     g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
-    g.P = C; g.ldp = ldc; g.plane_stride = 0;
-    g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = Kb;
+    if (chunks < 1 || (chunks > 1 && W.fmt != 0)) { fprintf(stderr, "[fast_hip] gemm_big: K chunks need F16 tiles\n"); abort(); }
+    g.P = C; g.ldp = ldc; g.plane_stride = plane_stride;
+    g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb;
+    g.steps_per_chunk = (Kb + chunks - 1) / chunks;
+    g.S = (Kb + g.steps_per_chunk - 1) / g.steps_per_chunk;
     const int MT = (M + 127) / 128, NT = (N + 128 * WPW - 1) / (128 * WPW);
     const int m_patches = (MT + 7) / 8, n_patches = ((NT + 7) / 8 + 3) / 4;
-    const dim3 grid(8 * 32 * m_patches * n_patches), block(256);
+    const dim3 grid(W.fmt == 0 && g.S > 1 ? MT * NT * g.S : 8 * 32 * m_patches * n_patches), block(256);
     const size_t lds = (size_t)2 * (4 + 4 * WPW) * 256 * sizeof(half8);
     static bool attr_set = false;
     if (!attr_set) {
@@ -415,6 +445,9 @@ void launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &
         else hipLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), g);
     }
     HIP_CHECK(hipGetLastError());
+    return W.fmt == 0 ? g.S : 1;
 }
+
+void set_big_gemm_split(int mode) { g_big_split = mode; }
 
 }  // namespace lmhip

@@ -172,7 +172,10 @@ size_t max_planes_elems(SFTState *s)
     size_t mx = 0;
     for (const Sh &sh : shapes) {
         GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0);
-        const size_t e = (size_t)p.S * s->BN * sh.N;
+        // whichever kernel the product takes (the choice can be forced at run time): the planes of the streaming kernel, or
+        // up to four K chunks of the large-M one; the LM head writes the logits directly unless the streaming kernel splits K
+        const bool head = sh.N == s->V && sh.K == s->D;
+        const size_t e = (size_t)(head ? (p.S > 1 ? p.S : 0) : std::max(p.S, 4)) * s->BN * sh.N;
         if (e > mx) mx = e;
     }
     return mx;
@@ -225,11 +228,14 @@ WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int th
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr,
             const ScaleGroups *sg = nullptr)
 {
-    if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch, final output
+    if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch; final output, or a few K chunks as planes
         float *C = out ? out : at<float>(s->planes);
-        if (!out && (size_t)s->BN * N > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
-        launch_gemm_big(A, inv, f16_image_of(W, N, K), C, N, s->BN, N, K);
-        return Planes{C, 1, (size_t)s->BN * N, N, nullptr};
+        const WeightOp Wf = f16_image_of(W, N, K);
+        const int chunks = out ? 1 : big_gemm_chunks(s->BN, N, K, Wf.fmt);
+        const size_t stride = (size_t)s->BN * N;
+        if (!out && chunks * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
+        const int planes = launch_gemm_big(A, inv, Wf, C, N, s->BN, N, K, chunks, stride);
+        return Planes{C, planes, stride, N, nullptr};
     }
     GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
     float *P = out ? out : at<float>(s->planes);

@@ -44,6 +44,9 @@ CASES = [
     # unpacked into LDS by the kernel itself, with row scales (forward image) and column scales (transposed image).
     # Row counts that are not multiples of the 128-row block.
     C1.with_(name="big_m_f16", batch=4, seq=64),
+    # ... with the K steps of every product cut into three chunks over the grid (planes added by the consumer), which
+    # the measured rule only does at sizes the oracle cannot follow; K of 4, 12 and 64 steps, 200 ragged rows
+    C1.with_(name="big_m_f16_chunks", batch=5, seq=40),
     C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
     C1.with_(name="big_m_q8_lds", NL=1, batch=2, seq=160, weight_format="q8_0"),
@@ -86,6 +89,7 @@ def test_train_steps_match_oracle(cfg):
     # the "big_m" cases pin every product to the LDS-tiled large-M kernel (by itself it is only chosen for
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
     lib.load().hip_gemm_force_large_m(2 if cfg.name.endswith("_lds") else 1 if "big_m" in cfg.name else 0)
+    lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
     with SFTState(cfg, model) as st:
         for i, (tok, tgt) in enumerate(batches):
             loss = st.train_step(tok, tgt, lr)
@@ -108,6 +112,7 @@ def test_train_steps_match_oracle(cfg):
         assert rel(d_gpu, d_ref) < 0.1
         assert (np.sign(d_gpu) == np.sign(d_ref)).mean() > 0.97
     lib.load().hip_gemm_force_large_m(0)
+    lib.load().hip_gemm_large_m_split(1)
 
 
 def test_q8_tiles_hold_the_dequantised_values_in_both_images():
