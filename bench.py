@@ -119,6 +119,19 @@ def decode_bench(args, cfg, L):
     tms, wb, fl = C.c_double(0), C.c_double(0), C.c_double(0)
     n = L.hip_gemm_profile_read2(C.byref(tms), C.byref(wb), C.byref(fl))
     L.hip_gemm_profile_enable(0)
+    batch = None
+    if args.decode_batch > 1 and f16:
+        # the same prompt decoded in lock step by `decode_batch` copies (qwen3_generate_fast_batch); a never-emitted EOS id
+        # keeps every copy going; the timed call includes the prefill of its prompt and the allocation of its caches
+        inf.set_eos([cfg.V + 1])
+        prompt = rng.integers(1, cfg.V, args.prompt_len).astype(np.uint32)
+        inf.generate_batch(prompt, 2, args.decode_batch)               # builds the tiled weight images once
+        tb = time.perf_counter()
+        got = inf.generate_batch(prompt, args.steps, args.decode_batch)
+        dtb = time.perf_counter() - tb
+        steps_b = args.prompt_len + got.shape[1] - 1
+        batch = {"batch": args.decode_batch, "ms_per_step": round(dtb / steps_b * 1e3, 3),
+                 "tokens_per_s": round(args.decode_batch * steps_b / dtb, 1), "steps": steps_b}
     inf.free()
     gbs = wb.value / (tms.value * 1e-3) / 1e9 if tms.value > 0 else 0.0
     out = {"metric": "greedy decode tokens/s, batch 1", "value": round(args.steps / dt, 1), "unit": "tokens/s", "n_gpus": 1,
@@ -132,6 +145,8 @@ def decode_bench(args, cfg, L):
                         "launches_per_step": n // prof_steps, "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                         "weight_bytes_per_step": wb.value / prof_steps, "matvec_ms_per_step": round(tms.value / prof_steps, 3)},
            "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}
+    if batch:
+        out["batched"] = batch
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = decode_cpu_baseline(cfg)
     print(json.dumps(out))
@@ -148,6 +163,8 @@ def main():
                     help="time greedy token-by-token generation (include/inference_hip.h) on the configuration's model "
                          "instead of the training step: a step is one token")
     ap.add_argument("--prompt-len", type=int, default=16)
+    ap.add_argument("--decode-batch", type=int, default=0,
+                    help="with --decode: also time this many copies of one prompt decoded in lock step")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the library's plain copy kernel (1 GiB in, 1 GiB out, 5 launches): "
                          "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")

@@ -49,6 +49,15 @@ void inference_state_free(InferenceState *state);                    /* src/nn/f
 int inference_generate(InferenceState *state, const uint32_t *prompt_tokens, int prompt_len,
                        uint32_t *output_tokens, int max_gen_len);
 
+/* qwen3_generate_fast_batch (src/nn/fast_inference.h:70-72; impl src/nn/fast_inference.c:895-1000) on the weights of a
+ * state: batch_size copies of one prompt, prefilled and decoded greedily in lock step, every weight read once per step
+ * for all of them.  Runs with its own KV caches (the state's position and cache are left alone); F16 weights only and
+ * batch_size <= 32, as in the reference, but for either model type and with the state's adapters.  A sequence ends at
+ * one of the state's EOS ids or at token 0 (:944-947); the loop ends when all have.  output_tokens: [batch_size][max_gen_len].
+ * Returns the number of tokens written per sequence (0: arguments refused). */
+int inference_generate_batch(InferenceState *state, const uint32_t *prompt_tokens, int prompt_len, uint32_t *output_tokens,
+                             int max_gen_len, int batch_size);
+
 ModelType inference_state_model_type(InferenceState *state);         /* src/nn/fast_inference.h:31 */
 int  inference_state_vocab_size(InferenceState *state);              /* src/nn/fast_inference.h:34 */
 void inference_state_reset(InferenceState *state);                   /* src/nn/fast_inference.h:37: position := 0 */

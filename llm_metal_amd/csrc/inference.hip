@@ -110,6 +110,8 @@ __global__ __launch_bounds__(1024) void k_add_norm(float *__restrict__ x, const 
                                                    float *__restrict__ ln, int D, float eps)
 {
     __shared__ float sm[16];
+    x += (size_t)blockIdx.x * D; ln += (size_t)blockIdx.x * D;           // one workgroup per vector of a batch
+    if (branch) branch += (size_t)blockIdx.x * D;
     float inv_b = 1.f;
     if (branch && g_branch) {
         float ss = 0.f;
@@ -552,6 +554,166 @@ int inference_generate(InferenceState *s, const uint32_t *prompt_tokens, int pro
         next = argmax_to_host(s);
         output_tokens[n_gen++] = (uint32_t)next;
     }
+    return n_gen;
+}
+
+namespace {
+
+// act[b][i] = silu | gelu (gu[b][i]) * gu[b][IS + i]: the gated activation of a batch from the [gate | up] product
+__global__ __launch_bounds__(TB) void k_glu_batch(const float *__restrict__ gu, float *__restrict__ act, int IS, int gelu)
+{
+    const int b = blockIdx.y, i = blockIdx.x * TB + threadIdx.x;
+    if (i >= IS) return;
+    const float g = gu[(size_t)b * 2 * IS + i], u = gu[(size_t)b * 2 * IS + IS + i];
+    float a;
+    if (gelu) {                                                           // shaders/q8_kernels.metal:349-362
+        float t = 0.7978845608f * (g + 0.044715f * g * g * g);
+        t = fminf(fmaxf(t, -15.f), 15.f);
+        a = 0.5f * g * (1.0f + tanhf(t));
+    } else a = g / (1.0f + expf(-g));                                     // :337-347
+    act[(size_t)b * IS + i] = a * u;
+}
+
+// Scratch and KV caches of a batch of B sequences decoded in lock step (BatchState of src/nn/fast_inference.c:699-776).
+struct BatchRun {
+    int B;
+    MetalBuf *x, *branch, *ln, *qkv, *att, *gu, *act, *logits, *best, *lora_t;
+    std::vector<MetalBuf *> kc, vc;                                      // [layer * B + item]
+    int *best_host;
+};
+
+void batch_free(BatchRun &r)
+{
+    for (MetalBuf *b : {r.x, r.branch, r.ln, r.qkv, r.att, r.gu, r.act, r.logits, r.best, r.lora_t}) metal_buf_free(b);
+    for (MetalBuf *b : r.kc) metal_buf_free(b);
+    for (MetalBuf *b : r.vc) metal_buf_free(b);
+    if (r.best_host) hipHostFree(r.best_host);
+}
+
+// One step for B tokens at the same position: forward_token_batch, src/nn/fast_inference.c:808-893.  Every product
+// reads its weight once for all B vectors (matrix cores over the tiled image, gemm_f32a_exact); what is per sequence
+// -- adapter terms, per-head RMSNorm, RoPE, cache store, attention -- is one launch per sequence and layer.
+void forward_token_batch(InferenceState *s, BatchRun &r, const int *tokens, int pos)
+{
+    const int D = s->D, Hq = s->Hq, Hkv = s->Hkv, hd = s->hd, IS = s->IS, B = r.B;
+    const int qd = Hq * hd, kd = Hkv * hd, nqkv = qd + 2 * kd;
+    const bool gemma = s->model_type == MODEL_GEMMA3;
+    for (int b = 0; b < B; b++)
+        hipLaunchKernelGGL(k_embed_row, dim3((D + TB - 1) / TB), dim3(TB), 0, stream(), dptr_as<float>(s->emb), tokens[b], s->emb_scale,
+                           dptr_as<float>(r.x) + (size_t)b * D, D);
+    auto add_norm_b = [&](MetalBuf *branch, MetalBuf *g_branch, MetalBuf *g) {
+        hipLaunchKernelGGL(k_add_norm, dim3(B), dim3(1024), 0, stream(), dptr_as<float>(r.x), branch ? dptr_as<float>(branch) : nullptr,
+                           g_branch ? dptr_as<float>(g_branch) : nullptr, dptr_as<float>(g), dptr_as<float>(r.ln), D, s->eps);
+    };
+    auto product = [&](const WMat *w, MetalBuf *in, MetalBuf *out) {
+        gemm_f32a_exact(dptr_as<float>(in), w->mbuf, dptr_as<float>(out), B, w->rows, w->cols);
+        mark_written(out);
+    };
+    MetalBuf *pending = nullptr, *pending_g = nullptr;
+    for (int L = 0; L < s->NL; L++) {
+        const InferenceState::Layer &lw = s->layers[L];
+        add_norm_b(pending, pending_g, lw.g_in);
+        product(&lw.qkv, r.ln, r.qkv);
+        for (int b = 0; b < B; b++) {
+            HeadPost a{};
+            a.qkv = dptr_as<float>(r.qkv) + (size_t)b * nqkv;
+            a.g_q = lw.g_q ? dptr_as<float>(lw.g_q) : nullptr; a.g_k = lw.g_k ? dptr_as<float>(lw.g_k) : nullptr;
+            MetalBuf *kc = r.kc[(size_t)L * B + b], *vc = r.vc[(size_t)L * B + b];
+            a.kc = dptr_as<float>(kc); a.vc = dptr_as<float>(vc);
+            a.Hq = Hq; a.Hkv = Hkv; a.pos = pos;
+            a.rope = dptr_as<float2>(s->rope_tabs) + ((size_t)s->theta_slot[L] * s->max_seq + pos) * (hd / 2); a.eps = s->eps;
+            if (!s->lora.empty()) {
+                const InferenceState::Lora &lr = s->lora[L];
+                float *t = dptr_as<float>(r.lora_t) + (size_t)b * 2 * s->R;
+                hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R), dim3(64), 0, stream(), dptr_as<float>(r.ln) + (size_t)b * D,
+                                   dptr_as<float>(lr.Aq), dptr_as<float>(lr.Av), t, s->R, D);
+                a.t = t; a.Bq = dptr_as<float>(lr.Bq); a.Bv = dptr_as<float>(lr.Bv); a.R = s->R; a.sc = s->scaling;
+            }
+            attention_decode_fused(a, kc, vc, dptr_as<float>(r.att) + (size_t)b * qd, hd, s->max_seq);
+        }
+        mark_written(r.att);
+        product(lw.o, r.att, r.branch);
+        add_norm_b(r.branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
+        product(&lw.gu, r.ln, r.gu);
+        hipLaunchKernelGGL(k_glu_batch, dim3((IS + TB - 1) / TB, B), dim3(TB), 0, stream(), dptr_as<float>(r.gu), dptr_as<float>(r.act), IS,
+                           gemma ? 1 : 0);
+        product(lw.down, r.act, r.branch);
+        pending = r.branch;
+        pending_g = gemma ? lw.g_post_ff : nullptr;
+    }
+    add_norm_b(pending, pending_g, s->g_final);
+    product(s->lm_head, r.ln, r.logits);
+    HIP_CHECK(hipGetLastError());
+}
+
+// argmax of every sequence's logits, computed on the GPU; one wait for all of them
+void argmax_batch(InferenceState *s, BatchRun &r, int *out)
+{
+    for (int b = 0; b < r.B; b++) {
+        float *pv = dptr_as<float>(r.best) + r.B + (size_t)b * 2 * AM_WGS;
+        int *pi = reinterpret_cast<int *>(pv) + AM_WGS;
+        hipLaunchKernelGGL(k_argmax_part, dim3(AM_WGS), dim3(TB), 0, stream(), dptr_as<float>(r.logits) + (size_t)b * s->V, s->V, pv, pi);
+        hipLaunchKernelGGL(k_argmax_final, dim3(1), dim3(AM_WGS), 0, stream(), pv, pi, dptr_as<int>(r.best) + b);
+    }
+    HIP_CHECK(hipMemcpyAsync(r.best_host, dptr(r.best), (size_t)r.B * sizeof(int), hipMemcpyDeviceToHost, stream()));
+    HIP_CHECK(hipStreamSynchronize(stream()));
+    for (int b = 0; b < r.B; b++) out[b] = r.best_host[b];
+}
+
+}  // namespace
+
+// qwen3_generate_fast_batch, src/nn/fast_inference.c:895-1000, on a state's weights: batch_size copies of one prompt are
+// prefilled and then decoded greedily in lock step, so that a step reads every weight once for all of them.  The loop
+// ends when every sequence has emitted an end token (the state's EOS ids, or token 0 as in the reference, :944-947),
+// after max_gen_len tokens or when the cache is full; sequences that have ended keep being stepped and written, as in
+// the reference.  output_tokens: [batch_size][max_gen_len].  Returns the tokens written per sequence, 0 when the
+// arguments do not fit (F16 weights only, 1 <= batch_size <= 32, prompt within the cache).
+int inference_generate_batch(InferenceState *s, const uint32_t *prompt_tokens, int prompt_len, uint32_t *output_tokens,
+                             int max_gen_len, int batch_size)
+{
+    const int B = batch_size;
+    if (!s->use_fp16) { fprintf(stderr, "[BatchGen] F16 weights only\n"); return 0; }
+    if (B < 1 || B > 32 || prompt_len <= 0 || max_gen_len <= 0 || prompt_len > s->max_seq) return 0;
+    for (int i = 0; i < prompt_len; i++)
+        if (prompt_tokens[i] >= (uint32_t)s->V) { fprintf(stderr, "[BatchGen] token %u outside the vocabulary (%d)\n", prompt_tokens[i], s->V); return 0; }
+    const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS, V = s->V;
+    BatchRun r{};
+    r.B = B;
+    r.x = fbuf((size_t)B * D); r.branch = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
+    r.qkv = fbuf((size_t)B * (qd + 2 * kd)); r.att = fbuf((size_t)B * qd);
+    r.gu = fbuf((size_t)B * 2 * IS); r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
+    r.best = metal_buf_create(((size_t)B + (size_t)B * 2 * AM_WGS) * sizeof(int));
+    r.lora_t = s->lora.empty() ? nullptr : fbuf((size_t)B * 2 * s->R);
+    HIP_CHECK(hipHostMalloc((void **)&r.best_host, (size_t)B * sizeof(int), hipHostMallocDefault));
+    const size_t cache_bytes = (size_t)s->Hkv * s->max_seq * s->hd * sizeof(float);
+    for (int i = 0; i < s->NL * B; i++) { r.kc.push_back(metal_buf_create(cache_bytes)); r.vc.push_back(metal_buf_create(cache_bytes)); }
+
+    int tokens[32], next[32], active[32];
+    for (int i = 0; i < prompt_len; i++) {                               // prefill: the same token for every sequence (:910-916)
+        for (int b = 0; b < B; b++) tokens[b] = (int)prompt_tokens[i];
+        forward_token_batch(s, r, tokens, i);
+    }
+    int cur_len = prompt_len;
+    argmax_batch(s, r, next);
+    for (int b = 0; b < B; b++) { output_tokens[(size_t)b * max_gen_len] = (uint32_t)next[b]; active[b] = 1; }
+    int n_gen = 1;
+    for (int gen = 1; gen < max_gen_len && cur_len < s->max_seq; gen++) {
+        int any_active = 0;
+        for (int b = 0; b < B; b++) {
+            bool ended = next[b] == 0;
+            for (int e = 0; e < s->n_eos; e++) ended |= next[b] == s->eos[e];
+            if (active[b] && ended) active[b] = 0;
+            any_active |= active[b];
+        }
+        if (!any_active) break;
+        forward_token_batch(s, r, next, cur_len);
+        cur_len++;
+        argmax_batch(s, r, next);
+        for (int b = 0; b < B; b++) output_tokens[(size_t)b * max_gen_len + n_gen] = (uint32_t)next[b];
+        n_gen++;
+    }
+    metal_flush();
+    batch_free(r);
     return n_gen;
 }
 

@@ -276,6 +276,13 @@ class InferenceState:
         n = self.L.inference_generate(self.h, _vp(prompt), len(prompt), _vp(out), max_gen_len)
         return out[:n]
 
+    def generate_batch(self, prompt, max_gen_len, batch):
+        """[batch, n] tokens: the same prompt decoded greedily `batch` times in lock step."""
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.zeros((batch, max_gen_len), dtype=np.uint32)
+        n = self.L.inference_generate_batch(self.h, _vp(prompt), len(prompt), _vp(out), max_gen_len, batch)
+        return out[:, :n]
+
     def set_eos(self, ids):
         a = np.ascontiguousarray(ids, dtype=np.int32)
         self.L.inference_state_set_eos(self.h, _vp(a), len(a))

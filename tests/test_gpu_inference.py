@@ -71,6 +71,55 @@ def test_forward_token_logits_and_greedy_generation(cfg, fmt):
         assert inf.forward_token_argmax(c.V) == -1 and inf.position() == 0
 
 
+@pytest.mark.parametrize("cfg,with_lora", [(C1.with_(seq=8), False), (TINY_GEMMA, False), (C1.with_(seq=8), True)],
+                         ids=["qwen3", "gemma3", "qwen3_adapters"])
+def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, with_lora):
+    """inference_generate_batch (qwen3_generate_fast_batch, src/nn/fast_inference.c:895-1000): B copies of one prompt
+    in lock step, weights read once per step.  Every copy must produce the single-sequence greedy tokens (wherever the
+    choice was not a near-tie: the batched products keep 22 bits of the activations, the single ones all 24), the
+    oracle's decode chain must agree with them, and an end token stops the loop once all copies have emitted it."""
+    say("batched generation", cfg.name, with_lora)
+    c = cfg
+    model = make_model(c, seed=17, gamma_jitter=0.1)
+    tok, _ = make_batch(c, seed=18)
+    prompt = [int(t) for t in tok[:4]]
+    B, n = 5, 12
+
+    def check(inf, lora):
+        single = [int(g) for g in inf.generate(prompt, n)]
+        assert len(single) == n
+        pos = inf.position()
+        got = inf.generate_batch(prompt, n, B)
+        assert got.shape == (B, n) and inf.position() == pos          # its own caches: the state's are left alone
+        lo = oracle_decode(c, model, "f16", prompt + single[:-1], max_seq=32, precision="f32", lora=lora)[len(prompt) - 1:]
+        srt = np.sort(lo, axis=1)
+        clear = (srt[:, -1] - srt[:, -2]) > 1e-3 * np.abs(lo).max()
+        first_tie = n if clear.all() else int(np.argmin(clear))        # after a near-tie the sequences may part ways
+        assert first_tie >= 4
+        for b in range(B):
+            assert [int(t) for t in got[b, :first_tie]] == single[:first_tie], b
+            assert np.array_equal(got[b], got[0])                      # identical inputs, identical arithmetic
+        assert (lo.argmax(1)[:first_tie] == np.asarray(single)[:first_tie]).all()
+        # an end token: every copy emits it at the same step, and the loop stops after it
+        inf.set_eos([single[2]])
+        stop = single.index(single[2])
+        got2 = inf.generate_batch(prompt, n, 3)
+        assert got2.shape == (3, stop + 1) and [int(t) for t in got2[1]] == single[:stop + 1]
+        # refused: too many copies, a token outside the vocabulary
+        assert inf.generate_batch(prompt, n, 33).shape[1] == 0
+        assert inf.generate_batch([c.V], n, 2).shape[1] == 0
+
+    if with_lora:
+        with SFTState(c, model) as sft:
+            with InferenceState(sft=sft, max_seq=32) as inf:
+                check(inf, model["lora"])
+    else:
+        with InferenceState(c, model, max_seq=32, use_fp16=True) as inf:
+            check(inf, None)
+        with InferenceState(c, model, max_seq=32, use_fp16=False) as q8:
+            assert q8.generate_batch(prompt, n, 2).shape[1] == 0       # F16 weights only, as in the reference
+
+
 def test_eos_ids_from_config_json(tmp_path, capfd):
     c = C1.with_(seq=4)
     model = make_model(c, seed=9)
