@@ -175,6 +175,9 @@ typedef struct {
     float clip_eps;
     int accurate;                         /* full-parameter only: 1 = accumulate, apply once; 0 = SGD per completion with lr/G */
 } GRPOCompletions;
+/* new_logprobs: optional, [G][seq_len].  A state built with batch B takes B completions per forward / backward pass
+ * (every weight is streamed once per pass, not once per completion); the F16 accumulators are then rounded once per
+ * pass instead of once per completion.  Full-parameter SGD after every completion (accurate == 0) needs batch 1. */
 void grpo_apply_completions(SFTState *state, const GRPOCompletions *c, float lr, float *new_logprobs);
 /* "LORA" adapter file, src/nn/fast_sft.c:1255-1285 */
 void sft_save_lora(SFTState *state, const char *path);

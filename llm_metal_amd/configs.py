@@ -69,7 +69,8 @@ C1 = SFTConfig("c1_tiny_qwen3", QWEN3, NL=2, D=256, Hq=4, Hkv=2, hd=64, IS=768, 
 C2 = SFTConfig("c2_gemma3_1b", GEMMA3, NL=26, D=1152, Hq=4, Hkv=1, hd=256, IS=6912, V=262144, tied=True)
 C3 = SFTConfig("c3_qwen3_4b_f16", QWEN3, NL=36, D=2560, Hq=32, Hkv=8, hd=128, IS=9728, V=151936)
 C4 = C3.with_(name="c4_qwen3_4b_q8", batch=4, seq=512, weight_format="q8_0")
-C5 = C2.with_(name="c5_gemma3_1b_grpo", batch=1, seq=160, R=0)
+# the group of four 160-token sequences is one batch: a pass streams every weight once for the whole group
+C5 = C2.with_(name="c5_gemma3_1b_grpo", batch=4, seq=160, R=0)
 # config 3's step on Q8_0 weights: the dequant-fused weight-streaming GEMM at M = 64
 C3Q = C3.with_(name="c3_qwen3_4b_q8_seq64", weight_format="q8_0")
 

@@ -42,10 +42,12 @@ struct WeightPrefetch {
     int depth;                    // K steps fetched per product workgroup (its waves' first steps)
 };
 
+constexpr uint32_t ZERO_ROW_TOKEN = 0xFFFFFFFFu;
+
 struct NormRowsArgs {
     // source of the residual stream row: token gather (emb != null) or x_prev
     const float *emb; const uint32_t *tokens; float emb_scale;
-    int n_valid;                  // gather only: rows >= n_valid read as zero (0 = every row is valid)
+    int zero_rows;                // gather only: rows whose token id is ZERO_ROW_TOKEN read as zero (padding of a short sequence)
     const float *x_prev;
     // optional branch added to it: planes, optionally RMS-normalised with g_branch first
     Planes branch; const float *g_branch; float *branch_raw_out;

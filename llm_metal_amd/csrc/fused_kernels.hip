@@ -65,8 +65,9 @@ __global__ __launch_bounds__(NT) void k_norm_rows(NormRowsArgs a)
     const size_t r = blockIdx.x;
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
-    const bool padded = a.emb && a.n_valid > 0 && (int)r >= a.n_valid;      // zero rows past the sequence
-    const float *base = a.emb ? a.emb + (size_t)(padded ? 0u : a.tokens[r]) * D : a.x_prev + r * D;
+    const uint32_t tok = a.emb ? a.tokens[r] : 0u;
+    const bool padded = a.emb && a.zero_rows && tok == ZERO_ROW_TOKEN;      // zero rows past the end of a sequence
+    const float *base = a.emb ? a.emb + (size_t)(padded ? 0u : tok) * D : a.x_prev + r * D;
     size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {

@@ -253,7 +253,7 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
     return Planes{P, p.S, stride, N, out ? nullptr : inv};
 }
 
-void forward_impl(SFTState *s, bool gather, int n_valid = 0)
+void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
 {
     const int BN = s->BN, D = s->D, IS = s->IS, qd = s->qd, kd = s->kd, R = s->R;
     const size_t xsz = (size_t)BN * D;
@@ -270,7 +270,7 @@ void forward_impl(SFTState *s, bool gather, int n_valid = 0)
         // x_in = x (+ previous FFN branch); ln1 = RN(x_in; g_in)        [src/nn/fast_sft.c:631-635, 732-740]
         NormRowsArgs n1{};
         if (L == 0) {
-            if (gather) { n1.emb = at<float>(s->emb); n1.tokens = at<uint32_t>(s->tokens); n1.emb_scale = s->emb_scale; n1.n_valid = n_valid; }
+            if (gather) { n1.emb = at<float>(s->emb); n1.tokens = at<uint32_t>(s->tokens); n1.emb_scale = s->emb_scale; n1.zero_rows = zero_rows; }
             else n1.x_prev = at<float>(s->x_in_host);
         } else {
             n1.x_prev = at<float>(s->xs, (size_t)(2 * L - 1) * xsz);
@@ -1109,48 +1109,59 @@ WMat *sft_get_lm_head(SFTState *s)
 // new_logprobs (optional, [G][rows]) receives the policy's log-probabilities of the actions.
 void grpo_apply_completions(SFTState *s, const GRPOCompletions *c, float lr, float *new_logprobs)
 {
-    if (s->B != 1) { fprintf(stderr, "[FastGRPO] the state must be built with batch 1\n"); return; }
-    const int G = c->group_size, seq_len = s->BN;
+    const int G = c->group_size, seq_len = s->N, B = s->B;
     if (G <= 0) return;
+    const bool accurate = s->full_param && c->accurate;
+    if (B > 1 && s->full_param && !accurate) {
+        fprintf(stderr, "[FastGRPO] SGD after every completion needs a state built with batch 1 (the weights change between completions)\n");
+        return;
+    }
     if (s->step_in_flight) { metal_flush(); s->step_in_flight = 0; }
     if (!ids_in_vocab(s, c->prompt, (size_t)(c->prompt_len > 0 ? c->prompt_len : 0), "prompt token")) return;
     for (int i = 0; i < G; i++)
         if (!ids_in_vocab(s, c->gen_tokens[i], (size_t)(c->gen_lengths[i] > 0 ? c->gen_lengths[i] : 0), "completion token")) return;
-    const bool accurate = s->full_param && c->accurate;
     if (accurate) sft_alloc_grad_accum(s);
     if (!s->grpo_old_lp) {
-        s->grpo_old_lp = host_buf((size_t)seq_len * 4, (void **)&s->grpo_old_lp_cpu);
-        s->grpo_advs = host_buf((size_t)seq_len * 4, (void **)&s->grpo_advs_cpu);
-        s->grpo_new_lp = host_buf((size_t)seq_len * 4, (void **)&s->grpo_new_lp_cpu);
+        s->grpo_old_lp = host_buf((size_t)s->BN * 4, (void **)&s->grpo_old_lp_cpu);
+        s->grpo_advs = host_buf((size_t)s->BN * 4, (void **)&s->grpo_advs_cpu);
+        s->grpo_new_lp = host_buf((size_t)s->BN * 4, (void **)&s->grpo_new_lp_cpu);
     }
     if (!s->full_param) {
         if (!s->lora_acc) s->lora_acc = fbuf(s->lora_n);
         HIP_CHECK(hipMemsetAsync(dptr(s->lora_acc), 0, s->lora_n * 4, stream()));
     }
-    for (int i = 0; i < G; i++) {
-        int comp_len = c->gen_lengths[i];                  // [:388-400]
-        if (comp_len > seq_len) comp_len = seq_len;
-        int prompt_use = seq_len - comp_len;
-        if (prompt_use > c->prompt_len) prompt_use = c->prompt_len;
-        if (prompt_use < 0) prompt_use = 0;
-        int total = prompt_use + comp_len;
-        if (total > seq_len) { comp_len = seq_len - prompt_use; total = seq_len; }
-        if (new_logprobs) memset(new_logprobs + (size_t)i * seq_len, 0, (size_t)seq_len * 4);
-        if (total <= 0) continue;                          // nothing but zero rows: no gradient
-        const int prompt_start = c->prompt_len - prompt_use;
-        memset(s->tokens_cpu, 0, (size_t)seq_len * 4);
-        memset(s->targets_cpu, 0, (size_t)seq_len * 4);    // actions                      [:430-443]
-        memset(s->grpo_old_lp_cpu, 0, (size_t)seq_len * 4);
-        memset(s->grpo_advs_cpu, 0, (size_t)seq_len * 4);
-        for (int t = 0; t < prompt_use; t++) s->tokens_cpu[t] = c->prompt[prompt_start + t];
-        for (int t = 0; t < comp_len; t++) {
-            const int pos = prompt_use + t;
-            s->tokens_cpu[pos] = c->gen_tokens[i][t];
-            s->targets_cpu[pos] = c->gen_tokens[i][t];
-            s->grpo_old_lp_cpu[pos] = c->gen_logprobs[i][t];
-            s->grpo_advs_cpu[pos] = c->advantages[i];
+    // A state built with batch B takes B completions per pass (one forward and backward for all of them: every weight
+    // is streamed once per pass instead of once per completion); sequence slots beyond the group are all zero rows.
+    for (int i0 = 0; i0 < G; i0 += B) {
+        int any = 0;
+        for (int b = 0; b < B; b++) {
+            const int i = i0 + b;
+            uint32_t *tok = s->tokens_cpu + (size_t)b * seq_len, *act = s->targets_cpu + (size_t)b * seq_len;
+            float *olp = s->grpo_old_lp_cpu + (size_t)b * seq_len, *adv = s->grpo_advs_cpu + (size_t)b * seq_len;
+            for (int t = 0; t < seq_len; t++) { tok[t] = ZERO_ROW_TOKEN; act[t] = 0; olp[t] = 0.f; adv[t] = 0.f; }
+            if (i >= G) continue;
+            int comp_len = c->gen_lengths[i];                  // [:388-400]
+            if (comp_len > seq_len) comp_len = seq_len;
+            int prompt_use = seq_len - comp_len;
+            if (prompt_use > c->prompt_len) prompt_use = c->prompt_len;
+            if (prompt_use < 0) prompt_use = 0;
+            int total = prompt_use + comp_len;
+            if (total > seq_len) { comp_len = seq_len - prompt_use; total = seq_len; }
+            if (new_logprobs) memset(new_logprobs + (size_t)i * seq_len, 0, (size_t)seq_len * 4);
+            if (total <= 0) continue;                          // nothing but zero rows: no gradient
+            any = 1;
+            const int prompt_start = c->prompt_len - prompt_use;
+            for (int t = 0; t < prompt_use; t++) tok[t] = c->prompt[prompt_start + t];
+            for (int t = 0; t < comp_len; t++) {               // actions                      [:430-443]
+                const int pos = prompt_use + t;
+                tok[pos] = c->gen_tokens[i][t];
+                act[pos] = c->gen_tokens[i][t];
+                olp[pos] = c->gen_logprobs[i][t];
+                adv[pos] = c->advantages[i];
+            }
         }
-        forward_impl(s, true, total < seq_len ? total : 0);
+        if (!any) continue;
+        forward_impl(s, true, true);
         CeArgs ce{};
         ce.logits = at<float>(s->logits); ce.V = s->V; ce.targets = at<uint32_t>(s->targets); ce.losses = at<float>(s->losses);
         ce.dl16 = at<half_t>(s->dl16); ce.inv_scale = at<float>(s->dl_inv); ce.rows_total = s->BN;
@@ -1165,7 +1176,9 @@ void grpo_apply_completions(SFTState *s, const GRPOCompletions *c, float lr, flo
             metal_enqueue_add_scaled(s->lora_acc, s->lora_grad, 1.0f, (int)s->lora_n);
         }
         metal_flush();
-        if (new_logprobs) memcpy(new_logprobs + (size_t)i * seq_len, s->grpo_new_lp_cpu, (size_t)seq_len * 4);
+        if (new_logprobs)
+            for (int b = 0; b < B && i0 + b < G; b++)
+                memcpy(new_logprobs + (size_t)(i0 + b) * seq_len, s->grpo_new_lp_cpu + (size_t)b * seq_len, (size_t)seq_len * 4);
     }
     if (accurate) {                                                               // [:479-481]
         sft_apply_grad_sgd(s, lr);

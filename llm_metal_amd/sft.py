@@ -209,7 +209,7 @@ class SFTState:
 
     def grpo_apply_completions(self, prompt, gen_tokens, gen_logprobs, advantages, clip_eps, lr, accurate=True):
         """Phases 3-4 of a GRPO step over already sampled completions.  Returns the policy's
-        log-probabilities of the actions, [G, rows] (zero outside the completion positions)."""
+        log-probabilities of the actions, [G, seq].  A state built with batch B runs B completions per pass."""
         G = len(gen_tokens)
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
         toks = [np.ascontiguousarray(t, dtype=np.uint32) for t in gen_tokens]
@@ -220,7 +220,7 @@ class SFTState:
         lp = (C.c_void_p * G)(*[p.ctypes.data for p in lps])
         c = _lib.GRPOCompletions(prompt.ctypes.data, len(prompt), G, tp, lens.ctypes.data, lp, adv.ctypes.data,
                                  clip_eps, 1 if accurate else 0)
-        new_lp = np.zeros((G, self.c.BN), dtype=np.float32)
+        new_lp = np.zeros((G, self.c.seq), dtype=np.float32)
         self.L.grpo_apply_completions(self.h, C.byref(c), lr, _vp(new_lp))
         return new_lp
 

@@ -135,9 +135,14 @@ def _oracle_sequence(cfg, used, prompt, toks_i):
     return x, use, comp
 
 
-@pytest.mark.parametrize("cfg", [FULL_G.with_(name="grpo_full_gemma", seq=48), FULL_Q.with_(name="grpo_full_qwen", seq=32)],
+# the last two run the whole group (4 completions) and three of the four per pass: a state built with batch B takes B
+# completions per forward / backward, the oracle stays sequential (one F16 rounding of G per completion instead of per pass)
+@pytest.mark.parametrize("cfg", [FULL_G.with_(name="grpo_full_gemma", seq=48), FULL_Q.with_(name="grpo_full_qwen", seq=32),
+                                 FULL_G.with_(name="grpo_full_gemma_batch4", seq=48, batch=4),
+                                 FULL_Q.with_(name="grpo_full_qwen_batch3", seq=32, batch=3)],
                          ids=lambda c: c.name)
 def test_grpo_accumulate_and_apply(cfg):
+    gpu_cfg, cfg = cfg, cfg.with_(batch=1)                 # the oracle follows one completion at a time
     rng = np.random.default_rng(5)
     G = 4
     prompt, toks, adv = _completions(cfg, rng, G, 12, [cfg.seq - 12, cfg.seq - 20, 5, cfg.seq + 7])   # exact, short, tiny, too long
@@ -167,7 +172,7 @@ def test_grpo_accumulate_and_apply(cfg):
         r = oracle.full_param_pass(cfg, used, ga, x_rows=x, grpo=dict(actions=act, old_lp=olp, advs=advs, clip_eps=clip, dl_scale=1.0 / G))
         want_lp[i] = r["new_lp"]
     oracle.apply_grad_sgd(cfg, used, ga, lr)
-    with SFTState(cfg, model) as st:
+    with SFTState(gpu_cfg, model) as st:
         got_lp = st.grpo_apply_completions(prompt, toks, old, adv, clip, lr, accurate=True)
         for i, t in enumerate(toks):
             _, use, comp = _oracle_sequence(cfg, used, prompt, t)
@@ -181,7 +186,8 @@ def test_grpo_accumulate_and_apply(cfg):
             assert rel(d_gpu, d_ref) < 3e-2, (L, k, rel(d_gpu, d_ref))
 
 
-def test_grpo_lora_mode_sums_adapter_gradients_then_adamw():
+@pytest.mark.parametrize("batch", [1, 2], ids=["one_per_pass", "two_per_pass"])
+def test_grpo_lora_mode_sums_adapter_gradients_then_adamw(batch):
     cfg = C1.with_(name="grpo_lora", seq=32)
     rng = np.random.default_rng(6)
     G = 3
@@ -201,7 +207,7 @@ def test_grpo_lora_mode_sums_adapter_gradients_then_adamw():
         r = oracle.full_param_pass(cfg, used, None, x_rows=x, lora=lora,
                                    grpo=dict(actions=act, old_lp=olp, advs=advs, clip_eps=clip, dl_scale=1.0 / G))
         acc += r["grad"]
-    with SFTState(cfg, model) as st:
+    with SFTState(cfg.with_(batch=batch), model) as st:
         st.grpo_apply_completions(prompt, toks, old, adv, clip, lr)
         assert st.step_count() == 1
         gn = float(np.sqrt((acc.astype(np.float64) ** 2).sum()))

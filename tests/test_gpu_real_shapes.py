@@ -109,10 +109,12 @@ def test_q8_step_at_2048_rows_matches_oracle_fixture(policy):
         L.hip_gemm_force_large_m(0)
 
 
-def test_grpo_full_parameter_at_real_widths_matches_oracle_fixture():
+@pytest.mark.parametrize("batch", [1, 2], ids=["one_completion_per_pass", "group_in_one_pass"])
+def test_grpo_full_parameter_at_real_widths_matches_oracle_fixture(batch):
     """Config 5's shape on two layers: Gemma3-1B widths, full-parameter, 160 rows per completion, F16 accumulation
-    over the group and one apply (grpo_apply_completions, src/nn/fast_grpo.c:376-495)."""
-    cfg = rw.C5_WIDTHS
+    over the group and one apply (grpo_apply_completions, src/nn/fast_grpo.c:376-495); the fixture's two completions
+    one per pass (as the reference runs them) and both in one pass (as the benchmark runs its group of four)."""
+    cfg = rw.C5_WIDTHS.with_(batch=batch)
     model = make_model(cfg, seed=rw.MODEL_SEED, gamma_jitter=rw.GAMMA_JITTER)
     g = _golden("real_width_c5.npz", model)
     used = oracle.weights_as_used(model)
