@@ -59,9 +59,10 @@ def cpu_baseline(cfg, budget_s=20.0):
     dt = time.perf_counter() - t0
     scale = cfg.frozen_params / small.frozen_params
     est = dt * scale
-    return {"value": cfg.BN / est, "unit": "tokens/s", "cores": 1, "kind": "port",
+    return {"value": cfg.BN / est, "unit": "tokens/s", "cores": 1, "host_cores_total": os.cpu_count(), "kind": "port",
             "sample": f"oracle full step on {nl} of {cfg.NL} layers + {v} of {cfg.V} vocab rows "
-                      f"({dt:.1f} s measured), scaled by the frozen-parameter ratio {scale:.1f}"}
+                      f"({dt:.1f} s measured), scaled by the frozen-parameter ratio {scale:.1f}; one thread "
+                      f"(the reference's CPU path has no threading) of the box's {os.cpu_count()} logical cores"}
 
 
 def decode_cpu_baseline(cfg):
@@ -82,7 +83,7 @@ def decode_cpu_baseline(cfg):
         op("f32", "or_f16_batch_matvec", w, x, y, w.shape[0], w.shape[1], 1)
     dt = time.perf_counter() - t0
     scale = cfg.frozen_params / small.frozen_params
-    return {"value": 1.0 / (dt * scale), "unit": "tokens/s", "cores": 1, "kind": "port",
+    return {"value": 1.0 / (dt * scale), "unit": "tokens/s", "cores": 1, "host_cores_total": os.cpu_count(), "kind": "port",
             "sample": f"oracle matrix-vector products of one token on {nl} of {cfg.NL} layers + {v} of {cfg.V} vocab rows "
                       f"({dt:.2f} s measured), scaled by the frozen-parameter ratio {scale:.1f}"}
 
@@ -263,6 +264,9 @@ def main():
                 "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}
     roofline["traffic"] = measured_traffic(cfg.name)
+    roofline["traffic_source"] = ("profiles/c3_gemm_hbm_traffic_pmc.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
+                                  "scaled by the same counters on a copy kernel of known size; not re-measured in this run"
+                                  if roofline["traffic"] is not None else "no hardware-counter summary is committed for this workload")
     st.free()
 
     metric = ("SFT train tokens/s, Qwen3-4B LoRA r16 seq64; % of HBM-BW / MFMA peak" if cfg.name == "c3_qwen3_4b_f16" else
