@@ -134,7 +134,9 @@ void launch_lora_grads(const LoraGradArgs &a);
 struct GluArgs {
     Planes in;                    // fwd: [rows][gate | up]; bwd: [rows][d act]
     int IS, gelu;
-    float *gate_pre, *up_val;     // fwd: written; bwd: read
+    float *gate_pre, *up_val;     // fwd: written; bwd: read; rows ld_gu floats apart (the two are the halves of one [rows][2 IS] array)
+    size_t ld_gu;
+    int in_place;                 // fwd, one workgroup per row only: `in` is that array (one plane, factors applied): nothing to copy
     half_t *out16; float *inv_scale;                // tiled; fwd: act [rows, IS]; bwd: [rows, dgate | dup]
     ScaleGroups sg;               // sg.cols != 0: inv_scale is [rows][sg.groups]
 };

@@ -740,8 +740,10 @@ __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
         act[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (v < nv) {
             const float4 g = gu[t], u = gu[MAXV + t];
-            st4(a.gate_pre + r * IS + 4 * v, g);
-            st4(a.up_val + r * IS + 4 * v, u);
+            if (!a.in_place) {                                // in place: the product wrote [gate | up] where they are kept
+                st4(a.gate_pre + r * a.ld_gu + 4 * v, g);
+                st4(a.up_val + r * a.ld_gu + 4 * v, u);
+            }
             act[t] = make_float4(act_fwd(g.x, a.gelu) * u.x, act_fwd(g.y, a.gelu) * u.y,
                                  act_fwd(g.z, a.gelu) * u.z, act_fwd(g.w, a.gelu) * u.w);
             amax = fmaxf(amax, amax4(act[t]));
@@ -784,8 +786,10 @@ __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
         act[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (v < nv) {
             const float4 g = gu[t], u = gu[MAXC + t];
-            st4(a.gate_pre + r * IS + c0 + 4 * v, g);
-            st4(a.up_val + r * IS + c0 + 4 * v, u);
+            if (!a.in_place) {
+                st4(a.gate_pre + r * a.ld_gu + c0 + 4 * v, g);
+                st4(a.up_val + r * a.ld_gu + c0 + 4 * v, u);
+            }
             act[t] = make_float4(act_fwd(g.x, GELU) * u.x, act_fwd(g.y, GELU) * u.y,
                                  act_fwd(g.z, GELU) * u.z, act_fwd(g.w, GELU) * u.w);
             amax = fmaxf(amax, amax4(act[t]));
@@ -829,7 +833,7 @@ __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
             const int v = threadIdx.x + t * RB;
             rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
             gs[t] = us[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (v < nv) { gs[t] = ld4(a.gate_pre + r * IS + 4 * v); us[t] = ld4(a.up_val + r * IS + 4 * v); }
+            if (v < nv) { gs[t] = ld4(a.gate_pre + r * a.ld_gu + 4 * v); us[t] = ld4(a.up_val + r * a.ld_gu + 4 * v); }
         }
         planes_at4_multi<MAXV, 5>(a.in, rows, cols, ok, dys);
     }
@@ -876,7 +880,7 @@ __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
             const int v = threadIdx.x + t * GC, j = c0 + 4 * v;
             rows[t] = r; cols[t] = j < IS ? j : j - IS; ok[t] = v < nv;
             gs[t] = us[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (v < nv) { gs[t] = ld4(a.gate_pre + r * IS + cols[t]); us[t] = ld4(a.up_val + r * IS + cols[t]); }
+            if (v < nv) { gs[t] = ld4(a.gate_pre + r * a.ld_gu + cols[t]); us[t] = ld4(a.up_val + r * a.ld_gu + cols[t]); }
         }
         planes_at4_multi<MAXC, 5>(a.in, rows, cols, ok, dys);
     }
@@ -1240,6 +1244,8 @@ void launch_glu_fwd(const GluArgs &a, int rows)
 {
     require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_fwd: FFN width must be a multiple of 4, <= 12288");
     require(!a.in.scale_groups, "glu_fwd: input planes with grouped row factors are not supported");
+    require(!a.in_place || (a.in.S == 1 && !a.in.row_scale && a.in.p == a.gate_pre && (size_t)a.in.ld == a.ld_gu),
+            "glu_fwd: in place needs the product's one finished plane to be the kept [gate | up] array");
     if (a.sg.cols) {
         require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC * MAXC && (long)a.sg.cols * a.sg.groups >= a.IS && (long)a.sg.cols * (a.sg.groups - 1) < a.IS,
                 "glu_fwd: column groups do not fit the row");

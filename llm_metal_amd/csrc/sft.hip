@@ -60,7 +60,7 @@ struct SFTState {
     // saved activations (layer-strided arenas)
     MetalBuf *xs;                        // [2*NL + 1][BN*D]: x_in[L] = 2L, x_mid[L] = 2L+1, x_final = 2NL
     MetalBuf *ln1_16, *ln1_inv;          // [NL][BN*D] f16, [NL][BN]
-    MetalBuf *q_pre, *k_pre, *q_fin, *k_fin, *v_sav, *probs, *gate_pre, *up_val, *tq, *tv, *o_raw, *ff_raw;
+    MetalBuf *q_pre, *k_pre, *q_fin, *k_fin, *v_sav, *probs, *gu_sav, *tq, *tv, *o_raw, *ff_raw;   // gu_sav: [NL][BN][gate (IS) | up (IS)]
     MetalBuf *kT, *vT;                   // k_fin / v_sav once more, per head and transposed, for the matrix-core attention
     // transients
     MetalBuf *a16, *a16_inv;             // largest fp16 operand (BN x max K) and its row factors
@@ -331,10 +331,15 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
         launch_norm_rows(n2, BN);
 
         // [gate | up] = ln2 [Wg; Wu]^T; act = silu|gelu(gate) * up              [:715-725]
-        Planes pg = gemm(s, ln2, ln2inv, wop(s, W_GU, L, false), 2 * IS, D);
+        // [gate | up] of the layer are kept for the backward as one [BN][2 IS] array, which is the product's own output
+        // layout: the large-M kernel writes it there, the streaming kernel's planes are summed into it by the GLU kernel
+        float *gu_keep = at<float>(s->gu_sav, (size_t)L * BN * 2 * IS);
+        const WeightOp wgu = wop(s, W_GU, L, false);
+        const bool direct = use_big_gemm(BN, 2 * IS, D, wgu.fmt);
+        Planes pg = gemm(s, ln2, ln2inv, wgu, 2 * IS, D, direct ? gu_keep : nullptr);
         GluArgs ga{};
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
-        ga.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); ga.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
+        ga.gate_pre = gu_keep; ga.up_val = gu_keep + IS; ga.ld_gu = (size_t)2 * IS; ga.in_place = direct;
         ga.sg = scale_groups_for(s, wop(s, W_D, L, false), D, IS);
         ga.out16 = act16; ga.inv_scale = ga.sg.cols ? at<float>(s->group_inv) : actinv;
         launch_glu_fwd(ga, BN);
@@ -416,7 +421,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
                         s->wd, s->wdT, s->gd, L * s->st_d, L * s->st_dT);
         GluArgs gb{};
         gb.in = pd; gb.IS = IS; gb.gelu = gemma;
-        gb.gate_pre = at<float>(s->gate_pre, (size_t)L * BN * IS); gb.up_val = at<float>(s->up_val, (size_t)L * BN * IS);
+        gb.gate_pre = at<float>(s->gu_sav, (size_t)L * BN * 2 * IS); gb.up_val = gb.gate_pre + IS; gb.ld_gu = (size_t)2 * IS;
         if (mode == BWD_LORA) gb.sg = scale_groups_for(s, wop(s, W_GU, L, true), D, 2 * IS);
         gb.out16 = a16; gb.inv_scale = gb.sg.cols ? at<float>(s->group_inv) : ainv;
         launch_glu_bwd(gb, BN);
@@ -722,7 +727,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     if (attn_mfma_supported(s->hd, s->N)) {
         s->kT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N)); s->vT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N));
     }
-    s->gate_pre = fbuf((size_t)NL * BN * IS); s->up_val = fbuf((size_t)NL * BN * IS);
+    s->gu_sav = fbuf((size_t)NL * BN * 2 * IS);
     s->tq = fbuf((size_t)NL * BN * (R ? R : 1)); s->tv = fbuf((size_t)NL * BN * (R ? R : 1));
     const bool gemma = s->model_type == MODEL_GEMMA3;
     s->o_raw = gemma ? fbuf((size_t)NL * xsz) : nullptr; s->ff_raw = gemma ? fbuf((size_t)NL * xsz) : nullptr;
@@ -778,7 +783,7 @@ void sft_state_free(SFTState *s)
                        s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
-                       s->gate_pre, s->up_val, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->group_inv, s->ones, s->planes,
+                       s->gu_sav, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->group_inv, s->ones, s->planes,
                        s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
                        s->dq, s->dk, s->dv, s->dq_f, s->dh, s->ce_part,
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
