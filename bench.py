@@ -160,6 +160,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="c3_qwen3_4b_f16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seq", type=int, default=0, help="override the configuration's sequence length (experiments only)")
+    ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch (experiments only)")
     ap.add_argument("--decode", action="store_true",
                     help="time greedy token-by-token generation (include/inference_hip.h) on the configuration's model "
                          "instead of the training step: a step is one token")
@@ -175,6 +177,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     cfg = CONFIGS[args.config]
+    if args.seq or args.batch:
+        cfg = cfg.with_(seq=args.seq or cfg.seq, batch=args.batch or cfg.batch)
 
     from llm_metal_amd import lib
     from llm_metal_amd.sft import SFTState
