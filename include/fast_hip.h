@@ -163,6 +163,10 @@ void hip_gemm_force_large_m(int policy);
  * rule (three chunks when the 128 x 256 output blocks leave a third of the CUs idle and K >= 4096), 0 = never, n > 1 =
  * always n. */
 void hip_gemm_large_m_split(int mode);
+/* Training attention without the [seq, seq] probability matrices in memory (running softmax in the forward, the
+ * probabilities formed again in the backward): -1 = for head_dim 64 / 128 and sequences of at least 128 positions
+ * (default), 0 = never, 1 = whenever the head size allows.  Read when a training state is created. */
+void hip_attention_flash(int mode);
 /* Timing aid for benchmarks: when enabled, every GEMM launch is bracketed by HIP events on the
  * library's stream.  hip_gemm_profile_read (after metal_flush) returns the number of launches recorded
  * since the last enable and adds up their durations (ms) and weight bytes; _read2 also their flops. */

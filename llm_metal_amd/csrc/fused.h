@@ -105,6 +105,28 @@ bool attn_mfma_supported(int hd, int seq);
 void launch_attn_fwd_mfma(const AttnFwdArgs &a);
 void launch_attn_bwd_mfma(const AttnBwdArgs &a);
 
+// The same attention without the [seq, seq] matrices in memory (attn_flash.hip): head_dim 64 or 128, any sequence
+// length.  The forward saves the operands of the backward (bf16-pair fragments of q, k, v), the output and one
+// number per query row; the backward needs the window again (nothing saved carries it).
+struct AttnFlashArgs {
+    const float *q, *k, *v;       // forward: [rows][Hq*hd], [rows][Hkv*hd] x2 (post-RoPE)
+    Planes dO;                    // backward: [rows][Hq*hd]
+    int Hq, Hkv, hd, seq, batch, window; float scale;
+    uint4 *q_rt, *q_pt, *k_rt, *k_pt, *v_rt, *v_pt;    // written by the forward, attn_flash_tile_elems() each
+    uint4 *do_rt, *do_pt;         // backward scratch, as q_rt
+    float *O, *lse;               // written by the forward: [rows][Hq*hd], [batch][Hq][ceil(seq/32)*32]
+    float *D;                     // backward scratch, as lse
+    half_t *out16;                // forward: tiled [rows, Hq*hd], unit scale
+    float *dq, *dk, *dv;          // backward: [rows][Hq*hd], [rows][Hkv*hd] x2
+    float *dkp, *dvp;             // backward scratch: [Hq/Hkv][rows][Hkv*hd] each
+};
+// -1: head_dim 64/128 and at least 128 positions (default); 0: never; 1: whenever the head size allows
+void set_attn_flash_mode(int mode);
+bool attn_flash_supported(int hd, int seq, int Hq, int Hkv);
+size_t attn_flash_tile_elems(int hd, int seq, int heads, int batch);     // 16-byte elements of one RT or PT image
+void launch_attn_fwd_flash(const AttnFlashArgs &a);
+void launch_attn_bwd_flash(const AttnFlashArgs &a);
+
 struct QkvBwdArgs {
     const float *dq, *dk, *dv;    // post-RoPE-domain gradients
     const float *q_pre, *k_pre, *g_q, *g_k; float eps;

@@ -62,6 +62,10 @@ struct SFTState {
     MetalBuf *ln1_16, *ln1_inv;          // [NL][BN*D] f16, [NL][BN]
     MetalBuf *q_pre, *k_pre, *q_fin, *k_fin, *v_sav, *probs, *gu_sav, *tq, *tv, *o_raw, *ff_raw;   // gu_sav: [NL][BN][gate (IS) | up (IS)]
     MetalBuf *kT, *vT;                   // k_fin / v_sav once more, per head and transposed, for the matrix-core attention
+    // attention without saved probabilities (attn_flash.hip; probs, kT, vT, dO_red, dscore are then not allocated):
+    // per layer the bf16-pair fragments of q, k, v ([RT | PT] each), the output and the row statistics
+    int use_flash;
+    MetalBuf *fa_q, *fa_k, *fa_v, *fa_O, *fa_lse, *fa_do, *fa_D, *fa_dkp, *fa_dvp;
     // transients
     MetalBuf *a16, *a16_inv;             // largest fp16 operand (BN x max K) and its row factors
     MetalBuf *group_inv;                 // row factors per column group [BN][MAX_SCALE_GROUPS]: never the buffer the
@@ -224,6 +228,24 @@ WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int th
     return pf;
 }
 
+// The flash attention's buffers of layer L
+AttnFlashArgs flash_args(SFTState *s, int L)
+{
+    AttnFlashArgs f{};
+    const size_t eq = attn_flash_tile_elems(s->hd, s->N, s->Hq, s->B), ek = attn_flash_tile_elems(s->hd, s->N, s->Hkv, s->B);
+    const size_t stat = (size_t)s->B * s->Hq * ((s->N + 31) / 32) * 32;
+    f.Hq = s->Hq; f.Hkv = s->Hkv; f.hd = s->hd; f.seq = s->N; f.batch = s->B;
+    f.window = (s->window > 0 && s->layer_local[L]) ? s->window : 0;
+    f.scale = 1.0f / sqrtf((float)s->hd);
+    f.q_rt = at<uint4>(s->fa_q, (size_t)L * 2 * eq); f.q_pt = f.q_rt + eq;
+    f.k_rt = at<uint4>(s->fa_k, (size_t)L * 2 * ek); f.k_pt = f.k_rt + ek;
+    f.v_rt = at<uint4>(s->fa_v, (size_t)L * 2 * ek); f.v_pt = f.v_rt + ek;
+    f.do_rt = at<uint4>(s->fa_do); f.do_pt = f.do_rt + eq;
+    f.O = at<float>(s->fa_O, (size_t)L * s->BN * s->qd); f.lse = at<float>(s->fa_lse, (size_t)L * stat); f.D = at<float>(s->fa_D);
+    f.dkp = at<float>(s->fa_dkp); f.dvp = at<float>(s->fa_dvp);
+    return f;
+}
+
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr,
             const ScaleGroups *sg = nullptr)
@@ -301,15 +323,21 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
         if (s->kT) { qa.kT = at<float>(s->kT, (size_t)L * st_kt); qa.vT = at<float>(s->vT, (size_t)L * st_kt); }
         // causal GQA attention                                               [:678-689]
         half_t *attn16 = s->full_param ? at<half_t>(s->attn16, L * s->st_attn) : a16;
-        float *probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
+        float *probs = s->probs ? at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N) : nullptr;
         const float attn_scale = 1.0f / sqrtf((float)s->hd);
         launch_qkv_post(qa, BN);
+        if (s->use_flash) {
+            AttnFlashArgs f = flash_args(s, L);
+            f.q = qa.q_fin; f.k = qa.k_fin; f.v = qa.v_out; f.out16 = attn16;
+            launch_attn_fwd_flash(f);
+        }
         AttnFwdArgs aa{};
         aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
         aa.scale = attn_scale; aa.probs = probs; aa.out16 = attn16; aa.kT = qa.kT;
         aa.window = (s->window > 0 && s->layer_local[L]) ? s->window : 0;
-        if (attn_mfma_supported(s->hd, s->N)) {
+        if (s->use_flash) {
+        } else if (attn_mfma_supported(s->hd, s->N)) {
             aa.pf = prefetch_for(s, wop(s, W_O, L, false), D, qd, 256, ((s->N + 31) / 32) * s->Hq);
             launch_attn_fwd_mfma(aa);
         } else launch_attn_fwd(aa);
@@ -446,16 +474,21 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
                         s->wo, s->woT, s->go, L * s->st_o, L * s->st_oT);
         AttnBwdArgs ab{};
         ab.dO = pdo;
-        ab.probs = at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N);
+        ab.probs = s->probs ? at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N) : nullptr;
         ab.q = at<float>(s->q_fin, (size_t)L * BN * qd); ab.k = at<float>(s->k_fin, (size_t)L * BN * kd);
         ab.v = at<float>(s->v_sav, (size_t)L * BN * kd);
         ab.Hq = s->Hq; ab.Hkv = s->Hkv; ab.hd = s->hd; ab.seq = s->N; ab.batch = s->B;
         ab.scale = 1.0f / sqrtf((float)s->hd);
         ab.vT = s->vT ? at<float>(s->vT, (size_t)L * s->B * kd * attn_ldt(s->N)) : nullptr;
-        ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore);
+        if (!s->use_flash) { ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore); }
         const size_t keepL = R ? (size_t)L : 0;                 // LoRA mode keeps dv, dq_f and dh of every layer
         ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv, keepL * BN * kd);
-        if (attn_mfma_supported(s->hd, s->N)) launch_attn_bwd_mfma(ab); else launch_attn_bwd(ab);
+        if (s->use_flash) {
+            AttnFlashArgs f = flash_args(s, L);
+            f.dO = pdo; f.dq = ab.dq; f.dk = ab.dk; f.dv = ab.dv;
+            launch_attn_bwd_flash(f);
+        } else if (attn_mfma_supported(s->hd, s->N)) launch_attn_bwd_mfma(ab);
+        else launch_attn_bwd(ab);
 
         // inverse RoPE, QK-norm backward, dh; LoRA gradients                  [:912-966]
         QkvBwdArgs qb{};
@@ -723,8 +756,16 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->ln1_16 = hbuf((size_t)NL * s->st_ln1); s->ln1_inv = fbuf((size_t)NL * BN);
     s->q_pre = fbuf((size_t)NL * BN * qd); s->k_pre = fbuf((size_t)NL * BN * kd);
     s->q_fin = fbuf((size_t)NL * BN * qd); s->k_fin = fbuf((size_t)NL * BN * kd); s->v_sav = fbuf((size_t)NL * BN * kd);
-    s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
-    if (attn_mfma_supported(s->hd, s->N)) {
+    s->use_flash = attn_flash_supported(s->hd, s->N, s->Hq, s->Hkv);
+    if (s->use_flash) {
+        const size_t eq = attn_flash_tile_elems(s->hd, s->N, s->Hq, s->B), ek = attn_flash_tile_elems(s->hd, s->N, s->Hkv, s->B);
+        const size_t stat = (size_t)s->B * s->Hq * ((s->N + 31) / 32) * 32;
+        s->fa_q = metal_buf_create((size_t)NL * 2 * eq * 16); s->fa_k = metal_buf_create((size_t)NL * 2 * ek * 16);
+        s->fa_v = metal_buf_create((size_t)NL * 2 * ek * 16); s->fa_do = metal_buf_create(2 * eq * 16);
+        s->fa_O = fbuf((size_t)NL * BN * qd); s->fa_lse = fbuf((size_t)NL * stat); s->fa_D = fbuf(stat);
+        s->fa_dkp = fbuf((size_t)(s->Hq / s->Hkv) * BN * kd); s->fa_dvp = fbuf((size_t)(s->Hq / s->Hkv) * BN * kd);
+    } else s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
+    if (!s->use_flash && attn_mfma_supported(s->hd, s->N)) {
         s->kT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N)); s->vT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N));
     }
     s->gu_sav = fbuf((size_t)NL * BN * 2 * IS);
@@ -743,7 +784,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->logits = fbuf((size_t)BN * V); s->dlogits = nullptr;
     s->dl16 = hbuf(tiled_elems(BN, V)); s->dl_inv = fbuf(BN);
     s->dx[0] = fbuf(xsz); s->dx[1] = fbuf(xsz);
-    s->dO_red = fbuf((size_t)BN * qd); s->dscore = fbuf((size_t)s->B * s->Hq * s->N * s->N);
+    if (!s->use_flash) { s->dO_red = fbuf((size_t)BN * qd); s->dscore = fbuf((size_t)s->B * s->Hq * s->N * s->N); }
     const size_t keep = R ? NL : 1;
     s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf(keep * BN * kd);
     s->dq_f = fbuf(keep * BN * qd); s->dh = fbuf(keep * BN * (R ? 2 * R : 1));
@@ -788,7 +829,8 @@ void sft_state_free(SFTState *s)
                        s->dq, s->dk, s->dv, s->dq_f, s->dh, s->ce_part,
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
                        s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
-                       s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf};
+                       s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf,
+                       s->fa_q, s->fa_k, s->fa_v, s->fa_O, s->fa_lse, s->fa_do, s->fa_D, s->fa_dkp, s->fa_dvp};
     for (MetalBuf *b : s->views_out) metal_buf_free(b);
     for (MetalBuf *b : all) metal_buf_free(b);
     for (WMat &w : s->wmats_out) metal_buf_free(w.mbuf);

@@ -61,6 +61,20 @@ CASES = [
     TINY_GEMMA3.with_(name="gemma_window8", window=8),
     C1.with_(name="window_seq300", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
     C1.with_(name="window7_small_heads", NL=1, D=64, Hq=4, Hkv=2, hd=16, IS=96, V=512, seq=40, window=7),
+    # attention without saved probabilities (running softmax, probabilities formed again in the backward), which the
+    # measured rule takes from 128 positions on ("seq512", "seq300_hd128", "window_seq300", "gemma_many_rows" above):
+    # forced on for short and ragged sequences, several sequences per batch, one KV head for four query heads, windows
+    # that cut inside a 32-key block and that skip whole blocks; and forced off ("_noflash") so that the long sequences
+    # keep covering the kernels with saved probabilities
+    C1.with_(name="c1_flash"),
+    C1.with_(name="hd128_flash", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
+    C1.with_(name="ragged_seq40_flash", NL=2, batch=2, seq=40, R=4, alpha=8.0),
+    C1.with_(name="seq17_mqa_flash", NL=1, Hq=4, Hkv=1, seq=17, V=1024),
+    C1.with_(name="c1_batch3_flash", batch=3, seq=32),
+    C1.with_(name="window24_flash", window=24),
+    C1.with_(name="seq333_window50_flash", NL=1, batch=2, seq=333, V=1024, window=50),
+    C1.with_(name="seq512_noflash", NL=1, seq=512, V=1024),
+    C1.with_(name="window_seq300_noflash", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
     # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
     TINY_GEMMA3.with_(name="gemma_many_rows", NL=2, batch=4, seq=128),
 ]
@@ -90,6 +104,7 @@ def test_train_steps_match_oracle(cfg):
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
     lib.load().hip_gemm_force_large_m(2 if cfg.name.endswith("_lds") else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
+    lib.load().hip_attention_flash(1 if cfg.name.endswith("_flash") else 0 if cfg.name.endswith("_noflash") else -1)
     with SFTState(cfg, model) as st:
         for i, (tok, tgt) in enumerate(batches):
             loss = st.train_step(tok, tgt, lr)
@@ -113,6 +128,7 @@ def test_train_steps_match_oracle(cfg):
         assert (np.sign(d_gpu) == np.sign(d_ref)).mean() > 0.97
     lib.load().hip_gemm_force_large_m(0)
     lib.load().hip_gemm_large_m_split(1)
+    lib.load().hip_attention_flash(-1)
 
 
 def test_q8_tiles_hold_the_dequantised_values_in_both_images():
