@@ -163,6 +163,10 @@ void hip_gemm_force_large_m(int policy);
  * rule (three chunks when the 128 x 256 output blocks leave a third of the CUs idle and K >= 4096), 0 = never, n > 1 =
  * always n. */
 void hip_gemm_large_m_split(int mode);
+/* A training state with frozen Q8_0 weights whose products run on the large-M kernel keeps the F16 image of every
+ * weight it has used (made once instead of once per product) when the images of all its weights fit this many MB
+ * (default 65536; the 4B model needs 16 GB); 0 = never keep them. */
+void hip_gemm_image_budget_mb(int mb);
 /* Training attention without the [seq, seq] probability matrices in memory (running softmax in the forward, the
  * probabilities formed again in the backward): -1 = for head_dim 64 / 128 and sequences of at least 128 positions
  * (default), 0 = never, 1 = whenever the head size allows.  Read when a training state is created. */

@@ -72,7 +72,10 @@ double weight_stream_bytes(const WeightOp &W, int N, int K);
 // C[m][n] (row stride ldc) = a_inv_scale[m] * sum_k A[m][k] W[n][k] in one launch of 128 x 128 output blocks staged
 // through LDS (gemm_big.hip): the path for M of several hundred rows and more, where the product is MFMA bound.
 // W as plain F16 tiles: itself when F16, else dequantised once into a scratch image that the next call overwrites
-WeightOp f16_image_of(const WeightOp &W, int N, int K);
+// `keep`: the image goes there (tiled_elems(N, K) halves, the caller's) instead of the scratch arena; with
+// f16_part_only only the tiles that are F16 in W are written (the Q8_0 part of `keep` holds its image from before).
+WeightOp f16_image_of(const WeightOp &W, int N, int K, void *keep = nullptr, bool f16_part_only = false);
+bool large_m_unpacks_q8();                                // the large-M policy that reads Q8_0 tiles itself is in force
 // chunks > 1 (F16 tiles only): the K steps are cut into that many chunks, chunk c writing the plane at C + c * plane_stride;
 // big_gemm_chunks: what the measured rule picks for a product
 int big_gemm_chunks(int M, int N, int K, int fmt);

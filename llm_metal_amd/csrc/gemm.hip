@@ -103,12 +103,14 @@ __global__ void reduce_planes(const float *__restrict__ P, int S, size_t plane_s
 // F16 tile image of a Q8_0 (or mixed Q8_0 / F16) weight operand: one wave per 32 x 64 tile loads the tile the way
 // the streaming GEMM does (codes unpacked and scaled in registers, F16 tiles as they are) and stores the four operand
 // vectors of every lane at the tile's place in a plain F16 operand, out[(nb * Kb + kt) * 256 + j * 64 + lane].
-__global__ __launch_bounds__(256) void q8_operand_to_f16(lmhip::WeightOp W, int Nb, int Kb, half8 *__restrict__ out)
+// f16_only: only the tiles that are F16 in W (adapter rows of a fused matrix) are copied; the rest of `out` is kept.
+__global__ __launch_bounds__(256) void q8_operand_to_f16(lmhip::WeightOp W, int Nb, int Kb, half8 *__restrict__ out, int f16_only)
 {
     const int lane = threadIdx.x & 63;
     const size_t tile = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (tile >= (size_t)Nb * Kb) return;
     const int nb = (int)(tile / Kb), kt = (int)(tile % Kb);
+    if (f16_only && (W.fmt == 1 ? nb < W.nbq : kt < W.kbq)) return;
     half8 w[4];
     if (W.fmt == 1) {
         if (nb < W.nbq) lmhip::load_w_q8_rows(w, W, nb, Kb, kt, lane);
@@ -359,16 +361,19 @@ bool use_big_gemm(int M, int N, int K, int fmt)
 
 // The operand as plain F16 tiles: W itself when it is F16, else an image in the library's scratch arena (valid until
 // the next call).
-WeightOp f16_image_of(const WeightOp &W, int N, int K)
+WeightOp f16_image_of(const WeightOp &W, int N, int K, void *keep, bool f16_part_only)
 {
     if (W.fmt == 0 || g_big_policy == 2) return W;        // policy 2: the large-M kernel unpacks the Q8_0 tiles into LDS itself
     const int Nb = tiled_rb(N), Kb = tiled_kb(K);
     const size_t tiles = (size_t)Nb * Kb;
-    half8 *img = (half8 *)scratch(SCR_WF16, tiles * 256 * sizeof(half8));
-    hipLaunchKernelGGL(q8_operand_to_f16, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, stream(), W, Nb, Kb, img);
-    HIP_CHECK(hipGetLastError());
+    half8 *img = keep ? (half8 *)keep : (half8 *)scratch(SCR_WF16, tiles * 256 * sizeof(half8));
+    if (!(f16_part_only && !W.w16)) {
+        hipLaunchKernelGGL(q8_operand_to_f16, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, stream(), W, Nb, Kb, img, f16_part_only ? 1 : 0);
+        HIP_CHECK(hipGetLastError());
+    }
     return weight_f16(reinterpret_cast<const half_t *>(img));
 }
+bool large_m_unpacks_q8() { return g_big_policy == 2; }
 
 bool gemm_prof_begin(double wbytes, double flops, hipEvent_t *a, hipEvent_t *b)
 {

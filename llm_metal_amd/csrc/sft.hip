@@ -18,6 +18,7 @@
 #include <math.h>
 #include <string.h>
 #include <vector>
+#include <unordered_map>
 
 using namespace lmhip;
 
@@ -89,6 +90,11 @@ struct SFTState {
     MetalBuf *grpo_old_lp, *grpo_advs, *grpo_new_lp;   // host-visible [BN] inputs/outputs of the policy gradient
     float *grpo_old_lp_cpu, *grpo_advs_cpu, *grpo_new_lp_cpu;
     MetalBuf *lora_acc;                  // LoRA gradients summed over the completions of a GRPO group
+    // Q8_0 states whose products run on the large-M kernel keep the F16 image of every frozen weight they have used
+    // (dequantised once, not once per product), as long as all of them fit the budget
+    std::unordered_map<const void *, half_t *> img_slots;
+    MetalBuf *img_arena;
+    size_t img_used, img_cap;
     int step_in_flight, step_rejected;   // sft_enqueue_train_step without its sft_finish_train_step yet; ids refused
     std::vector<LayerW> layers_out;      // row-major F16 copies handed out by sft_get_layers
     std::vector<WMat> wmats_out;
@@ -246,13 +252,40 @@ AttnFlashArgs flash_args(SFTState *s, int L)
     return f;
 }
 
+// F16 tiles of a weight for the large-M kernel.  A Q8_0 weight of a LoRA state is frozen, so its image is made once
+// and kept (16 GB for the 4B model's two orientations; MI355X has the room, and the product then reads what it would
+// read anyway); only the adapter rows of the fused QKV matrix, which every step changes, are copied again.  Without
+// room within the budget for all the state's weights the image is made per product in the scratch arena.
+size_t g_image_budget = (size_t)64 << 30;
+WeightOp resident_image(SFTState *s, const WeightOp &W, int N, int K)
+{
+    if (W.fmt == 0 || s->full_param || large_m_unpacks_q8() || !g_image_budget) return f16_image_of(W, N, K);
+    if (!s->img_arena) {
+        if (s->img_cap == (size_t)-1) return f16_image_of(W, N, K);            // found too large before
+        const int NL = s->NL;
+        size_t need = 0;
+        const int shp[5][2] = {{s->nq_ext, s->D}, {s->D, s->qd}, {2 * s->IS, s->D}, {s->D, s->IS}, {s->V, s->D}};
+        for (int k = 0; k < 5; k++) need += (tiled_elems(shp[k][0], shp[k][1]) + tiled_elems(shp[k][1], shp[k][0])) * (k == 4 ? 1 : NL);
+        if (need * sizeof(half_t) > g_image_budget) { s->img_cap = (size_t)-1; return f16_image_of(W, N, K); }
+        s->img_arena = hbuf(need); s->img_cap = need; s->img_used = 0;
+    }
+    auto it = s->img_slots.find(W.q);
+    if (it != s->img_slots.end()) return f16_image_of(W, N, K, it->second, true);
+    const size_t elems = tiled_elems(N, K);
+    if (s->img_used + elems > s->img_cap) return f16_image_of(W, N, K);
+    half_t *slot = at<half_t>(s->img_arena, s->img_used);
+    s->img_used += elems;
+    s->img_slots.emplace(W.q, slot);
+    return f16_image_of(W, N, K, slot, false);
+}
+
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr,
             const ScaleGroups *sg = nullptr)
 {
     if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch; final output, or a few K chunks as planes
         float *C = out ? out : at<float>(s->planes);
-        const WeightOp Wf = f16_image_of(W, N, K);
+        const WeightOp Wf = resident_image(s, W, N, K);
         const int chunks = out ? 1 : big_gemm_chunks(s->BN, N, K, Wf.fmt);
         const size_t stride = (size_t)s->BN * N;
         if (!out && chunks * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
@@ -830,7 +863,7 @@ void sft_state_free(SFTState *s)
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
                        s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
                        s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf,
-                       s->fa_q, s->fa_k, s->fa_v, s->fa_O, s->fa_lse, s->fa_do, s->fa_D, s->fa_dkp, s->fa_dvp};
+                       s->fa_q, s->fa_k, s->fa_v, s->fa_O, s->fa_lse, s->fa_do, s->fa_D, s->fa_dkp, s->fa_dvp, s->img_arena};
     for (MetalBuf *b : s->views_out) metal_buf_free(b);
     for (MetalBuf *b : all) metal_buf_free(b);
     for (WMat &w : s->wmats_out) metal_buf_free(w.mbuf);
@@ -1051,6 +1084,8 @@ MetalBuf *sft_get_lora_weight_buf(SFTState *s, int layer, int sub)
     return i < s->lora_views.size() ? s->lora_views[i] : nullptr;
 }
 float sft_get_lora_scaling(SFTState *s) { return s->lora_scaling; }
+
+void hip_gemm_image_budget_mb(int mb) { g_image_budget = mb > 0 ? (size_t)mb << 20 : 0; }
 
 // Sliding-window attention on the local layers.  The reference stores Gemma3's window (src/nn/gemma3.c:20, 99) and
 // never applies it: its attention kernels see every earlier key on every layer (shaders/q8_kernels.metal:769-855), which

@@ -49,6 +49,7 @@ CASES = [
     C1.with_(name="big_m_f16_chunks", batch=5, seq=40),
     C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
+    C1.with_(name="big_m_q8_noimg", NL=1, batch=2, seq=160, weight_format="q8_0"),      # no room to keep the images: made per product
     C1.with_(name="big_m_q8_lds", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8_lds", NL=2, batch=3, seq=100, weight_format="q8_0"),
     # a wide FFN: the GLU kernels split each row into column groups of two (forward) and four (backward) K chunks with
@@ -105,6 +106,7 @@ def test_train_steps_match_oracle(cfg):
     lib.load().hip_gemm_force_large_m(2 if cfg.name.endswith("_lds") else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
     lib.load().hip_attention_flash(1 if cfg.name.endswith("_flash") else 0 if cfg.name.endswith("_noflash") else -1)
+    lib.load().hip_gemm_image_budget_mb(0 if cfg.name.endswith("_noimg") else 65536)
     with SFTState(cfg, model) as st:
         for i, (tok, tgt) in enumerate(batches):
             loss = st.train_step(tok, tgt, lr)
@@ -129,6 +131,7 @@ def test_train_steps_match_oracle(cfg):
     lib.load().hip_gemm_force_large_m(0)
     lib.load().hip_gemm_large_m_split(1)
     lib.load().hip_attention_flash(-1)
+    lib.load().hip_gemm_image_budget_mb(65536)
 
 
 def test_q8_tiles_hold_the_dequantised_values_in_both_images():
