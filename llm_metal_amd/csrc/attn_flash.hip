@@ -140,6 +140,136 @@ __global__ __launch_bounds__(256) void k_fa_split(FaSplitArgs a)
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// The QKV epilogue for this attention: what k_qkv_post does (plane sums, LoRA term sc * (x A^T) B^T, pre-norm copy,
+// per-head RMSNorm, half-split RoPE; src/nn/fast_sft.c:639-669, shaders/q8_kernels.metal:495-538) on a tile of 32
+// positions of one head, which then leaves the workgroup as the RT and PT fragments directly: no fp32 copy of the
+// final q, k, v is written and read again.  grid (blocks of 32 positions, Hq + 2 Hkv, batch), block 256.
+// RK: the LoRA rank compiled in (16), or -1 for any rank up to 64 (0 included).
+template <int HD, int RK>
+__global__ __launch_bounds__(256) void k_qkv_post_tile(QkvPostArgs a, uint4 *q_rt, uint4 *q_pt, uint4 *k_rt, uint4 *k_pt, uint4 *v_rt, uint4 *v_pt, int batch)
+{
+    constexpr int LDS_LD = HD + 4, NJ = HD / 16, TILE = HD / 8 * 64, TPR = HD / 4, HALF = HD / 2;
+    __shared__ float Xs[32 * LDS_LD];
+    __shared__ float Ts[32 * 64];
+    __shared__ float Inv[32];
+    const int blk = blockIdx.x, slot = blockIdx.y, b = blockIdx.z, nblk = gridDim.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l31 = lane & 31, hh = lane >> 5;
+    const int N = a.seq, qd = a.Hq * HD, kd = a.Hkv * HD, R = RK >= 0 ? RK : a.R;
+    const int kind = slot < a.Hq ? 0 : (slot < a.Hq + a.Hkv ? 1 : 2);     // 0 q, 1 k, 2 v
+    const int h = kind == 0 ? slot : (kind == 1 ? slot - a.Hq : slot - a.Hq - a.Hkv);
+    const int col0 = kind == 0 ? h * HD : (kind == 1 ? qd + h * HD : qd + kd + h * HD);
+    const int t0 = qd + 2 * kd + (kind == 2 ? R : 0);
+    const bool lora = R > 0 && kind != 1;
+    const size_t r0 = (size_t)b * N;
+    {   // ---- the tile and its rows of x A^T
+        float4 xv[HD / 32];
+        size_t rows[HD / 32]; int cols[HD / 32]; bool ok[HD / 32];
+#pragma unroll
+        for (int u = 0; u < HD / 32; u++) {
+            const int idx = tid + 256 * u, rr = idx / TPR, c4 = idx % TPR;
+            ok[u] = blk * 32 + rr < N; rows[u] = r0 + (ok[u] ? blk * 32 + rr : 0); cols[u] = col0 + 4 * c4;
+        }
+        planes_at4_multi<HD / 32, (HD <= 128 ? 5 : 3)>(a.qkv, rows, cols, ok, xv);
+#pragma unroll
+        for (int u = 0; u < HD / 32; u++) { const int idx = tid + 256 * u; st4(Xs + (idx / TPR) * LDS_LD + 4 * (idx % TPR), xv[u]); }
+        if (lora)
+            for (int idx = tid; idx < 32 * R; idx += 256) {
+                const int rr = idx / R, k = idx % R;
+                const bool okr = blk * 32 + rr < N;
+                const float t = okr ? planes_at(a.qkv, r0 + blk * 32 + rr, t0 + k) : 0.f;
+                Ts[rr * 64 + k] = t;
+                if (okr && h == 0) (kind == 0 ? a.tq : a.tv)[(r0 + blk * 32 + rr) * R + k] = t;
+            }
+    }
+    __syncthreads();
+    {   // ---- LoRA term, pre-norm copy: a thread owns one column of HD for 32 * HD / 256 rows
+        constexpr int PARTS = 256 / HD, RPP = 32 / PARTS;
+        const int d = tid % HD, part = tid / HD;
+        float *pre = kind == 0 ? a.q_pre : a.k_pre;
+        const int W = kind == 0 ? qd : kd;
+        if (lora) {
+            const float *B = (kind == 0 ? a.Bq : a.Bv) + (size_t)(h * HD + d) * R;
+            if constexpr (RK == 16) {
+                float4 w[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) w[i] = ld4(B + 4 * i);
+#pragma unroll
+                for (int q = 0; q < RPP; q++) {
+                    const int rr = part * RPP + q;
+                    const float *t = Ts + rr * 64;
+                    float acc = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) { acc += t[4 * i] * w[i].x; acc += t[4 * i + 1] * w[i].y; acc += t[4 * i + 2] * w[i].z; acc += t[4 * i + 3] * w[i].w; }
+                    Xs[rr * LDS_LD + d] += a.sc * acc;
+                }
+            } else {
+                for (int q = 0; q < RPP; q++) {
+                    const int rr = part * RPP + q;
+                    float acc = 0.f;
+                    for (int k = 0; k < R; k++) acc += Ts[rr * 64 + k] * B[k];
+                    Xs[rr * LDS_LD + d] += a.sc * acc;
+                }
+            }
+        }
+        if (kind != 2)
+#pragma unroll
+            for (int q = 0; q < RPP; q++) {
+                const int rr = part * RPP + q;
+                if (blk * 32 + rr < N) pre[(r0 + blk * 32 + rr) * W + h * HD + d] = Xs[rr * LDS_LD + d];
+            }
+    }
+    __syncthreads();
+    if (kind != 2) {
+        {   // ---- 1 / rms of every row: eight threads per row
+            const int rr = tid >> 3, part = tid & 7;
+            float ss = 0.f;
+#pragma unroll
+            for (int c = 0; c < HD / 32; c++) { const float4 v = ld4(Xs + rr * LDS_LD + 32 * c + 4 * part); ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+            ss += __shfl_xor(ss, 1, WAVE); ss += __shfl_xor(ss, 2, WAVE); ss += __shfl_xor(ss, 4, WAVE);
+            if (part == 0) Inv[rr] = rsqrtf(ss / (float)HD + a.eps);
+        }
+        __syncthreads();
+        {   // ---- weight, RoPE on the pairs (d, d + HD/2): a thread owns one pair for 32 * HALF / 256 rows
+            constexpr int PARTS = 256 / HALF, RPP = 32 / PARTS;
+            const int d = tid % HALF, part = tid / HALF;
+            const float *g = kind == 0 ? a.g_q : a.g_k;
+            const float g0 = g[d], g1 = g[d + HALF];
+#pragma unroll
+            for (int q = 0; q < RPP; q++) {
+                const int rr = part * RPP + q, pos = blk * 32 + rr;
+                if (pos >= N) continue;
+                const float inv = Inv[rr];
+                const float n0 = Xs[rr * LDS_LD + d] * inv * g0, n1 = Xs[rr * LDS_LD + d + HALF] * inv * g1;
+                const float2 cs = a.rope[(size_t)pos * HALF + d];
+                Xs[rr * LDS_LD + d] = n0 * cs.x - n1 * cs.y;
+                Xs[rr * LDS_LD + d + HALF] = n0 * cs.y + n1 * cs.x;
+            }
+        }
+        __syncthreads();
+    }
+    // ---- the tile as fragments
+    const int H = kind == 0 ? a.Hq : a.Hkv;
+    const size_t tile = (((size_t)b * H + h) * nblk + blk) * TILE + lane;
+    uint4 *rt = (kind == 0 ? q_rt : kind == 1 ? k_rt : v_rt) + tile, *pt = (kind == 0 ? q_pt : kind == 1 ? k_pt : v_pt) + tile;
+    for (int p = wave; p < HD / 8; p += 4) {
+        if (p < NJ) {
+            const float *src = Xs + l31 * LDS_LD + 16 * p + 8 * hh;
+            const HL f = split8(ld4(src), ld4(src + 4));
+            rt[(2 * p) * 64] = __builtin_bit_cast(uint4, f.hi);
+            rt[(2 * p + 1) * 64] = __builtin_bit_cast(uint4, f.lo);
+        } else {
+            const int q = p - NJ, db = q >> 1, u = q & 1;
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = Xs[pt_row(u, hh, e) * LDS_LD + 32 * db + l31];
+            const HL f = split8(x);
+            pt[(2 * q) * 64] = __builtin_bit_cast(uint4, f.hi);
+            pt[(2 * q + 1) * 64] = __builtin_bit_cast(uint4, f.lo);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 struct FaArgs {
     const uint4 *q_rt, *q_pt, *k_rt, *k_pt, *v_rt, *v_pt, *do_rt, *do_pt;
     int Hq, Hkv, seq, batch, window;
@@ -571,14 +701,32 @@ size_t attn_flash_tile_elems(int hd, int seq, int heads, int batch)
     return (size_t)batch * heads * ((seq + 31) / 32) * (hd / 8) * 64;       // uint4 (16 bytes) each
 }
 
+template <int HD>
+void qkv_post_hd(const QkvPostArgs &a, const AttnFlashArgs &f)
+{
+    const dim3 grid((f.seq + 31) / 32, a.Hq + 2 * a.Hkv, f.batch);
+    if (a.R == 16) LAUNCH((k_qkv_post_tile<HD, 16>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+    else LAUNCH((k_qkv_post_tile<HD, -1>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+}
+
+void launch_qkv_post_flash(const QkvPostArgs &a, const AttnFlashArgs &f)
+{
+    if (!(f.hd == 64 || f.hd == 128) || a.hd != f.hd || a.R < 0 || a.R > 64 || (a.R & 1) || a.qkv.scale_groups || (a.qkv.ld & 3) || a.seq != f.seq) {
+        fprintf(stderr, "[fast_hip] qkv_post_flash: unsupported shape (hd %d, rank %d)\n", a.hd, a.R); abort();
+    }
+    if (f.hd == 64) qkv_post_hd<64>(a, f); else qkv_post_hd<128>(a, f);
+}
+
 void launch_attn_fwd_flash(const AttnFlashArgs &f)
 {
     if (!(f.hd == 64 || f.hd == 128)) { fprintf(stderr, "[fast_hip] attn_fwd_flash: unsupported head size %d\n", f.hd); abort(); }
-    FaSplitArgs sp{};
-    sp.seq = f.seq; sp.batch = f.batch;
-    sp.X = f.q; sp.ldx = (size_t)f.Hq * f.hd; sp.H = f.Hq; sp.rt = f.q_rt; sp.pt = f.q_pt; split(sp, f.hd);
-    sp.X = f.k; sp.ldx = (size_t)f.Hkv * f.hd; sp.H = f.Hkv; sp.rt = f.k_rt; sp.pt = f.k_pt; split(sp, f.hd);
-    sp.X = f.v; sp.rt = f.v_rt; sp.pt = f.v_pt; split(sp, f.hd);
+    if (f.q) {                                            // fp32 q, k, v given: split them here (else launch_qkv_post_flash has)
+        FaSplitArgs sp{};
+        sp.seq = f.seq; sp.batch = f.batch;
+        sp.X = f.q; sp.ldx = (size_t)f.Hq * f.hd; sp.H = f.Hq; sp.rt = f.q_rt; sp.pt = f.q_pt; split(sp, f.hd);
+        sp.X = f.k; sp.ldx = (size_t)f.Hkv * f.hd; sp.H = f.Hkv; sp.rt = f.k_rt; sp.pt = f.k_pt; split(sp, f.hd);
+        sp.X = f.v; sp.rt = f.v_rt; sp.pt = f.v_pt; split(sp, f.hd);
+    }
     FaArgs a{};
     a.q_rt = f.q_rt; a.k_rt = f.k_rt; a.v_pt = f.v_pt;
     a.Hq = f.Hq; a.Hkv = f.Hkv; a.seq = f.seq; a.batch = f.batch; a.window = f.window;

@@ -124,7 +124,11 @@ struct AttnFlashArgs {
 void set_attn_flash_mode(int mode);
 bool attn_flash_supported(int hd, int seq, int Hq, int Hkv);
 size_t attn_flash_tile_elems(int hd, int seq, int heads, int batch);     // 16-byte elements of one RT or PT image
+// q, k, v null: the fragments are there already (launch_qkv_post_flash)
 void launch_attn_fwd_flash(const AttnFlashArgs &a);
+// The QKV epilogue (launch_qkv_post) writing this attention's fragments instead of fp32 q_fin / k_fin / v_out: uses
+// a.qkv, B, rank, norm weights, rope, q_pre, k_pre, tq, tv of `a` and the fragment pointers of `f`.
+void launch_qkv_post_flash(const QkvPostArgs &a, const AttnFlashArgs &f);
 void launch_attn_bwd_flash(const AttnFlashArgs &a);
 
 struct QkvBwdArgs {

@@ -358,12 +358,12 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
         half_t *attn16 = s->full_param ? at<half_t>(s->attn16, L * s->st_attn) : a16;
         float *probs = s->probs ? at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N) : nullptr;
         const float attn_scale = 1.0f / sqrtf((float)s->hd);
-        launch_qkv_post(qa, BN);
-        if (s->use_flash) {
+        if (s->use_flash) {                                  // epilogue and attention on bf16-pair fragments, no fp32 q / k / v
             AttnFlashArgs f = flash_args(s, L);
-            f.q = qa.q_fin; f.k = qa.k_fin; f.v = qa.v_out; f.out16 = attn16;
+            f.out16 = attn16;
+            launch_qkv_post_flash(qa, f);
             launch_attn_fwd_flash(f);
-        }
+        } else launch_qkv_post(qa, BN);
         AttnFwdArgs aa{};
         aa.q = qa.q_fin; aa.k = qa.k_fin; aa.v = qa.v_out;
         aa.Hq = s->Hq; aa.Hkv = s->Hkv; aa.hd = s->hd; aa.seq = s->N; aa.batch = s->B;
