@@ -62,7 +62,7 @@ __global__ __launch_bounds__(NT) void k_norm_rows(NormRowsArgs a)
         prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_block_row(blockIdx.x, a.rows_launched);
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
     const uint32_t tok = a.emb ? a.tokens[r] : 0u;
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
-    const size_t row = blockIdx.x;
+    const size_t row = xcd_block_row(blockIdx.x, a.rows_launched);
     const int hd = a.hd, half = hd / 2, qd = a.Hq * hd, kd = a.Hkv * hd, R = a.R;
     const int n = qd + 2 * kd + 2 * R;
     float *dhp = buf + n;
@@ -719,7 +719,7 @@ __device__ __forceinline__ float act_fwd(float g, int gelu)
 __global__ __launch_bounds__(RB) void k_glu_fwd(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_block_row(blockIdx.x, gridDim.x);
     const int IS = a.IS, nv = IS >> 2;
     float4 act[MAXV];
     float amax = 0.f;
@@ -821,7 +821,7 @@ __device__ __forceinline__ void act_bwd(float dy, float g, float u, int gelu, fl
 __global__ __launch_bounds__(RB) void k_glu_bwd(GluArgs a)
 {
     __shared__ float sm[16];
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_block_row(blockIdx.x, gridDim.x);
     const int IS = a.IS, nv = IS >> 2;
     float4 dg[MAXV], du[MAXV];
     float amax = 0.f;
@@ -922,7 +922,7 @@ __global__ __launch_bounds__(NT) void k_norm_bwd_rows(NormBwdArgs a)
         prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
-    const size_t r = blockIdx.x;
+    const size_t r = xcd_block_row(blockIdx.x, a.rows_launched);
     const int D = a.D, nv = D >> 2;
     float4 dy[MAXV], x[MAXV], g[MAXV];
     float ss = 0.f, dot = 0.f;

@@ -107,10 +107,20 @@ __global__ void reduce_planes(const float *__restrict__ P, int S, size_t plane_s
 __global__ __launch_bounds__(256) void q8_operand_to_f16(lmhip::WeightOp W, int Nb, int Kb, half8 *__restrict__ out, int f16_only)
 {
     const int lane = threadIdx.x & 63;
-    const size_t tile = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (tile >= (size_t)Nb * Kb) return;
-    const int nb = (int)(tile / Kb), kt = (int)(tile % Kb);
-    if (f16_only && (W.fmt == 1 ? nb < W.nbq : kt < W.kbq)) return;
+    const size_t t = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    int nb, kt;
+    if (!f16_only) {
+        if (t >= (size_t)Nb * Kb) return;
+        nb = (int)(t / Kb); kt = (int)(t % Kb);
+    } else if (W.fmt == 1) {                               // the row blocks from nbq on
+        if (t >= (size_t)(Nb - W.nbq) * Kb) return;
+        nb = W.nbq + (int)(t / Kb); kt = (int)(t % Kb);
+    } else {                                              // the K steps from kbq on, of every row block
+        const int kf = Kb - W.kbq;
+        if (kf <= 0 || t >= (size_t)Nb * kf) return;
+        nb = (int)(t / kf); kt = W.kbq + (int)(t % kf);
+    }
+    const size_t tile = (size_t)nb * Kb + kt;
     half8 w[4];
     if (W.fmt == 1) {
         if (nb < W.nbq) lmhip::load_w_q8_rows(w, W, nb, Kb, kt, lane);
@@ -367,8 +377,10 @@ WeightOp f16_image_of(const WeightOp &W, int N, int K, void *keep, bool f16_part
     const int Nb = tiled_rb(N), Kb = tiled_kb(K);
     const size_t tiles = (size_t)Nb * Kb;
     half8 *img = keep ? (half8 *)keep : (half8 *)scratch(SCR_WF16, tiles * 256 * sizeof(half8));
-    if (!(f16_part_only && !W.w16)) {
-        hipLaunchKernelGGL(q8_operand_to_f16, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, stream(), W, Nb, Kb, img, f16_part_only ? 1 : 0);
+    size_t todo = tiles;
+    if (f16_part_only) todo = !W.w16 ? 0 : W.fmt == 1 ? (size_t)(Nb - W.nbq) * Kb : (size_t)Nb * (Kb - W.kbq);
+    if (todo) {
+        hipLaunchKernelGGL(q8_operand_to_f16, dim3((unsigned)((todo + 3) / 4)), dim3(256), 0, stream(), W, Nb, Kb, img, f16_part_only ? 1 : 0);
         HIP_CHECK(hipGetLastError());
     }
     return weight_f16(reinterpret_cast<const half_t *>(img));

@@ -156,6 +156,18 @@ __device__ __forceinline__ void prefetch_weight_tiles(const WeightPrefetch &pf, 
     asm volatile("" :: "v"(sink));                        // the loads have a use, and nothing is stored
 }
 
+// Row of workgroup `id` in a one-workgroup-per-row kernel over `rows` rows.  Workgroup ids go to the eight XCDs in
+// turn, and such a kernel writes its row of a tiled fp16 operand as 16-byte pieces 512 bytes apart, which only fill
+// whole memory lines together with the other 31 rows of the 32-row block.  So within every run of 256 ids XCD x gets
+// the 32 rows of one block, one after the other: the pieces meet in that XCD's L2 instead of reaching memory as
+// partial lines from eight L2s.  Rows beyond the last whole run of 256 keep their id.
+__device__ __forceinline__ int xcd_block_row(int id, int rows)
+{
+    if (id >= (rows & ~255)) return id;
+    const int in = id & 255;
+    return (id & ~255) + ((in & 7) << 5) + (in >> 3);
+}
+
 __device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 __device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
 __device__ __forceinline__ float amax4(float4 v) { return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))); }
