@@ -422,15 +422,16 @@ __global__ __launch_bounds__(TB) void k_attn_bwd_dkv(AttnBwdArgs a)
 // row [dq | dk | dv | dh_q | dh_v] as one scaled fp16 operand so that a single GEMM
 // against [Wq; Wk; Wv; A_q; A_v]^T yields dq Wq + dk Wk + dv Wv + dh_q A_q + dh_v A_v
 // (src/nn/fast_sft.c:953-971).
-// NP, RK: pairs per lane and LoRA rank compiled in, as in k_qkv_post.
-template <int NP, int RK>
-__global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
+// NP, RK: pairs per lane and LoRA rank compiled in, as in k_qkv_post.  NT: threads per row (1024, or 256 from a few
+// hundred rows on, as in k_norm_rows).
+template <int NP, int RK, int NT = RB>
+__global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
 {
-    extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [16 waves][32] partials
+    extern __shared__ float buf[];                       // [qd + 2kd + 2R] then [NT / 64 waves][32] partials
     __shared__ float sm[16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
-        prefetch_weight_tiles<RB>(a.pf, blockIdx.x - a.rows_launched);
+        prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t row = xcd_block_row(blockIdx.x, a.rows_launched);
@@ -442,7 +443,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
     // issued before the first reduction, so their latency is paid once per trip instead of once per head.
     constexpr int SU = 3;
     const int nslots = a.Hq + a.Hkv;
-    for (int s0 = wave; s0 < nslots; s0 += (RB / 64) * SU) {
+    for (int s0 = wave; s0 < nslots; s0 += (NT / 64) * SU) {
         float g0[SU][NP], g1[SU][NP], p0[SU][NP], p1[SU][NP], w0[SU][NP], w1[SU][NP];
         float2 cs[NP];
 #pragma unroll
@@ -452,7 +453,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         }
 #pragma unroll
         for (int u = 0; u < SU; u++) {
-            const int slot = min(s0 + (RB / 64) * u, nslots - 1);      // clamped: the extra work is not stored
+            const int slot = min(s0 + (NT / 64) * u, nslots - 1);      // clamped: the extra work is not stored
             const int isk = slot >= a.Hq, h = isk ? slot - a.Hq : slot;
             const int W = isk ? kd : qd;
             const float *gin = (isk ? a.dk : a.dq) + row * W + h * hd;
@@ -471,7 +472,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         }
 #pragma unroll
         for (int u = 0; u < SU; u++) {
-            const int slot = s0 + (RB / 64) * u;
+            const int slot = s0 + (NT / 64) * u;
             float y0[NP], y1[NP];
             float ss = 0.f, dot = 0.f;
 #pragma unroll
@@ -500,7 +501,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
             }
         }
     }
-    for (int c = threadIdx.x; c < kd; c += RB) buf[qd + kd + c] = a.dv[row * kd + c];
+    for (int c = threadIdx.x; c < kd; c += NT) buf[qd + kd + c] = a.dv[row * kd + c];
     __syncthreads();
     // dh[r] = sc * sum_c d[c] * B[c][r].  Rank 16 (the common case): four threads share a row of B (16 floats, one
     // float4 each) and 256 such groups split the columns, so a thread keeps 4 + 4 sums and a wave reduces over its 16
@@ -512,13 +513,13 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
             // two plain loops (q columns, then v columns), so that the loads of B of eight trips can be in flight at once:
             // every workgroup reads all of B, and what bounds it is how much of that one CU keeps in flight
 #pragma unroll 8
-            for (int c = threadIdx.x >> 2; c < qd; c += RB / 4) {
+            for (int c = threadIdx.x >> 2; c < qd; c += NT / 4) {
                 const float x = buf[c];
                 const float4 w = ld4(a.Bq + (size_t)c * 16 + 4 * sub);
                 aq[0] += x * w.x; aq[1] += x * w.y; aq[2] += x * w.z; aq[3] += x * w.w;
             }
 #pragma unroll 4
-            for (int c = threadIdx.x >> 2; c < kd; c += RB / 4) {
+            for (int c = threadIdx.x >> 2; c < kd; c += NT / 4) {
                 const float x = buf[qd + kd + c];
                 const float4 w = ld4(a.Bv + (size_t)c * 16 + 4 * sub);
                 av[0] += x * w.x; av[1] += x * w.y; av[2] += x * w.z; av[3] += x * w.w;
@@ -537,7 +538,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
 #pragma unroll
         for (int r = 0; r < 32; r++) acc[r] = 0.f;
 #pragma unroll 4
-        for (int c = threadIdx.x; c < qd + kd; c += RB) {
+        for (int c = threadIdx.x; c < qd + kd; c += NT) {
             const int isv = c >= qd;
             const float x = buf[isv ? c + kd : c];
             const float *Br = isv ? a.Bv + (size_t)(c - qd) * R : a.Bq + (size_t)c * R;
@@ -567,7 +568,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         if (threadIdx.x < 2 * R) {
             const int isv = threadIdx.x >= R, rr = isv ? threadIdx.x - R : threadIdx.x;
             float s = 0.f;
-            for (int w = 0; w < RB / 64; w++) s += dhp[w * 32 + (isv ? 16 : 0) + rr];
+            for (int w = 0; w < NT / 64; w++) s += dhp[w * 32 + (isv ? 16 : 0) + rr];
             s *= a.sc;
             buf[qd + 2 * kd + threadIdx.x] = s;
             a.dh[row * 2 * R + threadIdx.x] = s;
@@ -575,7 +576,7 @@ __global__ __launch_bounds__(RB) void k_qkv_bwd_rows(QkvBwdArgs a)
         __syncthreads();
     }
     float amax = 0.f;
-    for (int c = threadIdx.x; c < n; c += RB) amax = fmaxf(amax, fabsf(buf[c]));
+    for (int c = threadIdx.x; c < n; c += NT) amax = fmaxf(amax, fabsf(buf[c]));
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
     write_f16_tiled(buf, n, a.out16, row, s);
@@ -1066,10 +1067,14 @@ __global__ __launch_bounds__(256) void k_ce_rows(CeArgs a)
     const int Kb = tiled_kb(V);
     for (int c = c_beg + threadIdx.x; c < c_end; c += 256) {
         half8 hv;
+        // V % 4 == 0 (checked by the launcher): the eight logits are two aligned 16-byte loads, each inside the row or not
+        const float4 lo4 = c * 8 < V ? ld4(lg + c * 8) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 hi4 = c * 8 + 4 < V ? ld4(lg + c * 8 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float x[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const int i = c * 8 + e;
-            hv[e] = (i < V) ? f2h((expf(lg[i] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
+            hv[e] = (i < V) ? f2h((expf(x[e] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
         }
         *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
     }
@@ -1215,6 +1220,7 @@ void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
     QkvBwdArgs b = a;
     b.rows_launched = rows;
     const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
+    if (rows >= MANY_ROWS && a.R == 16 && a.hd <= 128 && !a.pf.base) { LAUNCH((k_qkv_bwd_rows<1, 16, TB>), grid, dim3(TB), n * 4, b); return; }
     if (a.hd <= 128) {
         if (a.R == 16) LAUNCH((k_qkv_bwd_rows<1, 16>), grid, dim3(RB), n * 4, b);
         else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<1, 0>), grid, dim3(RB), n * 4, b);
