@@ -263,7 +263,8 @@ def main():
                 "peak": MFMA_PEAK_TFS if compute_bound else HBM_PEAK_GBS,
                 "unit": "TFLOP/s" if compute_bound else "GB/s",
                 "frac": round(tfs / MFMA_PEAK_TFS if compute_bound else gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "gemm_tiled", "launches_per_step": n // prof_steps,
+                "kernel": ("gemm_big_f16" if cfg.BN >= 1024 else "gemm_tiled + gemm_big_f16" if compute_bound else "gemm_tiled"),
+                "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                 "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}
@@ -278,7 +279,9 @@ def main():
     out = {"metric": metric,
            "value": round(toks, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-           "dtype": "f16 weights x f16 activations, f32 accumulate", "data": "synthetic",
+           "dtype": ("q8_0 weights as f16 images x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN >= 1024 else
+                     "q8_0 weights unpacked to f16 in registers x f16 activations, f32 accumulate" if cfg.weight_format != "f16" else
+                     "f16 weights x f16 activations, f32 accumulate"), "data": "synthetic",
            "config": {"workload": cfg.name, "rows_per_step": rows_per_step, "layers": cfg.NL, "lora_rank": cfg.R,
                       "frozen_params": cfg.frozen_params, "weight_format": cfg.weight_format},
            "roofline": roofline, "final_loss": round(float(loss), 5),
