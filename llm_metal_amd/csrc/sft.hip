@@ -349,8 +349,10 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
         qa.eps = s->eps; qa.rope = at<float2>(s->rope_tabs, (size_t)s->rope_slot[L] * s->N * (s->hd / 2));
         qa.Hq = s->Hq; qa.Hkv = s->Hkv; qa.hd = s->hd; qa.seq = s->N;
         qa.q_pre = at<float>(s->q_pre, (size_t)L * BN * qd); qa.k_pre = at<float>(s->k_pre, (size_t)L * BN * kd);
-        qa.q_fin = at<float>(s->q_fin, (size_t)L * BN * qd); qa.k_fin = at<float>(s->k_fin, (size_t)L * BN * kd);
-        qa.v_out = at<float>(s->v_sav, (size_t)L * BN * kd);
+        if (s->q_fin) {                                       // not kept by the attention that works on fragments
+            qa.q_fin = at<float>(s->q_fin, (size_t)L * BN * qd); qa.k_fin = at<float>(s->k_fin, (size_t)L * BN * kd);
+            qa.v_out = at<float>(s->v_sav, (size_t)L * BN * kd);
+        }
         qa.tq = at<float>(s->tq, (size_t)L * BN * (R ? R : 1)); qa.tv = at<float>(s->tv, (size_t)L * BN * (R ? R : 1));
         const size_t st_kt = (size_t)s->B * kd * attn_ldt(s->N);
         if (s->kT) { qa.kT = at<float>(s->kT, (size_t)L * st_kt); qa.vT = at<float>(s->vT, (size_t)L * st_kt); }
@@ -508,8 +510,10 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         AttnBwdArgs ab{};
         ab.dO = pdo;
         ab.probs = s->probs ? at<float>(s->probs, (size_t)L * s->B * s->Hq * s->N * s->N) : nullptr;
-        ab.q = at<float>(s->q_fin, (size_t)L * BN * qd); ab.k = at<float>(s->k_fin, (size_t)L * BN * kd);
-        ab.v = at<float>(s->v_sav, (size_t)L * BN * kd);
+        if (s->q_fin) {
+            ab.q = at<float>(s->q_fin, (size_t)L * BN * qd); ab.k = at<float>(s->k_fin, (size_t)L * BN * kd);
+            ab.v = at<float>(s->v_sav, (size_t)L * BN * kd);
+        }
         ab.Hq = s->Hq; ab.Hkv = s->Hkv; ab.hd = s->hd; ab.seq = s->N; ab.batch = s->B;
         ab.scale = 1.0f / sqrtf((float)s->hd);
         ab.vT = s->vT ? at<float>(s->vT, (size_t)L * s->B * kd * attn_ldt(s->N)) : nullptr;
@@ -788,7 +792,6 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->xs = fbuf((size_t)(2 * NL + 1) * xsz);
     s->ln1_16 = hbuf((size_t)NL * s->st_ln1); s->ln1_inv = fbuf((size_t)NL * BN);
     s->q_pre = fbuf((size_t)NL * BN * qd); s->k_pre = fbuf((size_t)NL * BN * kd);
-    s->q_fin = fbuf((size_t)NL * BN * qd); s->k_fin = fbuf((size_t)NL * BN * kd); s->v_sav = fbuf((size_t)NL * BN * kd);
     s->use_flash = attn_flash_supported(s->hd, s->N, s->Hq, s->Hkv);
     if (s->use_flash) {
         const size_t eq = attn_flash_tile_elems(s->hd, s->N, s->Hq, s->B), ek = attn_flash_tile_elems(s->hd, s->N, s->Hkv, s->B);
@@ -797,7 +800,10 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
         s->fa_v = metal_buf_create((size_t)NL * 2 * ek * 16); s->fa_do = metal_buf_create(2 * eq * 16);
         s->fa_O = fbuf((size_t)NL * BN * qd); s->fa_lse = fbuf((size_t)NL * stat); s->fa_D = fbuf(stat);
         s->fa_dkp = fbuf((size_t)(s->Hq / s->Hkv) * BN * kd); s->fa_dvp = fbuf((size_t)(s->Hq / s->Hkv) * BN * kd);
-    } else s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
+    } else {
+        s->probs = fbuf((size_t)NL * s->B * s->Hq * s->N * s->N);
+        s->q_fin = fbuf((size_t)NL * BN * qd); s->k_fin = fbuf((size_t)NL * BN * kd); s->v_sav = fbuf((size_t)NL * BN * kd);
+    }
     if (!s->use_flash && attn_mfma_supported(s->hd, s->N)) {
         s->kT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N)); s->vT = fbuf((size_t)NL * s->B * kd * attn_ldt(s->N));
     }

@@ -74,6 +74,7 @@ CASES = [
     C1.with_(name="c1_batch3_flash", batch=3, seq=32),
     C1.with_(name="window24_flash", window=24),
     C1.with_(name="seq333_window50_flash", NL=1, batch=2, seq=333, V=1024, window=50),
+    C1.with_(name="seq1100_flash", NL=1, D=128, Hq=2, Hkv=1, hd=64, IS=256, V=512, seq=1100),      # beyond the other kernels' 1024 keys
     C1.with_(name="seq512_noflash", NL=1, seq=512, V=1024),
     C1.with_(name="window_seq300_noflash", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
     # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
