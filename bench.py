@@ -162,6 +162,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seq", type=int, default=0, help="override the configuration's sequence length (experiments only)")
     ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch (experiments only)")
+    ap.add_argument("--q8-large-m", choices=("kept-image", "image-per-product", "unpack-in-lds"), default="kept-image",
+                    help="how products with >= 1024 rows read Q8_0 weights: the F16 image a state keeps once made (default), "
+                         "an F16 image made for every product, or Q8_0 tiles unpacked into LDS by the GEMM itself")
     ap.add_argument("--decode", action="store_true",
                     help="time greedy token-by-token generation (include/inference_hip.h) on the configuration's model "
                          "instead of the training step: a step is one token")
@@ -205,6 +208,10 @@ def main():
     t0 = time.perf_counter()
     model = make_model(cfg, seed=0, lora_b_std=0.0)          # timing runs: B = 0 as the reference initialises it
     t_gen = time.perf_counter() - t0
+    if args.q8_large_m == "image-per-product":
+        L.hip_gemm_image_budget_mb(0)
+    elif args.q8_large_m == "unpack-in-lds" and cfg.weight_format != "f16" and cfg.BN >= 1024:
+        L.hip_gemm_force_large_m(2)
     st = SFTState(cfg, model)
     t_init = time.perf_counter() - t0 - t_gen
     del model
@@ -263,7 +270,8 @@ def main():
                 "peak": MFMA_PEAK_TFS if compute_bound else HBM_PEAK_GBS,
                 "unit": "TFLOP/s" if compute_bound else "GB/s",
                 "frac": round(tfs / MFMA_PEAK_TFS if compute_bound else gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": ("gemm_big_f16" if cfg.BN >= 1024 else "gemm_tiled + gemm_big_f16" if compute_bound else "gemm_tiled"),
+                "kernel": ("gemm_big<1>, gemm_big<2>" if cfg.BN >= 1024 and cfg.weight_format != "f16" and args.q8_large_m == "unpack-in-lds" else
+                           "gemm_big_f16" if cfg.BN >= 1024 else "gemm_tiled + gemm_big_f16" if compute_bound else "gemm_tiled"),
                 "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                 "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
@@ -279,11 +287,14 @@ def main():
     out = {"metric": metric,
            "value": round(toks, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-           "dtype": ("q8_0 weights as f16 images x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN >= 1024 else
+           "dtype": ("q8_0 weights unpacked to f16 in LDS x f16 activations, f32 accumulate"
+                     if cfg.weight_format != "f16" and cfg.BN >= 1024 and args.q8_large_m == "unpack-in-lds" else
+                     "q8_0 weights as f16 images x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN >= 1024 else
                      "q8_0 weights unpacked to f16 in registers x f16 activations, f32 accumulate" if cfg.weight_format != "f16" else
                      "f16 weights x f16 activations, f32 accumulate"), "data": "synthetic",
            "config": {"workload": cfg.name, "rows_per_step": rows_per_step, "layers": cfg.NL, "lora_rank": cfg.R,
-                      "frozen_params": cfg.frozen_params, "weight_format": cfg.weight_format},
+                      "frozen_params": cfg.frozen_params, "weight_format": cfg.weight_format,
+                      **({"q8_large_m": args.q8_large_m} if cfg.weight_format != "f16" and cfg.BN >= 1024 else {})},
            "roofline": roofline, "final_loss": round(float(loss), 5),
            "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}
     if not args.no_cpu_baseline:
