@@ -164,8 +164,8 @@ void hip_gemm_force_large_m(int policy);
  * always n. */
 void hip_gemm_large_m_split(int mode);
 /* A training state with frozen Q8_0 weights whose products run on the large-M kernel keeps the F16 image of every
- * weight it has used (made once instead of once per product) when the images of all its weights fit this many MB
- * (default 65536; the 4B model needs 16 GB); 0 = never keep them. */
+ * weight it has used (made once instead of once per product) while they fit this many MB per state (default 65536;
+ * the 4B model needs 16 GB); weights beyond that, or all with 0, get an image per product. */
 void hip_gemm_image_budget_mb(int mb);
 /* Training attention without the [seq, seq] probability matrices in memory (running softmax in the forward, the
  * probabilities formed again in the backward): -1 = for head_dim 64 / 128 and sequences of at least 128 positions

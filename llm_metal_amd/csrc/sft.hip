@@ -92,9 +92,8 @@ struct SFTState {
     MetalBuf *lora_acc;                  // LoRA gradients summed over the completions of a GRPO group
     // Q8_0 states whose products run on the large-M kernel keep the F16 image of every frozen weight they have used
     // (dequantised once, not once per product), as long as all of them fit the budget
-    std::unordered_map<const void *, half_t *> img_slots;
-    MetalBuf *img_arena;
-    size_t img_used, img_cap;
+    std::unordered_map<const void *, MetalBuf *> img_slots;
+    size_t img_bytes;
     int step_in_flight, step_rejected;   // sft_enqueue_train_step without its sft_finish_train_step yet; ids refused
     std::vector<LayerW> layers_out;      // row-major F16 copies handed out by sft_get_layers
     std::vector<WMat> wmats_out;
@@ -254,29 +253,20 @@ AttnFlashArgs flash_args(SFTState *s, int L)
 
 // F16 tiles of a weight for the large-M kernel.  A Q8_0 weight of a LoRA state is frozen, so its image is made once
 // and kept (16 GB for the 4B model's two orientations; MI355X has the room, and the product then reads what it would
-// read anyway); only the adapter rows of the fused QKV matrix, which every step changes, are copied again.  Without
-// room within the budget for all the state's weights the image is made per product in the scratch arena.
+// read anyway); only the adapter rows of the fused QKV matrix, which every step changes, are copied again.  A weight
+// whose image no longer fits the budget gets one per product in the scratch arena.
 size_t g_image_budget = (size_t)64 << 30;
 WeightOp resident_image(SFTState *s, const WeightOp &W, int N, int K)
 {
     if (W.fmt == 0 || s->full_param || large_m_unpacks_q8() || !g_image_budget) return f16_image_of(W, N, K);
-    if (!s->img_arena) {
-        if (s->img_cap == (size_t)-1) return f16_image_of(W, N, K);            // found too large before
-        const int NL = s->NL;
-        size_t need = 0;
-        const int shp[5][2] = {{s->nq_ext, s->D}, {s->D, s->qd}, {2 * s->IS, s->D}, {s->D, s->IS}, {s->V, s->D}};
-        for (int k = 0; k < 5; k++) need += (tiled_elems(shp[k][0], shp[k][1]) + tiled_elems(shp[k][1], shp[k][0])) * (k == 4 ? 1 : NL);
-        if (need * sizeof(half_t) > g_image_budget) { s->img_cap = (size_t)-1; return f16_image_of(W, N, K); }
-        s->img_arena = hbuf(need); s->img_cap = need; s->img_used = 0;
-    }
     auto it = s->img_slots.find(W.q);
-    if (it != s->img_slots.end()) return f16_image_of(W, N, K, it->second, true);
-    const size_t elems = tiled_elems(N, K);
-    if (s->img_used + elems > s->img_cap) return f16_image_of(W, N, K);
-    half_t *slot = at<half_t>(s->img_arena, s->img_used);
-    s->img_used += elems;
+    if (it != s->img_slots.end()) return f16_image_of(W, N, K, at<half_t>(it->second), true);
+    const size_t bytes = tiled_elems(N, K) * sizeof(half_t);
+    if (s->img_bytes + bytes > g_image_budget) return f16_image_of(W, N, K);   // no room: this weight's image is made per product
+    MetalBuf *slot = metal_buf_create(bytes);
+    s->img_bytes += bytes;
     s->img_slots.emplace(W.q, slot);
-    return f16_image_of(W, N, K, slot, false);
+    return f16_image_of(W, N, K, at<half_t>(slot), false);
 }
 
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
@@ -869,8 +859,9 @@ void sft_state_free(SFTState *s)
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
                        s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
                        s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf,
-                       s->fa_q, s->fa_k, s->fa_v, s->fa_O, s->fa_lse, s->fa_do, s->fa_D, s->fa_dkp, s->fa_dvp, s->img_arena};
+                       s->fa_q, s->fa_k, s->fa_v, s->fa_O, s->fa_lse, s->fa_do, s->fa_D, s->fa_dkp, s->fa_dvp};
     for (MetalBuf *b : s->views_out) metal_buf_free(b);
+    for (auto &kv : s->img_slots) metal_buf_free(kv.second);
     for (MetalBuf *b : all) metal_buf_free(b);
     for (WMat &w : s->wmats_out) metal_buf_free(w.mbuf);
     delete s;
