@@ -26,14 +26,21 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFS = 2500.0          # dense fp16 MFMA
 
 
+TRAFFIC_SUMMARIES = {"c3_qwen3_4b_f16": ("c3_gemm_hbm_traffic_pmc.txt", "traffic_bytes_per_gemm_launch_c3"),
+                     "c4_qwen3_4b_q8": ("c4_gemm_hbm_traffic_pmc.txt", "traffic_bytes_per_gemm_launch_c4")}
+
+
 def measured_traffic(cfg_name):
     """HBM bytes per GEMM launch from the committed hardware-counter summary of this workload (two rocprofv3
     --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by a copy kernel of known size), or None when there is none."""
-    path = os.path.join(ROOT, "profiles", "c3_gemm_hbm_traffic_pmc.txt")
-    if cfg_name != "c3_qwen3_4b_f16" or not os.path.exists(path):
+    if cfg_name not in TRAFFIC_SUMMARIES:
+        return None
+    name, key = TRAFFIC_SUMMARIES[cfg_name]
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(path):
         return None
     for line in open(path):
-        if line.startswith("traffic_bytes_per_gemm_launch_c3"):
+        if line.startswith(key):
             return float(line.split("=")[1])
     return None
 
@@ -277,7 +284,7 @@ def main():
                 "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}
     roofline["traffic"] = measured_traffic(cfg.name)
-    roofline["traffic_source"] = ("profiles/c3_gemm_hbm_traffic_pmc.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
+    roofline["traffic_source"] = (f"profiles/{TRAFFIC_SUMMARIES.get(cfg.name, ('',))[0]}: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
                                   "scaled by the same counters on a copy kernel of known size; not re-measured in this run"
                                   if roofline["traffic"] is not None else "no hardware-counter summary is committed for this workload")
     st.free()
