@@ -168,8 +168,9 @@ void hip_gemm_large_m_split(int mode);
  * the 4B model needs 16 GB); weights beyond that, or all with 0, get an image per product. */
 void hip_gemm_image_budget_mb(int mb);
 /* Training attention without the [seq, seq] probability matrices in memory (running softmax in the forward, the
- * probabilities formed again in the backward): -1 = for head_dim 64 / 128 and sequences of at least 128 positions
- * (default), 0 = never, 1 = whenever the head size allows.  Read when a training state is created. */
+ * probabilities formed again in the backward): -1 = for head_dim 64 / 128 when ceil(seq / 128) * query heads * batch
+ * is at least 128 or the sequence is longer than 1024 (default, the measured rule), 0 = never, 1 = whenever the head
+ * size allows.  Read when a training state is created. */
 void hip_attention_flash(int mode);
 /* Timing aid for benchmarks: when enabled, every GEMM launch is bracketed by HIP events on the
  * library's stream.  hip_gemm_profile_read (after metal_flush) returns the number of launches recorded

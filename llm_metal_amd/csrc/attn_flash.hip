@@ -690,10 +690,14 @@ int g_flash_mode = -1;
 
 void set_attn_flash_mode(int mode) { g_flash_mode = mode < 0 ? -1 : mode > 0 ? 1 : 0; }
 
-bool attn_flash_supported(int hd, int seq, int Hq, int Hkv)
+// The measured rule (Qwen3-4B widths, MI355X; step time without / with saved probabilities): these kernels run one
+// workgroup per 128 queries of a head and want at least half the CUs' worth of them -- 1 x 512 positions x 32 heads = 128
+// workgroups 28.6 / 29.0 ms, 2 x 512 44.8 / 49.2, 1 x 1024 48.6 / 56.2, 4 x 256 43.1 / 45.2, 8 x 128 42.2 / 43.7, against
+// 1 x 256 (64 workgroups) 18.4 / 17.5 and 1 x 128 12.5 / 11.7 -- and take every sequence beyond the other kernels' 1024 keys.
+bool attn_flash_supported(int hd, int seq, int Hq, int Hkv, int batch)
 {
-    if (g_flash_mode == 0 || !(hd == 64 || hd == 128) || seq < 1 || Hkv < 1 || Hq % Hkv) return false;
-    return g_flash_mode == 1 || seq >= 128;
+    if (g_flash_mode == 0 || !(hd == 64 || hd == 128) || seq < 1 || Hkv < 1 || Hq % Hkv || batch < 1) return false;
+    return g_flash_mode == 1 || seq > 1024 || (long)((seq + 127) / 128) * Hq * batch >= 128;
 }
 
 size_t attn_flash_tile_elems(int hd, int seq, int heads, int batch)

@@ -120,9 +120,10 @@ struct AttnFlashArgs {
     float *dq, *dk, *dv;          // backward: [rows][Hq*hd], [rows][Hkv*hd] x2
     float *dkp, *dvp;             // backward scratch: [Hq/Hkv][rows][Hkv*hd] each
 };
-// -1: head_dim 64/128 and at least 128 positions (default); 0: never; 1: whenever the head size allows
+// -1: head_dim 64/128 and enough (128-query block, head, sequence) workgroups for half the CUs, or more than 1024
+// positions (default); 0: never; 1: whenever the head size allows
 void set_attn_flash_mode(int mode);
-bool attn_flash_supported(int hd, int seq, int Hq, int Hkv);
+bool attn_flash_supported(int hd, int seq, int Hq, int Hkv, int batch);
 size_t attn_flash_tile_elems(int hd, int seq, int heads, int batch);     // 16-byte elements of one RT or PT image
 // q, k, v null: the fragments are there already (launch_qkv_post_flash)
 void launch_attn_fwd_flash(const AttnFlashArgs &a);

@@ -782,7 +782,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->xs = fbuf((size_t)(2 * NL + 1) * xsz);
     s->ln1_16 = hbuf((size_t)NL * s->st_ln1); s->ln1_inv = fbuf((size_t)NL * BN);
     s->q_pre = fbuf((size_t)NL * BN * qd); s->k_pre = fbuf((size_t)NL * BN * kd);
-    s->use_flash = attn_flash_supported(s->hd, s->N, s->Hq, s->Hkv);
+    s->use_flash = attn_flash_supported(s->hd, s->N, s->Hq, s->Hkv, s->B);
     if (s->use_flash) {
         const size_t eq = attn_flash_tile_elems(s->hd, s->N, s->Hq, s->B), ek = attn_flash_tile_elems(s->hd, s->N, s->Hkv, s->B);
         const size_t stat = (size_t)s->B * s->Hq * ((s->N + 31) / 32) * 32;

@@ -81,17 +81,20 @@ def _check_sampled(g, key, tensor, tol):
     assert rel(tensor[idx], g[key + "_sample"]) < tol, (key, rel(tensor[idx], g[key + "_sample"]))
 
 
-@pytest.mark.parametrize("policy", [0, 2], ids=["measured_rule", "q8_unpacked_in_lds"])
-def test_q8_step_at_2048_rows_matches_oracle_fixture(policy):
+@pytest.mark.parametrize("policy,attention", [(0, -1), (2, -1), (0, 0)],
+                         ids=["measured_rule", "q8_unpacked_in_lds", "attention_with_saved_probabilities"])
+def test_q8_step_at_2048_rows_matches_oracle_fixture(policy, attention):
     """Config 4's shape on one layer: Q8_0 weights, 4 x 512 rows.  Policy 0 is what the benchmark runs (every product
-    on the large-M kernel over an F16 image of the operand); policy 2 keeps the operand quantised and unpacks the
-    Q8_0 tiles into LDS inside the large-M kernel."""
+    on the large-M kernel over an F16 image of the operand, attention without saved probabilities); policy 2 keeps the
+    operand quantised and unpacks the Q8_0 tiles into LDS inside the large-M kernel; the third case pins the attention
+    kernels that save the probabilities, which the rule leaves at this shape."""
     cfg = rw.C4_WIDTHS
     model = make_model(cfg, seed=rw.MODEL_SEED, gamma_jitter=rw.GAMMA_JITTER)
     g = _golden("real_width_c4.npz", model)
     tok, tgt = make_batch(cfg, seed=rw.BATCH_SEED)
     L = lib.load()
     L.hip_gemm_force_large_m(policy)
+    L.hip_attention_flash(attention)
     try:
         with SFTState(cfg, model) as st:
             loss = st.train_step(tok, tgt, 1e-4)
@@ -107,6 +110,7 @@ def test_q8_step_at_2048_rows_matches_oracle_fixture(policy):
                 _check_sampled(g, "delta_" + k, after[k] - before[k], 0.1)
     finally:
         L.hip_gemm_force_large_m(0)
+        L.hip_attention_flash(-1)
 
 
 @pytest.mark.parametrize("batch", [1, 2], ids=["one_completion_per_pass", "group_in_one_pass"])

@@ -63,10 +63,10 @@ CASES = [
     C1.with_(name="window_seq300", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
     C1.with_(name="window7_small_heads", NL=1, D=64, Hq=4, Hkv=2, hd=16, IS=96, V=512, seq=40, window=7),
     # attention without saved probabilities (running softmax, probabilities formed again in the backward), which the
-    # measured rule takes from 128 positions on ("seq512", "seq300_hd128", "window_seq300", "gemma_many_rows" above):
-    # forced on for short and ragged sequences, several sequences per batch, one KV head for four query heads, windows
-    # that cut inside a 32-key block and that skip whole blocks; and forced off ("_noflash") so that the long sequences
-    # keep covering the kernels with saved probabilities
+    # measured rule takes when there are enough (128-query block, head, sequence) workgroups or more than 1024 positions
+    # (config 4's shape, and "seq1100" below): forced on for short, ragged and long sequences, several sequences per
+    # batch, one KV head for four query heads, windows that cut inside a 32-key block and that skip whole blocks; the
+    # cases above cover the kernels with saved probabilities at the same lengths
     C1.with_(name="c1_flash"),
     C1.with_(name="hd128_flash", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
     C1.with_(name="ragged_seq40_flash", NL=2, batch=2, seq=40, R=4, alpha=8.0),
@@ -74,9 +74,10 @@ CASES = [
     C1.with_(name="c1_batch3_flash", batch=3, seq=32),
     C1.with_(name="window24_flash", window=24),
     C1.with_(name="seq333_window50_flash", NL=1, batch=2, seq=333, V=1024, window=50),
-    C1.with_(name="seq1100_flash", NL=1, D=128, Hq=2, Hkv=1, hd=64, IS=256, V=512, seq=1100),      # beyond the other kernels' 1024 keys
-    C1.with_(name="seq512_noflash", NL=1, seq=512, V=1024),
-    C1.with_(name="window_seq300_noflash", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
+    C1.with_(name="seq512_flash", NL=1, seq=512, V=1024),
+    C1.with_(name="seq300_hd128_flash", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300),
+    C1.with_(name="window_seq300_flash", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300, window=100),
+    C1.with_(name="seq1100", NL=1, D=128, Hq=2, Hkv=1, hd=64, IS=256, V=512, seq=1100),             # by the rule: beyond 1024 keys
     # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
     TINY_GEMMA3.with_(name="gemma_many_rows", NL=2, batch=4, seq=128),
 ]
