@@ -362,11 +362,14 @@ int gemm_profiling() { return g_prof_on; }
 int g_big_policy = 0;                                     // 0 measured rule, 1 always, -1 never, 2 always and Q8_0 tiles stay quantised
 bool use_big_gemm(int M, int N, int K, int fmt)
 {
-    (void)K;
     if (g_big_policy) return g_big_policy > 0;
     const long blocks = (long)((M + 127) / 128) * ((N + 255) / 256);
-    if (M >= 1024) return blocks >= 160;                  // either format (Q8_0 through its F16 image)
-    return fmt == 0 && M >= 512 && blocks >= 224;
+    const int cus = num_cus() > 0 ? num_cus() : 256;
+    const bool long_k = fmt == 0 && blocks * 8 <= cus && K >= 65536;      // few blocks, cut into many K chunks (big_gemm_chunks)
+    if (M >= 1024) return blocks >= 160 || long_k;        // either format (Q8_0 through its F16 image)
+    // 640 rows, F16 (Gemma3-1B shapes): 135 blocks 24 us against 31 on the streaming kernel, 270 blocks ahead as well;
+    // 25-30 blocks of short K lose by a factor of two to four
+    return fmt == 0 && M >= 512 && (blocks >= 128 || long_k);
 }
 
 // The operand as plain F16 tiles: W itself when it is F16, else an image in the library's scratch arena (valid until

@@ -17,6 +17,7 @@
 #include "gemm.h"
 #include "gemm_kernel.h"
 #include <hip/hip_ext.h>
+#include <algorithm>
 
 namespace lmhip {
 namespace {
@@ -404,6 +405,10 @@ int big_gemm_chunks(int M, int N, int K, int fmt)
     if (g_big_split > 1) return g_big_split;
     const long blocks = (long)((M + 127) / 128) * ((N + 128 * WPW - 1) / (128 * WPW));
     const int cus = num_cus() > 0 ? num_cus() : 256;
+    // a handful of blocks over a very long K (the LM head's backward at a few hundred rows: 25 blocks, K = 262 144): as
+    // many chunks as it takes to give every CU a block, each still thousands of columns long (640 rows: 930 us on the
+    // streaming kernel, 3 680 / 1 340 / 840 / 640 us with 1 / 3 / 5 / 8-10 chunks)
+    if (blocks * 8 <= cus && K >= 65536) return (int)std::min<long>(std::min<long>(cus / blocks, K / 8192), 16);
     return (blocks * 3 <= cus * 2 && K >= 4096) ? 3 : 1;
 }
 

@@ -18,6 +18,7 @@
 #include <math.h>
 #include <string.h>
 #include <vector>
+#include <algorithm>
 #include <unordered_map>
 
 using namespace lmhip;
@@ -184,7 +185,7 @@ size_t max_planes_elems(SFTState *s)
         // whichever kernel the product takes (the choice can be forced at run time): the planes of the streaming kernel, or
         // up to four K chunks of the large-M one; the LM head writes the logits directly unless the streaming kernel splits K
         const bool head = sh.N == s->V && sh.K == s->D;
-        const size_t e = (size_t)(head ? (p.S > 1 ? p.S : 0) : std::max(p.S, 4)) * s->BN * sh.N;
+        const size_t e = (size_t)(head ? (p.S > 1 ? p.S : 0) : std::max({p.S, 4, big_gemm_chunks(s->BN, sh.N, sh.K, 0)})) * s->BN * sh.N;
         if (e > mx) mx = e;
     }
     return mx;

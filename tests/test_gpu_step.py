@@ -136,6 +136,23 @@ def test_train_steps_match_oracle(cfg):
     lib.load().hip_gemm_image_budget_mb(65536)
 
 
+def test_lm_head_backward_over_many_k_chunks():
+    """512 rows and a 65 536-token vocabulary: the LM head's backward is four 128 x 256 blocks over K = 65 536, which the
+    measured rule gives to the large-M kernel cut into eight K chunks (planes added by the consumer); the forward takes
+    the same kernel uncut.  One step against the oracle (its LM head alone is 9 GFLOP of scalar code)."""
+    cfg = C1.with_(name="long_k_head", NL=1, D=64, Hq=2, Hkv=1, hd=32, IS=128, V=65536, batch=4, seq=128)
+    model = make_model(cfg, seed=21, gamma_jitter=0.1)
+    tok, tgt = make_batch(cfg, seed=30)
+    r = run_oracle(cfg, model, [(tok, tgt)], 1e-4)[0]
+    with SFTState(cfg, model) as st:
+        loss = st.train_step(tok, tgt, 1e-4)
+        assert abs(loss - r["loss"]) <= 1e-3 * abs(r["loss"]), (loss, r["loss"])
+        assert abs(st.grad_norm() - r["grad_norm"]) <= 1e-2 * r["grad_norm"]
+        for gv, rv in zip(lora_views(cfg, st.lora_grads()), lora_views(cfg, r["grad"])):
+            for k in ("A_q", "B_q", "A_v", "B_v"):
+                assert rel(gv[k], rv[k]) < 1e-2, (k, rel(gv[k], rv[k]))
+
+
 def test_q8_tiles_hold_the_dequantised_values_in_both_images():
     """Q8_0 weights stay quantised on the device (int8 tiles with row scales, transposed twin with column
     scales).  Read back through the dequantising accessor, both images must equal half(d * q) of the
