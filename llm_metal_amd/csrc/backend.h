@@ -51,9 +51,11 @@ struct HeadPost {
     int Hq, Hkv, R, pos;
     const float2 *rope;                  // (cos, sin) of the hd/2 rotary pairs at position pos
     float eps, sc;
+    size_t qkv_step, cache_step, t_step; // floats from one sequence's qkv / caches / t to the next when several are decoded at once
 };
-// infer_kernels.hip: that and the attention over the cache rows 0 .. pos in one launch (out [Hq*hd])
-void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq);
+// infer_kernels.hip: that and the attention over the cache rows 0 .. pos in one launch (out [Hq*hd]); with copies > 1
+// for that many sequences at position pos, whose caches lie cache_step floats apart inside Kc and Vc (out [copies, Hq*hd])
+void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq, int copies = 1);
 
 // infer_kernels.hip: y[i] = act(gate_i . x) * (up_i . x) for W = [gate; up] of 2 * rows rows (F16, or Q8_0 blocks when q8)
 void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q8, int gelu);

@@ -98,6 +98,29 @@ void launch_rows_to_f16(const float *X, int ldx, half_t *out_tiled, float *inv_s
 // C[M, N] fp32 = A[M, K] fp32 * W^T on the matrix cores with A kept to 22 bits: every row goes in twice, as its fp16
 // image and as the fp16 image of the rounding residual.  W: row-major F16 [N, K] buffer (its tiled image is cached).
 void gemm_f32a_exact(const float *A, struct ::MetalBuf *W, float *C, int M, int N, int K);
+// Its three parts, for callers that fold the first or the last into kernels of their own: the cached tiled image of W;
+// rows m and M + m of the tiled operand a16 [2M, K] and their factors inv [2M] from A [M, K]; launch_gemm over
+// plan_gemm(2M, N, K) into planes of [2M, N]; C [M, N] from the planes.
+const half_t *tiled_weight_of(struct ::MetalBuf *W, int N, int K);
+void launch_rows_to_f16_split(const float *A, half_t *a16, float *inv, int M, int K);
+void launch_reduce_planes_split(const float *P, int S, size_t plane_stride, int ldp, const float *inv, float *C, int M, int N);
+// element (m, n) of such a product: the planes of row m and of row M + m summed, each sum times its row's factor
+__device__ __forceinline__ float split_planes_value(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
+                                                    const float *__restrict__ inv, int M, int m, int n)
+{
+    const float *ph = P + (size_t)m * ldp + n, *pl = P + (size_t)(M + m) * ldp + n;
+    float hi = 0.f, lo = 0.f;
+    int p = 0;
+    for (; p + 8 <= S; p += 8) {                          // eight planes' loads in flight; summed in plane order
+        float h[8], l[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) { h[q] = ph[(p + q) * plane_stride]; l[q] = pl[(p + q) * plane_stride]; }
+#pragma unroll
+        for (int q = 0; q < 8; q++) { hi += h[q]; lo += l[q]; }
+    }
+    for (; p < S; p++) { hi += ph[p * plane_stride]; lo += pl[p * plane_stride]; }
+    return fmaf(lo, inv[M + m], hi * inv[m]);
+}
 void launch_reduce_planes(const float *P, int S, size_t plane_stride, int ldp, const float *row_scale, float *C, int M, int N);
 // dst (tiled, Kb_dst K blocks) <- src row-major F16 [rows, cols]:
 //   element (r, c) goes to tiled(row_off + r, k_off + c), or tiled(row_off + c, k_off + r) when transposed

@@ -74,6 +74,57 @@ __global__ __launch_bounds__(256) void rows_to_f16_split(
     if (threadIdx.x == 0) { inv_scale[row] = inv; inv_scale[M + row] = 1.0f / s2; }
 }
 
+// The same for rows a workgroup of 1024 threads can hold in registers (K <= 8192 * CPT, K % 4 == 0, X 16-byte aligned):
+// a thread owns CPT chunks of 8 consecutive elements, each one 16-byte store into the tiled image, and the row is read
+// once.  Same values as rows_to_f16_split.
+template <int CPT>
+__global__ __launch_bounds__(1024) void rows_to_f16_split_vec(
+    const float *__restrict__ X, int ldx, half_t *__restrict__ out, float *__restrict__ inv_scale, int M, int K, int Kb)
+{
+    __shared__ float sm[16];
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    const int row = blockIdx.x;
+    const float *x = X + (size_t)row * ldx;
+    float v[CPT][8];
+    float amax = 0.f;
+#pragma unroll
+    for (int u = 0; u < CPT; u++) {
+        const int k0 = (threadIdx.x + 1024 * u) * 8;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+        if (k0 < K) a = *reinterpret_cast<const float4 *>(x + k0);
+        if (k0 + 4 < K) b = *reinterpret_cast<const float4 *>(x + k0 + 4);
+        v[u][0] = a.x; v[u][1] = a.y; v[u][2] = a.z; v[u][3] = a.w; v[u][4] = b.x; v[u][5] = b.y; v[u][6] = b.z; v[u][7] = b.w;
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[u][e]));
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax), inv = 1.0f / s;
+    float lmax = 0.f;
+#pragma unroll
+    for (int u = 0; u < CPT; u++) {
+        const int k0 = (threadIdx.x + 1024 * u) * 8;
+        half8 h;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            h[e] = f2h(v[u][e] * s);
+            v[u][e] = v[u][e] - h2f(h[e]) * inv;                            // what the rounding lost, exact in fp32
+            lmax = fmaxf(lmax, fabsf(v[u][e]));
+        }
+        if (k0 < Kb * 64) *reinterpret_cast<half8 *>(out + lmhip::tiled_index(row, k0, Kb)) = h;
+    }
+    lmax = block_max(lmax, sm);
+    const float s2 = row_scale_for(lmax);
+#pragma unroll
+    for (int u = 0; u < CPT; u++) {
+        const int k0 = (threadIdx.x + 1024 * u) * 8;
+        half8 l;
+#pragma unroll
+        for (int e = 0; e < 8; e++) l[e] = f2h(v[u][e] * s2);
+        if (k0 < Kb * 64) *reinterpret_cast<half8 *>(out + lmhip::tiled_index(M + row, k0, Kb)) = l;
+    }
+    if (threadIdx.x == 0) { inv_scale[row] = inv; inv_scale[M + row] = 1.0f / s2; }
+}
+
 // C[m, n] = sum over planes of row m and of row M + m, each times its row factor
 __global__ void reduce_planes_split(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
                                     const float *__restrict__ row_scale, float *__restrict__ C, int M, int N)
@@ -81,12 +132,7 @@ __global__ void reduce_planes_split(const float *__restrict__ P, int S, size_t p
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)M * N) return;
     const int m = (int)(idx / N), n = (int)(idx % N);
-    float hi = 0.f, lo = 0.f;
-    for (int p = 0; p < S; p++) {
-        hi += P[p * plane_stride + (size_t)m * ldp + n];
-        lo += P[p * plane_stride + (size_t)(M + m) * ldp + n];
-    }
-    C[idx] = fmaf(lo, row_scale[M + m], hi * row_scale[m]);
+    C[idx] = lmhip::split_planes_value(P, S, plane_stride, ldp, row_scale, M, m, n);
 }
 
 __global__ void reduce_planes(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
@@ -459,6 +505,22 @@ void gemm_f32a(const float *A, const half_t *Wt, float *C, int M, int Nout, int 
 
 namespace lmhip {
 
+const half_t *tiled_weight_of(MetalBuf *W, int N, int K) { return tiled_copy_of(W, N, K, 0); }
+
+void launch_rows_to_f16_split(const float *A, half_t *a16, float *inv, int M, int K)
+{
+    const bool vec = K % 4 == 0 && ((uintptr_t)A & 15) == 0;
+    if (vec && K <= 8192) hipLaunchKernelGGL(rows_to_f16_split_vec<1>, dim3(M), dim3(1024), 0, stream(), A, K, a16, inv, M, K, tiled_kb(K));
+    else if (vec && K <= 16384) hipLaunchKernelGGL(rows_to_f16_split_vec<2>, dim3(M), dim3(1024), 0, stream(), A, K, a16, inv, M, K, tiled_kb(K));
+    else hipLaunchKernelGGL(rows_to_f16_split, dim3(M), dim3(256), 0, stream(), A, K, a16, inv, M, K, tiled_kb(K));
+}
+
+void launch_reduce_planes_split(const float *P, int S, size_t plane_stride, int ldp, const float *inv, float *C, int M, int N)
+{
+    const size_t n = (size_t)M * N;
+    hipLaunchKernelGGL(reduce_planes_split, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(), P, S, plane_stride, ldp, inv, C, M, N);
+}
+
 // C[M, N] fp32 = A[M, K] fp32 * W^T, W an F16 [N, K] weight buffer, with A split into value and residual rows
 void gemm_f32a_exact(const float *A, MetalBuf *W, float *C, int M, int N, int K)
 {
@@ -466,13 +528,12 @@ void gemm_f32a_exact(const float *A, MetalBuf *W, float *C, int M, int N, int K)
     const int M2 = 2 * M;
     half_t *a16 = (half_t *)scratch(SCR_A16, tiled_elems(M2, K) * sizeof(half_t));
     float *inv = (float *)scratch(SCR_SCALE, (size_t)M2 * sizeof(float));
-    hipLaunchKernelGGL(rows_to_f16_split, dim3(M), dim3(256), 0, stream(), A, K, a16, inv, M, K, tiled_kb(K));
+    launch_rows_to_f16_split(A, a16, inv, M, K);
     GemmPlan p = plan_gemm(M2, N, K);
     const size_t plane = (size_t)M2 * N;
     float *P = (float *)scratch(SCR_PARTIAL, plane * p.S * sizeof(float));
     launch_gemm(a16, nullptr, Wt, P, N, plane, M2, N, K, p);
-    const size_t n = (size_t)M * N;
-    hipLaunchKernelGGL(reduce_planes_split, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream(), P, p.S, plane, N, inv, C, M, N);
+    launch_reduce_planes_split(P, p.S, plane, N, inv, C, M, N);
     HIP_CHECK(hipGetLastError());
 }
 

@@ -370,6 +370,16 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hq0 = blockIdx.x * gpw, hkv = hq0 / G, split = blockIdx.y;
     const int j0 = split * SL, nj = min(SL, n_attend - j0);
+    // blockIdx.z: one of several sequences decoded in lock step (FUSED only), each with its own product row, adapter
+    // terms, caches and output; slice results are kept per (sequence, query head)
+    const int z = blockIdx.z, Hq_all = gridDim.x * gpw;
+    if (FUSED) {
+        hp.qkv += (size_t)z * hp.qkv_step; hp.kc += (size_t)z * hp.cache_step; hp.vc += (size_t)z * hp.cache_step;
+        if (hp.R) hp.t += (size_t)z * hp.t_step;
+        Kc = hp.kc; Vc = hp.vc;
+        out += (size_t)z * Hq_all * hd;
+    }
+    const int hqz0 = z * Hq_all + hq0;                    // first (sequence, query head) of this workgroup
     const float *kbase = Kc + ((size_t)hkv * max_seq + j0) * hd;
     const float *vbase = Vc + ((size_t)hkv * max_seq + j0) * hd;
 
@@ -488,21 +498,20 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
                 if (g0 + u >= gpw) continue;
                 float s = 0.f;
                 for (int pp = 0; pp < parts; pp++) s += red[(pp * 4 + u) * hd + tid];
-                const int hq = hq0 + g0 + u;
-                if (nsplit == 1) out[(size_t)hq * hd + tid] = s / ml[gpw + g0 + u];
-                else part_o[((size_t)hq * nsplit + split) * hd + tid] = s;
+                if (nsplit == 1) out[(size_t)(hq0 + g0 + u) * hd + tid] = s / ml[gpw + g0 + u];
+                else part_o[((size_t)(hqz0 + g0 + u) * nsplit + split) * hd + tid] = s;
             }
         }
         __syncthreads();
     }
     if (nsplit > 1 && tid < gpw) {
-        const int hq = hq0 + tid;
+        const int hq = hqz0 + tid;
         part_ml[((size_t)hq * nsplit + split) * 2] = ml[tid];
         part_ml[((size_t)hq * nsplit + split) * 2 + 1] = ml[gpw + tid];
     }
 }
 
-// merge of the slices of one query head: grid = Hq, block = hd threads (<= 256)
+// merge of the slices of one query head: grid = Hq (times the sequences of a batch), block = hd threads (<= 256)
 __global__ __launch_bounds__(TB) void k_attn_combine(const float *__restrict__ part_o, const float *__restrict__ part_ml,
                                                      float *__restrict__ out, int hd, int nsplit)
 {
@@ -557,47 +566,48 @@ void kv_store(const float *k, const float *v, MetalBuf *kc, MetalBuf *vc, int Hk
 
 // floats of slice results the attention over n_attend keys leaves for its merge kernel: per (query head, slice) hd sums and
 // (max, sum of exponentials); none for a single slice
-size_t attention_partial_floats(int Hq, int hd, int n_attend)
+size_t attention_partial_floats(int Hq, int hd, int n_attend, int copies = 1)
 {
     const int nsplit = (n_attend + SL - 1) / SL;
-    return nsplit > 1 ? (size_t)Hq * nsplit * (hd + 2) : 0;
+    return nsplit > 1 ? (size_t)copies * Hq * nsplit * (hd + 2) : 0;
 }
 
 // The launches of one attention over device pointers whose shapes the caller has checked.  `partials` holds
-// attention_partial_floats(...) floats (unused when that is 0).
+// attention_partial_floats(...) floats (unused when that is 0).  copies > 1 (only with hp): that many sequences at the
+// same position in one launch, their operands hp's steps apart and their outputs Hq * hd floats apart.
 void attention_launch(const float *Q, const float *Kc, const float *Vc, float *out, float *partials, int n_attend, int hd, int max_seq,
-                      int Hq, int G, const HeadPost *hp)
+                      int Hq, int G, const HeadPost *hp, int copies = 1)
 {
     const int nsplit = (n_attend + SL - 1) / SL;
     // short contexts are bound by latency: one query head per workgroup; long ones by cache bytes: the whole group
     const int gpw = n_attend <= 128 ? 1 : G;
     const size_t lds = ((size_t)gpw * hd + (size_t)gpw * SL + 2 * gpw + 4 * 1024) * 4;
-    float *po = nsplit > 1 ? partials : nullptr, *pml = nsplit > 1 ? partials + (size_t)Hq * nsplit * hd : nullptr;
+    float *po = nsplit > 1 ? partials : nullptr, *pml = nsplit > 1 ? partials + (size_t)copies * Hq * nsplit * hd : nullptr;
     const float scale = 1.0f / sqrtf((float)hd);
     const bool vec4 = hd % 4 == 0 && (((uintptr_t)Vc) & 15) == 0;
-    const dim3 grid(Hq / gpw, nsplit);
+    const dim3 grid(Hq / gpw, nsplit, copies);
     const HeadPost none{};
 #define ATTN_LAUNCH(V_, F_) LAUNCH((k_attn_decode<V_, F_>), grid, dim3(TB), lds, Q, Kc, Vc, out, po, pml, \
                                    n_attend, hd, max_seq, G, gpw, scale, nsplit, F_ ? *hp : none)
     if (hp) { if (vec4) ATTN_LAUNCH(4, true); else ATTN_LAUNCH(1, true); }
     else { if (vec4) ATTN_LAUNCH(4, false); else ATTN_LAUNCH(1, false); }
 #undef ATTN_LAUNCH
-    if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq), dim3(TB), 0, po, pml, out, hd, nsplit);
+    if (nsplit > 1) LAUNCH(k_attn_combine, dim3(Hq * copies), dim3(TB), 0, po, pml, out, hd, nsplit);
 }
 
 void attention(const float *Q, MetalBuf *Kc, MetalBuf *Vc, float *out, int n_attend, int hd, int max_seq, int Hq, int G, const char *fn,
-               const HeadPost *hp = nullptr)
+               const HeadPost *hp = nullptr, int copies = 1)
 {
     if (Hq <= 0 || n_attend <= 0) return;
     if (G <= 0 || Hq % G) { fprintf(stderr, "[fast_hip] %s: %d query heads are not a multiple of the group ratio %d; launch skipped\n", fn, Hq, G); return; }
     const int Hkv = Hq / G;
-    REQUIRE_BYTES(Kc, (size_t)Hkv * max_seq * hd * 4, fn);
-    REQUIRE_BYTES(Vc, (size_t)Hkv * max_seq * hd * 4, fn);
+    REQUIRE_BYTES(Kc, (size_t)copies * Hkv * max_seq * hd * 4, fn);
+    REQUIRE_BYTES(Vc, (size_t)copies * Hkv * max_seq * hd * 4, fn);
     if (n_attend > max_seq) { fprintf(stderr, "[fast_hip] %s: n_attend %d exceeds the cache (%d); launch skipped\n", fn, n_attend, max_seq); return; }
     if (hd > 256 || G > 16) { fprintf(stderr, "[fast_hip] %s: head_dim %d / group ratio %d not supported (<= 256 / <= 16); launch skipped\n", fn, hd, G); return; }
-    const size_t pf = attention_partial_floats(Hq, hd, n_attend);
+    const size_t pf = attention_partial_floats(Hq, hd, n_attend, copies);
     float *partials = pf ? (float *)scratch(SCR_MISC, pf * sizeof(float)) : nullptr;
-    attention_launch(Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, partials, n_attend, hd, max_seq, Hq, G, hp);
+    attention_launch(Q, dptr_as<float>(Kc), dptr_as<float>(Vc), out, partials, n_attend, hd, max_seq, Hq, G, hp, copies);
 }
 
 // ---- the attention once more for callers that cannot allocate ------------------------------------------------
@@ -845,12 +855,13 @@ void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q
 }
 
 
-void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq)
+void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq, int copies)
 {
-    if (hp.Hkv <= 0 || hp.Hq % hp.Hkv || (hd & 1) || hp.pos < 0 || hp.pos >= max_seq) {
+    if (hp.Hkv <= 0 || hp.Hq % hp.Hkv || (hd & 1) || hp.pos < 0 || hp.pos >= max_seq || copies < 1 || copies > 65535 ||
+        (copies > 1 && (hp.cache_step != (size_t)hp.Hkv * max_seq * hd || hp.qkv_step < (size_t)(hp.Hq + 2 * hp.Hkv) * hd))) {
         fprintf(stderr, "[fast_hip] attention_decode_fused: unsupported shape\n"); abort();
     }
-    attention(hp.qkv, Kc, Vc, out, hp.pos + 1, hd, max_seq, hp.Hq, hp.Hq / hp.Hkv, "attention_decode_fused", &hp);
+    attention(hp.qkv, Kc, Vc, out, hp.pos + 1, hd, max_seq, hp.Hq, hp.Hq / hp.Hkv, "attention_decode_fused", &hp, copies);
     mark_written(Kc); mark_written(Vc);
 }
 

@@ -133,11 +133,104 @@ __global__ __launch_bounds__(64) void k_lora_down(const float *__restrict__ ln, 
                                                   const float *__restrict__ Av, float *__restrict__ t, int R, int D)
 {
     const int r = blockIdx.x;
+    ln += (size_t)blockIdx.y * D; t += (size_t)blockIdx.y * 2 * R;       // one vector of a batch per blockIdx.y
     const float *a = r < R ? Aq + (size_t)r * D : Av + (size_t)(r - R) * D;
     float s = 0.f;
     for (int i = threadIdx.x; i < D; i += 64) s = fmaf(a[i], ln[i], s);
     s = wave_sum(s);
     if (threadIdx.x == 0) t[r] = s;
+}
+
+// A product of the batched step as the GEMM leaves it (gemm_f32a_exact without its last part): S planes of [2B, N], rows
+// b and B + b the value and residual images of sequence b, inv their factors.
+struct SplitPlanes {
+    const float *P, *inv;
+    size_t plane;
+    int S, N;
+};
+__device__ __forceinline__ float planes_at(const SplitPlanes &p, int B, int b, int n)
+{
+    return split_planes_value(p.P, p.S, p.plane, p.N, p.inv, B, b, n);
+}
+
+// act[b][i] = silu | gelu (gate) * up from the planes of the [gate | up] product of a batch
+__global__ __launch_bounds__(TB) void k_glu_planes(SplitPlanes gu, float *__restrict__ act, int B, int IS, int gelu)
+{
+    const int b = blockIdx.y, i = blockIdx.x * TB + threadIdx.x;
+    if (i >= IS) return;
+    const float g = planes_at(gu, B, b, i), u = planes_at(gu, B, b, IS + i);
+    float a;
+    if (gelu) {                                                           // shaders/q8_kernels.metal:349-362
+        float t = 0.7978845608f * (g + 0.044715f * g * g * g);
+        t = fminf(fmaxf(t, -15.f), 15.f);
+        a = 0.5f * g * (1.0f + tanhf(t));
+    } else a = g / (1.0f + expf(-g));                                     // :337-347
+    act[(size_t)b * IS + i] = a * u;
+}
+
+// k_add_norm for row blockIdx.x of a batch, with the branch taken from a product's planes (br.P) or absent, and with
+// ln also written as the next product's operand: rows b and B + b of the tiled fp16 image a16 [2B, D] and their factors
+// (what rows_to_f16_split makes of ln, element for element).  A thread holds elements tid + 1024 u, u < EPT, so
+// 1024 EPT >= the padded row; the sums run in k_add_norm's order.
+template <int EPT>
+__global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, SplitPlanes br, const float *__restrict__ g_branch,
+                                                         const float *__restrict__ g, float *__restrict__ ln,
+                                                         half_t *__restrict__ a16, float *__restrict__ inv_out, int B, int D, float eps)
+{
+    __shared__ float sm[16];
+    const int b = blockIdx.x, Kb = tiled_kb(D);
+    x += (size_t)b * D;
+    float bv[EPT], v[EPT];
+    float inv_b = 1.f;
+    if (br.P) {
+#pragma unroll
+        for (int u = 0; u < EPT; u++) { const int i = threadIdx.x + 1024 * u; bv[u] = i < D ? planes_at(br, B, b, i) : 0.f; }
+        if (g_branch) {
+            float ss = 0.f;
+#pragma unroll
+            for (int u = 0; u < EPT; u++) ss += bv[u] * bv[u];
+            inv_b = rsqrtf(block_sum(ss, sm) / (float)D + eps);
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < EPT; u++) {
+        const int i = threadIdx.x + 1024 * u;
+        v[u] = 0.f;
+        if (i < D) {
+            v[u] = x[i];
+            if (br.P) { v[u] += g_branch ? bv[u] * inv_b * g_branch[i] : bv[u]; x[i] = v[u]; }
+        }
+        ss += v[u] * v[u];
+    }
+    const float inv = rsqrtf(block_sum(ss, sm) / (float)D + eps);
+    float amax = 0.f;
+#pragma unroll
+    for (int u = 0; u < EPT; u++) {
+        const int i = threadIdx.x + 1024 * u;
+        v[u] = i < D ? v[u] * inv * g[i] : 0.f;
+        if (ln && i < D) ln[(size_t)b * D + i] = v[u];
+        amax = fmaxf(amax, fabsf(v[u]));
+    }
+    amax = block_max(amax, sm);
+    const float s = row_scale_for(amax), is = 1.0f / s;
+    float lmax = 0.f;
+#pragma unroll
+    for (int u = 0; u < EPT; u++) {
+        const int i = threadIdx.x + 1024 * u;
+        const half_t h = f2h(v[u] * s);
+        if (i < Kb * 64) a16[tiled_index(b, i, Kb)] = h;
+        v[u] = v[u] - h2f(h) * is;
+        lmax = fmaxf(lmax, fabsf(v[u]));
+    }
+    lmax = block_max(lmax, sm);
+    const float s2 = row_scale_for(lmax);
+#pragma unroll
+    for (int u = 0; u < EPT; u++) {
+        const int i = threadIdx.x + 1024 * u;
+        if (i < Kb * 64) a16[tiled_index(B + b, i, Kb)] = f2h(v[u] * s2);
+    }
+    if (threadIdx.x == 0) { inv_out[b] = is; inv_out[B + b] = 1.0f / s2; }
 }
 
 MetalBuf *fbuf(size_t n) { return metal_buf_create(n * sizeof(float)); }
@@ -559,102 +652,133 @@ int inference_generate(InferenceState *s, const uint32_t *prompt_tokens, int pro
 
 namespace {
 
-// act[b][i] = silu | gelu (gu[b][i]) * gu[b][IS + i]: the gated activation of a batch from the [gate | up] product
-__global__ __launch_bounds__(TB) void k_glu_batch(const float *__restrict__ gu, float *__restrict__ act, int IS, int gelu)
+// the embedding rows of a batch of tokens, scaled: x[b] = emb[tokens.id[b]] * scale
+struct TokenIds { int id[32]; };
+__global__ __launch_bounds__(TB) void k_embed_rows(const float *__restrict__ emb, TokenIds tokens, float scale, float *__restrict__ x, int D)
 {
-    const int b = blockIdx.y, i = blockIdx.x * TB + threadIdx.x;
-    if (i >= IS) return;
-    const float g = gu[(size_t)b * 2 * IS + i], u = gu[(size_t)b * 2 * IS + IS + i];
-    float a;
-    if (gelu) {                                                           // shaders/q8_kernels.metal:349-362
-        float t = 0.7978845608f * (g + 0.044715f * g * g * g);
-        t = fminf(fmaxf(t, -15.f), 15.f);
-        a = 0.5f * g * (1.0f + tanhf(t));
-    } else a = g / (1.0f + expf(-g));                                     // :337-347
-    act[(size_t)b * IS + i] = a * u;
+    const int i = blockIdx.x * TB + threadIdx.x, b = blockIdx.y;
+    if (i < D) x[(size_t)b * D + i] = emb[(size_t)tokens.id[b] * D + i] * scale;
+}
+
+// k_argmax_part and k_argmax_final for every vector of a batch at once (blockIdx.y: the vector)
+__global__ __launch_bounds__(TB) void k_argmax_part_batch(const float *__restrict__ v, int n, float *__restrict__ pv, int *__restrict__ pi)
+{
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    v += (size_t)blockIdx.y * n; pv += (size_t)blockIdx.y * AM_WGS; pi += (size_t)blockIdx.y * AM_WGS;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = blockIdx.x * TB + threadIdx.x; i < n; i += AM_WGS * TB) am_pick(best, idx, v[i], i);
+    am_block(best, idx, bv, bi);
+    if (threadIdx.x == 0) { pv[blockIdx.x] = best; pi[blockIdx.x] = idx; }
+}
+
+__global__ __launch_bounds__(AM_WGS) void k_argmax_final_batch(const float *__restrict__ pv, const int *__restrict__ pi, int *__restrict__ out)
+{
+    __shared__ float bv[AM_WGS / 64];
+    __shared__ int bi[AM_WGS / 64];
+    float best = pv[(size_t)blockIdx.x * AM_WGS + threadIdx.x];
+    int idx = pi[(size_t)blockIdx.x * AM_WGS + threadIdx.x];
+    am_block(best, idx, bv, bi);
+    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
 }
 
 // Scratch and KV caches of a batch of B sequences decoded in lock step (BatchState of src/nn/fast_inference.c:699-776).
 struct BatchRun {
     int B;
-    MetalBuf *x, *branch, *ln, *qkv, *att, *gu, *act, *logits, *best, *lora_t;
-    std::vector<MetalBuf *> kc, vc;                                      // [layer * B + item]
+    MetalBuf *x, *ln, *qkv, *att, *act, *logits, *best, *lora_t;
+    MetalBuf *a16, *inv_ln, *inv_br, *planes;                            // a product's operand, its factors (of ln | of att and act), its planes
+    std::vector<MetalBuf *> kc, vc;                                      // per layer: [B][Hkv, max_seq, hd]
     int *best_host;
 };
 
 void batch_free(BatchRun &r)
 {
-    for (MetalBuf *b : {r.x, r.branch, r.ln, r.qkv, r.att, r.gu, r.act, r.logits, r.best, r.lora_t}) metal_buf_free(b);
+    for (MetalBuf *b : {r.x, r.ln, r.qkv, r.att, r.act, r.logits, r.best, r.lora_t, r.a16, r.inv_ln, r.inv_br, r.planes}) metal_buf_free(b);
     for (MetalBuf *b : r.kc) metal_buf_free(b);
     for (MetalBuf *b : r.vc) metal_buf_free(b);
     if (r.best_host) hipHostFree(r.best_host);
 }
 
 // One step for B tokens at the same position: forward_token_batch, src/nn/fast_inference.c:808-893.  Every product
-// reads its weight once for all B vectors (matrix cores over the tiled image, gemm_f32a_exact); what is per sequence
-// -- adapter terms, per-head RMSNorm, RoPE, cache store, attention -- is one launch per sequence and layer.
+// reads its weight once for all B vectors (matrix cores over the tiled image, the arithmetic of gemm_f32a_exact); what
+// is per sequence -- adapter terms, per-head RMSNorm, RoPE, cache store, attention -- has the sequence as a grid
+// dimension, so a layer is the same 11 launches (12 with adapters) for any B.  A product's planes are summed by the kernel
+// that consumes them and the norm kernel writes the next product's operand itself, where a row is one workgroup's.
 void forward_token_batch(InferenceState *s, BatchRun &r, const int *tokens, int pos)
 {
     const int D = s->D, Hq = s->Hq, Hkv = s->Hkv, hd = s->hd, IS = s->IS, B = r.B;
     const int qd = Hq * hd, kd = Hkv * hd, nqkv = qd + 2 * kd;
     const bool gemma = s->model_type == MODEL_GEMMA3;
-    for (int b = 0; b < B; b++)
-        hipLaunchKernelGGL(k_embed_row, dim3((D + TB - 1) / TB), dim3(TB), 0, stream(), dptr_as<float>(s->emb), tokens[b], s->emb_scale,
-                           dptr_as<float>(r.x) + (size_t)b * D, D);
-    auto add_norm_b = [&](MetalBuf *branch, MetalBuf *g_branch, MetalBuf *g) {
-        hipLaunchKernelGGL(k_add_norm, dim3(B), dim3(1024), 0, stream(), dptr_as<float>(r.x), branch ? dptr_as<float>(branch) : nullptr,
-                           g_branch ? dptr_as<float>(g_branch) : nullptr, dptr_as<float>(g), dptr_as<float>(r.ln), D, s->eps);
+    TokenIds ids{};
+    for (int b = 0; b < B; b++) ids.id[b] = tokens[b];
+    hipLaunchKernelGGL(k_embed_rows, dim3((D + TB - 1) / TB, B), dim3(TB), 0, stream(), dptr_as<float>(s->emb), ids, s->emb_scale,
+                       dptr_as<float>(r.x), D);
+    half_t *a16 = dptr_as<half_t>(r.a16);
+    float *inv_ln = dptr_as<float>(r.inv_ln), *inv_br = dptr_as<float>(r.inv_br), *P = dptr_as<float>(r.planes);
+    // x += branch (the planes `br` of the product before, none at the start); ln = RMSNorm(x) as fp32 (only the adapters
+    // read it) and as the operand of the next product
+    auto add_norm_b = [&](const SplitPlanes &br, MetalBuf *g_branch, MetalBuf *g) {
+        float *ln = s->lora.empty() ? nullptr : dptr_as<float>(r.ln);
+        const float *gb = g_branch ? dptr_as<float>(g_branch) : nullptr;
+        if (tiled_kb(D) * 64 <= 4096)
+            hipLaunchKernelGGL(k_add_norm_split<4>, dim3(B), dim3(1024), 0, stream(), dptr_as<float>(r.x), br, gb, dptr_as<float>(g), ln,
+                               a16, inv_ln, B, D, s->eps);
+        else
+            hipLaunchKernelGGL(k_add_norm_split<8>, dim3(B), dim3(1024), 0, stream(), dptr_as<float>(r.x), br, gb, dptr_as<float>(g), ln,
+                               a16, inv_ln, B, D, s->eps);
     };
-    auto product = [&](const WMat *w, MetalBuf *in, MetalBuf *out) {
-        gemm_f32a_exact(dptr_as<float>(in), w->mbuf, dptr_as<float>(out), B, w->rows, w->cols);
-        mark_written(out);
+    // planes of (the operand in a16) x w^T; `inv`: the factors that operand's rows were split with
+    auto product = [&](const WMat *w, const float *inv) {
+        const GemmPlan p = plan_gemm(2 * B, w->rows, w->cols);
+        const size_t plane = (size_t)2 * B * w->rows;
+        launch_gemm(a16, nullptr, tiled_weight_of(w->mbuf, w->rows, w->cols), P, w->rows, plane, 2 * B, w->rows, w->cols, p);
+        return SplitPlanes{P, inv, plane, p.S, w->rows};
     };
-    MetalBuf *pending = nullptr, *pending_g = nullptr;
+    auto split = [&](MetalBuf *in, int K) { launch_rows_to_f16_split(dptr_as<float>(in), a16, inv_br, B, K); };
+    SplitPlanes pending{};                                               // FFN branch of the layer before, added by the next norm kernel
+    MetalBuf *pending_g = nullptr;
     for (int L = 0; L < s->NL; L++) {
         const InferenceState::Layer &lw = s->layers[L];
         add_norm_b(pending, pending_g, lw.g_in);
-        product(&lw.qkv, r.ln, r.qkv);
-        for (int b = 0; b < B; b++) {
-            HeadPost a{};
-            a.qkv = dptr_as<float>(r.qkv) + (size_t)b * nqkv;
-            a.g_q = lw.g_q ? dptr_as<float>(lw.g_q) : nullptr; a.g_k = lw.g_k ? dptr_as<float>(lw.g_k) : nullptr;
-            MetalBuf *kc = r.kc[(size_t)L * B + b], *vc = r.vc[(size_t)L * B + b];
-            a.kc = dptr_as<float>(kc); a.vc = dptr_as<float>(vc);
-            a.Hq = Hq; a.Hkv = Hkv; a.pos = pos;
-            a.rope = dptr_as<float2>(s->rope_tabs) + ((size_t)s->theta_slot[L] * s->max_seq + pos) * (hd / 2); a.eps = s->eps;
-            if (!s->lora.empty()) {
-                const InferenceState::Lora &lr = s->lora[L];
-                float *t = dptr_as<float>(r.lora_t) + (size_t)b * 2 * s->R;
-                hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R), dim3(64), 0, stream(), dptr_as<float>(r.ln) + (size_t)b * D,
-                                   dptr_as<float>(lr.Aq), dptr_as<float>(lr.Av), t, s->R, D);
-                a.t = t; a.Bq = dptr_as<float>(lr.Bq); a.Bv = dptr_as<float>(lr.Bv); a.R = s->R; a.sc = s->scaling;
-            }
-            attention_decode_fused(a, kc, vc, dptr_as<float>(r.att) + (size_t)b * qd, hd, s->max_seq);
+        const SplitPlanes qkv = product(&lw.qkv, inv_ln);
+        launch_reduce_planes_split(qkv.P, qkv.S, qkv.plane, qkv.N, qkv.inv, dptr_as<float>(r.qkv), B, qkv.N);
+        HeadPost a{};
+        a.qkv = dptr_as<float>(r.qkv); a.qkv_step = (size_t)nqkv;
+        a.g_q = lw.g_q ? dptr_as<float>(lw.g_q) : nullptr; a.g_k = lw.g_k ? dptr_as<float>(lw.g_k) : nullptr;
+        a.kc = dptr_as<float>(r.kc[L]); a.vc = dptr_as<float>(r.vc[L]); a.cache_step = (size_t)Hkv * s->max_seq * hd;
+        a.Hq = Hq; a.Hkv = Hkv; a.pos = pos;
+        a.rope = dptr_as<float2>(s->rope_tabs) + ((size_t)s->theta_slot[L] * s->max_seq + pos) * (hd / 2); a.eps = s->eps;
+        if (!s->lora.empty()) {
+            const InferenceState::Lora &lr = s->lora[L];
+            hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R, B), dim3(64), 0, stream(), dptr_as<float>(r.ln), dptr_as<float>(lr.Aq),
+                               dptr_as<float>(lr.Av), dptr_as<float>(r.lora_t), s->R, D);
+            a.t = dptr_as<float>(r.lora_t); a.t_step = (size_t)2 * s->R;
+            a.Bq = dptr_as<float>(lr.Bq); a.Bv = dptr_as<float>(lr.Bv); a.R = s->R; a.sc = s->scaling;
         }
-        mark_written(r.att);
-        product(lw.o, r.att, r.branch);
-        add_norm_b(r.branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
-        product(&lw.gu, r.ln, r.gu);
-        hipLaunchKernelGGL(k_glu_batch, dim3((IS + TB - 1) / TB, B), dim3(TB), 0, stream(), dptr_as<float>(r.gu), dptr_as<float>(r.act), IS,
-                           gemma ? 1 : 0);
-        product(lw.down, r.act, r.branch);
-        pending = r.branch;
+        attention_decode_fused(a, r.kc[L], r.vc[L], dptr_as<float>(r.att), hd, s->max_seq, B);
+        split(r.att, qd);
+        const SplitPlanes o = product(lw.o, inv_br);
+        add_norm_b(o, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
+        const SplitPlanes gu = product(&lw.gu, inv_ln);
+        hipLaunchKernelGGL(k_glu_planes, dim3((IS + TB - 1) / TB, B), dim3(TB), 0, stream(), gu, dptr_as<float>(r.act), B, IS, gemma ? 1 : 0);
+        split(r.act, IS);
+        pending = product(lw.down, inv_br);
         pending_g = gemma ? lw.g_post_ff : nullptr;
     }
     add_norm_b(pending, pending_g, s->g_final);
-    product(s->lm_head, r.ln, r.logits);
+    const SplitPlanes lg = product(s->lm_head, inv_ln);
+    launch_reduce_planes_split(lg.P, lg.S, lg.plane, lg.N, lg.inv, dptr_as<float>(r.logits), B, lg.N);
     HIP_CHECK(hipGetLastError());
 }
 
 // argmax of every sequence's logits, computed on the GPU; one wait for all of them
 void argmax_batch(InferenceState *s, BatchRun &r, int *out)
 {
-    for (int b = 0; b < r.B; b++) {
-        float *pv = dptr_as<float>(r.best) + r.B + (size_t)b * 2 * AM_WGS;
-        int *pi = reinterpret_cast<int *>(pv) + AM_WGS;
-        hipLaunchKernelGGL(k_argmax_part, dim3(AM_WGS), dim3(TB), 0, stream(), dptr_as<float>(r.logits) + (size_t)b * s->V, s->V, pv, pi);
-        hipLaunchKernelGGL(k_argmax_final, dim3(1), dim3(AM_WGS), 0, stream(), pv, pi, dptr_as<int>(r.best) + b);
-    }
+    float *pv = dptr_as<float>(r.best) + r.B;                            // [B][AM_WGS] values, then as many indices
+    int *pi = reinterpret_cast<int *>(pv) + (size_t)r.B * AM_WGS;
+    hipLaunchKernelGGL(k_argmax_part_batch, dim3(AM_WGS, r.B), dim3(TB), 0, stream(), dptr_as<float>(r.logits), s->V, pv, pi);
+    hipLaunchKernelGGL(k_argmax_final_batch, dim3(r.B), dim3(AM_WGS), 0, stream(), pv, pi, dptr_as<int>(r.best));
     HIP_CHECK(hipMemcpyAsync(r.best_host, dptr(r.best), (size_t)r.B * sizeof(int), hipMemcpyDeviceToHost, stream()));
     HIP_CHECK(hipStreamSynchronize(stream()));
     for (int b = 0; b < r.B; b++) out[b] = r.best_host[b];
@@ -674,19 +798,28 @@ int inference_generate_batch(InferenceState *s, const uint32_t *prompt_tokens, i
     const int B = batch_size;
     if (!s->use_fp16) { fprintf(stderr, "[BatchGen] F16 weights only\n"); return 0; }
     if (B < 1 || B > 32 || prompt_len <= 0 || max_gen_len <= 0 || prompt_len > s->max_seq) return 0;
+    if (s->D > 8192) { fprintf(stderr, "[BatchGen] hidden size %d not supported (<= 8192)\n", s->D); return 0; }
     for (int i = 0; i < prompt_len; i++)
         if (prompt_tokens[i] >= (uint32_t)s->V) { fprintf(stderr, "[BatchGen] token %u outside the vocabulary (%d)\n", prompt_tokens[i], s->V); return 0; }
     const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS, V = s->V;
     BatchRun r{};
     r.B = B;
-    r.x = fbuf((size_t)B * D); r.branch = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
+    r.x = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
     r.qkv = fbuf((size_t)B * (qd + 2 * kd)); r.att = fbuf((size_t)B * qd);
-    r.gu = fbuf((size_t)B * 2 * IS); r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
+    r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
+    size_t a16_elems = 0, plane_floats = 0;                              // the largest operand and planes of the step's products
+    const int shapes[5][2] = {{qd + 2 * kd, D}, {D, qd}, {2 * IS, D}, {D, IS}, {V, D}};
+    for (const auto &nk : shapes) {
+        a16_elems = std::max(a16_elems, tiled_elems(2 * B, nk[1]));
+        plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1]).S * 2 * B * nk[0]);
+    }
+    r.a16 = metal_buf_create(a16_elems * sizeof(half_t)); r.planes = fbuf(plane_floats);
+    r.inv_ln = fbuf((size_t)2 * B); r.inv_br = fbuf((size_t)2 * B);
     r.best = metal_buf_create(((size_t)B + (size_t)B * 2 * AM_WGS) * sizeof(int));
     r.lora_t = s->lora.empty() ? nullptr : fbuf((size_t)B * 2 * s->R);
     HIP_CHECK(hipHostMalloc((void **)&r.best_host, (size_t)B * sizeof(int), hipHostMallocDefault));
     const size_t cache_bytes = (size_t)s->Hkv * s->max_seq * s->hd * sizeof(float);
-    for (int i = 0; i < s->NL * B; i++) { r.kc.push_back(metal_buf_create(cache_bytes)); r.vc.push_back(metal_buf_create(cache_bytes)); }
+    for (int L = 0; L < s->NL; L++) { r.kc.push_back(metal_buf_create(cache_bytes * B)); r.vc.push_back(metal_buf_create(cache_bytes * B)); }
 
     int tokens[32], next[32], active[32];
     for (int i = 0; i < prompt_len; i++) {                               // prefill: the same token for every sequence (:910-916)

@@ -71,19 +71,25 @@ def test_forward_token_logits_and_greedy_generation(cfg, fmt):
         assert inf.forward_token_argmax(c.V) == -1 and inf.position() == 0
 
 
-@pytest.mark.parametrize("cfg,with_lora", [(C1.with_(seq=8), False), (TINY_GEMMA, False), (C1.with_(seq=8), True)],
-                         ids=["qwen3", "gemma3", "qwen3_adapters"])
-def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, with_lora):
+@pytest.mark.parametrize("cfg,with_lora,n_prompt", [(C1.with_(seq=8), False, 4), (TINY_GEMMA, False, 4), (C1.with_(seq=8), True, 4),
+                                                    (C1.with_(seq=8), True, 270)],
+                         ids=["qwen3", "gemma3", "qwen3_adapters", "qwen3_adapters_two_key_slices"])
+def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, with_lora, n_prompt):
     """inference_generate_batch (qwen3_generate_fast_batch, src/nn/fast_inference.c:895-1000): B copies of one prompt
     in lock step, weights read once per step.  Every copy must produce the single-sequence greedy tokens (wherever the
     choice was not a near-tie: the batched products keep 22 bits of the activations, the single ones all 24), the
-    oracle's decode chain must agree with them, and an end token stops the loop once all copies have emitted it."""
-    say("batched generation", cfg.name, with_lora)
+    oracle's decode chain must agree with them, and an end token stops the loop once all copies have emitted it.
+    The 270-token prompt puts the context beyond one slice of keys, where every copy's slice results are merged."""
+    say("batched generation", cfg.name, with_lora, n_prompt)
     c = cfg
     model = make_model(c, seed=17, gamma_jitter=0.1)
-    tok, _ = make_batch(c, seed=18)
-    prompt = [int(t) for t in tok[:4]]
+    if n_prompt <= 8:
+        tok, _ = make_batch(c, seed=18)
+        prompt = [int(t) for t in tok[:n_prompt]]
+    else:
+        prompt = [int(t) for t in np.random.default_rng(18).integers(1, c.V, n_prompt)]
     B, n = 5, 12
+    max_seq = 32 if n_prompt <= 8 else n_prompt + n + 6
 
     def check(inf, lora):
         single = [int(g) for g in inf.generate(prompt, n)]
@@ -91,7 +97,7 @@ def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, wit
         pos = inf.position()
         got = inf.generate_batch(prompt, n, B)
         assert got.shape == (B, n) and inf.position() == pos          # its own caches: the state's are left alone
-        lo = oracle_decode(c, model, "f16", prompt + single[:-1], max_seq=32, precision="f32", lora=lora)[len(prompt) - 1:]
+        lo = oracle_decode(c, model, "f16", prompt + single[:-1], max_seq=max_seq, precision="f32", lora=lora)[len(prompt) - 1:]
         srt = np.sort(lo, axis=1)
         clear = (srt[:, -1] - srt[:, -2]) > 1e-3 * np.abs(lo).max()
         first_tie = n if clear.all() else int(np.argmin(clear))        # after a near-tie the sequences may part ways
@@ -111,12 +117,12 @@ def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, wit
 
     if with_lora:
         with SFTState(c, model) as sft:
-            with InferenceState(sft=sft, max_seq=32) as inf:
+            with InferenceState(sft=sft, max_seq=max_seq) as inf:
                 check(inf, model["lora"])
     else:
-        with InferenceState(c, model, max_seq=32, use_fp16=True) as inf:
+        with InferenceState(c, model, max_seq=max_seq, use_fp16=True) as inf:
             check(inf, None)
-        with InferenceState(c, model, max_seq=32, use_fp16=False) as q8:
+        with InferenceState(c, model, max_seq=max_seq, use_fp16=False) as q8:
             assert q8.generate_batch(prompt, n, 2).shape[1] == 0       # F16 weights only, as in the reference
 
 
