@@ -263,24 +263,31 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq)
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), m_tiles = (M + 63) / 64;
     const int cus = num_cus() > 0 ? num_cus() : 256;
     GemmPlan p{};
-    p.nb = g_force_nb ? g_force_nb : (Nb >= 2 ? 2 : 1);
-    if (nbq & 1) p.nb = 1;                                 // a workgroup must not straddle the Q8_0 / F16 boundary
     p.nw = 4;
-    p.n_tiles = (Nb + p.nb - 1) / p.nb;
     p.m_tiles = m_tiles;
-    const int base = p.n_tiles * m_tiles;
-    // about twelve waves per CU in flight, whatever the workgroup size
-    int S = g_force_S ? g_force_S : (3 * cus + base - 1) / base;
-    if (S < 1) S = 1;
-    int steps = (Kb + S - 1) / S;
-    if (!g_force_S) {
-        if (steps < p.nw) steps = p.nw;
-        if (steps > 10 * p.nw) steps = 10 * p.nw;
-    }
-    steps = (steps + p.nw - 1) / p.nw * p.nw;              // whole steps for each wave
-    if (steps > Kb) steps = Kb;
-    p.steps = steps;
-    p.S = (Kb + steps - 1) / steps;
+    auto split = [&](int nb) {
+        p.nb = nb;
+        p.n_tiles = (Nb + nb - 1) / nb;
+        const int base = p.n_tiles * m_tiles;
+        // about twelve waves per CU in flight, whatever the workgroup size
+        int S = g_force_S ? g_force_S : (3 * cus + base - 1) / base;
+        if (S < 1) S = 1;
+        int steps = (Kb + S - 1) / S;
+        if (!g_force_S) {
+            if (steps < p.nw) steps = p.nw;
+            if (steps > 10 * p.nw) steps = 10 * p.nw;
+        }
+        steps = (steps + p.nw - 1) / p.nw * p.nw;          // whole steps for each wave
+        if (steps > Kb) steps = Kb;
+        p.steps = steps;
+        p.S = (Kb + steps - 1) / steps;
+    };
+    int nb = g_force_nb ? g_force_nb : (Nb >= 2 ? 2 : 1);
+    if (nbq & 1) nb = 1;                                   // a workgroup must not straddle the Q8_0 / F16 boundary
+    split(nb);
+    // a product too small to give every CU a workgroup of 64 weight rows (K is short as well) takes 32-row workgroups:
+    // measured on 1152 x 1024 .. 1568 x 1152 at 64 rows, 4.3-4.6 us against 5.2-5.5
+    if (!g_force_nb && p.nb == 2 && m_tiles == 1 && p.n_tiles * p.S < cus) split(1);
     // rotate the K order unless the activation matrix is too big to stay in an XCD's L2
     p.rotate = (size_t)tiled_rb(M) * 32 * Kb * 64 * 2 <= (size_t)4 << 20;
     return p;
