@@ -59,6 +59,15 @@ void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, floa
 
 // infer_kernels.hip: y[i] = act(gate_i . x) * (up_i . x) for W = [gate; up] of 2 * rows rows (F16, or Q8_0 blocks when q8)
 void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q8, int gelu);
+// The vector of a product as the sum and norm before it left it: RMSNorm(xr + br; g) with br optional; xr + br goes to
+// x_out (another buffer than xr) when that is given.
+struct NormIn {
+    const float *xr, *br, *g;
+    float *x_out;
+    float eps;
+};
+// infer_kernels.hip: y = W . RMSNorm(xr + br; g) (glu 0), or the gated pair product of matvec_glu over it (1 SiLU, 2 GELU)
+void matvec_norm(MetalBuf *W, const NormIn &nin, MetalBuf *y, int rows, int cols, int q8, int glu);
 
 }  // namespace lmhip
 

@@ -93,26 +93,38 @@ const int8_t *q8_split_of(MetalBuf *W, int rows, int nb, const half_t **scales)
 // (q + 128, one v_cvt_f32_ubyte each) and the bias is taken out with the lane's sum of x, once per step for all rows.
 // GLU (1 SiLU, 2 GELU; R = 2): the matrix is [gate; up] with `rows` rows each; a wave takes gate row i and up row i and
 // writes act(gate . x) * (up . x), the gated product the FFN forms next, in place of the two sums.
-template <int FMT, int R, int U, int XLDS, int GLU = 0>
+// NORM (with XLDS): the vector is RMSNorm(v; g) of v = xr + br (br may be null), which every workgroup forms for itself
+// while its first weights are on their way: v g goes to LDS, the sum of squares through one block reduction, and the
+// factor rsqrt(mean + eps) onto the finished sums; workgroup 0 also writes v to x_out (not xr: the others still read it).
+// residual_add + rms_norm of shaders/q8_kernels.metal:133-158, 369-375 without a launch of their own.
+// REPS (NORM only): row groups a wave takes one after the other, so that fewer workgroups form the vector.
+template <int FMT, int R, int U, int XLDS, int GLU = 0, int NORM = 0, int REPS = 1>
 __global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, const half_t *__restrict__ scales,
-                                               const float *__restrict__ x, float *__restrict__ y, int rows, int cols)
+                                               const float *__restrict__ x, float *__restrict__ y, int rows, int cols, NormIn nin)
 {
     static_assert(GLU == 0 || R == 2, "the gated variant pairs two rows");
+    static_assert(NORM == 0 || XLDS == 1, "the normed vector is staged in LDS");
     extern __shared__ float xs[];                               // [cols] when XLDS
+    __shared__ float red[16];
     struct Stage {
         half8   w16[FMT == 0 ? R : 1][U];
         uint2v  w8[FMT == 1 ? R : 1][U];
         float   dsc[FMT == 1 ? R : 1][U];
         float4v x0[XLDS ? 1 : U], x1[XLDS ? 1 : U];
     };
+    static_assert(REPS == 1 || NORM == 1, "row groups in turn only where the vector is formed in the kernel");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row0 = (blockIdx.x * 4 + wave) * (GLU ? 1 : R);
+    int row0 = ((blockIdx.x * REPS) * 4 + wave) * (GLU ? 1 : R);
     size_t roff[R];                                             // element offset of each row (clamped: extra rows are not stored)
-#pragma unroll
-    for (int r = 0; r < R; r++) roff[r] = GLU ? ((size_t)r * rows + min(row0, rows - 1)) * cols : (size_t)min(row0 + r, rows - 1) * cols;
     float acc[R];
+    auto set_rows = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r] = 0.f;
+        for (int r = 0; r < R; r++) {
+            roff[r] = GLU ? ((size_t)r * rows + min(row0, rows - 1)) * cols : (size_t)min(row0 + r, rows - 1) * cols;
+            acc[r] = 0.f;
+        }
+    };
+    set_rows();
 
     auto load = [&](Stage &g, int c) __attribute__((always_inline)) {
 #pragma unroll
@@ -171,27 +183,58 @@ __global__ __launch_bounds__(TB) void k_matvec(const void *__restrict__ Wp, cons
 
     Stage cur;
     load(cur, lane * 8);
-    if (XLDS) {
+    float norm_inv = 1.f;
+    if (NORM) {
+        float ss = 0.f;
+        for (int i0 = tid * 4; i0 < cols; i0 += TB * 16) {      // four groups of a thread requested together
+            float4v v[4], b[4], gg[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = min(i0 + u * TB * 4, cols - 4);
+                v[u] = *reinterpret_cast<const float4v *>(&nin.xr[i]);
+                if (nin.br) b[u] = *reinterpret_cast<const float4v *>(&nin.br[i]);
+                gg[u] = *reinterpret_cast<const float4v *>(&nin.g[i]);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = i0 + u * TB * 4;
+                if (i >= cols) break;
+                if (nin.br) v[u] += b[u];
+                ss += v[u][0] * v[u][0] + v[u][1] * v[u][1] + v[u][2] * v[u][2] + v[u][3] * v[u][3];
+                *reinterpret_cast<float4v *>(&xs[i]) = v[u] * gg[u];
+                if (blockIdx.x == 0 && nin.x_out) *reinterpret_cast<float4v *>(&nin.x_out[i]) = v[u];
+            }
+        }
+        norm_inv = rsqrtf(block_sum(ss, red) / (float)cols + nin.eps);      // its barriers also publish xs
+    } else if (XLDS) {
         for (int i = tid * 4; i < cols; i += TB * 4)
             *reinterpret_cast<float4v *>(&xs[i]) = *reinterpret_cast<const float4v *>(&x[i]);
         __syncthreads();
     }
-    for (int c = lane * 8; c < cols; c += 512 * U) {
-        Stage nxt;
-        load(nxt, c + 512 * U);
-        use(cur, c);
-        cur = nxt;
-    }
-    if (GLU) {
-        const float g = wave_sum(acc[0]), u = wave_sum(acc[R - 1]);
-        if (lane == 0 && row0 < rows)                           // the expressions of silu_mul / gelu_mul
-            y[row0] = (GLU == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + tanhf(gelu_inner(g)))) * u;
-        return;
-    }
+#pragma unroll 1
+    for (int rep = 0; rep < REPS; rep++) {
+        if (rep) {                                              // the next group of rows, with the same vector
+            row0 += 4 * (GLU ? 1 : R);
+            set_rows();
+            load(cur, lane * 8);
+        }
+        for (int c = lane * 8; c < cols; c += 512 * U) {
+            Stage nxt;
+            load(nxt, c + 512 * U);
+            use(cur, c);
+            cur = nxt;
+        }
+        if (GLU) {
+            const float g = wave_sum(acc[0]) * norm_inv, u = wave_sum(acc[R - 1]) * norm_inv;
+            if (lane == 0 && row0 < rows)                       // the expressions of silu_mul / gelu_mul
+                y[row0] = (GLU == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + tanhf(gelu_inner(g)))) * u;
+        } else {
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        const float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < rows) y[row0 + r] = s;
+            for (int r = 0; r < R; r++) {
+                const float s = wave_sum(acc[r]) * norm_inv;
+                if (lane == 0 && row0 + r < rows) y[row0 + r] = s;
+            }
+        }
     }
 }
 
@@ -222,8 +265,8 @@ void launch_matvec(const void *W, const half_t *scales, const float *x, float *y
     const bool prof = gemm_prof_begin((double)rows * cols * (FMT == 0 ? 2.0 : 34.0 / 32.0), 2.0 * rows * cols, &ev_a, &ev_b);
 #define MATVEC_LAUNCH(R_, U_, XL_, RPW_, L_) do { \
     const dim3 grid((rows + RPW_ - 1) / RPW_); \
-    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, R_, U_, XL_>), grid, dim3(TB), L_, stream(), ev_a, ev_b, 0, W, scales, x, y, rows, cols); \
-    else hipLaunchKernelGGL((k_matvec<FMT, R_, U_, XL_>), grid, dim3(TB), L_, stream(), W, scales, x, y, rows, cols); \
+    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, R_, U_, XL_>), grid, dim3(TB), L_, stream(), ev_a, ev_b, 0, W, scales, x, y, rows, cols, NormIn{}); \
+    else hipLaunchKernelGGL((k_matvec<FMT, R_, U_, XL_>), grid, dim3(TB), L_, stream(), W, scales, x, y, rows, cols, NormIn{}); \
     HIP_CHECK(hipGetLastError()); } while (0)
     if (rows >= 32768 && lds <= 40 * 1024) MATVEC_LAUNCH(4, 2, 1, 16, lds);
     else if (rows >= 32768) MATVEC_LAUNCH(4, 2, 0, 16, 0);
@@ -240,11 +283,30 @@ void launch_matvec_glu(const void *W, const half_t *scales, const float *x, floa
     const bool prof = gemm_prof_begin(2.0 * rows * cols * (FMT == 0 ? 2.0 : 34.0 / 32.0), 4.0 * rows * cols, &ev_a, &ev_b);
     const dim3 grid((rows + 3) / 4);
 #define GLU_LAUNCH(G_) do { \
-    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, 2, 2, 0, G_>), grid, dim3(TB), 0, stream(), ev_a, ev_b, 0, W, scales, x, y, rows, cols); \
-    else hipLaunchKernelGGL((k_matvec<FMT, 2, 2, 0, G_>), grid, dim3(TB), 0, stream(), W, scales, x, y, rows, cols); \
+    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, 2, 2, 0, G_>), grid, dim3(TB), 0, stream(), ev_a, ev_b, 0, W, scales, x, y, rows, cols, NormIn{}); \
+    else hipLaunchKernelGGL((k_matvec<FMT, 2, 2, 0, G_>), grid, dim3(TB), 0, stream(), W, scales, x, y, rows, cols, NormIn{}); \
     HIP_CHECK(hipGetLastError()); } while (0)
     if (gelu) GLU_LAUNCH(2); else GLU_LAUNCH(1);
 #undef GLU_LAUNCH
+}
+
+// Either product over RMSNorm(xr + br; g), formed by the kernel itself (NORM): glu 0 plain rows, 1 SiLU, 2 GELU pairs.
+template <int FMT>
+void launch_matvec_norm(const void *W, const half_t *scales, const NormIn &nin, float *y, int rows, int cols, int glu)
+{
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+    const double mats = glu ? 2.0 : 1.0;
+    const bool prof = gemm_prof_begin(mats * rows * cols * (FMT == 0 ? 2.0 : 34.0 / 32.0), 2.0 * mats * rows * cols, &ev_a, &ev_b);
+    const size_t lds = (size_t)cols * 4;
+#define NORM_LAUNCH(G_, RPW_, REPS_) do { \
+    const dim3 grid((rows + RPW_ * REPS_ - 1) / (RPW_ * REPS_)); \
+    if (prof) hipExtLaunchKernelGGL((k_matvec<FMT, 2, 2, 1, G_, 1, REPS_>), grid, dim3(TB), lds, stream(), ev_a, ev_b, 0, W, scales, nullptr, y, rows, cols, nin); \
+    else hipLaunchKernelGGL((k_matvec<FMT, 2, 2, 1, G_, 1, REPS_>), grid, dim3(TB), lds, stream(), W, scales, nullptr, y, rows, cols, nin); \
+    HIP_CHECK(hipGetLastError()); } while (0)
+    // measured at 9728 x 2560 pairs and 6144 x 2560 rows: two row groups per wave for the pairs (2432 workgroups forming
+    // the vector cost what the norm's own launch did), one for the rows (384 workgroups leave CUs idle)
+    if (glu == 0) NORM_LAUNCH(0, 8, 1); else if (glu == 1) NORM_LAUNCH(1, 4, 2); else NORM_LAUNCH(2, 4, 2);
+#undef NORM_LAUNCH
 }
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -854,6 +916,28 @@ void matvec_glu(MetalBuf *W, MetalBuf *x, MetalBuf *y, int rows, int cols, int q
     mark_written(y);
 }
 
+// The same products (glu 0: y[i] = W_i . ln for `rows` rows) over ln = RMSNorm(xr + br; g), the sum and the norm formed
+// inside the launch: what k_add_norm followed by a matrix-vector product computes, src/nn/fast_inference.c:386-398,
+// 437-452.  nin.x_out receives xr + br and must not be xr.
+void matvec_norm(MetalBuf *W, const NormIn &nin, MetalBuf *y, int rows, int cols, int q8, int glu)
+{
+    if (rows <= 0 || cols <= 0 || (cols & 31) || cols > 12288 || !aligned16(dptr(W)) || !nin.xr || !nin.g || nin.x_out == nin.xr ||
+        !aligned16(nin.xr) || !aligned16(nin.g) || (nin.br && !aligned16(nin.br)) || (nin.x_out && !aligned16(nin.x_out))) {
+        fprintf(stderr, "[fast_hip] matvec_norm: unsupported shape %d x %d or operands\n", rows, cols); abort();
+    }
+    const int wrows = glu ? 2 * rows : rows;
+    REQUIRE_BYTES(y, (size_t)rows * 4, "matvec_norm");
+    if (q8) {
+        REQUIRE_BYTES(W, (size_t)wrows * (cols / 32) * 34, "matvec_norm");
+        const half_t *scales = nullptr;
+        const int8_t *q = q8_split_of(W, wrows, cols / 32, &scales);
+        launch_matvec_norm<1>(q, scales, nin, dptr_as<float>(y), rows, cols, glu);
+    } else {
+        REQUIRE_BYTES(W, (size_t)wrows * cols * 2, "matvec_norm");
+        launch_matvec_norm<0>(dptr(W), nullptr, nin, dptr_as<float>(y), rows, cols, glu);
+    }
+    mark_written(y);
+}
 
 void attention_decode_fused(const HeadPost &hp, MetalBuf *Kc, MetalBuf *Vc, float *out, int hd, int max_seq, int copies)
 {

@@ -33,7 +33,7 @@ struct InferenceState {
     std::vector<float> thetas;
     MetalBuf *rope_tabs;                 // (cos, sin) [distinct thetas][max_seq][hd/2], as rope forms them
     std::vector<int> theta_slot;         // table of each layer
-    MetalBuf *x, *branch, *ln, *qkv, *att, *gu, *gate_v, *up_v, *logits, *best;   // gate_v / up_v: the halves of gu
+    MetalBuf *x, *x2, *branch, *ln, *qkv, *att, *gu, *gate_v, *up_v, *logits, *best;   // gate_v / up_v: the halves of gu
     float *logits_host;
     int *best_host;
     std::vector<MetalBuf *> kc, vc;
@@ -241,9 +241,9 @@ void matvec(InferenceState *s, const WMat *w, MetalBuf *x, MetalBuf *y)
     else metal_enqueue_q8_matvec(w->mbuf, x, y, w->rows, w->nb);
 }
 
-void add_norm(InferenceState *s, MetalBuf *branch, MetalBuf *g_branch, MetalBuf *g)
+void add_norm(InferenceState *s, MetalBuf *x, MetalBuf *branch, MetalBuf *g_branch, MetalBuf *g)
 {
-    hipLaunchKernelGGL(k_add_norm, dim3(1), dim3(1024), 0, stream(), dptr_as<float>(s->x), branch ? dptr_as<float>(branch) : nullptr,
+    hipLaunchKernelGGL(k_add_norm, dim3(1), dim3(1024), 0, stream(), dptr_as<float>(x), branch ? dptr_as<float>(branch) : nullptr,
                        g_branch ? dptr_as<float>(g_branch) : nullptr, dptr_as<float>(g), dptr_as<float>(s->ln), s->D, s->eps);
 }
 
@@ -255,10 +255,25 @@ void forward_token(InferenceState *s, int token, int pos)
     hipLaunchKernelGGL(k_embed_row, dim3((D + TB - 1) / TB), dim3(TB), 0, stream(), dptr_as<float>(s->emb), token, s->emb_scale,
                        dptr_as<float>(s->x), D);
     MetalBuf *pending = nullptr, *pending_g = nullptr;           // FFN branch of the previous layer, added by the next norm kernel
+    // Where the branch enters the sum as it is (Qwen3), the product after a norm forms sum and norm itself
+    // (matvec_norm) and the sum goes to the other of two residual buffers; the Q|K|V product only without adapters,
+    // whose down-projection reads the normed vector too.
+    MetalBuf *x = s->x, *x_other = s->x2;
+    const bool fuse_ffn = !gemma && D <= 12288, fuse_qkv = fuse_ffn && s->lora.empty();
+    const int q8 = s->use_fp16 ? 0 : 1;
+    auto normed_product = [&](MetalBuf *W, MetalBuf *branch, MetalBuf *g, MetalBuf *y, int rows, int glu) {
+        NormIn n{dptr_as<float>(x), branch ? dptr_as<float>(branch) : nullptr, dptr_as<float>(g), branch ? dptr_as<float>(x_other) : nullptr,
+                 s->eps};
+        matvec_norm(W, n, y, rows, D, q8, glu);
+        if (branch) std::swap(x, x_other);
+    };
     for (int L = 0; L < s->NL; L++) {
         const InferenceState::Layer &lw = s->layers[L];
-        add_norm(s, pending, pending_g, lw.g_in);
-        matvec(s, &lw.qkv, s->ln, s->qkv);
+        if (fuse_qkv) normed_product(lw.qkv.mbuf, pending, lw.g_in, s->qkv, lw.qkv.rows, 0);
+        else {
+            add_norm(s, x, pending, pending_g, lw.g_in);
+            matvec(s, &lw.qkv, s->ln, s->qkv);
+        }
         // LoRA on q and v, per-head RMSNorm and RoPE on q and k, k and v into the caches, and the attention over the
         // cache: one launch (infer_kernels.hip: k_attn_decode<.., FUSED>)
         HeadPost a{};
@@ -277,15 +292,18 @@ void forward_token(InferenceState *s, int token, int pos)
         attention_decode_fused(a, s->kc[L], s->vc[L], dptr_as<float>(s->att), hd, s->max_seq);
         mark_written(s->att);
         matvec(s, lw.o, s->att, s->branch);
-        // x += o (Gemma3: RMSNorm(o; g_post_attn)); ln = RMSNorm(x; g_pre_ff | g_post_attn)
-        add_norm(s, s->branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
+        // x += o (Gemma3: RMSNorm(o; g_post_attn)); ln = RMSNorm(x; g_pre_ff | g_post_attn);
         // act = silu | gelu (gate) * up, formed in the epilogue of the [gate; up] product
-        matvec_glu(lw.gu.mbuf, s->ln, s->gate_v, s->IS, D, s->use_fp16 ? 0 : 1, gemma ? 1 : 0);
+        if (fuse_ffn) normed_product(lw.gu.mbuf, s->branch, lw.g_post_attn, s->gate_v, s->IS, 1);
+        else {
+            add_norm(s, x, s->branch, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
+            matvec_glu(lw.gu.mbuf, s->ln, s->gate_v, s->IS, D, q8, gemma ? 1 : 0);
+        }
         matvec(s, lw.down, s->gate_v, s->branch);
         pending = s->branch;
         pending_g = gemma ? lw.g_post_ff : nullptr;
     }
-    add_norm(s, pending, pending_g, s->g_final);
+    add_norm(s, x, pending, pending_g, s->g_final);
     HIP_CHECK(hipGetLastError());
     matvec(s, s->lm_head, s->ln, s->logits);
 }
@@ -344,7 +362,7 @@ InferenceState *new_state(ModelType mt, int D, int Hq, int Hkv, int hd, int IS, 
     }
     default_eos(s);
     const int qd = Hq * hd, kd = Hkv * hd;
-    s->x = fbuf(D); s->branch = fbuf(D); s->ln = fbuf(D);
+    s->x = fbuf(D); s->x2 = fbuf(D); s->branch = fbuf(D); s->ln = fbuf(D);
     s->qkv = fbuf(qd + 2 * kd); s->att = fbuf(qd);
     s->gu = fbuf(2 * (size_t)IS);
     s->gate_v = metal_buf_view(s->gu, 0, (size_t)IS * 4); s->up_v = metal_buf_view(s->gu, (size_t)IS * 4, (size_t)IS * 4);
@@ -575,7 +593,7 @@ void inference_state_free(InferenceState *s)
 {
     if (!s) return;
     metal_flush();
-    for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t, s->rope_tabs})
+    for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->x2, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t, s->rope_tabs})
         metal_buf_free(b);
     for (MetalBuf *b : s->kc) metal_buf_free(b);
     for (MetalBuf *b : s->vc) metal_buf_free(b);
