@@ -163,6 +163,10 @@ void hip_gemm_force_large_m(int policy);
  * rule (three chunks when the 128 x 256 output blocks leave a third of the CUs idle and K >= 4096), 0 = never, n > 1 =
  * always n. */
 void hip_gemm_large_m_split(int mode);
+/* Output block of the large-M kernel on F16 tiles: 0 = by the measured rule (256 x 256 where that leaves at least 0.8
+ * as much of the GPU on useful work as 128 x 256 does, counting partial rounds of blocks and partial tiles), 1 = always
+ * 128 x 256, 2 = always 256 x 256. */
+void hip_gemm_large_m_block(int mode);
 /* A training state with frozen Q8_0 weights whose products run on the large-M kernel keeps the F16 image of every
  * weight it has used (made once instead of once per product) while they fit this many MB per state (default 65536;
  * the 4B model needs 16 GB); weights beyond that, or all with 0, get an image per product. */

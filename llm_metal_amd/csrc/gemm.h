@@ -80,6 +80,7 @@ bool large_m_unpacks_q8();                                // the large-M policy 
 // big_gemm_chunks: what the measured rule picks for a product
 int big_gemm_chunks(int M, int N, int K, int fmt);
 void set_big_gemm_split(int mode);     // 1 measured rule, 0 never, n > 1 always n chunks
+void set_big_gemm_block(int mode);     // F16 tiles: 0 block shape by the measured rule, 1 always 128 x 256, 2 always 256 x 256
 // Returns the number of planes written (fewer than `chunks` when K has too few steps for that many).
 int launch_gemm_big(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K,
                     int chunks = 1, size_t plane_stride = 0);

@@ -574,6 +574,7 @@ void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, i
 
 void hip_gemm_force_large_m(int policy) { g_big_policy = policy; }
 void hip_gemm_large_m_split(int mode) { set_big_gemm_split(mode); }
+void hip_gemm_large_m_block(int mode) { set_big_gemm_block(mode); }
 
 void hip_gemm_profile_enable(int on)
 {

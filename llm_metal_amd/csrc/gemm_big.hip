@@ -23,6 +23,7 @@ namespace lmhip {
 namespace {
 
 int g_big_split = 1;                  // 1: K chunks by the measured rule (big_gemm_chunks), 0: never, n > 1: always n
+int g_big_block = 0;                  // F16 tiles: 0 block shape by the measured rule, 1 always 128 x 256, 2 always 256 x 256
 constexpr int WPW = 2;               // weight row blocks each wave fetches per K step: the block is 128 x (WPW * 128)
 constexpr int PF = 3;                // K steps whose operands are in flight in registers ahead of the one being multiplied
 
@@ -392,6 +393,143 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
         }
 }
 
+// The same product on a 256 x 256 block: four waves of 128 x 128 (sixteen accumulator tiles each, in the accumulation
+// registers), so that a wave reads 0.5 KB of LDS per MFMA instead of 0.75 and a block fetches half as many operand bytes
+// per flop.  K goes in half steps of 32 (two of a tile's four 1 KB slices per row block) through four 32 KB LDS buffers:
+// half step h is multiplied out of buffer h % 4 while h + 1 .. h + 3 are in flight; one barrier per half step with the
+// wait before it written by hand (vmcnt <= 16: the two half steps after the next may still be out).  The copies are
+// LDS-direct loads issued as assembly, right after the barrier: the compiler does not count them among its own loads
+// (it cannot tell which LDS bytes a pending copy writes and would wait for all of them before every LDS read).
+// In its loop this block runs at 1.5 PFLOP/s (60 % of the MFMA peak) against 1.1 for 128 x 256, but there are half as
+// many blocks: launch_gemm_big picks the one that loses less to partial rounds and partial tiles.
+__global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
+{
+    constexpr int HB = 16 * 2 * 64;                       // half8 per buffer: [16 row blocks][2 slices][64 lanes]
+    __shared__ half8 lb0[HB], lb1[HB], lb2[HB], lb3[HB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int MT = (g.M + 255) >> 8, NT = (g.N + 255) >> 8;
+    const int m_patches = (MT + 7) >> 3;
+    int mt, nt, chunk = 0;
+    if (g.S > 1) {
+        const int t = blockIdx.x % (MT * NT);
+        chunk = blockIdx.x / (MT * NT); mt = t % MT; nt = t / MT;
+    } else {
+        const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3, patch = seq >> 5, in_patch = seq & 31;
+        mt = (patch % m_patches) * 8 + (in_patch & 7);
+        nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
+        if (mt >= MT || nt >= NT) return;
+    }
+    const int nb0 = nt * 8, mb0 = mt * 8;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int k_beg = chunk * g.steps_per_chunk, nsteps = min(g.Kb, k_beg + g.steps_per_chunk) - k_beg;
+    const int nhalf = 2 * nsteps, last = nhalf - 1;
+    // this wave's share of a half step: both slices of A row blocks w, 4 + w and of W row blocks w, 4 + w
+    const half8 *src[4];
+    src[0] = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[1] = g.A + ((size_t)min(mb0 + 4 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[2] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + wave, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[3] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + 4 + wave, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
+    const int dst[4] = {wave, 4 + wave, 8 + wave, 12 + wave};
+    float *const Cp = g.P + (size_t)chunk * g.plane_stride;
+
+    float16v acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    typedef __attribute__((address_space(3))) void lds_void;
+    uint32_t loff[4][2];                                   // byte offsets inside a buffer of this wave's eight 1 KB pieces
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) loff[u][j] = __builtin_amdgcn_readfirstlane((uint32_t)((dst[u] * 2 + j) * 64 * 16));
+    auto request = [&](half8 (&buf)[HB], int hs) __attribute__((always_inline)) {
+        const size_t o = (size_t)(hs >> 1) * 256 + (hs & 1) * 128;
+        const uint32_t base = (uint32_t)(uintptr_t)(lds_void *)buf;
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[u] + o + j * 64), "s"(base + loff[u][j]) : "m0");
+    };
+    auto step = [&](int hs, half8 (&cur)[HB], half8 (&free_buf)[HB]) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        request(free_buf, min(hs + 3, last));
+        half8 a[2][4], w[2][4];
+        auto read = [&](int j) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[j & 1][i] = cur[((4 * wm + i) * 2 + j) * 64 + lane];
+#pragma unroll
+            for (int k = 0; k < 4; k++) w[j & 1][k] = cur[((8 + 4 * wn + k) * 2 + j) * 64 + lane];
+        };
+        read(0);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if (j + 1 < 2) read(j + 1);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 1][i], w[j & 1][k], acc[i][k], 0, 0, 0);
+        }
+        // issue order: the 8 LDS reads of slice 0, then under each MFMA one LDS read of slice 1
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+    request(lb0, 0);
+    request(lb1, min(1, last));
+    request(lb2, min(2, last));
+    const int full = nhalf / 4 * 4;                         // nhalf is even: the rest is 0 or 2 half steps
+    for (int h0 = 0; h0 < full; h0 += 4) {
+        step(h0, lb0, lb3);
+        step(h0 + 1, lb1, lb0);
+        step(h0 + 2, lb2, lb1);
+        step(h0 + 3, lb3, lb2);
+    }
+    if (full < nhalf) { step(full, lb0, lb3); step(full + 1, lb1, lb0); }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    if (mb0 * 32 + 256 <= g.M && (nb0 + 8) * 32 <= g.N) {  // a block inside the matrix: stores without tests, factors first
+        float sc[4][16];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                sc[i][v] = g.a_inv_scale ? g.a_inv_scale[(mb0 + 4 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3)] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = (mb0 + 4 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                float *row = Cp + (size_t)m * g.ldp + (nb0 + 4 * wn) * 32 + r;
+#pragma unroll
+                for (int k = 0; k < 4; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = (mb0 + 4 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (m >= g.M) continue;
+            const float sc = g.a_inv_scale ? g.a_inv_scale[m] : 1.0f;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int n = (nb0 + 4 * wn + k) * 32 + r;
+                if (n < g.N) Cp[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
+            }
+        }
+}
+
 }  // namespace
 
 // How many K chunks the large-M kernel should cut a product with F16 tiles into: three when its 128 x 256 output blocks
@@ -432,6 +570,23 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
     const int MT = (M + 127) / 128, NT = (N + 128 * WPW - 1) / (128 * WPW);
     const int m_patches = (MT + 7) / 8, n_patches = ((NT + 7) / 8 + 3) / 4;
     const dim3 grid(W.fmt == 0 && g.S > 1 ? MT * NT * g.S : 8 * 32 * m_patches * n_patches), block(256);
+    // F16 tiles: 128 x 256 or 256 x 256 blocks, whichever keeps more of the GPU on useful work -- the share of the last
+    // round's CUs that have a block times the share of the tiles' area that lies inside the matrix; the wide block is
+    // faster in its loop and wins from 0.8 of the other's share (measured at 2048 rows: 200 / 240 / 608 wide blocks win
+    // against 400 / 480 / 1216, 304 and 128 lose against 608 and 256)
+    bool wide = false;
+    dim3 grid256(1);
+    if (W.fmt == 0) {
+        const int cus = num_cus() > 0 ? num_cus() : 256;
+        auto share = [&](int bm, int bn) {
+            const long tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn, blocks = tm * tn * g.S;
+            return (double)M * N / ((double)tm * bm * tn * bn) * (double)blocks / (double)((blocks + cus - 1) / cus * cus);
+        };
+        // (its gain is in the loop: below 32 K steps per block the larger prologue and epilogue take it back)
+        wide = g_big_block == 2 || (g_big_block == 0 && g.steps_per_chunk >= 20 && share(256, 256) >= 0.9 * share(128, 128 * WPW));
+        const int MX = (M + 255) / 256, NX = (N + 255) / 256;
+        grid256 = dim3(g.S > 1 ? MX * NX * g.S : 8 * 32 * ((MX + 7) / 8) * (((NX + 7) / 8 + 3) / 4));
+    }
     const size_t lds = (size_t)2 * (4 + 4 * WPW) * 256 * sizeof(half8);
     static bool attr_set = false;
     if (!attr_set) {
@@ -441,11 +596,13 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
     }
     hipEvent_t ev_a = nullptr, ev_b = nullptr;
     if (gemm_prof_begin(weight_stream_bytes(W, N, K), 2.0 * M * N * K, &ev_a, &ev_b)) {
-        if (W.fmt == 0) hipExtLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), ev_a, ev_b, 0, g);
+        if (W.fmt == 0 && wide) hipExtLaunchKernelGGL(gemm_big_f16_256, grid256, block, 0, stream(), ev_a, ev_b, 0, g);
+        else if (W.fmt == 0) hipExtLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), ev_a, ev_b, 0, g);
         else if (W.fmt == 1) hipExtLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
         else hipExtLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
     } else {
-        if (W.fmt == 0) hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), g);
+        if (W.fmt == 0 && wide) hipLaunchKernelGGL(gemm_big_f16_256, grid256, block, 0, stream(), g);
+        else if (W.fmt == 0) hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), g);
         else if (W.fmt == 1) hipLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), g);
         else hipLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), g);
     }
@@ -454,5 +611,6 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
 }
 
 void set_big_gemm_split(int mode) { g_big_split = mode; }
+void set_big_gemm_block(int mode) { g_big_block = mode; }
 
 }  // namespace lmhip

@@ -47,6 +47,10 @@ CASES = [
     # ... with the K steps of every product cut into three chunks over the grid (planes added by the consumer), which
     # the measured rule only does at sizes the oracle cannot follow; K of 4, 12 and 64 steps, 200 ragged rows
     C1.with_(name="big_m_f16_chunks", batch=5, seq=40),
+    C1.with_(name="big_m_f16_wide", batch=4, seq=64),                    # the 256 x 256 block of the large-M kernel
+    C1.with_(name="big_m_f16_wide_chunks", batch=5, seq=40),             # ragged in rows (200) and three K chunks
+    C1.with_(name="big_m_q8_wide", NL=1, batch=2, seq=160, weight_format="q8_0"),   # over the kept F16 images, 320 rows
+    TINY_GEMMA3.with_(name="gemma_big_m_q8_wide", NL=2, batch=3, seq=100, weight_format="q8_0"),
     C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
     C1.with_(name="big_m_q8_noimg", NL=1, batch=2, seq=160, weight_format="q8_0"),      # no room to keep the images: made per product
@@ -107,6 +111,7 @@ def test_train_steps_match_oracle(cfg):
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
     lib.load().hip_gemm_force_large_m(2 if cfg.name.endswith("_lds") else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
+    lib.load().hip_gemm_large_m_block(2 if "_wide" in cfg.name else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_attention_flash(1 if cfg.name.endswith("_flash") else 0 if cfg.name.endswith("_noflash") else -1)
     lib.load().hip_gemm_image_budget_mb(0 if cfg.name.endswith("_noimg") else 65536)
     with SFTState(cfg, model) as st:
@@ -132,6 +137,7 @@ def test_train_steps_match_oracle(cfg):
         assert (np.sign(d_gpu) == np.sign(d_ref)).mean() > 0.97
     lib.load().hip_gemm_force_large_m(0)
     lib.load().hip_gemm_large_m_split(1)
+    lib.load().hip_gemm_large_m_block(0)
     lib.load().hip_attention_flash(-1)
     lib.load().hip_gemm_image_budget_mb(65536)
 
