@@ -395,17 +395,18 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
 
 // The same product on a 256 x 256 block: four waves of 128 x 128 (sixteen accumulator tiles each, in the accumulation
 // registers), so that a wave reads 0.5 KB of LDS per MFMA instead of 0.75 and a block fetches half as many operand bytes
-// per flop.  K goes in half steps of 32 (two of a tile's four 1 KB slices per row block) through four 32 KB LDS buffers:
-// half step h is multiplied out of buffer h % 4 while h + 1 .. h + 3 are in flight; one barrier per half step with the
-// wait before it written by hand (vmcnt <= 16: the two half steps after the next may still be out).  The copies are
-// LDS-direct loads issued as assembly, right after the barrier: the compiler does not count them among its own loads
-// (it cannot tell which LDS bytes a pending copy writes and would wait for all of them before every LDS read).
-// In its loop this block runs at 1.5 PFLOP/s (60 % of the MFMA peak) against 1.1 for 128 x 256, but there are half as
-// many blocks: launch_gemm_big picks the one that loses less to partial rounds and partial tiles.
+// per flop.  K goes in half steps of 32 (two of a tile's four 1 KB slices per row block) through five 32 KB LDS buffers
+// (all 160 KB of a CU): half step h is multiplied out of buffer h % 5 while h + 1 .. h + 4 are in LDS or on their way.
+// The copies are LDS-direct loads issued as assembly, right after the barrier: the compiler does not count them among
+// its own loads (it cannot tell which LDS bytes a pending copy writes and would wait for all of them before every LDS
+// read); the wait before the barrier is written by hand.
+// In its loop this block runs at 1.5-1.7 PFLOP/s (60-67 % of the MFMA peak; 8192 x 8192 x 8192: 1 667 TFLOP/s) against 1.1
+// for 128 x 256, but there are half as many blocks: launch_gemm_big picks the one that loses less to partial rounds and
+// partial tiles.
 __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
 {
     constexpr int HB = 16 * 2 * 64;                       // half8 per buffer: [16 row blocks][2 slices][64 lanes]
-    __shared__ half8 lb0[HB], lb1[HB], lb2[HB], lb3[HB];
+    __shared__ half8 lb0[HB], lb1[HB], lb2[HB], lb3[HB], lb4[HB];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int MT = (g.M + 255) >> 8, NT = (g.N + 255) >> 8;
@@ -456,45 +457,53 @@ __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
             for (int j = 0; j < 2; j++)
                 asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[u] + o + j * 64), "s"(base + loff[u][j]) : "m0");
     };
-    auto step = [&](int hs, half8 (&cur)[HB], half8 (&free_buf)[HB]) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        request(free_buf, min(hs + 3, last));
-        half8 a[2][4], w[2][4];
-        auto read = [&](int j) {
+    half8 a0[4], w0[4];                                    // fragments of slice 0 of the half step about to be multiplied
+    auto read = [&](half8 (&a)[4], half8 (&w)[4], const half8 (&cur)[HB], int j) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) a[j & 1][i] = cur[((4 * wm + i) * 2 + j) * 64 + lane];
+        for (int i = 0; i < 4; i++) a[i] = cur[((4 * wm + i) * 2 + j) * 64 + lane];
 #pragma unroll
-            for (int k = 0; k < 4; k++) w[j & 1][k] = cur[((8 + 4 * wn + k) * 2 + j) * 64 + lane];
-        };
-        read(0);
+        for (int k = 0; k < 4; k++) w[k] = cur[((8 + 4 * wn + k) * 2 + j) * 64 + lane];
+    };
+    auto multiply = [&](const half8 (&a)[4], const half8 (&w)[4]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            if (j + 1 < 2) read(j + 1);
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int k = 0; k < 4; k++)
-                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 1][i], w[j & 1][k], acc[i][k], 0, 0, 0);
-        }
-        // issue order: the 8 LDS reads of slice 0, then under each MFMA one LDS read of slice 1
-        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+            for (int k = 0; k < 4; k++) acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
+    };
+    // Half step hs is multiplied out of buffer hs % 5.  The barrier that ends half step hs - 1 has found hs and hs + 1 in
+    // LDS (every wave waited for its own copies of them), so slice 0 of hs + 1 is read while slice 1 of hs is multiplied
+    // and no half step starts by waiting out an LDS round trip; hs + 4 is requested into the buffer hs - 1 left.
+    auto step = [&](int hs, const half8 (&cur)[HB], const half8 (&nxt)[HB], half8 (&free_buf)[HB]) __attribute__((always_inline)) {
+        request(free_buf, min(hs + 4, last));
+        half8 a1[4], w1[4];
+        read(a1, w1, cur, 1);
+        multiply(a0, w0);
+        read(a0, w0, nxt, 0);
+        multiply(a1, w1);
+        // issue order: under each MFMA of slice 0 one LDS read of slice 1, under each of slice 1 one of the next slice 0
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
         for (int i = 0; i < 32; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i < 6 || (i >= 16 && i < 24)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
-    request(lb0, 0);
-    request(lb1, min(1, last));
-    request(lb2, min(2, last));
-    const int full = nhalf / 4 * 4;                         // nhalf is even: the rest is 0 or 2 half steps
-    for (int h0 = 0; h0 < full; h0 += 4) {
-        step(h0, lb0, lb3);
-        step(h0 + 1, lb1, lb0);
-        step(h0 + 2, lb2, lb1);
-        step(h0 + 3, lb3, lb2);
+    request(lb0, 0); request(lb1, min(1, last)); request(lb2, min(2, last)); request(lb3, min(3, last));
+    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+    read(a0, w0, lb0, 0);
+    const int full = nhalf / 5 * 5;
+    for (int h0 = 0; h0 < full; h0 += 5) {
+        step(h0, lb0, lb1, lb4);
+        step(h0 + 1, lb1, lb2, lb0);
+        step(h0 + 2, lb2, lb3, lb1);
+        step(h0 + 3, lb3, lb4, lb2);
+        step(h0 + 4, lb4, lb0, lb3);
     }
-    if (full < nhalf) { step(full, lb0, lb3); step(full + 1, lb1, lb0); }
+    if (full < nhalf) step(full, lb0, lb1, lb4);
+    if (full + 1 < nhalf) step(full + 1, lb1, lb2, lb0);
+    if (full + 2 < nhalf) step(full + 2, lb2, lb3, lb1);
+    if (full + 3 < nhalf) step(full + 3, lb3, lb4, lb2);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     if (mb0 * 32 + 256 <= g.M && (nb0 + 8) * 32 <= g.N) {  // a block inside the matrix: stores without tests, factors first
