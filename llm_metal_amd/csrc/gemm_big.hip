@@ -576,26 +576,52 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
     g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb;
     g.steps_per_chunk = (Kb + chunks - 1) / chunks;
     g.S = (Kb + g.steps_per_chunk - 1) / g.steps_per_chunk;
-    const int MT = (M + 127) / 128, NT = (N + 128 * WPW - 1) / (128 * WPW);
-    const int m_patches = (MT + 7) / 8, n_patches = ((NT + 7) / 8 + 3) / 4;
-    const dim3 grid(W.fmt == 0 && g.S > 1 ? MT * NT * g.S : 8 * 32 * m_patches * n_patches), block(256);
-    // F16 tiles: 128 x 256 or 256 x 256 blocks, whichever keeps more of the GPU on useful work -- the share of the last
-    // round's CUs that have a block times the share of the tiles' area that lies inside the matrix; the wide block is
-    // faster in its loop and wins from 0.8 of the other's share (measured at 2048 rows: 200 / 240 / 608 wide blocks win
-    // against 400 / 480 / 1216, 304 and 128 lose against 608 and 256)
-    bool wide = false;
-    dim3 grid256(1);
+    const dim3 block(256);
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+    const bool prof = gemm_prof_begin(weight_stream_bytes(W, N, K), 2.0 * M * N * K, &ev_a, &ev_b);
+    // grid of either block shape: with K chunks one workgroup per (chunk, block); else whole patches of 8 x 32 ids (see
+    // the kernels), the ids past the matrix returning at once
+    auto grid_of = [&](const GemmKArgs &a, int bm, int bn) {
+        const int mt = (a.M + bm - 1) / bm, nt = (a.N + bn - 1) / bn;
+        return dim3(W.fmt == 0 && a.S > 1 ? mt * nt * a.S : 8 * 32 * ((mt + 7) / 8) * (((nt + 7) / 8 + 3) / 4));
+    };
     if (W.fmt == 0) {
+        // 128 x 256 or 256 x 256 blocks, whichever keeps more of the GPU on useful work -- the share of the last round's
+        // CUs that have a block times the share of the tiles' area that lies inside the matrix.  The wide block is faster
+        // in its loop and wins from 0.9 of the other's share, given 20 K steps per block to win them in (below, its larger
+        // prologue and epilogue take the gain back).  Measured at 2048 rows inside the step: 200 and 240 wide blocks win
+        // against 400 and 480, 4752 against 9504; 608, 304 and 128 lose against 1216, 608 and 256.
         const int cus = num_cus() > 0 ? num_cus() : 256;
         auto share = [&](int bm, int bn) {
             const long tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn, blocks = tm * tn * g.S;
             return (double)M * N / ((double)tm * bm * tn * bn) * (double)blocks / (double)((blocks + cus - 1) / cus * cus);
         };
-        // (its gain is in the loop: below 32 K steps per block the larger prologue and epilogue take it back)
-        wide = g_big_block == 2 || (g_big_block == 0 && g.steps_per_chunk >= 20 && share(256, 256) >= 0.9 * share(128, 128 * WPW));
-        const int MX = (M + 255) / 256, NX = (N + 255) / 256;
-        grid256 = dim3(g.S > 1 ? MX * NX * g.S : 8 * 32 * ((MX + 7) / 8) * (((NX + 7) / 8 + 3) / 4));
+        const bool deep = g.steps_per_chunk >= 20;
+        const bool wide = g_big_block == 2 || (g_big_block == 0 && deep && share(256, 256) >= 0.9 * share(128, 128 * WPW));
+        // A product of at least two full rounds of wide blocks whose last round would be half empty or less: the columns
+        // of the full rounds go to wide blocks, the rest to 128 x 256 blocks in a launch of their own
+        const int MX = (M + 255) / 256, NX = (N + 255) / 256, full = MX * NX / cus, rest = MX * NX % cus;
+        const int wide_cols = full * cus / MX * 256;
+        auto launch = [&](const GemmKArgs &a, bool w, hipEvent_t e0, hipEvent_t e1) {
+            const dim3 grid = w ? grid_of(a, 256, 256) : grid_of(a, 128, 128 * WPW);
+            if (prof && w) hipExtLaunchKernelGGL(gemm_big_f16_256, grid, block, 0, stream(), e0, e1, 0, a);
+            else if (prof) hipExtLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), e0, e1, 0, a);
+            else if (w) hipLaunchKernelGGL(gemm_big_f16_256, grid, block, 0, stream(), a);
+            else hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), a);
+        };
+        if (g_big_block == 0 && !wide && deep && g.S == 1 && full >= 2 && rest > 0 && rest * 2 <= cus && wide_cols < N) {
+            GemmKArgs g1 = g, g2 = g;
+            g1.N = wide_cols; g1.Nb = wide_cols / 32;
+            g2.N = N - wide_cols; g2.Nb = tiled_rb(g2.N);
+            g2.W.w16 = W.w16 + (size_t)(wide_cols / 32) * Kb * 2048;
+            g2.P = C + wide_cols;
+            launch(g1, true, ev_a, nullptr);
+            launch(g2, false, nullptr, ev_b);
+        } else launch(g, wide, ev_a, ev_b);
+        HIP_CHECK(hipGetLastError());
+        return g.S;
     }
+    const dim3 grid = grid_of(g, 128, 128 * WPW);
     const size_t lds = (size_t)2 * (4 + 4 * WPW) * 256 * sizeof(half8);
     static bool attr_set = false;
     if (!attr_set) {
@@ -603,20 +629,15 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_big<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_set = true;
     }
-    hipEvent_t ev_a = nullptr, ev_b = nullptr;
-    if (gemm_prof_begin(weight_stream_bytes(W, N, K), 2.0 * M * N * K, &ev_a, &ev_b)) {
-        if (W.fmt == 0 && wide) hipExtLaunchKernelGGL(gemm_big_f16_256, grid256, block, 0, stream(), ev_a, ev_b, 0, g);
-        else if (W.fmt == 0) hipExtLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), ev_a, ev_b, 0, g);
-        else if (W.fmt == 1) hipExtLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
+    if (prof) {
+        if (W.fmt == 1) hipExtLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
         else hipExtLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), ev_a, ev_b, 0, g);
     } else {
-        if (W.fmt == 0 && wide) hipLaunchKernelGGL(gemm_big_f16_256, grid256, block, 0, stream(), g);
-        else if (W.fmt == 0) hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), g);
-        else if (W.fmt == 1) hipLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), g);
+        if (W.fmt == 1) hipLaunchKernelGGL(gemm_big<1>, grid, block, lds, stream(), g);
         else hipLaunchKernelGGL(gemm_big<2>, grid, block, lds, stream(), g);
     }
     HIP_CHECK(hipGetLastError());
-    return W.fmt == 0 ? g.S : 1;
+    return 1;
 }
 
 void set_big_gemm_split(int mode) { g_big_split = mode; }
