@@ -249,26 +249,23 @@ __global__ __launch_bounds__(256) void gemm_big(GemmKArgs g)
 
 // F16 weight tiles need no unpacking, so their steps go from L2/HBM straight into LDS (global_load_lds_dwordx4: a
 // wave-uniform LDS base in M0, lane i's 16 bytes land at base + 16 i -- the [j][lane] order of the tiles) and never
-// pass through registers or ds_write.  Three LDS buffers (distinct objects, so that the compiler knows that a read of
-// one does not have to wait for a load into another): step kt is multiplied out of buffer kt % 3 while the loads of
-// steps kt + 1 and kt + 2 are in flight.  One barrier per step; the wait before it is written by hand (vmcnt <= 12: the
-// twelve loads of the step after may still be out), because a fence would wait for all of them.
-constexpr int DMA_LOADS = 4 + 4 * WPW;                    // per wave and step
-static_assert(DMA_LOADS == 12, "the hand-written wait below counts twelve loads per step");
-
+// pass through registers or ds_write.  K goes in half steps of 32 (two of a tile's four 1 KB slices per row block)
+// through six 24 KB LDS buffers, distinct objects: half step h is multiplied out of buffer h % 6 while h + 1 .. h + 5
+// are in LDS or on their way.  The copies are issued as assembly right after the barrier, so the compiler does not count
+// them among its own loads (it cannot tell which LDS bytes a pending copy writes and would wait for all of them before
+// every LDS read); the wait before the barrier is written by hand: the barrier that ends half step h - 1 finds h and
+// h + 1 in LDS -- every wave has waited for its own copies of them -- so slice 0 of h + 1 is read under the MFMAs of
+// slice 1 of h and no half step starts by waiting out an LDS round trip; h + 5 is requested into the buffer h - 1 left.
 __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
 {
-    constexpr int NBLK = 4 + 4 * WPW, BUF = NBLK * 256, NW = 2 * WPW;
-    __shared__ half8 lb0[BUF], lb1[BUF], lb2[BUF];
+    constexpr int HB = 12 * 2 * 64;                       // half8 per buffer: [4 A + 8 W row blocks][2 slices][64 lanes]
+    __shared__ half8 lb0[HB], lb1[HB], lb2[HB], lb3[HB], lb4[HB], lb5[HB];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int MT = (g.M + 127) >> 7, NT = (g.N + 128 * WPW - 1) / (128 * WPW);
+    const int MT = (g.M + 127) >> 7, NT = (g.N + 255) >> 8;
     const int m_patches = (MT + 7) >> 3;
     int mt, nt, chunk = 0;
     if (g.S > 1) {
-        // K chunks: the grid is S * MT * NT workgroups, id = (chunk * NT + nt) * MT + mt.  The hardware deals ids to the
-        // XCDs in turn, so (MT a multiple of 8) an XCD takes the row blocks mt = xcd (mod 8) of every column block and
-        // chunk: equal shares, and an activation row block is fetched into one L2 only.
         const int t = blockIdx.x % (MT * NT);
         chunk = blockIdx.x / (MT * NT); mt = t % MT; nt = t / MT;
     } else {
@@ -277,104 +274,102 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
         nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
         if (mt >= MT || nt >= NT) return;
     }
-    const int nb0 = nt * 4 * WPW, mb0 = mt * 4;
+    const int nb0 = nt * 8, mb0 = mt * 4;
     const int wm = wave >> 1, wn = wave & 1;
     const int k_beg = chunk * g.steps_per_chunk, nsteps = min(g.Kb, k_beg + g.steps_per_chunk) - k_beg;
-    const half8 *asrc = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
-    const half8 *wsrc[WPW];
-#pragma unroll
-    for (int u = 0; u < WPW; u++)
-        wsrc[u] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + wave * WPW + u, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
+    const int nhalf = 2 * nsteps, last = nhalf - 1;
+    const half8 *src[3];
+    src[0] = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[1] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + 2 * wave, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[2] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + 2 * wave + 1, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
+    const int dst[3] = {wave, 4 + 2 * wave, 5 + 2 * wave};
     float *const Cp = g.P + (size_t)chunk * g.plane_stride;
 
-    float16v acc[2][NW];
+    float16v acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < NW; j++)
+        for (int j = 0; j < 4; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     typedef __attribute__((address_space(3))) void lds_void;
-    auto request = [&](half8 (&buf)[BUF], int kt) __attribute__((always_inline)) {
-        const size_t o = (size_t)kt * 256;
+    uint32_t loff[3][2];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            __builtin_amdgcn_global_load_lds(asrc + o + j * 64, (lds_void *)(buf + (wave * 4 + j) * 64), 16, 0, 0);
+    for (int u = 0; u < 3; u++)
 #pragma unroll
-        for (int u = 0; u < WPW; u++)
+        for (int j = 0; j < 2; j++) loff[u][j] = __builtin_amdgcn_readfirstlane((uint32_t)((dst[u] * 2 + j) * 64 * 16));
+    auto request = [&](half8 (&buf)[HB], int hs) __attribute__((always_inline)) {
+        const size_t o = (size_t)(hs >> 1) * 256 + (hs & 1) * 128;
+        const uint32_t base = (uint32_t)(uintptr_t)(lds_void *)buf;
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                __builtin_amdgcn_global_load_lds(wsrc[u] + o + j * 64, (lds_void *)(buf + ((4 + wave * WPW + u) * 4 + j) * 64), 16, 0, 0);
+        for (int u = 0; u < 3; u++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[u] + o + j * 64), "s"(base + loff[u][j]) : "m0");
     };
-    const int last = nsteps - 1;
-    // one K step: `cur` holds step kt; `free_buf` held step kt - 1 and takes step kt + 2
-    auto step = [&](int kt, half8 (&cur)[BUF], half8 (&free_buf)[BUF]) __attribute__((always_inline)) {
-        // lgkmcnt(0): every LDS read this wave issued for step kt - 1 has returned before the barrier lets other waves
-        // overwrite that buffer (the MFMAs that consume them are not memory operations and may be scheduled past this
-        // statement, so their own waits do not order the reuse)
-        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        request(free_buf, min(kt + 2, last));
-        half8 a[2][2], w[2][NW];
-        auto read = [&](int j) {
+    half8 a0[2], w0[4];
+    auto read = [&](half8 (&a)[2], half8 (&w)[4], const half8 (&cur)[HB], int j) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) a[j & 1][i] = cur[((2 * wm + i) * 4 + j) * 64 + lane];
+        for (int i = 0; i < 2; i++) a[i] = cur[((2 * wm + i) * 2 + j) * 64 + lane];
 #pragma unroll
-            for (int k = 0; k < NW; k++) w[j & 1][k] = cur[((4 + NW * wn + k) * 4 + j) * 64 + lane];
-        };
-        read(0);
+        for (int k = 0; k < 4; k++) w[k] = cur[((4 + 4 * wn + k) * 2 + j) * 64 + lane];
+    };
+    auto multiply = [&](const half8 (&a)[2], const half8 (&w)[4]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            if (j + 1 < 4) read(j + 1);
+        for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int k = 0; k < 4; k++) acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
+    };
+    auto step = [&](int hs, const half8 (&cur)[HB], const half8 (&nxt)[HB], half8 (&free_buf)[HB]) __attribute__((always_inline)) {
+        request(free_buf, min(hs + 5, last));
+        half8 a1[2], w1[4];
+        read(a1, w1, cur, 1);
+        multiply(a0, w0);
+        read(a0, w0, nxt, 0);
+        multiply(a1, w1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
-                for (int k = 0; k < NW; k++)
-                    acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 1][i], w[j & 1][k], acc[i][k], 0, 0, 0);
-        }
-        // issue order: the 6 LDS reads of slice 0, then under each MFMA one LDS read of the next slice and one of the
-        // twelve requests
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-#pragma unroll
-        for (int i = 0; i < 32; i++) {
+        for (int i = 0; i < 16; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 24 && (i & 7) < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (i < 4 || (i >= 8 && i < 14)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
-    request(lb0, 0);
-    request(lb1, min(1, last));
-    const int full = nsteps / 3 * 3;
-    for (int kt0 = 0; kt0 < full; kt0 += 3) {
-        step(kt0, lb0, lb2);
-        step(kt0 + 1, lb1, lb0);
-        step(kt0 + 2, lb2, lb1);
+    request(lb0, 0); request(lb1, min(1, last)); request(lb2, min(2, last)); request(lb3, min(3, last)); request(lb4, min(4, last));
+    asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+    read(a0, w0, lb0, 0);
+    const int full = nhalf / 6 * 6;
+    for (int h0 = 0; h0 < full; h0 += 6) {
+        step(h0, lb0, lb1, lb5);
+        step(h0 + 1, lb1, lb2, lb0);
+        step(h0 + 2, lb2, lb3, lb1);
+        step(h0 + 3, lb3, lb4, lb2);
+        step(h0 + 4, lb4, lb5, lb3);
+        step(h0 + 5, lb5, lb0, lb4);
     }
-    if (full < nsteps) step(full, lb0, lb2);
-    if (full + 1 < nsteps) step(full + 1, lb1, lb0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the repeated requests of the last steps land before the LDS is given back
+    if (full < nhalf) step(full, lb0, lb1, lb5);
+    if (full + 1 < nhalf) step(full + 1, lb1, lb2, lb0);
+    if (full + 2 < nhalf) step(full + 2, lb2, lb3, lb1);
+    if (full + 3 < nhalf) step(full + 3, lb3, lb4, lb2);
+    if (full + 4 < nhalf) step(full + 4, lb4, lb5, lb3);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    if (mb0 * 32 + 128 <= g.M && (nb0 + 4 * WPW) * 32 <= g.N) {
+    if (mb0 * 32 + 128 <= g.M && (nb0 + 8) * 32 <= g.N) {
         float sc[2][16];
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) sc[i][v] = 1.0f;
-        if (g.a_inv_scale) {
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int v = 0; v < 16; v++)
-                    sc[i][v] = g.a_inv_scale[(mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3)];
-        }
+            for (int v = 0; v < 16; v++)
+                sc[i][v] = g.a_inv_scale ? g.a_inv_scale[(mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3)] : 1.0f;
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = (mb0 + 2 * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-                float *row = Cp + (size_t)m * g.ldp + (nb0 + NW * wn) * 32 + r;
+                float *row = Cp + (size_t)m * g.ldp + (nb0 + 4 * wn) * 32 + r;
 #pragma unroll
-                for (int k = 0; k < NW; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
+                for (int k = 0; k < 4; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
             }
         return;
     }
@@ -386,12 +381,13 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
             if (m >= g.M) continue;
             const float sc = g.a_inv_scale ? g.a_inv_scale[m] : 1.0f;
 #pragma unroll
-            for (int k = 0; k < NW; k++) {
-                const int n = (nb0 + NW * wn + k) * 32 + r;
+            for (int k = 0; k < 4; k++) {
+                const int n = (nb0 + 4 * wn + k) * 32 + r;
                 if (n < g.N) Cp[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
             }
         }
 }
+
 
 // The same product on a 256 x 256 block: four waves of 128 x 128 (sixteen accumulator tiles each, in the accumulation
 // registers), so that a wave reads 0.5 KB of LDS per MFMA instead of 0.75 and a block fetches half as many operand bytes
@@ -400,8 +396,8 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
 // The copies are LDS-direct loads issued as assembly, right after the barrier: the compiler does not count them among
 // its own loads (it cannot tell which LDS bytes a pending copy writes and would wait for all of them before every LDS
 // read); the wait before the barrier is written by hand.
-// In its loop this block runs at 1.5-1.7 PFLOP/s (60-67 % of the MFMA peak; 8192 x 8192 x 8192: 1 667 TFLOP/s) against 1.1
-// for 128 x 256, but there are half as many blocks: launch_gemm_big picks the one that loses less to partial rounds and
+// In its loop this block runs at 1.5-1.7 PFLOP/s (60-67 % of the MFMA peak; 8192 x 8192 x 8192: 1 667 TFLOP/s against 1 387
+// for 128 x 256), but there are half as many blocks: launch_gemm_big picks the one that loses less to partial rounds and
 // partial tiles.
 __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
 {
@@ -609,7 +605,7 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
             else if (w) hipLaunchKernelGGL(gemm_big_f16_256, grid, block, 0, stream(), a);
             else hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), a);
         };
-        if (g_big_block == 0 && !wide && deep && g.S == 1 && full >= 2 && rest > 0 && rest * 2 <= cus && wide_cols < N) {
+        if (g_big_block == 0 && !wide && deep && g.S == 1 && full >= 1 && rest > 0 && rest * 2 <= cus && wide_cols < N) {
             GemmKArgs g1 = g, g2 = g;
             g1.N = wide_cols; g1.Nb = wide_cols / 32;
             g2.N = N - wide_cols; g2.Nb = tiled_rb(g2.N);
