@@ -143,7 +143,13 @@ __global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, con
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l31 = lane & 31, h = lane >> 5;
     const int KbG = tiled_kb(N_in), MbG = tiled_rb(M_out), NbX = tiled_rb(N_in);
-    const int nk = blockIdx.x * 4 + wave, mb0 = blockIdx.y * 2;
+    // Workgroup ids go to the eight XCDs in turn; an XCD takes a contiguous share of the (row pair, column group) list,
+    // so the workgroups that read the same two row blocks of Y^T run on one XCD, one after the other, and fetch them
+    // into one L2 instead of one each
+    const int gx = (KbG + 3) >> 2, gy = (MbG + 1) >> 1, per_xcd = (gx * gy + 7) >> 3;
+    const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (item >= gx * gy || (int)(blockIdx.x >> 3) >= per_xcd) return;
+    const int nk = (item % gx) * 4 + wave, mb0 = (item / gx) * 2;
     const bool active = nk < KbG;                         // a wave past the last column block still fetches its share of Y
     const half8 *xp[2], *yp[2];
 #pragma unroll
@@ -331,7 +337,8 @@ void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const 
                   int M_out, int N_in, int T, int sgd, float lr)
 {
     if (M_out <= 0 || N_in <= 0 || T <= 0) return;
-    const dim3 grid((tiled_kb(N_in) + 3) / 4, (tiled_rb(M_out) + 1) / 2);
+    const int items = ((tiled_kb(N_in) + 3) / 4) * ((tiled_rb(M_out) + 1) / 2);
+    const dim3 grid((items + 7) / 8 * 8);                 // whole rounds of the eight XCDs; k_wgrad maps ids to tiles
     const half8 *x8 = reinterpret_cast<const half8 *>(XT), *y8 = reinterpret_cast<const half8 *>(YT);
     if (sgd) LAUNCH(k_wgrad<1>, grid, dim3(256), 0, x8, x_inv, y8, y_inv, target_tiled, M_out, N_in, tiled_kb(T), lr);
     else     LAUNCH(k_wgrad<0>, grid, dim3(256), 0, x8, x_inv, y8, y_inv, target_tiled, M_out, N_in, tiled_kb(T), lr);
