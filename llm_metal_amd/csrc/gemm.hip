@@ -125,6 +125,17 @@ __global__ __launch_bounds__(1024) void rows_to_f16_split_vec(
     if (threadIdx.x == 0) { inv_scale[row] = inv; inv_scale[M + row] = 1.0f / s2; }
 }
 
+// pseudo-random fp16 values in (-1, 1) for the timing entry points: constant operands would flatter the matrix cores,
+// whose power (and with it the clock the GPU holds) depends on how many operand bits toggle
+__global__ void fill_random_f16(half_t *p, size_t n, uint32_t seed)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t x = (uint32_t)i * 2654435761u ^ seed;
+    x ^= x >> 15; x *= 2246822519u; x ^= x >> 13; x *= 3266489917u; x ^= x >> 16;
+    p[i] = (half_t)(((int)(x & 0xffff) - 32768) * (1.0f / 32768.0f));
+}
+
 // C[m, n] = sum over planes of row m and of row M + m, each times its row factor
 __global__ void reduce_planes_split(const float *__restrict__ P, int S, size_t plane_stride, int ldp,
                                     const float *__restrict__ row_scale, float *__restrict__ C, int M, int N)
@@ -625,7 +636,12 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters
     const int nbuf = (int)((size_t)1200 * 1024 * 1024 / wb) + 1;
     HIP_CHECK(hipMalloc(&A, ab)); HIP_CHECK(hipMalloc(&W, wb * nbuf)); HIP_CHECK(hipMalloc(&D, db * nbuf));
     HIP_CHECK(hipMalloc(&P, pb)); HIP_CHECK(hipMalloc(&inv, (size_t)M * 4));
-    HIP_CHECK(hipMemsetAsync(A, 0x11, ab, stream())); HIP_CHECK(hipMemsetAsync(W, 0x11, wb * nbuf, stream()));
+    if (wf == 0) {                                         // F16 tiles: random values (Q8_0 tiles keep a constant pattern)
+        hipLaunchKernelGGL(fill_random_f16, dim3((unsigned)((ab / 2 + 255) / 256)), dim3(256), 0, stream(), (half_t *)A, ab / 2, 1u);
+        hipLaunchKernelGGL(fill_random_f16, dim3((unsigned)((wb * nbuf / 2 + 255) / 256)), dim3(256), 0, stream(), (half_t *)W, wb * nbuf / 2, 2u);
+    } else {
+        HIP_CHECK(hipMemsetAsync(A, 0x11, ab, stream())); HIP_CHECK(hipMemsetAsync(W, 0x11, wb * nbuf, stream()));
+    }
     HIP_CHECK(hipMemsetAsync(D, 0x11, db * nbuf, stream()));
     HIP_CHECK(hipMemsetAsync(inv, 0, (size_t)M * 4, stream()));
     hipEvent_t e0, e1;

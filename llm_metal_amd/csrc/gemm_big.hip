@@ -396,9 +396,9 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
 // The copies are LDS-direct loads issued as assembly, right after the barrier: the compiler does not count them among
 // its own loads (it cannot tell which LDS bytes a pending copy writes and would wait for all of them before every LDS
 // read); the wait before the barrier is written by hand.
-// In its loop this block runs at 1.5-1.7 PFLOP/s (60-67 % of the MFMA peak; 8192 x 8192 x 8192: 1 667 TFLOP/s against 1 387
-// for 128 x 256), but there are half as many blocks: launch_gemm_big picks the one that loses less to partial rounds and
-// partial tiles.
+// 8192 x 8192 x 8192 on random operands: 1 227 TFLOP/s against 1 083 for 128 x 256 (constant operands, which toggle few
+// bits and let the GPU hold a higher clock, give 1 667 and 1 387).  There are half as many blocks: launch_gemm_big picks
+// the shape that loses less to partial rounds and partial tiles.
 __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
 {
     constexpr int HB = 16 * 2 * 64;                       // half8 per buffer: [16 row blocks][2 slices][64 lanes]
