@@ -260,6 +260,7 @@ struct ProfRec { hipEvent_t a, b; double wbytes, flops; };
 int g_prof_on = 0;
 std::vector<ProfRec> g_prof;
 int g_force_nb = 0, g_force_S = 0;
+int g_wide_wg = 1;                     // eight-wave workgroups where K would be cut into ten or more chunks
 
 }  // namespace
 
@@ -281,7 +282,7 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq)
         p.n_tiles = (Nb + nb - 1) / nb;
         const int base = p.n_tiles * m_tiles;
         // about twelve waves per CU in flight, whatever the workgroup size
-        int S = g_force_S ? g_force_S : (3 * cus + base - 1) / base;
+        int S = g_force_S ? g_force_S : (12 * cus / p.nw + base - 1) / base;
         if (S < 1) S = 1;
         int steps = (Kb + S - 1) / S;
         if (!g_force_S) {
@@ -299,6 +300,9 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq)
     // a product too small to give every CU a workgroup of 64 weight rows (K is short as well) takes 32-row workgroups:
     // measured on 1152 x 1024 .. 1568 x 1152 at 64 rows, 4.3-4.6 us against 5.2-5.5
     if (!g_force_nb && p.nb == 2 && m_tiles == 1 && p.n_tiles * p.S < cus) split(1);
+    // few weight rows under a long K would be cut into ten or more chunks: eight waves per workgroup split K among
+    // themselves instead and leave half as many planes to write and to add
+    if (g_wide_wg && !g_force_S && m_tiles == 1 && p.S >= 20) { p.nw = 8; split(p.nb); }
     // rotate the K order unless the activation matrix is too big to stay in an XCD's L2
     p.rotate = (size_t)tiled_rb(M) * 32 * Kb * 64 * 2 <= (size_t)4 << 20;
     return p;
@@ -309,7 +313,7 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
 {
     if (M <= 0 || N <= 0 || K <= 0) return;
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
-    bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2) && p.nw == 4 && W.fmt >= 0 && W.fmt <= 2;
+    bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2) && (p.nw == 4 || (p.nw == 8 && p.m_tiles == 1)) && W.fmt >= 0 && W.fmt <= 2;
     if (W.fmt == 0) ok = ok && W.w16;
     if (W.fmt == 1) ok = ok && W.q && W.d && W.nbq >= 0 && W.nbq <= Nb && (W.nbq == Nb || (W.w16 && (W.nbq % p.nb) == 0));
     if (W.fmt == 2) ok = ok && W.q && W.d && W.kbq >= 0 && W.kbq <= Kb && (W.kbq == Kb || W.w16);
@@ -341,6 +345,9 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         if (p.m_tiles > 1) { \
             if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV, 1>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
             else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV, 1>), grid, block, lds, stream(), g); \
+        } else if (p.nw == 8) { \
+            if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 8, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
+            else hipLaunchKernelGGL((gemm_tiled<NBV, 8, ROT, SC, WFV>), grid, block, lds, stream(), g); \
         } else { \
             if (g_prof_on) hipExtLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), ev_a, ev_b, 0, g); \
             else hipLaunchKernelGGL((gemm_tiled<NBV, 4, ROT, SC, WFV>), grid, block, lds, stream(), g); \

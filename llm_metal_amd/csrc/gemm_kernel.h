@@ -78,6 +78,15 @@ __device__ __forceinline__ void load_w_q8_cols(half8 (&w)[4], const WeightOp &W,
     w[3] = q8_unpack8(r1[2], r1[3]) * s3;
 }
 
+// First register of the segment that wave w of nw still holds after `rounds` rounds of the accumulator exchange (see the
+// end of gemm_tiled): every round halves the segment, the wave whose bit nw >> (round + 1) is set keeps the upper half.
+__host__ __device__ constexpr int exchange_seg_lo(int regs, int nw, int w, int rounds)
+{
+    int lo = 0, len = regs;
+    for (int r = 0; r < rounds; r++) { len >>= 1; if (w & (nw >> (r + 1))) lo += len; }
+    return lo;
+}
+
 // grid: x = ceil(Nb / NB) weight-row tiles, y = S (K chunks), z = ceil(M / 64); block = NW waves of 64.
 // Kb = number of 64-wide K steps of the (padded) reduction; Nb, Mb = 32-row blocks of W and A.
 //
@@ -88,8 +97,9 @@ __device__ __forceinline__ void load_w_q8_cols(half8 (&w)[4], const WeightOp &W,
 // it all workgroups of a chunk ask L2 for the same activation lines at the same moment.
 // SCALE: multiply row m of the result by a_inv_scale[m] here (used when the output is final, S == 1);
 // otherwise the consumer of the partial planes applies the row factors.
-// NW = 4: the waves of a workgroup split its K chunk and add their accumulators through LDS; each then stores a quarter
-// of the tile.
+// NW = 4 or 8: the waves of a workgroup split its K chunk and add their accumulators through LDS; each then stores its
+// part of the tile.  Eight waves cut K into half as many chunks for the same number of waves in flight: half the planes
+// to write and for the consumer to add.
 // WF: weight format (WeightOp::fmt).  1: row blocks below W.nbq are Q8_0 tiles, the rest F16 tiles
 // (the trainable LoRA rows of the fused QKV weight); the planner keeps W.nbq a multiple of NB, so a
 // workgroup is of one kind.  2: K steps below W.kbq are Q8_0 tiles with column scales, the rest F16.
@@ -162,47 +172,46 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
                     acc[mb][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mb][j], w[b][j], acc[mb][b], 0, 0, 0);
     }
 
-    // Add the four waves' accumulators through LDS so that every wave ends up with the finished sums of a quarter of
-    // the tile and stores that quarter: the registers are numbered i = (mb * NB + b) * 16 + v; in round one the waves
-    // w and w ^ 2 exchange halves (waves 0, 1 keep the lower half), in round two the waves w and w ^ 1 exchange quarters
-    // of the half they kept.  Wave w finishes the registers [w * Q, (w + 1) * Q).
-    static_assert(NW == 4, "the exchange below is written for four waves");
-    constexpr int REGS = 2 * NB * 16, H = REGS / 2, Q = REGS / 4;
+    // Add the waves' accumulators through LDS so that every wave ends up with the finished sums of 1 / NW of the tile and
+    // stores that part.  The registers are numbered i = (mb * NB + b) * 16 + v.  In round r the waves w and
+    // w ^ (NW >> (r + 1)) exchange halves of the segment both still hold (the wave without that bit keeps the lower half),
+    // so after log2(NW) rounds wave w holds the sums of [seg_lo(w), seg_lo(w) + REGS / NW); the last round's addition
+    // is done on the way to memory.
+    static_assert(NW == 4 || NW == 8, "the exchange below is written for four or eight waves");
+    constexpr int REGS = 2 * NB * 16, ROUNDS = NW == 4 ? 2 : 3;
 #define ACC_AT(i) acc[(i) / (NB * 16)][((i) / 16) % NB][(i) % 16]
-    {
-        float *mine = red + (size_t)wave * H * 64;
-        const float *theirs = red + (size_t)(wave ^ 2) * H * 64;
-        if (wave < 2) {
-#pragma unroll
-            for (int k = 0; k < H; k++) mine[k * 64 + lane] = ACC_AT(H + k);
-        } else {
-#pragma unroll
-            for (int k = 0; k < H; k++) mine[k * 64 + lane] = ACC_AT(k);
-        }
-        __syncthreads();
-        if (wave < 2) {
-#pragma unroll
-            for (int k = 0; k < H; k++) ACC_AT(k) += theirs[k * 64 + lane];
-        } else {
-#pragma unroll
-            for (int k = 0; k < H; k++) ACC_AT(H + k) += theirs[k * 64 + lane];
-        }
-        __syncthreads();                                  // all have read before the slots are written again
-    }
-    float *Pp = g.P + (size_t)by * g.plane_stride;
-    float *mine = red + (size_t)wave * Q * 64;
-    const float *theirs = red + (size_t)(wave ^ 1) * Q * 64;
-#define QUARTER_GIVE(W) if (wave == (W)) { _Pragma("unroll") for (int k = 0; k < Q; k++) mine[k * 64 + lane] = ACC_AT(((W) ^ 1) * Q + k); }
-    QUARTER_GIVE(0) QUARTER_GIVE(1) QUARTER_GIVE(2) QUARTER_GIVE(3)
-#undef QUARTER_GIVE
+    // what wave W gives away in round R: the half of its segment that it does not keep
+#define GIVE(W, R) if constexpr ((W) < NW) { if (wave == (W)) { \
+        constexpr int half = REGS >> ((R) + 1), bit = NW >> ((R) + 1), lo = exchange_seg_lo(REGS, NW, (W), (R)); \
+        constexpr int give_lo = ((W) & bit) ? lo : lo + half; \
+        float *mine = red + (size_t)(W) * half * 64; \
+        _Pragma("unroll") for (int k = 0; k < half; k++) mine[k * 64 + lane] = ACC_AT(give_lo + k); } }
+#define TAKE(W, R) if constexpr ((W) < NW) { if (wave == (W)) { \
+        constexpr int half = REGS >> ((R) + 1), bit = NW >> ((R) + 1), keep_lo = exchange_seg_lo(REGS, NW, (W), (R) + 1); \
+        const float *theirs = red + (size_t)((W) ^ bit) * half * 64; \
+        _Pragma("unroll") for (int k = 0; k < half; k++) ACC_AT(keep_lo + k) += theirs[k * 64 + lane]; } }
+#define ALL_WAVES(OP, R) OP(0, R) OP(1, R) OP(2, R) OP(3, R) OP(4, R) OP(5, R) OP(6, R) OP(7, R)
+    ALL_WAVES(GIVE, 0)
     __syncthreads();
+    ALL_WAVES(TAKE, 0)
+    __syncthreads();                                      // all have read before the slots are written again
+    if constexpr (ROUNDS == 3) {
+        ALL_WAVES(GIVE, 1)
+        __syncthreads();
+        ALL_WAVES(TAKE, 1)
+        __syncthreads();
+    }
+    ALL_WAVES(GIVE, ROUNDS - 1)
+    __syncthreads();
+    float *Pp = g.P + (size_t)by * g.plane_stride;
     // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8*(v/4) + 4*(lane/32) + v%4.  SCALE: the row factors
     // are fetched here, where the K loop's registers are free (holding them through the loop costs a wave of occupancy).
     // A tile inside the matrix stores without bounds tests: under a test per element the compiler puts each LDS read into
     // the branch of its store, and the sixteen read-wait-store groups run one after the other.
     const bool inside = (mb0 + 2) * 32 <= M && (nb0 + NB) * 32 <= N;
-#define QUARTER_STORE(W) if (wave == (W)) { \
-        constexpr int i0 = (W) * Q; \
+#define PART_STORE(W, R) if constexpr ((W) < NW) { if (wave == (W)) { \
+        constexpr int Q = REGS / NW, i0 = exchange_seg_lo(REGS, NW, (W), ROUNDS); \
+        const float *theirs = red + (size_t)((W) ^ 1) * Q * 64; \
         float sc[Q], sres[Q]; \
         if (SCALE) { \
             /* all factors requested before the first store (row clamped): a load under the store's condition would make \
@@ -228,9 +237,12 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
                 const int m = (mb0 + mb) * 32 + 8 * (v >> 2) + 4 * h + (v & 3), n = (nb0 + b) * 32 + r; \
                 if (m < M && n < N) Pp[(size_t)m * g.ldp + n] = sres[k]; \
             } \
-        } }
-    QUARTER_STORE(0) QUARTER_STORE(1) QUARTER_STORE(2) QUARTER_STORE(3)
-#undef QUARTER_STORE
+        } } }
+    ALL_WAVES(PART_STORE, 0)
+#undef PART_STORE
+#undef ALL_WAVES
+#undef TAKE
+#undef GIVE
 #undef ACC_AT
 }
 
