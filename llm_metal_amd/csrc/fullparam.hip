@@ -131,24 +131,47 @@ __global__ __launch_bounds__(256) void k_transpose_scaled_pair(TransposeJob j0, 
     transpose_scaled_block(j.in, j.in_inv, T, j.F, j.out, j.out_inv, first ? blockIdx.x : blockIdx.x - nb0);
 }
 
+// Up to eight operands in one launch (both operands of the four weight gradients of a layer): workgroup id -> job by the
+// jobs' first ids.
+struct TransposeJobs { TransposeJob j[8]; int first[9]; int n; };
+__global__ __launch_bounds__(256) void k_transpose_scaled_jobs(TransposeJobs js, int T)
+{
+    int k = 0;
+#pragma unroll
+    for (int i = 1; i < 8; i++) if (i < js.n && (int)blockIdx.x >= js.first[i]) k = i;      // uniform per workgroup
+    const TransposeJob &j = js.j[k];
+    transpose_scaled_block(j.in, j.in_inv, T, j.F, j.out, j.out_inv, blockIdx.x - js.first[k]);
+}
+
 // Target[m][n] (tiled [M_out, N_in] F16) <- half(float(Target) + alpha * sum_t Y[t][m] X[t][n])
 // with XT = tiled [N_in, T], YT = tiled [M_out, T] and their row factors.  SGD: alpha = -lr, else 1.
 // grid: x = ceil(Kb / 4) (each wave one 64-wide column block), y = ceil(Mb / 2); block 256.
 // The MFMA's first operand supplies the rows of its result, so feeding X there puts four
 // consecutive n into each lane's registers: exactly the 8-byte groups of the tiled target.
+// One to four weight gradients per launch (the four matrices of a layer in accumulate mode).  Workgroup ids go to the
+// eight XCDs in turn; an XCD takes a contiguous share of the list of (matrix, row pair, column group) items, so the
+// workgroups that read the same two row blocks of Y^T run on one XCD, one after the other, and fetch them into one L2
+// instead of one each.
+struct WgradJob { const half8 *XT; const float *x_inv; const half8 *YT; const float *y_inv; half_t *target; int M_out, N_in; };
+struct WgradJobs { WgradJob j[4]; int first[5]; int n; };
+
 template <int SGD>
-__global__ __launch_bounds__(256) void k_wgrad(const half8 *__restrict__ XT, const float *__restrict__ x_inv,
-                                               const half8 *__restrict__ YT, const float *__restrict__ y_inv,
-                                               half_t *__restrict__ target, int M_out, int N_in, int Kt, float lr)
+__global__ __launch_bounds__(256) void k_wgrad(WgradJobs js, int Kt, float lr)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l31 = lane & 31, h = lane >> 5;
+    const int total = js.first[js.n], per_xcd = (total + 7) >> 3;
+    int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (item >= total || (int)(blockIdx.x >> 3) >= per_xcd) return;
+    int k = 0;
+#pragma unroll
+    for (int i = 1; i < 4; i++) if (i < js.n && item >= js.first[i]) k = i;                  // uniform per workgroup
+    item -= js.first[k];
+    const half8 *__restrict__ XT = js.j[k].XT, *__restrict__ YT = js.j[k].YT;
+    const float *__restrict__ x_inv = js.j[k].x_inv, *__restrict__ y_inv = js.j[k].y_inv;
+    half_t *__restrict__ target = js.j[k].target;
+    const int M_out = js.j[k].M_out, N_in = js.j[k].N_in;
     const int KbG = tiled_kb(N_in), MbG = tiled_rb(M_out), NbX = tiled_rb(N_in);
-    // Workgroup ids go to the eight XCDs in turn; an XCD takes a contiguous share of the (row pair, column group) list,
-    // so the workgroups that read the same two row blocks of Y^T run on one XCD, one after the other, and fetch them
-    // into one L2 instead of one each
-    const int gx = (KbG + 3) >> 2, gy = (MbG + 1) >> 1, per_xcd = (gx * gy + 7) >> 3;
-    const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (item >= gx * gy || (int)(blockIdx.x >> 3) >= per_xcd) return;
+    const int gx = (KbG + 3) >> 2;
     const int nk = (item % gx) * 4 + wave, mb0 = (item / gx) * 2;
     const bool active = nk < KbG;                         // a wave past the last column block still fetches its share of Y
     const half8 *xp[2], *yp[2];
@@ -333,15 +356,47 @@ void launch_transpose_scaled_pair(const half_t *in0, const float *in0_inv, int F
     LAUNCH(k_transpose_scaled_pair, dim3(nb0 + tiled_kb(F1)), dim3(256), 0, j0, j1, T, nb0);
 }
 
+void launch_transpose_scaled_jobs(const TransposeOperand *ops, int n, int T)
+{
+    if (n <= 0 || n > 8 || T <= 0) { fprintf(stderr, "[fast_hip] transpose_scaled_jobs: %d operands\n", n); abort(); }
+    TransposeJobs js{};
+    js.n = n;
+    int total = 0;
+    for (int i = 0; i < n; i++) {
+        if (ops[i].F <= 0) { fprintf(stderr, "[fast_hip] transpose_scaled_jobs: empty operand\n"); abort(); }
+        js.j[i] = TransposeJob{reinterpret_cast<const half8 *>(ops[i].in), ops[i].in_inv, ops[i].F, reinterpret_cast<half8 *>(ops[i].out), ops[i].out_inv};
+        js.first[i] = total;
+        total += tiled_kb(ops[i].F);
+    }
+    js.first[n] = total;
+    LAUNCH(k_transpose_scaled_jobs, dim3(total), dim3(256), 0, js, T);
+}
+
+void launch_wgrads(const WgradOperands *w, int n, int T, int sgd, float lr)
+{
+    if (n <= 0 || n > 4 || T <= 0) { fprintf(stderr, "[fast_hip] wgrads: %d matrices\n", n); abort(); }
+    WgradJobs js{};
+    js.n = n;
+    int total = 0;
+    for (int i = 0; i < n; i++) {
+        if (w[i].M_out <= 0 || w[i].N_in <= 0) { fprintf(stderr, "[fast_hip] wgrads: empty matrix\n"); abort(); }
+        js.j[i] = WgradJob{reinterpret_cast<const half8 *>(w[i].XT), w[i].x_inv, reinterpret_cast<const half8 *>(w[i].YT), w[i].y_inv,
+                           w[i].target_tiled, w[i].M_out, w[i].N_in};
+        js.first[i] = total;
+        total += ((tiled_kb(w[i].N_in) + 3) / 4) * ((tiled_rb(w[i].M_out) + 1) / 2);
+    }
+    for (int i = n; i <= 4; i++) js.first[i] = total;
+    const dim3 grid((total + 7) / 8 * 8);                 // whole rounds of the eight XCDs; k_wgrad maps ids to tiles
+    if (sgd) LAUNCH(k_wgrad<1>, grid, dim3(256), 0, js, tiled_kb(T), lr);
+    else     LAUNCH(k_wgrad<0>, grid, dim3(256), 0, js, tiled_kb(T), lr);
+}
+
 void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,
                   int M_out, int N_in, int T, int sgd, float lr)
 {
     if (M_out <= 0 || N_in <= 0 || T <= 0) return;
-    const int items = ((tiled_kb(N_in) + 3) / 4) * ((tiled_rb(M_out) + 1) / 2);
-    const dim3 grid((items + 7) / 8 * 8);                 // whole rounds of the eight XCDs; k_wgrad maps ids to tiles
-    const half8 *x8 = reinterpret_cast<const half8 *>(XT), *y8 = reinterpret_cast<const half8 *>(YT);
-    if (sgd) LAUNCH(k_wgrad<1>, grid, dim3(256), 0, x8, x_inv, y8, y_inv, target_tiled, M_out, N_in, tiled_kb(T), lr);
-    else     LAUNCH(k_wgrad<0>, grid, dim3(256), 0, x8, x_inv, y8, y_inv, target_tiled, M_out, N_in, tiled_kb(T), lr);
+    const WgradOperands w{XT, x_inv, YT, y_inv, target_tiled, M_out, N_in};
+    launch_wgrads(&w, 1, T, sgd, lr);
 }
 
 void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr)

@@ -215,10 +215,16 @@ void launch_transpose_scaled(const half_t *in_tiled, const float *in_inv, int T,
 // two operands [T, F0] and [T, F1] in one launch
 void launch_transpose_scaled_pair(const half_t *in0, const float *in0_inv, int F0, half_t *out0, float *out0_inv,
                                   const half_t *in1, const float *in1_inv, int F1, half_t *out1, float *out1_inv, int T);
+// up to eight operands [T, F] in one launch
+struct TransposeOperand { const half_t *in; const float *in_inv; int F; half_t *out; float *out_inv; };
+void launch_transpose_scaled_jobs(const TransposeOperand *ops, int n, int T);
 // target (tiled [M_out, N_in] F16) <- half(target + alpha * Y^T X), XT/YT = transposed operands over T tokens;
 // sgd: alpha = -lr (f16_sgd_fused), else alpha = 1 (f16_grad_accum)
 void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,
                   int M_out, int N_in, int T, int sgd, float lr);
+// the same for up to four matrices in one launch
+struct WgradOperands { const half_t *XT; const float *x_inv; const half_t *YT; const float *y_inv; half_t *target_tiled; int M_out, N_in; };
+void launch_wgrads(const WgradOperands *w, int n, int T, int sgd, float lr);
 // G != null: W = half(W - lr G), G = 0 (f16_sgd_apply); always: WT (tiled [N_in, M_out]) <- W^T
 void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr);
 void launch_untile_f16(const half_t *src_tiled, int Kb, int row_off, int k_off, int transpose, int rows, int cols, half_t *dst);

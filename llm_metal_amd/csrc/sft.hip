@@ -87,6 +87,9 @@ struct SFTState {
     MetalBuf *ln2_16, *ln2_inv, *act16, *act_inv, *attn16, *lnf16, *lnf_inv;
     size_t st_act, st_attn;
     MetalBuf *xT, *xT_inv, *yT, *yT_inv; // transposed operands of the weight gradient being formed
+    // accumulate mode: the loss-gradient operands of a layer's four products (down, gate|up, o, qkv) stay until its
+    // backward has run, and all eight operands of its weight gradients are transposed in one launch
+    MetalBuf *dy16[4], *dy_inv[4], *lyT[4], *lyT_inv[4], *lxT[4], *lxT_inv[4];
     MetalBuf *gqkv, *go, *ggu, *gd, *glm;   // F16 gradient accumulators, tiled like the weights (sft_alloc_grad_accum)
     MetalBuf *grpo_old_lp, *grpo_advs, *grpo_new_lp;   // host-visible [BN] inputs/outputs of the policy gradient
     float *grpo_old_lp_cpu, *grpo_advs_cpu, *grpo_new_lp_cpu;
@@ -453,6 +456,14 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
     float *ainv = at<float>(s->a16_inv);
     const bool gemma = s->model_type == MODEL_GEMMA3;
     int cur = 0;                                          // dx ping-pong
+    // Accumulate mode: each of a layer's four loss-gradient operands (of down, gate|up, o, qkv) has a buffer of its own,
+    // so that all four weight gradients can be formed after the layer's last row kernel: one launch transposes their
+    // eight operands instead of four launches of two (the weights do not change before the apply, so the order of the
+    // reference's f16_grad_accum calls, src/nn/fast_sft.c:804-946, does not matter).  Otherwise one buffer serves all.
+    const bool defer = mode == BWD_ACCUM && s->dy16[0];
+    half_t *d16[4];
+    float *dinv[4];
+    for (int i = 0; i < 4; i++) { d16[i] = defer ? at<half_t>(s->dy16[i]) : a16; dinv[i] = defer ? at<float>(s->dy_inv[i]) : ainv; }
 
     // dx = RNB(x_final, dlogits Wlm; g_final)                                [:777-790]
     Planes p = gemm(s, at<half_t>(s->dl16), at<float>(s->dl_inv), wop(s, W_LM, 0, true), D, s->V);
@@ -463,24 +474,24 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
     nb.dy = p; nb.x_saved = at<float>(s->xs, (size_t)(2 * NL) * xsz); nb.g = at<float>(s->g_final);
     nb.eps = s->eps; nb.D = D; nb.dx_prev = nullptr; nb.dx_out = at<float>(s->dx[cur]); nb.clamp = 0.f;
     if (gemma) { nb.branch_raw = at<float>(s->ff_raw, (size_t)(NL - 1) * xsz); nb.g_branch = at<float>(s->g_post_ff, (size_t)(NL - 1) * D); }
-    nb.d16 = a16; nb.inv_scale = ainv;
+    nb.d16 = d16[0]; nb.inv_scale = dinv[0];
     if (mode == BWD_LORA) nb.pf = prefetch_for(s, wop(s, W_D, NL - 1, true), IS, D, 1024);
     launch_norm_bwd_rows(nb, BN);
 
     for (int L = NL - 1; L >= 0; L--) {
         // FFN: d act = d Wd; (dgate, dup); dln2 = dgate Wg + dup Wu; dx += RNB(x_mid, dln2)   [:798-874]
-        Planes pd = gemm(s, a16, ainv, wop(s, W_D, L, true), IS, D);
-        if (mode != BWD_LORA)                                                 // [:804-811, 842-849]
+        Planes pd = gemm(s, d16[0], dinv[0], wop(s, W_D, L, true), IS, D);
+        if (mode != BWD_LORA && !defer)                                       // [:804-811, 842-849]
             weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->act16, L * s->st_act), at<float>(s->act_inv, (size_t)L * BN), IS,
                         s->wd, s->wdT, s->gd, L * s->st_d, L * s->st_dT);
         GluArgs gb{};
         gb.in = pd; gb.IS = IS; gb.gelu = gemma;
         gb.gate_pre = at<float>(s->gu_sav, (size_t)L * BN * 2 * IS); gb.up_val = gb.gate_pre + IS; gb.ld_gu = (size_t)2 * IS;
         if (mode == BWD_LORA) gb.sg = scale_groups_for(s, wop(s, W_GU, L, true), D, 2 * IS);
-        gb.out16 = a16; gb.inv_scale = gb.sg.cols ? at<float>(s->group_inv) : ainv;
+        gb.out16 = d16[1]; gb.inv_scale = gb.sg.cols ? at<float>(s->group_inv) : dinv[1];
         launch_glu_bwd(gb, BN);
-        Planes pgu = gemm(s, a16, gb.inv_scale, wop(s, W_GU, L, true), D, 2 * IS, nullptr, &gb.sg);
-        if (mode != BWD_LORA)                                                 // gate and up as one matrix [:817-833, 853-869]
+        Planes pgu = gemm(s, d16[1], gb.inv_scale, wop(s, W_GU, L, true), D, 2 * IS, nullptr, &gb.sg);
+        if (mode != BWD_LORA && !defer)                                       // gate and up as one matrix [:817-833, 853-869]
             weight_grad(s, mode, lr, a16, ainv, 2 * IS, at<half_t>(s->ln2_16, L * s->st_ln1), at<float>(s->ln2_inv, (size_t)L * BN), D,
                         s->wgu, s->wguT, s->ggu, L * s->st_gu, L * s->st_guT);
         NormBwdArgs n2{};
@@ -488,14 +499,14 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         n2.g = gemma ? at<float>(s->g_pre_ff, (size_t)L * D) : at<float>(s->g_post_attn, (size_t)L * D);
         n2.eps = s->eps; n2.D = D; n2.dx_prev = at<float>(s->dx[cur]); n2.dx_out = at<float>(s->dx[cur ^ 1]); n2.clamp = 0.f;
         if (gemma) { n2.branch_raw = at<float>(s->o_raw, (size_t)L * xsz); n2.g_branch = at<float>(s->g_post_attn, (size_t)L * D); }
-        n2.d16 = a16; n2.inv_scale = ainv;
+        n2.d16 = d16[2]; n2.inv_scale = dinv[2];
         if (mode == BWD_LORA) n2.pf = prefetch_for(s, wop(s, W_O, L, true), qd, D, 1024);
         launch_norm_bwd_rows(n2, BN);
         cur ^= 1;
 
         // attention: dO = d Wo; dq, dk, dv                                    [:877-911]
-        Planes pdo = gemm(s, a16, ainv, wop(s, W_O, L, true), qd, D);
-        if (mode != BWD_LORA)                                                 // [:883-901]
+        Planes pdo = gemm(s, d16[2], dinv[2], wop(s, W_O, L, true), qd, D);
+        if (mode != BWD_LORA && !defer)                                       // [:883-901]
             weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->attn16, L * s->st_attn), at<float>(s->ones), qd,
                         s->wo, s->woT, s->go, L * s->st_o, L * s->st_oT);
         AttnBwdArgs ab{};
@@ -529,23 +540,44 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         qb.R = R; qb.sc = s->lora_scaling;
         qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
         qb.dq_f = at<float>(s->dq_f, keepL * BN * qd); qb.dv_f = nullptr; qb.dh = at<float>(s->dh, keepL * BN * (R ? 2 * R : 1));
-        qb.out16 = a16; qb.inv_scale = ainv;
+        qb.out16 = d16[3]; qb.inv_scale = dinv[3];
         if (mode == BWD_LORA) qb.pf = prefetch_for(s, wop(s, W_QKV, L, true), D, s->nq_ext, 1024);
         launch_qkv_bwd(qb, BN);
+        if (defer) {
+            // the layer's four weight gradients: eight transposes in one launch, then G += dY^T X for the four matrices in one
+            const int m_out[4] = {D, 2 * IS, D, s->nq_ext}, n_in[4] = {IS, D, qd, D};
+            const half_t *x16[4] = {at<half_t>(s->act16, L * s->st_act), at<half_t>(s->ln2_16, L * s->st_ln1),
+                                    at<half_t>(s->attn16, L * s->st_attn), at<half_t>(s->ln1_16, (size_t)L * s->st_ln1)};
+            const float *xinv[4] = {at<float>(s->act_inv, (size_t)L * BN), at<float>(s->ln2_inv, (size_t)L * BN), at<float>(s->ones),
+                                    at<float>(s->ln1_inv, (size_t)L * BN)};
+            MetalBuf *G[4] = {s->gd, s->ggu, s->go, s->gqkv};
+            const size_t goff[4] = {L * s->st_d, L * s->st_gu, L * s->st_o, L * s->st_qkv};
+            TransposeOperand ops[8];
+            for (int i = 0; i < 4; i++) {
+                ops[2 * i] = TransposeOperand{d16[i], dinv[i], m_out[i], at<half_t>(s->lyT[i]), at<float>(s->lyT_inv[i])};
+                ops[2 * i + 1] = TransposeOperand{x16[i], xinv[i], n_in[i], at<half_t>(s->lxT[i]), at<float>(s->lxT_inv[i])};
+            }
+            launch_transpose_scaled_jobs(ops, 8, BN);
+            WgradOperands wg[4];
+            for (int i = 0; i < 4; i++)
+                wg[i] = WgradOperands{at<half_t>(s->lxT[i]), at<float>(s->lxT_inv[i]), at<half_t>(s->lyT[i]), at<float>(s->lyT_inv[i]),
+                                      at<half_t>(G[i], goff[i]), m_out[i], n_in[i]};
+            launch_wgrads(wg, 4, BN, 0, 0.f);
+        }
         // full-parameter: W_q, W_k, W_v are updated BEFORE the dX product, which then multiplies with the
         // new weights in SGD mode, as the reference does                       [:922-946]
-        if (mode != BWD_LORA)
+        if (mode != BWD_LORA && !defer)
             weight_grad(s, mode, lr, a16, ainv, s->nq_ext, at<half_t>(s->ln1_16, (size_t)L * s->st_ln1), at<float>(s->ln1_inv, (size_t)L * BN), D,
                         s->wqkv, s->wqkvT, s->gqkv, L * s->st_qkv, L * s->st_qkvT);
 
         // dln1 = [dq|dk|dv|dh] [Wq;Wk;Wv;A_q;A_v]; dx += RNB(x_in, dln1; g_in); clamp     [:956-980]
-        Planes pl = gemm(s, a16, ainv, wop(s, W_QKV, L, true), D, s->nq_ext);
+        Planes pl = gemm(s, d16[3], dinv[3], wop(s, W_QKV, L, true), D, s->nq_ext);
         NormBwdArgs n1{};
         n1.dy = pl; n1.x_saved = at<float>(s->xs, (size_t)(2 * L) * xsz); n1.g = at<float>(s->g_in, (size_t)L * D);
         n1.eps = s->eps; n1.D = D; n1.dx_prev = at<float>(s->dx[cur]); n1.dx_out = at<float>(s->dx[cur ^ 1]); n1.clamp = 1e6f;
         if (L > 0) {
             if (gemma) { n1.branch_raw = at<float>(s->ff_raw, (size_t)(L - 1) * xsz); n1.g_branch = at<float>(s->g_post_ff, (size_t)(L - 1) * D); }
-            n1.d16 = a16; n1.inv_scale = ainv;
+            n1.d16 = d16[0]; n1.inv_scale = dinv[0];
         }
         if (mode == BWD_LORA && L > 0) n1.pf = prefetch_for(s, wop(s, W_D, L - 1, true), IS, D, 1024);
         launch_norm_bwd_rows(n1, BN);
@@ -861,6 +893,8 @@ void sft_state_free(SFTState *s)
                        s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
                        s->grpo_old_lp, s->grpo_advs, s->grpo_new_lp, s->lora_acc, s->lm_head_out.mbuf,
                        s->fa_q, s->fa_k, s->fa_v, s->fa_O, s->fa_lse, s->fa_do, s->fa_D, s->fa_dkp, s->fa_dvp};
+    for (int i = 0; i < 4; i++)
+        for (MetalBuf *b : {s->dy16[i], s->dy_inv[i], s->lyT[i], s->lyT_inv[i], s->lxT[i], s->lxT_inv[i]}) metal_buf_free(b);
     for (MetalBuf *b : s->views_out) metal_buf_free(b);
     for (auto &kv : s->img_slots) metal_buf_free(kv.second);
     for (MetalBuf *b : all) metal_buf_free(b);
@@ -951,6 +985,13 @@ void sft_alloc_grad_accum(SFTState *s)
     s->ggu = hbuf(s->NL * s->st_gu);   s->gd = hbuf(s->NL * s->st_d);
     s->glm = hbuf(tiled_elems(s->V, s->D));
     for (MetalBuf *b : {s->gqkv, s->go, s->ggu, s->gd, s->glm}) HIP_CHECK(hipMemsetAsync(dptr(b), 0, b->size, stream()));
+    const int m_out[4] = {s->D, 2 * s->IS, s->D, s->nq_ext}, n_in[4] = {s->IS, s->D, s->qd, s->D};
+    for (int i = 0; i < 4; i++) {
+        s->dy16[i] = hbuf(tiled_elems(s->BN, m_out[i])); s->dy_inv[i] = fbuf(s->BN);
+        HIP_CHECK(hipMemsetAsync(dptr(s->dy16[i]), 0, s->dy16[i]->size, stream()));      // row and K padding must read as zero
+        s->lyT[i] = hbuf(tiled_elems(m_out[i], s->BN)); s->lyT_inv[i] = fbuf((size_t)tiled_kb(m_out[i]) * 64);
+        s->lxT[i] = hbuf(tiled_elems(n_in[i], s->BN));  s->lxT_inv[i] = fbuf((size_t)tiled_kb(n_in[i]) * 64);
+    }
     const double mb = 2.0 * ((double)s->NL * (s->st_qkv + s->st_o + s->st_gu + s->st_d) + (double)tiled_elems(s->V, s->D)) / (1024.0 * 1024.0);
     printf("[FastSFT] Grad accum buffers allocated: %.2f MB\n", mb);
 }
