@@ -286,12 +286,15 @@ __global__ __launch_bounds__(256) void k_wgrad(WgradJobs js, int Kt, float lr)
 
 // 64 x 64 blocks of W (tiled [Mo, Ni]):  if G: W = half(W - lr * G), G = 0 (f16_sgd_apply);
 // then the block is written, transposed, into WT (tiled [Ni, Mo]).
-// grid: x = K blocks of W, y = ceil(row tiles / 2); block 256.
+// grid: x = K blocks of W, y = ceil(row tiles / 2), z = matrices of this shape (the layers of an arena, st / stT half8
+// apart in W and G / in WT); block 256.
 __global__ __launch_bounds__(256) void k_apply_retile(half8 *__restrict__ W, half8 *__restrict__ G, half8 *__restrict__ WT,
-                                                       int Mo, int Ni, float lr)
+                                                       int Mo, int Ni, float lr, size_t st, size_t stT)
 {
     __shared__ half_t t[64][72];
     const int tid = threadIdx.x, bx = blockIdx.x, by = blockIdx.y;
+    W += blockIdx.z * st; WT += blockIdx.z * stT;
+    if (G) G += blockIdx.z * st;
     const int KbW = tiled_kb(Ni), MbW = tiled_rb(Mo), KbT = tiled_kb(Mo), NbT = tiled_rb(Ni);
     for (int q = tid; q < 512; q += 256) {
         const int th = q >> 8, qq = q & 255, mbt = by * 2 + th;
@@ -399,11 +402,13 @@ void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const 
     launch_wgrads(&w, 1, T, sgd, lr);
 }
 
-void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr)
+void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr,
+                         int matrices, size_t stride, size_t strideT)
 {
-    if (M_out <= 0 || N_in <= 0) return;
-    LAUNCH(k_apply_retile, dim3(tiled_kb(N_in), (tiled_rb(M_out) + 1) / 2), dim3(256), 0, reinterpret_cast<half8 *>(W_tiled),
-           reinterpret_cast<half8 *>(G_tiled), reinterpret_cast<half8 *>(WT_tiled), M_out, N_in, lr);
+    if (M_out <= 0 || N_in <= 0 || matrices <= 0) return;
+    if (matrices > 65535 || (stride & 7) || (strideT & 7)) { fprintf(stderr, "[fast_hip] apply_retile: bad strides\n"); abort(); }
+    LAUNCH(k_apply_retile, dim3(tiled_kb(N_in), (tiled_rb(M_out) + 1) / 2, matrices), dim3(256), 0, reinterpret_cast<half8 *>(W_tiled),
+           reinterpret_cast<half8 *>(G_tiled), reinterpret_cast<half8 *>(WT_tiled), M_out, N_in, lr, stride / 8, strideT / 8);
 }
 
 void launch_untile_f16(const half_t *src_tiled, int Kb, int row_off, int k_off, int transpose, int rows, int cols, half_t *dst)

@@ -225,8 +225,10 @@ void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const 
 // the same for up to four matrices in one launch
 struct WgradOperands { const half_t *XT; const float *x_inv; const half_t *YT; const float *y_inv; half_t *target_tiled; int M_out, N_in; };
 void launch_wgrads(const WgradOperands *w, int n, int T, int sgd, float lr);
-// G != null: W = half(W - lr G), G = 0 (f16_sgd_apply); always: WT (tiled [N_in, M_out]) <- W^T
-void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr);
+// G != null: W = half(W - lr G), G = 0 (f16_sgd_apply); always: WT (tiled [N_in, M_out]) <- W^T.  `matrices` of the same
+// shape in one launch, `stride` halves apart in W and G and `strideT` in WT (the layers of an arena).
+void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int M_out, int N_in, float lr,
+                         int matrices = 1, size_t stride = 0, size_t strideT = 0);
 void launch_untile_f16(const half_t *src_tiled, int Kb, int row_off, int k_off, int transpose, int rows, int cols, half_t *dst);
 
 }  // namespace lmhip

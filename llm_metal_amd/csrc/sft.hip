@@ -1001,12 +1001,11 @@ void sft_alloc_grad_accum(SFTState *s)
 void sft_apply_grad_sgd(SFTState *s, float lr)
 {
     if (!s->gqkv) return;
-    for (int L = 0; L < s->NL; L++) {
-        launch_apply_retile(at<half_t>(s->wqkv, L * s->st_qkv), at<half_t>(s->gqkv, L * s->st_qkv), at<half_t>(s->wqkvT, L * s->st_qkvT), s->nq_ext, s->D, lr);
-        launch_apply_retile(at<half_t>(s->wo, L * s->st_o), at<half_t>(s->go, L * s->st_o), at<half_t>(s->woT, L * s->st_oT), s->D, s->qd, lr);
-        launch_apply_retile(at<half_t>(s->wgu, L * s->st_gu), at<half_t>(s->ggu, L * s->st_gu), at<half_t>(s->wguT, L * s->st_guT), 2 * s->IS, s->D, lr);
-        launch_apply_retile(at<half_t>(s->wd, L * s->st_d), at<half_t>(s->gd, L * s->st_d), at<half_t>(s->wdT, L * s->st_dT), s->D, s->IS, lr);
-    }
+    // one launch per arena: the layers of a kind have one shape and lie at equal distances
+    launch_apply_retile(at<half_t>(s->wqkv), at<half_t>(s->gqkv), at<half_t>(s->wqkvT), s->nq_ext, s->D, lr, s->NL, s->st_qkv, s->st_qkvT);
+    launch_apply_retile(at<half_t>(s->wo), at<half_t>(s->go), at<half_t>(s->woT), s->D, s->qd, lr, s->NL, s->st_o, s->st_oT);
+    launch_apply_retile(at<half_t>(s->wgu), at<half_t>(s->ggu), at<half_t>(s->wguT), 2 * s->IS, s->D, lr, s->NL, s->st_gu, s->st_guT);
+    launch_apply_retile(at<half_t>(s->wd), at<half_t>(s->gd), at<half_t>(s->wdT), s->D, s->IS, lr, s->NL, s->st_d, s->st_dT);
     launch_apply_retile(at<half_t>(s->wlm), at<half_t>(s->glm), at<half_t>(s->wlmT), s->V, s->D, lr);
     metal_flush();
 }
