@@ -10,8 +10,9 @@
 // per consumer), and both go to LDS in the same [j][lane][8 halves] order, so a wave reads any row block back
 // with conflict-free 16-byte loads.  LDS is double buffered and the operands travel three steps ahead in registers:
 // during the MFMAs of step k the loads of step k+3 are issued and step k+1 is written to the other buffer; one
-// barrier per step.  That is the kernel for Q8_0 tiles (gemm_big<1>, <2>); F16 tiles take gemm_big_f16 below, whose
-// operands reach LDS without passing through registers.
+// barrier per step.  That is the kernel for Q8_0 tiles (gemm_big<1>, <2>); F16 tiles take gemm_big_f16 (the same block)
+// or gemm_big_f16_256 (a 256 x 256 block) below, whose operands reach LDS without passing through registers, and
+// launch_gemm_big chooses between the two block shapes, or gives each a part of the columns.
 #include "backend.h"
 #include "devutil.h"
 #include "gemm.h"
