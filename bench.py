@@ -280,7 +280,7 @@ def main():
                 "peak": MFMA_PEAK_TFS if compute_bound else HBM_PEAK_GBS,
                 "unit": "TFLOP/s" if compute_bound else "GB/s",
                 "frac": round(tfs / MFMA_PEAK_TFS if compute_bound else gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": ("gemm_big<1>, gemm_big<2>" if cfg.BN >= 1024 and cfg.weight_format != "f16" and args.q8_large_m == "unpack-in-lds" else
+                "kernel": ("gemm_big_q8<1>, gemm_big_q8<2>" if cfg.BN >= 1024 and cfg.weight_format != "f16" and args.q8_large_m == "unpack-in-lds" else
                            "gemm_big_f16_256, gemm_big_f16" if cfg.BN >= 1024 else
                            "gemm_tiled + gemm_big_f16_256, gemm_big_f16" if compute_bound else "gemm_tiled"),
                 "launches_per_step": n // prof_steps,

@@ -79,6 +79,8 @@ bool large_m_unpacks_q8();                                // the large-M policy 
 // chunks > 1 (F16 tiles only): the K steps are cut into that many chunks, chunk c writing the plane at C + c * plane_stride;
 // big_gemm_chunks: what the measured rule picks for a product
 int big_gemm_chunks(int M, int N, int K, int fmt);
+// the same for any operand: Q8_0 tiles that the 256 x 256 dequant-fused kernel can take are cut into chunks as well
+int big_gemm_chunks_for(int M, int N, int K, const WeightOp &W);
 void set_big_gemm_split(int mode);     // 1 measured rule, 0 never, n > 1 always n chunks
 void set_big_gemm_block(int mode);     // F16 tiles: 0 block shape by the measured rule, 1 always 128 x 256, 2 always 256 x 256
 // Returns the number of planes written (fewer than `chunks` when K has too few steps for that many).

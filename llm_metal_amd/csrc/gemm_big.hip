@@ -536,6 +536,219 @@ __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
         }
 }
 
+// The 256 x 256 block over Q8_0 weight tiles that stay quantised all the way into LDS: the dequant-fused product for
+// many activation rows.  A half step of a weight row block is ONE 1 KB piece (16 int8 per lane: both 8-value slices), its
+// 64 fp16 scales another 128 bytes, so a block's half step is 16 KB of activations + 8 KB of weights instead of 32 KB and
+// six buffers fit; the copies are LDS-direct loads as in gemm_big_f16_256 (the scales as one dword per lane, lanes 32-63
+// fetching the same 128 bytes again into the second half of a 256-byte slot, which keeps every lane active and inside
+// the array).  A wave unpacks its fragments on the way from LDS to the MFMA: bytes to exact fp16 integers with
+// v_perm_b32, times the scale with packed fp16 multiplies -- the values an F16 image of the dequantised weight holds.
+// WF 1: scales per (row, 32 columns), all row blocks of the launch Q8_0 (the caller gives F16 row blocks to another
+// launch).  WF 2: the transposed image, scales per (column, 32 rows); K steps from W.kbq on are F16 tiles (the adapter
+// rows of the fused QKV weight): at most a step or two at the end of K, multiplied straight from memory after the loop.
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+// BM: rows of the block.  The launcher uses 256 (four waves of 128 x 128); with 128 (four waves of 64 x 128) a wave unpacks
+// as many weight fragments for half as many MFMAs, and 192 such blocks took 68 us where the F16 kernel's take 45.
+// TAIL (WF 1): the launch has a column block of F16 tiles at its end (only then does the loop carry that case).
+template <int WF, int BM, bool TAIL = false>
+__global__ __launch_bounds__(256) void gemm_big_q8(GemmKArgs g)
+{
+    constexpr int AB = BM / 32, MI = BM / 64, AU = BM / 128;  // A row blocks per block; accumulator tile rows and A pieces per wave
+    constexpr int HB = (2 * AB + 8) * 64;                 // 16-byte units per buffer: A [AB blocks][2 slices][64], Wq [8 blocks][64]
+    __shared__ uint4v lb0[HB], lb1[HB], lb2[HB], lb3[HB], lb4[HB], lb5[HB];
+    __shared__ half_t scl[6][8][128];                      // scales of the weight row blocks of the half step in buffer i
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int MT = (g.M + BM - 1) / BM, NT = (g.N + 255) >> 8;
+    const int m_patches = (MT + 7) >> 3;
+    int mt, nt, chunk = 0;
+    if (g.S > 1) {
+        const int t = blockIdx.x % (MT * NT);
+        chunk = blockIdx.x / (MT * NT); mt = t % MT; nt = t / MT;
+    } else {
+        const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3, patch = seq >> 5, in_patch = seq & 31;
+        mt = (patch % m_patches) * 8 + (in_patch & 7);
+        nt = ((patch / m_patches) * 4 + (in_patch >> 3)) * 8 + xcd;
+        if (mt >= MT || nt >= NT) return;
+    }
+    const int nb0 = nt * 8, mb0 = mt * AB;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int k_beg = chunk * g.steps_per_chunk, k_end = min(g.Kb, k_beg + g.steps_per_chunk);
+    const int kq_end = WF == 2 ? min(k_end, g.W.kbq) : k_end;              // Q8_0 steps of this chunk: [k_beg, kq_end)
+    const int nsteps = kq_end - k_beg, nhalf = 2 * nsteps, last = nhalf - 1;
+    const int kstride = WF == 2 ? g.W.kbq : g.Kb;                           // K blocks per row block of the Q8_0 tile arrays
+    // A column block from row block W.nbq on holds F16 tiles (WF 1: the adapter rows at the end of the fused QKV weight;
+    // W.nbq is a multiple of 8 and at most one row block follows it, the rest of the block lies outside the matrix): its
+    // one row block travels as two 1 KB slices per half step in the places of a piece and a scale copy.
+    const bool f16_cols = TAIL && WF == 1 && nb0 >= g.W.nbq;
+    // this wave's share of a half step: both slices of A row blocks w (, 4 + w); the piece and the scales of W row blocks w, 4 + w
+    const uint4v *asrc[AU], *qsrc[2];
+    const uint32_t *dsrc[2];
+#pragma unroll
+    for (int u = 0; u < AU; u++)
+        asrc[u] = reinterpret_cast<const uint4v *>(g.A) + ((size_t)min(mb0 + 4 * u + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const size_t tile0 = (size_t)min(nb0 + 4 * u + wave, (WF == 1 ? min(g.Nb, g.W.nbq) : g.Nb) - 1) * kstride + k_beg;
+        qsrc[u] = reinterpret_cast<const uint4v *>(g.W.q) + tile0 * 128 + lane;
+        dsrc[u] = reinterpret_cast<const uint32_t *>(g.W.d + tile0 * 64) + (lane & 31);
+    }
+    const uint4v *fsrc = f16_cols ? reinterpret_cast<const uint4v *>(g.W.w16) + ((size_t)min(nb0 - g.W.nbq, g.Nb - g.W.nbq - 1) * g.Kb + k_beg) * 256 + lane : nullptr;
+    float *const Cp = g.P + (size_t)chunk * g.plane_stride;
+
+    float16v acc[MI][4];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    typedef __attribute__((address_space(3))) void lds_void;
+    uint32_t aoff[AU][2], qoff[2], doff[2];                // byte offsets of this wave's pieces inside a buffer / a scale slot
+#pragma unroll
+    for (int u = 0; u < AU; u++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) aoff[u][j] = __builtin_amdgcn_readfirstlane((uint32_t)((((4 * u + wave) * 2 + j) * 64) * 16));
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        qoff[u] = __builtin_amdgcn_readfirstlane((uint32_t)((2 * AB * 64 + (4 * u + wave) * 64) * 16));
+        doff[u] = __builtin_amdgcn_readfirstlane((uint32_t)((4 * u + wave) * 256));
+    }
+    const uint32_t scl0 = (uint32_t)(uintptr_t)(lds_void *)&scl[0][0][0];
+    auto request = [&](uint4v (&buf)[HB], int slot, int hs) __attribute__((always_inline)) {
+        const int kt = hs >> 1, jh = hs & 1;
+        const uint32_t base = (uint32_t)(uintptr_t)(lds_void *)buf, sbase = scl0 + (uint32_t)slot * (8 * 256);
+#pragma unroll
+        for (int u = 0; u < AU; u++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(asrc[u] + (size_t)kt * 256 + (2 * jh + j) * 64), "s"(base + aoff[u][j]) : "m0");
+        if (f16_cols) {                                    // the same four copies: slice j of the F16 row block into W place w (j = 0) / 4 + w (j = 1)
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(fsrc + (size_t)kt * 256 + (2 * jh + j) * 64), "s"(base + qoff[j]) : "m0");
+        } else {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(qsrc[u] + (size_t)kt * 128 + jh * 64), "s"(base + qoff[u]) : "m0");
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" :: "v"(dsrc[u] + (size_t)kt * 32), "s"(sbase + doff[u]) : "m0");
+            }
+        }
+    };
+    half8 a0[MI], w0[4];                                   // fragments of slice 0 of the half step about to be multiplied
+    // slice j (0 / 1) of the half step in `cur` / scale slot `slot`: A as it lies, W unpacked
+    auto read = [&](half8 (&a)[MI], half8 (&w)[4], const uint4v (&cur)[HB], int slot, int jh, int j) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < MI; i++) a[i] = __builtin_bit_cast(half8, cur[((MI * wm + i) * 2 + j) * 64 + lane]);
+        if (f16_cols) {                                    // (wave 0's copies; every fragment of the block is that one row block)
+#pragma unroll
+            for (int k = 0; k < 4; k++) w[k] = __builtin_bit_cast(half8, cur[2 * AB * 64 + (j ? 4 : 0) * 64 + lane]);
+            return;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int blk = 4 * wn + k;
+            const uint2v q = reinterpret_cast<const uint2v *>(&cur[2 * AB * 64 + blk * 64 + lane])[j];
+            half8 sc;
+            if (WF == 1) sc = bcast8(scl[slot][blk][lane]);
+            else sc = reinterpret_cast<const half8 *>(&scl[slot][blk][0])[h * 4 + 2 * jh + j];
+            w[k] = q8_unpack8(q[0], q[1]) * sc;
+        }
+    };
+    auto multiply = [&](const half8 (&a)[MI], const half8 (&w)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) acc[i][k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[k], acc[i][k], 0, 0, 0);
+    };
+    // Half step hs is multiplied out of buffer hs % 6 (see gemm_big_f16_256): the barrier that ends half step hs - 1 has
+    // found hs and hs + 1 in LDS, slice 0 of hs + 1 is read and unpacked while slice 1 of hs is multiplied, hs + 5 is
+    // requested into the buffer hs - 1 left.  Eight copies per wave and half step.
+    auto step = [&](int hs, const uint4v (&cur)[HB], int slot, const uint4v (&nxt)[HB], int nslot, uint4v (&free_buf)[HB], int fslot)
+        __attribute__((always_inline)) {
+        request(free_buf, fslot, min(hs + 5, last));
+        half8 a1[MI], w1[4];
+        read(a1, w1, cur, slot, hs & 1, 1);
+        multiply(a0, w0);
+        read(a0, w0, nxt, nslot, (hs + 1) & 1, 0);
+        multiply(a1, w1);
+        if (BM == 256) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+    if (nhalf > 0) {
+        request(lb0, 0, 0); request(lb1, 1, min(1, last)); request(lb2, 2, min(2, last)); request(lb3, 3, min(3, last));
+        request(lb4, 4, min(4, last));
+        if (BM == 256) asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+        read(a0, w0, lb0, 0, 0, 0);
+        const int full = nhalf / 6 * 6;
+        for (int h0 = 0; h0 < full; h0 += 6) {
+            step(h0, lb0, 0, lb1, 1, lb5, 5);
+            step(h0 + 1, lb1, 1, lb2, 2, lb0, 0);
+            step(h0 + 2, lb2, 2, lb3, 3, lb1, 1);
+            step(h0 + 3, lb3, 3, lb4, 4, lb2, 2);
+            step(h0 + 4, lb4, 4, lb5, 5, lb3, 3);
+            step(h0 + 5, lb5, 5, lb0, 0, lb4, 4);
+        }
+        if (full < nhalf) step(full, lb0, 0, lb1, 1, lb5, 5);
+        if (full + 1 < nhalf) step(full + 1, lb1, 1, lb2, 2, lb0, 0);
+        if (full + 2 < nhalf) step(full + 2, lb2, 2, lb3, 3, lb1, 1);
+        if (full + 3 < nhalf) step(full + 3, lb3, 3, lb4, 4, lb2, 2);
+        if (full + 4 < nhalf) step(full + 4, lb4, 4, lb5, 5, lb3, 3);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    if (WF == 2) {
+        // the F16 K steps at the end of this chunk (adapter rows): operands straight from memory
+        for (int kt = max(kq_end, k_beg); kt < k_end; kt++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                half8 a[MI], w[4];
+#pragma unroll
+                for (int i = 0; i < MI; i++) a[i] = g.A[((size_t)min(mb0 + MI * wm + i, g.Mb - 1) * g.Kb + kt) * 256 + j * 64 + lane];
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    w[k] = reinterpret_cast<const half8 *>(g.W.w16)[((size_t)min(nb0 + 4 * wn + k, g.Nb - 1) * (g.Kb - g.W.kbq) + kt - g.W.kbq) * 256 + j * 64 + lane];
+                multiply(a, w);
+            }
+        }
+    }
+
+    if (mb0 * 32 + BM <= g.M && (nb0 + 8) * 32 <= g.N) {   // a block inside the matrix: stores without tests, factors first
+        float sc[MI][16];
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                sc[i][v] = g.a_inv_scale ? g.a_inv_scale[(mb0 + MI * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3)] : 1.0f;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = (mb0 + MI * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+                float *row = Cp + (size_t)m * g.ldp + (nb0 + 4 * wn) * 32 + r;
+#pragma unroll
+                for (int k = 0; k < 4; k++) row[k * 32] = acc[i][k][v] * sc[i][v];
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = (mb0 + MI * wm + i) * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (m >= g.M) continue;
+            const float sc = g.a_inv_scale ? g.a_inv_scale[m] : 1.0f;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int n = (nb0 + 4 * wn + k) * 32 + r;
+                if (n < g.N) Cp[(size_t)m * g.ldp + n] = acc[i][k][v] * sc;
+            }
+        }
+}
+
 }  // namespace
 
 // How many K chunks the large-M kernel should cut a product with F16 tiles into: three when its 128 x 256 output blocks
@@ -556,6 +769,33 @@ int big_gemm_chunks(int M, int N, int K, int fmt)
     return (blocks * 3 <= cus * 2 && K >= 4096) ? 3 : 1;
 }
 
+// Whether a Q8_0 operand can run on gemm_big_q8: the row blocks of a row-scaled operand all quantised, or one F16 row
+// block (the adapter rows of the fused QKV weight) that begins a column block of its own; at most two F16 K steps at the
+// end of a column-scaled one.
+bool q8_wide_ok(const WeightOp &W, int N, int K)
+{
+    if (g_big_block == 1) return false;
+    if (W.fmt == 1) return W.nbq >= tiled_rb(N) || (W.nbq % 8 == 0 && tiled_rb(N) - W.nbq == 1 && W.w16);
+    if (W.fmt == 2) return W.kbq >= 1 && tiled_kb(K) - W.kbq <= 2;
+    return false;
+}
+
+// K chunks for any operand: big_gemm_chunks for F16 tiles; for Q8_0 tiles on the 256 x 256 block, two or three chunks
+// where they fill at least half as many CUs again as one does (each chunk 20 K steps or more), else one.
+int big_gemm_chunks_for(int M, int N, int K, const WeightOp &W)
+{
+    if (W.fmt == 0) return big_gemm_chunks(M, N, K, 0);
+    if (g_big_split == 0 || !q8_wide_ok(W, N, K)) return 1;
+    if (g_big_split > 1) return g_big_split;
+    const int cus = num_cus() > 0 ? num_cus() : 256;
+    const long blocks = (long)((M + 255) / 256) * ((N + 255) / 256);
+    auto share = [&](int c) { return (double)(blocks * c) / (double)((blocks * c + cus - 1) / cus * cus); };
+    int best = 1;
+    for (int c = 2; c <= 3; c++)
+        if (tiled_kb(K) / c >= 20 && share(c) >= 1.5 * share(1) && share(c) > share(best)) best = c;
+    return best;
+}
+
 int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W, float *C, int ldc, int M, int N, int K,
                     int chunks, size_t plane_stride)
 {
@@ -568,7 +808,8 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
     if (!ok) { fprintf(stderr, "[fast_hip] gemm_big: bad launch M=%d N=%d K=%d ldc=%d fmt=%d\n", M, N, K, ldc, W.fmt); abort(); }
     GemmKArgs g{};
     g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
-    if (chunks < 1 || (chunks > 1 && W.fmt != 0)) { fprintf(stderr, "[fast_hip] gemm_big: K chunks need F16 tiles\n"); abort(); }
+    const bool q8_wide = W.fmt != 0 && q8_wide_ok(W, N, K);
+    if (chunks < 1 || (chunks > 1 && W.fmt != 0 && !q8_wide)) { fprintf(stderr, "[fast_hip] gemm_big: K chunks need F16 tiles or the 256 x 256 Q8_0 kernel\n"); abort(); }
     g.P = C; g.ldp = ldc; g.plane_stride = plane_stride;
     g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb;
     g.steps_per_chunk = (Kb + chunks - 1) / chunks;
@@ -580,9 +821,9 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
     // the kernels), the ids past the matrix returning at once
     auto grid_of = [&](const GemmKArgs &a, int bm, int bn) {
         const int mt = (a.M + bm - 1) / bm, nt = (a.N + bn - 1) / bn;
-        return dim3(W.fmt == 0 && a.S > 1 ? mt * nt * a.S : 8 * 32 * ((mt + 7) / 8) * (((nt + 7) / 8 + 3) / 4));
+        return dim3(a.S > 1 ? mt * nt * a.S : 8 * 32 * ((mt + 7) / 8) * (((nt + 7) / 8 + 3) / 4));
     };
-    if (W.fmt == 0) {
+    if (W.fmt == 0 || q8_wide) {
         // 128 x 256 or 256 x 256 blocks, whichever keeps more of the GPU on useful work -- the share of the last round's
         // CUs that have a block times the share of the tiles' area that lies inside the matrix.  The wide block is faster
         // in its loop and wins from 0.9 of the other's share, given 20 K steps per block to win them in (below, its larger
@@ -594,24 +835,28 @@ int launch_gemm_big(const half_t *A, const float *a_inv_scale, const WeightOp &W
             return (double)M * N / ((double)tm * bm * tn * bn) * (double)blocks / (double)((blocks + cus - 1) / cus * cus);
         };
         const bool deep = g.steps_per_chunk >= 20;
-        const bool wide = g_big_block == 2 || (g_big_block == 0 && deep && share(256, 256) >= 0.9 * share(128, 128 * WPW));
-        // A product of at least two full rounds of wide blocks whose last round would be half empty or less: the columns
+        // (Q8_0 tiles: the wide block only, see gemm_big_q8)
+        const bool wide = W.fmt != 0 || g_big_block == 2 || (g_big_block == 0 && deep && share(256, 256) >= 0.9 * share(128, 128 * WPW));
+        // A product of at least one full round of wide blocks whose last round would be half empty or less: the columns
         // of the full rounds go to wide blocks, the rest to 128 x 256 blocks in a launch of their own
         const int MX = (M + 255) / 256, NX = (N + 255) / 256, full = MX * NX / cus, rest = MX * NX % cus;
         const int wide_cols = full * cus / MX * 256;
         auto launch = [&](const GemmKArgs &a, bool w, hipEvent_t e0, hipEvent_t e1) {
             const dim3 grid = w ? grid_of(a, 256, 256) : grid_of(a, 128, 128 * WPW);
-            if (prof && w) hipExtLaunchKernelGGL(gemm_big_f16_256, grid, block, 0, stream(), e0, e1, 0, a);
-            else if (prof) hipExtLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), e0, e1, 0, a);
-            else if (w) hipLaunchKernelGGL(gemm_big_f16_256, grid, block, 0, stream(), a);
-            else hipLaunchKernelGGL(gemm_big_f16, grid, block, 0, stream(), a);
+#define BIG_LAUNCH(KERNEL) do { if (prof) hipExtLaunchKernelGGL((KERNEL), grid, block, 0, stream(), e0, e1, 0, a); \
+                                else hipLaunchKernelGGL((KERNEL), grid, block, 0, stream(), a); } while (0)
+            if (W.fmt == 0) { if (w) BIG_LAUNCH(gemm_big_f16_256); else BIG_LAUNCH(gemm_big_f16); }
+            else if (W.fmt == 1) { if (a.W.nbq < a.Nb) BIG_LAUNCH((gemm_big_q8<1, 256, true>)); else BIG_LAUNCH((gemm_big_q8<1, 256>)); }
+            else BIG_LAUNCH((gemm_big_q8<2, 256>));
+#undef BIG_LAUNCH
         };
         if (g_big_block == 0 && !wide && deep && g.S == 1 && full >= 1 && rest > 0 && rest * 2 <= cus && wide_cols < N) {
             GemmKArgs g1 = g, g2 = g;
-            g1.N = wide_cols; g1.Nb = wide_cols / 32;
+            const int rb = wide_cols / 32;                 // weight row blocks that go to the wide launch
+            g1.N = wide_cols; g1.Nb = rb;
             g2.N = N - wide_cols; g2.Nb = tiled_rb(g2.N);
-            g2.W.w16 = W.w16 + (size_t)(wide_cols / 32) * Kb * 2048;
             g2.P = C + wide_cols;
+            g2.W.w16 = W.w16 + (size_t)rb * Kb * 2048;    // (F16 tiles: Q8_0 products are all wide)
             launch(g1, true, ev_a, nullptr);
             launch(g2, false, nullptr, ev_b);
         } else launch(g, wide, ev_a, ev_b);

@@ -280,7 +280,7 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
     if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch; final output, or a few K chunks as planes
         float *C = out ? out : at<float>(s->planes);
         const WeightOp Wf = resident_image(s, W, N, K);
-        const int chunks = out ? 1 : big_gemm_chunks(s->BN, N, K, Wf.fmt);
+        const int chunks = out ? 1 : big_gemm_chunks_for(s->BN, N, K, Wf);
         const size_t stride = (size_t)s->BN * N;
         if (!out && chunks * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
         const int planes = launch_gemm_big(A, inv, Wf, C, N, s->BN, N, K, chunks, stride);

@@ -51,6 +51,10 @@ CASES = [
     C1.with_(name="big_m_f16_wide_chunks", batch=5, seq=40),             # ragged in rows (200) and three K chunks
     C1.with_(name="big_m_q8_wide", NL=1, batch=2, seq=160, weight_format="q8_0"),   # over the kept F16 images, 320 rows
     TINY_GEMMA3.with_(name="gemma_big_m_q8_wide", NL=2, batch=3, seq=100, weight_format="q8_0"),
+    # Q8_0 tiles quantised all the way into LDS, unpacked by the 256 x 256 kernel itself; also in three K chunks
+    C1.with_(name="big_m_q8_wide_lds", NL=1, batch=2, seq=160, weight_format="q8_0"),
+    C1.with_(name="big_m_q8_wide_lds_chunks", NL=1, batch=2, seq=160, weight_format="q8_0"),
+    TINY_GEMMA3.with_(name="gemma_big_m_q8_wide_lds", NL=2, batch=3, seq=100, weight_format="q8_0"),
     C1.with_(name="big_m_q8", NL=1, batch=2, seq=160, weight_format="q8_0"),
     TINY_GEMMA3.with_(name="gemma_big_m_q8", NL=2, batch=3, seq=100, weight_format="q8_0"),
     C1.with_(name="big_m_q8_noimg", NL=1, batch=2, seq=160, weight_format="q8_0"),      # no room to keep the images: made per product
@@ -109,7 +113,7 @@ def test_train_steps_match_oracle(cfg):
     from llm_metal_amd import lib
     # the "big_m" cases pin every product to the LDS-tiled large-M kernel (by itself it is only chosen for
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
-    lib.load().hip_gemm_force_large_m(2 if cfg.name.endswith("_lds") else 1 if "big_m" in cfg.name else 0)
+    lib.load().hip_gemm_force_large_m(2 if "_lds" in cfg.name else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
     lib.load().hip_gemm_large_m_block(2 if "_wide" in cfg.name else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_attention_flash(1 if cfg.name.endswith("_flash") else 0 if cfg.name.endswith("_noflash") else -1)
