@@ -1022,15 +1022,18 @@ __global__ __launch_bounds__(256) void k_ce_partial(CeArgs a)
     int c_beg, c_end;
     ce_chunk_range(V, chunk, c_beg, c_end);
     const int e_beg = min(c_beg * 8, V), e_end = min(c_end * 8, V);     // V % 4 == 0 is checked by the launcher
-    float mx = -1e30f;
-    for (int i = e_beg + 4 * threadIdx.x; i < e_end; i += 4 * 256) { const float4 x = ld4(lg + i); mx = fmaxf(mx, fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w))); }
-    mx = block_max(mx, sm);
-    float sum = 0.f;
+    // one pass over the piece: every thread keeps a running maximum and the sum of exponentials relative to it, rescaled
+    // when the maximum moves; the threads' pairs are then brought to the piece's maximum
+    float tm = -1e30f, ts = 0.f;
+#pragma unroll 4
     for (int i = e_beg + 4 * threadIdx.x; i < e_end; i += 4 * 256) {
         const float4 x = ld4(lg + i);
-        sum += expf(x.x - mx) + expf(x.y - mx) + expf(x.z - mx) + expf(x.w - mx);
+        const float m4 = fmaxf(fmaxf(x.x, x.y), fmaxf(x.z, x.w));
+        if (m4 > tm) { ts *= expf(tm - m4); tm = m4; }
+        ts += expf(x.x - tm) + expf(x.y - tm) + expf(x.z - tm) + expf(x.w - tm);
     }
-    sum = block_sum(sum, sm);
+    const float mx = block_max(tm, sm);
+    const float sum = block_sum(ts * expf(tm - mx), sm);   // a thread without elements: 0 * exp(-1e30 - mx) = 0
     if (threadIdx.x == 0) a.partials[r * CE_CHUNKS + chunk] = make_float2(mx, sum);
 }
 
@@ -1068,18 +1071,100 @@ __global__ __launch_bounds__(256) void k_ce_rows(CeArgs a)
     int c_beg, c_end;
     ce_chunk_range(V, chunk, c_beg, c_end);
     const int Kb = tiled_kb(V);
-    for (int c = c_beg + threadIdx.x; c < c_end; c += 256) {
-        half8 hv;
-        // V % 4 == 0 (checked by the launcher): the eight logits are two aligned 16-byte loads, each inside the row or not
-        const float4 lo4 = c * 8 < V ? ld4(lg + c * 8) : make_float4(0.f, 0.f, 0.f, 0.f);
-        const float4 hi4 = c * 8 + 4 < V ? ld4(lg + c * 8 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-        const float x[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+    // four groups of eight logits per thread and trip, all eight loads issued before the first exponential
+    constexpr int U = 4;
+    for (int cb = c_beg + threadIdx.x; cb < c_end; cb += 256 * U) {
+        float4 lo4[U], hi4[U];
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const int i = c * 8 + e;
-            hv[e] = (i < V) ? f2h((expf(x[e] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
+        for (int u = 0; u < U; u++) {
+            const int c = cb + 256 * u;
+            // V % 4 == 0 (checked by the launcher): the eight logits are two aligned 16-byte loads, each inside the row or not
+            lo4[u] = (c < c_end && c * 8 < V) ? ld4(lg + c * 8) : make_float4(0.f, 0.f, 0.f, 0.f);
+            hi4[u] = (c < c_end && c * 8 + 4 < V) ? ld4(lg + c * 8 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = cb + 256 * u;
+            if (c >= c_end) break;
+            const float x[8] = {lo4[u].x, lo4[u].y, lo4[u].z, lo4[u].w, hi4[u].x, hi4[u].y, hi4[u].z, hi4[u].w};
+            half8 hv;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int i = c * 8 + e;
+                hv[e] = (i < V) ? f2h((expf(x[e] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
+            }
+            *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
+        }
+    }
+}
+
+// The second launch for many rows: a workgroup takes eight consecutive rows of one piece, thread t row t & 7, so that the
+// eight 16-byte groups that share a 128-byte line of the tiled gradient (the same columns of eight rows) are written by
+// eight neighbouring lanes as one line; a row is still read in runs of 256 bytes (eight groups) per wave.
+__global__ __launch_bounds__(256) void k_ce_rows8(CeArgs a, int rows)
+{
+    __shared__ float s_lse[8];
+    __shared__ uint32_t s_tgt[8];
+    const int chunk = blockIdx.x, V = a.V, sub = threadIdx.x & 7;
+    const size_t r = (size_t)blockIdx.y * 8 + sub;
+    if (threadIdx.x < 8 && r < (size_t)rows) {
+        const float *lg = a.logits + r * V;
+        const uint32_t tgt = a.targets[r];
+        float mx = -1e30f;
+        float2 part[CE_CHUNKS];
+#pragma unroll
+        for (int c = 0; c < CE_CHUNKS; c++) { part[c] = a.partials[r * CE_CHUNKS + c]; mx = fmaxf(mx, part[c].x); }
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < CE_CHUNKS; c++) sum += part[c].y * expf(part[c].x - mx);
+        const float lse = logf(sum) + mx;
+        s_lse[sub] = lse; s_tgt[sub] = tgt;
+        if (chunk == 0) {                                  // as in k_ce_rows
+            float coef = 1.0f / (float)a.rows_total;
+            if (a.grpo) {
+                const float new_lp = lg[tgt] - lse;
+                const float ratio = expf(new_lp - a.old_lp[r]);
+                const float clipped = fminf(fmaxf(ratio, 1.0f - a.clip_eps), 1.0f + a.clip_eps);
+                const float adv = a.advs[r];
+                const float w = (adv >= 0.f) ? ((ratio <= clipped) ? -adv : 0.f) : ((ratio >= clipped) ? -adv : 0.f);
+                coef = w * ratio * a.dl_scale;
+                a.new_lp[r] = new_lp;
+            } else {
+                a.losses[r] = lse - lg[tgt];
+            }
+            a.inv_scale[r] = coef * (1.0f / 1024.0f);
+        }
+    }
+    __syncthreads();
+    if (r >= (size_t)rows) return;
+    const float lse = s_lse[sub];
+    const uint32_t tgt = s_tgt[sub];
+    const float *lg = a.logits + r * V;
+    int c_beg, c_end;
+    ce_chunk_range(V, chunk, c_beg, c_end);
+    const int Kb = tiled_kb(V);
+    constexpr int U = 4;
+    for (int cb = c_beg + (threadIdx.x >> 3); cb < c_end; cb += 32 * U) {
+        float4 lo4[U], hi4[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = cb + 32 * u;
+            lo4[u] = (c < c_end && c * 8 < V) ? ld4(lg + c * 8) : make_float4(0.f, 0.f, 0.f, 0.f);
+            hi4[u] = (c < c_end && c * 8 + 4 < V) ? ld4(lg + c * 8 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = cb + 32 * u;
+            if (c >= c_end) break;
+            const float x[8] = {lo4[u].x, lo4[u].y, lo4[u].z, lo4[u].w, hi4[u].x, hi4[u].y, hi4[u].z, hi4[u].w};
+            half8 hv;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int i = c * 8 + e;
+                hv[e] = (i < V) ? f2h((expf(x[e] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
+            }
+            *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
+        }
     }
 }
 
@@ -1299,7 +1384,8 @@ void launch_ce_rows(const CeArgs &a, int rows)
     require(a.V % 4 == 0, "ce_rows: vocabulary size must be a multiple of 4");
     require(a.partials != nullptr, "ce_rows: partials scratch missing");
     LAUNCH(k_ce_partial, dim3(CE_CHUNKS, rows), dim3(256), 0, a);
-    LAUNCH(k_ce_rows, dim3(CE_CHUNKS, rows), dim3(256), 0, a);
+    if (rows >= MANY_ROWS) LAUNCH(k_ce_rows8, dim3(CE_CHUNKS, (rows + 7) / 8), dim3(256), 0, a, rows);
+    else LAUNCH(k_ce_rows, dim3(CE_CHUNKS, rows), dim3(256), 0, a);
 }
 
 void launch_adamw(const AdamArgs &a)
