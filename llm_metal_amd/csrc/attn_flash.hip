@@ -499,13 +499,13 @@ __global__ __launch_bounds__(256) void k_fa_fwd(FaArgs a)
                 const float4 v4 = make_float4(o[db][4 * g] * inv, o[db][4 * g + 1] * inv, o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
                 st4(a.O + row * qd + d, v4);
                 half4 h4 = {f2h(v4.x), f2h(v4.y), f2h(v4.z), f2h(v4.w)};
-                *reinterpret_cast<half4 *>(a.out16 + tiled_index((int)row, d, Kb)) = h4;
+                *reinterpret_cast<half4 *>(a.out16 + tiled_a_index((int)row, d, Kb)) = h4;
             }
     }
     if (h == a.Hq - 1 && Kb * 64 > qd)                      // zero the K padding of the operand rows once
         for (int idx = lane; idx < 32 * (Kb * 64 - qd); idx += 64) {
             const int rr = idx / (Kb * 64 - qd), c = qd + idx % (Kb * 64 - qd);
-            if (32 * qb + rr < N) a.out16[tiled_index((int)((size_t)b * N + 32 * qb + rr), c, Kb)] = (half_t)0;
+            if (32 * qb + rr < N) a.out16[tiled_a_index((int)((size_t)b * N + 32 * qb + rr), c, Kb)] = (half_t)0;
         }
 }
 

@@ -398,13 +398,13 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
             const int i = i0 + 8 * (v >> 2) + 4 * hh + (v & 3);
             if (i >= N) continue;
             if (BWD) a.out32[(r0 + i) * qd + h * HD + d] = acc[v];
-            else a.out16[tiled_index((int)(r0 + i), h * HD + d, Kb)] = f2h(acc[v]);
+            else a.out16[tiled_a_index((int)(r0 + i), h * HD + d, Kb)] = f2h(acc[v]);
         }
     }
     if (!BWD && h == a.Hq - 1)                             // zero the K padding of the operand rows once
         for (int idx = tid; idx < 32 * (Kb * 64 - qd); idx += 256) {
             const int rr = idx / (Kb * 64 - qd), c = qd + idx % (Kb * 64 - qd);
-            if (i0 + rr < N) a.out16[tiled_index((int)(r0 + i0 + rr), c, Kb)] = (half_t)0;
+            if (i0 + rr < N) a.out16[tiled_a_index((int)(r0 + i0 + rr), c, Kb)] = (half_t)0;
         }
 }
 

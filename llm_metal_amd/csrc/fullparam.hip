@@ -56,7 +56,7 @@ __device__ __forceinline__ void transpose_scaled_block(const half8 *__restrict__
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int tb = tb0 + u, token = tb * 32 + (lp & 31);
-                hb[u] = in[((size_t)min(tb, TbIn - 1) * KbIn + fb) * 256 + tid];
+                hb[u] = in[((size_t)min(tb, TbIn - 1) * KbIn + fb) * 256 + (tid & ~63) + a_lane(tid & 63)];
                 sb[u] = in_inv[min(token, T - 1)];
                 if (token >= T) sb[u] = 0.f;
             }
@@ -83,7 +83,7 @@ __device__ __forceinline__ void transpose_scaled_block(const half8 *__restrict__
 #pragma unroll
         for (int th = 0; th < 2; th++) {
             const int tile = tb2 * 2 + th, token = tb2 * 64 + th * 32 + (lp & 31);
-            h[th] = in[((size_t)min(tile, TbIn - 1) * KbIn + fb) * 256 + tid];
+            h[th] = in[((size_t)min(tile, TbIn - 1) * KbIn + fb) * 256 + (tid & ~63) + a_lane(tid & 63)];
             sc[th] = in_inv[min(token, T - 1)];
             if (tile >= TbIn || token >= T) { sc[th] = 0.f; h[th] = half8{0, 0, 0, 0, 0, 0, 0, 0}; }
         }

@@ -25,13 +25,13 @@ constexpr int MAXV_ROW = MAXV;                            // (the name the row k
 __device__ __forceinline__ void st_tiled4(half_t *out, size_t row, int k, int Kb, float4 v, float s)
 {
     half4 h = {f2h(v.x * s), f2h(v.y * s), f2h(v.z * s), f2h(v.w * s)};
-    *reinterpret_cast<half4 *>(out + tiled_index((int)row, k, Kb)) = h;
+    *reinterpret_cast<half4 *>(out + tiled_a_index((int)row, k, Kb)) = h;
 }
 
 // zero the K padding [n, Kb*64) of a tiled row
 __device__ __forceinline__ void zero_tiled_pad(half_t *out, size_t row, int n, int Kb)
 {
-    for (int i = n + threadIdx.x; i < Kb * 64; i += blockDim.x) out[tiled_index((int)row, i, Kb)] = (half_t)0;
+    for (int i = n + threadIdx.x; i < Kb * 64; i += blockDim.x) out[tiled_a_index((int)row, i, Kb)] = (half_t)0;
 }
 
 // Row `row` of a tiled fp16 operand [*, n] from fp32 values in LDS, scaled by s.
@@ -42,7 +42,7 @@ __device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t
         half8 hv;
 #pragma unroll
         for (int e = 0; e < 8; e++) { const int i = c * 8 + e; hv[e] = (i < n) ? f2h(vals[i] * s) : (half_t)0; }
-        *reinterpret_cast<half8 *>(out + tiled_index((int)row, c * 8, Kb)) = hv;
+        *reinterpret_cast<half8 *>(out + tiled_a_index((int)row, c * 8, Kb)) = hv;
     }
 }
 
@@ -320,10 +320,10 @@ __global__ __launch_bounds__(64) void k_attn_fwd(AttnFwdArgs a)
         float acc = 0.f;
 #pragma unroll 8
         for (int j = lo; j <= i; j++) acc += sc[j] * a.v[(r0 + j) * kd + hk * hd + d];
-        a.out16[tiled_index((int)(r0 + i), h * hd + d, Kb)] = f2h(acc);
+        a.out16[tiled_a_index((int)(r0 + i), h * hd + d, Kb)] = f2h(acc);
     }
     if (h == a.Hq - 1)                                    // zero the K padding of this row once
-        for (int c = qd + lane; c < Kb * 64; c += 64) a.out16[tiled_index((int)(r0 + i), c, Kb)] = (half_t)0;
+        for (int c = qd + lane; c < Kb * 64; c += 64) a.out16[tiled_a_index((int)(r0 + i), c, Kb)] = (half_t)0;
 }
 
 // attn_bwd_dq, shaders/q8_kernels.metal:857-925.  Also leaves the plane-summed dO
@@ -613,7 +613,7 @@ __global__ __launch_bounds__(TB) void k_lora_grads(LoraGradArgs a)
             const int Kb = tiled_kb(a.D);
 #pragma unroll 8
             for (int i = 0; i < a.rows; i++)
-                s += a.dh[(size_t)i * 2 * a.R + hc] * (h2f(a.ln16[tiled_index(i, d, Kb)]) * a.ln_inv_scale[i]);
+                s += a.dh[(size_t)i * 2 * a.R + hc] * (h2f(a.ln16[tiled_a_index(i, d, Kb)]) * a.ln_inv_scale[i]);
         } else {
             const int c = (int)(o / a.R), r = (int)(o % a.R);
             const float *dy = which == 1 ? a.dq_f : a.dv_f;
@@ -691,7 +691,7 @@ __global__ __launch_bounds__(256) void k_lora_grads_rank(LoraGradArgs a)
             if (d < a.D) {
 #pragma unroll 4
                 for (int i = 0; i < nr; i++) {
-                    const float x = h2f(a.ln16[tiled_index(i0 + i, d, Kb)]) * a.ln_inv_scale[i0 + i];
+                    const float x = h2f(a.ln16[tiled_a_index(i0 + i, d, Kb)]) * a.ln_inv_scale[i0 + i];
 #pragma unroll
                     for (int r = 0; r < R; r++) { aq[r] += ts[i * 2 * R + r] * x; av[r] += ts[i * 2 * R + R + r] * x; }
                 }
@@ -1093,7 +1093,7 @@ __global__ __launch_bounds__(256) void k_ce_rows(CeArgs a)
                 const int i = c * 8 + e;
                 hv[e] = (i < V) ? f2h((expf(x[e] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
             }
-            *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
+            *reinterpret_cast<half8 *>(a.dl16 + tiled_a_index((int)r, c * 8, Kb)) = hv;
         }
     }
 }
@@ -1163,7 +1163,7 @@ __global__ __launch_bounds__(256) void k_ce_rows8(CeArgs a, int rows)
                 const int i = c * 8 + e;
                 hv[e] = (i < V) ? f2h((expf(x[e] - lse) - ((uint32_t)i == tgt ? 1.0f : 0.0f)) * 1024.0f) : (half_t)0;
             }
-            *reinterpret_cast<half8 *>(a.dl16 + tiled_index((int)r, c * 8, Kb)) = hv;
+            *reinterpret_cast<half8 *>(a.dl16 + tiled_a_index((int)r, c * 8, Kb)) = hv;
         }
     }
 }

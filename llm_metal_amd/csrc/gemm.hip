@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void rows_to_f16_scaled(
     amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
     for (int i = threadIdx.x; i < Kb * 64; i += blockDim.x)
-        out[lmhip::tiled_index(row, i, Kb)] = (i < K) ? f2h(x[i] * s) : (half_t)0;
+        out[lmhip::tiled_a_index(row, i, Kb)] = (i < K) ? f2h(x[i] * s) : (half_t)0;
     if (threadIdx.x == 0) inv_scale[row] = 1.0f / s;
 }
 
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void rows_to_f16_split(
     float lmax = 0.f;
     for (int i = threadIdx.x; i < Kb * 64; i += blockDim.x) {
         const half_t h = (i < K) ? f2h(x[i] * s) : (half_t)0;
-        out[lmhip::tiled_index(row, i, Kb)] = h;
+        out[lmhip::tiled_a_index(row, i, Kb)] = h;
         if (i < K) lmax = fmaxf(lmax, fabsf(x[i] - h2f(h) * inv));
     }
     lmax = block_max(lmax, sm);
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void rows_to_f16_split(
     for (int i = threadIdx.x; i < Kb * 64; i += blockDim.x) {
         half_t l = (half_t)0;
         if (i < K) { const half_t h = f2h(x[i] * s); l = f2h((x[i] - h2f(h) * inv) * s2); }
-        out[lmhip::tiled_index(M + row, i, Kb)] = l;
+        out[lmhip::tiled_a_index(M + row, i, Kb)] = l;
     }
     if (threadIdx.x == 0) { inv_scale[row] = inv; inv_scale[M + row] = 1.0f / s2; }
 }
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(1024) void rows_to_f16_split_vec(
             v[u][e] = v[u][e] - h2f(h[e]) * inv;                            // what the rounding lost, exact in fp32
             lmax = fmaxf(lmax, fabsf(v[u][e]));
         }
-        if (k0 < Kb * 64) *reinterpret_cast<half8 *>(out + lmhip::tiled_index(row, k0, Kb)) = h;
+        if (k0 < Kb * 64) *reinterpret_cast<half8 *>(out + lmhip::tiled_a_index(row, k0, Kb)) = h;
     }
     lmax = block_max(lmax, sm);
     const float s2 = row_scale_for(lmax);
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(1024) void rows_to_f16_split_vec(
         half8 l;
 #pragma unroll
         for (int e = 0; e < 8; e++) l[e] = f2h(v[u][e] * s2);
-        if (k0 < Kb * 64) *reinterpret_cast<half8 *>(out + lmhip::tiled_index(M + row, k0, Kb)) = l;
+        if (k0 < Kb * 64) *reinterpret_cast<half8 *>(out + lmhip::tiled_a_index(M + row, k0, Kb)) = l;
     }
     if (threadIdx.x == 0) { inv_scale[row] = inv; inv_scale[M + row] = 1.0f / s2; }
 }

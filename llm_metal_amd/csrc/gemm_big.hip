@@ -50,7 +50,7 @@ __device__ __forceinline__ int tile_kind(const GemmKArgs &g, int nb, int kt)
 template <int WF>
 __device__ __forceinline__ void fetch(Stage &s, const GemmKArgs &g, int mb, const int (&nb)[WPW], int kt, int lane)
 {
-    const half8 *ap = g.A + ((size_t)mb * g.Kb + kt) * 256 + lane;
+    const half8 *ap = g.A + ((size_t)mb * g.Kb + kt) * 256 + a_lane(lane);
 #pragma unroll
     for (int j = 0; j < 4; j++) s.a[j] = ap[j * 64];
 #pragma unroll
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
     const int k_beg = chunk * g.steps_per_chunk, nsteps = min(g.Kb, k_beg + g.steps_per_chunk) - k_beg;
     const int nhalf = 2 * nsteps, last = nhalf - 1;
     const half8 *src[3];
-    src[0] = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[0] = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + a_lane(lane);
     src[1] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + 2 * wave, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
     src[2] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + 2 * wave + 1, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
     const int dst[3] = {wave, 4 + 2 * wave, 5 + 2 * wave};
@@ -424,8 +424,8 @@ __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
     const int nhalf = 2 * nsteps, last = nhalf - 1;
     // this wave's share of a half step: both slices of A row blocks w, 4 + w and of W row blocks w, 4 + w
     const half8 *src[4];
-    src[0] = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
-    src[1] = g.A + ((size_t)min(mb0 + 4 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+    src[0] = g.A + ((size_t)min(mb0 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + a_lane(lane);
+    src[1] = g.A + ((size_t)min(mb0 + 4 + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + a_lane(lane);
     src[2] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + wave, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
     src[3] = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(nb0 + 4 + wave, g.Nb - 1) * g.Kb + k_beg) * 256 + lane;
     const int dst[4] = {wave, 4 + wave, 8 + wave, 12 + wave};
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256) void gemm_big_q8(GemmKArgs g)
     const uint32_t *dsrc[2];
 #pragma unroll
     for (int u = 0; u < AU; u++)
-        asrc[u] = reinterpret_cast<const uint4v *>(g.A) + ((size_t)min(mb0 + 4 * u + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + lane;
+        asrc[u] = reinterpret_cast<const uint4v *>(g.A) + ((size_t)min(mb0 + 4 * u + wave, g.Mb - 1) * g.Kb + k_beg) * 256 + a_lane(lane);
 #pragma unroll
     for (int u = 0; u < 2; u++) {
         const size_t tile0 = (size_t)min(nb0 + 4 * u + wave, (WF == 1 ? min(g.Nb, g.W.nbq) : g.Nb) - 1) * kstride + k_beg;
@@ -707,7 +707,7 @@ __global__ __launch_bounds__(256) void gemm_big_q8(GemmKArgs g)
             for (int j = 0; j < 4; j++) {
                 half8 a[MI], w[4];
 #pragma unroll
-                for (int i = 0; i < MI; i++) a[i] = g.A[((size_t)min(mb0 + MI * wm + i, g.Mb - 1) * g.Kb + kt) * 256 + j * 64 + lane];
+                for (int i = 0; i < MI; i++) a[i] = g.A[((size_t)min(mb0 + MI * wm + i, g.Mb - 1) * g.Kb + kt) * 256 + j * 64 + a_lane(lane)];
 #pragma unroll
                 for (int k = 0; k < 4; k++)
                     w[k] = reinterpret_cast<const half8 *>(g.W.w16)[((size_t)min(nb0 + 4 * wn + k, g.Nb - 1) * (g.Kb - g.W.kbq) + kt - g.W.kbq) * 256 + j * 64 + lane];

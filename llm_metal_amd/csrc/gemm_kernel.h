@@ -130,7 +130,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 #pragma unroll
     for (int b = 0; b < NB; b++) nbi[b] = min(nb0 + b, Nb - 1);
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++) ap[mb] = g.A + (size_t)min(mb0 + mb, g.Mb - 1) * Kb * 256 + lane;
+    for (int mb = 0; mb < 2; mb++) ap[mb] = g.A + (size_t)min(mb0 + mb, g.Mb - 1) * Kb * 256 + a_lane(lane);
     const bool q8_rows = WF == 1 && nb0 < g.W.nbq;
 
     float16v acc[2][NB];

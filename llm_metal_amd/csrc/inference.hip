@@ -219,7 +219,7 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
     for (int u = 0; u < EPT; u++) {
         const int i = threadIdx.x + 1024 * u;
         const half_t h = f2h(v[u] * s);
-        if (i < Kb * 64) a16[tiled_index(b, i, Kb)] = h;
+        if (i < Kb * 64) a16[tiled_a_index(b, i, Kb)] = h;
         v[u] = v[u] - h2f(h) * is;
         lmax = fmaxf(lmax, fabsf(v[u]));
     }
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
 #pragma unroll
     for (int u = 0; u < EPT; u++) {
         const int i = threadIdx.x + 1024 * u;
-        if (i < Kb * 64) a16[tiled_index(B + b, i, Kb)] = f2h(v[u] * s2);
+        if (i < Kb * 64) a16[tiled_a_index(B + b, i, Kb)] = f2h(v[u] * s2);
     }
     if (threadIdx.x == 0) { inv_out[b] = is; inv_out[B + b] = 1.0f / s2; }
 }
