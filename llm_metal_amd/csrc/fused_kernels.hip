@@ -1140,9 +1140,10 @@ __global__ __launch_bounds__(256) void k_ce_rows8(CeArgs a, int rows)
     const float lse = s_lse[sub];
     const uint32_t tgt = s_tgt[sub];
     const float *lg = a.logits + r * V;
-    int c_beg, c_end;
-    ce_chunk_range(V, chunk, c_beg, c_end);
-    const int Kb = tiled_kb(V);
+    // pieces of whole tiles (eight groups), not the first launch's pieces: a wave then writes both column halves of its
+    // rows, 256 contiguous bytes per slice of a tile
+    const int Kb = tiled_kb(V), tiles_per = (Kb + CE_CHUNKS - 1) / CE_CHUNKS;
+    const int c_beg = min(chunk * tiles_per, Kb) * 8, c_end = min((chunk + 1) * tiles_per, Kb) * 8;
     constexpr int U = 4;
     for (int cb = c_beg + (threadIdx.x >> 3); cb < c_end; cb += 32 * U) {
         float4 lo4[U], hi4[U];
