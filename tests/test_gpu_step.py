@@ -39,6 +39,9 @@ CASES = [
     # long sequences: 16 key blocks per query block (config 4's 512), and a ragged length beyond 256
     C1.with_(name="seq512", NL=1, seq=512, V=1024),
     C1.with_(name="seq300_hd128", NL=1, D=256, Hq=2, Hkv=1, hd=128, IS=512, V=1024, seq=300),
+    # many rows, ragged: 525 rows (not a multiple of the eight rows that a cross-entropy workgroup takes, nor of a tile)
+    # and a vocabulary that ends inside a tile; the row kernels' many-row variants
+    C1.with_(name="rows525_v1000", NL=1, batch=7, seq=75, V=1000),
     # every product through the LDS-tiled large-M GEMM: F16 tiles; Q8_0 operands dequantised once per product into an
     # F16 image (what the measured rule does from 1024 rows on); and, in the "_lds" cases, Q8_0 tiles kept quantised and
     # unpacked into LDS by the kernel itself, with row scales (forward image) and column scales (transposed image).
