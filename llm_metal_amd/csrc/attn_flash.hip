@@ -83,7 +83,8 @@ struct FaSplitArgs {
     const float *O; float *D;            // optional: D[batch][H][nblk * 32] = rowsum(X o O), O [rows][H * HD]
 };
 
-template <int HD>
+// NBP: planes fetched per batch of loads (1 when the product left a single plane: fewer registers, more workgroups per CU)
+template <int HD, int NBP>
 __global__ __launch_bounds__(256) void k_fa_split(FaSplitArgs a)
 {
     constexpr int LDS_LD = HD + 4, NJ = HD / 16, TILE = HD / 8 * 64, TPR = HD / 4;      // TPR: threads per row
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void k_fa_split(FaSplitArgs a)
         if (a.X) {
 #pragma unroll
             for (int u = 0; u < HD / 32; u++) xv[u] = ok[u] ? ld4(a.X + rows[u] * a.ldx + cols[u]) : make_float4(0.f, 0.f, 0.f, 0.f);
-        } else planes_at4_multi<HD / 32, (HD <= 128 ? 5 : 3)>(a.Xpl, rows, cols, ok, xv);
+        } else planes_at4_multi<HD / 32, NBP>(a.Xpl, rows, cols, ok, xv);
 #pragma unroll
         for (int u = 0; u < HD / 32; u++) {
             const int idx = tid + 256 * u, rr = idx / TPR, c4 = idx % TPR;
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(256) void k_fa_split(FaSplitArgs a)
 // positions of one head, which then leaves the workgroup as the RT and PT fragments directly: no fp32 copy of the
 // final q, k, v is written and read again.  grid (blocks of 32 positions, Hq + 2 Hkv, batch), block 256.
 // RK: the LoRA rank compiled in (16), or -1 for any rank up to 64 (0 included).
-template <int HD, int RK>
+template <int HD, int RK, int NBP>                           // NBP as in k_fa_split
 __global__ __launch_bounds__(256) void k_qkv_post_tile(QkvPostArgs a, uint4 *q_rt, uint4 *q_pt, uint4 *k_rt, uint4 *k_pt, uint4 *v_rt, uint4 *v_pt, int batch)
 {
     constexpr int LDS_LD = HD + 4, NJ = HD / 16, TILE = HD / 8 * 64, TPR = HD / 4, HALF = HD / 2;
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(256) void k_qkv_post_tile(QkvPostArgs a, uint4 *q_r
             const int idx = tid + 256 * u, rr = idx / TPR, c4 = idx % TPR;
             ok[u] = blk * 32 + rr < N; rows[u] = r0 + (ok[u] ? blk * 32 + rr : 0); cols[u] = col0 + 4 * c4;
         }
-        planes_at4_multi<HD / 32, (HD <= 128 ? 5 : 3)>(a.qkv, rows, cols, ok, xv);
+        planes_at4_multi<HD / 32, NBP>(a.qkv, rows, cols, ok, xv);
 #pragma unroll
         for (int u = 0; u < HD / 32; u++) { const int idx = tid + 256 * u; st4(Xs + (idx / TPR) * LDS_LD + 4 * (idx % TPR), xv[u]); }
         if (lora)
@@ -670,7 +671,12 @@ __global__ __launch_bounds__(256) void k_fa_sum_groups(const float4 *dkp, const 
 }
 
 template <int HD>
-void split_hd(const FaSplitArgs &a) { LAUNCH(k_fa_split<HD>, dim3((a.seq + 31) / 32, a.H, a.batch), dim3(256), 0, a); }
+void split_hd(const FaSplitArgs &a)
+{
+    const dim3 grid((a.seq + 31) / 32, a.H, a.batch);
+    if (a.X || a.Xpl.S <= 1) LAUNCH((k_fa_split<HD, 1>), grid, dim3(256), 0, a);
+    else LAUNCH((k_fa_split<HD, (HD <= 128 ? 5 : 3)>), grid, dim3(256), 0, a);
+}
 
 void split(const FaSplitArgs &a, int hd) { if (hd == 64) split_hd<64>(a); else split_hd<128>(a); }
 
@@ -709,8 +715,14 @@ template <int HD>
 void qkv_post_hd(const QkvPostArgs &a, const AttnFlashArgs &f)
 {
     const dim3 grid((f.seq + 31) / 32, a.Hq + 2 * a.Hkv, f.batch);
-    if (a.R == 16) LAUNCH((k_qkv_post_tile<HD, 16>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
-    else LAUNCH((k_qkv_post_tile<HD, -1>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+    constexpr int NBM = HD <= 128 ? 5 : 3;
+    if (a.qkv.S <= 1) {
+        if (a.R == 16) LAUNCH((k_qkv_post_tile<HD, 16, 1>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+        else LAUNCH((k_qkv_post_tile<HD, -1, 1>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+    } else {
+        if (a.R == 16) LAUNCH((k_qkv_post_tile<HD, 16, NBM>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+        else LAUNCH((k_qkv_post_tile<HD, -1, NBM>), grid, dim3(256), 0, a, f.q_rt, f.q_pt, f.k_rt, f.k_pt, f.v_rt, f.v_pt, f.batch);
+    }
 }
 
 void launch_qkv_post_flash(const QkvPostArgs &a, const AttnFlashArgs &f)
