@@ -1310,6 +1310,11 @@ void launch_qkv_bwd(const QkvBwdArgs &a, int rows)
     b.rows_launched = rows;
     const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
     if (rows >= MANY_ROWS && a.R == 16 && a.hd <= 128 && !a.pf.base) { LAUNCH((k_qkv_bwd_rows<1, 16, TB>), grid, dim3(TB), n * 4, b); return; }
+    if (rows >= MANY_ROWS && a.R == 0 && !a.pf.base) {      // full-parameter mode: a handful of heads, no adapter projection
+        if (a.hd <= 128) LAUNCH((k_qkv_bwd_rows<1, 0, TB>), grid, dim3(TB), n * 4, b);
+        else LAUNCH((k_qkv_bwd_rows<MAXP, 0, TB>), grid, dim3(TB), n * 4, b);
+        return;
+    }
     if (a.hd <= 128) {
         if (a.R == 16) LAUNCH((k_qkv_bwd_rows<1, 16>), grid, dim3(RB), n * 4, b);
         else if (a.R == 0) LAUNCH((k_qkv_bwd_rows<1, 0>), grid, dim3(RB), n * 4, b);
