@@ -515,6 +515,7 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
     const int parts = max(1, TB / dpt), part = tid / dpt, d = (tid % dpt) * VEC;
     const bool active = part < parts;
     typedef float vecf __attribute__((ext_vector_type(VEC)));
+    constexpr int PT = 8;
     for (int g0 = 0; g0 < gpw; g0 += 4) {
         int gq[4];
 #pragma unroll
@@ -525,11 +526,11 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
 #pragma unroll
             for (int e = 0; e < VEC; e++) o[u][e] = 0.f;
         if (active)
-            for (int jj = part; jj < nj; jj += 4 * parts) {                    // four independent loads per trip
-                float v[4][VEC];
-                int jt[4];
+            for (int jj = part; jj < nj; jj += PT * parts) {                   // PT independent loads per trip
+                float v[PT][VEC];
+                int jt[PT];
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
+                for (int t = 0; t < PT; t++) {
                     jt[t] = min(jj + t * parts, nj - 1);
                     const float live = (jj + t * parts < nj) ? 1.f : 0.f;
                     if (VEC == 1) v[t][0] = vbase[(size_t)jt[t] * hd + d] * live;
@@ -540,7 +541,7 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
                     }
                 }
 #pragma unroll
-                for (int t = 0; t < 4; t++)
+                for (int t = 0; t < PT; t++)
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
                         const float w = sc[gq[u] * SL + jt[t]];
