@@ -52,6 +52,9 @@ struct HeadPost {
     const float2 *rope;                  // (cos, sin) of the hd/2 rotary pairs at position pos
     float eps, sc;
     size_t qkv_step, cache_step, t_step; // floats from one sequence's qkv / caches / t to the next when several are decoded at once
+    // weights of the product that follows, requested ahead by pf_wgs extra workgroups while the few attention workgroups
+    // run (pf_wgs == 0: none)
+    const char *pf_base; size_t pf_bytes; int pf_wgs;
 };
 // infer_kernels.hip: that and the attention over the cache rows 0 .. pos in one launch (out [Hq*hd]); with copies > 1
 // for that many sequences at position pos, whose caches lie cache_step floats apart inside Kc and Vc (out [copies, Hq*hd])

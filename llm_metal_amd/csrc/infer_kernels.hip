@@ -430,11 +430,28 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
     extern __shared__ float sm[];
     float *qs = sm, *sc = qs + gpw * hd, *ml = sc + gpw * SL, *red = ml + 2 * gpw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int head_groups = FUSED ? (int)gridDim.x - hp.pf_wgs : (int)gridDim.x;
+    if (FUSED && (int)blockIdx.x >= head_groups) {       // a workgroup that only asks for the next product's weights
+        if (blockIdx.y == 0 && blockIdx.z == 0) {
+            const size_t per = ((hp.pf_bytes + hp.pf_wgs - 1) / hp.pf_wgs + 4095) & ~(size_t)4095;
+            const size_t beg = (size_t)(blockIdx.x - head_groups) * per, end = min(hp.pf_bytes, beg + per);
+            unsigned sink = 0u;
+            for (size_t o = beg + threadIdx.x * 16; o < end; o += 8 * 4096) {
+                uint4 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = (o + u * 4096 < end) ? *reinterpret_cast<const uint4 *>(hp.pf_base + o + u * 4096) : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+                for (int u = 0; u < 8; u++) sink ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+            }
+            asm volatile("" :: "v"(sink));
+        }
+        return;
+    }
     const int hq0 = blockIdx.x * gpw, hkv = hq0 / G, split = blockIdx.y;
     const int j0 = split * SL, nj = min(SL, n_attend - j0);
     // blockIdx.z: one of several sequences decoded in lock step (FUSED only), each with its own product row, adapter
     // terms, caches and output; slice results are kept per (sequence, query head)
-    const int z = blockIdx.z, Hq_all = gridDim.x * gpw;
+    const int z = blockIdx.z, Hq_all = head_groups * gpw;
     if (FUSED) {
         hp.qkv += (size_t)z * hp.qkv_step; hp.kc += (size_t)z * hp.cache_step; hp.vc += (size_t)z * hp.cache_step;
         if (hp.R) hp.t += (size_t)z * hp.t_step;
@@ -650,10 +667,13 @@ void attention_launch(const float *Q, const float *Kc, const float *Vc, float *o
     float *po = nsplit > 1 ? partials : nullptr, *pml = nsplit > 1 ? partials + (size_t)copies * Hq * nsplit * hd : nullptr;
     const float scale = 1.0f / sqrtf((float)hd);
     const bool vec4 = hd % 4 == 0 && (((uintptr_t)Vc) & 15) == 0;
-    const dim3 grid(Hq / gpw, nsplit, copies);
+    HeadPost post{};
+    if (hp) post = *hp;
+    if ((Hq / gpw) * nsplit * copies > 128 || !post.pf_base || !post.pf_bytes) post.pf_wgs = 0;      // no spare CUs, or nothing to ask for
+    const dim3 grid(Hq / gpw + post.pf_wgs, nsplit, copies);
     const HeadPost none{};
 #define ATTN_LAUNCH(V_, F_) LAUNCH((k_attn_decode<V_, F_>), grid, dim3(TB), lds, Q, Kc, Vc, out, po, pml, \
-                                   n_attend, hd, max_seq, G, gpw, scale, nsplit, F_ ? *hp : none)
+                                   n_attend, hd, max_seq, G, gpw, scale, nsplit, F_ ? post : none)
     if (hp) { if (vec4) ATTN_LAUNCH(4, true); else ATTN_LAUNCH(1, true); }
     else { if (vec4) ATTN_LAUNCH(4, false); else ATTN_LAUNCH(1, false); }
 #undef ATTN_LAUNCH
