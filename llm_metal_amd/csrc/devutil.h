@@ -90,3 +90,22 @@ __device__ __forceinline__ float gelu_inner(float g)
 
 __device__ __forceinline__ half_t f2h(float x) { return (half_t)x; }      // v_cvt_f16_f32: round to nearest even
 __device__ __forceinline__ float  h2f(half_t x) { return (float)x; }
+
+// Workgroup `wg` of `nwgs` reads its share of [base, base + bytes) with 16-byte loads, eight in flight per thread, and
+// throws the values away: what a launch with spare CUs does for the weights of the product that follows it (the data then
+// waits in the memory-side cache).  bytes % 16 == 0; block of 256 threads or more.
+__device__ __forceinline__ void request_bytes_ahead(const char *base, size_t bytes, int wg, int nwgs)
+{
+    const size_t row = (size_t)blockDim.x * 16;
+    const size_t per = ((bytes + nwgs - 1) / nwgs + row - 1) / row * row;
+    const size_t beg = (size_t)wg * per, end = bytes < beg + per ? bytes : beg + per;
+    unsigned sink = 0u;
+    for (size_t o = beg + (size_t)threadIdx.x * 16; o < end; o += 8 * row) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = (o + u * row < end) ? *reinterpret_cast<const uint4 *>(base + o + u * row) : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int u = 0; u < 8; u++) sink ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    asm volatile("" :: "v"(sink));
+}

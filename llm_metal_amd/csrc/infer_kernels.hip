@@ -432,19 +432,7 @@ __global__ __launch_bounds__(TB) void k_attn_decode(const float *__restrict__ Q,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int head_groups = FUSED ? (int)gridDim.x - hp.pf_wgs : (int)gridDim.x;
     if (FUSED && (int)blockIdx.x >= head_groups) {       // a workgroup that only asks for the next product's weights
-        if (blockIdx.y == 0 && blockIdx.z == 0) {
-            const size_t per = ((hp.pf_bytes + hp.pf_wgs - 1) / hp.pf_wgs + 4095) & ~(size_t)4095;
-            const size_t beg = (size_t)(blockIdx.x - head_groups) * per, end = min(hp.pf_bytes, beg + per);
-            unsigned sink = 0u;
-            for (size_t o = beg + threadIdx.x * 16; o < end; o += 8 * 4096) {
-                uint4 v[8];
-#pragma unroll
-                for (int u = 0; u < 8; u++) v[u] = (o + u * 4096 < end) ? *reinterpret_cast<const uint4 *>(hp.pf_base + o + u * 4096) : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-                for (int u = 0; u < 8; u++) sink ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
-            }
-            asm volatile("" :: "v"(sink));
-        }
+        if (blockIdx.y == 0 && blockIdx.z == 0) request_bytes_ahead(hp.pf_base, hp.pf_bytes, blockIdx.x - head_groups, hp.pf_wgs);
         return;
     }
     const int hq0 = blockIdx.x * gpw, hkv = hq0 / G, split = blockIdx.y;
