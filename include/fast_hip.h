@@ -159,6 +159,10 @@ void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
  * F16 image made once per product); 2: always the large-M kernel with Q8_0 tiles kept quantised and unpacked into LDS
  * by the kernel itself; -1: never (always the weight-streaming kernel). */
 void hip_gemm_force_large_m(int policy);
+/* Products of up to 64 activation rows with F16 weights: 1 (default) = the kernel whose workgroups stream their operands
+ * into an LDS ring (gemm_ring: one or two workgroups per CU, 4 to 6 K chunks), 0 = the kernel with one K step per wave in
+ * registers (gemm_tiled: 13 to 19 K chunks), which every other product takes.  Same results up to the order of the sums. */
+void hip_gemm_ring(int on);
 /* K chunks of the large-M kernel on F16 tiles (each chunk writes a plane, the consumer adds them): 1 = by the measured
  * rule (three chunks when the 128 x 256 output blocks leave a third of the CUs idle and K >= 4096), 0 = never, n > 1 =
  * always n. */

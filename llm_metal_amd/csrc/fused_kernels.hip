@@ -765,8 +765,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
 // columns [c * sg.cols, (c + 1) * sg.cols) and scales them by a factor of its own, inv_scale[row * groups + c].  The
 // GEMM that reads the operand cuts K into chunks that do not straddle groups, so every plane of its result belongs to
 // one factor.  64 rows then occupy the whole GPU instead of 64 CUs.
-constexpr int GC = 256, MAXC = 2;                         // threads of a column-group workgroup; float4 per thread
-template <int GELU>                                       // compile-time: the kernel's code stays one straight run
+constexpr int MAXC = 2;                                   // float4 per thread of a column-group workgroup
+constexpr int GC_MAX = 512;                               // its threads: 256 for groups of up to 2048 columns, 512 up to 4096
+template <int GELU, int GC>                               // compile-time: the kernel's code stays one straight run
 __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
 {
     __shared__ float sm[16];
@@ -869,7 +870,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
 // The same with the columns of the output row [dgate | dup] split among workgroups (grid (rows, groups), block GC), as
 // in k_glu_fwd_cols.  A group may lie in either half or straddle the middle, so a thread computes the half its output
 // column belongs to; the inputs of a column are then read twice in all, by different workgroups.
-template <int GELU>
+template <int GELU, int GC>
 __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
 {
     __shared__ float sm[16];
@@ -1347,10 +1348,15 @@ void launch_glu_fwd(const GluArgs &a, int rows)
     require(!a.in_place || (a.in.S == 1 && !a.in.row_scale && a.in.p == a.gate_pre && (size_t)a.in.ld == a.ld_gu),
             "glu_fwd: in place needs the product's one finished plane to be the kept [gate | up] array");
     if (a.sg.cols) {
-        require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC * MAXC && (long)a.sg.cols * a.sg.groups >= a.IS && (long)a.sg.cols * (a.sg.groups - 1) < a.IS,
+        require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC_MAX * MAXC && (long)a.sg.cols * a.sg.groups >= a.IS && (long)a.sg.cols * (a.sg.groups - 1) < a.IS,
                 "glu_fwd: column groups do not fit the row");
-        if (a.gelu) LAUNCH(k_glu_fwd_cols<1>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
-        else LAUNCH(k_glu_fwd_cols<0>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        if (a.sg.cols <= 4 * 256 * MAXC) {
+            if (a.gelu) LAUNCH((k_glu_fwd_cols<1, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+            else LAUNCH((k_glu_fwd_cols<0, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+        } else {
+            if (a.gelu) LAUNCH((k_glu_fwd_cols<1, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+            else LAUNCH((k_glu_fwd_cols<0, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+        }
         return;
     }
     // many rows: one plane per batch of loads keeps the kernel within 64 registers, so that two workgroups share a CU and
@@ -1363,10 +1369,15 @@ void launch_glu_bwd(const GluArgs &a, int rows)
     require(a.IS % 4 == 0 && a.IS <= 4 * RB * MAXV && a.in.ld % 4 == 0, "glu_bwd: FFN width must be a multiple of 4, <= 12288");
     require(!a.in.scale_groups, "glu_bwd: input planes with grouped row factors are not supported");
     if (a.sg.cols) {
-        require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC * MAXC && (long)a.sg.cols * a.sg.groups >= 2 * a.IS && (long)a.sg.cols * (a.sg.groups - 1) < 2 * a.IS,
+        require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC_MAX * MAXC && (long)a.sg.cols * a.sg.groups >= 2 * a.IS && (long)a.sg.cols * (a.sg.groups - 1) < 2 * a.IS,
                 "glu_bwd: column groups do not fit the row");
-        if (a.gelu) LAUNCH(k_glu_bwd_cols<1>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
-        else LAUNCH(k_glu_bwd_cols<0>, dim3(rows, a.sg.groups), dim3(GC), 0, a);
+        if (a.sg.cols <= 4 * 256 * MAXC) {
+            if (a.gelu) LAUNCH((k_glu_bwd_cols<1, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+            else LAUNCH((k_glu_bwd_cols<0, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+        } else {
+            if (a.gelu) LAUNCH((k_glu_bwd_cols<1, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+            else LAUNCH((k_glu_bwd_cols<0, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+        }
         return;
     }
     if (rows >= MANY_ROWS) { LAUNCH((k_glu_bwd<RB, MAXV, 1, 8>), dim3(rows), dim3(RB), 0, a); return; }

@@ -27,6 +27,7 @@
 #include "gemm_kernel.h"
 #include <hip/hip_ext.h>
 #include <vector>
+#include <algorithm>
 
 namespace {
 
@@ -261,6 +262,7 @@ int g_prof_on = 0;
 std::vector<ProfRec> g_prof;
 int g_force_nb = 0, g_force_S = 0;
 int g_wide_wg = 1;                     // eight-wave workgroups where K would be cut into ten or more chunks
+int g_ring = 1;                        // gemm_ring for one-tile products with F16 weights
 
 }  // namespace
 
@@ -270,13 +272,44 @@ namespace lmhip {
 // (activation bytes through L1/L2 = weight bytes), about three workgroups per CU, chunks of at
 // least 4 and at most 40 K steps (long chunks gain nothing and short ones spread the
 // activation reads over more L2 lines); beyond that, splitting K only adds plane traffic.
-GemmPlan plan_gemm(int M, int N, int K, int nbq)
+// K chunks for gemm_ring.  Measured on MI355X (256 CUs; Qwen3-4B and Gemma3-1B layer shapes at 64 rows, cold weights):
+// the launch is fastest when every CU has the same number of workgroups — one for up to 256 of them, two for up to 512
+// (64 KB of LDS each) — and loses when some CUs have one more than others (320 workgroups: 9.2 us against 8.1 for 240
+// on 2560 x 4096) or when not all are resident at once (beyond 512).  Among equally balanced splits the one with fewer
+// planes wins: a plane costs the product its stores and the consumer its loads (the more the shorter K is).
+static int ring_chunks(int n_tiles, int Kb, int K, int cus)
+{
+    int best = 1;
+    double best_score = -1e9;
+    for (int S = 1; S <= 32 && S <= Kb; S++) {
+        const int steps = (Kb + S - 1) / S;
+        if ((Kb + steps - 1) / steps != S) continue;       // this S does not exist (the last chunk would be empty)
+        const long wgs = (long)n_tiles * S;
+        const long slots = wgs <= 2L * cus ? cus : 2L * cus;
+        double eff = (double)wgs / (double)(slots * ((wgs + slots - 1) / slots));
+        if (wgs > 2L * cus) eff *= 0.85;
+        const double score = eff - 0.05 * S * (K > 2560 ? 2560.0 / K : 1.0);
+        if (score > best_score + 1e-9) { best_score = score; best = S; }
+    }
+    return best;
+}
+
+GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
 {
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), m_tiles = (M + 63) / 64;
     const int cus = num_cus() > 0 ? num_cus() : 256;
     GemmPlan p{};
     p.nw = 4;
     p.m_tiles = m_tiles;
+    if (g_ring && fmt == 0 && m_tiles == 1 && !g_force_nb) {
+        p.ring = 1; p.kg = 2; p.nw = 8; p.nb = 2;
+        p.n_tiles = (Nb + 1) / 2;
+        const int S = g_force_S ? std::min(g_force_S, Kb) : ring_chunks(p.n_tiles, Kb, K, cus);
+        p.steps = (Kb + S - 1) / S;
+        p.S = (Kb + p.steps - 1) / p.steps;
+        p.rotate = 0;
+        return p;
+    }
     auto split = [&](int nb) {
         p.nb = nb;
         p.n_tiles = (Nb + nb - 1) / nb;
@@ -321,6 +354,36 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         fprintf(stderr, "[fast_hip] gemm: bad launch M=%d N=%d K=%d ldp=%d fmt=%d nbq=%d kbq=%d plan(nb=%d S=%d steps=%d)\n",
                 M, N, K, ldp, W.fmt, W.nbq, W.kbq, p.nb, p.S, p.steps);
         abort();
+    }
+    if (p.ring) {
+        if (W.fmt != 0 || p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (Nb + 1) / 2 ||
+            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb) {
+            fprintf(stderr, "[fast_hip] gemm_ring: bad launch M=%d N=%d K=%d fmt=%d plan(kg=%d S=%d steps=%d tiles=%d)\n", M, N, K, W.fmt, p.kg, p.S, p.steps, p.n_tiles);
+            abort();
+        }
+        ProfRec rrec{};
+        hipEvent_t ra = nullptr, rb = nullptr;
+        if (g_prof_on) {
+            HIP_CHECK(hipEventCreate(&rrec.a)); HIP_CHECK(hipEventCreate(&rrec.b));
+            rrec.wbytes = weight_stream_bytes(W, N, K); rrec.flops = 2.0 * M * N * K;
+            ra = rrec.a; rb = rrec.b;
+        }
+        GemmKArgs g{};
+        g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
+        g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
+        g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
+        g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1;
+        const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(256 * p.kg);
+#define RING_LAUNCH(KGV, SC) do { \
+            if (g_prof_on) hipExtLaunchKernelGGL((gemm_ring<KGV, SC>), rgrid, rblock, 0, stream(), ra, rb, 0, g); \
+            else hipLaunchKernelGGL((gemm_ring<KGV, SC>), rgrid, rblock, 0, stream(), g); } while (0)
+#define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1); else RING_LAUNCH(KGV, 0); } while (0)
+        if (p.kg == 1) RING_PICK(1); else if (p.kg == 2) RING_PICK(2); else RING_PICK(4);
+#undef RING_PICK
+#undef RING_LAUNCH
+        HIP_CHECK(hipGetLastError());
+        if (g_prof_on) g_prof.push_back(rrec);
+        return;
     }
     dim3 grid(p.n_tiles, p.S, p.m_tiles), block(p.nw * 64);
     if (p.m_tiles > 1) grid = dim3((unsigned)(((size_t)p.n_tiles * p.S + 7) / 8 * 8 * p.m_tiles), 1, 1);   // see gemm_tiled
@@ -422,6 +485,8 @@ void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, in
 }
 
 int gemm_profiling() { return g_prof_on; }
+void set_gemm_ring(int on) { g_ring = on; }
+int gemm_ring_enabled() { return g_ring; }
 
 // Which kernel multiplies an [M, K] activation block with an [N, K] weight.  Measured on MI355X (Qwen3-4B shapes):
 // the 128 x 256 LDS-tiled kernel wins for F16 weights once there is about one block per CU (2048 rows: 490-650
@@ -591,6 +656,7 @@ void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, i
 }
 
 void hip_gemm_force_large_m(int policy) { g_big_policy = policy; }
+void hip_gemm_ring(int on) { lmhip::set_gemm_ring(on); }
 void hip_gemm_large_m_split(int mode) { set_big_gemm_split(mode); }
 void hip_gemm_large_m_block(int mode) { set_big_gemm_block(mode); }
 
@@ -631,7 +697,7 @@ int hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double 
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S)
 {
     g_force_nb = nb == 128 ? 0 : nb; g_force_S = S;
-    GemmPlan p = plan_gemm(M, N, K);
+    GemmPlan p = plan_gemm(M, N, K, 0, wf);
     g_force_nb = 0; g_force_S = 0;
     if (used_nb) *used_nb = p.nb;
     if (used_S) *used_S = p.S;

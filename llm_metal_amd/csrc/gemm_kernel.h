@@ -246,4 +246,118 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 #undef ACC_AT
 }
 
+// ---- the same product for one 64-row tile of activations and F16 weights: workgroups that own their loads --------------
+// gemm_ring<KG, SCALE>: one workgroup of 4 KG waves per (64 weight rows, K chunk).  Where gemm_tiled puts twelve waves on a
+// CU, each with one K step in registers, and then adds the waves' accumulators through LDS (32 KB per workgroup, all
+// workgroups of a launch at the same moment), this kernel gives the CU one or two workgroups whose loads go straight
+// into LDS (global_load_lds_dwordx4: no registers, so the bytes in flight do not depend on the number of waves) and
+// splits the 64 x 64 output among the waves as 2 x 2 quadrants of 32 x 32 times KG groups that take every KG-th K step:
+//   * a K step is one 16 KB stage: [weight row block 0 | 1 | activation row block 0 | 1], 4 KB each; wave (q, kg)
+//     requests block q of its group's stage (four 1 KB pieces) and multiplies weight block q & 1 with activation block
+//     q >> 1: every byte is fetched once per workgroup and read from LDS twice;
+//   * the ring holds two rounds of KG stages; round r + 2 is requested when round r has been read;
+//   * at the end the KG groups exchange 16 / KG accumulator registers per lane (4 KB per wave instead of 12) and every
+//     wave stores its part.
+// A workgroup covers a K chunk that four-wave workgroups would cut into three, so a product leaves 4 to 6 planes where it
+// left 13 to 19, and the launch runs one workgroup per CU (plan_gemm), which keeps the CUs' shares of the stream equal.
+// Weight loads are non-temporal (streamed once), activation loads are not (every workgroup of a chunk reads them).
+// The LDS-direct loads are issued as assembly: the compiler cannot tell which LDS bytes a pending load writes and would
+// wait for all of them before every LDS read; the waits are written by hand below.
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+template <int KG, int SCALE>
+__global__ __launch_bounds__(256 * KG) void gemm_ring(GemmKArgs g)
+{
+    static_assert(KG == 1 || KG == 2 || KG == 4, "K groups per workgroup");
+    constexpr int LOADS_PER_ROUND = 4;                    // LDS-direct loads a wave issues per round: the four 1 KB pieces of its block
+    __shared__ half8 ring[2 * KG * 1024];                 // [round parity][K group][block 0..3][slice 0..3][64 lanes]
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int q = wv & 3, kg = wv >> 2, qm = q >> 1, qn = q & 1;
+    const int r = lane & 31, h = lane >> 5;
+    const int tile = blockIdx.x % g.n_tiles, chunk = blockIdx.x / g.n_tiles;
+    const int kb_beg = chunk * g.steps_per_chunk;
+    const int nsteps = min(g.Kb, kb_beg + g.steps_per_chunk) - kb_beg;
+    const int rounds = (nsteps + KG - 1) / KG;
+    // q = 0, 1: weight row blocks 2 tile + q; q = 2, 3: activation row blocks q - 2 (clamped: rows beyond M or N are not stored)
+    const half8 *src = q < 2 ? reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(2 * tile + q, g.Nb - 1) * g.Kb + kb_beg) * 256 + lane
+                             : g.A + ((size_t)min(q - 2, g.Mb - 1) * g.Kb + kb_beg) * 256 + a_lane(lane);
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)ring;
+    auto request = [&](int round) __attribute__((always_inline)) {
+        const int step = min(round * KG + kg, nsteps - 1);    // a group without a step in the last round loads the last step again
+        const uint32_t sb = base + (uint32_t)(((round & 1) * KG + kg) * 16384 + q * 4096);
+#pragma unroll
+        for (int j = 0; j < LOADS_PER_ROUND; j++) {
+            if (q < 2) asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src + (size_t)step * 256 + j * 64), "s"(sb + (uint32_t)(j * 1024)) : "m0", "memory");
+            else asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src + (size_t)step * 256 + j * 64), "s"(sb + (uint32_t)(j * 1024)) : "m0", "memory");
+        }
+    };
+    float16v acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    request(0);
+    if (rounds > 1) request(1);
+    for (int rd = 0; rd < rounds; rd++) {
+        // in flight at this point: this wave's loads of round rd and, if there is one, of round rd + 1; loads retire in
+        // order, so all but the LOADS_PER_ROUND newest having retired means round rd has landed
+        if (rd + 1 < rounds) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS_PER_ROUND) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                     // ... and every other wave's as well
+        const half8 *st = ring + ((rd & 1) * KG + kg) * 1024;
+        half8 w[4], a[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = st[(qn * 4 + j) * 64 + lane];
+#pragma unroll
+        for (int j = 0; j < 4; j++) a[j] = st[((2 + qm) * 4 + j) * 64 + lane];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                     // all waves have read the stages of this round: they may be refilled
+        if (rd + 2 < rounds) request(rd + 2);
+        if (rd * KG + kg < nsteps) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j], w[j], acc, 0, 0, 0);
+        }
+    }
+    // Exchange: wave (q, kg) ends up with registers [kg Q, kg Q + Q) of quadrant q, Q = 16 / KG, summed over the groups.
+    constexpr int Q = 16 / KG;
+    float res[Q];
+#pragma unroll
+    for (int k = 0; k < Q; k++) res[k] = acc[kg * Q + k];
+    if constexpr (KG > 1) {
+        float *ex = reinterpret_cast<float *>(ring);       // [q][owner][giver][Q][64 lanes]; the ring is free (last barrier above)
+#pragma unroll
+        for (int o = 0; o < KG; o++)
+            if (o != kg) {
+#pragma unroll
+                for (int k = 0; k < Q; k++) ex[(((q * KG + o) * KG + kg) * Q + k) * 64 + lane] = acc[o * Q + k];
+            }
+        __syncthreads();
+#pragma unroll
+        for (int gv = 0; gv < KG; gv++)
+            if (gv != kg) {
+#pragma unroll
+                for (int k = 0; k < Q; k++) res[k] += ex[(((q * KG + kg) * KG + gv) * Q + k) * 64 + lane];
+            }
+    }
+    // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8 (v / 4) + 4 (lane / 32) + v % 4
+    float *Pp = g.P + (size_t)chunk * g.plane_stride;
+    const int n = (tile * 2 + qn) * 32 + r;
+    const bool inside = 64 <= g.M && (tile + 1) * 64 <= g.N;
+    float sc[Q];
+    if (SCALE) {
+#pragma unroll
+        for (int k = 0; k < Q; k++) { const int v = kg * Q + k; sc[k] = g.a_inv_scale[min(qm * 32 + 8 * (v >> 2) + 4 * h + (v & 3), g.M - 1)]; }
+#pragma unroll
+        for (int k = 0; k < Q; k++) res[k] *= sc[k];
+    }
+    if (inside) {
+#pragma unroll
+        for (int k = 0; k < Q; k++) { const int v = kg * Q + k; Pp[(size_t)(qm * 32 + 8 * (v >> 2) + 4 * h + (v & 3)) * g.ldp + n] = res[k]; }
+    } else {
+#pragma unroll
+        for (int k = 0; k < Q; k++) {
+            const int v = kg * Q + k, m = qm * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (m < g.M && n < g.N) Pp[(size_t)m * g.ldp + n] = res[k];
+        }
+    }
+}
+
 }  // namespace lmhip

@@ -183,14 +183,18 @@ size_t max_planes_elems(SFTState *s)
     const Sh shapes[] = {{s->nq_ext, s->D}, {s->D, s->qd}, {2 * s->IS, s->D}, {s->D, s->IS}, {s->V, s->D},
                          {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->nq_ext}};
     size_t mx = 0;
+    const int ring_was = gemm_ring_enabled();             // the kernel family can be switched at run time: room for either
+    for (int ring = 0; ring < 2; ring++)
     for (const Sh &sh : shapes) {
-        GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0);
+        set_gemm_ring(ring);
+        GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0, s->q8_native ? 1 : 0);
         // whichever kernel the product takes (the choice can be forced at run time): the planes of the streaming kernel, or
         // up to four K chunks of the large-M one; the LM head writes the logits directly unless the streaming kernel splits K
         const bool head = sh.N == s->V && sh.K == s->D;
         const size_t e = (size_t)(head ? (p.S > 1 ? p.S : 0) : std::max({p.S, 4, big_gemm_chunks(s->BN, sh.N, sh.K, 0)})) * s->BN * sh.N;
         if (e > mx) mx = e;
     }
+    set_gemm_ring(ring_was);
     return mx;
 }
 
@@ -198,15 +202,15 @@ constexpr int MAX_SCALE_GROUPS = 64;                      // group_inv holds thi
 
 // Column groups for the row kernel that writes the operand [BN, K] of the product with W [N, K]: as many groups as it
 // takes to put about two workgroups on every CU, each a power-of-two number of the GEMM's K chunks and at most 2048
-// columns wide.  None (cols = 0) when the product does not leave planes (large M, S == 1) or the rows alone fill the GPU.
+// columns wide (a single chunk: up to 4096).  None (cols = 0) when the product does not leave planes (large M, S == 1) or the rows alone fill the GPU.
 ScaleGroups scale_groups_for(SFTState *s, const WeightOp &W, int N, int K)
 {
     ScaleGroups none{0, 1, 0};
     if (s->full_param || use_big_gemm(s->BN, N, K, W.fmt)) return none;      // weight gradients take one factor per row
-    const GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
+    const GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0, W.fmt);
     const int plane_cols = p.steps * 64, cus = num_cus() > 0 ? num_cus() : 256;
     const int want = (2 * cus + s->BN - 1) / s->BN;
-    if (p.S <= 1 || want <= 1 || plane_cols > 2048) return none;
+    if (p.S <= 1 || want <= 1 || plane_cols > 4096) return none;
     int shift = 0;
     while ((plane_cols << (shift + 1)) <= 2048 && ((p.S + (2 << shift) - 1) >> (shift + 1)) >= want) shift++;
     ScaleGroups g{plane_cols << shift, (p.S + (1 << shift) - 1) >> shift, shift};
@@ -224,15 +228,20 @@ WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int th
     constexpr int mb = 16, depth = 4, wgs1024 = 160;
     WeightPrefetch pf{};
     if (s->full_param || W.fmt != 0 || !W.w16 || use_big_gemm(s->BN, N, K, W.fmt)) return pf;
-    const GemmPlan p = plan_gemm(s->BN, N, K, 0);
+    const GemmPlan p = plan_gemm(s->BN, N, K, 0, W.fmt);
     if (p.m_tiles != 1 || unit <= 0) return pf;
     int wgs = wgs1024 * (1024 / threads);
     wgs = (wgs + unit - 1) / unit * unit;
     pf.base = reinterpret_cast<const char *>(W.w16);
     pf.Kb = tiled_kb(K); pf.Nb = tiled_rb(N);
     pf.nb = p.nb; pf.steps = p.steps; pf.S = p.S; pf.n_tiles = p.n_tiles; pf.rotate = p.rotate;
-    pf.wgs = wgs; pf.depth = depth;
-    const long covered = std::min<long>((long)mb * 1024 * 1024 / ((long)p.nb * depth * 4096), (long)p.n_tiles * p.S);
+    // few workgroups with long chunks (gemm_ring): the same bytes reach further into each chunk
+    const long total = (long)p.n_tiles * p.S;
+    int d = depth;
+    if (total * p.nb * depth * 4096 < (long)mb * 1024 * 1024) d = (int)std::min<long>(p.steps, (long)mb * 1024 * 1024 / (total * p.nb * 4096));
+    if (d < depth) d = std::min(depth, p.steps);
+    pf.wgs = wgs; pf.depth = d;
+    const long covered = std::min<long>((long)mb * 1024 * 1024 / ((long)p.nb * d * 4096), total);
     pf.per_wg = (int)((covered + wgs - 1) / wgs);
     return pf;
 }
@@ -286,7 +295,7 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
         const int planes = launch_gemm_big(A, inv, Wf, C, N, s->BN, N, K, chunks, stride);
         return Planes{C, planes, stride, N, nullptr};
     }
-    GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0);
+    GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0, W.fmt);
     float *P = out ? out : at<float>(s->planes);
     const size_t stride = (size_t)s->BN * N;
     if (!out && (size_t)p.S * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
@@ -418,7 +427,7 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
     nf.ln16 = lnf; nf.inv_scale = lnfinv; nf.D = D; nf.eps = s->eps;
     nf.pf = prefetch_for(s, wop(s, W_LM, 0, false), s->V, D, 1024);
     launch_norm_rows(nf, BN);
-    GemmPlan pl = plan_gemm(BN, s->V, D);
+    GemmPlan pl = plan_gemm(BN, s->V, D, 0, s->q8_native ? 1 : 0);
     if (pl.S == 1 || use_big_gemm(BN, s->V, D, s->q8_native ? 1 : 0)) {
         gemm(s, lnf, lnfinv, wop(s, W_LM, 0, false), s->V, D, at<float>(s->logits));
     } else {
