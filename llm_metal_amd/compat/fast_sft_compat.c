@@ -5,109 +5,46 @@
  *
  *   cc -DFAST_METAL_H -I<reference>/src/nn -I<this repo>/include -c fast_sft_compat.c
  *
- * Only field reads: the seven matrices and the norm vectors of every block
- * (what src/nn/fast_sft.c:212-239 and :327-356 hand to layers_convert_upload),
- * the per-layer RoPE base (:310-313) and, when the model carries attached
- * adapters, their A and B tensors (:96-98, 110-112).
+ * The struct reads themselves are in model_ref_compat.h, shared with
+ * fast_inference_compat.c.
  */
 #include "fast_sft_compat.h"
-#include <stdlib.h>
-#include <string.h>
+#include "model_ref_compat.h"
 
-typedef struct {
-    ModelType type;
-    int NL, D, Hq, Hkv, hd, IS, V;
-    LoRALinear **q_loras, **v_loras;
-    Embedding *token_emb;
-    const float *lm_head, *final_norm_g;
-} Dims;
-
-static void fill_layer(LayerWeightRef *r, const Dims *d, GroupedQueryAttention *attn,
-                       Linear *gate, Linear *up, Linear *down,
-                       RMSNorm *in, RMSNorm *post_attn, RMSNorm *pre_ff, RMSNorm *post_ff)
+/* Attached adapters of another rank, or attached to some layers only, are not used: say so (the reference takes the
+ * attached adapters of every layer that has them, src/nn/fast_sft.c:96-112; this pipeline keeps all layers at one rank). */
+static float *attached_or_warn(const Dims *d, int rank)
 {
-    const int qd = d->Hq * d->hd, kd = d->Hkv * d->hd;
-    r->q_proj = (WeightRef){ attn->q_proj->weight->data, qd, d->D };
-    r->k_proj = (WeightRef){ attn->k_proj->weight->data, kd, d->D };
-    r->v_proj = (WeightRef){ attn->v_proj->weight->data, kd, d->D };
-    r->o_proj = (WeightRef){ attn->o_proj->weight->data, d->D, qd };
-    r->gate_proj = (WeightRef){ gate->weight->data, d->IS, d->D };
-    r->up_proj = (WeightRef){ up->weight->data, d->IS, d->D };
-    r->down_proj = (WeightRef){ down->weight->data, d->D, d->IS };
-    r->input_norm_g = in->gamma->data;
-    r->post_attn_norm_g = post_attn->gamma->data;
-    r->pre_ff_norm_g = pre_ff ? pre_ff->gamma->data : NULL;
-    r->post_ff_norm_g = post_ff ? post_ff->gamma->data : NULL;
-    r->q_norm_g = attn->q_norm->gamma->data;
-    r->k_norm_g = attn->k_norm->gamma->data;
-    r->d_model = d->D;
-    r->head_dim = d->hd;
+    float *lora = pack_attached_lora(d, rank);
+    if (!lora && rank > 0 && d->q_loras && d->v_loras)
+        fprintf(stderr, "[FastSFT] the model's attached adapters are ignored (a layer without them, or a rank other than %d): "
+                        "starting from A ~ U(-1,1)/sqrt(d_model), B = 0\n", rank);
+    return lora;
 }
 
-/* A_q | B_q | A_v | B_v per layer from the model's attached adapters, or NULL when it has none
- * (or their rank differs from the one asked for). */
-static float *pack_attached_lora(const Dims *d, int rank)
-{
-    if (rank <= 0 || !d->q_loras || !d->v_loras) return NULL;
-    const size_t a = (size_t)rank * d->D, bq = (size_t)d->Hq * d->hd * rank, bv = (size_t)d->Hkv * d->hd * rank;
-    for (int L = 0; L < d->NL; L++)
-        if (!d->q_loras[L] || !d->v_loras[L] || d->q_loras[L]->rank != rank || d->v_loras[L]->rank != rank) return NULL;
-    float *flat = malloc((2 * a + bq + bv) * d->NL * sizeof(float)), *p = flat;
-    if (!flat) return NULL;
-    for (int L = 0; L < d->NL; L++) {
-        memcpy(p, d->q_loras[L]->lora_A->data, a * sizeof(float));  p += a;
-        memcpy(p, d->q_loras[L]->lora_B->data, bq * sizeof(float)); p += bq;
-        memcpy(p, d->v_loras[L]->lora_A->data, a * sizeof(float));  p += a;
-        memcpy(p, d->v_loras[L]->lora_B->data, bv * sizeof(float)); p += bv;
-    }
-    return flat;
-}
-
-static SFTState *create(const Dims *d, LayerWeightRef *refs, float *thetas, int seq_len, int rank, float alpha)
+static SFTState *create(ModelDesc *m, int have, int seq_len, int rank, float alpha)
 {
     SFTState *s = NULL;
-    if (refs && thetas) {
-        float *lora = pack_attached_lora(d, rank);
-        SFTModelRef ref = { d->type, d->NL, d->D, d->Hq, d->Hkv, d->hd, d->IS, d->V, thetas, refs,
-                            d->token_emb->weight->data, d->lm_head, d->final_norm_g, lora };
+    if (have == 0) {
+        float *lora = attached_or_warn(&m->d, rank);
+        const SFTModelRef ref = model_desc_ref(m, lora);
         s = sft_state_create_from_ref(&ref, /* batch */ 1, seq_len, rank, alpha, /* F16 weights */ 1);
         free(lora);
+        model_desc_free(m);
     }
-    free(refs);
-    free(thetas);
     return s;
 }
 
-static SFTState *create_qwen3(Qwen3Model *m, int seq_len, int rank, float alpha)
+static SFTState *create_qwen3(Qwen3Model *model, int seq_len, int rank, float alpha)
 {
-    const Dims d = { MODEL_QWEN3, m->n_layers, m->d_model, m->n_q_heads, m->n_kv_heads, m->head_dim,
-                     m->intermediate_size, m->vocab_size, m->q_loras, m->v_loras, m->token_emb,
-                     m->lm_head->weight->data, m->final_norm->gamma->data };
-    LayerWeightRef *refs = calloc((size_t)d.NL, sizeof *refs);
-    float *thetas = malloc((size_t)d.NL * sizeof *thetas);
-    for (int i = 0; refs && thetas && i < d.NL; i++) {
-        Qwen3Block *b = m->blocks[i];
-        fill_layer(&refs[i], &d, b->attn, b->gate_proj, b->up_proj, b->down_proj, b->input_norm, b->post_attn_norm, NULL, NULL);
-        thetas[i] = m->rope_theta;
-    }
-    return create(&d, refs, thetas, seq_len, rank, alpha);
+    ModelDesc m;
+    return create(&m, model_desc_qwen3(&m, model), seq_len, rank, alpha);
 }
 
-static SFTState *create_gemma3(Gemma3Model *m, int seq_len, int rank, float alpha)
+static SFTState *create_gemma3(Gemma3Model *model, int seq_len, int rank, float alpha)
 {
-    /* the head is tied to the embedding table (src/nn/fast_sft.c:351) */
-    const Dims d = { MODEL_GEMMA3, m->n_layers, m->d_model, m->n_q_heads, m->n_kv_heads, m->head_dim,
-                     m->intermediate_size, m->vocab_size, m->q_loras, m->v_loras, m->token_emb,
-                     m->token_emb->weight->data, m->final_norm->gamma->data };
-    LayerWeightRef *refs = calloc((size_t)d.NL, sizeof *refs);
-    float *thetas = malloc((size_t)d.NL * sizeof *thetas);
-    for (int i = 0; refs && thetas && i < d.NL; i++) {
-        Gemma3Block *b = m->blocks[i];
-        fill_layer(&refs[i], &d, b->attn, b->gate_proj, b->up_proj, b->down_proj, b->input_norm, b->post_attn_norm,
-                   b->pre_ff_norm, b->post_ff_norm);
-        thetas[i] = (i % 6) != 0 ? m->local_rope_theta : m->global_rope_theta;      /* src/nn/fast_sft.c:310-313 */
-    }
-    return create(&d, refs, thetas, seq_len, rank, alpha);
+    ModelDesc m;
+    return create(&m, model_desc_gemma3(&m, model), seq_len, rank, alpha);
 }
 
 SFTState *sft_state_create(Qwen3Model *model, int seq_len, int lora_rank, float lora_alpha)
