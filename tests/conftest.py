@@ -16,3 +16,20 @@ def pytest_configure(config):
 def _oracle_built():
     from oracle import oracle
     oracle.build()
+
+
+@pytest.fixture(autouse=True)
+def _default_kernel_policies(request):
+    """The library's kernel-family switches are process-global: whatever a GPU test sets, the next test starts from the
+    defaults again, also when the test failed half way."""
+    yield
+    if request.node.get_closest_marker("gpu") is None:
+        return
+    from llm_metal_amd import lib
+    L = lib.load()
+    L.hip_gemm_force_large_m(0)
+    L.hip_gemm_large_m_split(1)
+    L.hip_gemm_large_m_block(0)
+    L.hip_gemm_ring(1)
+    L.hip_attention_flash(-1)
+    L.hip_gemm_image_budget_mb(65536)

@@ -7,7 +7,7 @@ import sys
 import numpy as np
 import pytest
 
-from llm_metal_amd.configs import C1, GEMMA3, SFTConfig
+from llm_metal_amd.configs import C1, C3, GEMMA3, SFTConfig
 from llm_metal_amd.sft import InferenceState, SFTState
 from llm_metal_amd.synth import make_batch, make_model
 from tests.decode_chain import oracle_decode
@@ -124,6 +124,50 @@ def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, wit
             check(inf, None)
         with InferenceState(c, model, max_seq=max_seq, use_fp16=False) as q8:
             assert q8.generate_batch(prompt, n, 2).shape[1] == 0       # F16 weights only, as in the reference
+
+
+# Qwen3-4B's widths (hidden 2560, 32 / 8 heads of 128, FFN 9728): the instantiations that `bench.py --decode` launches --
+# two weight rows per wave with the SiLU gate and the norm inside the launch at 19456 x 2560, the norm-fused Q|K|V
+# product at 6144 x 2560, the attention kernel with four-key steps, the fused per-head prologue and the O weights asked
+# for ahead at 32 / 8 heads of 128, and, for the batch, the matrix-core products on split rows.  Two layers, vocabulary cut.
+C3_DECODE = C3.with_(name="c3_decode_widths", NL=2, V=8192, seq=24)
+
+
+@pytest.mark.parametrize("fmt,with_lora", [("f16", False), ("q8_0", False), ("f16", True)], ids=["f16", "q8_0", "f16_adapters"])
+def test_decode_at_the_benchmarked_widths(fmt, with_lora):
+    say("decode at config 3's widths", fmt, with_lora)
+    c = C3_DECODE.with_(weight_format=fmt)
+    model = make_model(c, seed=27, gamma_jitter=0.1)
+    toks = [int(t) for t in np.random.default_rng(28).integers(1, c.V, 16)]
+    lora = model["lora"] if with_lora else None
+    ref = oracle_decode(c, model, fmt, toks, max_seq=64, precision="f32", lora=lora)
+
+    def check(inf):
+        got = np.stack([inf.forward_token(t) for t in toks])
+        assert maxrel(got, ref) < 5e-4, maxrel(got, ref)
+        # greedy generation from a prompt: the tokens are the argmax of the oracle's logits wherever that is not a near-tie
+        prompt = toks[:5]
+        gen = [int(g) for g in inf.generate(prompt, 8)]
+        lo = oracle_decode(c, model, fmt, prompt + gen[:-1], max_seq=64, precision="f32", lora=lora)[len(prompt) - 1:]
+        srt = np.sort(lo, axis=1)
+        clear = (srt[:, -1] - srt[:, -2]) > 1e-3 * np.abs(lo).max()
+        first_tie = len(gen) if clear.all() else int(np.argmin(clear))
+        assert first_tie >= 3 and (lo.argmax(1)[:first_tie] == np.asarray(gen)[:first_tie]).all()
+        if fmt == "f16":
+            # eight copies in lock step (the products on the matrix cores): every copy the single-sequence tokens
+            got8 = inf.generate_batch(prompt, 8, 8)
+            assert got8.shape == (8, 8)
+            for b in range(8):
+                assert np.array_equal(got8[b], got8[0])
+                assert [int(t) for t in got8[b, :first_tie]] == gen[:first_tie], b
+
+    if with_lora:
+        with SFTState(c, model) as sft:
+            with InferenceState(sft=sft, max_seq=64) as inf:
+                check(inf)
+    else:
+        with InferenceState(c, model, max_seq=64, use_fp16=(fmt == "f16")) as inf:
+            check(inf)
 
 
 def test_eos_ids_from_config_json(tmp_path, capfd):

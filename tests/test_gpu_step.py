@@ -91,6 +91,12 @@ CASES = [
     C1.with_(name="seq1100", NL=1, D=128, Hq=2, Hkv=1, hd=64, IS=256, V=512, seq=1100),             # by the rule: beyond 1024 keys
     # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
     TINY_GEMMA3.with_(name="gemma_many_rows", NL=2, batch=4, seq=128),
+    # products of up to 64 rows on F16 weights take gemm_ring by default; the register-staged streaming kernel that they
+    # took before (and that Q8_0 weights and several row tiles still take) on the same shapes
+    C1.with_(name="c1_tiled"),
+    TINY_GEMMA3.with_(name="gemma_tiled"),
+    C1.with_(name="wide_ffn_groups_tiled", NL=1, IS=4224, V=1024, seq=64),
+    C1.with_(name="ragged_seq40_tiled", NL=2, batch=2, seq=40, R=4, alpha=8.0),
 ]
 
 
@@ -117,6 +123,7 @@ def test_train_steps_match_oracle(cfg):
     # the "big_m" cases pin every product to the LDS-tiled large-M kernel (by itself it is only chosen for
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
     lib.load().hip_gemm_force_large_m(2 if "_lds" in cfg.name else 1 if "big_m" in cfg.name else 0)
+    lib.load().hip_gemm_ring(0 if cfg.name.endswith("_tiled") else 1)
     lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
     lib.load().hip_gemm_large_m_block(2 if "_wide" in cfg.name else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_attention_flash(1 if cfg.name.endswith("_flash") else 0 if cfg.name.endswith("_noflash") else -1)
