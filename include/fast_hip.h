@@ -57,6 +57,8 @@ size_t metal_buf_size(MetalBuf *b);
 /* Extension: the address kernels use for the buffer (device memory, or the device view of pinned host memory once
  * metal_buf_ptr was called).  For callers that pass plain device pointers to hip_attention_noalloc. */
 void *hip_buf_device_ptr(MetalBuf *b);
+/* free and total bytes of the current device's memory (hipMemGetInfo): lets a caller see that a call allocated nothing */
+void hip_mem_info(size_t *free_bytes, size_t *total_bytes);
 /* Non-owning window [offset, offset+size) of another buffer. */
 MetalBuf *metal_buf_view(MetalBuf *parent, size_t offset, size_t size);
 

@@ -18,8 +18,8 @@
  *  - Embedding gather, loss scaling, global-norm clipping and AdamW run on the
  *    device; the host touches only tokens, targets and the per-row losses.
  *
- * Limits (a constructor prints the reason and returns NULL, a product that does
- * not fit aborts with a message):
+ * Limits (sft_state_create_from_ref checks all of them before it uploads anything,
+ * prints the reason and returns NULL):
  *  - d_model, FFN width, vocabulary and head_dim multiples of 4; n_q_heads a
  *    multiple of n_kv_heads; Q8_0 additionally needs d_model, FFN width and
  *    n_q_heads * head_dim to be multiples of 32;

@@ -133,6 +133,14 @@ size_t metal_buf_size(MetalBuf *b) { return b ? b->size : 0; }
 
 void *hip_buf_device_ptr(MetalBuf *b) { return b ? lmhip::dptr(b) : nullptr; }
 
+void hip_mem_info(size_t *free_bytes, size_t *total_bytes)
+{
+    size_t f = 0, t = 0;
+    HIP_CHECK(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+}
+
 void *metal_buf_ptr(MetalBuf *b)
 {
     if (!b) return nullptr;

@@ -685,6 +685,22 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
         return nullptr;
     }
 
+    // upper limits of the row kernels (each would stop the process at its first launch, after all weights are uploaded)
+    {
+        const char *why = nullptr;
+        if (D > 12288 || IS > 12288) why = "d_model and the FFN width must be at most 12288 (a workgroup keeps a row in registers)";
+        else if (s->hd > 512) why = "head_dim must be at most 512";
+        else if ((long)(qd + 2 * kd + 2 * R + 16 * 32) * 4 > 64 * 1024) why = "(n_q_heads + 2 n_kv_heads) * head_dim + 2 rank must be at most 15872 (a row of dq | dk | dv | dh is staged in 64 KB of LDS)";
+        else if (seq_len > 4096) why = "seq_len must be at most 4096";
+        else if (batch < 1 || seq_len < 1 || NL < 1) why = "batch, seq_len and the number of layers must be positive";
+        if (why) {
+            fprintf(stderr, "[FastSFT] unsupported dims: %s\n", why);
+            delete s;
+            fast_metal_shutdown();
+            return nullptr;
+        }
+    }
+
     // ---- frozen weights: tiled arenas plus transposed images for the dX products ----
     // Q8_0 weights stay quantised when the fused QKV matrix splits into quantised and LoRA parts on tile
     // boundaries; otherwise (and in full-parameter mode, which rewrites the weights) they are stored as the

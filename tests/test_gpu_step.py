@@ -156,6 +156,18 @@ def test_train_steps_match_oracle(cfg):
     lib.load().hip_gemm_image_budget_mb(65536)
 
 
+@pytest.mark.parametrize("bad", [dict(hd=516, Hq=1, Hkv=1), dict(seq=4097), dict(Hq=120, Hkv=8, hd=128, D=256), dict(R=18)],
+                         ids=["head_dim_516", "seq_4097", "qkv_row_beyond_lds", "rank_18"])
+def test_dimensions_beyond_the_limits_are_refused_at_creation(bad, capfd):
+    """The limits of include/sft_hip.h: the constructor says which one and returns NULL (nothing uploaded, no abort at the
+    first launch)."""
+    cfg = C1.with_(name="refused", NL=1, V=256, **bad)
+    model = make_model(cfg, seed=3)
+    with pytest.raises(RuntimeError):
+        SFTState(cfg, model)
+    assert "unsupported dims" in capfd.readouterr().err
+
+
 def test_lm_head_backward_over_many_k_chunks():
     """512 rows and a 65 536-token vocabulary: the LM head's backward is four 128 x 256 blocks over K = 65 536, which the
     measured rule gives to the large-M kernel cut into eight K chunks (planes added by the consumer); the forward takes

@@ -44,6 +44,35 @@ def test_no_alloc_attention_matches_the_allocating_entry_point_on_consecutive_ca
         dev.close()
 
 
+def test_no_alloc_attention_leaves_device_memory_as_it_was():
+    """What the entry point exists for: between two readings of the device's free memory, calls at several sizes (with and
+    without slice partials) allocate nothing.  fast_metal_init has resolved the fixed array's address on this device
+    before, so the calls themselves resolve nothing either (a caller under graph capture must have initialised the
+    library on its device first)."""
+    import ctypes as C
+    dev = Dev()
+    try:
+        L = dev.L
+        rng = np.random.default_rng(12)
+        Hq, G, hd, max_seq = 32, 4, 128, 4096
+        Q = dev.up(rng.standard_normal(Hq * hd).astype(F))
+        Kc = dev.up(rng.standard_normal((Hq // G, max_seq, hd)).astype(F))
+        Vc = dev.up(rng.standard_normal((Hq // G, max_seq, hd)).astype(F))
+        out = dev.empty(Hq * hd * 4)
+        ptrs = [L.hip_buf_device_ptr(b.h) for b in (Q, Kc, Vc, out)]
+        L.metal_flush()
+        free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        L.hip_mem_info(C.byref(free0), C.byref(total))
+        for n_attend in (4096, 100, 2500, 257):
+            assert L.hip_attention_noalloc(*ptrs, n_attend, hd, max_seq, Hq, G) == 0
+        L.metal_flush()
+        L.hip_mem_info(C.byref(free1), C.byref(total))
+        assert free1.value == free0.value, (free0.value, free1.value)
+        assert np.isfinite(out.read(F)).all()
+    finally:
+        dev.close()
+
+
 def test_no_alloc_attention_refuses_what_does_not_fit(capfd):
     dev = Dev()
     try:
