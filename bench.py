@@ -26,23 +26,31 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFS = 2500.0          # dense fp16 MFMA
 
 
-TRAFFIC_SUMMARIES = {"c3_qwen3_4b_f16": ("c3_gemm_hbm_traffic_pmc.txt", "traffic_bytes_per_gemm_launch_c3"),
-                     "c4_qwen3_4b_q8": ("c4_gemm_hbm_traffic_pmc.txt", "traffic_bytes_per_gemm_launch_c4")}
+TRAFFIC_SUMMARIES = {"c3_qwen3_4b_f16": ("c3_gemm_hbm_traffic_pmc.txt", "c3"),
+                     "c2_gemma3_1b": ("c2_gemm_hbm_traffic_pmc.txt", "c2"),
+                     "c4_qwen3_4b_q8": ("c4_gemm_hbm_traffic_pmc.txt", "c4"),
+                     "c5_gemma3_1b_grpo": ("c5_step_hbm_traffic_pmc.txt", "c5")}
 
 
-def measured_traffic(cfg_name):
-    """HBM bytes per GEMM launch from the committed hardware-counter summary of this workload (two rocprofv3
-    --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by a copy kernel of known size), or None when there is none."""
+def measured_traffic(cfg_name, kernels):
+    """HBM bytes per timed launch from the committed hardware-counter summary of this workload (two rocprofv3
+    --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by a copy kernel of known size), or None when there is none, or when
+    the summary was made for another kernel than the one that runs now (its `traffic_kernel_*` line)."""
     if cfg_name not in TRAFFIC_SUMMARIES:
         return None
-    name, key = TRAFFIC_SUMMARIES[cfg_name]
+    name, tag = TRAFFIC_SUMMARIES[cfg_name]
     path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
         return None
+    value, kernel = None, None
     for line in open(path):
-        if line.startswith(key):
-            return float(line.split("=")[1])
-    return None
+        if line.startswith(f"traffic_bytes_per_gemm_launch_{tag}"):
+            value = float(line.split("=")[1])
+        if line.startswith(f"traffic_kernel_{tag}"):
+            kernel = line.split("=")[1].strip()
+    if kernel is not None and kernel not in kernels:
+        return None
+    return value
 
 
 def cpu_baseline(cfg, budget_s=20.0):
@@ -285,15 +293,18 @@ def main():
                 "frac": round(tfs / MFMA_PEAK_TFS if compute_bound else gbs / HBM_PEAK_GBS, 4), "traffic": None,
                 "kernel": ("gemm_big_q8<1>, gemm_big_q8<2>" if cfg.BN >= 1024 and cfg.weight_format != "f16" and args.q8_large_m == "unpack-in-lds" else
                            "gemm_big_f16_256, gemm_big_f16" if cfg.BN >= 1024 else
-                           "gemm_tiled + gemm_big_f16_256, gemm_big_f16" if compute_bound else "gemm_tiled"),
+                           # full-parameter pass: the products, the weight gradients (F16 read-modify-write of the accumulators), the
+                           # apply (W, G and the transposed image) and the operand transposes (time only) are timed together
+                           "gemm_tiled, gemm_big_f16*, k_wgrad, k_apply_retile, k_transpose_scaled_jobs" if cfg.R == 0 else
+                           "gemm_ring" if cfg.BN <= 64 and cfg.weight_format == "f16" and args.gemm_ring else "gemm_tiled"),
                 "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                 "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
                 "gemm_ms_per_step": round(tms.value / prof_steps, 3)}
-    roofline["traffic"] = measured_traffic(cfg.name)
+    roofline["traffic"] = measured_traffic(cfg.name, roofline["kernel"])
     roofline["traffic_source"] = (f"profiles/{TRAFFIC_SUMMARIES.get(cfg.name, ('',))[0]}: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, "
                                   "scaled by the same counters on a copy kernel of known size; not re-measured in this run"
-                                  if roofline["traffic"] is not None else "no hardware-counter summary is committed for this workload")
+                                  if roofline["traffic"] is not None else "no hardware-counter summary of the kernel that runs now is committed for this workload")
     st.free()
 
     metric = ("SFT train tokens/s, Qwen3-4B LoRA r16 seq64; % of HBM-BW / MFMA peak" if cfg.name == "c3_qwen3_4b_f16" else

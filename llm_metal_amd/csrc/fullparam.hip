@@ -18,6 +18,7 @@
 #include "devutil.h"
 #include "gemm.h"
 #include "fused.h"
+#include <hip/hip_ext.h>
 
 using namespace lmhip;
 
@@ -29,6 +30,14 @@ namespace {
 
 #define LAUNCH(kern, grid, block, lds, ...) do { \
     hipLaunchKernelGGL(kern, grid, block, lds, stream(), __VA_ARGS__); HIP_CHECK(hipGetLastError()); } while (0)
+// The same, timed with the products when per-launch events are being recorded (hip_gemm_profile_enable): `bytes` are the
+// HBM bytes the launch has to move at least (the F16 targets it reads and writes; operand transposes move none that the
+// step's arithmetic asks for, so their time counts and their bytes do not), `flops` its multiply-adds times two.
+#define LAUNCH_TIMED(bytes, flops, kern, grid, block, lds, ...) do { \
+    hipEvent_t ev_a_ = nullptr, ev_b_ = nullptr; \
+    if (gemm_prof_begin((bytes), (flops), &ev_a_, &ev_b_)) hipExtLaunchKernelGGL(kern, grid, block, lds, stream(), ev_a_, ev_b_, 0, __VA_ARGS__); \
+    else hipLaunchKernelGGL(kern, grid, block, lds, stream(), __VA_ARGS__); \
+    HIP_CHECK(hipGetLastError()); } while (0)
 
 // in:  tiled [T tokens, F features] fp16, value(t, f) = in[t][f] * in_inv[t]
 // out: tiled [F, T] fp16, value(f, t) = out[f][t] * out_inv[f]; zero in the K (token) padding and in
@@ -345,7 +354,7 @@ namespace lmhip {
 void launch_transpose_scaled(const half_t *in_tiled, const float *in_inv, int T, int F, half_t *out_tiled, float *out_inv)
 {
     if (T <= 0 || F <= 0) return;
-    LAUNCH(k_transpose_scaled, dim3(tiled_kb(F)), dim3(256), 0, reinterpret_cast<const half8 *>(in_tiled), in_inv, T, F,
+    LAUNCH_TIMED(0.0, 0.0, k_transpose_scaled, dim3(tiled_kb(F)), dim3(256), 0, reinterpret_cast<const half8 *>(in_tiled), in_inv, T, F,
            reinterpret_cast<half8 *>(out_tiled), out_inv);
 }
 
@@ -356,7 +365,7 @@ void launch_transpose_scaled_pair(const half_t *in0, const float *in0_inv, int F
     const TransposeJob j0{reinterpret_cast<const half8 *>(in0), in0_inv, F0, reinterpret_cast<half8 *>(out0), out0_inv};
     const TransposeJob j1{reinterpret_cast<const half8 *>(in1), in1_inv, F1, reinterpret_cast<half8 *>(out1), out1_inv};
     const int nb0 = tiled_kb(F0);
-    LAUNCH(k_transpose_scaled_pair, dim3(nb0 + tiled_kb(F1)), dim3(256), 0, j0, j1, T, nb0);
+    LAUNCH_TIMED(0.0, 0.0, k_transpose_scaled_pair, dim3(nb0 + tiled_kb(F1)), dim3(256), 0, j0, j1, T, nb0);
 }
 
 void launch_transpose_scaled_jobs(const TransposeOperand *ops, int n, int T)
@@ -372,7 +381,7 @@ void launch_transpose_scaled_jobs(const TransposeOperand *ops, int n, int T)
         total += tiled_kb(ops[i].F);
     }
     js.first[n] = total;
-    LAUNCH(k_transpose_scaled_jobs, dim3(total), dim3(256), 0, js, T);
+    LAUNCH_TIMED(0.0, 0.0, k_transpose_scaled_jobs, dim3(total), dim3(256), 0, js, T);
 }
 
 void launch_wgrads(const WgradOperands *w, int n, int T, int sgd, float lr)
@@ -390,8 +399,11 @@ void launch_wgrads(const WgradOperands *w, int n, int T, int sgd, float lr)
     }
     for (int i = n; i <= 4; i++) js.first[i] = total;
     const dim3 grid((total + 7) / 8 * 8);                 // whole rounds of the eight XCDs; k_wgrad maps ids to tiles
-    if (sgd) LAUNCH(k_wgrad<1>, grid, dim3(256), 0, js, tiled_kb(T), lr);
-    else     LAUNCH(k_wgrad<0>, grid, dim3(256), 0, js, tiled_kb(T), lr);
+    double weights = 0.0;
+    for (int i = 0; i < n; i++) weights += (double)w[i].M_out * w[i].N_in;
+    // the F16 target is read and written once: 4 bytes per weight
+    if (sgd) LAUNCH_TIMED(4.0 * weights, 2.0 * T * weights, k_wgrad<1>, grid, dim3(256), 0, js, tiled_kb(T), lr);
+    else     LAUNCH_TIMED(4.0 * weights, 2.0 * T * weights, k_wgrad<0>, grid, dim3(256), 0, js, tiled_kb(T), lr);
 }
 
 void launch_wgrad(const half_t *XT, const float *x_inv, const half_t *YT, const float *y_inv, half_t *target_tiled,
@@ -407,7 +419,9 @@ void launch_apply_retile(half_t *W_tiled, half_t *G_tiled, half_t *WT_tiled, int
 {
     if (M_out <= 0 || N_in <= 0 || matrices <= 0) return;
     if (matrices > 65535 || (stride & 7) || (strideT & 7)) { fprintf(stderr, "[fast_hip] apply_retile: bad strides\n"); abort(); }
-    LAUNCH(k_apply_retile, dim3(tiled_kb(N_in), (tiled_rb(M_out) + 1) / 2, matrices), dim3(256), 0, reinterpret_cast<half8 *>(W_tiled),
+    // W read and written, the transposed image written, and with an accumulator G read and cleared: 10 (6) bytes per weight
+    const double weights = (double)M_out * N_in * matrices;
+    LAUNCH_TIMED((G_tiled ? 10.0 : 6.0) * weights, 0.0, k_apply_retile, dim3(tiled_kb(N_in), (tiled_rb(M_out) + 1) / 2, matrices), dim3(256), 0, reinterpret_cast<half8 *>(W_tiled),
            reinterpret_cast<half8 *>(G_tiled), reinterpret_cast<half8 *>(WT_tiled), M_out, N_in, lr, stride / 8, strideT / 8);
 }
 
