@@ -53,6 +53,42 @@ def measured_traffic(cfg_name, kernels):
     return value
 
 
+def gemm_shapes(cfg, L):
+    """One line per product shape of a LoRA step at cfg.BN rows (F16 weights): microseconds per launch, launched back to
+    back on the library's stream with the weights rotated through more than 1 GB (nothing is found in a cache), for
+    (a) the weight loads of gemm_ring alone on its grid, (b) gemm_ring, (c) gemm_tiled; and a fit  t = t0 + bytes / rate
+    over the layer shapes.  An empty kernel launched the same way takes about 3 us, which every figure includes."""
+    import ctypes as C
+    D, qd, kd, IS, V, R = cfg.D, cfg.Hq * cfg.hd, cfg.Hkv * cfg.hd, cfg.IS, cfg.V, cfg.R
+    nq = qd + 2 * kd + 2 * R
+    shapes = [("qkv forward", nq, D), ("o forward", D, qd), ("gate|up forward", 2 * IS, D), ("down forward", D, IS),
+              ("down backward", IS, D), ("gate|up backward", D, 2 * IS), ("o backward", qd, D), ("qkv backward", D, nq),
+              ("lm_head forward", V, D), ("lm_head backward", D, V)]
+    rows = []
+    for name, N, K in shapes:
+        nb, S = C.c_int(0), C.c_int(0)
+        it = 20 if N * K > 2e8 else 100
+        L.hip_gemm_ring(1)
+        t_read = L.hip_gemm_time_shape(cfg.BN, N, K, -1, 0, 0, it, C.byref(nb), C.byref(S)) * 1e3
+        t_ring = L.hip_gemm_time_shape(cfg.BN, N, K, 0, 0, 0, it, C.byref(nb), C.byref(S)) * 1e3
+        s_ring = S.value
+        L.hip_gemm_ring(0)
+        t_tiled = L.hip_gemm_time_shape(cfg.BN, N, K, 0, 0, 0, it, C.byref(nb), C.byref(S)) * 1e3
+        s_tiled = S.value
+        L.hip_gemm_ring(1)
+        mb = 2.0 * N * K / 1e6
+        rows.append({"product": name, "N": N, "K": K, "MB": round(mb, 1), "weights_only_us": round(t_read, 2), "gemm_ring_us": round(t_ring, 2),
+                     "ring_chunks": s_ring, "gemm_tiled_us": round(t_tiled, 2), "tiled_chunks": s_tiled,
+                     "weights_only_GBs": round(mb / t_read * 1e3), "gemm_ring_GBs": round(mb / t_ring * 1e3), "gemm_tiled_GBs": round(mb / t_tiled * 1e3)})
+    layer = rows[:8]
+    x = np.array([r["MB"] for r in layer]); fits = {}
+    for key in ("weights_only_us", "gemm_ring_us", "gemm_tiled_us"):
+        y = np.array([r[key] for r in layer])
+        slope, t0 = np.polyfit(x, y, 1)
+        fits[key] = {"t0_us": round(float(t0), 2), "rate_GBs": round(1e3 / float(slope))}
+    print(json.dumps({"workload": cfg.name, "rows": cfg.BN, "shapes": rows, "fit_over_layer_shapes": fits}))
+
+
 def cpu_baseline(cfg, budget_s=20.0):
     """Times the CPU oracle (scalar port of the reference's arithmetic, 1 thread) on a bounded
     sample of the same workload: the full step on a model with fewer layers and a truncated
@@ -190,6 +226,8 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=16)
     ap.add_argument("--decode-batch", type=int, default=0,
                     help="with --decode: also time this many copies of one prompt decoded in lock step")
+    ap.add_argument("--gemm-shapes", action="store_true",
+                    help="time every product shape of the configuration alone, with cold weights: the weight loads only, gemm_ring, gemm_tiled")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the library's plain copy kernel (1 GiB in, 1 GiB out, 5 launches): "
                          "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
@@ -223,6 +261,8 @@ def main():
 
     if args.decode:
         return decode_bench(args, cfg, L)
+    if args.gemm_shapes:
+        return gemm_shapes(cfg, L)
 
     t0 = time.perf_counter()
     model = make_model(cfg, seed=0, lora_b_std=0.0)          # timing runs: B = 0 as the reference initialises it

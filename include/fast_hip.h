@@ -190,7 +190,7 @@ int  hip_gemm_profile_read(double *total_ms, double *total_weight_bytes);
 int  hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double *total_flops);
 /* Microbenchmark of the GEMM alone at one shape (M rows, N x K weight) on synthetic operands,
  * rotating through > 1 GB of distinct weight images.  nb / S = 0: planner's choice, else forced
- * tile height (1, 2; 128 = the large-M kernel) and K split (for the large-M kernel: K chunks, F16 tiles only).  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
+ * tile height (1, 2; 128 = the large-M kernel; -1 = no product at all, only the weight loads of gemm_ring on its grid) and K split (for the large-M kernel: K chunks, F16 tiles only).  wf: weight format, 0 F16, 1 Q8_0 with row scales (forward image),
  * 2 Q8_0 with column scales (transposed image).  Returns average ms per launch. */
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S);
 

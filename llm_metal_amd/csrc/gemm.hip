@@ -700,6 +700,8 @@ int hip_gemm_profile_read2(double *total_ms, double *total_weight_bytes, double 
 // Returns the average milliseconds per launch.
 double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters, int *used_nb, int *used_S)
 {
+    const bool read_only = nb == -1;                       // the weight loads of gemm_ring alone (ring_weights_only)
+    if (read_only) nb = 0;
     g_force_nb = nb == 128 ? 0 : nb; g_force_S = S;
     GemmPlan p = plan_gemm(M, N, K, 0, wf);
     g_force_nb = 0; g_force_S = 0;
@@ -735,7 +737,11 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters
     };
     const bool big = nb == 128;                            // nb = 128 selects the large-M kernel (one launch, 128-row blocks)
     auto run = [&](int i) {
-        if (big) launch_gemm_big((half_t *)A, (float *)inv, op(i), (float *)P, N, M, N, K, S > 0 ? S : 1, (size_t)M * N);
+        if (read_only && p.ring) {
+            GemmKArgs g{};
+            g.W = op(i); g.P = (float *)P; g.Nb = tiled_rb(N); g.Kb = tiled_kb(K); g.steps_per_chunk = p.steps; g.n_tiles = p.n_tiles; g.S = p.S;
+            hipLaunchKernelGGL((ring_weights_only<2>), dim3((unsigned)(p.n_tiles * p.S)), dim3(512), 0, stream(), g);
+        } else if (big) launch_gemm_big((half_t *)A, (float *)inv, op(i), (float *)P, N, M, N, K, S > 0 ? S : 1, (size_t)M * N);
         else launch_gemm((half_t *)A, nullptr, op(i), (float *)P, N, (size_t)M * N, M, N, K, p);
     };
     for (int i = 0; i < 3; i++) run(i);

@@ -360,4 +360,36 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(GemmKArgs g)
     }
 }
 
+// The weight loads of gemm_ring alone, on the same grid and through the same LDS ring: what a launch needs just to pull its
+// weight bytes into LDS (timing reference for the product; nothing is multiplied or stored).
+template <int KG>
+__global__ __launch_bounds__(256 * KG) void ring_weights_only(GemmKArgs g)
+{
+    __shared__ half8 ring[2 * KG * 1024];
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int q = wv & 3, kg = wv >> 2;
+    const int tile = blockIdx.x % g.n_tiles, chunk = blockIdx.x / g.n_tiles;
+    const int kb_beg = chunk * g.steps_per_chunk;
+    const int nsteps = min(g.Kb, kb_beg + g.steps_per_chunk) - kb_beg;
+    const int rounds = (nsteps + KG - 1) / KG;
+    if (q >= 2) return;
+    const half8 *src = reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(2 * tile + q, g.Nb - 1) * g.Kb + kb_beg) * 256 + lane;
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)ring;
+    auto request = [&](int round) __attribute__((always_inline)) {
+        const int step = min(round * KG + kg, nsteps - 1);
+        const uint32_t sb = base + (uint32_t)(((round & 1) * KG + kg) * 16384 + q * 4096);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src + (size_t)step * 256 + j * 64), "s"(sb + (uint32_t)(j * 1024)) : "m0", "memory");
+    };
+    request(0);
+    if (rounds > 1) request(1);
+    for (int rd = 0; rd < rounds; rd++) {
+        if (rd + 1 < rounds) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");    // four loads per round and wave, as in gemm_ring
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (rd + 2 < rounds) request(rd + 2);
+    }
+    if (ring[lane][0] == (half_t)12345.0f) g.P[0] = 1.f;   // the loads have a use
+}
+
 }  // namespace lmhip
