@@ -300,13 +300,16 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
     for (int u = 0; u < 3; u++)
 #pragma unroll
         for (int j = 0; j < 2; j++) loff[u][j] = __builtin_amdgcn_readfirstlane((uint32_t)((dst[u] * 2 + j) * 64 * 16));
+    constexpr int LOADS = 3 * 2, AHEAD = 5, LANDED = 2;   // copies per request and wave; requests in flight after a request; how many of them a barrier needs
+    constexpr int WAIT = (AHEAD - LANDED) * LOADS;
+    static_assert(WAIT == 18 && AHEAD * LOADS < 64, "the hand-written waits count this wave's LDS-direct loads; vmcnt has six bits");
     auto request = [&](half8 (&buf)[HB], int hs) __attribute__((always_inline)) {
         const size_t o = (size_t)(hs >> 1) * 256 + (hs & 1) * 128;
         const uint32_t base = (uint32_t)(uintptr_t)(lds_void *)buf;
 #pragma unroll
         for (int u = 0; u < 3; u++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < 2; j++)                    // LOADS of these
                 asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[u] + o + j * 64), "s"(base + loff[u][j]) : "m0");
     };
     half8 a0[2], w0[4];
@@ -335,10 +338,12 @@ __global__ __launch_bounds__(256) void gemm_big_f16(GemmKArgs g)
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (i < 4 || (i >= 8 && i < 14)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // In flight here: this wave's copies of half steps hs + 1 .. hs + 5, LOADS each, oldest first.  The barrier must find
+        // hs + 1 and hs + 2 in LDS, so all but the newest three requests have to have retired (loads retire in order).
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(WAIT) : "memory");
     };
     request(lb0, 0); request(lb1, min(1, last)); request(lb2, min(2, last)); request(lb3, min(3, last)); request(lb4, min(4, last));
-    asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(WAIT) : "memory");   // five requests out: the first two have landed
     read(a0, w0, lb0, 0);
     const int full = nhalf / 6 * 6;
     for (int h0 = 0; h0 < full; h0 += 6) {
@@ -454,6 +459,9 @@ __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
             for (int j = 0; j < 2; j++)
                 asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[u] + o + j * 64), "s"(base + loff[u][j]) : "m0");
     };
+    constexpr int LOADS = 4 * 2, AHEAD = 4, LANDED = 2;    // copies per request and wave; requests in flight after a request; how many a barrier needs
+    constexpr int WAIT = (AHEAD - LANDED) * LOADS;
+    static_assert(WAIT == 16 && AHEAD * LOADS < 64, "the hand-written waits count this wave's LDS-direct loads; vmcnt has six bits");
     half8 a0[4], w0[4];                                    // fragments of slice 0 of the half step about to be multiplied
     auto read = [&](half8 (&a)[4], half8 (&w)[4], const half8 (&cur)[HB], int j) __attribute__((always_inline)) {
 #pragma unroll
@@ -484,10 +492,11 @@ __global__ __launch_bounds__(256) void gemm_big_f16_256(GemmKArgs g)
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (i < 6 || (i >= 16 && i < 24)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // in flight: this wave's copies of hs + 1 .. hs + 4, 8 each (4 pieces x 2 slices); hs + 1 and hs + 2 must have landed
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(WAIT) : "memory");
     };
     request(lb0, 0); request(lb1, min(1, last)); request(lb2, min(2, last)); request(lb3, min(3, last));
-    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(WAIT) : "memory");   // four requests out: the first two have landed
     read(a0, w0, lb0, 0);
     const int full = nhalf / 5 * 5;
     for (int h0 = 0; h0 < full; h0 += 5) {
@@ -554,6 +563,10 @@ template <int WF, int BM, bool TAIL = false>
 __global__ __launch_bounds__(256) void gemm_big_q8(GemmKArgs g)
 {
     constexpr int AB = BM / 32, MI = BM / 64, AU = BM / 128;  // A row blocks per block; accumulator tile rows and A pieces per wave
+    // LDS-direct copies a wave issues per request (2 per A piece; 2 weight pieces + 2 scale pieces, or 4 F16 pieces), requests
+    // in flight after a request (six buffers), and how many of them a barrier needs in LDS: the hand-written waits below
+    constexpr int Q8_LOADS = 2 * AU + 4, Q8_AHEAD = 5, Q8_LANDED = 2, Q8_WAIT = (Q8_AHEAD - Q8_LANDED) * Q8_LOADS;
+    static_assert(Q8_WAIT == (BM == 256 ? 24 : 18) && Q8_AHEAD * Q8_LOADS < 64, "the waits count this wave's LDS-direct loads; vmcnt has six bits");
     constexpr int HB = (2 * AB + 8) * 64;                 // 16-byte units per buffer: A [AB blocks][2 slices][64], Wq [8 blocks][64]
     __shared__ uint4v lb0[HB], lb1[HB], lb2[HB], lb3[HB], lb4[HB], lb5[HB];
     __shared__ half_t scl[6][8][128];                      // scales of the weight row blocks of the half step in buffer i
@@ -675,14 +688,13 @@ __global__ __launch_bounds__(256) void gemm_big_q8(GemmKArgs g)
         multiply(a0, w0);
         read(a0, w0, nxt, nslot, (hs + 1) & 1, 0);
         multiply(a1, w1);
-        if (BM == 256) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // in flight: this wave's copies of hs + 1 .. hs + 5, Q8_LOADS each; hs + 1 and hs + 2 must have landed
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(Q8_WAIT) : "memory");
     };
     if (nhalf > 0) {
         request(lb0, 0, 0); request(lb1, 1, min(1, last)); request(lb2, 2, min(2, last)); request(lb3, 3, min(3, last));
         request(lb4, 4, min(4, last));
-        if (BM == 256) asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(18)\n\ts_barrier" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(Q8_WAIT) : "memory");   // five requests out: the first two have landed
         read(a0, w0, lb0, 0, 0, 0);
         const int full = nhalf / 6 * 6;
         for (int h0 = 0; h0 < full; h0 += 6) {

@@ -275,7 +275,11 @@ WeightOp resident_image(SFTState *s, const WeightOp &W, int N, int K)
     auto it = s->img_slots.find(W.q);
     if (it != s->img_slots.end()) return f16_image_of(W, N, K, at<half_t>(it->second), true);
     const size_t bytes = tiled_elems(N, K) * sizeof(half_t);
-    if (s->img_bytes + bytes > g_image_budget) return f16_image_of(W, N, K);   // no room: this weight's image is made per product
+    // no room in the budget, or on the device (2 GB kept free for everything allocated later): this weight's image is
+    // made per product in the scratch arena instead
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    if (s->img_bytes + bytes > g_image_budget || free_b < bytes + ((size_t)2 << 30)) return f16_image_of(W, N, K);
     MetalBuf *slot = metal_buf_create(bytes);
     s->img_bytes += bytes;
     s->img_slots.emplace(W.q, slot);
