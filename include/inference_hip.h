@@ -54,9 +54,17 @@ int inference_generate(InferenceState *state, const uint32_t *prompt_tokens, int
  * for all of them.  Runs with its own KV caches (the state's position and cache are left alone); F16 weights only and
  * batch_size <= 32, as in the reference, but for either model type and with the state's adapters.  A sequence ends at
  * one of the state's EOS ids or at token 0 (:944-947); the loop ends when all have.  output_tokens: [batch_size][max_gen_len].
- * Returns the number of tokens written per sequence (0: arguments refused). */
+ * Returns the number of tokens written per sequence (0: arguments refused).  The batch's caches and scratch stay with
+ * the state until inference_state_free or a call with another batch_size, so repeated calls allocate nothing. */
 int inference_generate_batch(InferenceState *state, const uint32_t *prompt_tokens, int prompt_len, uint32_t *output_tokens,
                              int max_gen_len, int batch_size);
+
+/* One lock-step step of the same batch path with a token of its own per sequence -- the call a sampling caller makes
+ * where the reference's forward_token_batch (src/nn/fast_inference.c:808-893, static there) takes tokens_b[b]; no
+ * public counterpart in the reference.  tokens[b] enters sequence b at position pos; logits ([batch_size][vocab], host)
+ * may be NULL.  pos = 0 starts new sequences; otherwise pos must follow the step before on the same batch_size (a step
+ * of this call or the end of inference_generate_batch).  Returns 0, -1 when the arguments do not fit. */
+int inference_step_batch(InferenceState *state, const int *tokens, int batch_size, int pos, float *logits);
 
 ModelType inference_state_model_type(InferenceState *state);         /* src/nn/fast_inference.h:31 */
 int  inference_state_vocab_size(InferenceState *state);              /* src/nn/fast_inference.h:34 */

@@ -25,6 +25,11 @@ using namespace lmhip;
 
 extern "C" MetalBuf *sft_get_token_emb_buf(SFTState *s);
 
+namespace {
+struct BatchRun;
+void batch_release(BatchRun *r);
+}
+
 struct InferenceState {
     int D, Hq, Hkv, hd, IS, V, NL, max_seq, cur_len, use_fp16;
     ModelType model_type;
@@ -49,6 +54,7 @@ struct InferenceState {
     int R;
     float scaling;
     MetalBuf *lora_t;                    // [2R]: A_q ln | A_v ln
+    BatchRun *batch;                     // scratch and caches of the lock-step batch path, kept from call to call (NULL until used)
 };
 
 namespace {
@@ -596,6 +602,7 @@ void inference_state_free(InferenceState *s)
 {
     if (!s) return;
     metal_flush();
+    batch_release(s->batch);
     for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->x2, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t, s->rope_tabs})
         metal_buf_free(b);
     for (MetalBuf *b : s->kc) metal_buf_free(b);
@@ -706,19 +713,21 @@ __global__ __launch_bounds__(AM_WGS) void k_argmax_final_batch(const float *__re
 
 // Scratch and KV caches of a batch of B sequences decoded in lock step (BatchState of src/nn/fast_inference.c:699-776).
 struct BatchRun {
-    int B;
+    int B, R, len;                                                       // sequences; adapter rank the scratch was sized for; positions held by the caches
     MetalBuf *x, *ln, *qkv, *att, *act, *logits, *best, *lora_t;
     MetalBuf *a16, *inv_ln, *inv_br, *planes;                            // a product's operand, its factors (of ln | of att and act), its planes
     std::vector<MetalBuf *> kc, vc;                                      // per layer: [B][Hkv, max_seq, hd]
     int *best_host;
 };
 
-void batch_free(BatchRun &r)
+void batch_release(BatchRun *r)
 {
-    for (MetalBuf *b : {r.x, r.ln, r.qkv, r.att, r.act, r.logits, r.best, r.lora_t, r.a16, r.inv_ln, r.inv_br, r.planes}) metal_buf_free(b);
-    for (MetalBuf *b : r.kc) metal_buf_free(b);
-    for (MetalBuf *b : r.vc) metal_buf_free(b);
-    if (r.best_host) hipHostFree(r.best_host);
+    if (!r) return;
+    for (MetalBuf *b : {r->x, r->ln, r->qkv, r->att, r->act, r->logits, r->best, r->lora_t, r->a16, r->inv_ln, r->inv_br, r->planes}) metal_buf_free(b);
+    for (MetalBuf *b : r->kc) metal_buf_free(b);
+    for (MetalBuf *b : r->vc) metal_buf_free(b);
+    if (r->best_host) hipHostFree(r->best_host);
+    delete r;
 }
 
 // One step for B tokens at the same position: forward_token_batch, src/nn/fast_inference.c:808-893.  Every product
@@ -805,6 +814,51 @@ void argmax_batch(InferenceState *s, BatchRun &r, int *out)
     for (int b = 0; b < r.B; b++) out[b] = r.best_host[b];
 }
 
+// The state's batch run for B sequences: the one kept from the call before when that had the same B and rank (its buffers
+// are strided by B), else a new one in its place.  Caches are not cleared: a step at position pos reads what steps
+// 0..pos-1 of the same run wrote.
+BatchRun &batch_acquire(InferenceState *s, int B)
+{
+    const int R = s->lora.empty() ? 0 : s->R;
+    if (s->batch && s->batch->B == B && s->batch->R == R) return *s->batch;
+    metal_flush();
+    batch_release(s->batch);
+    s->batch = new BatchRun{};
+    BatchRun &r = *s->batch;
+    const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS, V = s->V;
+    r.B = B; r.R = R; r.len = 0;
+    r.x = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
+    r.qkv = fbuf((size_t)B * (qd + 2 * kd)); r.att = fbuf((size_t)B * qd);
+    r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
+    size_t a16_elems = 0, plane_floats = 0;                              // the largest operand and planes of the step's products
+    const int shapes[5][2] = {{qd + 2 * kd, D}, {D, qd}, {2 * IS, D}, {D, IS}, {V, D}};
+    for (const auto &nk : shapes) {
+        a16_elems = std::max(a16_elems, tiled_elems(2 * B, nk[1]));
+        for (int ring = 0; ring < 2; ring++) {                           // either kernel policy may be switched in later
+            const int was = gemm_ring_enabled();
+            set_gemm_ring(ring);
+            plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1]).S * 2 * B * nk[0]);
+            set_gemm_ring(was);
+        }
+    }
+    r.a16 = metal_buf_create(a16_elems * sizeof(half_t)); r.planes = fbuf(plane_floats);
+    r.inv_ln = fbuf((size_t)2 * B); r.inv_br = fbuf((size_t)2 * B);
+    r.best = metal_buf_create(((size_t)B + (size_t)B * 2 * AM_WGS) * sizeof(int));
+    r.lora_t = R ? fbuf((size_t)B * 2 * R) : nullptr;
+    HIP_CHECK(hipHostMalloc((void **)&r.best_host, (size_t)B * sizeof(int), hipHostMallocDefault));
+    const size_t cache_bytes = (size_t)s->Hkv * s->max_seq * s->hd * sizeof(float);
+    for (int L = 0; L < s->NL; L++) { r.kc.push_back(metal_buf_create(cache_bytes * B)); r.vc.push_back(metal_buf_create(cache_bytes * B)); }
+    return r;
+}
+
+bool batch_args_ok(InferenceState *s, int B)
+{
+    if (!s->use_fp16) { fprintf(stderr, "[BatchGen] F16 weights only\n"); return false; }
+    if (B < 1 || B > 32) return false;
+    if (s->D > 8192) { fprintf(stderr, "[BatchGen] hidden size %d not supported (<= 8192)\n", s->D); return false; }
+    return true;
+}
+
 }  // namespace
 
 // qwen3_generate_fast_batch, src/nn/fast_inference.c:895-1000, on a state's weights: batch_size copies of one prompt are
@@ -817,31 +871,10 @@ int inference_generate_batch(InferenceState *s, const uint32_t *prompt_tokens, i
                              int max_gen_len, int batch_size)
 {
     const int B = batch_size;
-    if (!s->use_fp16) { fprintf(stderr, "[BatchGen] F16 weights only\n"); return 0; }
-    if (B < 1 || B > 32 || prompt_len <= 0 || max_gen_len <= 0 || prompt_len > s->max_seq) return 0;
-    if (s->D > 8192) { fprintf(stderr, "[BatchGen] hidden size %d not supported (<= 8192)\n", s->D); return 0; }
+    if (!batch_args_ok(s, B) || prompt_len <= 0 || max_gen_len <= 0 || prompt_len > s->max_seq) return 0;
     for (int i = 0; i < prompt_len; i++)
         if (prompt_tokens[i] >= (uint32_t)s->V) { fprintf(stderr, "[BatchGen] token %u outside the vocabulary (%d)\n", prompt_tokens[i], s->V); return 0; }
-    const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS, V = s->V;
-    BatchRun r{};
-    r.B = B;
-    r.x = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
-    r.qkv = fbuf((size_t)B * (qd + 2 * kd)); r.att = fbuf((size_t)B * qd);
-    r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
-    size_t a16_elems = 0, plane_floats = 0;                              // the largest operand and planes of the step's products
-    const int shapes[5][2] = {{qd + 2 * kd, D}, {D, qd}, {2 * IS, D}, {D, IS}, {V, D}};
-    for (const auto &nk : shapes) {
-        a16_elems = std::max(a16_elems, tiled_elems(2 * B, nk[1]));
-        plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1]).S * 2 * B * nk[0]);
-    }
-    r.a16 = metal_buf_create(a16_elems * sizeof(half_t)); r.planes = fbuf(plane_floats);
-    r.inv_ln = fbuf((size_t)2 * B); r.inv_br = fbuf((size_t)2 * B);
-    r.best = metal_buf_create(((size_t)B + (size_t)B * 2 * AM_WGS) * sizeof(int));
-    r.lora_t = s->lora.empty() ? nullptr : fbuf((size_t)B * 2 * s->R);
-    HIP_CHECK(hipHostMalloc((void **)&r.best_host, (size_t)B * sizeof(int), hipHostMallocDefault));
-    const size_t cache_bytes = (size_t)s->Hkv * s->max_seq * s->hd * sizeof(float);
-    for (int L = 0; L < s->NL; L++) { r.kc.push_back(metal_buf_create(cache_bytes * B)); r.vc.push_back(metal_buf_create(cache_bytes * B)); }
-
+    BatchRun &r = batch_acquire(s, B);
     int tokens[32], next[32], active[32];
     for (int i = 0; i < prompt_len; i++) {                               // prefill: the same token for every sequence (:910-916)
         for (int b = 0; b < B; b++) tokens[b] = (int)prompt_tokens[i];
@@ -866,9 +899,30 @@ int inference_generate_batch(InferenceState *s, const uint32_t *prompt_tokens, i
         for (int b = 0; b < B; b++) output_tokens[(size_t)b * max_gen_len + n_gen] = (uint32_t)next[b];
         n_gen++;
     }
-    metal_flush();
-    batch_free(r);
+    r.len = cur_len;
     return n_gen;
+}
+
+// One lock-step step with a token of its own for every sequence (what forward_token_batch, src/nn/fast_inference.c:808-893,
+// is given by a sampling caller): tokens[b] enters sequence b at position pos, logits [batch_size][vocab] come back when
+// `logits` is not NULL.  Positions run 0, 1, 2, ... on the state's kept batch caches; pos = 0 starts new sequences, any
+// other pos must be the one after the step before (of this call or of inference_generate_batch with the same batch_size).
+// Returns 0, or -1 when the arguments do not fit.
+int inference_step_batch(InferenceState *s, const int *tokens, int batch_size, int pos, float *logits)
+{
+    const int B = batch_size;
+    if (!s || !tokens || !batch_args_ok(s, B) || pos < 0 || pos >= s->max_seq) return -1;
+    for (int b = 0; b < B; b++)
+        if (tokens[b] < 0 || tokens[b] >= s->V) { fprintf(stderr, "[BatchGen] token %d outside the vocabulary (%d)\n", tokens[b], s->V); return -1; }
+    BatchRun &r = batch_acquire(s, B);
+    if (pos != 0 && pos != r.len) { fprintf(stderr, "[BatchGen] step at position %d, but the batch's caches hold %d\n", pos, r.len); return -1; }
+    forward_token_batch(s, r, tokens, pos);
+    r.len = pos + 1;
+    if (logits) {
+        HIP_CHECK(hipMemcpyAsync(logits, dptr(r.logits), (size_t)B * s->V * sizeof(float), hipMemcpyDeviceToHost, stream()));
+        HIP_CHECK(hipStreamSynchronize(stream()));
+    }
+    return 0;
 }
 
 void inference_state_set_eos(InferenceState *s, const int *eos_tokens, int n_eos)

@@ -141,6 +141,7 @@ def load():
         "inference_state_create_from_ref": (vp, [C.POINTER(SFTModelRef), i, i]),
         "inference_state_create_from_sft": (vp, [vp, i]), "inference_state_refresh_from_sft": (None, [vp]),
         "inference_state_free": (None, [vp]), "inference_generate": (i, [vp, vp, i, vp, i]), "inference_generate_batch": (i, [vp, vp, i, vp, i, i]),
+        "inference_step_batch": (i, [vp, vp, i, i, vp]),
         "inference_state_model_type": (i, [vp]), "inference_state_vocab_size": (i, [vp]),
         "inference_state_reset": (None, [vp]), "inference_forward_token": (C.POINTER(C.c_float), [vp, i]),
         "inference_forward_token_argmax": (i, [vp, i]), "inference_state_set_lora": (None, [vp, vp]),

@@ -283,6 +283,14 @@ class InferenceState:
         n = self.L.inference_generate_batch(self.h, _vp(prompt), len(prompt), _vp(out), max_gen_len, batch)
         return out[:, :n]
 
+    def step_batch(self, tokens, pos, want_logits=True):
+        """One lock-step step with a token per sequence at position `pos`; [batch, V] logits (None if not asked for)."""
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        out = np.empty((len(t), self.V), dtype=np.float32) if want_logits else None
+        if self.L.inference_step_batch(self.h, _vp(t), len(t), int(pos), _vp(out) if want_logits else None) != 0:
+            raise RuntimeError("inference_step_batch refused its arguments")
+        return out
+
     def set_eos(self, ids):
         a = np.ascontiguousarray(ids, dtype=np.int32)
         self.L.inference_state_set_eos(self.h, _vp(a), len(a))

@@ -126,6 +126,46 @@ def test_batched_generation_decodes_every_copy_like_the_single_sequence(cfg, wit
             assert q8.generate_batch(prompt, n, 2).shape[1] == 0       # F16 weights only, as in the reference
 
 
+@pytest.mark.parametrize("with_lora", [False, True], ids=["plain", "adapters"])
+def test_batch_steps_with_a_token_of_their_own_per_sequence(with_lora):
+    """inference_step_batch: sequence b of a lock-step batch is fed its own tokens (forward_token_batch with distinct
+    tokens_b, src/nn/fast_inference.c:808-893).  Each sequence's logits must match the single-sequence path run on that
+    sequence alone, to the 22 bits the batched products keep of the activations; the batch's caches survive from call to
+    call, and a greedy batch run afterwards reuses them without disturbing its result."""
+    say("batch steps with distinct tokens", with_lora)
+    c = C1.with_(seq=8)
+    model = make_model(c, seed=31, gamma_jitter=0.1)
+    B, n = 4, 9
+    seqs = np.random.default_rng(32).integers(1, c.V, (B, n))
+
+    def check(inf):
+        greedy_before = inf.generate_batch([int(t) for t in seqs[0, :3]], 5, B)
+        batch_logits = np.stack([inf.step_batch(seqs[:, i], i) for i in range(n)], axis=1)      # [B, n, V]
+        for b in range(B):
+            inf.reset()
+            single = np.stack([inf.forward_token(int(t)) for t in seqs[b]])
+            assert maxrel(batch_logits[b], single) < 1e-4, b
+        # a step that does not follow the one before is refused; pos = 0 restarts
+        with pytest.raises(RuntimeError):
+            inf.step_batch(seqs[:, 0], n + 3)
+        again = inf.step_batch(seqs[:, 0], 0)
+        assert np.array_equal(again, batch_logits[:, 0])
+        with pytest.raises(RuntimeError):
+            inf.step_batch([c.V] * B, 1)
+        assert np.array_equal(inf.generate_batch([int(t) for t in seqs[0, :3]], 5, B), greedy_before)
+        # another batch size takes new caches
+        two = inf.step_batch(seqs[:2, 0], 0)
+        assert maxrel(two, batch_logits[:2, 0]) < 1e-4
+
+    if with_lora:
+        with SFTState(c, model) as sft:
+            with InferenceState(sft=sft, max_seq=32) as inf:
+                check(inf)
+    else:
+        with InferenceState(c, model, max_seq=32, use_fp16=True) as inf:
+            check(inf)
+
+
 # Qwen3-4B's widths (hidden 2560, 32 / 8 heads of 128, FFN 9728): the instantiations that `bench.py --decode` launches --
 # two weight rows per wave with the SiLU gate and the norm inside the launch at 19456 x 2560, the norm-fused Q|K|V
 # product at 6144 x 2560, the attention kernel with four-key steps, the fused per-head prologue and the O weights asked
