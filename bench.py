@@ -143,13 +143,18 @@ def decode_bench(args, cfg, L):
     """Greedy generation, one token per step; the matrix-vector kernel is the dominant kernel and every one of its
     launches is timed with HIP events on the library's stream in a second pass."""
     import ctypes as C
-    from llm_metal_amd.sft import InferenceState
+    from llm_metal_amd.sft import InferenceState, SFTState
     f16 = cfg.weight_format == "f16"
     t0 = time.perf_counter()
     model = make_model(cfg, seed=0)
     t_gen = time.perf_counter() - t0
     max_seq = args.prompt_len + args.warmup + 2 * args.steps + 8
-    inf = InferenceState(cfg, model, max_seq=max_seq, use_fp16=f16)
+    sft = None
+    if args.decode_from_sft:                               # the generation state reads the training state's tiles in place
+        sft = SFTState(cfg, model)
+        inf = InferenceState(sft=sft, max_seq=max_seq)
+    else:
+        inf = InferenceState(cfg, model, max_seq=max_seq, use_fp16=f16)
     t_init = time.perf_counter() - t0 - t_gen
     del model
     rng = np.random.default_rng(3)
@@ -172,12 +177,12 @@ def decode_bench(args, cfg, L):
     n = L.hip_gemm_profile_read2(C.byref(tms), C.byref(wb), C.byref(fl))
     L.hip_gemm_profile_enable(0)
     batch = None
-    if args.decode_batch > 1 and f16:
+    if args.decode_batch > 1 and (f16 or sft is not None):
         # the same prompt decoded in lock step by `decode_batch` copies (qwen3_generate_fast_batch); a never-emitted EOS id
-        # keeps every copy going; the timed call includes the prefill of its prompt and the allocation of its caches
+        # keeps every copy going; the timed call includes the prefill of its prompt
         inf.set_eos([cfg.V + 1])
         prompt = rng.integers(1, cfg.V, args.prompt_len).astype(np.uint32)
-        inf.generate_batch(prompt, 2, args.decode_batch)               # builds the tiled weight images once
+        inf.generate_batch(prompt, 2, args.decode_batch)               # builds the tiled weight images and the caches once
         tb = time.perf_counter()
         got = inf.generate_batch(prompt, args.steps, args.decode_batch)
         dtb = time.perf_counter() - tb
@@ -185,15 +190,19 @@ def decode_bench(args, cfg, L):
         batch = {"batch": args.decode_batch, "ms_per_step": round(dtb / steps_b * 1e3, 3),
                  "tokens_per_s": round(args.decode_batch * steps_b / dtb, 1), "steps": steps_b}
     inf.free()
+    if sft is not None:
+        sft.free()
     gbs = wb.value / (tms.value * 1e-3) / 1e9 if tms.value > 0 else 0.0
     out = {"metric": "greedy decode tokens/s, batch 1", "value": round(args.steps / dt, 1), "unit": "tokens/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt / args.steps * 1e3, 3), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "f16 weights x f32 activations, f32 accumulate" if f16 else
            "q8_0 weights x f32 activations, f32 accumulate", "data": "synthetic",
            "config": {"workload": cfg.name + "_decode", "layers": cfg.NL, "frozen_params": cfg.frozen_params,
-                      "weight_format": cfg.weight_format, "prompt_len": args.prompt_len},
+                      "weight_format": cfg.weight_format, "prompt_len": args.prompt_len,
+                      "weights": "own row-major matrices" if sft is None else "the training state's tiles, read in place"},
            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "k_matvec",
+                        "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                        "kernel": "k_matvec" if sft is None else ("gemm_ring" if f16 else "gemm_tiled"),
                         "launches_per_step": n // prof_steps, "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                         "weight_bytes_per_step": wb.value / prof_steps, "matvec_ms_per_step": round(tms.value / prof_steps, 3)},
            "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}
@@ -224,6 +233,8 @@ def main():
                     help="time greedy token-by-token generation (include/inference_hip.h) on the configuration's model "
                          "instead of the training step: a step is one token")
     ap.add_argument("--prompt-len", type=int, default=16)
+    ap.add_argument("--decode-from-sft", action="store_true",
+                    help="with --decode: a generation state made from a training state (inference_state_create_from_sft)")
     ap.add_argument("--decode-batch", type=int, default=0,
                     help="with --decode: also time this many copies of one prompt decoded in lock step")
     ap.add_argument("--gemm-shapes", action="store_true",

@@ -4,6 +4,8 @@
 #include "backend.h"
 #include "devutil.h"
 
+struct SFTState;
+
 namespace lmhip {
 
 // ---- tiled fp16 operand layout ------------------------------------------------
@@ -53,6 +55,16 @@ struct WeightOp {
     int fmt, nbq, kbq;
 };
 inline WeightOp weight_f16(const half_t *w) { return WeightOp{w, nullptr, nullptr, 0, 0, 0}; }
+
+// A training state's own forward images and norm gammas of one layer, nothing copied (sft.hip): what a generation
+// state made from the training state reads.  qkv holds the rows Q | K | V (any adapter rows behind them are not part
+// of the product), gu the rows gate | up.  The gammas are windows on the training state's arenas and belong to it.
+struct BorrowedLayer {
+    WeightOp qkv, o, gu, down;
+    struct ::MetalBuf *g_in, *g_post_attn, *g_pre_ff, *g_post_ff, *g_q, *g_k;
+};
+void sft_borrow_layer(::SFTState *s, int L, BorrowedLayer *out);
+WeightOp sft_borrow_lm_head(::SFTState *s);
 
 struct GemmPlan {
     int nb;        // 32-row weight blocks per wave (1 or 2)

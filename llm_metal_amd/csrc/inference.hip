@@ -28,6 +28,10 @@ extern "C" MetalBuf *sft_get_token_emb_buf(SFTState *s);
 namespace {
 struct BatchRun;
 void batch_release(BatchRun *r);
+// a state on a training state's tiles: one token through the lock-step path with a run of one sequence
+void step_on_tiles(InferenceState *s, int token, int pos);
+const float *logits_on_tiles(InferenceState *s);
+int argmax_on_tiles(InferenceState *s);
 }
 
 struct InferenceState {
@@ -44,6 +48,14 @@ struct InferenceState {
     std::vector<MetalBuf *> kc, vc;
     // per layer: fused [Wq; Wk; Wv] and [Wgate; Wup] (owned), Wo and Wdown and the norm gammas (owned, or the SFT state's)
     struct Layer { WMat qkv, gu; WMat *o, *down; MetalBuf *g_in, *g_post_attn, *g_pre_ff, *g_post_ff, *g_q, *g_k; };
+    // A state made from a training state owns no weights at all: `borrowed` holds the training state's tiled images
+    // (F16 or Q8_0 tiles, the operands of its own forward), read in place, so whatever training writes there is what the
+    // next token sees.  Such a state has no row-major matrices for the matrix-vector kernels; every step, also of a
+    // single sequence, goes through the matrix-core products of the lock-step batch path (`single`: its run of one).
+    int borrows_tiles;
+    std::vector<BorrowedLayer> borrowed;
+    WeightOp borrowed_lm;
+    BatchRun *single;
     std::vector<Layer> layers;
     WMat *lm_head;
     MetalBuf *g_final, *emb;
@@ -343,7 +355,7 @@ void default_eos(InferenceState *s)
 }
 
 InferenceState *new_state(ModelType mt, int D, int Hq, int Hkv, int hd, int IS, int V, int NL, int max_seq, int use_fp16,
-                          const float *thetas)
+                          const float *thetas, bool matvec_path = true)
 {
     if (fast_metal_init() != 0) { fprintf(stderr, "[FastGen] no GPU: fast_metal_init failed\n"); return nullptr; }
     if (Hkv <= 0 || Hq % Hkv || hd > 256 || (hd & 1) || Hq / Hkv > 16 || max_seq <= 0 || (IS & 3)) {
@@ -371,15 +383,17 @@ InferenceState *new_state(ModelType mt, int D, int Hq, int Hkv, int hd, int IS, 
     }
     default_eos(s);
     const int qd = Hq * hd, kd = Hkv * hd;
-    s->x = fbuf(D); s->x2 = fbuf(D); s->branch = fbuf(D); s->ln = fbuf(D);
-    s->qkv = fbuf(qd + 2 * kd); s->att = fbuf(qd);
-    s->gu = fbuf(2 * (size_t)IS);
-    s->gate_v = metal_buf_view(s->gu, 0, (size_t)IS * 4); s->up_v = metal_buf_view(s->gu, (size_t)IS * 4, (size_t)IS * 4);
-    s->logits = fbuf(V); s->best = metal_buf_create((4 + 2 * AM_WGS) * sizeof(int));   // result, then the per-workgroup (value, index) pairs
     HIP_CHECK(hipHostMalloc((void **)&s->logits_host, (size_t)V * 4, hipHostMallocDefault));
     HIP_CHECK(hipHostMalloc((void **)&s->best_host, sizeof(int), hipHostMallocDefault));
-    const size_t cache_bytes = (size_t)Hkv * max_seq * hd * sizeof(float);
-    for (int L = 0; L < NL; L++) { s->kc.push_back(metal_buf_create(cache_bytes)); s->vc.push_back(metal_buf_create(cache_bytes)); }
+    if (matvec_path) {                                                    // scratch and caches of the matrix-vector pipeline
+        s->x = fbuf(D); s->x2 = fbuf(D); s->branch = fbuf(D); s->ln = fbuf(D);
+        s->qkv = fbuf(qd + 2 * kd); s->att = fbuf(qd);
+        s->gu = fbuf(2 * (size_t)IS);
+        s->gate_v = metal_buf_view(s->gu, 0, (size_t)IS * 4); s->up_v = metal_buf_view(s->gu, (size_t)IS * 4, (size_t)IS * 4);
+        s->logits = fbuf(V); s->best = metal_buf_create((4 + 2 * AM_WGS) * sizeof(int));   // result, then the per-workgroup (value, index) pairs
+        const size_t cache_bytes = (size_t)Hkv * max_seq * hd * sizeof(float);
+        for (int L = 0; L < NL; L++) { s->kc.push_back(metal_buf_create(cache_bytes)); s->vc.push_back(metal_buf_create(cache_bytes)); }
+    }
     s->R = 0; s->scaling = 0.f; s->lora_t = nullptr;
     s->sft = nullptr; s->owns_weights = 0;
     s->layers.resize(NL);
@@ -547,49 +561,35 @@ InferenceState *inference_state_create_from_sft(SFTState *sft, int max_seq_len)
 {
     InferenceState *s = new_state(sft_get_model_type(sft), sft_get_d_model(sft), sft_get_n_q_heads(sft), sft_get_n_kv_heads(sft),
                                   sft_get_head_dim(sft), sft_get_intermediate_size(sft), sft_get_vocab_size(sft),
-                                  sft_get_n_layers(sft), max_seq_len, 1, sft_get_rope_thetas(sft));
+                                  sft_get_n_layers(sft), max_seq_len, 1, sft_get_rope_thetas(sft), false);
     if (!s) return nullptr;
+    if (s->D > 8192) { fprintf(stderr, "[FastGen] hidden size %d not supported for a state on a training state's weights (<= 8192)\n", s->D); inference_state_free(s); return nullptr; }
     s->sft = sft;
     s->g_final = sft_get_final_norm_g(sft);
     s->emb = sft_get_token_emb_buf(sft);
-    inference_state_refresh_from_sft(s);
+    s->borrows_tiles = 1;
+    s->borrowed.resize(s->NL);
+    for (int L = 0; L < s->NL; L++) {
+        sft_borrow_layer(sft, L, &s->borrowed[L]);
+        const BorrowedLayer &b = s->borrowed[L];
+        InferenceState::Layer &lw = s->layers[L];
+        lw.g_in = b.g_in; lw.g_post_attn = b.g_post_attn; lw.g_pre_ff = b.g_pre_ff; lw.g_post_ff = b.g_post_ff; lw.g_q = b.g_q; lw.g_k = b.g_k;
+    }
+    s->borrowed_lm = sft_borrow_lm_head(sft);
+    s->use_fp16 = s->borrowed_lm.fmt == 0;
     inference_state_set_lora(s, sft);
     return s;
 }
 
-void inference_state_refresh_from_sft(InferenceState *s)
-{
-    if (!s || !s->sft) return;
-    LayerW *src = sft_get_layers(s->sft);                                 // row-major F16 copies, refreshed by the call
-    const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS;
-    for (int L = 0; L < s->NL; L++) {
-        InferenceState::Layer &lw = s->layers[L];
-        if (!lw.qkv.mbuf) {
-            lw.qkv = WMat{metal_buf_create((size_t)(qd + 2 * kd) * D * 2), qd + 2 * kd, D, D / 32};
-            lw.gu = WMat{metal_buf_create((size_t)2 * IS * D * 2), 2 * IS, D, D / 32};
-        }
-        struct Part { WMat *w; MetalBuf *dst; size_t row0; };
-        const Part parts[5] = {{src[L].q_proj, lw.qkv.mbuf, 0}, {src[L].k_proj, lw.qkv.mbuf, (size_t)qd},
-                               {src[L].v_proj, lw.qkv.mbuf, (size_t)(qd + kd)}, {src[L].gate_proj, lw.gu.mbuf, 0},
-                               {src[L].up_proj, lw.gu.mbuf, (size_t)IS}};
-        for (const Part &p : parts) {
-            HIP_CHECK(hipMemcpyAsync((char *)dptr(p.dst) + p.row0 * D * 2, dptr(p.w->mbuf), (size_t)p.w->rows * D * 2,
-                                     hipMemcpyDeviceToDevice, stream()));
-            mark_written(p.dst);
-        }
-        lw.o = src[L].o_proj; lw.down = src[L].down_proj;
-        lw.g_in = src[L].input_norm_g; lw.g_post_attn = src[L].post_attn_norm_g;
-        lw.g_pre_ff = src[L].pre_ff_norm_g; lw.g_post_ff = src[L].post_ff_norm_g;
-        lw.g_q = src[L].q_norm_g; lw.g_k = src[L].k_norm_g;
-    }
-    s->lm_head = sft_get_lm_head(s->sft);
-}
+// Kept for callers written against copies: a state made from a training state reads that state's weights in place, so
+// there is nothing to refresh after a full-parameter update.
+void inference_state_refresh_from_sft(InferenceState *s) { (void)s; }
 
 void inference_state_set_lora(InferenceState *s, SFTState *sft)
 {
     const int R = sft_get_lora_rank(sft);
     if (R == 0) return;                                                   // full-parameter state: no adapters
-    if (!s->lora_t) s->lora_t = fbuf(2 * (size_t)R);
+    if (!s->lora_t && !s->borrows_tiles) s->lora_t = fbuf(2 * (size_t)R);
     s->lora.resize(s->NL);
     for (int L = 0; L < s->NL; L++)
         s->lora[L] = InferenceState::Lora{sft_get_lora_weight_buf(sft, L, 0), sft_get_lora_weight_buf(sft, L, 1),
@@ -603,6 +603,7 @@ void inference_state_free(InferenceState *s)
     if (!s) return;
     metal_flush();
     batch_release(s->batch);
+    batch_release(s->single);
     for (MetalBuf *b : {s->gate_v, s->up_v, s->x, s->x2, s->branch, s->ln, s->qkv, s->att, s->gu, s->logits, s->best, s->lora_t, s->rope_tabs})
         metal_buf_free(b);
     for (MetalBuf *b : s->kc) metal_buf_free(b);
@@ -638,20 +639,27 @@ static bool token_ok(InferenceState *s, int token)
     return true;
 }
 
+static void step_token(InferenceState *s, int token, int pos)
+{
+    if (s->borrows_tiles) step_on_tiles(s, token, pos);
+    else forward_token(s, token, pos);
+}
+static int argmax_host(InferenceState *s) { return s->borrows_tiles ? argmax_on_tiles(s) : argmax_to_host(s); }
+
 const float *inference_forward_token(InferenceState *s, int token)
 {
     if (!token_ok(s, token)) return nullptr;
-    forward_token(s, token, s->cur_len);
+    step_token(s, token, s->cur_len);
     s->cur_len++;
-    return logits_to_host(s);
+    return s->borrows_tiles ? logits_on_tiles(s) : logits_to_host(s);
 }
 
 int inference_forward_token_argmax(InferenceState *s, int token)
 {
     if (!token_ok(s, token)) return -1;
-    forward_token(s, token, s->cur_len);
+    step_token(s, token, s->cur_len);
     s->cur_len++;
-    return argmax_to_host(s);
+    return argmax_host(s);
 }
 
 int inference_generate(InferenceState *s, const uint32_t *prompt_tokens, int prompt_len, uint32_t *output_tokens, int max_gen_len)
@@ -660,19 +668,19 @@ int inference_generate(InferenceState *s, const uint32_t *prompt_tokens, int pro
     if (prompt_len <= 0 || max_gen_len <= 0 || prompt_len > s->max_seq) return 0;
     for (int i = 0; i < prompt_len; i++) {
         if (!token_ok(s, (int)prompt_tokens[i])) return 0;
-        forward_token(s, (int)prompt_tokens[i], i);                      // prefill: only the last logits are looked at
+        step_token(s, (int)prompt_tokens[i], i);                      // prefill: only the last logits are looked at
         s->cur_len = i + 1;
     }
-    int next = argmax_to_host(s);
+    int next = argmax_host(s);
     output_tokens[0] = (uint32_t)next;
     int n_gen = 1;
     for (int gen = 1; gen < max_gen_len && s->cur_len < s->max_seq; gen++) {
         bool is_eos = false;
         for (int e = 0; e < s->n_eos; e++) is_eos |= next == s->eos[e];
         if (is_eos) break;
-        forward_token(s, next, s->cur_len);
+        step_token(s, next, s->cur_len);
         s->cur_len++;
-        next = argmax_to_host(s);
+        next = argmax_host(s);
         output_tokens[n_gen++] = (uint32_t)next;
     }
     return n_gen;
@@ -758,20 +766,24 @@ void forward_token_batch(InferenceState *s, BatchRun &r, const int *tokens, int 
             hipLaunchKernelGGL(k_add_norm_split<8>, dim3(B), dim3(1024), 0, stream(), dptr_as<float>(r.x), br, gb, dptr_as<float>(g), ln,
                                a16, inv_ln, B, D, s->eps);
     };
-    // planes of (the operand in a16) x w^T; `inv`: the factors that operand's rows were split with
-    auto product = [&](const WMat *w, const float *inv) {
-        const GemmPlan p = plan_gemm(2 * B, w->rows, w->cols);
-        const size_t plane = (size_t)2 * B * w->rows;
-        launch_gemm(a16, nullptr, tiled_weight_of(w->mbuf, w->rows, w->cols), P, w->rows, plane, 2 * B, w->rows, w->cols, p);
-        return SplitPlanes{P, inv, plane, p.S, w->rows};
+    // planes of (the operand in a16) x w^T; `inv`: the factors that operand's rows were split with.  The weight: the
+    // tiled image of the state's own row-major matrix (made on first use), or the training state's tiles
+    auto product = [&](const WMat *w, const WeightOp *tiles, int rows, int cols, const float *inv) {
+        const WeightOp op = tiles ? *tiles : weight_f16(tiled_weight_of(w->mbuf, rows, cols));
+        const GemmPlan p = plan_gemm(2 * B, rows, cols, op.fmt ? op.nbq : 0, op.fmt);
+        const size_t plane = (size_t)2 * B * rows;
+        launch_gemm(a16, nullptr, op, P, rows, plane, 2 * B, rows, cols, p);
+        return SplitPlanes{P, inv, plane, p.S, rows};
     };
+    const bool bt = s->borrows_tiles;
     auto split = [&](MetalBuf *in, int K) { launch_rows_to_f16_split(dptr_as<float>(in), a16, inv_br, B, K); };
     SplitPlanes pending{};                                               // FFN branch of the layer before, added by the next norm kernel
     MetalBuf *pending_g = nullptr;
     for (int L = 0; L < s->NL; L++) {
         const InferenceState::Layer &lw = s->layers[L];
+        const BorrowedLayer *bl = bt ? &s->borrowed[L] : nullptr;
         add_norm_b(pending, pending_g, lw.g_in);
-        const SplitPlanes qkv = product(&lw.qkv, inv_ln);
+        const SplitPlanes qkv = product(&lw.qkv, bt ? &bl->qkv : nullptr, nqkv, D, inv_ln);
         launch_reduce_planes_split(qkv.P, qkv.S, qkv.plane, qkv.N, qkv.inv, dptr_as<float>(r.qkv), B, qkv.N);
         HeadPost a{};
         a.qkv = dptr_as<float>(r.qkv); a.qkv_step = (size_t)nqkv;
@@ -788,16 +800,16 @@ void forward_token_batch(InferenceState *s, BatchRun &r, const int *tokens, int 
         }
         attention_decode_fused(a, r.kc[L], r.vc[L], dptr_as<float>(r.att), hd, s->max_seq, B);
         split(r.att, qd);
-        const SplitPlanes o = product(lw.o, inv_br);
+        const SplitPlanes o = product(lw.o, bt ? &bl->o : nullptr, D, qd, inv_br);
         add_norm_b(o, gemma ? lw.g_post_attn : nullptr, gemma ? lw.g_pre_ff : lw.g_post_attn);
-        const SplitPlanes gu = product(&lw.gu, inv_ln);
+        const SplitPlanes gu = product(&lw.gu, bt ? &bl->gu : nullptr, 2 * IS, D, inv_ln);
         hipLaunchKernelGGL(k_glu_planes, dim3((IS + TB - 1) / TB, B), dim3(TB), 0, stream(), gu, dptr_as<float>(r.act), B, IS, gemma ? 1 : 0);
         split(r.act, IS);
-        pending = product(lw.down, inv_br);
+        pending = product(lw.down, bt ? &bl->down : nullptr, D, IS, inv_br);
         pending_g = gemma ? lw.g_post_ff : nullptr;
     }
     add_norm_b(pending, pending_g, s->g_final);
-    const SplitPlanes lg = product(s->lm_head, inv_ln);
+    const SplitPlanes lg = product(s->lm_head, bt ? &s->borrowed_lm : nullptr, s->V, D, inv_ln);
     launch_reduce_planes_split(lg.P, lg.S, lg.plane, lg.N, lg.inv, dptr_as<float>(r.logits), B, lg.N);
     HIP_CHECK(hipGetLastError());
 }
@@ -817,14 +829,14 @@ void argmax_batch(InferenceState *s, BatchRun &r, int *out)
 // The state's batch run for B sequences: the one kept from the call before when that had the same B and rank (its buffers
 // are strided by B), else a new one in its place.  Caches are not cleared: a step at position pos reads what steps
 // 0..pos-1 of the same run wrote.
-BatchRun &batch_acquire(InferenceState *s, int B)
+BatchRun &batch_acquire(InferenceState *s, BatchRun *&slot, int B)
 {
     const int R = s->lora.empty() ? 0 : s->R;
-    if (s->batch && s->batch->B == B && s->batch->R == R) return *s->batch;
+    if (slot && slot->B == B && slot->R == R) return *slot;
     metal_flush();
-    batch_release(s->batch);
-    s->batch = new BatchRun{};
-    BatchRun &r = *s->batch;
+    batch_release(slot);
+    slot = new BatchRun{};
+    BatchRun &r = *slot;
     const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS, V = s->V;
     r.B = B; r.R = R; r.len = 0;
     r.x = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
@@ -832,12 +844,13 @@ BatchRun &batch_acquire(InferenceState *s, int B)
     r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
     size_t a16_elems = 0, plane_floats = 0;                              // the largest operand and planes of the step's products
     const int shapes[5][2] = {{qd + 2 * kd, D}, {D, qd}, {2 * IS, D}, {D, IS}, {V, D}};
+    const int fmt = s->borrows_tiles ? s->borrowed_lm.fmt : 0;
     for (const auto &nk : shapes) {
         a16_elems = std::max(a16_elems, tiled_elems(2 * B, nk[1]));
         for (int ring = 0; ring < 2; ring++) {                           // either kernel policy may be switched in later
             const int was = gemm_ring_enabled();
             set_gemm_ring(ring);
-            plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1]).S * 2 * B * nk[0]);
+            plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1], fmt ? tiled_rb(nk[0]) : 0, fmt).S * 2 * B * nk[0]);
             set_gemm_ring(was);
         }
     }
@@ -851,9 +864,28 @@ BatchRun &batch_acquire(InferenceState *s, int B)
     return r;
 }
 
+void step_on_tiles(InferenceState *s, int token, int pos)
+{
+    BatchRun &r = batch_acquire(s, s->single, 1);
+    forward_token_batch(s, r, &token, pos);
+    r.len = pos + 1;
+}
+const float *logits_on_tiles(InferenceState *s)
+{
+    HIP_CHECK(hipMemcpyAsync(s->logits_host, dptr(s->single->logits), (size_t)s->V * 4, hipMemcpyDeviceToHost, stream()));
+    HIP_CHECK(hipStreamSynchronize(stream()));
+    return s->logits_host;
+}
+int argmax_on_tiles(InferenceState *s)
+{
+    int best = 0;
+    argmax_batch(s, *s->single, &best);
+    return best;
+}
+
 bool batch_args_ok(InferenceState *s, int B)
 {
-    if (!s->use_fp16) { fprintf(stderr, "[BatchGen] F16 weights only\n"); return false; }
+    if (!s->use_fp16 && !s->borrows_tiles) { fprintf(stderr, "[BatchGen] F16 weights only\n"); return false; }
     if (B < 1 || B > 32) return false;
     if (s->D > 8192) { fprintf(stderr, "[BatchGen] hidden size %d not supported (<= 8192)\n", s->D); return false; }
     return true;
@@ -874,7 +906,7 @@ int inference_generate_batch(InferenceState *s, const uint32_t *prompt_tokens, i
     if (!batch_args_ok(s, B) || prompt_len <= 0 || max_gen_len <= 0 || prompt_len > s->max_seq) return 0;
     for (int i = 0; i < prompt_len; i++)
         if (prompt_tokens[i] >= (uint32_t)s->V) { fprintf(stderr, "[BatchGen] token %u outside the vocabulary (%d)\n", prompt_tokens[i], s->V); return 0; }
-    BatchRun &r = batch_acquire(s, B);
+    BatchRun &r = batch_acquire(s, s->batch, B);
     int tokens[32], next[32], active[32];
     for (int i = 0; i < prompt_len; i++) {                               // prefill: the same token for every sequence (:910-916)
         for (int b = 0; b < B; b++) tokens[b] = (int)prompt_tokens[i];
@@ -914,7 +946,7 @@ int inference_step_batch(InferenceState *s, const int *tokens, int batch_size, i
     if (!s || !tokens || !batch_args_ok(s, B) || pos < 0 || pos >= s->max_seq) return -1;
     for (int b = 0; b < B; b++)
         if (tokens[b] < 0 || tokens[b] >= s->V) { fprintf(stderr, "[BatchGen] token %d outside the vocabulary (%d)\n", tokens[b], s->V); return -1; }
-    BatchRun &r = batch_acquire(s, B);
+    BatchRun &r = batch_acquire(s, s->batch, B);
     if (pos != 0 && pos != r.len) { fprintf(stderr, "[BatchGen] step at position %d, but the batch's caches hold %d\n", pos, r.len); return -1; }
     forward_token_batch(s, r, tokens, pos);
     r.len = pos + 1;

@@ -102,6 +102,7 @@ struct SFTState {
     std::vector<LayerW> layers_out;      // row-major F16 copies handed out by sft_get_layers
     std::vector<WMat> wmats_out;
     std::vector<MetalBuf *> views_out;
+    std::vector<MetalBuf *> gamma_views; // [NL][6] windows on the norm gammas for a generation state that borrows them
     WMat lm_head_out;
 };
 
@@ -925,6 +926,7 @@ void sft_state_free(SFTState *s)
     for (int i = 0; i < 4; i++)
         for (MetalBuf *b : {s->dy16[i], s->dy_inv[i], s->lyT[i], s->lyT_inv[i], s->lxT[i], s->lxT_inv[i]}) metal_buf_free(b);
     for (MetalBuf *b : s->views_out) metal_buf_free(b);
+    for (MetalBuf *b : s->gamma_views) metal_buf_free(b);
     for (auto &kv : s->img_slots) metal_buf_free(kv.second);
     for (MetalBuf *b : all) metal_buf_free(b);
     for (WMat &w : s->wmats_out) metal_buf_free(w.mbuf);
@@ -1377,3 +1379,21 @@ int sft_load_lora(SFTState *s, const char *path)
 }
 
 }  // extern "C"
+
+// internal: see BorrowedLayer
+void lmhip::sft_borrow_layer(SFTState *s, int L, BorrowedLayer *out)
+{
+    if (s->gamma_views.empty()) {
+        s->gamma_views.resize((size_t)6 * s->NL, nullptr);
+        const bool gemma = s->model_type == MODEL_GEMMA3;
+        MetalBuf *arena[6] = {s->g_in, s->g_post_attn, gemma ? s->g_pre_ff : nullptr, gemma ? s->g_post_ff : nullptr, s->g_q, s->g_k};
+        const int dim[6] = {s->D, s->D, s->D, s->D, s->hd, s->hd};
+        for (int l = 0; l < s->NL; l++)
+            for (int g = 0; g < 6; g++)
+                if (arena[g]) s->gamma_views[(size_t)l * 6 + g] = metal_buf_view(arena[g], (size_t)l * dim[g] * 4, (size_t)dim[g] * 4);
+    }
+    MetalBuf **g = &s->gamma_views[(size_t)L * 6];
+    *out = BorrowedLayer{wop(s, W_QKV, L, false), wop(s, W_O, L, false), wop(s, W_GU, L, false), wop(s, W_D, L, false),
+                         g[0], g[1], g[2], g[3], g[4], g[5]};
+}
+WeightOp lmhip::sft_borrow_lm_head(SFTState *s) { return wop(s, W_LM, 0, false); }

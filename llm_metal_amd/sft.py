@@ -298,6 +298,11 @@ class InferenceState:
     def load_eos(self, path):
         self.L.inference_state_load_eos(self.h, str(path).encode())
 
+    def attach_lora(self, sft):
+        """inference_state_set_lora: a state with its own weights reads the training state's adapters from then on."""
+        self.L.inference_state_set_lora(self.h, sft.h)
+        self._keep.append(sft)
+
     def refresh_from_sft(self):
         self.L.inference_state_refresh_from_sft(self.h)
 
