@@ -33,12 +33,17 @@ InferenceState *inference_state_create_from_ref(const SFTModelRef *model, int ma
  * tensors that already have the wanted format are used bit for bit (no dequantise -> requantise). */
 InferenceState *inference_state_create_from_file(const char *path, ModelType model_type, int max_seq_len, int use_fp16);
 
-/* src/nn/fast_inference.h:49 (impl src/nn/fast_inference.c:527-610): shares the SFT state's weights (row-major F16
- * copies handed out by sft_get_layers / sft_get_lm_head), embedding table, final norm and LoRA adapters; the SFT
- * state must outlive it.  After a full-parameter update call inference_state_refresh_from_sft. */
+/* src/nn/fast_inference.h:49 (impl src/nn/fast_inference.c:527-610, owns_weights = 0 at :596-603): the state owns no
+ * weights.  It reads the SFT state's own operands in place -- the F16 or Q8_0 tiles of its forward products, embedding
+ * table, norm gammas and LoRA adapter buffers -- so it allocates only caches and scratch, and whatever training writes
+ * (adapters, or every matrix in full-parameter mode) is what the next token is computed with.  The SFT state must
+ * outlive it.  There are no row-major matrices for the matrix-vector kernels in such a state: every step, also of a
+ * single sequence, runs the products of the lock-step batch path on the matrix cores (22 bits of the activations kept;
+ * Q8_0 tiles enter as half(d * q), as in training), at about 1.8x the time per token of a state with its own weights.
+ * A caller that wants the fastest single-sequence decode with a training state's adapters builds a state of its own
+ * (inference_state_create_from_ref) and attaches them with inference_state_set_lora.  Hidden size <= 8192. */
 InferenceState *inference_state_create_from_sft(SFTState *sft, int max_seq_len);
-/* re-reads the weights of the SFT state this state was created from (no counterpart in the reference, whose shared
- * buffers are the training weights themselves) */
+/* does nothing (kept for callers written against weight copies): the shared buffers are the training weights themselves */
 void inference_state_refresh_from_sft(InferenceState *state);
 
 void inference_state_free(InferenceState *state);                    /* src/nn/fast_inference.h:21 */
