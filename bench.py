@@ -225,6 +225,8 @@ def main():
     ap.add_argument("--q8-large-m", choices=("kept-image", "image-per-product", "unpack-in-lds"), default="kept-image",
                     help="how products with >= 1024 rows read Q8_0 weights: the F16 image a state keeps once made (default), "
                          "an F16 image made for every product, or Q8_0 tiles unpacked into LDS by the GEMM itself")
+    ap.add_argument("--attn-bwd-one-launch", type=int, choices=(0, 1), default=1,
+                    help="0: up to 64 positions too, the attention backward is two launches (dQ, then dK / dV) (comparisons only)")
     ap.add_argument("--gemm-ring", type=int, choices=(0, 1), default=1,
                     help="0: the products of up to 64 rows take the register-staged streaming kernel (gemm_tiled) instead of gemm_ring (comparisons only)")
     ap.add_argument("--attention", choices=("auto", "flash", "saved-probs"), default="auto",
@@ -280,6 +282,7 @@ def main():
     t_gen = time.perf_counter() - t0
     L.hip_attention_flash({"auto": -1, "flash": 1, "saved-probs": 0}[args.attention])
     L.hip_gemm_ring(args.gemm_ring)
+    L.hip_attention_backward_one_launch(args.attn_bwd_one_launch)
     if args.q8_large_m == "image-per-product":
         L.hip_gemm_image_budget_mb(0)
     elif args.q8_large_m == "unpack-in-lds" and cfg.weight_format != "f16" and cfg.BN >= 1024:

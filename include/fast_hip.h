@@ -182,6 +182,9 @@ void hip_gemm_image_budget_mb(int mb);
  * is at least 128 or the sequence is longer than 1024 (default, the measured rule), 0 = never, 1 = whenever the head
  * size allows.  Read when a training state is created. */
 void hip_attention_flash(int mode);
+/* 1 (default): for sequences of at most 64 positions the attention backward is one launch (dQ, and dK / dV as shares per
+ * query block and query head that the next kernel sums); 0: dQ, then dK / dV, as for longer sequences */
+void hip_attention_backward_one_launch(int on);
 /* Timing aid for benchmarks: when enabled, every GEMM launch is bracketed by HIP events on the
  * library's stream.  hip_gemm_profile_read (after metal_flush) returns the number of launches recorded
  * since the last enable and adds up their durations (ms) and weight bytes; _read2 also their flops. */

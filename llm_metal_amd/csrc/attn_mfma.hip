@@ -182,6 +182,9 @@ struct AttnTileArgs {
     half_t *out16;                // forward: tiled [rows, Hq*hd]
     WeightPrefetch pf;            // weights of the product that follows: fetched by the grid slices z >= batch
     int window;                   // forward: > 0 masks keys older than i - window + 1 (the saved zeros carry it into the backward)
+    // dQ with the block's share of dK / dV in the same launch (sequences of at most 64 keys): q [rows][Hq*hd], and the
+    // shares [query block][Hq][rows_total][hd] that the consumer of dk / dv sums (attn_dkv_part_index)
+    const float *q; float *dkp, *dvp; int rows_total;
 };
 
 // Row step: eight threads per row, thread `part` owns the keys 32 m + 4 part + (0..3) for m < M32 and keeps them in
@@ -210,9 +213,11 @@ __device__ __forceinline__ void load_probs(float4 (&p)[M32], const AttnTileArgs 
     }
 }
 
-template <int BWD, int M32>
+// DKV (dQ only): the probabilities go to LDS as well (Ps, laid out like the finished rows of Xs), for the dV share
+// formed after phase 3, and dscore stays out of memory: nothing reads it.
+template <int BWD, int M32, int DKV = 0>
 __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int xlo, int nk, int N, int i0, int b, int h, int tid,
-                                         const float4 (&p_early)[BWD ? M32 : 1])
+                                         const float4 (&p_early)[BWD ? M32 : 1], float *Ps = nullptr)
 {
     const int rr = tid >> 3, part = tid & 7, i = i0 + rr;
     const bool row_ok = i < N;
@@ -267,8 +272,14 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
             __bf16 *xh = reinterpret_cast<__bf16 *>(Xs + rr * ldx) + j;
             *reinterpret_cast<u32x2 *>(xh) = u32x2{pack_hi(o.x, o.y), pack_hi(o.z, o.w)};
             *reinterpret_cast<u32x2 *>(xh + xlo) = u32x2{pack_hi(rest(o.x), rest(o.y)), pack_hi(rest(o.z), rest(o.w))};
+            if constexpr (BWD && DKV) {
+                const float4 pv = p[m];
+                __bf16 *ph = reinterpret_cast<__bf16 *>(Ps + rr * ldx) + j;
+                *reinterpret_cast<u32x2 *>(ph) = u32x2{pack_hi(pv.x, pv.y), pack_hi(pv.z, pv.w)};
+                *reinterpret_cast<u32x2 *>(ph + xlo) = u32x2{pack_hi(rest(pv.x), rest(pv.y)), pack_hi(rest(pv.z), rest(pv.w))};
+            }
         }
-        if (row_ok && j < N) {
+        if (!DKV && row_ok && j < N) {
             if ((N & 3) == 0) *reinterpret_cast<float4 *>(gdst + 32 * m) = o;
             else { const float *q = &o.x; for (int c = 0; c < 4; c++) if (j + c < N) gdst[32 * m + c] = q[c]; }
         }
@@ -278,7 +289,7 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
 // grid (query blocks of 32, Hq, batch), block 256; LDS: Ahi, Alo [32][HD+8] bf16, Xs[32][ldx] fp32 / bf16 pairs
 // M32: 32-key blocks a row can hold (2, 8, 16 or 32: sequences up to 64, 256, 512, 1024); a template parameter so
 // that the kernel's code is one straight run (the kernel runs once per workgroup, and what it skips it still fetches).
-template <int BWD, int HD, int M32>
+template <int BWD, int HD, int M32, int DKV = 0>
 __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
 {
     extern __shared__ float lds[];
@@ -298,6 +309,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     const int N32 = (N + 31) & ~31, ldx = N32 + 4;
     __bf16 *Ahi = reinterpret_cast<__bf16 *>(lds), *Alo = Ahi + 32 * lda;
     float *Xs = lds + 32 * lda;                           // behind the two bf16 images of A
+    float *Ps = Xs + 32 * ldx;                            // DKV only
 
     // ---- the first B pass and the first C chunk of this wave do not depend on anything computed here:
     //      request them before the A rows are staged (waves without a tile of their own read tile 0)
@@ -316,6 +328,21 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     b_tile_load<CB>(bt0, b_item(0), ldt);
     float4 p_early[BWD ? M32 : 1];
     if constexpr (BWD && M32 <= 8) load_probs<M32>(p_early, a, N, i0, b, h, tid);
+    // DKV: this lane's q values for the shares formed at the end (query rows 16 u + 8 hh + e of the block, head column
+    // dt * 32 + l31 for the wave's blocks dt = wave, wave + 4): requested now, used last
+    constexpr int NDT = DKV ? (HD + 127) / 128 : 1;
+    float q_early[NDT][2][8];
+    if constexpr (BWD && DKV) {
+#pragma unroll
+        for (int t = 0; t < NDT; t++)
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int i = i0 + 16 * u + 8 * hh + e, d = min((wave + 4 * t) * 32, HD - 32) + l31;
+                    q_early[t][u][e] = a.q[(r0 + min(i, N - 1)) * qd + h * HD + d];
+                }
+    }
     CRing cring;
     const float *c_lane0 = a.C + r0 * kd + hk * HD + l31;
     c_ring_start<M32>(cring, c_lane0 + (wave * 32 < HD ? wave * 32 : 0), (size_t)kd, nk, hh, N);
@@ -342,7 +369,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
 #pragma unroll
         for (int u = 0; u < HD / 32; u++) {
             const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
-            if (BWD && i0 + rr < N) st4(a.A_out + (r0 + i0 + rr) * qd + h * HD + 4 * c4, av[u]);
+            if (BWD && !DKV && i0 + rr < N) st4(a.A_out + (r0 + i0 + rr) * qd + h * HD + 4 * c4, av[u]);
             *reinterpret_cast<u32x2 *>(Ahi + rr * lda + 4 * c4) = u32x2{pack_hi(av[u].x, av[u].y), pack_hi(av[u].z, av[u].w)};
             *reinterpret_cast<u32x2 *>(Alo + rr * lda + 4 * c4) = u32x2{pack_hi(rest(av[u].x), rest(av[u].y)), pack_hi(rest(av[u].z), rest(av[u].w))};
         }
@@ -382,7 +409,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     __syncthreads();
 
     // ---- row step
-    row_step<BWD, M32>(a, Xs, ldx, N32, nk, N, i0, b, h, tid, p_early);    // whole rows of N entries are written
+    row_step<BWD, M32, DKV>(a, Xs, ldx, N32, nk, N, i0, b, h, tid, p_early, Ps);    // whole rows of N entries are written
     __syncthreads();
 
     // ---- phase 3: Y = X C, one 32-column block of the head per wave and round
@@ -399,6 +426,56 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
             if (i >= N) continue;
             if (BWD) a.out32[(r0 + i) * qd + h * HD + d] = acc[v];
             else a.out16[tiled_a_index((int)(r0 + i), h * HD + d, Kb)] = f2h(acc[v]);
+        }
+    }
+    if constexpr (BWD && DKV) {
+        // ---- the block's share of dK and dV of its query head, for the keys it sees:
+        //      dKp[j, d] = sum_{i in block} dS[i, j] q[i, d],   dVp[j, d] = sum_{i in block} P[i, j] dO[i, d].
+        // A wave takes the head columns dt * 32 ..; in an instruction lane (l31, hh) reduces over the query rows
+        // 16 u + 8 hh + 0..7 of the block: its key's dS / P values come from LDS a row apart each (the finished rows
+        // are stored by query), dO likewise from the staged A rows, q from memory.
+        const __bf16 *Xh = reinterpret_cast<const __bf16 *>(Xs), *Ph = reinterpret_cast<const __bf16 *>(Ps);
+        const int ldh = 2 * ldx;
+#pragma unroll
+        for (int t = 0; t < NDT; t++) {
+            const int dt = wave + 4 * t;
+            if (dt * 32 >= HD) break;
+            const int d = dt * 32 + l31;
+            HL qB[2], oB[2];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                float qv[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int i = i0 + 16 * u + 8 * hh + e;
+                    qv[e] = i < N ? q_early[t][u][e] : 0.f;
+                    oB[u].hi[e] = Ahi[(16 * u + 8 * hh + e) * lda + d];
+                    oB[u].lo[e] = Alo[(16 * u + 8 * hh + e) * lda + d];
+                }
+                qB[u] = split8(qv);
+            }
+            for (int jb = 0; jb < nkb; jb++) {
+                HL sA[2], pA[2];
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const int o = (16 * u + 8 * hh + e) * ldh + jb * 32 + l31;
+                        sA[u].hi[e] = Xh[o]; sA[u].lo[e] = Xh[o + N32];
+                        pA[u].hi[e] = Ph[o]; pA[u].lo[e] = Ph[o + N32];
+                    }
+                float16v aK = zero16(), aV = zero16();
+#pragma unroll
+                for (int u = 0; u < 2; u++) { mfma3(aK, sA[u], qB[u]); mfma3(aV, pA[u], oB[u]); }
+                const size_t base = (((size_t)qb * a.Hq + h) * a.rows_total + r0) * HD + d;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int jj = jb * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
+                    if (jj >= N) continue;
+                    a.dkp[base + (size_t)jj * HD] = aK[v];
+                    a.dvp[base + (size_t)jj * HD] = aV[v];
+                }
+            }
         }
     }
     if (!BWD && h == a.Hq - 1)                             // zero the K padding of the operand rows once
@@ -473,22 +550,23 @@ __global__ __launch_bounds__(256) void k_attn_dkv_tile(AttnDkvArgs a)
     }
 }
 
-size_t tile_lds_bytes(int hd, int seq) { return (size_t)32 * (hd + 8 + ((seq + 31) & ~31) + 4) * sizeof(float); }
+size_t tile_lds_bytes(int hd, int seq, int dkv = 0) { return (size_t)32 * (hd + 8 + (1 + dkv) * (((seq + 31) & ~31) + 4)) * sizeof(float); }
 
-template <int BWD, int HD, int M32>
+template <int BWD, int HD, int M32, int DKV = 0>
 void launch_tile_m(const AttnTileArgs &a)
 {
     static bool attr_set = false;
-    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_attn_tile<BWD, HD, M32>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); attr_set = true; }
-    const size_t lds = tile_lds_bytes(HD, a.seq);
+    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_attn_tile<BWD, HD, M32, DKV>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); attr_set = true; }
+    const size_t lds = tile_lds_bytes(HD, a.seq, DKV);
     const int per_z = ((a.seq + 31) / 32) * a.Hq;
     const int extra = a.pf.base ? a.pf.wgs / per_z : 0;   // the planner made pf.wgs a multiple of per_z
-    LAUNCH((k_attn_tile<BWD, HD, M32>), dim3((a.seq + 31) / 32, a.Hq, a.batch + extra), dim3(256), lds, a);
+    LAUNCH((k_attn_tile<BWD, HD, M32, DKV>), dim3((a.seq + 31) / 32, a.Hq, a.batch + extra), dim3(256), lds, a);
 }
 
 template <int BWD, int HD>
 void launch_tile_hd(const AttnTileArgs &a)
 {
+    if (BWD && a.dkp) { launch_tile_m<BWD, HD, 2, BWD>(a); return; }     // at most 64 keys (the caller checked)
     if (a.seq <= 64) launch_tile_m<BWD, HD, 2>(a);
     else if (a.seq <= 256) launch_tile_m<BWD, HD, 8>(a);
     else if (a.seq <= 512) launch_tile_m<BWD, HD, 16>(a);
@@ -509,6 +587,13 @@ void launch_tile(const AttnTileArgs &a)
 
 
 }  // namespace
+
+namespace { int g_bwd_one_launch = 1; }
+void set_attn_bwd_one_launch(int on) { g_bwd_one_launch = on ? 1 : 0; }
+bool attn_bwd_one_launch(int hd, int seq)
+{
+    return g_bwd_one_launch && attn_mfma_supported(hd, seq) && seq <= 64 && tile_lds_bytes(hd, seq, 1) <= 150 * 1024;
+}
 
 bool attn_mfma_supported(int hd, int seq)
 {
@@ -533,6 +618,12 @@ void launch_attn_bwd_mfma(const AttnBwdArgs &g)
     a.Apl = g.dO; a.BT = g.vT; a.C = g.k;
     a.Hq = g.Hq; a.Hkv = g.Hkv; a.hd = g.hd; a.seq = g.seq; a.batch = g.batch; a.scale = g.scale;
     a.probs = const_cast<float *>(g.probs); a.dscore = g.dscore; a.A_out = g.dO_red; a.out32 = g.dq;
+    if (g.dkp) {                                          // one launch: the consumer of dk / dv sums the shares
+        if (g.seq > 64) { fprintf(stderr, "[fast_hip] attn_bwd_mfma: dK / dV shares need a sequence of at most 64\n"); abort(); }
+        a.q = g.q; a.dkp = g.dkp; a.dvp = g.dvp; a.rows_total = g.batch * g.seq;
+        launch_tile<1>(a);
+        return;
+    }
     launch_tile<1>(a);
     AttnDkvArgs d{};
     d.probs = g.probs; d.dscore = g.dscore; d.q = g.q; d.dO = g.dO_red;
@@ -542,3 +633,5 @@ void launch_attn_bwd_mfma(const AttnBwdArgs &g)
 }
 
 }  // namespace lmhip
+
+extern "C" void hip_attention_backward_one_launch(int on) { lmhip::set_attn_bwd_one_launch(on); }

@@ -97,6 +97,9 @@ struct AttnBwdArgs {
     const float *vT;              // v transposed per head [batch][Hkv][hd/4][attn_ldt(seq)][4] (matrix-core path only)
     float *dO_red, *dscore;       // scratch: [rows][Hq*hd], [batch][Hq][seq][seq]
     float *dq, *dk, *dv;          // [rows][Hq*hd], [rows][Hkv*hd] x2 (post-RoPE domain)
+    // matrix-core path, at most 64 keys: not null -> one launch that leaves dk / dv as shares per (query block, query
+    // head), [ceil(seq/32)][Hq][rows][hd] each, for launch_qkv_bwd to sum (dk, dv, dO_red, dscore are then not written)
+    float *dkp, *dvp;
 };
 void launch_attn_bwd(const AttnBwdArgs &a);
 // The same two operations on the fp32 matrix cores (attn_mfma.hip): head_dim a multiple of 32 and a
@@ -104,6 +107,10 @@ void launch_attn_bwd(const AttnBwdArgs &a);
 bool attn_mfma_supported(int hd, int seq);
 void launch_attn_fwd_mfma(const AttnFwdArgs &a);
 void launch_attn_bwd_mfma(const AttnBwdArgs &a);
+// dQ and the dK / dV shares in one launch (AttnBwdArgs::dkp): on by default wherever the matrix-core path runs on at
+// most 64 keys; the switch is for comparisons with the two-launch path
+void set_attn_bwd_one_launch(int on);
+bool attn_bwd_one_launch(int hd, int seq);
 
 // The same attention without the [seq, seq] matrices in memory (attn_flash.hip): head_dim 64 or 128, any sequence
 // length.  The forward saves the operands of the backward (bf16-pair fragments of q, k, v), the output and one
@@ -134,6 +141,10 @@ void launch_attn_bwd_flash(const AttnFlashArgs &a);
 
 struct QkvBwdArgs {
     const float *dq, *dk, *dv;    // post-RoPE-domain gradients
+    // not null: dk and dv come as shares [query block][Hq][rows_total][hd] instead (AttnBwdArgs::dkp): key row j of
+    // KV head hk is the sum over the query heads of its group and over the query blocks from j / 32 on; the summed dv
+    // is also written to dv_f
+    const float *dkp, *dvp; int rows_total;
     const float *q_pre, *k_pre, *g_q, *g_k; float eps;
     const float2 *rope;
     const float *Bq, *Bv; int R; float sc;

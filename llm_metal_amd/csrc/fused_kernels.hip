@@ -425,6 +425,32 @@ __global__ __launch_bounds__(TB) void k_attn_bwd_dkv(AttnBwdArgs a)
 // (src/nn/fast_sft.c:953-971).
 // NP, RK: pairs per lane and LoRA rank compiled in, as in k_qkv_post.  NT: threads per row (1024, or 256 from a few
 // hundred rows on, as in k_norm_rows).
+// dk or dv of (row, KV head hk, column d) from the shares the one-launch attention backward leaves
+// ([query block][Hq][rows_total][hd]): the query heads of the group, and the query blocks that see the key
+__device__ __forceinline__ float kv_share_sum(const QkvBwdArgs &a, const float *shares, size_t row, int pos, int hk, int d)
+{
+    const int ratio = a.Hq / a.Hkv, nqb = (a.seq + 31) >> 5;
+    float v[2][4];
+    float s = 0.f;
+    const size_t st_h = (size_t)a.rows_total * a.hd, st_qb = st_h * a.Hq;
+    const float *p = shares + ((size_t)hk * ratio * a.rows_total + row) * a.hd + d;
+    const int qb0 = pos >> 5;
+    for (int g0 = 0; g0 < ratio; g0 += 4) {
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const bool ok = qb0 + q < nqb && g0 + g < ratio;
+                v[q][g] = ok ? p[(size_t)(qb0 + q) * st_qb + (size_t)(g0 + g) * st_h] : 0.f;
+            }
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) s += v[q][g];
+    }
+    return s;
+}
+
 template <int NP, int RK, int NT = RB>
 __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
 {
@@ -444,9 +470,10 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
     // issued before the first reduction, so their latency is paid once per trip instead of once per head.
     constexpr int SU = 3;
     const int nslots = a.Hq + a.Hkv;
-    for (int s0 = wave; s0 < nslots; s0 += (NT / 64) * SU) {
-        float g0[SU][NP], g1[SU][NP], p0[SU][NP], p1[SU][NP], w0[SU][NP], w1[SU][NP];
-        float2 cs[NP];
+    float g0[SU][NP], g1[SU][NP], p0[SU][NP], p1[SU][NP], w0[SU][NP], w1[SU][NP];
+    float2 cs[NP];
+    // the loads of one trip; with `defer_shares` the dk values of a K head are left for take_shares()
+    auto load_trip = [&](int s0, bool defer_shares) __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             const int d = lane + 64 * p;
@@ -460,17 +487,34 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
             const float *gin = (isk ? a.dk : a.dq) + row * W + h * hd;
             const float *xp = (isk ? a.k_pre : a.q_pre) + row * W + h * hd;
             const float *g = isk ? a.g_k : a.g_q;
+            const bool shares = isk && a.dkp;                          // uniform per wave
 #pragma unroll
             for (int p = 0; p < NP; p++) {
                 const int d = lane + 64 * p;
                 g0[u][p] = g1[u][p] = p0[u][p] = p1[u][p] = w0[u][p] = w1[u][p] = 0.f;
                 if (d < half) {
-                    g0[u][p] = gin[d]; g1[u][p] = gin[d + half];
+                    if (shares) { if (!defer_shares) { g0[u][p] = buf[qd + h * hd + d]; g1[u][p] = buf[qd + h * hd + d + half]; } }
+                    else { g0[u][p] = gin[d]; g1[u][p] = gin[d + half]; }
                     p0[u][p] = xp[d]; p1[u][p] = xp[d + half];
                     w0[u][p] = g[d]; w1[u][p] = g[d + half];
                 }
             }
         }
+    };
+    auto take_shares = [&](int s0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < SU; u++) {
+            const int slot = min(s0 + (NT / 64) * u, nslots - 1);
+            if (slot < a.Hq) continue;
+            const int h = slot - a.Hq;
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int d = lane + 64 * p;
+                if (d < half) { g0[u][p] = buf[qd + h * hd + d]; g1[u][p] = buf[qd + h * hd + d + half]; }
+            }
+        }
+    };
+    auto finish_trip = [&](int s0) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < SU; u++) {
             const int slot = s0 + (NT / 64) * u;
@@ -501,8 +545,27 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
                 if (!isk) { a.dq_f[row * qd + h * hd + d] = d0; a.dq_f[row * qd + h * hd + d + half] = d1; }
             }
         }
+    };
+    constexpr int TRIP = (NT / 64) * SU;
+    const bool first = wave < nslots;
+    if (first) load_trip(wave, true);
+    if (a.dkp) {
+        // dk and dv arrive as shares: their sums are formed by all threads while the loads of the first trip are on
+        // their way.  dk waits in its place in the row (the wave that owns a head reads it there before it writes the
+        // head's result), dv is final.
+        for (int c = threadIdx.x; c < 2 * kd; c += NT) {
+            const int isv = c >= kd, cc = isv ? c - kd : c;
+            const float v = kv_share_sum(a, isv ? a.dvp : a.dkp, row, pos, cc / hd, cc % hd);
+            buf[qd + c] = v;
+            if (isv) a.dv_f[row * kd + cc] = v;
+        }
+        __syncthreads();
+        if (first) take_shares(wave);
     }
-    for (int c = threadIdx.x; c < kd; c += NT) buf[qd + kd + c] = a.dv[row * kd + c];
+    if (first) finish_trip(wave);
+    for (int s0 = wave + TRIP; s0 < nslots; s0 += TRIP) { load_trip(s0, false); finish_trip(s0); }
+    if (!a.dvp)
+        for (int c = threadIdx.x; c < kd; c += NT) buf[qd + kd + c] = a.dv[row * kd + c];
     __syncthreads();
     // dh[r] = sc * sum_c d[c] * B[c][r].  Rank 16 (the common case): four threads share a row of B (16 floats, one
     // float4 each) and 256 such groups split the columns, so a thread keeps 4 + 4 sums and a wave reduces over its 16

@@ -75,6 +75,7 @@ struct SFTState {
     MetalBuf *ones;                      // [BN] of 1.0f
     MetalBuf *planes;
     MetalBuf *logits, *dlogits, *dl16, *dl_inv;
+    MetalBuf *dkp, *dvp;                 // dk / dv as shares per (query block, query head) where one launch forms dq and them (at most 64 keys)
     MetalBuf *dx[2], *dO_red, *dscore, *dq, *dk, *dv, *dq_f, *dh;   // LoRA mode: dv, dq_f, dh are kept per layer until the
                                                                    // adapter gradients of all layers are formed in one launch
     MetalBuf *ce_part;
@@ -536,6 +537,8 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         if (!s->use_flash) { ab.dO_red = at<float>(s->dO_red); ab.dscore = at<float>(s->dscore); }
         const size_t keepL = R ? (size_t)L : 0;                 // LoRA mode keeps dv, dq_f and dh of every layer
         ab.dq = at<float>(s->dq); ab.dk = at<float>(s->dk); ab.dv = at<float>(s->dv, keepL * BN * kd);
+        const bool kv_shares = !s->use_flash && s->dkp && attn_bwd_one_launch(s->hd, s->N);
+        if (kv_shares) { ab.dkp = at<float>(s->dkp); ab.dvp = at<float>(s->dvp); }
         if (s->use_flash) {
             AttnFlashArgs f = flash_args(s, L);
             f.dO = pdo; f.dq = ab.dq; f.dk = ab.dk; f.dv = ab.dv;
@@ -554,6 +557,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         qb.R = R; qb.sc = s->lora_scaling;
         qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
         qb.dq_f = at<float>(s->dq_f, keepL * BN * qd); qb.dv_f = nullptr; qb.dh = at<float>(s->dh, keepL * BN * (R ? 2 * R : 1));
+        if (kv_shares) { qb.dkp = ab.dkp; qb.dvp = ab.dvp; qb.rows_total = BN; qb.dv_f = ab.dv; }
         qb.out16 = d16[3]; qb.inv_scale = dinv[3];
         if (mode == BWD_LORA) qb.pf = prefetch_for(s, wop(s, W_QKV, L, true), D, s->nq_ext, 1024);
         launch_qkv_bwd(qb, BN);
@@ -877,6 +881,10 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->dl16 = hbuf(tiled_elems(BN, V)); s->dl_inv = fbuf(BN);
     s->dx[0] = fbuf(xsz); s->dx[1] = fbuf(xsz);
     if (!s->use_flash) { s->dO_red = fbuf((size_t)BN * qd); s->dscore = fbuf((size_t)s->B * s->Hq * s->N * s->N); }
+    if (!s->use_flash && attn_mfma_supported(s->hd, s->N) && s->N <= 64) {
+        const size_t n = (size_t)((s->N + 31) / 32) * s->Hq * BN * s->hd;
+        s->dkp = fbuf(n); s->dvp = fbuf(n);
+    }
     const size_t keep = R ? NL : 1;
     s->dq = fbuf((size_t)BN * qd); s->dk = fbuf((size_t)BN * kd); s->dv = fbuf(keep * BN * kd);
     s->dq_f = fbuf(keep * BN * qd); s->dh = fbuf(keep * BN * (R ? 2 * R : 1));
@@ -917,7 +925,7 @@ void sft_state_free(SFTState *s)
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
                        s->gu_sav, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->group_inv, s->ones, s->planes,
-                       s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore,
+                       s->logits, s->dlogits, s->dl16, s->dl_inv, s->dx[0], s->dx[1], s->dO_red, s->dscore, s->dkp, s->dvp,
                        s->dq, s->dk, s->dv, s->dq_f, s->dh, s->ce_part,
                        s->ln2_16, s->ln2_inv, s->act16, s->act_inv, s->attn16, s->lnf16, s->lnf_inv,
                        s->xT, s->xT_inv, s->yT, s->yT_inv, s->gqkv, s->go, s->ggu, s->gd, s->glm,
