@@ -86,7 +86,7 @@ def gemm_shapes(cfg, L):
         y = np.array([r[key] for r in layer])
         slope, t0 = np.polyfit(x, y, 1)
         fits[key] = {"t0_us": round(float(t0), 2), "rate_GBs": round(1e3 / float(slope))}
-    print(json.dumps({"workload": cfg.name, "rows": cfg.BN, "shapes": rows, "fit_over_layer_shapes": fits}))
+    emit({"workload": cfg.name, "rows": cfg.BN, "shapes": rows, "fit_over_layer_shapes": fits})
 
 
 def cpu_baseline(cfg, budget_s=20.0):
@@ -210,10 +210,51 @@ def decode_bench(args, cfg, L):
         out["batched"] = batch
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = decode_cpu_baseline(cfg)
-    print(json.dumps(out))
+    emit(out)
+
+
+class _LibraryStdoutToStderr:
+    """The library reports like the reference does, with printf on stdout ("[FastSFT] Grad accum buffers allocated ...").
+    While this is active, file descriptor 1 is stderr, so that the one JSON line is all this program writes to stdout."""
+
+    def __enter__(self):
+        import ctypes
+        self.libc = ctypes.CDLL(None)
+        sys.stdout.flush()
+        self.saved = os.dup(1)
+        os.dup2(2, 1)
+        return self
+
+    def __exit__(self, *exc):
+        self.libc.fflush(None)
+        sys.stdout.flush()
+        os.dup2(self.saved, 1)
+        os.close(self.saved)
+
+
+def emit(obj):
+    """The result line, on the real stdout."""
+    line = json.dumps(obj)
+    if _REAL_STDOUT is not None:
+        os.write(_REAL_STDOUT, (line + "\n").encode())
+    else:
+        print(line)
+
+
+_REAL_STDOUT = None
 
 
 def main():
+    global _REAL_STDOUT
+    with _LibraryStdoutToStderr() as redirect:
+        _REAL_STDOUT = redirect.saved
+        try:
+            return _main()
+        finally:
+            _REAL_STDOUT = None
+
+
+def _main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -268,8 +309,8 @@ def main():
         L.metal_flush()
         L.metal_buf_free(src), L.metal_buf_free(dst)
         L.fast_metal_shutdown()
-        print(json.dumps({"copy_calibration": {"kernel": "k_copy", "bytes_read_per_launch": 4 * n,
-                                               "bytes_written_per_launch": 4 * n, "launches": 5}}))
+        emit({"copy_calibration": {"kernel": "k_copy", "bytes_read_per_launch": 4 * n,
+                                   "bytes_written_per_launch": 4 * n, "launches": 5}})
         return
 
     if args.decode:
@@ -378,7 +419,7 @@ def main():
            "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
-    print(json.dumps(out))
+    emit(out)
 
 
 if __name__ == "__main__":
