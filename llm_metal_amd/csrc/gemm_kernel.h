@@ -41,22 +41,26 @@ __device__ __forceinline__ half8 bcast8(half_t d)
 
 // Weight registers of one 64-wide K step for row block `nb`: w[j] feeds the j-th MFMA of the step.
 // FMT 0: F16 tiles, `kb_stride` K blocks per row block, K block `kt`.
+// SHARED: the workgroups of several activation row tiles read the same weight tile through one L2 (gemm_tiled's MTILES),
+// so the loads are ordinary ones; a tile that only one workgroup reads is streamed past the caches.
+template <int SHARED = 0>
 __device__ __forceinline__ void load_w_f16(half8 (&w)[4], const half_t *W16, int nb, int kb_stride, int kt, int lane)
 {
     const half8 *p = reinterpret_cast<const half8 *>(W16) + ((size_t)nb * kb_stride + kt) * 256 + lane;
 #pragma unroll
-    for (int j = 0; j < 4; j++) w[j] = __builtin_nontemporal_load(&p[j * 64]);     // streamed once
+    for (int j = 0; j < 4; j++) w[j] = SHARED ? p[j * 64] : __builtin_nontemporal_load(&p[j * 64]);
 }
 
 // FMT 1: Q8_0, one scale per (row, 32 columns): the 32 weights of a lane share one scale.
 // The products d * q are rounded to fp16 once, which is what a stored F16 image of the
 // dequantised weight would hold.
+template <int SHARED = 0>
 __device__ __forceinline__ void load_w_q8_rows(half8 (&w)[4], const WeightOp &W, int nb, int kb_stride, int kt, int lane)
 {
     const size_t tile = (size_t)nb * kb_stride + kt;
     const uint4v *q = reinterpret_cast<const uint4v *>(W.q) + tile * 128 + lane;
-    const uint4v r0 = __builtin_nontemporal_load(&q[0]), r1 = __builtin_nontemporal_load(&q[64]);
-    const half8 d = bcast8(__builtin_nontemporal_load(&W.d[tile * 64 + lane]));
+    const uint4v r0 = SHARED ? q[0] : __builtin_nontemporal_load(&q[0]), r1 = SHARED ? q[64] : __builtin_nontemporal_load(&q[64]);
+    const half8 d = bcast8(SHARED ? W.d[tile * 64 + lane] : __builtin_nontemporal_load(&W.d[tile * 64 + lane]));
     w[0] = q8_unpack8(r0[0], r0[1]) * d;
     w[1] = q8_unpack8(r0[2], r0[3]) * d;
     w[2] = q8_unpack8(r1[0], r1[1]) * d;
@@ -65,11 +69,12 @@ __device__ __forceinline__ void load_w_q8_rows(half8 (&w)[4], const WeightOp &W,
 
 // FMT 2: Q8_0 of the transposed matrix: one scale per (column, 32 rows), so a tile (32 rows) has 64
 // column scales and a lane multiplies its weight (j, e) by the scale of column (lane / 32) * 32 + 8 j + e.
+template <int SHARED = 0>
 __device__ __forceinline__ void load_w_q8_cols(half8 (&w)[4], const WeightOp &W, int nb, int kb_stride, int kt, int lane)
 {
     const size_t tile = (size_t)nb * kb_stride + kt;
     const uint4v *q = reinterpret_cast<const uint4v *>(W.q) + tile * 128 + lane;
-    const uint4v r0 = __builtin_nontemporal_load(&q[0]), r1 = __builtin_nontemporal_load(&q[64]);
+    const uint4v r0 = SHARED ? q[0] : __builtin_nontemporal_load(&q[0]), r1 = SHARED ? q[64] : __builtin_nontemporal_load(&q[64]);
     const half8 *sc = reinterpret_cast<const half8 *>(W.d + tile * 64 + (lane >> 5) * 32);
     const half8 s0 = sc[0], s1 = sc[1], s2 = sc[2], s3 = sc[3];
     w[0] = q8_unpack8(r0[0], r0[1]) * s0;
@@ -150,13 +155,13 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
         half8 a[2][4], w[NB][4];
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            if (WF == 0) load_w_f16(w[b], g.W.w16, nbi[b], Kb, kt, lane);
+            if (WF == 0) load_w_f16<MTILES>(w[b], g.W.w16, nbi[b], Kb, kt, lane);
             else if (WF == 1) {
-                if (q8_rows) load_w_q8_rows(w[b], g.W, nbi[b], Kb, kt, lane);
-                else load_w_f16(w[b], g.W.w16, nbi[b] - g.W.nbq, Kb, kt, lane);
+                if (q8_rows) load_w_q8_rows<MTILES>(w[b], g.W, nbi[b], Kb, kt, lane);
+                else load_w_f16<MTILES>(w[b], g.W.w16, nbi[b] - g.W.nbq, Kb, kt, lane);
             } else {
-                if (kt < g.W.kbq) load_w_q8_cols(w[b], g.W, nbi[b], g.W.kbq, kt, lane);
-                else load_w_f16(w[b], g.W.w16, nbi[b], Kb - g.W.kbq, kt - g.W.kbq, lane);
+                if (kt < g.W.kbq) load_w_q8_cols<MTILES>(w[b], g.W, nbi[b], g.W.kbq, kt, lane);
+                else load_w_f16<MTILES>(w[b], g.W.w16, nbi[b], Kb - g.W.kbq, kt - g.W.kbq, lane);
             }
         }
 #pragma unroll
