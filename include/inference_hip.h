@@ -39,7 +39,7 @@ InferenceState *inference_state_create_from_file(const char *path, ModelType mod
  * (adapters, or every matrix in full-parameter mode) is what the next token is computed with.  The SFT state must
  * outlive it.  There are no row-major matrices for the matrix-vector kernels in such a state: every step, also of a
  * single sequence, runs the products of the lock-step batch path on the matrix cores (22 bits of the activations kept;
- * Q8_0 tiles enter as half(d * q), as in training), at about 1.8x the time per token of a state with its own weights.
+ * Q8_0 tiles enter as half(d * q), as in training), at about 1.6x the time per token of a state with its own weights.
  * A caller that wants the fastest single-sequence decode with a training state's adapters builds a state of its own
  * (inference_state_create_from_ref) and attaches them with inference_state_set_lora.  Hidden size <= 8192. */
 InferenceState *inference_state_create_from_sft(SFTState *sft, int max_seq_len);

@@ -154,7 +154,23 @@ __global__ __launch_bounds__(64) void k_lora_down(const float *__restrict__ ln, 
     ln += (size_t)blockIdx.y * D; t += (size_t)blockIdx.y * 2 * R;       // one vector of a batch per blockIdx.y
     const float *a = r < R ? Aq + (size_t)r * D : Av + (size_t)(r - R) * D;
     float s = 0.f;
-    for (int i = threadIdx.x; i < D; i += 64) s = fmaf(a[i], ln[i], s);
+    if ((D & 3) == 0) {                                                   // 16-byte loads, eight pairs of them in flight per lane
+        const float4 *a4 = reinterpret_cast<const float4 *>(a), *l4 = reinterpret_cast<const float4 *>(ln);
+        const int n4 = D >> 2;
+        for (int i0 = threadIdx.x; i0 < n4; i0 += 64 * 8) {
+            float4 av[8], lv[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int i = i0 + 64 * u;
+                av[u] = lv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (i < n4) { av[u] = a4[i]; lv[u] = l4[i]; }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += av[u].x * lv[u].x + av[u].y * lv[u].y + av[u].z * lv[u].z + av[u].w * lv[u].w;
+        }
+    } else {
+        for (int i = threadIdx.x; i < D; i += 64) s = fmaf(a[i], ln[i], s);
+    }
     s = wave_sum(s);
     if (threadIdx.x == 0) t[r] = s;
 }
@@ -757,7 +773,7 @@ void forward_token_batch(InferenceState *s, BatchRun &r, const int *tokens, int 
     // x += branch (the planes `br` of the product before, none at the start); ln = RMSNorm(x) as fp32 (only the adapters
     // read it) and as the operand of the next product
     auto add_norm_b = [&](const SplitPlanes &br, MetalBuf *g_branch, MetalBuf *g) {
-        float *ln = s->lora.empty() ? nullptr : dptr_as<float>(r.ln);
+        float *ln = (s->lora.empty() || s->borrows_tiles) ? nullptr : dptr_as<float>(r.ln);      // fp32 copy: only k_lora_down reads it
         const float *gb = g_branch ? dptr_as<float>(g_branch) : nullptr;
         if (tiled_kb(D) * 64 <= 4096)
             hipLaunchKernelGGL(k_add_norm_split<4>, dim3(B), dim3(1024), 0, stream(), dptr_as<float>(r.x), br, gb, dptr_as<float>(g), ln,
@@ -783,19 +799,26 @@ void forward_token_batch(InferenceState *s, BatchRun &r, const int *tokens, int 
         const InferenceState::Layer &lw = s->layers[L];
         const BorrowedLayer *bl = bt ? &s->borrowed[L] : nullptr;
         add_norm_b(pending, pending_g, lw.g_in);
-        const SplitPlanes qkv = product(&lw.qkv, bt ? &bl->qkv : nullptr, nqkv, D, inv_ln);
+        // a training state's fused matrix continues with the rows of A_q and A_v (their fp16 images, as its own forward
+        // reads them): the product then yields the adapters' down-projections as well, and no launch forms them
+        const bool t_in_product = bt && !s->lora.empty();
+        const int nq_rows = nqkv + (t_in_product ? 2 * s->R : 0);
+        const SplitPlanes qkv = product(&lw.qkv, bt ? &bl->qkv : nullptr, nq_rows, D, inv_ln);
         launch_reduce_planes_split(qkv.P, qkv.S, qkv.plane, qkv.N, qkv.inv, dptr_as<float>(r.qkv), B, qkv.N);
         HeadPost a{};
-        a.qkv = dptr_as<float>(r.qkv); a.qkv_step = (size_t)nqkv;
+        a.qkv = dptr_as<float>(r.qkv); a.qkv_step = (size_t)nq_rows;
         a.g_q = lw.g_q ? dptr_as<float>(lw.g_q) : nullptr; a.g_k = lw.g_k ? dptr_as<float>(lw.g_k) : nullptr;
         a.kc = dptr_as<float>(r.kc[L]); a.vc = dptr_as<float>(r.vc[L]); a.cache_step = (size_t)Hkv * s->max_seq * hd;
         a.Hq = Hq; a.Hkv = Hkv; a.pos = pos;
         a.rope = dptr_as<float2>(s->rope_tabs) + ((size_t)s->theta_slot[L] * s->max_seq + pos) * (hd / 2); a.eps = s->eps;
         if (!s->lora.empty()) {
             const InferenceState::Lora &lr = s->lora[L];
-            hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R, B), dim3(64), 0, stream(), dptr_as<float>(r.ln), dptr_as<float>(lr.Aq),
-                               dptr_as<float>(lr.Av), dptr_as<float>(r.lora_t), s->R, D);
-            a.t = dptr_as<float>(r.lora_t); a.t_step = (size_t)2 * s->R;
+            if (t_in_product) { a.t = dptr_as<float>(r.qkv) + nqkv; a.t_step = (size_t)nq_rows; }
+            else {
+                hipLaunchKernelGGL(k_lora_down, dim3(2 * s->R, B), dim3(64), 0, stream(), dptr_as<float>(r.ln), dptr_as<float>(lr.Aq),
+                                   dptr_as<float>(lr.Av), dptr_as<float>(r.lora_t), s->R, D);
+                a.t = dptr_as<float>(r.lora_t); a.t_step = (size_t)2 * s->R;
+            }
             a.Bq = dptr_as<float>(lr.Bq); a.Bv = dptr_as<float>(lr.Bv); a.R = s->R; a.sc = s->scaling;
         }
         attention_decode_fused(a, r.kc[L], r.vc[L], dptr_as<float>(r.att), hd, s->max_seq, B);
@@ -840,17 +863,18 @@ BatchRun &batch_acquire(InferenceState *s, BatchRun *&slot, int B)
     const int D = s->D, qd = s->Hq * s->hd, kd = s->Hkv * s->hd, IS = s->IS, V = s->V;
     r.B = B; r.R = R; r.len = 0;
     r.x = fbuf((size_t)B * D); r.ln = fbuf((size_t)B * D);
-    r.qkv = fbuf((size_t)B * (qd + 2 * kd)); r.att = fbuf((size_t)B * qd);
+    r.qkv = fbuf((size_t)B * (qd + 2 * kd + 2 * R)); r.att = fbuf((size_t)B * qd);
     r.act = fbuf((size_t)B * IS); r.logits = fbuf((size_t)B * V);
     size_t a16_elems = 0, plane_floats = 0;                              // the largest operand and planes of the step's products
-    const int shapes[5][2] = {{qd + 2 * kd, D}, {D, qd}, {2 * IS, D}, {D, IS}, {V, D}};
+    const int shapes[5][2] = {{qd + 2 * kd + (s->borrows_tiles ? 2 * R : 0), D}, {D, qd}, {2 * IS, D}, {D, IS}, {V, D}};
     const int fmt = s->borrows_tiles ? s->borrowed_lm.fmt : 0;
     for (const auto &nk : shapes) {
         a16_elems = std::max(a16_elems, tiled_elems(2 * B, nk[1]));
         for (int ring = 0; ring < 2; ring++) {                           // either kernel policy may be switched in later
             const int was = gemm_ring_enabled();
             set_gemm_ring(ring);
-            plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1], fmt ? tiled_rb(nk[0]) : 0, fmt).S * 2 * B * nk[0]);
+            const int nbq = !fmt ? 0 : &nk == &shapes[0] ? tiled_rb(qd + 2 * kd) : tiled_rb(nk[0]);   // the adapter rows are F16 tiles
+            plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1], nbq, fmt).S * 2 * B * nk[0]);
             set_gemm_ring(was);
         }
     }
