@@ -268,6 +268,8 @@ def _main():
                          "an F16 image made for every product, or Q8_0 tiles unpacked into LDS by the GEMM itself")
     ap.add_argument("--attn-bwd-one-launch", type=int, choices=(0, 1), default=1,
                     help="0: up to 64 positions too, the attention backward is two launches (dQ, then dK / dV) (comparisons only)")
+    ap.add_argument("--half-planes", type=int, choices=(0, 1), default=1,
+                    help="0: fp32 K-split planes for every product (comparisons only)")
     ap.add_argument("--gemm-ring", type=int, choices=(0, 1), default=1,
                     help="0: the products of up to 64 rows take the register-staged streaming kernel (gemm_tiled) instead of gemm_ring (comparisons only)")
     ap.add_argument("--attention", choices=("auto", "flash", "saved-probs"), default="auto",
@@ -323,6 +325,7 @@ def _main():
     t_gen = time.perf_counter() - t0
     L.hip_attention_flash({"auto": -1, "flash": 1, "saved-probs": 0}[args.attention])
     L.hip_gemm_ring(args.gemm_ring)
+    L.hip_gemm_half_planes(args.half_planes)
     L.hip_attention_backward_one_launch(args.attn_bwd_one_launch)
     if args.q8_large_m == "image-per-product":
         L.hip_gemm_image_budget_mb(0)
@@ -411,6 +414,8 @@ def _main():
                      if cfg.weight_format != "f16" and cfg.BN >= 1024 and args.q8_large_m == "unpack-in-lds" else
                      "q8_0 weights as f16 images x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN >= 1024 else
                      "q8_0 weights unpacked to f16 in registers x f16 activations, f32 accumulate" if cfg.weight_format != "f16" else
+                     "f16 weights x f16 activations, f32 accumulate (the K-chunk sums of five products per layer leave as f16)"
+                     if cfg.R > 0 and cfg.BN <= 64 and args.half_planes and args.gemm_ring else
                      "f16 weights x f16 activations, f32 accumulate"), "data": "synthetic",
            "config": {"workload": cfg.name, "rows_per_step": rows_per_step, "layers": cfg.NL, "lora_rank": cfg.R,
                       "frozen_params": cfg.frozen_params, "weight_format": cfg.weight_format,

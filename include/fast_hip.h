@@ -165,6 +165,12 @@ void hip_gemm_force_large_m(int policy);
  * into an LDS ring (gemm_ring: one or two workgroups per CU, 4 to 6 K chunks), 0 = the kernel with one K step per wave in
  * registers (gemm_tiled: 13 to 19 K chunks), which every other product takes.  Same results up to the order of the sums. */
 void hip_gemm_ring(int on);
+/* 1 (default): a LoRA training state of at most 64 rows on F16 weights stores the K-split planes of five of its eight
+ * products per layer (gate|up and down forward; down, gate|up and O backward) as halves: every chunk sum, formed in fp32,
+ * leaves times a power of two derived from the weight matrix (8192 times its largest row sum of |w| stays below the fp16
+ * maximum) and is summed in fp32 again by the kernel that consumes the planes.  Half the plane bytes, 11 significant
+ * bits per chunk sum.  0: fp32 planes everywhere.  Read when a product is launched. */
+void hip_gemm_half_planes(int on);
 /* K chunks of the large-M kernel on F16 tiles (each chunk writes a plane, the consumer adds them): 1 = by the measured
  * rule (three chunks when the 128 x 256 output blocks leave a third of the CUs idle and K >= 4096), 0 = never, n > 1 =
  * always n. */

@@ -19,6 +19,10 @@ struct Planes {
     // scale_groups != 0: the operand rows were scaled in that many groups of columns, each the K range of 2^group_shift
     // planes, and plane s is multiplied by row_scale[row * scale_groups + (s >> group_shift)] before it is added
     int group_shift, scale_groups;
+    // not 0: the planes hold halves (p points at them, stride and ld count halves), each the chunk's fp32 sum times a
+    // power of two that keeps it below the fp16 maximum for any operand row; a value read is multiplied by half_unscale,
+    // the inverse of that factor.  Only kernels that read their planes through planes_at4_multi may be given such planes.
+    float half_unscale;
 };
 
 // How a row kernel splits the columns of an fp16 operand row [*, K] among workgroups, each with a power-of-two scale of

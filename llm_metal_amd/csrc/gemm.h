@@ -85,8 +85,17 @@ int gemm_ring_enabled();            // 1 (default): products of up to 64 rows wi
 // P[s][m][n] (s < plan.S, plane s at P + s*plane_stride, row stride ldp) =
 //   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k],  A and W in the tiled layout.
 // Pass a_inv_scale = null to leave the row factors to the consumer of the planes.
+// half_scale != 0 (ring plans only, a_inv_scale null): the planes are written as halves, each chunk sum times half_scale
+// (see gemm_ring); plane_stride and ldp then count halves, and only planes_at4_multi reads such planes.
 void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const WeightOp &W,
-                 float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p);
+                 float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p, float half_scale = 0.f);
+// Largest sum of |w| over a row of a tiled F16 matrix [N, K]: with operand rows scaled below 8192 (row_scale_for), no
+// chunk sum of a product with this matrix exceeds 8192 times it.  Synchronises the stream.
+float tiled_max_row_l1(const half_t *W_tiled, int N, int K);
+// the power of two by which chunk sums of products with a matrix of that row bound are multiplied to leave as halves
+float half_plane_scale(float max_row_l1);
+void set_gemm_half_planes(int on);
+int gemm_half_planes_enabled();     // 1 (default): LoRA training states store the K-split planes of their frozen-weight ring products as halves
 inline void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const half_t *W_tiled,
                         float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p)
 {

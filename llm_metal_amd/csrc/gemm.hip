@@ -346,8 +346,9 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
 }
 
 void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
-                 float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p)
+                 float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p, float half_scale)
 {
+    if (half_scale != 0.f && (!p.ring || a_inv_scale)) { fprintf(stderr, "[fast_hip] gemm: half planes need a ring plan without row factors\n"); abort(); }
     if (M <= 0 || N <= 0 || K <= 0) return;
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
     bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2) && (p.nw == 4 || (p.nw == 8 && p.m_tiles == 1)) && W.fmt >= 0 && W.fmt <= 2;
@@ -376,12 +377,12 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
         g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
         g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
-        g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1;
+        g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1; g.half_scale = half_scale;
         const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(256 * p.kg);
-#define RING_LAUNCH(KGV, SC) do { \
-            if (g_prof_on) hipExtLaunchKernelGGL((gemm_ring<KGV, SC>), rgrid, rblock, 0, stream(), ra, rb, 0, g); \
-            else hipLaunchKernelGGL((gemm_ring<KGV, SC>), rgrid, rblock, 0, stream(), g); } while (0)
-#define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1); else RING_LAUNCH(KGV, 0); } while (0)
+#define RING_LAUNCH(KGV, SC, HP) do { \
+            if (g_prof_on) hipExtLaunchKernelGGL((gemm_ring<KGV, SC, HP>), rgrid, rblock, 0, stream(), ra, rb, 0, g); \
+            else hipLaunchKernelGGL((gemm_ring<KGV, SC, HP>), rgrid, rblock, 0, stream(), g); } while (0)
+#define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1, 0); else if (half_scale != 0.f) RING_LAUNCH(KGV, 0, 1); else RING_LAUNCH(KGV, 0, 0); } while (0)
         if (p.kg == 1) RING_PICK(1); else if (p.kg == 2) RING_PICK(2); else RING_PICK(4);
 #undef RING_PICK
 #undef RING_LAUNCH
@@ -489,6 +490,53 @@ void launch_untile_q8(const uint8_t *q_tiles, const half_t *d_tiles, int fmt, in
 }
 
 int gemm_profiling() { return g_prof_on; }
+namespace {
+int g_half_planes = 1;
+// one workgroup (a wave) per 32-row block of a tiled F16 matrix: the largest sum of |w| over one of its rows
+__global__ __launch_bounds__(64) void k_tiled_row_l1(const half8 *__restrict__ W, int N, int Kb, float *__restrict__ out)
+{
+    const int lane = threadIdx.x;
+    const half8 *p = W + (size_t)blockIdx.x * Kb * 256 + lane;
+    float s = 0.f;
+    for (int kt = 0; kt < Kb; kt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const half8 v = p[(size_t)kt * 256 + j * 64];
+#pragma unroll
+            for (int e = 0; e < 8; e++) s += fabsf((float)v[e]);
+        }
+    if ((int)blockIdx.x * 32 + (lane & 31) >= N) s = 0.f; // rows of the last block past the matrix hold anything
+    s += __shfl_xor(s, 32, 64);                           // the two column halves of a row
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) s = fmaxf(s, __shfl_xor(s, o, 64));
+    if (lane == 0) atomicMax(reinterpret_cast<int *>(out), __float_as_int(s));   // sums are >= 0: integer order is float order
+}
+}  // namespace
+
+float tiled_max_row_l1(const half_t *W_tiled, int N, int K)
+{
+    float *slot = (float *)scratch(SCR_MISC, sizeof(float));
+    HIP_CHECK(hipMemsetAsync(slot, 0, sizeof(float), stream()));
+    hipLaunchKernelGGL(k_tiled_row_l1, dim3(tiled_rb(N)), dim3(64), 0, stream(), reinterpret_cast<const half8 *>(W_tiled), N, tiled_kb(K), slot);
+    float v = 0.f;
+    HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream()));
+    HIP_CHECK(hipStreamSynchronize(stream()));
+    return v;
+}
+
+float half_plane_scale(float max_row_l1)
+{
+    // |chunk sum| < 8192 * max_row_l1; the largest power of two s with 8192 * max_row_l1 * s <= 32768 (half the fp16 range)
+    if (!(max_row_l1 > 0.f) || !(max_row_l1 < 1e30f)) return 1.0f;
+    int e;
+    frexpf(4.0f / max_row_l1, &e);                        // 4 / l1 = f * 2^e, f in [0.5, 1)
+    int pw = e - 1;
+    pw = pw > 24 ? 24 : (pw < -100 ? -100 : pw);
+    return ldexpf(1.0f, pw);
+}
+void set_gemm_half_planes(int on) { g_half_planes = on ? 1 : 0; }
+int gemm_half_planes_enabled() { return g_half_planes; }
+
 void set_gemm_ring(int on) { g_ring = on; }
 int gemm_ring_enabled() { return g_ring; }
 
@@ -661,6 +709,7 @@ void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, i
 
 void hip_gemm_force_large_m(int policy) { g_big_policy = policy; }
 void hip_gemm_ring(int on) { lmhip::set_gemm_ring(on); }
+void hip_gemm_half_planes(int on) { lmhip::set_gemm_half_planes(on); }
 void hip_gemm_large_m_split(int mode) { set_big_gemm_split(mode); }
 void hip_gemm_large_m_block(int mode) { set_big_gemm_block(mode); }
 

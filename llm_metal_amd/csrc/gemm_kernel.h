@@ -11,6 +11,7 @@ struct GemmKArgs {
     float *P; int ldp; size_t plane_stride;
     int M, N, Mb, Nb, Kb, steps_per_chunk;
     int n_tiles, S, m_tiles;                             // set (m_tiles > 1) when the grid is the 1-D one described at gemm_tiled
+    float half_scale;                                    // gemm_ring<.., .., 1>: the planes are halves, each sum times this power of two
 };
 
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -270,9 +271,13 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 // wait for all of them before every LDS read; the waits are written by hand below.
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-template <int KG, int SCALE>
+// HALFP (with SCALE 0): the chunk's sums leave as halves, times g.half_scale -- a power of two that the caller derives from
+// the weight matrix so that no sum of 8192-bounded operand values can pass the fp16 maximum; plane_stride and ldp then
+// count halves.  Half the bytes to write here and for the consumer to read; 11 significant bits per chunk sum.
+template <int KG, int SCALE, int HALFP = 0>
 __global__ __launch_bounds__(256 * KG) void gemm_ring(GemmKArgs g)
 {
+    static_assert(!(SCALE && HALFP), "final outputs stay fp32");
     static_assert(KG == 1 || KG == 2 || KG == 4, "K groups per workgroup");
     constexpr int LOADS_PER_ROUND = 4;                    // LDS-direct loads a wave issues per round: the four 1 KB pieces of its block
     __shared__ half8 ring[2 * KG * 1024];                 // [round parity][K group][block 0..3][slice 0..3][64 lanes]
@@ -343,9 +348,18 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(GemmKArgs g)
             }
     }
     // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8 (v / 4) + 4 (lane / 32) + v % 4
-    float *Pp = g.P + (size_t)chunk * g.plane_stride;
     const int n = (tile * 2 + qn) * 32 + r;
     const bool inside = 64 <= g.M && (tile + 1) * 64 <= g.N;
+    if constexpr (HALFP) {
+        half_t *Ph = reinterpret_cast<half_t *>(g.P) + (size_t)chunk * g.plane_stride;
+#pragma unroll
+        for (int k = 0; k < Q; k++) {
+            const int v = kg * Q + k, m = qm * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (inside || (m < g.M && n < g.N)) Ph[(size_t)m * g.ldp + n] = f2h(res[k] * g.half_scale);
+        }
+        return;
+    }
+    float *Pp = g.P + (size_t)chunk * g.plane_stride;
     float sc[Q];
     if (SCALE) {
 #pragma unroll

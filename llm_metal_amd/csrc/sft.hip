@@ -104,6 +104,10 @@ struct SFTState {
     std::vector<WMat> wmats_out;
     std::vector<MetalBuf *> views_out;
     std::vector<MetalBuf *> gamma_views; // [NL][6] windows on the norm gammas for a generation state that borrows them
+    // LoRA states of at most 64 rows on F16 weights: per frozen matrix (kind, as stored / transposed, layer) the power of
+    // two with which the chunk sums of its products leave as halves (half_plane_scale of the matrix's largest row sum of
+    // |w|); empty when the state's products do not take that path
+    std::vector<float> half_scale[5][2];
     WMat lm_head_out;
 };
 
@@ -289,8 +293,20 @@ WeightOp resident_image(SFTState *s, const WeightOp &W, int N, int K)
 }
 
 // P = A16 * W^T as K-split planes in the state's plane buffer (operands tiled)
+// The factor for the half planes of a product with matrix `kind` of layer L (0: fp32 planes).  Only where the consumer of
+// the planes reads them through planes_at4_multi and the operand rows are scaled below 8192: gate|up and down forward,
+// and the three frozen backward products.  (The O forward takes the attention output at unit scale, the Q|K|V products
+// contain the adapter rows, which change.)
+float half_scale_for(SFTState *s, int kind, int L, bool T)
+{
+    if (!gemm_half_planes_enabled() || kind < 0 || kind >= 5) return 0.f;
+    const std::vector<float> &v = s->half_scale[kind][T ? 1 : 0];
+    return (size_t)L < v.size() ? v[L] : 0.f;
+}
+
+// hscale != 0 (see half_scale_for): the planes of a ring product are written as halves
 Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, int N, int K, float *out = nullptr,
-            const ScaleGroups *sg = nullptr)
+            const ScaleGroups *sg = nullptr, float hscale = 0.f)
 {
     if (use_big_gemm(s->BN, N, K, W.fmt)) {                 // one launch; final output, or a few K chunks as planes
         float *C = out ? out : at<float>(s->planes);
@@ -307,14 +323,16 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
     if (!out && (size_t)p.S * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
     if (out && p.S != 1) { fprintf(stderr, "[fast_sft] direct GEMM output needs S == 1\n"); abort(); }
     // a direct (final) output gets its row factors in the GEMM epilogue; planes leave them to the consumer
-    launch_gemm(A, out ? inv : nullptr, W, P, N, stride, s->BN, N, K, p);
+    if (out || !p.ring) hscale = 0.f;
+    launch_gemm(A, out ? inv : nullptr, W, P, N, stride, s->BN, N, K, p, hscale);
+    const float unscale = hscale != 0.f ? 1.0f / hscale : 0.f;
     if (sg && sg->cols) {
         if (out || sg->cols != (p.steps * 64) << sg->shift || sg->groups != (p.S + (1 << sg->shift) - 1) >> sg->shift) {
             fprintf(stderr, "[fast_sft] column groups of the operand do not match the K chunks of the product\n"); abort();
         }
-        return Planes{P, p.S, stride, N, inv, sg->shift, sg->groups};
+        return Planes{P, p.S, stride, N, inv, sg->shift, sg->groups, unscale};
     }
-    return Planes{P, p.S, stride, N, out ? nullptr : inv};
+    return Planes{P, p.S, stride, N, out ? nullptr : inv, 0, 0, unscale};
 }
 
 void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
@@ -408,7 +426,7 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
         float *gu_keep = at<float>(s->gu_sav, (size_t)L * BN * 2 * IS);
         const WeightOp wgu = wop(s, W_GU, L, false);
         const bool direct = use_big_gemm(BN, 2 * IS, D, wgu.fmt);
-        Planes pg = gemm(s, ln2, ln2inv, wgu, 2 * IS, D, direct ? gu_keep : nullptr);
+        Planes pg = gemm(s, ln2, ln2inv, wgu, 2 * IS, D, direct ? gu_keep : nullptr, nullptr, half_scale_for(s, W_GU, L, false));
         GluArgs ga{};
         ga.in = pg; ga.IS = IS; ga.gelu = gemma;
         ga.gate_pre = gu_keep; ga.up_val = gu_keep + IS; ga.ld_gu = (size_t)2 * IS; ga.in_place = direct;
@@ -417,7 +435,7 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
         launch_glu_fwd(ga, BN);
 
         // ff = act Wd^T, added by the next row kernel                          [:730-740]
-        pending = gemm(s, act16, ga.inv_scale, wop(s, W_D, L, false), D, IS, nullptr, &ga.sg);
+        pending = gemm(s, act16, ga.inv_scale, wop(s, W_D, L, false), D, IS, nullptr, &ga.sg, half_scale_for(s, W_D, L, false));
     }
 
     // x_final = x_mid + ff; ln = RN(x_final; g_final); logits = ln Wlm^T        [:744-751]
@@ -495,7 +513,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
 
     for (int L = NL - 1; L >= 0; L--) {
         // FFN: d act = d Wd; (dgate, dup); dln2 = dgate Wg + dup Wu; dx += RNB(x_mid, dln2)   [:798-874]
-        Planes pd = gemm(s, d16[0], dinv[0], wop(s, W_D, L, true), IS, D);
+        Planes pd = gemm(s, d16[0], dinv[0], wop(s, W_D, L, true), IS, D, nullptr, nullptr, half_scale_for(s, W_D, L, true));
         if (mode != BWD_LORA && !defer)                                       // [:804-811, 842-849]
             weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->act16, L * s->st_act), at<float>(s->act_inv, (size_t)L * BN), IS,
                         s->wd, s->wdT, s->gd, L * s->st_d, L * s->st_dT);
@@ -505,7 +523,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         if (mode == BWD_LORA) gb.sg = scale_groups_for(s, wop(s, W_GU, L, true), D, 2 * IS);
         gb.out16 = d16[1]; gb.inv_scale = gb.sg.cols ? at<float>(s->group_inv) : dinv[1];
         launch_glu_bwd(gb, BN);
-        Planes pgu = gemm(s, d16[1], gb.inv_scale, wop(s, W_GU, L, true), D, 2 * IS, nullptr, &gb.sg);
+        Planes pgu = gemm(s, d16[1], gb.inv_scale, wop(s, W_GU, L, true), D, 2 * IS, nullptr, &gb.sg, half_scale_for(s, W_GU, L, true));
         if (mode != BWD_LORA && !defer)                                       // gate and up as one matrix [:817-833, 853-869]
             weight_grad(s, mode, lr, a16, ainv, 2 * IS, at<half_t>(s->ln2_16, L * s->st_ln1), at<float>(s->ln2_inv, (size_t)L * BN), D,
                         s->wgu, s->wguT, s->ggu, L * s->st_gu, L * s->st_guT);
@@ -520,7 +538,9 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         cur ^= 1;
 
         // attention: dO = d Wo; dq, dk, dv                                    [:877-911]
-        Planes pdo = gemm(s, d16[2], dinv[2], wop(s, W_O, L, true), qd, D);
+        // (the wave-per-query attention kernels read their planes element by element: fp32 planes for them)
+        const bool dO_by4 = s->use_flash || attn_mfma_supported(s->hd, s->N);
+        Planes pdo = gemm(s, d16[2], dinv[2], wop(s, W_O, L, true), qd, D, nullptr, nullptr, dO_by4 ? half_scale_for(s, W_O, L, true) : 0.f);
         if (mode != BWD_LORA && !defer)                                       // [:883-901]
             weight_grad(s, mode, lr, a16, ainv, D, at<half_t>(s->attn16, L * s->st_attn), at<float>(s->ones), qd,
                         s->wo, s->woT, s->go, L * s->st_o, L * s->st_oT);
@@ -909,6 +929,18 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     // the fused QKV weight and its transpose carry fp16 images of A_q, A_v
     refresh_shadow(s);
     metal_flush();
+    // products of at most 64 rows on frozen F16 weights leave their K-split planes as halves: one factor per matrix
+    if (s->R > 0 && !s->q8_native && BN <= 64) {
+        struct Img { int kind; bool T; MetalBuf *arena; size_t st; int N, K; };
+        const Img imgs[] = {{W_GU, false, s->wgu, s->st_gu, 2 * IS, D}, {W_D, false, s->wd, s->st_d, D, IS},
+                            {W_D, true, s->wdT, s->st_dT, IS, D}, {W_GU, true, s->wguT, s->st_guT, D, 2 * IS},
+                            {W_O, true, s->woT, s->st_oT, qd, D}};
+        for (const Img &im : imgs) {
+            std::vector<float> &v = s->half_scale[im.kind][im.T ? 1 : 0];
+            v.resize(s->NL);
+            for (int L = 0; L < s->NL; L++) v[L] = half_plane_scale(tiled_max_row_l1(at<half_t>(im.arena, (size_t)L * im.st), im.N, im.K));
+        }
+    }
     return s;
 }
 
