@@ -3,6 +3,8 @@
 // activations that feed a GEMM are produced directly as scaled fp16 rows, GEMM
 // outputs arrive as K-split partial planes that the consumer sums on load.
 #pragma once
+#include <stdio.h>
+#include <stdlib.h>
 #include "backend.h"
 #include "devutil.h"
 #include "gemm.h"
@@ -10,20 +12,31 @@
 namespace lmhip {
 
 // K-split partial planes of a GEMM output: value(row, col) = row_scale[row] * sum_s p[s*stride + row*ld + col]
+// (40 bytes: with two ints and a pointer in front of it, it fits the arguments that reach a kernel preloaded, kargs.h)
 struct Planes {
     const float *p;
-    int S;
-    size_t stride;
-    int ld;
     const float *row_scale;   // value(row, col) is multiplied by row_scale[row] when non-null
+    uint32_t stride;          // elements between planes
+    int S;
+    int ld;
     // scale_groups != 0: the operand rows were scaled in that many groups of columns, each the K range of 2^group_shift
     // planes, and plane s is multiplied by row_scale[row * scale_groups + (s >> group_shift)] before it is added
-    int group_shift, scale_groups;
+    int16_t group_shift, scale_groups;
     // not 0: the planes hold halves (p points at them, stride and ld count halves), each the chunk's fp32 sum times a
     // power of two that keeps it below the fp16 maximum for any operand row; a value read is multiplied by half_unscale,
     // the inverse of that factor.  Only kernels that read their planes through planes_at4_multi may be given such planes.
     float half_unscale;
 };
+inline Planes make_planes(const float *p, int S, size_t stride, int ld, const float *row_scale, int group_shift = 0, int scale_groups = 0,
+                          float half_unscale = 0.f)
+{
+    if (stride > 0xffffffffull) { fprintf(stderr, "[fast_hip] planes: more than 2^32 elements per plane\n"); abort(); }
+    Planes P;
+    P.p = p; P.row_scale = row_scale; P.stride = (uint32_t)stride; P.S = S; P.ld = ld;
+    P.group_shift = (int16_t)group_shift; P.scale_groups = (int16_t)scale_groups; P.half_unscale = half_unscale;
+    return P;
+}
+static_assert(sizeof(Planes) == 40, "Planes is part of the kernels' preloaded arguments");
 
 // How a row kernel splits the columns of an fp16 operand row [*, K] among workgroups, each with a power-of-two scale of
 // its own: `cols` columns per group (a whole number of K chunks of the GEMM that consumes the operand), `groups` of
@@ -49,17 +62,20 @@ struct WeightPrefetch {
 constexpr uint32_t ZERO_ROW_TOKEN = 0xFFFFFFFFu;
 
 struct NormRowsArgs {
-    // source of the residual stream row: token gather (emb != null) or x_prev
-    const float *emb; const uint32_t *tokens; float emb_scale;
-    int zero_rows;                // gather only: rows whose token id is ZERO_ROW_TOKEN read as zero (padding of a short sequence)
-    const float *x_prev;
+    // (the first 56 bytes reach the kernel preloaded: what it needs to ask for the branch's planes and the row)
+    int rows_launched;            // set by the launcher
+    int D;
+    const float *x_prev;          // source of the residual stream row, unless it is gathered (emb != null)
     // optional branch added to it: planes, optionally RMS-normalised with g_branch first
-    Planes branch; const float *g_branch; float *branch_raw_out;
+    Planes branch;
+    const float *emb; const uint32_t *tokens; float emb_scale;      // token gather
+    int zero_rows;                // gather only: rows whose token id is ZERO_ROW_TOKEN read as zero (padding of a short sequence)
+    const float *g_branch; float *branch_raw_out;
     float *x_out;                 // new residual stream row (may be null when nothing was added)
     const float *g_norm;          // null: no normalised output wanted
     half_t *ln16; float *inv_scale;   // tiled [rows, D]
-    int D; float eps;
-    WeightPrefetch pf; int rows_launched;             // rows_launched: set by the launcher
+    float eps;
+    WeightPrefetch pf;
 };
 void launch_norm_rows(const NormRowsArgs &a, int rows);
 
@@ -174,23 +190,29 @@ int  lora_grad_blocks(int D, int qd, int kd, int R);
 void launch_lora_grads(const LoraGradArgs &a);
 
 struct GluArgs {
+    // (the first 56 bytes -- the planes, gate_pre, IS and sg.cols -- reach the column-group kernels preloaded, kargs.h)
     Planes in;                    // fwd: [rows][gate | up]; bwd: [rows][d act]
-    int IS, gelu;
-    float *gate_pre, *up_val;     // fwd: written; bwd: read; rows ld_gu floats apart (the two are the halves of one [rows][2 IS] array)
+    float *gate_pre;              // fwd: written; bwd: read; rows ld_gu floats apart (gate_pre and up_val are the halves of one [rows][2 IS] array)
+    int IS;
+    ScaleGroups sg;               // sg.cols != 0: inv_scale is [rows][sg.groups]
+    int gelu;
+    float *up_val;
     size_t ld_gu;
     int in_place;                 // fwd, one workgroup per row only: `in` is that array (one plane, factors applied): nothing to copy
     half_t *out16; float *inv_scale;                // tiled; fwd: act [rows, IS]; bwd: [rows, dgate | dup]
-    ScaleGroups sg;               // sg.cols != 0: inv_scale is [rows][sg.groups]
 };
 void launch_glu_fwd(const GluArgs &a, int rows);
 void launch_glu_bwd(const GluArgs &a, int rows);
 
 struct NormBwdArgs {
-    Planes dy; const float *x_saved, *g; float eps; int D;
+    int rows_launched; int D;                           // (first 56 bytes: preloaded, see NormRowsArgs)
+    const float *x_saved;
+    Planes dy;
+    const float *g; float eps;
     const float *dx_prev; float *dx_out; float clamp;   // clamp <= 0: none
     const float *branch_raw, *g_branch;                 // Gemma3: next GEMM input is RNB(branch_raw, dx_out)
     half_t *d16; float *inv_scale;                      // tiled [rows, D]; may be null on the last kernel of the backward
-    WeightPrefetch pf; int rows_launched;
+    WeightPrefetch pf;
 };
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows);
 

@@ -11,6 +11,7 @@
 // thread are independent so they are in flight together.
 #include "fused.h"
 #include "planes.h"
+#include "kargs.h"
 
 namespace lmhip {
 namespace {
@@ -55,19 +56,25 @@ __device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t
 // NT: threads per row.  1024 when a step has few rows (one row's loads all in flight at once); 256 from a few hundred
 // rows on, where eight resident workgroups per CU hide each other's reductions and barriers.
 template <int MAXV, bool GROUPED, int NT = RB>
-__global__ __launch_bounds__(NT) void k_norm_rows(NormRowsArgs a)
+__global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
 {
+    KARGS_HOT(NormRowsArgs, a);                           // rows_launched, D, x_prev, branch
     __shared__ float sm[16];
     if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
+        kargs_rest(a);
         prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
     const size_t r = xcd_block_row(blockIdx.x, a.rows_launched);
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
-    const uint32_t tok = a.emb ? a.tokens[r] : 0u;
-    const bool padded = a.emb && a.zero_rows && tok == ZERO_ROW_TOKEN;      // zero rows past the end of a sequence
-    const float *base = a.emb ? a.emb + (size_t)(padded ? 0u : tok) * D : a.x_prev + r * D;
+    // (x_prev, D and the branch's planes arrive preloaded: a row that is not gathered asks for all its data without
+    // waiting for the rest of the arguments)
+    const bool gather = a.x_prev == nullptr;
+    if (gather) kargs_rest(a);                            // the first layer's rows: emb, tokens
+    const uint32_t tok = gather ? a.tokens[r] : 0u;
+    const bool padded = gather && a.zero_rows && tok == ZERO_ROW_TOKEN;      // zero rows past the end of a sequence
+    const float *base = gather ? a.emb + (size_t)(padded ? 0u : tok) * D : a.x_prev + r * D;
     size_t rows[MAXV]; int cols[MAXV]; bool ok[MAXV];
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
@@ -76,9 +83,10 @@ __global__ __launch_bounds__(NT) void k_norm_rows(NormRowsArgs a)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv && !padded) x[t] = ld4(base + 4 * v);
     }
+    if (!gather) kargs_rest(a);                           // everything else, asked for behind the row's own loads
     if (a.branch.S > 0) // (many rows: a plane per round trip and 48 registers, so that eight workgroups fit a CU: 25.5 -> 22.7 us at 2048 x 2560)
     planes_at4_multi<MAXV, (MAXV == 1 ? 20 : NT == RB ? 6 : 1), GROUPED>(a.branch, rows, cols, ok, b);
-    if (a.emb && a.emb_scale != 1.0f) {
+    if (gather && a.emb_scale != 1.0f) {
 #pragma unroll
         for (int t = 0; t < MAXV; t++) { x[t].x *= a.emb_scale; x[t].y *= a.emb_scale; x[t].z *= a.emb_scale; x[t].w *= a.emb_scale; }
     }
@@ -831,8 +839,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
 constexpr int MAXC = 2;                                   // float4 per thread of a column-group workgroup
 constexpr int GC_MAX = 512;                               // its threads: 256 for groups of up to 2048 columns, 512 up to 4096
 template <int GELU, int GC>                               // compile-time: the kernel's code stays one straight run
-__global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
+__global__ __launch_bounds__(GC) void k_glu_fwd_cols(KARGS16)
 {
+    KARGS_HOT(GluArgs, a);                                // in, gate_pre, IS, sg.cols
     __shared__ float sm[16];
     const size_t r = blockIdx.x;
     const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(IS, c0 + a.sg.cols) - c0, nv = width >> 2;
@@ -845,6 +854,7 @@ __global__ __launch_bounds__(GC) void k_glu_fwd_cols(GluArgs a)
             const int v = threadIdx.x + t * GC;
             rows[t] = rows[MAXC + t] = r; cols[t] = c0 + 4 * v; cols[MAXC + t] = IS + c0 + 4 * v; ok[t] = ok[MAXC + t] = v < nv;
         }
+        kargs_rest(a);                                    // asked for beside the planes
         planes_at4_multi<2 * MAXC, 3>(a.in, rows, cols, ok, gu);
     }
 #pragma unroll
@@ -934,8 +944,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
 // in k_glu_fwd_cols.  A group may lie in either half or straddle the middle, so a thread computes the half its output
 // column belongs to; the inputs of a column are then read twice in all, by different workgroups.
 template <int GELU, int GC>
-__global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
+__global__ __launch_bounds__(GC) void k_glu_bwd_cols(KARGS16)
 {
+    KARGS_HOT(GluArgs, a);                                // in, gate_pre, IS, sg.cols; up_val = gate_pre + IS and ld_gu = 2 IS (checked by the launcher)
     __shared__ float sm[16];
     const size_t r = blockIdx.x;
     const int IS = a.IS, c0 = blockIdx.y * a.sg.cols, width = min(2 * IS, c0 + a.sg.cols) - c0, nv = width >> 2;
@@ -948,8 +959,9 @@ __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
             const int v = threadIdx.x + t * GC, j = c0 + 4 * v;
             rows[t] = r; cols[t] = j < IS ? j : j - IS; ok[t] = v < nv;
             gs[t] = us[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (v < nv) { gs[t] = ld4(a.gate_pre + r * a.ld_gu + cols[t]); us[t] = ld4(a.up_val + r * a.ld_gu + cols[t]); }
+            if (v < nv) { gs[t] = ld4(a.gate_pre + r * (size_t)(2 * IS) + cols[t]); us[t] = ld4(a.gate_pre + r * (size_t)(2 * IS) + IS + cols[t]); }
         }
+        kargs_rest(a);
         planes_at4_multi<MAXC, 5>(a.in, rows, cols, ok, dys);
     }
 #pragma unroll
@@ -983,10 +995,12 @@ __global__ __launch_bounds__(GC) void k_glu_bwd_cols(GluArgs a)
 // itself (Qwen3) or RNB(branch_raw, dx_out; g_branch) (Gemma3's post-norms,
 // src/nn/fast_sft.c:798-802, 877-881).
 template <int MAXV, bool GROUPED, int NT = RB>
-__global__ __launch_bounds__(NT) void k_norm_bwd_rows(NormBwdArgs a)
+__global__ __launch_bounds__(NT) void k_norm_bwd_rows(KARGS24)
 {
+    KARGS_HOT(NormBwdArgs, a);                            // rows_launched, D, x_saved, dy
     __shared__ float sm[32];
     if (blockIdx.x >= a.rows_launched) {
+        kargs_rest(a);
         prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
@@ -1000,9 +1014,12 @@ __global__ __launch_bounds__(NT) void k_norm_bwd_rows(NormBwdArgs a)
         const int v = threadIdx.x + t * NT;
         x[t] = g[t] = make_float4(0.f, 0.f, 0.f, 0.f);
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
-        if (v < nv) { x[t] = ld4(a.x_saved + r * D + 4 * v); g[t] = ld4(a.g + 4 * v); }
+        if (v < nv) x[t] = ld4(a.x_saved + r * D + 4 * v);
     }
+    kargs_rest(a);                                        // (g is not among the preloaded arguments: asked for behind the row's own loads)
     planes_at4_multi<MAXV, (MAXV == 1 ? 20 : NT == RB ? 4 : 3), GROUPED>(a.dy, rows, cols, ok, dy);      // (many rows: 92 registers instead of 108)
+#pragma unroll
+    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) g[t] = ld4(a.g + 4 * v); }
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         ss += sumsq4(x[t]);
@@ -1305,6 +1322,9 @@ __global__ void k_fill_f32(float *p, float v, size_t n)
 
 #define LAUNCH(kern, grid, block, lds, ...) do { \
     hipLaunchKernelGGL(kern, grid, block, lds, stream(), __VA_ARGS__); HIP_CHECK(hipGetLastError()); } while (0)
+// a kernel declared with KARGS<NQ> (kargs.h): its argument struct travels as NQ scalar words
+#define LAUNCHK(NQ, kern, grid, block, lds, args) do { \
+    launch_kargs<NQ>(kern, grid, block, lds, stream(), args); HIP_CHECK(hipGetLastError()); } while (0)
 
 void require(bool ok, const char *what)
 {
@@ -1317,13 +1337,14 @@ void launch_norm_rows(const NormRowsArgs &a, int rows)
 {
     require(a.D > 0 && a.D % 4 == 0 && a.D <= 4 * RB * MAXV, "norm_rows: hidden size must be a multiple of 4, <= 12288");
     require(a.branch.S == 0 || a.branch.ld % 4 == 0, "norm_rows: plane row length must be a multiple of 4");
+    require((a.emb != nullptr) != (a.x_prev != nullptr), "norm_rows: the row is either gathered (emb) or read (x_prev)");
     const bool grouped = a.branch.S > 0 && a.branch.scale_groups != 0;
     NormRowsArgs b = a;
     b.rows_launched = rows;
     const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
-    if (rows >= MANY_ROWS && !grouped && !a.pf.base && a.D <= 4 * TB * MAXV_ROW) { LAUNCH((k_norm_rows<MAXV_ROW, false, TB>), grid, dim3(TB), 0, b); return; }
-    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_rows<1, false>), grid, dim3(RB), 0, b); }
-    else { if (grouped) LAUNCH((k_norm_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
+    if (rows >= MANY_ROWS && !grouped && !a.pf.base && a.D <= 4 * TB * MAXV_ROW) { LAUNCHK(24, (k_norm_rows<MAXV_ROW, false, TB>), grid, dim3(TB), 0, b); return; }
+    if (a.D <= 4 * RB) { if (grouped) LAUNCHK(24, (k_norm_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCHK(24, (k_norm_rows<1, false>), grid, dim3(RB), 0, b); }
+    else { if (grouped) LAUNCHK(24, (k_norm_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCHK(24, (k_norm_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
 }
 
 void launch_rope_table(float2 *tab, int seq, int hd, float theta)
@@ -1414,11 +1435,11 @@ void launch_glu_fwd(const GluArgs &a, int rows)
         require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC_MAX * MAXC && (long)a.sg.cols * a.sg.groups >= a.IS && (long)a.sg.cols * (a.sg.groups - 1) < a.IS,
                 "glu_fwd: column groups do not fit the row");
         if (a.sg.cols <= 4 * 256 * MAXC) {
-            if (a.gelu) LAUNCH((k_glu_fwd_cols<1, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
-            else LAUNCH((k_glu_fwd_cols<0, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+            if (a.gelu) LAUNCHK(16, (k_glu_fwd_cols<1, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+            else LAUNCHK(16, (k_glu_fwd_cols<0, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
         } else {
-            if (a.gelu) LAUNCH((k_glu_fwd_cols<1, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
-            else LAUNCH((k_glu_fwd_cols<0, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+            if (a.gelu) LAUNCHK(16, (k_glu_fwd_cols<1, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+            else LAUNCHK(16, (k_glu_fwd_cols<0, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
         }
         return;
     }
@@ -1434,12 +1455,13 @@ void launch_glu_bwd(const GluArgs &a, int rows)
     if (a.sg.cols) {
         require(a.sg.cols % 64 == 0 && a.sg.cols <= 4 * GC_MAX * MAXC && (long)a.sg.cols * a.sg.groups >= 2 * a.IS && (long)a.sg.cols * (a.sg.groups - 1) < 2 * a.IS,
                 "glu_bwd: column groups do not fit the row");
+        require(a.ld_gu == (size_t)2 * a.IS && a.up_val == a.gate_pre + a.IS, "glu_bwd: gate and up are kept as one [rows][2 IS] array");
         if (a.sg.cols <= 4 * 256 * MAXC) {
-            if (a.gelu) LAUNCH((k_glu_bwd_cols<1, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
-            else LAUNCH((k_glu_bwd_cols<0, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+            if (a.gelu) LAUNCHK(16, (k_glu_bwd_cols<1, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
+            else LAUNCHK(16, (k_glu_bwd_cols<0, 256>), dim3(rows, a.sg.groups), dim3(256), 0, a);
         } else {
-            if (a.gelu) LAUNCH((k_glu_bwd_cols<1, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
-            else LAUNCH((k_glu_bwd_cols<0, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+            if (a.gelu) LAUNCHK(16, (k_glu_bwd_cols<1, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
+            else LAUNCHK(16, (k_glu_bwd_cols<0, 512>), dim3(rows, a.sg.groups), dim3(512), 0, a);
         }
         return;
     }
@@ -1454,9 +1476,9 @@ void launch_norm_bwd_rows(const NormBwdArgs &a, int rows)
     NormBwdArgs b = a;
     b.rows_launched = rows;
     const dim3 grid(rows + (a.pf.base ? a.pf.wgs : 0));
-    if (rows >= MANY_ROWS && !grouped && !a.pf.base && a.D <= 4 * TB * MAXV_ROW) { LAUNCH((k_norm_bwd_rows<MAXV_ROW, false, TB>), grid, dim3(TB), 0, b); return; }
-    if (a.D <= 4 * RB) { if (grouped) LAUNCH((k_norm_bwd_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_bwd_rows<1, false>), grid, dim3(RB), 0, b); }
-    else { if (grouped) LAUNCH((k_norm_bwd_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCH((k_norm_bwd_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
+    if (rows >= MANY_ROWS && !grouped && !a.pf.base && a.D <= 4 * TB * MAXV_ROW) { LAUNCHK(24, (k_norm_bwd_rows<MAXV_ROW, false, TB>), grid, dim3(TB), 0, b); return; }
+    if (a.D <= 4 * RB) { if (grouped) LAUNCHK(24, (k_norm_bwd_rows<1, true>), grid, dim3(RB), 0, b); else LAUNCHK(24, (k_norm_bwd_rows<1, false>), grid, dim3(RB), 0, b); }
+    else { if (grouped) LAUNCHK(24, (k_norm_bwd_rows<MAXV_ROW, true>), grid, dim3(RB), 0, b); else LAUNCHK(24, (k_norm_bwd_rows<MAXV_ROW, false>), grid, dim3(RB), 0, b); }
 }
 
 void launch_ce_rows(const CeArgs &a, int rows)

@@ -377,11 +377,9 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         g.A = reinterpret_cast<const half8 *>(A); g.a_inv_scale = a_inv_scale; g.W = W;
         g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
         g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
-        g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1; g.half_scale = half_scale;
+        g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1; g.half_scale = half_scale; g.w16_ring = W.w16;
         const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(256 * p.kg);
-#define RING_LAUNCH(KGV, SC, HP) do { \
-            if (g_prof_on) hipExtLaunchKernelGGL((gemm_ring<KGV, SC, HP>), rgrid, rblock, 0, stream(), ra, rb, 0, g); \
-            else hipLaunchKernelGGL((gemm_ring<KGV, SC, HP>), rgrid, rblock, 0, stream(), g); } while (0)
+#define RING_LAUNCH(KGV, SC, HP) launch_kargs<24>(gemm_ring<KGV, SC, HP>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
 #define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1, 0); else if (half_scale != 0.f) RING_LAUNCH(KGV, 0, 1); else RING_LAUNCH(KGV, 0, 0); } while (0)
         if (p.kg == 1) RING_PICK(1); else if (p.kg == 2) RING_PICK(2); else RING_PICK(4);
 #undef RING_PICK

@@ -1,16 +1,21 @@
 // The weight-streaming GEMM kernel (device code only; included by gemm.hip).
 #pragma once
+#include "kargs.h"
 #include "devutil.h"
 #include "gemm.h"
 
 namespace lmhip {
 
+// (ordered for kargs.h: what gemm_ring needs to request its first stages lies in the first 56 bytes)
 struct GemmKArgs {
-    const half8 *A; const float *a_inv_scale;
+    const half8 *A;
+    const half_t *w16_ring;                              // W.w16 once more, for gemm_ring
+    int Kb, Nb, Mb, n_tiles, steps_per_chunk, M;
+    int N, S, m_tiles;                                   // (m_tiles > 1: the grid is the 1-D one described at gemm_tiled)
+    int ldp;
+    const float *a_inv_scale;
     WeightOp W;
-    float *P; int ldp; size_t plane_stride;
-    int M, N, Mb, Nb, Kb, steps_per_chunk;
-    int n_tiles, S, m_tiles;                             // set (m_tiles > 1) when the grid is the 1-D one described at gemm_tiled
+    float *P; size_t plane_stride;
     float half_scale;                                    // gemm_ring<.., .., 1>: the planes are halves, each sum times this power of two
 };
 
@@ -275,9 +280,11 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 // the weight matrix so that no sum of 8192-bounded operand values can pass the fp16 maximum; plane_stride and ldp then
 // count halves.  Half the bytes to write here and for the consumer to read; 11 significant bits per chunk sum.
 template <int KG, int SCALE, int HALFP = 0>
-__global__ __launch_bounds__(256 * KG) void gemm_ring(GemmKArgs g)
+__global__ __launch_bounds__(256 * KG) void gemm_ring(KARGS24)
 {
     static_assert(!(SCALE && HALFP), "final outputs stay fp32");
+    const uint64_t kw[24] = {KLIST24};
+    const GemmKArgs g = kargs_unpack<GemmKArgs>(kw);
     static_assert(KG == 1 || KG == 2 || KG == 4, "K groups per workgroup");
     constexpr int LOADS_PER_ROUND = 4;                    // LDS-direct loads a wave issues per round: the four 1 KB pieces of its block
     __shared__ half8 ring[2 * KG * 1024];                 // [round parity][K group][block 0..3][slice 0..3][64 lanes]
@@ -289,7 +296,7 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(GemmKArgs g)
     const int nsteps = min(g.Kb, kb_beg + g.steps_per_chunk) - kb_beg;
     const int rounds = (nsteps + KG - 1) / KG;
     // q = 0, 1: weight row blocks 2 tile + q; q = 2, 3: activation row blocks q - 2 (clamped: rows beyond M or N are not stored)
-    const half8 *src = q < 2 ? reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)min(2 * tile + q, g.Nb - 1) * g.Kb + kb_beg) * 256 + lane
+    const half8 *src = q < 2 ? reinterpret_cast<const half8 *>(g.w16_ring) + ((size_t)min(2 * tile + q, g.Nb - 1) * g.Kb + kb_beg) * 256 + lane
                              : g.A + ((size_t)min(q - 2, g.Mb - 1) * g.Kb + kb_beg) * 256 + a_lane(lane);
     const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)ring;
     auto request = [&](int round) __attribute__((always_inline)) {

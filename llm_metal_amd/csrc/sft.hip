@@ -315,7 +315,7 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
         const size_t stride = (size_t)s->BN * N;
         if (!out && chunks * stride > s->planes_cap) { fprintf(stderr, "[fast_sft] plane buffer too small\n"); abort(); }
         const int planes = launch_gemm_big(A, inv, Wf, C, N, s->BN, N, K, chunks, stride);
-        return Planes{C, planes, stride, N, nullptr};
+        return make_planes(C, planes, stride, N, nullptr);
     }
     GemmPlan p = plan_gemm(s->BN, N, K, (W.fmt == 1 && W.nbq < tiled_rb(N)) ? W.nbq : 0, W.fmt);
     float *P = out ? out : at<float>(s->planes);
@@ -330,9 +330,9 @@ Planes gemm(SFTState *s, const half_t *A, const float *inv, const WeightOp &W, i
         if (out || sg->cols != (p.steps * 64) << sg->shift || sg->groups != (p.S + (1 << sg->shift) - 1) >> sg->shift) {
             fprintf(stderr, "[fast_sft] column groups of the operand do not match the K chunks of the product\n"); abort();
         }
-        return Planes{P, p.S, stride, N, inv, sg->shift, sg->groups, unscale};
+        return make_planes(P, p.S, stride, N, inv, sg->shift, sg->groups, unscale);
     }
-    return Planes{P, p.S, stride, N, out ? nullptr : inv, 0, 0, unscale};
+    return make_planes(P, p.S, stride, N, out ? nullptr : inv, 0, 0, unscale);
 }
 
 void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
@@ -342,7 +342,7 @@ void forward_impl(SFTState *s, bool gather, bool zero_rows = false)
     half_t *a16 = at<half_t>(s->a16);
     float *ainv = at<float>(s->a16_inv);
     const bool gemma = s->model_type == MODEL_GEMMA3;
-    Planes pending{nullptr, 0, 0, 0, nullptr};                    // FFN output of the previous layer, not yet added
+    Planes pending = make_planes(nullptr, 0, 0, 0, nullptr);                    // FFN output of the previous layer, not yet added
 
     for (int L = 0; L < s->NL; L++) {
         float *x_in = at<float>(s->xs, (size_t)(2 * L) * xsz), *x_mid = at<float>(s->xs, (size_t)(2 * L + 1) * xsz);
