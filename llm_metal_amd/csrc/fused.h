@@ -3,6 +3,7 @@
 // activations that feed a GEMM are produced directly as scaled fp16 rows, GEMM
 // outputs arrive as K-split partial planes that the consumer sums on load.
 #pragma once
+#include <cstddef>
 #include <stdio.h>
 #include <stdlib.h>
 #include "backend.h"
@@ -62,9 +63,11 @@ struct WeightPrefetch {
 constexpr uint32_t ZERO_ROW_TOKEN = 0xFFFFFFFFu;
 
 struct NormRowsArgs {
-    // (the first 56 bytes reach the kernel preloaded: what it needs to ask for the branch's planes and the row)
+    // (the first 56 bytes reach the kernel preloaded: all that the workgroups beyond the rows need, which ask for the next
+    // product's weights and are the last to finish; the rows' workgroups read the rest from the argument segment)
     int rows_launched;            // set by the launcher
     int D;
+    WeightPrefetch pf;
     const float *x_prev;          // source of the residual stream row, unless it is gathered (emb != null)
     // optional branch added to it: planes, optionally RMS-normalised with g_branch first
     Planes branch;
@@ -75,8 +78,8 @@ struct NormRowsArgs {
     const float *g_norm;          // null: no normalised output wanted
     half_t *ln16; float *inv_scale;   // tiled [rows, D]
     float eps;
-    WeightPrefetch pf;
 };
+static_assert(offsetof(NormRowsArgs, x_prev) == 56, "NormRowsArgs: preloaded part");
 void launch_norm_rows(const NormRowsArgs &a, int rows);
 
 // The matrix-core attention reads K and V once more from copies laid out [batch][Hkv][hd/4][attn_ldt(seq)][4]:
@@ -206,14 +209,15 @@ void launch_glu_bwd(const GluArgs &a, int rows);
 
 struct NormBwdArgs {
     int rows_launched; int D;                           // (first 56 bytes: preloaded, see NormRowsArgs)
+    WeightPrefetch pf;
     const float *x_saved;
     Planes dy;
     const float *g; float eps;
     const float *dx_prev; float *dx_out; float clamp;   // clamp <= 0: none
     const float *branch_raw, *g_branch;                 // Gemma3: next GEMM input is RNB(branch_raw, dx_out)
     half_t *d16; float *inv_scale;                      // tiled [rows, D]; may be null on the last kernel of the backward
-    WeightPrefetch pf;
 };
+static_assert(offsetof(NormBwdArgs, x_saved) == 56, "NormBwdArgs: preloaded part");
 void launch_norm_bwd_rows(const NormBwdArgs &a, int rows);
 
 struct CeArgs {

@@ -58,20 +58,17 @@ __device__ __forceinline__ void write_f16_tiled(const float *vals, int n, half_t
 template <int MAXV, bool GROUPED, int NT = RB>
 __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
 {
-    KARGS_HOT(NormRowsArgs, a);                           // rows_launched, D, x_prev, branch
+    KARGS_HOT(NormRowsArgs, a);                           // rows_launched, D, pf
     __shared__ float sm[16];
-    if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights
-        kargs_rest(a);
-        prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
+    if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights; they are the last
+        prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);      // to finish and have nothing to wait for
         return;
     }
+    kargs_rest(a);
     const size_t r = xcd_block_row(blockIdx.x, a.rows_launched);
     const int D = a.D, nv = D >> 2;
     float4 x[MAXV], b[MAXV];
-    // (x_prev, D and the branch's planes arrive preloaded: a row that is not gathered asks for all its data without
-    // waiting for the rest of the arguments)
     const bool gather = a.x_prev == nullptr;
-    if (gather) kargs_rest(a);                            // the first layer's rows: emb, tokens
     const uint32_t tok = gather ? a.tokens[r] : 0u;
     const bool padded = gather && a.zero_rows && tok == ZERO_ROW_TOKEN;      // zero rows past the end of a sequence
     const float *base = gather ? a.emb + (size_t)(padded ? 0u : tok) * D : a.x_prev + r * D;
@@ -83,7 +80,6 @@ __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv && !padded) x[t] = ld4(base + 4 * v);
     }
-    if (!gather) kargs_rest(a);                           // everything else, asked for behind the row's own loads
     if (a.branch.S > 0) // (many rows: a plane per round trip and 48 registers, so that eight workgroups fit a CU: 25.5 -> 22.7 us at 2048 x 2560)
     planes_at4_multi<MAXV, (MAXV == 1 ? 20 : NT == RB ? 6 : 1), GROUPED>(a.branch, rows, cols, ok, b);
     if (gather && a.emb_scale != 1.0f) {
@@ -997,13 +993,13 @@ __global__ __launch_bounds__(GC) void k_glu_bwd_cols(KARGS16)
 template <int MAXV, bool GROUPED, int NT = RB>
 __global__ __launch_bounds__(NT) void k_norm_bwd_rows(KARGS24)
 {
-    KARGS_HOT(NormBwdArgs, a);                            // rows_launched, D, x_saved, dy
+    KARGS_HOT(NormBwdArgs, a);                            // rows_launched, D, pf
     __shared__ float sm[32];
-    if (blockIdx.x >= a.rows_launched) {
-        kargs_rest(a);
+    if (blockIdx.x >= a.rows_launched) {                  // these set the kernel's duration: nothing to wait for
         prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);
         return;
     }
+    kargs_rest(a);
     const size_t r = xcd_block_row(blockIdx.x, a.rows_launched);
     const int D = a.D, nv = D >> 2;
     float4 dy[MAXV], x[MAXV], g[MAXV];
@@ -1016,7 +1012,6 @@ __global__ __launch_bounds__(NT) void k_norm_bwd_rows(KARGS24)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv) x[t] = ld4(a.x_saved + r * D + 4 * v);
     }
-    kargs_rest(a);                                        // (g is not among the preloaded arguments: asked for behind the row's own loads)
     planes_at4_multi<MAXV, (MAXV == 1 ? 20 : NT == RB ? 4 : 3), GROUPED>(a.dy, rows, cols, ok, dy);      // (many rows: 92 registers instead of 108)
 #pragma unroll
     for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) g[t] = ld4(a.g + 4 * v); }
