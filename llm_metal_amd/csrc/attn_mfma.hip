@@ -213,11 +213,14 @@ __device__ __forceinline__ void load_probs(float4 (&p)[M32], const AttnTileArgs 
     }
 }
 
-// DKV (dQ only): the probabilities go to LDS as well (Ps, laid out like the finished rows of Xs), for the dV share
-// formed after phase 3, and dscore stays out of memory: nothing reads it.
+// DKV (dQ only): dS and the probabilities also go to LDS by key (Ts: four images -- upper and lower parts of dS, then of
+// P -- of [keys][DKV_TS] halves each, 32 query rows and padding per key), for the shares of dK and dV formed after phase
+// 3, whose matrix-core operands are eight consecutive query rows of one key: one 16-byte read each.  dscore stays out of
+// memory: nothing reads it.
+constexpr int DKV_TS = 40;                                 // halves per key: 80 bytes apart, so that eight lanes' 16-byte reads cover all banks
 template <int BWD, int M32, int DKV = 0>
 __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int ldx, int xlo, int nk, int N, int i0, int b, int h, int tid,
-                                         const float4 (&p_early)[BWD ? M32 : 1], float *Ps = nullptr)
+                                         const float4 (&p_early)[BWD ? M32 : 1], uint16_t *Ts = nullptr)
 {
     const int rr = tid >> 3, part = tid & 7, i = i0 + rr;
     const bool row_ok = i < N;
@@ -273,10 +276,14 @@ __device__ __forceinline__ void row_step(const AttnTileArgs &a, float *Xs, int l
             *reinterpret_cast<u32x2 *>(xh) = u32x2{pack_hi(o.x, o.y), pack_hi(o.z, o.w)};
             *reinterpret_cast<u32x2 *>(xh + xlo) = u32x2{pack_hi(rest(o.x), rest(o.y)), pack_hi(rest(o.z), rest(o.w))};
             if constexpr (BWD && DKV) {
-                const float4 pv = p[m];
-                __bf16 *ph = reinterpret_cast<__bf16 *>(Ps + rr * ldx) + j;
-                *reinterpret_cast<u32x2 *>(ph) = u32x2{pack_hi(pv.x, pv.y), pack_hi(pv.z, pv.w)};
-                *reinterpret_cast<u32x2 *>(ph + xlo) = u32x2{pack_hi(rest(pv.x), rest(pv.y)), pack_hi(rest(pv.z), rest(pv.w))};
+                const float ov[4] = {o.x, o.y, o.z, o.w}, pv[4] = {p[m].x, p[m].y, p[m].z, p[m].w};
+                const int img = xlo * DKV_TS;                          // xlo: the keys rounded up to 32
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    uint16_t *t = Ts + (j + c) * DKV_TS + rr;
+                    t[0] = (uint16_t)(__float_as_uint(ov[c]) >> 16); t[img] = (uint16_t)(__float_as_uint(rest(ov[c])) >> 16);
+                    t[2 * img] = (uint16_t)(__float_as_uint(pv[c]) >> 16); t[3 * img] = (uint16_t)(__float_as_uint(rest(pv[c])) >> 16);
+                }
             }
         }
         if (!DKV && row_ok && j < N) {
@@ -309,10 +316,10 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     const int N32 = (N + 31) & ~31, ldx = N32 + 4;
     __bf16 *Ahi = reinterpret_cast<__bf16 *>(lds), *Alo = Ahi + 32 * lda;
     float *Xs = lds + 32 * lda;                           // behind the two bf16 images of A
-    float *Ps = Xs + 32 * ldx;                            // DKV only
+    uint16_t *Ts = reinterpret_cast<uint16_t *>(Xs + 32 * ldx);      // DKV only: dS and P by key (row_step)
 
     // ---- the first B pass and the first C chunk of this wave do not depend on anything computed here:
-    //      request them before the A rows are staged (waves without a tile of their own read tile 0)
+    //      request them before the A rows are staged
     // Work items of a wave in phase 1: (key block jb = wave + 4 (q / NCB), column pass c = q % NCB), q = 0 .. nitems - 1.
     // This lane's part of the transposed B matrix for an item: key jb * 32 + l31, columns c * CB + hh * CB/2 ...
     constexpr int CB = HD > 128 ? 128 : HD, NCB = HD / CB;
@@ -325,7 +332,7 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
         return a.BT + ((((size_t)b * a.Hkv + hk) * (HD / 4) + c * (CB / 4) + hh * (CB / 8)) * ldt + min(jb * 32 + l31, N - 1)) * 4;
     };
     BTile<CB> bt0, bt1;
-    b_tile_load<CB>(bt0, b_item(0), ldt);
+    if (nitems) b_tile_load<CB>(bt0, b_item(0), ldt);     // (uniform per wave; a wave without an item asks for nothing)
     float4 p_early[BWD ? M32 : 1];
     if constexpr (BWD && M32 <= 8) load_probs<M32>(p_early, a, N, i0, b, h, tid);
     // DKV: this lane's q values for the shares formed at the end (query rows 16 u + 8 hh + e of the block, head column
@@ -357,7 +364,9 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
                 const int idx = tid + 256 * u, rr = idx / (HD >> 2), c4 = idx % (HD >> 2);
                 ok[u] = i0 + rr < N; rows[u] = r0 + (ok[u] ? i0 + rr : 0); cols[u] = h * HD + 4 * c4;
             }
-            planes_at4_multi<HD / 32, (HD <= 128 ? 5 : 3)>(a.Apl, rows, cols, ok, av);
+            // (a head of 256 columns: eight positions per thread; planes of halves take half the registers, so ten of
+            // them -- the chunks of the short products of a model with such heads -- travel in one round trip)
+            planes_at4_multi<HD / 32, (HD <= 128 ? 5 : 3), false, (HD <= 128 ? 5 : 5)>(a.Apl, rows, cols, ok, av);
         } else {
 #pragma unroll
             for (int u = 0; u < HD / 32; u++) {
@@ -375,6 +384,11 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
         }
     }
     __syncthreads();
+    // a head of 256 columns at up to 64 keys: the C values of the wave's second column block are asked for now and
+    // arrive during phase 1 and the row step (at the start of the kernel they would not fit among a wave's 63 loads in flight)
+    constexpr bool RING2 = HD > 128 && M32 == 2;
+    CRing cring2;
+    if constexpr (RING2) c_ring_start<M32>(cring2, c_lane0 + (wave + 4) * 32, (size_t)kd, nk, hh, N);
 
     // ---- phase 1: X = A B^T, one 32-key block per wave and round; the B values of the next item are on their way
     auto put_x = [&](const float16v &acc, int jb) {
@@ -409,16 +423,12 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
     __syncthreads();
 
     // ---- row step
-    row_step<BWD, M32, DKV>(a, Xs, ldx, N32, nk, N, i0, b, h, tid, p_early, Ps);    // whole rows of N entries are written
+    row_step<BWD, M32, DKV>(a, Xs, ldx, N32, nk, N, i0, b, h, tid, p_early, Ts);    // whole rows of N entries are written
     __syncthreads();
 
     // ---- phase 3: Y = X C, one 32-column block of the head per wave and round
     const int Kb = tiled_kb(qd);
-    for (int dt = wave; dt * 32 < HD; dt += 4) {
-        if (dt != wave) c_ring_start<M32>(cring, c_lane0 + dt * 32, (size_t)kd, nk, hh, N);
-        float16v acc;
-        if constexpr (M32 == 2) acc = tile_xc_2(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, lane, cring);
-        else acc = tile_xc(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
+    auto put_y = [&](const float16v &acc, int dt) __attribute__((always_inline)) {
         const int d = dt * 32 + l31;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
@@ -427,15 +437,26 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
             if (BWD) a.out32[(r0 + i) * qd + h * HD + d] = acc[v];
             else a.out16[tiled_a_index((int)(r0 + i), h * HD + d, Kb)] = f2h(acc[v]);
         }
+    };
+    if constexpr (RING2) {
+        put_y(tile_xc_2(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, lane, cring), wave);
+        put_y(tile_xc_2(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, lane, cring2), wave + 4);
+    } else {
+        for (int dt = wave; dt * 32 < HD; dt += 4) {
+            if (dt != wave) c_ring_start<M32>(cring, c_lane0 + dt * 32, (size_t)kd, nk, hh, N);
+            float16v acc;
+            if constexpr (M32 == 2) acc = tile_xc_2(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, lane, cring);
+            else acc = tile_xc(reinterpret_cast<const __bf16 *>(Xs), 2 * ldx, N32, nk, c_lane0 + dt * 32, (size_t)kd, N, lane, cring);
+            put_y(acc, dt);
+        }
     }
     if constexpr (BWD && DKV) {
         // ---- the block's share of dK and dV of its query head, for the keys it sees:
         //      dKp[j, d] = sum_{i in block} dS[i, j] q[i, d],   dVp[j, d] = sum_{i in block} P[i, j] dO[i, d].
         // A wave takes the head columns dt * 32 ..; in an instruction lane (l31, hh) reduces over the query rows
-        // 16 u + 8 hh + 0..7 of the block: its key's dS / P values come from LDS a row apart each (the finished rows
-        // are stored by query), dO likewise from the staged A rows, q from memory.
-        const __bf16 *Xh = reinterpret_cast<const __bf16 *>(Xs), *Ph = reinterpret_cast<const __bf16 *>(Ps);
-        const int ldh = 2 * ldx;
+        // 16 u + 8 hh + 0..7 of the block: its key's dS / P values are eight consecutive halves of the images by key,
+        // dO comes from the staged A rows a row apart each, q from memory.
+        const int img = N32 * DKV_TS;
 #pragma unroll
         for (int t = 0; t < NDT; t++) {
             const int dt = wave + 4 * t;
@@ -457,13 +478,11 @@ __global__ __launch_bounds__(256) void k_attn_tile(AttnTileArgs a)
             for (int jb = 0; jb < nkb; jb++) {
                 HL sA[2], pA[2];
 #pragma unroll
-                for (int u = 0; u < 2; u++)
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const int o = (16 * u + 8 * hh + e) * ldh + jb * 32 + l31;
-                        sA[u].hi[e] = Xh[o]; sA[u].lo[e] = Xh[o + N32];
-                        pA[u].hi[e] = Ph[o]; pA[u].lo[e] = Ph[o + N32];
-                    }
+                for (int u = 0; u < 2; u++) {
+                    const uint16_t *t = Ts + (jb * 32 + l31) * DKV_TS + 16 * u + 8 * hh;
+                    sA[u].hi = *reinterpret_cast<const bf16x8 *>(t); sA[u].lo = *reinterpret_cast<const bf16x8 *>(t + img);
+                    pA[u].hi = *reinterpret_cast<const bf16x8 *>(t + 2 * img); pA[u].lo = *reinterpret_cast<const bf16x8 *>(t + 3 * img);
+                }
                 float16v aK = zero16(), aV = zero16();
 #pragma unroll
                 for (int u = 0; u < 2; u++) { mfma3(aK, sA[u], qB[u]); mfma3(aV, pA[u], oB[u]); }
@@ -550,7 +569,11 @@ __global__ __launch_bounds__(256) void k_attn_dkv_tile(AttnDkvArgs a)
     }
 }
 
-size_t tile_lds_bytes(int hd, int seq, int dkv = 0) { return (size_t)32 * (hd + 8 + (1 + dkv) * (((seq + 31) & ~31) + 4)) * sizeof(float); }
+size_t tile_lds_bytes(int hd, int seq, int dkv = 0)
+{
+    const size_t n32 = (seq + 31) & ~31;
+    return (size_t)32 * (hd + 8 + n32 + 4) * sizeof(float) + (dkv ? 4 * n32 * DKV_TS * sizeof(uint16_t) : 0);
+}
 
 template <int BWD, int HD, int M32, int DKV = 0>
 void launch_tile_m(const AttnTileArgs &a)

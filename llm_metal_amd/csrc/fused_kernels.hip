@@ -431,28 +431,36 @@ __global__ __launch_bounds__(TB) void k_attn_bwd_dkv(AttnBwdArgs a)
 // hundred rows on, as in k_norm_rows).
 // dk or dv of (row, KV head hk, column d) from the shares the one-launch attention backward leaves
 // ([query block][Hq][rows_total][hd]): the query heads of the group, and the query blocks that see the key
-__device__ __forceinline__ float kv_share_sum(const QkvBwdArgs &a, const float *shares, size_t row, int pos, int hk, int d)
+// U elements of a thread at once (element u: shares[u], KV head hk[u], column d[u]; skipped unless on[u]): the loads of all
+// of them are issued before the first sum, one memory round trip per four query heads of the group for all U.
+template <int U>
+__device__ __forceinline__ void kv_share_sums(const QkvBwdArgs &a, const float *const (&shares)[U], size_t row, int pos, const int (&hk)[U],
+                                              const int (&d)[U], const bool (&on)[U], float (&s)[U])
 {
     const int ratio = a.Hq / a.Hkv, nqb = (a.seq + 31) >> 5;
-    float v[2][4];
-    float s = 0.f;
     const size_t st_h = (size_t)a.rows_total * a.hd, st_qb = st_h * a.Hq;
-    const float *p = shares + ((size_t)hk * ratio * a.rows_total + row) * a.hd + d;
     const int qb0 = pos >> 5;
+    const float *p[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) { p[u] = shares[u] + ((size_t)hk[u] * ratio * a.rows_total + row) * a.hd + d[u]; s[u] = 0.f; }
     for (int g0 = 0; g0 < ratio; g0 += 4) {
+        float v[U][2][4];
 #pragma unroll
-        for (int q = 0; q < 2; q++)
+        for (int u = 0; u < U; u++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const bool ok = qb0 + q < nqb && g0 + g < ratio;
-                v[q][g] = ok ? p[(size_t)(qb0 + q) * st_qb + (size_t)(g0 + g) * st_h] : 0.f;
-            }
+            for (int q = 0; q < 2; q++)
 #pragma unroll
-        for (int q = 0; q < 2; q++)
+                for (int g = 0; g < 4; g++) {
+                    const bool ok = on[u] && qb0 + q < nqb && g0 + g < ratio;
+                    v[u][q][g] = ok ? p[u][(size_t)(qb0 + q) * st_qb + (size_t)(g0 + g) * st_h] : 0.f;
+                }
 #pragma unroll
-            for (int g = 0; g < 4; g++) s += v[q][g];
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int q = 0; q < 2; q++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) s[u] += v[u][q][g];
     }
-    return s;
 }
 
 template <int NP, int RK, int NT = RB>
@@ -476,6 +484,7 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
     const int nslots = a.Hq + a.Hkv;
     float g0[SU][NP], g1[SU][NP], p0[SU][NP], p1[SU][NP], w0[SU][NP], w1[SU][NP];
     float2 cs[NP];
+    float amax = 0.f;                                      // over what this thread puts into the row's final values
     // the loads of one trip; with `defer_shares` the dk values of a K head are left for take_shares()
     auto load_trip = [&](int s0, bool defer_shares) __attribute__((always_inline)) {
 #pragma unroll
@@ -546,6 +555,7 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
                 const int c0 = (isk ? qd : 0) + h * hd + d;
                 buf[c0] = d0;
                 buf[c0 + half] = d1;
+                amax = fmaxf(amax, fmaxf(fabsf(d0), fabsf(d1)));
                 if (!isk) { a.dq_f[row * qd + h * hd + d] = d0; a.dq_f[row * qd + h * hd + d + half] = d1; }
             }
         }
@@ -555,13 +565,24 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
     if (first) load_trip(wave, true);
     if (a.dkp) {
         // dk and dv arrive as shares: their sums are formed by all threads while the loads of the first trip are on
-        // their way.  dk waits in its place in the row (the wave that owns a head reads it there before it writes the
-        // head's result), dv is final.
-        for (int c = threadIdx.x; c < 2 * kd; c += NT) {
-            const int isv = c >= kd, cc = isv ? c - kd : c;
-            const float v = kv_share_sum(a, isv ? a.dvp : a.dkp, row, pos, cc / hd, cc % hd);
-            buf[qd + c] = v;
-            if (isv) a.dv_f[row * kd + cc] = v;
+        // their way, SHU elements of a thread per round trip.  dk waits in its place in the row (the wave that owns a
+        // head reads it there before it writes the head's result), dv is final.
+        constexpr int SHU = NP == 1 ? 2 : 1;               // (wide heads: the first trip's values leave no registers for two)
+        for (int c0 = threadIdx.x; c0 < 2 * kd; c0 += SHU * NT) {
+            const float *sh[SHU]; int hk[SHU], dd[SHU], cc[SHU]; bool on[SHU], isv[SHU]; float v[SHU];
+#pragma unroll
+            for (int u = 0; u < SHU; u++) {
+                const int c = c0 + u * NT;
+                on[u] = c < 2 * kd; isv[u] = c >= kd; cc[u] = on[u] ? (isv[u] ? c - kd : c) : 0;
+                sh[u] = isv[u] ? a.dvp : a.dkp; hk[u] = cc[u] / hd; dd[u] = cc[u] % hd;
+            }
+            kv_share_sums<SHU>(a, sh, row, pos, hk, dd, on, v);
+#pragma unroll
+            for (int u = 0; u < SHU; u++) {
+                if (!on[u]) continue;
+                buf[qd + c0 + u * NT] = v[u];
+                if (isv[u]) { a.dv_f[row * kd + cc[u]] = v[u]; amax = fmaxf(amax, fabsf(v[u])); }
+            }
         }
         __syncthreads();
         if (first) take_shares(wave);
@@ -569,7 +590,7 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
     if (first) finish_trip(wave);
     for (int s0 = wave + TRIP; s0 < nslots; s0 += TRIP) { load_trip(s0, false); finish_trip(s0); }
     if (!a.dvp)
-        for (int c = threadIdx.x; c < kd; c += NT) buf[qd + kd + c] = a.dv[row * kd + c];
+        for (int c = threadIdx.x; c < kd; c += NT) { const float v = a.dv[row * kd + c]; buf[qd + kd + c] = v; amax = fmaxf(amax, fabsf(v)); }
     __syncthreads();
     // dh[r] = sc * sum_c d[c] * B[c][r].  Rank 16 (the common case): four threads share a row of B (16 floats, one
     // float4 each) and 256 such groups split the columns, so a thread keeps 4 + 4 sums and a wave reduces over its 16
@@ -640,12 +661,11 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
             s *= a.sc;
             buf[qd + 2 * kd + threadIdx.x] = s;
             a.dh[row * 2 * R + threadIdx.x] = s;
+            amax = fmaxf(amax, fabsf(s));
         }
         __syncthreads();
     }
-    float amax = 0.f;
-    for (int c = threadIdx.x; c < n; c += NT) amax = fmaxf(amax, fabsf(buf[c]));
-    amax = block_max(amax, sm);
+    amax = block_max(amax, sm);                           // (every entry of the row was written by a thread that also took it into its maximum)
     const float s = row_scale_for(amax);
     write_f16_tiled(buf, n, a.out16, row, s);
     if (threadIdx.x == 0) a.inv_scale[row] = 1.0f / s;

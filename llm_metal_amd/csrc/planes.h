@@ -49,8 +49,9 @@ __device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int co
 // Position t is read only when ok[t]; the sums are formed in plane order, exactly as planes_at4 forms them.
 // GROUPED: the planes carry a factor per group of planes (Planes::scale_groups != 0); all T positions must then lie in
 // row[0], and row[0] must be the same for the whole wave.
-// Planes of halves (Planes::half_unscale != 0) are read 8 bytes at a time and summed in fp32 the same way.
-template <int T, int NB, bool GROUPED = false>
+// Planes of halves (Planes::half_unscale != 0) are read 8 bytes at a time and summed in fp32 the same way, NBH planes per
+// round trip (twice NB holds the same number of registers).
+template <int T, int NB, bool GROUPED = false, int NBH = NB>
 __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (&row)[T], const int (&col)[T], const bool (&ok)[T], float4 (&s)[T])
 {
     if (P.half_unscale != 0.f) {                          // uniform
@@ -59,20 +60,20 @@ __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (
 #pragma unroll
         for (int t = 0; t < T; t++) { ph[t] = reinterpret_cast<const half_t *>(P.p) + row[t] * P.ld + col[t]; s[t] = make_float4(0.f, 0.f, 0.f, 0.f); }
         auto hbatch = [&](int i0) __attribute__((always_inline)) {
-            half4v v[T][NB];
+            half4v v[T][NBH];
 #pragma unroll
-            for (int i = 0; i < NB; i++)
+            for (int i = 0; i < NBH; i++)
 #pragma unroll
                 for (int t = 0; t < T; t++) {
                     v[t][i] = half4v{(_Float16)0, (_Float16)0, (_Float16)0, (_Float16)0};
                     if (ok[t] && i0 + i < P.S) v[t][i] = *reinterpret_cast<const half4v *>(ph[t] + (size_t)(i0 + i) * P.stride);
                 }
             if (GROUPED) {
-                static_assert(NB <= 64, "one lane per plane of a batch");
+                static_assert(NBH <= 64, "one lane per plane of a batch");
                 const int li = threadIdx.x & 63;
-                const float fl = (li < NB && i0 + li < P.S) ? P.row_scale[row[0] * P.scale_groups + ((i0 + li) >> P.group_shift)] : 0.f;
+                const float fl = (li < NBH && i0 + li < P.S) ? P.row_scale[row[0] * P.scale_groups + ((i0 + li) >> P.group_shift)] : 0.f;
 #pragma unroll
-                for (int i = 0; i < NB; i++) {
+                for (int i = 0; i < NBH; i++) {
                     const float f = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fl), i));
 #pragma unroll
                     for (int t = 0; t < T; t++) {
@@ -84,9 +85,9 @@ __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (
 #pragma unroll
             for (int t = 0; t < T; t++)
 #pragma unroll
-                for (int i = 0; i < NB; i++) { s[t].x += (float)v[t][i][0]; s[t].y += (float)v[t][i][1]; s[t].z += (float)v[t][i][2]; s[t].w += (float)v[t][i][3]; }
+                for (int i = 0; i < NBH; i++) { s[t].x += (float)v[t][i][0]; s[t].y += (float)v[t][i][1]; s[t].z += (float)v[t][i][2]; s[t].w += (float)v[t][i][3]; }
         };
-        for (int i0 = 0; i0 < P.S; i0 += NB) hbatch(i0);
+        for (int i0 = 0; i0 < P.S; i0 += NBH) hbatch(i0);
 #pragma unroll
         for (int t = 0; t < T; t++) {
             const float f = P.half_unscale * ((!GROUPED && P.row_scale && ok[t]) ? P.row_scale[row[t]] : 1.0f);
