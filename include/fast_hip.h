@@ -161,9 +161,10 @@ void hip_enqueue_q8_to_f16(MetalBuf *src, MetalBuf *dst, int rows, int cols);
  * F16 image made once per product); 2: always the large-M kernel with Q8_0 tiles kept quantised and unpacked into LDS
  * by the kernel itself; -1: never (always the weight-streaming kernel). */
 void hip_gemm_force_large_m(int policy);
-/* Products of up to 64 activation rows with F16 weights: 1 (default) = the kernel whose workgroups stream their operands
- * into an LDS ring (gemm_ring: one or two workgroups per CU, 4 to 6 K chunks), 0 = the kernel with one K step per wave in
- * registers (gemm_tiled: 13 to 19 K chunks), which every other product takes.  Same results up to the order of the sums. */
+/* Products of up to 64 activation rows: 1 (default) = the kernel whose workgroups stream their operands into an LDS ring
+ * (gemm_ring: one or two workgroups per CU, 4 to 6 K chunks; Q8_0 tiles travel quantised, 1.06 bytes per weight, and are
+ * unpacked to fp16 from LDS), 0 = the kernel with one K step per wave in registers (gemm_tiled: 13 to 19 K chunks, Q8_0
+ * unpacked in registers), which every product of more rows takes.  Same results up to the order of the sums. */
 void hip_gemm_ring(int on);
 /* 1 (default): a LoRA training state of at most 64 rows on F16 weights stores the K-split planes of five of its eight
  * products per layer (gate|up and down forward; down, gate|up and O backward) as halves: every chunk sum, formed in fp32,

@@ -48,13 +48,13 @@ struct ScaleGroups { int cols, groups, shift; };
 // request, while most CUs have nothing to do, the tiles that the product's workgroups ask for first (its workgroup g
 // starts with the K steps rot(g) .. rot(g) + 3 of its chunk).  Hardware counters show that the product fetches them
 // again from beyond L2 (no line survives a kernel boundary there), but it then finds them in the memory-side cache, and
-// its first K steps stop waiting for HBM.  Which XCD asks makes no difference.  F16 tiles only; base == null: nothing
-// to fetch.
+// its first K steps stop waiting for HBM.  Which XCD asks makes no difference.  F16 tiles, or the int8 tiles of a Q8_0
+// operand (their scales, 6 % of the bytes, are left to the product); base == null: nothing to fetch.
 struct WeightPrefetch {
-    const char *base;             // tiled F16 weight image
-    int Kb, Nb;                   // K steps and 32-row blocks of the image
+    const char *base;             // tiled F16 weight image, or the int8 tiles of a Q8_0 operand (rotate & 2)
+    int Kb, Nb;                   // K steps and 32-row blocks of the image (Q8_0: of its quantised part)
     int nb, steps, S, n_tiles;    // the product's plan: blocks per workgroup, K steps per chunk, chunks, row tiles
-    int rotate;
+    int rotate;                   // bit 0: the product rotates its K steps; bit 1: Q8_0 tiles of 2 KB, `depth` counts pairs of K steps
     int wgs;                      // prefetching workgroups
     int per_wg;                   // product workgroups each of them covers
     int depth;                    // K steps fetched per product workgroup (its waves' first steps)

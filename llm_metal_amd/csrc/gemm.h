@@ -73,14 +73,14 @@ struct GemmPlan {
     int steps;     // 64-wide K steps per chunk
     int n_tiles, m_tiles;
     int rotate;    // start each workgroup at a different K step of its chunk
-    int ring;      // gemm_ring (one 64-row tile of activations, F16 weights): kg K groups of four waves per workgroup
+    int ring;      // gemm_ring (one 64-row tile of activations; F16 or Q8_0 weights): kg K groups of four waves per workgroup
     int kg;
 };
 
 // nbq: Q8_0 row blocks of a fmt-1 operand (an odd count forces one row block per wave); fmt: WeightOp::fmt of the operand
 GemmPlan plan_gemm(int M, int N, int K, int nbq = 0, int fmt = 0);
 void set_gemm_ring(int on);
-int gemm_ring_enabled();            // 1 (default): products of up to 64 rows with F16 weights take gemm_ring; 0: gemm_tiled
+int gemm_ring_enabled();            // 1 (default): products of up to 64 rows take gemm_ring (Q8_0 tiles stay quantised up to LDS); 0: gemm_tiled
 
 // P[s][m][n] (s < plan.S, plane s at P + s*plane_stride, row stride ldp) =
 //   inv_scale[m] * sum_{k in chunk s} A[m][k] * W[n][k],  A and W in the tiled layout.

@@ -266,7 +266,7 @@ int g_prof_on = 0;
 std::vector<ProfRec> g_prof;
 int g_force_nb = 0, g_force_S = 0;
 int g_wide_wg = 1;                     // eight-wave workgroups where K would be cut into ten or more chunks
-int g_ring = 1;                        // gemm_ring for one-tile products with F16 weights
+int g_ring = 1;                        // gemm_ring for one-tile products (F16 or Q8_0 weights)
 
 }  // namespace
 
@@ -305,7 +305,7 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
     GemmPlan p{};
     p.nw = 4;
     p.m_tiles = m_tiles;
-    if (g_ring && fmt == 0 && m_tiles == 1 && !g_force_nb) {
+    if (g_ring && m_tiles == 1 && !g_force_nb) {            // any weight format: Q8_0 tiles travel through the ring quantised
         p.ring = 1; p.kg = 2; p.nw = 8; p.nb = 2;
         p.n_tiles = (Nb + 1) / 2;
         const int S = g_force_S ? std::min(g_force_S, Kb) : ring_chunks(p.n_tiles, Kb, K, cus);
@@ -353,7 +353,7 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
     bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2) && (p.nw == 4 || (p.nw == 8 && p.m_tiles == 1)) && W.fmt >= 0 && W.fmt <= 2;
     if (W.fmt == 0) ok = ok && W.w16;
-    if (W.fmt == 1) ok = ok && W.q && W.d && W.nbq >= 0 && W.nbq <= Nb && (W.nbq == Nb || (W.w16 && (W.nbq % p.nb) == 0));
+    if (W.fmt == 1) ok = ok && W.q && W.d && W.nbq >= 0 && W.nbq <= Nb && (W.nbq == Nb || (W.w16 && (p.ring || (W.nbq % p.nb) == 0)));
     if (W.fmt == 2) ok = ok && W.q && W.d && W.kbq >= 0 && W.kbq <= Kb && (W.kbq == Kb || W.w16);
     if (!ok) {
         fprintf(stderr, "[fast_hip] gemm: bad launch M=%d N=%d K=%d ldp=%d fmt=%d nbq=%d kbq=%d plan(nb=%d S=%d steps=%d)\n",
@@ -361,8 +361,8 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         abort();
     }
     if (p.ring) {
-        if (W.fmt != 0 || p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (Nb + 1) / 2 ||
-            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb) {
+        if (p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (Nb + 1) / 2 ||
+            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb || (W.fmt != 0 && (p.kg != 2 || half_scale != 0.f))) {
             fprintf(stderr, "[fast_hip] gemm_ring: bad launch M=%d N=%d K=%d fmt=%d plan(kg=%d S=%d steps=%d tiles=%d)\n", M, N, K, W.fmt, p.kg, p.S, p.steps, p.n_tiles);
             abort();
         }
@@ -381,7 +381,11 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(256 * p.kg);
 #define RING_LAUNCH(KGV, SC, HP) launch_kargs<24>(gemm_ring<KGV, SC, HP>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
 #define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1, 0); else if (half_scale != 0.f) RING_LAUNCH(KGV, 0, 1); else RING_LAUNCH(KGV, 0, 0); } while (0)
-        if (p.kg == 1) RING_PICK(1); else if (p.kg == 2) RING_PICK(2); else RING_PICK(4);
+#define RING_LAUNCH_Q8(SC, WFV) launch_kargs<24>(gemm_ring<2, SC, 0, WFV>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
+        if (W.fmt == 1) { if (a_inv_scale) RING_LAUNCH_Q8(1, 1); else RING_LAUNCH_Q8(0, 1); }
+        else if (W.fmt == 2) { if (a_inv_scale) RING_LAUNCH_Q8(1, 2); else RING_LAUNCH_Q8(0, 2); }
+        else if (p.kg == 1) RING_PICK(1); else if (p.kg == 2) RING_PICK(2); else RING_PICK(4);
+#undef RING_LAUNCH_Q8
 #undef RING_PICK
 #undef RING_LAUNCH
         HIP_CHECK(hipGetLastError());

@@ -257,7 +257,7 @@ __global__ __launch_bounds__(NW * 64, 2) void gemm_tiled(GemmKArgs g)
 #undef ACC_AT
 }
 
-// ---- the same product for one 64-row tile of activations and F16 weights: workgroups that own their loads --------------
+// ---- the same product for one 64-row tile of activations: workgroups that own their loads --------------
 // gemm_ring<KG, SCALE>: one workgroup of 4 KG waves per (64 weight rows, K chunk).  Where gemm_tiled puts twelve waves on a
 // CU, each with one K step in registers, and then adds the waves' accumulators through LDS (32 KB per workgroup, all
 // workgroups of a launch at the same moment), this kernel gives the CU one or two workgroups whose loads go straight
@@ -279,10 +279,20 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 // HALFP (with SCALE 0): the chunk's sums leave as halves, times g.half_scale -- a power of two that the caller derives from
 // the weight matrix so that no sum of 8192-bounded operand values can pass the fp16 maximum; plane_stride and ldp then
 // count halves.  Half the bytes to write here and for the consumer to read; 11 significant bits per chunk sum.
-template <int KG, int SCALE, int HALFP = 0>
+//
+// WF 1, 2: Q8_0 weights (WeightOp fmt 1 / 2) stay quantised on their way through the ring.  A weight tile's slot of a stage
+// then holds the tile's 2 KB of int8 as two 1 KB pieces, and behind them its 64 scales (128 bytes, fetched by eight lanes);
+// the waves that multiply the tile read their 32 bytes and their scale(s) from LDS and turn them into fp16 there, with
+// the arithmetic of load_w_q8_rows / load_w_q8_cols (the value an F16 image of the dequantised weight holds).  1.06 bytes
+// per weight from HBM instead of 2.  The F16 tiles that such an operand carries -- the adapter rows behind a fused Q | K | V
+// matrix (fmt 1: row blocks from nbq on), the K steps from kbq on of its transposed image (fmt 2) -- take the F16 way
+// through the same slot; which way is uniform per wave and stage.  Every wave issues four loads per round either way (a
+// quantised tile's fourth asks for its scales once more), so that one count serves the waits.
+template <int KG, int SCALE, int HALFP = 0, int WF = 0>
 __global__ __launch_bounds__(256 * KG) void gemm_ring(KARGS24)
 {
     static_assert(!(SCALE && HALFP), "final outputs stay fp32");
+    static_assert(WF >= 0 && WF <= 2, "weight format");
     const uint64_t kw[24] = {KLIST24};
     const GemmKArgs g = kargs_unpack<GemmKArgs>(kw);
     static_assert(KG == 1 || KG == 2 || KG == 4, "K groups per workgroup");
@@ -296,12 +306,44 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(KARGS24)
     const int nsteps = min(g.Kb, kb_beg + g.steps_per_chunk) - kb_beg;
     const int rounds = (nsteps + KG - 1) / KG;
     // q = 0, 1: weight row blocks 2 tile + q; q = 2, 3: activation row blocks q - 2 (clamped: rows beyond M or N are not stored)
-    const half8 *src = q < 2 ? reinterpret_cast<const half8 *>(g.w16_ring) + ((size_t)min(2 * tile + q, g.Nb - 1) * g.Kb + kb_beg) * 256 + lane
+    // the weight row block this wave requests (q < 2) and the one it multiplies (qn); fmt 1: from nbq on they are F16 tiles
+    const int wb_req = min(2 * tile + (q & 1), g.Nb - 1), wb_mul = min(2 * tile + qn, g.Nb - 1);
+    const bool req_q8_rows = WF == 1 && wb_req < g.W.nbq, mul_q8_rows = WF == 1 && wb_mul < g.W.nbq;
+    const half8 *src;
+    if (WF == 0) src = q < 2 ? reinterpret_cast<const half8 *>(g.w16_ring) + ((size_t)wb_req * g.Kb + kb_beg) * 256 + lane
                              : g.A + ((size_t)min(q - 2, g.Mb - 1) * g.Kb + kb_beg) * 256 + a_lane(lane);
+    else if (WF == 1) src = q < 2 ? reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)max(wb_req - g.W.nbq, 0) * g.Kb + kb_beg) * 256 + lane
+                                  : g.A + ((size_t)min(q - 2, g.Mb - 1) * g.Kb + kb_beg) * 256 + a_lane(lane);
+    else src = q < 2 ? reinterpret_cast<const half8 *>(g.W.w16) + (size_t)wb_req * (g.Kb - g.W.kbq) * 256 + lane     // (+ the F16 step's index)
+                     : g.A + ((size_t)min(q - 2, g.Mb - 1) * g.Kb + kb_beg) * 256 + a_lane(lane);
     const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)ring;
+    // a quantised tile: int8 at slot + 0 .. 2047, scales at + 2048 .. 2175 (and once more at + 2304)
+    auto request_q8 = [&](uint32_t sb, size_t tile_index) __attribute__((always_inline)) {
+        const uint8_t *qp = g.W.q + tile_index * 2048 + lane * 16;
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(qp), "s"(sb) : "m0", "memory");
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(qp + 1024), "s"(sb + 1024u) : "m0", "memory");
+        const half_t *dp = g.W.d + tile_index * 64 + (lane & 7) * 8;
+        if (lane < 8) {
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(dp), "s"(sb + 2048u) : "m0", "memory");
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(dp), "s"(sb + 2304u) : "m0", "memory");
+        }
+    };
     auto request = [&](int round) __attribute__((always_inline)) {
         const int step = min(round * KG + kg, nsteps - 1);    // a group without a step in the last round loads the last step again
         const uint32_t sb = base + (uint32_t)(((round & 1) * KG + kg) * 16384 + q * 4096);
+        if constexpr (WF == 1) {
+            if (q < 2 && req_q8_rows) { request_q8(sb, (size_t)wb_req * g.Kb + kb_beg + step); return; }
+        }
+        if constexpr (WF == 2) {
+            if (q < 2) {
+                const int kt = kb_beg + step;
+                if (kt < g.W.kbq) { request_q8(sb, (size_t)wb_req * g.W.kbq + kt); return; }
+#pragma unroll
+                for (int j = 0; j < LOADS_PER_ROUND; j++)
+                    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src + (size_t)(kt - g.W.kbq) * 256 + j * 64), "s"(sb + (uint32_t)(j * 1024)) : "m0", "memory");
+                return;
+            }
+        }
 #pragma unroll
         for (int j = 0; j < LOADS_PER_ROUND; j++) {
             if (q < 2) asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src + (size_t)step * 256 + j * 64), "s"(sb + (uint32_t)(j * 1024)) : "m0", "memory");
@@ -321,8 +363,24 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(KARGS24)
         __builtin_amdgcn_s_barrier();                     // ... and every other wave's as well
         const half8 *st = ring + ((rd & 1) * KG + kg) * 1024;
         half8 w[4], a[4];
+        const int kt_mul = kb_beg + min(rd * KG + kg, nsteps - 1);
+        if ((WF == 1 && mul_q8_rows) || (WF == 2 && kt_mul < g.W.kbq)) {
+            const uint8_t *sq = reinterpret_cast<const uint8_t *>(st) + qn * 4096;
+            const uint4v r0 = *reinterpret_cast<const uint4v *>(sq + lane * 16), r1 = *reinterpret_cast<const uint4v *>(sq + 1024 + lane * 16);
+            const half_t *sd = reinterpret_cast<const half_t *>(sq + 2048);
+            if (WF == 1) {
+                const half8 d = bcast8(sd[lane]);
+                w[0] = q8_unpack8(r0[0], r0[1]) * d; w[1] = q8_unpack8(r0[2], r0[3]) * d;
+                w[2] = q8_unpack8(r1[0], r1[1]) * d; w[3] = q8_unpack8(r1[2], r1[3]) * d;
+            } else {
+                const half8 *sc = reinterpret_cast<const half8 *>(sd + (lane >> 5) * 32);
+                w[0] = q8_unpack8(r0[0], r0[1]) * sc[0]; w[1] = q8_unpack8(r0[2], r0[3]) * sc[1];
+                w[2] = q8_unpack8(r1[0], r1[1]) * sc[2]; w[3] = q8_unpack8(r1[2], r1[3]) * sc[3];
+            }
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; j++) w[j] = st[(qn * 4 + j) * 64 + lane];
+            for (int j = 0; j < 4; j++) w[j] = st[(qn * 4 + j) * 64 + lane];
+        }
 #pragma unroll
         for (int j = 0; j < 4; j++) a[j] = st[((2 + qm) * 4 + j) * 64 + lane];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

@@ -184,12 +184,22 @@ __device__ __forceinline__ void prefetch_weight_tiles(const WeightPrefetch &pf, 
             if (j0 + u < pf.per_wg * per_g && g < total && w < pf.depth) {
                 const int x = g % pf.n_tiles, y = g / pf.n_tiles;
                 const int kb_beg = y * pf.steps, nsteps = min(pf.Kb, kb_beg + pf.steps) - kb_beg;
-                const int rot = pf.rotate ? (int)((x * 7u + y * 3u) % (unsigned)nsteps) : 0;
-                int kk = w + rot;
-                if (kk >= nsteps) kk -= nsteps;
-                if (w < nsteps) {
-                    const size_t tile = (size_t)min(x * pf.nb + b, pf.Nb - 1) * pf.Kb + kb_beg + kk;
-                    v[u] = *reinterpret_cast<const uint4 *>(pf.base + tile * 4096 + t16);
+                if (pf.rotate & 2) {
+                    // Q8_0 tiles (2 KB of int8 each, K steps of a row block side by side; Kb even): a 4 KB load takes the
+                    // pair of K steps that holds step kb_beg + 2 w
+                    const int kt = (kb_beg + 2 * w) & ~1;
+                    if (2 * w < nsteps && kt < pf.Kb) {
+                        const size_t tile = (size_t)min(x * pf.nb + b, pf.Nb - 1) * pf.Kb + kt;
+                        v[u] = *reinterpret_cast<const uint4 *>(pf.base + tile * 2048 + t16);
+                    }
+                } else {
+                    const int rot = pf.rotate ? (int)((x * 7u + y * 3u) % (unsigned)nsteps) : 0;
+                    int kk = w + rot;
+                    if (kk >= nsteps) kk -= nsteps;
+                    if (w < nsteps) {
+                        const size_t tile = (size_t)min(x * pf.nb + b, pf.Nb - 1) * pf.Kb + kb_beg + kk;
+                        v[u] = *reinterpret_cast<const uint4 *>(pf.base + tile * 4096 + t16);
+                    }
                 }
             }
         }

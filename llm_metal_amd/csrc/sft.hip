@@ -233,21 +233,29 @@ WeightPrefetch prefetch_for(SFTState *s, const WeightOp &W, int N, int K, int th
     // the row kernel by 1.5; less fetches too little, more (or fewer, longer-running workgroups) holds the row kernel up
     constexpr int mb = 16, depth = 4, wgs1024 = 160;
     WeightPrefetch pf{};
-    if (s->full_param || W.fmt != 0 || !W.w16 || use_big_gemm(s->BN, N, K, W.fmt)) return pf;
+    const bool q8 = W.fmt != 0;
+    if (s->full_param || (!q8 && !W.w16) || use_big_gemm(s->BN, N, K, W.fmt)) return pf;
     const GemmPlan p = plan_gemm(s->BN, N, K, 0, W.fmt);
     if (p.m_tiles != 1 || unit <= 0) return pf;
+    // Q8_0: the int8 tiles of the quantised part, two K steps per 4 KB load (an even number of K steps per row block)
+    const int kbq = !q8 ? tiled_kb(K) : W.fmt == 1 ? tiled_kb(K) : W.kbq;
+    const int nbq = W.fmt == 1 ? W.nbq : tiled_rb(N);
+    if (q8 && (!p.ring || !W.q || kbq <= 0 || (kbq & 1) || nbq <= 0)) return pf;
+    const long tile_bytes = q8 ? 2048 : 4096;
     int wgs = wgs1024 * (1024 / threads);
     wgs = (wgs + unit - 1) / unit * unit;
-    pf.base = reinterpret_cast<const char *>(W.w16);
-    pf.Kb = tiled_kb(K); pf.Nb = tiled_rb(N);
-    pf.nb = p.nb; pf.steps = p.steps; pf.S = p.S; pf.n_tiles = p.n_tiles; pf.rotate = p.rotate;
+    pf.base = q8 ? reinterpret_cast<const char *>(W.q) : reinterpret_cast<const char *>(W.w16);
+    pf.Kb = kbq; pf.Nb = nbq;
+    pf.nb = p.nb; pf.steps = p.steps; pf.S = p.S; pf.n_tiles = p.n_tiles; pf.rotate = (p.rotate ? 1 : 0) | (q8 ? 2 : 0);
     // few workgroups with long chunks (gemm_ring): the same bytes reach further into each chunk
     const long total = (long)p.n_tiles * p.S;
-    int d = depth;
-    if (total * p.nb * depth * 4096 < (long)mb * 1024 * 1024) d = (int)std::min<long>(p.steps, (long)mb * 1024 * 1024 / (total * p.nb * 4096));
-    if (d < depth) d = std::min(depth, p.steps);
-    pf.wgs = wgs; pf.depth = d;
-    const long covered = std::min<long>((long)mb * 1024 * 1024 / ((long)p.nb * d * 4096), total);
+    const int depth_q = q8 ? 2 * depth : depth;              // K steps: the same bytes
+    int d = depth_q;
+    if (total * p.nb * depth_q * tile_bytes < (long)mb * 1024 * 1024) d = (int)std::min<long>(p.steps, (long)mb * 1024 * 1024 / (total * p.nb * tile_bytes));
+    if (d < depth_q) d = std::min(depth_q, p.steps);
+    if (q8) d = (d + 1) & ~1;
+    pf.wgs = wgs; pf.depth = q8 ? d / 2 : d;                 // loads per row block of a product workgroup
+    const long covered = std::min<long>((long)mb * 1024 * 1024 / ((long)p.nb * d * tile_bytes), total);
     pf.per_wg = (int)((covered + wgs - 1) / wgs);
     return pf;
 }
