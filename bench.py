@@ -27,6 +27,7 @@ MFMA_PEAK_TFS = 2500.0          # dense fp16 MFMA
 
 
 TRAFFIC_SUMMARIES = {"c3_qwen3_4b_f16": ("c3_gemm_hbm_traffic_pmc.txt", "c3"),
+                     "c3_qwen3_4b_q8_seq64": ("c3_q8_step_trace_and_hbm_traffic.txt", "c3q"),
                      "c2_gemma3_1b": ("c2_gemm_hbm_traffic_pmc.txt", "c2"),
                      "c4_qwen3_4b_q8": ("c4_gemm_hbm_traffic_pmc.txt", "c4"),
                      "c5_gemma3_1b_grpo": ("c5_step_hbm_traffic_pmc.txt", "c5")}
@@ -202,7 +203,7 @@ def decode_bench(args, cfg, L):
                       "weights": "own row-major matrices" if sft is None else "the training state's tiles, read in place"},
            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                        "kernel": "k_matvec" if sft is None else ("gemm_ring" if f16 else "gemm_tiled"),
+                        "kernel": "k_matvec" if sft is None else "gemm_ring",
                         "launches_per_step": n // prof_steps, "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                         "weight_bytes_per_step": wb.value / prof_steps, "matvec_ms_per_step": round(tms.value / prof_steps, 3)},
            "setup_s": {"generate_weights": round(t_gen, 1), "upload_convert": round(t_init, 1)}}
@@ -394,7 +395,7 @@ def _main():
                            # full-parameter pass: the products, the weight gradients (F16 read-modify-write of the accumulators), the
                            # apply (W, G and the transposed image) and the operand transposes (time only) are timed together
                            "gemm_tiled, gemm_big_f16*, k_wgrad, k_apply_retile, k_transpose_scaled_jobs" if cfg.R == 0 else
-                           "gemm_ring" if cfg.BN <= 64 and cfg.weight_format == "f16" and args.gemm_ring else "gemm_tiled"),
+                           "gemm_ring" if cfg.BN <= 64 and args.gemm_ring else "gemm_tiled"),
                 "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),
                 "weight_bytes_per_step": wb.value / prof_steps, "flop_per_step": fl.value / prof_steps,
@@ -413,6 +414,7 @@ def _main():
            "dtype": ("q8_0 weights unpacked to f16 in LDS x f16 activations, f32 accumulate"
                      if cfg.weight_format != "f16" and cfg.BN >= 1024 and args.q8_large_m == "unpack-in-lds" else
                      "q8_0 weights as f16 images x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN >= 1024 else
+                     "q8_0 weights unpacked to f16 in LDS x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN <= 64 and args.gemm_ring else
                      "q8_0 weights unpacked to f16 in registers x f16 activations, f32 accumulate" if cfg.weight_format != "f16" else
                      "f16 weights x f16 activations, f32 accumulate (the K-chunk sums of five products per layer leave as f16)"
                      if cfg.R > 0 and cfg.BN <= 64 and args.half_planes and args.gemm_ring else
