@@ -305,24 +305,32 @@ __global__ __launch_bounds__(256) void k_apply_retile(half8 *__restrict__ W, hal
     W += blockIdx.z * st; WT += blockIdx.z * stT;
     if (G) G += blockIdx.z * st;
     const int KbW = tiled_kb(Ni), MbW = tiled_rb(Mo), KbT = tiled_kb(Mo), NbT = tiled_rb(Ni);
-    for (int q = tid; q < 512; q += 256) {
-        const int th = q >> 8, qq = q & 255, mbt = by * 2 + th;
-        const int j = qq >> 6, lp = qq & 63, ml = th * 32 + (lp & 31), n0 = (lp >> 5) * 32 + 8 * j;
-        half8 w = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (mbt < MbW) {
-            const size_t a = ((size_t)mbt * KbW + bx) * 256 + qq;
-            w = W[a];
-            if (G) {
-                const half8 g = G[a];
+    // both 32-row tiles of the block: their loads are issued together (one memory round trip for the thread's two pieces)
+    half8 w[2], g[2];
+    size_t at[2];
 #pragma unroll
-                for (int e = 0; e < 8; e++) w[e] = f2h(h2f(w[e]) - lr * h2f(g[e]));   // two roundings: contraction is off
-                W[a] = w;
-                const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-                G[a] = z;
-            }
+    for (int th = 0; th < 2; th++) {
+        const int mbt = by * 2 + th;
+        at[th] = ((size_t)min(mbt, MbW - 1) * KbW + bx) * 256 + tid;
+        w[th] = half8{0, 0, 0, 0, 0, 0, 0, 0}; g[th] = w[th];
+        if (mbt < MbW) {
+            w[th] = __builtin_nontemporal_load(&W[at[th]]);
+            if (G) g[th] = __builtin_nontemporal_load(&G[at[th]]);
+        }
+    }
+#pragma unroll
+    for (int th = 0; th < 2; th++) {
+        const int mbt = by * 2 + th;
+        const int j = tid >> 6, lp = tid & 63, ml = th * 32 + (lp & 31), n0 = (lp >> 5) * 32 + 8 * j;
+        if (mbt < MbW && G) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) w[th][e] = f2h(h2f(w[th][e]) - lr * h2f(g[th][e]));   // two roundings: contraction is off
+            __builtin_nontemporal_store(w[th], &W[at[th]]);
+            const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            __builtin_nontemporal_store(z, &G[at[th]]);
         }
 #pragma unroll
-        for (int e = 0; e < 8; e++) t[ml][n0 + e] = w[e];
+        for (int e = 0; e < 8; e++) t[ml][n0 + e] = w[th][e];
     }
     __syncthreads();
     for (int q = tid; q < 512; q += 256) {
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(256) void k_apply_retile(half8 *__restrict__ W, hal
         half8 o;
 #pragma unroll
         for (int e = 0; e < 8; e++) o[e] = t[m0 + e][nl];
-        WT[((size_t)nbt * KbT + by) * 256 + qq] = o;
+        __builtin_nontemporal_store(o, &WT[((size_t)nbt * KbT + by) * 256 + qq]);
     }
 }
 
