@@ -247,7 +247,7 @@ __global__ __launch_bounds__(256) void k_wgrad(WgradJobs js, int Kt, float lr)
                 for (int j4 = 0; j4 < 4; j4++) {
                     gp[mt][nh][j4] = reinterpret_cast<half4 *>(
                         target + ((((size_t)(mb0 + mt) * KbG + nk) * 4 + j4) * 64 + nh * 32 + l31) * 8 + 4 * h);
-                    g[mt][nh][j4] = *gp[mt][nh][j4];
+                    g[mt][nh][j4] = __builtin_nontemporal_load(gp[mt][nh][j4]);     // touched once per launch: past the caches, which hold the operands
                 }
         contract_tokens();
 #pragma unroll
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void k_wgrad(WgradJobs js, int Kt, float lr)
                         const float a = acc[mt][nh][4 * j4 + i] * sy[mt] * xs[i];
                         o[i] = SGD ? f2h(h2f(o[i]) - lr * a) : f2h(h2f(o[i]) + a);
                     }
-                    *gp[mt][nh][j4] = o;
+                    __builtin_nontemporal_store(o, gp[mt][nh][j4]);
                 }
         return;
     }
