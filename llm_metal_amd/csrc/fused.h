@@ -171,6 +171,9 @@ struct QkvBwdArgs {
     const float *q_pre, *k_pre, *g_q, *g_k; float eps;
     const float2 *rope;
     const float *Bq, *Bv; int R; float sc;
+    // optional fp16 copies of B_q and B_v (rank 16): every row's workgroup reads all of B for the projection dh, and that
+    // read is what a CU's path from L2 spends most of the kernel on; half the bytes.  null: the fp32 matrices are read
+    const half_t *Bq16, *Bv16;
     int Hq, Hkv, hd, seq;
     float *dq_f, *dv_f;           // pre-norm-domain dq [rows][Hq*hd], dv copy [rows][Hkv*hd] (for dB)
     float *dh;                    // [rows][2R] = sc * dq B_q | sc * dv B_v
@@ -239,6 +242,7 @@ struct AdamArgs {
     // transposed image wqkvT (kbT K blocks per row block)
     half_t *wqkv; size_t wqkv_layer_stride; half_t *wqkvT; size_t wqkvT_layer_stride;
     int a_row0, kbT;
+    half_t *p16;                  // optional: fp16 copy of the whole arena, same indexing (k_qkv_bwd_rows reads B_q, B_v there)
     int NL, D, qd, kd, R; size_t layer_size;
     float *grad_norm_out;         // [1]
 };
@@ -246,7 +250,8 @@ void launch_adamw(const AdamArgs &a);
 
 // fp16 shadow refresh only (after LoRA weights were written from outside)
 void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
-                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size, int a_row0, int kbT);
+                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size, int a_row0, int kbT,
+                        half_t *p16 = nullptr);
 
 void launch_fill_f32(float *p, float v, size_t n);
 

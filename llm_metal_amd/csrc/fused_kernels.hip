@@ -601,26 +601,82 @@ __global__ __launch_bounds__(NT) void k_qkv_bwd_rows(QkvBwdArgs a)
             float aq[4] = {0.f, 0.f, 0.f, 0.f}, av[4] = {0.f, 0.f, 0.f, 0.f};
             // two plain loops (q columns, then v columns), so that the loads of B of eight trips can be in flight at once:
             // every workgroup reads all of B, and what bounds it is how much of that one CU keeps in flight
+            if (a.Bq16 && NT == RB) {                      // (uniform; decided outside the loops so that each keeps its loads in flight)
+                // fp16 copies, a row per workgroup of 1024 threads: the fp32 loop's shape with 8-byte loads
+                typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 #pragma unroll 8
-            for (int c = threadIdx.x >> 2; c < qd; c += NT / 4) {
-                const float x = buf[c];
-                const float4 w = ld4(a.Bq + (size_t)c * 16 + 4 * sub);
-                aq[0] += x * w.x; aq[1] += x * w.y; aq[2] += x * w.z; aq[3] += x * w.w;
-            }
+                for (int c = threadIdx.x >> 2; c < qd; c += NT / 4) {
+                    const float x = buf[c];
+                    const half4v w = *reinterpret_cast<const half4v *>(a.Bq16 + (size_t)c * 16 + 4 * sub);
+                    aq[0] += x * (float)w[0]; aq[1] += x * (float)w[1]; aq[2] += x * (float)w[2]; aq[3] += x * (float)w[3];
+                }
 #pragma unroll 4
-            for (int c = threadIdx.x >> 2; c < kd; c += NT / 4) {
-                const float x = buf[qd + kd + c];
-                const float4 w = ld4(a.Bv + (size_t)c * 16 + 4 * sub);
-                av[0] += x * w.x; av[1] += x * w.y; av[2] += x * w.z; av[3] += x * w.w;
-            }
+                for (int c = threadIdx.x >> 2; c < kd; c += NT / 4) {
+                    const float x = buf[qd + kd + c];
+                    const half4v w = *reinterpret_cast<const half4v *>(a.Bv16 + (size_t)c * 16 + 4 * sub);
+                    av[0] += x * (float)w[0]; av[1] += x * (float)w[1]; av[2] += x * (float)w[2]; av[3] += x * (float)w[3];
+                }
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
+                for (int e = 0; e < 4; e++) {
 #pragma unroll
-                for (int o = 4; o < 64; o <<= 1) { aq[e] += __shfl_xor(aq[e], o, WAVE); av[e] += __shfl_xor(av[e], o, WAVE); }
-            }
-            if (lane < 4) {
+                    for (int o = 4; o < 64; o <<= 1) { aq[e] += __shfl_xor(aq[e], o, WAVE); av[e] += __shfl_xor(av[e], o, WAVE); }
+                }
+                if (lane < 4) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) { dhp[wave * 32 + 4 * lane + e] = aq[e]; dhp[wave * 32 + 16 + 4 * lane + e] = av[e]; }
+                    for (int e = 0; e < 4; e++) { dhp[wave * 32 + 4 * lane + e] = aq[e]; dhp[wave * 32 + 16 + 4 * lane + e] = av[e]; }
+                }
+            } else if (a.Bq16) {                           // 256 threads per row (many rows): the loads dominate, see below
+                // fp16 copies: two threads share a row of B (8 halves = 16 bytes each): half as many load instructions for
+                // half the bytes (a thread of a 256-thread workgroup walks 32 rows of B_q)
+                const int sub2 = threadIdx.x & 1;
+                float q8s[8], v8s[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) q8s[e] = v8s[e] = 0.f;
+#pragma unroll 8
+                for (int c = threadIdx.x >> 1; c < qd; c += NT / 2) {
+                    const float x = buf[c];
+                    const half8 w = *reinterpret_cast<const half8 *>(a.Bq16 + (size_t)c * 16 + 8 * sub2);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) q8s[e] += x * h2f(w[e]);
+                }
+#pragma unroll 2
+                for (int c = threadIdx.x >> 1; c < kd; c += NT / 2) {
+                    const float x = buf[qd + kd + c];
+                    const half8 w = *reinterpret_cast<const half8 *>(a.Bv16 + (size_t)c * 16 + 8 * sub2);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v8s[e] += x * h2f(w[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+#pragma unroll
+                    for (int o = 2; o < 64; o <<= 1) { q8s[e] += __shfl_xor(q8s[e], o, WAVE); v8s[e] += __shfl_xor(v8s[e], o, WAVE); }
+                }
+                if (lane < 2) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) { dhp[wave * 32 + 8 * lane + e] = q8s[e]; dhp[wave * 32 + 16 + 8 * lane + e] = v8s[e]; }
+                }
+            } else {
+#pragma unroll 8
+                for (int c = threadIdx.x >> 2; c < qd; c += NT / 4) {
+                    const float x = buf[c];
+                    const float4 w = ld4(a.Bq + (size_t)c * 16 + 4 * sub);
+                    aq[0] += x * w.x; aq[1] += x * w.y; aq[2] += x * w.z; aq[3] += x * w.w;
+                }
+#pragma unroll 4
+                for (int c = threadIdx.x >> 2; c < kd; c += NT / 4) {
+                    const float x = buf[qd + kd + c];
+                    const float4 w = ld4(a.Bv + (size_t)c * 16 + 4 * sub);
+                    av[0] += x * w.x; av[1] += x * w.y; av[2] += x * w.z; av[3] += x * w.w;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+#pragma unroll
+                    for (int o = 4; o < 64; o <<= 1) { aq[e] += __shfl_xor(aq[e], o, WAVE); av[e] += __shfl_xor(av[e], o, WAVE); }
+                }
+                if (lane < 4) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { dhp[wave * 32 + 4 * lane + e] = aq[e]; dhp[wave * 32 + 16 + 4 * lane + e] = av[e]; }
+                }
             }
         } else {
         float acc[32];
@@ -1288,6 +1344,7 @@ __global__ __launch_bounds__(1024) void k_grad_norm(const float *__restrict__ sl
 
 __device__ __forceinline__ void shadow_store(const AdamArgs &a, size_t idx, float pv)
 {
+    if (a.p16) a.p16[idx] = f2h(pv);
     const size_t L = idx / a.layer_size;
     size_t o = idx % a.layer_size;
     const size_t nA = (size_t)a.R * a.D, nBq = (size_t)a.qd * a.R;
@@ -1515,10 +1572,11 @@ void launch_adamw(const AdamArgs &a)
 }
 
 void launch_lora_shadow(const float *p, size_t n, half_t *wqkv, size_t wqkv_layer_stride, half_t *wqkvT,
-                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size, int a_row0, int kbT)
+                        size_t wqkvT_layer_stride, int D, int qd, int kd, int R, size_t layer_size, int a_row0, int kbT, half_t *p16)
 {
     if (!n) return;
     AdamArgs a{};
+    a.p16 = p16;
     a.p = const_cast<float *>(p); a.n = n; a.wqkv = wqkv; a.wqkv_layer_stride = wqkv_layer_stride;
     a.wqkvT = wqkvT; a.wqkvT_layer_stride = wqkvT_layer_stride;
     a.D = D; a.qd = qd; a.kd = kd; a.R = R; a.layer_size = layer_size; a.a_row0 = a_row0; a.kbT = kbT;

@@ -51,6 +51,7 @@ struct SFTState {
     // LoRA arena and optimiser state (fp32, device)
     size_t lsz, lora_n;
     MetalBuf *lora, *lora_grad, *adam_m, *adam_v, *sq_slots, *grad_norm;
+    MetalBuf *lora16;                    // fp16 copy of `lora`, refreshed wherever the adapters are written (B_q, B_v for the QKV backward rows)
     int slots_per_layer;
     std::vector<MetalBuf *> lora_views, grad_views;
 
@@ -583,6 +584,10 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         qb.Bq = at<float>(s->lora, L * s->lsz + (size_t)R * D);
         qb.Bv = at<float>(s->lora, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
         qb.R = R; qb.sc = s->lora_scaling;
+        if (R == 16) {
+            qb.Bq16 = at<half_t>(s->lora16, L * s->lsz + (size_t)R * D);
+            qb.Bv16 = at<half_t>(s->lora16, L * s->lsz + (size_t)2 * R * D + (size_t)qd * R);
+        }
         qb.Hq = s->Hq; qb.Hkv = s->Hkv; qb.hd = s->hd; qb.seq = s->N;
         qb.dq_f = at<float>(s->dq_f, keepL * BN * qd); qb.dv_f = nullptr; qb.dh = at<float>(s->dh, keepL * BN * (R ? 2 * R : 1));
         if (kv_shares) { qb.dkp = ab.dkp; qb.dvp = ab.dvp; qb.rows_total = BN; qb.dv_f = ab.dv; }
@@ -666,6 +671,7 @@ void enqueue_update(SFTState *s)
     a.a_row0 = s->q8_native ? 0 : s->qd + 2 * s->kd;
     a.kbT = s->q8_native ? tiled_kb(2 * s->R) : tiled_kb(s->nq_ext);
     a.grad_norm_out = at<float>(s->grad_norm);
+    a.p16 = at<half_t>(s->lora16);
     launch_adamw(a);
 }
 
@@ -674,7 +680,8 @@ void refresh_shadow(SFTState *s)
     if (!s->R) return;
     launch_lora_shadow(at<float>(s->lora), s->lora_n, at<half_t>(s->wqkv), s->st_qkv,
                        at<half_t>(s->wqkvT), s->st_qkvT, s->D, s->qd, s->kd, s->R, s->lsz,
-                       s->q8_native ? 0 : s->qd + 2 * s->kd, s->q8_native ? tiled_kb(2 * s->R) : tiled_kb(s->nq_ext));
+                       s->q8_native ? 0 : s->qd + 2 * s->kd, s->q8_native ? tiled_kb(2 * s->R) : tiled_kb(s->nq_ext),
+                       at<half_t>(s->lora16));
 }
 
 MetalBuf *host_buf(size_t bytes, void **cpu)
@@ -833,6 +840,7 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     s->lora_n = s->lsz * NL;
     s->slots_per_layer = R ? lora_grad_blocks(D, qd, kd, R) : 1;
     s->lora = fbuf(s->lora_n ? s->lora_n : 1); s->lora_grad = fbuf(s->lora_n ? s->lora_n : 1);
+    s->lora16 = hbuf(s->lora_n ? s->lora_n : 1);
     s->adam_m = fbuf(s->lora_n ? s->lora_n : 1); s->adam_v = fbuf(s->lora_n ? s->lora_n : 1);
     s->sq_slots = fbuf((size_t)s->slots_per_layer * NL); s->grad_norm = fbuf(4);
     HIP_CHECK(hipMemsetAsync(dptr(s->lora_grad), 0, s->lora_grad->size, stream()));
@@ -961,7 +969,7 @@ void sft_state_free(SFTState *s)
     MetalBuf *all[] = {s->wqkv, s->wqkvT, s->wo, s->woT, s->wgu, s->wguT, s->wd, s->wdT, s->wlm, s->wlmT, s->zqkv.q, s->zqkv.d, s->zqkv.qT, s->zqkv.dT, s->zo.q, s->zo.d, s->zo.qT, s->zo.dT,
                        s->zgu.q, s->zgu.d, s->zgu.qT, s->zgu.dT, s->zd.q, s->zd.d, s->zd.qT, s->zd.dT, s->zlm.q, s->zlm.d, s->zlm.qT, s->zlm.dT,
                        s->rope_tabs, s->g_in, s->g_post_attn, s->g_pre_ff, s->g_post_ff, s->g_q, s->g_k, s->g_final, s->emb,
-                       s->lora, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
+                       s->lora, s->lora16, s->lora_grad, s->adam_m, s->adam_v, s->sq_slots, s->grad_norm,
                        s->tokens, s->targets, s->losses, s->hyper, s->x_in_host,
                        s->xs, s->ln1_16, s->ln1_inv, s->q_pre, s->k_pre, s->q_fin, s->k_fin, s->v_sav, s->probs,
                        s->gu_sav, s->tq, s->tv, s->kT, s->vT, s->o_raw, s->ff_raw, s->a16, s->a16_inv, s->group_inv, s->ones, s->planes,
