@@ -91,10 +91,14 @@ CASES = [
     C1.with_(name="seq1100", NL=1, D=128, Hq=2, Hkv=1, hd=64, IS=256, V=512, seq=1100),             # by the rule: beyond 1024 keys
     # 512 rows and more: the row kernels run with 256 threads per row (norm-then-add ordering and GeGLU included)
     TINY_GEMMA3.with_(name="gemma_many_rows", NL=2, batch=4, seq=128),
-    # products of up to 64 rows on F16 weights take gemm_ring by default; the register-staged streaming kernel that they
-    # took before (and that Q8_0 weights and several row tiles still take) on the same shapes
+    # products of up to 64 rows take gemm_ring by default (Q8_0 tiles quantised up to LDS: the q8 cases above); the
+    # register-staged streaming kernel that they took before (and that several row tiles still take) on the same shapes,
+    # with F16 weights and with Q8_0 weights unpacked in registers (an odd number of Q8_0 row blocks among them)
     C1.with_(name="c1_tiled"),
     TINY_GEMMA3.with_(name="gemma_tiled"),
+    C1.with_(name="c1_q8_tiled", weight_format="q8_0"),
+    C1.with_(name="q8_odd_blocks_tiled", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format="q8_0"),
+    TINY_GEMMA3.with_(name="gemma_q8_tiled", weight_format="q8_0"),
     C1.with_(name="wide_ffn_groups_tiled", NL=1, IS=4224, V=1024, seq=64),
     C1.with_(name="ragged_seq40_tiled", NL=2, batch=2, seq=40, R=4, alpha=8.0),
     # up to 64 positions the attention backward is one launch by default (dQ with the shares of dK / dV per query block and
