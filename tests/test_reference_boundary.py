@@ -121,7 +121,8 @@ def reference_sources(dirs):
 @pytest.mark.skipif(not os.path.exists(LIB), reason="libllm_metal_hip.so is not built")
 def test_the_reference_tree_links_against_the_library(tmp_path):
     """./llm of the reference with fast_sft.c, fast_inference.c, fast_metal.m and metal_backend.m taken out and the
-    library plus the compat units put in: the link line of INTEGRATION.md.  No undefined symbol, and the binary starts."""
+    library plus the compat units put in: the link line a maintainer of the reference would use.  No undefined symbol, and
+    the binary starts."""
     exe = tmp_path / "llm_hip"
     r = subprocess.run([CLANG, "-std=c17", "-D_GNU_SOURCE", "-O1", "-w", "-DFAST_METAL_H",
                         "-include", os.path.join(COMPAT, "fast_inference_compat.h"), "-I", INC, "-I", os.path.join(REF, "src", "nn"),
