@@ -414,6 +414,8 @@ def _main():
            "dtype": ("q8_0 weights unpacked to f16 in LDS x f16 activations, f32 accumulate"
                      if cfg.weight_format != "f16" and cfg.BN >= 1024 and args.q8_large_m == "unpack-in-lds" else
                      "q8_0 weights as f16 images x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN >= 1024 else
+                     "q8_0 weights unpacked to f16 in LDS x f16 activations, f32 accumulate (the K-chunk sums of five products per layer leave as f16)"
+                     if cfg.weight_format != "f16" and cfg.BN <= 64 and args.gemm_ring and args.half_planes and cfg.R > 0 else
                      "q8_0 weights unpacked to f16 in LDS x f16 activations, f32 accumulate" if cfg.weight_format != "f16" and cfg.BN <= 64 and args.gemm_ring else
                      "q8_0 weights unpacked to f16 in registers x f16 activations, f32 accumulate" if cfg.weight_format != "f16" else
                      "f16 weights x f16 activations, f32 accumulate (the K-chunk sums of five products per layer leave as f16)"

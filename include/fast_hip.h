@@ -166,7 +166,7 @@ void hip_gemm_force_large_m(int policy);
  * unpacked to fp16 from LDS), 0 = the kernel with one K step per wave in registers (gemm_tiled: 13 to 19 K chunks, Q8_0
  * unpacked in registers), which every product of more rows takes.  Same results up to the order of the sums. */
 void hip_gemm_ring(int on);
-/* 1 (default): a LoRA training state of at most 64 rows on F16 weights stores the K-split planes of five of its eight
+/* 1 (default): a LoRA training state of at most 64 rows (frozen F16 or Q8_0 weights) stores the K-split planes of five of its eight
  * products per layer (gate|up and down forward; down, gate|up and O backward) as halves: every chunk sum, formed in fp32,
  * leaves times a power of two derived from the weight matrix (8192 times its largest row sum of |w| stays below the fp16
  * maximum) and is summed in fp32 again by the kernel that consumes the planes.  Half the plane bytes, 11 significant

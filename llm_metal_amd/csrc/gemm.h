@@ -91,6 +91,8 @@ void launch_gemm(const half_t *A_tiled, const float *a_inv_scale, const WeightOp
                  float *P, int ldp, size_t plane_stride, int M, int N, int K, const GemmPlan &p, float half_scale = 0.f);
 // Largest sum of |w| over a row of a tiled F16 matrix [N, K]: with operand rows scaled below 8192 (row_scale_for), no
 // chunk sum of a product with this matrix exceeds 8192 times it.  Synchronises the stream.
+// the same over the values a weight operand of any format multiplies with (0 when the operand mixes Q8_0 and F16 tiles)
+float weight_max_row_l1(const WeightOp &W, int N, int K);
 float tiled_max_row_l1(const half_t *W_tiled, int N, int K);
 // the power of two by which chunk sums of products with a matrix of that row bound are multiplied to leave as halves
 float half_plane_scale(float max_row_l1);

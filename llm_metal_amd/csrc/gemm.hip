@@ -362,7 +362,7 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
     }
     if (p.ring) {
         if (p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (Nb + 1) / 2 ||
-            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb || (W.fmt != 0 && (p.kg != 2 || half_scale != 0.f))) {
+            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb || (W.fmt != 0 && (p.kg != 2 || (half_scale != 0.f && a_inv_scale)))) {
             fprintf(stderr, "[fast_hip] gemm_ring: bad launch M=%d N=%d K=%d fmt=%d plan(kg=%d S=%d steps=%d tiles=%d)\n", M, N, K, W.fmt, p.kg, p.S, p.steps, p.n_tiles);
             abort();
         }
@@ -381,9 +381,9 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(256 * p.kg);
 #define RING_LAUNCH(KGV, SC, HP) launch_kargs<24>(gemm_ring<KGV, SC, HP>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
 #define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1, 0); else if (half_scale != 0.f) RING_LAUNCH(KGV, 0, 1); else RING_LAUNCH(KGV, 0, 0); } while (0)
-#define RING_LAUNCH_Q8(SC, WFV) launch_kargs<24>(gemm_ring<2, SC, 0, WFV>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
-        if (W.fmt == 1) { if (a_inv_scale) RING_LAUNCH_Q8(1, 1); else RING_LAUNCH_Q8(0, 1); }
-        else if (W.fmt == 2) { if (a_inv_scale) RING_LAUNCH_Q8(1, 2); else RING_LAUNCH_Q8(0, 2); }
+#define RING_LAUNCH_Q8(SC, HP, WFV) launch_kargs<24>(gemm_ring<2, SC, HP, WFV>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
+        if (W.fmt == 1) { if (a_inv_scale) RING_LAUNCH_Q8(1, 0, 1); else if (half_scale != 0.f) RING_LAUNCH_Q8(0, 1, 1); else RING_LAUNCH_Q8(0, 0, 1); }
+        else if (W.fmt == 2) { if (a_inv_scale) RING_LAUNCH_Q8(1, 0, 2); else if (half_scale != 0.f) RING_LAUNCH_Q8(0, 1, 2); else RING_LAUNCH_Q8(0, 0, 2); }
         else if (p.kg == 1) RING_PICK(1); else if (p.kg == 2) RING_PICK(2); else RING_PICK(4);
 #undef RING_LAUNCH_Q8
 #undef RING_PICK
@@ -513,7 +513,50 @@ __global__ __launch_bounds__(64) void k_tiled_row_l1(const half8 *__restrict__ W
     for (int o = 1; o < 32; o <<= 1) s = fmaxf(s, __shfl_xor(s, o, 64));
     if (lane == 0) atomicMax(reinterpret_cast<int *>(out), __float_as_int(s));   // sums are >= 0: integer order is float order
 }
+// the same for a Q8_0 operand (FMT 1: one scale per lane and tile; 2: one per column of the tile), of the values d * q
+template <int FMT>
+__global__ __launch_bounds__(64) void k_q8_row_l1(const uint8_t *__restrict__ q, const half_t *__restrict__ d, int N, int Kb, float *__restrict__ out)
+{
+    const int lane = threadIdx.x;
+    float s = 0.f;
+    for (int kt = 0; kt < Kb; kt++) {
+        const size_t tile = (size_t)blockIdx.x * Kb + kt;
+        const uint4v *qp = reinterpret_cast<const uint4v *>(q) + tile * 128 + lane;
+        const uint4v r[2] = {qp[0], qp[64]};
+        const half_t *sc = d + tile * 64 + (FMT == 1 ? lane : (lane >> 5) * 32);
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const int v = (int)(int8_t)((r[h][w] >> (8 * b)) & 0xffu);
+                    const int je = (2 * h + (w >> 1)) * 8 + (w & 1) * 4 + b;      // (j, e) of the byte, as load_w_q8_cols numbers them
+                    s += fabsf((float)v) * (float)(FMT == 1 ? sc[0] : sc[je]);
+                }
+    }
+    if ((int)blockIdx.x * 32 + (lane & 31) >= N) s = 0.f;
+    s += __shfl_xor(s, 32, 64);
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) s = fmaxf(s, __shfl_xor(s, o, 64));
+    if (lane == 0) atomicMax(reinterpret_cast<int *>(out), __float_as_int(s));
+}
 }  // namespace
+
+float weight_max_row_l1(const WeightOp &W, int N, int K)
+{
+    if (W.fmt == 0) return tiled_max_row_l1(W.w16, N, K);
+    // operands that are Q8_0 throughout (no F16 row blocks or K steps behind them)
+    if ((W.fmt == 1 && W.nbq != tiled_rb(N)) || (W.fmt == 2 && W.kbq != tiled_kb(K))) return 0.f;
+    float *slot = (float *)scratch(SCR_MISC, sizeof(float));
+    HIP_CHECK(hipMemsetAsync(slot, 0, sizeof(float), stream()));
+    if (W.fmt == 1) hipLaunchKernelGGL(k_q8_row_l1<1>, dim3(tiled_rb(N)), dim3(64), 0, stream(), W.q, W.d, N, tiled_kb(K), slot);
+    else hipLaunchKernelGGL(k_q8_row_l1<2>, dim3(tiled_rb(N)), dim3(64), 0, stream(), W.q, W.d, N, tiled_kb(K), slot);
+    float v = 0.f;
+    HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream()));
+    HIP_CHECK(hipStreamSynchronize(stream()));
+    return v;
+}
 
 float tiled_max_row_l1(const half_t *W_tiled, int N, int K)
 {

@@ -945,16 +945,17 @@ SFTState *sft_state_create_from_ref(const SFTModelRef *m, int batch, int seq_len
     // the fused QKV weight and its transpose carry fp16 images of A_q, A_v
     refresh_shadow(s);
     metal_flush();
-    // products of at most 64 rows on frozen F16 weights leave their K-split planes as halves: one factor per matrix
-    if (s->R > 0 && !s->q8_native && BN <= 64) {
-        struct Img { int kind; bool T; MetalBuf *arena; size_t st; int N, K; };
-        const Img imgs[] = {{W_GU, false, s->wgu, s->st_gu, 2 * IS, D}, {W_D, false, s->wd, s->st_d, D, IS},
-                            {W_D, true, s->wdT, s->st_dT, IS, D}, {W_GU, true, s->wguT, s->st_guT, D, 2 * IS},
-                            {W_O, true, s->woT, s->st_oT, qd, D}};
+    // products of at most 64 rows on frozen weights (F16 or Q8_0) leave their K-split planes as halves: one factor per matrix
+    if (s->R > 0 && BN <= 64) {
+        struct Img { int kind; bool T; int N, K; };
+        const Img imgs[] = {{W_GU, false, 2 * IS, D}, {W_D, false, D, IS}, {W_D, true, IS, D}, {W_GU, true, D, 2 * IS}, {W_O, true, qd, D}};
         for (const Img &im : imgs) {
             std::vector<float> &v = s->half_scale[im.kind][im.T ? 1 : 0];
             v.resize(s->NL);
-            for (int L = 0; L < s->NL; L++) v[L] = half_plane_scale(tiled_max_row_l1(at<half_t>(im.arena, (size_t)L * im.st), im.N, im.K));
+            for (int L = 0; L < s->NL; L++) {
+                const float l1 = weight_max_row_l1(wop(s, im.kind, L, im.T), im.N, im.K);
+                v[L] = l1 > 0.f ? half_plane_scale(l1) : 0.f;          // 0: that product keeps fp32 planes
+            }
         }
     }
     return s;

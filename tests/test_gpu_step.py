@@ -111,12 +111,13 @@ CASES = [
     C1.with_(name="ragged_seq40_two_launch", NL=2, batch=2, seq=40, R=4, alpha=8.0),
     C1.with_(name="hd256_mqa_seq50_two_launch", NL=2, D=128, Hq=4, Hkv=1, hd=256, IS=256, V=1024, batch=2, seq=50),
     C1.with_(name="window24_two_launch", window=24),
-    # LoRA states of up to 64 rows on F16 weights keep the K-split planes of five products per layer as halves by default;
+    # LoRA states of up to 64 rows (F16 or Q8_0 weights) keep the K-split planes of five products per layer as halves by default;
     # the same shapes with fp32 planes everywhere
     C1.with_(name="c1_f32_planes"),
     TINY_GEMMA3.with_(name="gemma_f32_planes"),
     C1.with_(name="wide_ffn_groups_f32_planes", NL=1, IS=4224, V=1024, seq=64),
     C1.with_(name="hd128_f32_planes", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
+    C1.with_(name="c1_q8_f32_planes", weight_format="q8_0"),
 ]
 
 
