@@ -14,6 +14,8 @@ V_CUT = 8192
 
 # Qwen3-4B widths, one layer, 64 rows, F16 (config 3)
 C3_WIDTHS = C3.with_(name="c3_widths", NL=1, V=V_CUT)
+# the same with Q8_0 weights (config 3's Q8_0 variant): the tiles stay quantised up to LDS in every product
+C3Q_WIDTHS = C3.with_(name="c3q_widths", NL=1, V=V_CUT, weight_format="q8_0")
 # Gemma3-1B widths, two layers (layer 0 global theta, layer 1 local), 64 rows, tied head (config 2)
 C2_WIDTHS = C2.with_(name="c2_widths", NL=2, V=V_CUT)
 # Qwen3-4B widths, Q8_0 weights, 4 x 512 rows (config 4): every product takes the large-M path

@@ -38,10 +38,10 @@ def f16(bits):
 
 # ---------------------------------------------------------------- real widths, few layers, against the oracle
 
-@pytest.mark.parametrize("cfg", [rw.C3_WIDTHS, rw.C2_WIDTHS], ids=lambda c: c.name)
+@pytest.mark.parametrize("cfg", [rw.C3_WIDTHS, rw.C2_WIDTHS, rw.C3Q_WIDTHS], ids=lambda c: c.name)
 def test_step_at_real_widths_matches_oracle(cfg):
     model = make_model(cfg, seed=rw.MODEL_SEED, gamma_jitter=rw.GAMMA_JITTER)
-    used = oracle.weights_as_used(model)
+    used = oracle.weights_as_used(model, "f16" if cfg.weight_format == "f16" else "q8")
     lora = model["lora"].copy()
     m, v, step = np.zeros_like(lora), np.zeros_like(lora), 0
     lr = 1e-4
