@@ -212,6 +212,24 @@ def test_config3_as_benchmarked(qwen3_4b_model):
         _zero_b_properties(C3, st, qwen3_4b_model)
 
 
+def test_config3_with_q8_weights_as_benchmarked_and_the_two_streaming_kernels_agree(qwen3_4b_model):
+    """1 x 64 rows on Q8_0 weights, all layers: the products take gemm_ring with the tiles quantised up to LDS (and planes
+    of halves); on the register-staged kernel with fp32 planes the step must give the same loss and gradient norm."""
+    from llm_metal_amd.configs import C3Q
+    L = lib.load()
+    with SFTState(C3Q, qwen3_4b_model) as st:
+        tok, tgt = make_batch(C3Q, seed=100)
+        out = {}
+        for ring in (1, 0):
+            L.hip_gemm_ring(ring)
+            st.set_lora(qwen3_4b_model["lora"])
+            out[ring] = (st.train_step(tok, tgt, 0.0), st.grad_norm())         # lr 0: the adapters stay put
+        L.hip_gemm_ring(1)
+        assert abs(out[0][0] - out[1][0]) <= 1e-3 * out[1][0], out
+        assert abs(out[0][1] - out[1][1]) <= 1e-2 * out[1][1], out
+        _zero_b_properties(C3Q, st, qwen3_4b_model)
+
+
 def test_config4_as_benchmarked_and_gemm_families_agree(qwen3_4b_model):
     """4 x 512 rows on Q8_0 weights: the measured rule sends every product to the large-M kernel; forced onto the
     weight-streaming kernel (policy -1) the step must give the same loss and gradient norm."""
