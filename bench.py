@@ -57,7 +57,8 @@ def measured_traffic(cfg_name, kernels):
 def gemm_shapes(cfg, L):
     """One line per product shape of a LoRA step at cfg.BN rows (F16 weights): microseconds per launch, launched back to
     back on the library's stream with the weights rotated through more than 1 GB (nothing is found in a cache), for
-    (a) the weight loads of gemm_ring alone on its grid, (b) gemm_ring, (c) gemm_tiled; and a fit  t = t0 + bytes / rate
+    (a) the weight loads of gemm_ring alone on its grid, (b) gemm_ring or, where the planner takes it, gemm_ring_wide (named in
+    `ring_kernel`), (c) gemm_tiled; and a fit  t = t0 + bytes / rate
     over the layer shapes.  An empty kernel launched the same way takes about 3 us, which every figure includes."""
     import ctypes as C
     D, qd, kd, IS, V, R = cfg.D, cfg.Hq * cfg.hd, cfg.Hkv * cfg.hd, cfg.IS, cfg.V, cfg.R
@@ -72,14 +73,14 @@ def gemm_shapes(cfg, L):
         L.hip_gemm_ring(1)
         t_read = L.hip_gemm_time_shape(cfg.BN, N, K, -1, 0, 0, it, C.byref(nb), C.byref(S)) * 1e3
         t_ring = L.hip_gemm_time_shape(cfg.BN, N, K, 0, 0, 0, it, C.byref(nb), C.byref(S)) * 1e3
-        s_ring = S.value
+        s_ring, wide = S.value, nb.value == 4
         L.hip_gemm_ring(0)
         t_tiled = L.hip_gemm_time_shape(cfg.BN, N, K, 0, 0, 0, it, C.byref(nb), C.byref(S)) * 1e3
         s_tiled = S.value
         L.hip_gemm_ring(1)
         mb = 2.0 * N * K / 1e6
         rows.append({"product": name, "N": N, "K": K, "MB": round(mb, 1), "weights_only_us": round(t_read, 2), "gemm_ring_us": round(t_ring, 2),
-                     "ring_chunks": s_ring, "gemm_tiled_us": round(t_tiled, 2), "tiled_chunks": s_tiled,
+                     "ring_chunks": s_ring, "ring_kernel": "gemm_ring_wide" if wide else "gemm_ring", "gemm_tiled_us": round(t_tiled, 2), "tiled_chunks": s_tiled,
                      "weights_only_GBs": round(mb / t_read * 1e3), "gemm_ring_GBs": round(mb / t_ring * 1e3), "gemm_tiled_GBs": round(mb / t_tiled * 1e3)})
     layer = rows[:8]
     x = np.array([r["MB"] for r in layer]); fits = {}
@@ -271,6 +272,8 @@ def _main():
                     help="0: up to 64 positions too, the attention backward is two launches (dQ, then dK / dV) (comparisons only)")
     ap.add_argument("--half-planes", type=int, choices=(0, 1), default=1,
                     help="0: fp32 K-split planes for every product (comparisons only)")
+    ap.add_argument("--gemm-ring-wide", type=int, choices=(0, 1), default=1,
+                    help="1: gemm_ring_wide (four weight row blocks per workgroup) where the product has the row tiles for it")
     ap.add_argument("--gemm-ring", type=int, choices=(0, 1), default=1,
                     help="0: the products of up to 64 rows take the register-staged streaming kernel (gemm_tiled) instead of gemm_ring (comparisons only)")
     ap.add_argument("--attention", choices=("auto", "flash", "saved-probs"), default="auto",
@@ -326,6 +329,7 @@ def _main():
     t_gen = time.perf_counter() - t0
     L.hip_attention_flash({"auto": -1, "flash": 1, "saved-probs": 0}[args.attention])
     L.hip_gemm_ring(args.gemm_ring)
+    L.hip_gemm_ring_wide(args.gemm_ring_wide)
     L.hip_gemm_half_planes(args.half_planes)
     L.hip_attention_backward_one_launch(args.attn_bwd_one_launch)
     if args.q8_large_m == "image-per-product":
@@ -395,6 +399,7 @@ def _main():
                            # full-parameter pass: the products, the weight gradients (F16 read-modify-write of the accumulators), the
                            # apply (W, G and the transposed image) and the operand transposes (time only) are timed together
                            "gemm_tiled, gemm_big_f16*, k_wgrad, k_apply_retile, k_transpose_scaled_jobs" if cfg.R == 0 else
+                           "gemm_ring, gemm_ring_wide" if 32 < cfg.BN <= 64 and args.gemm_ring and args.gemm_ring_wide and cfg.weight_format == "f16" else
                            "gemm_ring" if cfg.BN <= 64 and args.gemm_ring else "gemm_tiled"),
                 "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),

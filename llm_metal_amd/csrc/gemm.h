@@ -75,11 +75,13 @@ struct GemmPlan {
     int rotate;    // start each workgroup at a different K step of its chunk
     int ring;      // gemm_ring (one 64-row tile of activations; F16 or Q8_0 weights): kg K groups of four waves per workgroup
     int kg;
+    int wide;      // ring plans: gemm_ring_wide, four weight row blocks per workgroup (nb = 4), one K group
 };
 
 // nbq: Q8_0 row blocks of a fmt-1 operand (an odd count forces one row block per wave); fmt: WeightOp::fmt of the operand
 GemmPlan plan_gemm(int M, int N, int K, int nbq = 0, int fmt = 0);
 void set_gemm_ring(int on);
+void set_gemm_ring_wide(int on);     // 1: products with enough row tiles take gemm_ring_wide; 2: every F16 product of 33 to 64 rows (tests)
 int gemm_ring_enabled();            // 1 (default): products of up to 64 rows take gemm_ring (Q8_0 tiles stay quantised up to LDS); 0: gemm_tiled
 
 // P[s][m][n] (s < plan.S, plane s at P + s*plane_stride, row stride ldp) =

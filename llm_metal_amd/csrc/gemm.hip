@@ -267,6 +267,7 @@ std::vector<ProfRec> g_prof;
 int g_force_nb = 0, g_force_S = 0;
 int g_wide_wg = 1;                     // eight-wave workgroups where K would be cut into ten or more chunks
 int g_ring = 1;                        // gemm_ring for one-tile products (F16 or Q8_0 weights)
+int g_ring_wide = 1;                   // gemm_ring_wide where the product has enough row tiles for it
 
 }  // namespace
 
@@ -312,6 +313,19 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
         p.steps = (Kb + S - 1) / S;
         p.S = (Kb + p.steps - 1) / p.steps;
         p.rotate = 0;
+        // four weight row blocks per workgroup (up to three workgroups per CU) with the same K chunks, when those
+        // workgroups still fill the CUs: F16 weights, both activation blocks in use
+        if (g_ring_wide && fmt == 0 && M > 32 && (!g_force_S || g_ring_wide == 2)) {
+            const int nt4 = (Nb + 3) / 4;
+            bool wide = g_ring_wide == 2 || (long)nt4 * p.S >= (long)cus * 7 / 8;
+            // under a very long K (the lm_head backward) twice the chunks, up to 16, cost little: the planes stay a few percent of
+            // the weights (2560 x 151936: 157 -> 139 us; with 28 chunks on 1152 x 262144 it loses, 122 -> 126 us)
+            if (!wide && !g_force_S && K >= 32768 && 2 * p.S <= 16) {
+                const int steps2 = (Kb + 2 * p.S - 1) / (2 * p.S), S2 = (Kb + steps2 - 1) / steps2;
+                if ((long)nt4 * S2 >= (long)cus * 7 / 8) { wide = true; p.steps = steps2; p.S = S2; }
+            }
+            if (wide) { p.wide = 1; p.nb = 4; p.kg = 1; p.nw = 8; p.n_tiles = nt4; }
+        }
         return p;
     }
     auto split = [&](int nb) {
@@ -351,7 +365,8 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
     if (half_scale != 0.f && (!p.ring || a_inv_scale)) { fprintf(stderr, "[fast_hip] gemm: half planes need a ring plan without row factors\n"); abort(); }
     if (M <= 0 || N <= 0 || K <= 0) return;
     const int Kb = tiled_kb(K), Nb = tiled_rb(N), Mb = tiled_rb(M);
-    bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2) && (p.nw == 4 || (p.nw == 8 && p.m_tiles == 1)) && W.fmt >= 0 && W.fmt <= 2;
+    bool ok = ldp >= N && p.S >= 1 && p.steps >= 1 && (p.nb == 1 || p.nb == 2 || (p.ring && p.wide && p.nb == 4)) &&
+              (p.nw == 4 || (p.nw == 8 && p.m_tiles == 1)) && W.fmt >= 0 && W.fmt <= 2;
     if (W.fmt == 0) ok = ok && W.w16;
     if (W.fmt == 1) ok = ok && W.q && W.d && W.nbq >= 0 && W.nbq <= Nb && (W.nbq == Nb || (W.w16 && (p.ring || (W.nbq % p.nb) == 0)));
     if (W.fmt == 2) ok = ok && W.q && W.d && W.kbq >= 0 && W.kbq <= Kb && (W.kbq == Kb || W.w16);
@@ -361,7 +376,8 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         abort();
     }
     if (p.ring) {
-        if (p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (Nb + 1) / 2 ||
+        if (p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (p.wide ? (Nb + 3) / 4 : (Nb + 1) / 2) ||
+            (p.wide && (W.fmt != 0 || p.kg != 1 || M <= 32)) ||
             (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb || (W.fmt != 0 && (p.kg != 2 || (half_scale != 0.f && a_inv_scale)))) {
             fprintf(stderr, "[fast_hip] gemm_ring: bad launch M=%d N=%d K=%d fmt=%d plan(kg=%d S=%d steps=%d tiles=%d)\n", M, N, K, W.fmt, p.kg, p.S, p.steps, p.n_tiles);
             abort();
@@ -378,7 +394,15 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         g.P = P; g.ldp = ldp; g.plane_stride = plane_stride;
         g.M = M; g.N = N; g.Mb = Mb; g.Nb = Nb; g.Kb = Kb; g.steps_per_chunk = p.steps;
         g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1; g.half_scale = half_scale; g.w16_ring = W.w16;
-        const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(256 * p.kg);
+        const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(p.wide ? 512 : 256 * p.kg);
+        if (p.wide) {
+#define WIDE_LAUNCH(SC, HP) launch_kargs<24>(gemm_ring_wide<SC, HP>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
+            if (a_inv_scale) WIDE_LAUNCH(1, 0); else if (half_scale != 0.f) WIDE_LAUNCH(0, 1); else WIDE_LAUNCH(0, 0);
+#undef WIDE_LAUNCH
+            HIP_CHECK(hipGetLastError());
+            if (g_prof_on) g_prof.push_back(rrec);
+            return;
+        }
 #define RING_LAUNCH(KGV, SC, HP) launch_kargs<24>(gemm_ring<KGV, SC, HP>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
 #define RING_PICK(KGV) do { if (a_inv_scale) RING_LAUNCH(KGV, 1, 0); else if (half_scale != 0.f) RING_LAUNCH(KGV, 0, 1); else RING_LAUNCH(KGV, 0, 0); } while (0)
 #define RING_LAUNCH_Q8(SC, HP, WFV) launch_kargs<24>(gemm_ring<2, SC, HP, WFV>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
@@ -583,6 +607,7 @@ void set_gemm_half_planes(int on) { g_half_planes = on ? 1 : 0; }
 int gemm_half_planes_enabled() { return g_half_planes; }
 
 void set_gemm_ring(int on) { g_ring = on; }
+void set_gemm_ring_wide(int on) { g_ring_wide = on; }
 int gemm_ring_enabled() { return g_ring; }
 
 // Which kernel multiplies an [M, K] activation block with an [N, K] weight.  Measured on MI355X (Qwen3-4B shapes):
@@ -754,6 +779,7 @@ void metal_enqueue_f16_matmul_nt(MetalBuf *A, MetalBuf *W, MetalBuf *C, int M, i
 
 void hip_gemm_force_large_m(int policy) { g_big_policy = policy; }
 void hip_gemm_ring(int on) { lmhip::set_gemm_ring(on); }
+void hip_gemm_ring_wide(int on) { lmhip::set_gemm_ring_wide(on); }
 void hip_gemm_half_planes(int on) { lmhip::set_gemm_half_planes(on); }
 void hip_gemm_large_m_split(int mode) { set_big_gemm_split(mode); }
 void hip_gemm_large_m_block(int mode) { set_big_gemm_block(mode); }
@@ -797,8 +823,10 @@ double hip_gemm_time_shape(int M, int N, int K, int nb, int wf, int S, int iters
     const bool read_only = nb == -1;                       // the weight loads of gemm_ring alone (ring_weights_only)
     if (read_only) nb = 0;
     g_force_nb = nb == 128 ? 0 : nb; g_force_S = S;
+    const int wide_was = g_ring_wide;
+    if (read_only) g_ring_wide = 0;                        // ring_weights_only walks gemm_ring's grid of two row blocks per workgroup
     GemmPlan p = plan_gemm(M, N, K, 0, wf);
-    g_force_nb = 0; g_force_S = 0;
+    g_force_nb = 0; g_force_S = 0; g_ring_wide = wide_was;
     if (used_nb) *used_nb = p.nb;
     if (used_S) *used_S = p.S;
     void *A = nullptr, *W = nullptr, *D = nullptr, *P = nullptr, *inv = nullptr;

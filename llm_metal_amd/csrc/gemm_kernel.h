@@ -448,6 +448,92 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(KARGS24)
     }
 }
 
+// gemm_ring with four weight row blocks per workgroup instead of two and one K group (F16 weights, more than 32
+// activation rows): a stage is four weight tiles and the two activation tiles, 24 KB, so the bytes a workgroup pulls into
+// LDS per weight byte are 1.5 instead of 2 -- and it is those stage bytes, weights and activation tiles together, that a
+// launch's time follows.  Eight waves: 4 x 2 output quadrants of 32 x 32; the 24 pieces of a stage are requested three per
+// wave; 48 KB of ring, up to three workgroups per CU; a workgroup walks its K chunk one step per round and every wave
+// stores its whole quadrant (no exchange).  Rounds and waits as in gemm_ring.
+template <int SCALE, int HALFP>
+__global__ __launch_bounds__(512) void gemm_ring_wide(KARGS24)
+{
+    static_assert(!(SCALE && HALFP), "final outputs stay fp32");
+    const uint64_t kw[24] = {KLIST24};
+    const GemmKArgs g = kargs_unpack<GemmKArgs>(kw);
+    constexpr int WB = 4, LOADS_PER_ROUND = 3, STAGE = (WB + 2) * 256;      // half8 elements per stage (24 KB)
+    __shared__ half8 wring[2 * STAGE];                    // [round parity][weight block 0..3, activation block 0, 1][slice][64 lanes]
+    const int lane = threadIdx.x & 63, q = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int qn = q & 3, qm = q >> 2;
+    const int r = lane & 31, h = lane >> 5;
+    const int tile = blockIdx.x % g.n_tiles, chunk = blockIdx.x / g.n_tiles;
+    const int kb_beg = chunk * g.steps_per_chunk;
+    const int nsteps = min(g.Kb, kb_beg + g.steps_per_chunk) - kb_beg;
+    // wave q requests the pieces 3 q .. 3 q + 2 of a stage: piece p = slice p % 4 of block p / 4 (blocks 0 .. 3: weight
+    // row blocks 4 tile + b; 4, 5: activation row blocks; clamped: rows beyond M or N are not stored)
+    const half8 *src[LOADS_PER_ROUND];
+    uint32_t off[LOADS_PER_ROUND];
+    bool is_w[LOADS_PER_ROUND];
+#pragma unroll
+    for (int i = 0; i < LOADS_PER_ROUND; i++) {
+        const int p = q * LOADS_PER_ROUND + i, b = p >> 2, j = p & 3;
+        is_w[i] = b < WB;
+        src[i] = is_w[i] ? reinterpret_cast<const half8 *>(g.w16_ring) + ((size_t)min(WB * tile + b, g.Nb - 1) * g.Kb + kb_beg) * 256 + j * 64 + lane
+                         : g.A + ((size_t)min(b - WB, g.Mb - 1) * g.Kb + kb_beg) * 256 + j * 64 + a_lane(lane);
+        off[i] = (uint32_t)(b * 4096 + j * 1024);
+    }
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)wring;
+    auto request = [&](int step) __attribute__((always_inline)) {
+        const uint32_t sb = base + (uint32_t)((step & 1) * STAGE * 16);
+#pragma unroll
+        for (int i = 0; i < LOADS_PER_ROUND; i++) {
+            if (is_w[i]) asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src[i] + (size_t)step * 256), "s"(sb + off[i]) : "m0", "memory");
+            else asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[i] + (size_t)step * 256), "s"(sb + off[i]) : "m0", "memory");
+        }
+    };
+    float16v acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    request(0);
+    if (nsteps > 1) request(1);
+    for (int rd = 0; rd < nsteps; rd++) {
+        // in flight: this wave's three loads of step rd and, if there is one, of step rd + 1 (loads retire in order)
+        if (rd + 1 < nsteps) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS_PER_ROUND) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        const half8 *st = wring + (rd & 1) * STAGE;
+        half8 w[4], a[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = st[(qn * 4 + j) * 64 + lane];
+#pragma unroll
+        for (int j = 0; j < 4; j++) a[j] = st[((WB + qm) * 4 + j) * 64 + lane];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                     // all waves have read this step's stage: it may be refilled
+        if (rd + 2 < nsteps) request(rd + 2);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j], w[j], acc, 0, 0, 0);
+    }
+    // D layout of v_mfma_f32_32x32x16: column = lane & 31, row = 8 (v / 4) + 4 (lane / 32) + v % 4
+    const int n = (tile * WB + qn) * 32 + r;
+    const bool inside = 64 <= g.M && (tile + 1) * 32 * WB <= g.N;
+    if constexpr (HALFP) {
+        half_t *Ph = reinterpret_cast<half_t *>(g.P) + (size_t)chunk * g.plane_stride;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = qm * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+            if (inside || (m < g.M && n < g.N)) Ph[(size_t)m * g.ldp + n] = f2h(acc[v] * g.half_scale);
+        }
+        return;
+    }
+    float *Pp = g.P + (size_t)chunk * g.plane_stride;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const int m = qm * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        float o = acc[v];
+        if (SCALE) o *= g.a_inv_scale[min(m, g.M - 1)];
+        if (inside || (m < g.M && n < g.N)) Pp[(size_t)m * g.ldp + n] = o;
+    }
+}
+
 // The weight loads of gemm_ring alone, on the same grid and through the same LDS ring: what a launch needs just to pull its
 // weight bytes into LDS (timing reference for the product; nothing is multiplied or stored).
 template <int KG>

@@ -117,7 +117,7 @@ def load():
         "hip_enqueue_q8_dequant": (None, [vp, vp, i, i]), "hip_enqueue_q8_to_f16": (None, [vp, vp, i, i]),
         "hip_gemm_time_shape": (C.c_double, [i, i, i, i, i, i, i, C.POINTER(i), C.POINTER(i)]),
         "hip_matvec_time_shape": (C.c_double, [i, i, i, i, i]),
-        "hip_gemm_profile_enable": (None, [i]), "hip_gemm_force_large_m": (None, [i]), "hip_gemm_ring": (None, [i]), "hip_gemm_half_planes": (None, [i]), "hip_mem_info": (None, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]), "hip_gemm_large_m_split": (None, [i]), "hip_gemm_large_m_block": (None, [i]), "hip_attention_flash": (None, [i]), "hip_attention_backward_one_launch": (None, [i]), "hip_gemm_image_budget_mb": (None, [i]), "hip_gemm_profile_read": (i, [C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+        "hip_gemm_profile_enable": (None, [i]), "hip_gemm_force_large_m": (None, [i]), "hip_gemm_ring": (None, [i]), "hip_gemm_ring_wide": (None, [i]), "hip_gemm_half_planes": (None, [i]), "hip_mem_info": (None, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]), "hip_gemm_large_m_split": (None, [i]), "hip_gemm_large_m_block": (None, [i]), "hip_attention_flash": (None, [i]), "hip_attention_backward_one_launch": (None, [i]), "hip_gemm_image_budget_mb": (None, [i]), "hip_gemm_profile_read": (i, [C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "hip_gemm_profile_read2": (i, [C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "wmat_create_f16": (C.POINTER(WMat), [vp, i, i]), "wmat_create_q8": (C.POINTER(WMat), [vp, i, i]),
         "wmat_convert": (C.POINTER(WMat), [vp, i, i, i]), "wmat_free": (None, [C.POINTER(WMat)]),

@@ -31,6 +31,7 @@ def _default_kernel_policies(request):
     L.hip_gemm_large_m_split(1)
     L.hip_gemm_large_m_block(0)
     L.hip_gemm_ring(1)
+    L.hip_gemm_ring_wide(1)
     L.hip_gemm_half_planes(1)
     L.hip_attention_flash(-1)
     L.hip_attention_backward_one_launch(1)

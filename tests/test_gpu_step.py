@@ -118,6 +118,13 @@ CASES = [
     C1.with_(name="wide_ffn_groups_f32_planes", NL=1, IS=4224, V=1024, seq=64),
     C1.with_(name="hd128_f32_planes", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
     C1.with_(name="c1_q8_f32_planes", weight_format="q8_0"),
+    # gemm_ring_wide (four weight row blocks per workgroup) forced onto every F16 product of 33 to 64 rows: whole tiles,
+    # ragged row counts, matrices whose last tile is partial, half and fp32 planes
+    C1.with_(name="c1_ringwide"),
+    TINY_GEMMA3.with_(name="gemma_ringwide"),
+    C1.with_(name="wide_ffn_groups_ringwide", NL=1, IS=4224, V=1024, seq=64),
+    C1.with_(name="ragged_seq40_ringwide", NL=2, batch=1, seq=40, R=4, alpha=8.0),
+    C1.with_(name="hd128_ringwide_f32_planes", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
 ]
 
 
@@ -145,6 +152,7 @@ def test_train_steps_match_oracle(cfg):
     # F16 weights at sizes the oracle cannot follow); everything else takes the measured rule
     lib.load().hip_gemm_force_large_m(2 if "_lds" in cfg.name else 1 if "big_m" in cfg.name else 0)
     lib.load().hip_gemm_ring(0 if cfg.name.endswith("_tiled") else 1)
+    lib.load().hip_gemm_ring_wide(2 if "_ringwide" in cfg.name else 1)
     lib.load().hip_attention_backward_one_launch(0 if cfg.name.endswith("_two_launch") else 1)
     lib.load().hip_gemm_half_planes(0 if cfg.name.endswith("_f32_planes") else 1)
     lib.load().hip_gemm_large_m_split(3 if cfg.name.endswith("_chunks") else 1)
