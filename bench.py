@@ -399,7 +399,7 @@ def _main():
                            # full-parameter pass: the products, the weight gradients (F16 read-modify-write of the accumulators), the
                            # apply (W, G and the transposed image) and the operand transposes (time only) are timed together
                            "gemm_tiled, gemm_big_f16*, k_wgrad, k_apply_retile, k_transpose_scaled_jobs" if cfg.R == 0 else
-                           "gemm_ring, gemm_ring_wide" if 32 < cfg.BN <= 64 and args.gemm_ring and args.gemm_ring_wide and cfg.weight_format == "f16" else
+                           "gemm_ring, gemm_ring_wide" if 32 < cfg.BN <= 64 and args.gemm_ring and args.gemm_ring_wide else
                            "gemm_ring" if cfg.BN <= 64 and args.gemm_ring else "gemm_tiled"),
                 "launches_per_step": n // prof_steps,
                 "avg_launch_us": round(tms.value * 1e3 / max(n, 1), 2),

@@ -166,9 +166,9 @@ void hip_gemm_force_large_m(int policy);
  * unpacked to fp16 from LDS), 0 = the kernel with one K step per wave in registers (gemm_tiled: 13 to 19 K chunks, Q8_0
  * unpacked in registers), which every product of more rows takes.  Same results up to the order of the sums. */
 void hip_gemm_ring(int on);
-/* gemm_ring with four weight row blocks per workgroup (1.5 instead of 2 bytes into LDS per weight byte) for the F16 products
- * of 33 to 64 rows that have enough row tiles to fill the CUs with such workgroups: 1 = on, 0 = off, 2 = for every such product
- * whatever its size (tests). */
+/* gemm_ring with four weight row blocks per workgroup (1.5 instead of 2 bytes into LDS per F16 weight byte; Q8_0 tiles
+ * likewise quantised up to LDS) for the products of 33 to 64 rows that have enough row tiles to give every CU such a
+ * workgroup: 1 = on, 0 = off, 2 = for every product of 33 to 64 rows whatever its size (tests). */
 void hip_gemm_ring_wide(int on);
 /* 1 (default): a LoRA training state of at most 64 rows (frozen F16 or Q8_0 weights) stores the K-split planes of five of its eight
  * products per layer (gate|up and down forward; down, gate|up and O backward) as halves: every chunk sum, formed in fp32,

@@ -313,11 +313,13 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
         p.steps = (Kb + S - 1) / S;
         p.S = (Kb + p.steps - 1) / p.steps;
         p.rotate = 0;
-        // four weight row blocks per workgroup (up to three workgroups per CU) with the same K chunks, when those
-        // workgroups still fill the CUs: F16 weights, both activation blocks in use
-        if (g_ring_wide && fmt == 0 && M > 32 && (!g_force_S || g_ring_wide == 2)) {
+        // four weight row blocks per workgroup (up to three workgroups per CU) with the same K chunks, when every CU
+        // still gets such a workgroup (with 0.9 of them -- 9728 x 2560 and 6176 x 2560 in three and five chunks -- the
+        // products alone gain 2-7 %, the step nothing with F16 weights and it loses 1 % with Q8_0); both activation
+        // blocks in use
+        if (g_ring_wide && M > 32 && (!g_force_S || g_ring_wide == 2)) {
             const int nt4 = (Nb + 3) / 4;
-            bool wide = g_ring_wide == 2 || (long)nt4 * p.S >= (long)cus * 7 / 8;
+            bool wide = g_ring_wide == 2 || (long)nt4 * p.S >= (long)cus;
             // under a very long K (the lm_head backward) twice the chunks, up to 16, cost little: the planes stay a few percent of
             // the weights (2560 x 151936: 157 -> 139 us; with 28 chunks on 1152 x 262144 it loses, 122 -> 126 us)
             if (!wide && !g_force_S && K >= 32768 && 2 * p.S <= 16) {
@@ -377,8 +379,8 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
     }
     if (p.ring) {
         if (p.m_tiles != 1 || M > 64 || (p.kg != 1 && p.kg != 2 && p.kg != 4) || p.n_tiles != (p.wide ? (Nb + 3) / 4 : (Nb + 1) / 2) ||
-            (p.wide && (W.fmt != 0 || p.kg != 1 || M <= 32)) ||
-            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb || (W.fmt != 0 && (p.kg != 2 || (half_scale != 0.f && a_inv_scale)))) {
+            (p.wide && (p.kg != 1 || M <= 32)) ||
+            (long)p.S * p.steps < Kb || (long)(p.S - 1) * p.steps >= Kb || (W.fmt != 0 && ((!p.wide && p.kg != 2) || (half_scale != 0.f && a_inv_scale)))) {
             fprintf(stderr, "[fast_hip] gemm_ring: bad launch M=%d N=%d K=%d fmt=%d plan(kg=%d S=%d steps=%d tiles=%d)\n", M, N, K, W.fmt, p.kg, p.S, p.steps, p.n_tiles);
             abort();
         }
@@ -396,8 +398,10 @@ void launch_gemm(const half_t *A, const float *a_inv_scale, const WeightOp &W,
         g.n_tiles = p.n_tiles; g.S = p.S; g.m_tiles = 1; g.half_scale = half_scale; g.w16_ring = W.w16;
         const dim3 rgrid((unsigned)(p.n_tiles * p.S)), rblock(p.wide ? 512 : 256 * p.kg);
         if (p.wide) {
-#define WIDE_LAUNCH(SC, HP) launch_kargs<24>(gemm_ring_wide<SC, HP>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
-            if (a_inv_scale) WIDE_LAUNCH(1, 0); else if (half_scale != 0.f) WIDE_LAUNCH(0, 1); else WIDE_LAUNCH(0, 0);
+#define WIDE_LAUNCH(SC, HP, WFV) launch_kargs<24>(gemm_ring_wide<SC, HP, WFV>, rgrid, rblock, 0, stream(), g, g_prof_on ? ra : nullptr, g_prof_on ? rb : nullptr)
+#define WIDE_PICK(WFV) do { if (a_inv_scale) WIDE_LAUNCH(1, 0, WFV); else if (half_scale != 0.f) WIDE_LAUNCH(0, 1, WFV); else WIDE_LAUNCH(0, 0, WFV); } while (0)
+            if (W.fmt == 1) WIDE_PICK(1); else if (W.fmt == 2) WIDE_PICK(2); else WIDE_PICK(0);
+#undef WIDE_PICK
 #undef WIDE_LAUNCH
             HIP_CHECK(hipGetLastError());
             if (g_prof_on) g_prof.push_back(rrec);

@@ -448,16 +448,21 @@ __global__ __launch_bounds__(256 * KG) void gemm_ring(KARGS24)
     }
 }
 
-// gemm_ring with four weight row blocks per workgroup instead of two and one K group (F16 weights, more than 32
-// activation rows): a stage is four weight tiles and the two activation tiles, 24 KB, so the bytes a workgroup pulls into
-// LDS per weight byte are 1.5 instead of 2 -- and it is those stage bytes, weights and activation tiles together, that a
-// launch's time follows.  Eight waves: 4 x 2 output quadrants of 32 x 32; the 24 pieces of a stage are requested three per
-// wave; 48 KB of ring, up to three workgroups per CU; a workgroup walks its K chunk one step per round and every wave
-// stores its whole quadrant (no exchange).  Rounds and waits as in gemm_ring.
-template <int SCALE, int HALFP>
+// gemm_ring with four weight row blocks per workgroup instead of two and one K group (more than 32 activation rows): a
+// stage is four weight tiles and the two activation tiles, 24 KB of LDS, so the bytes a workgroup pulls into LDS per F16
+// weight byte are 1.5 instead of 2 (Q8_0: 16.5 KB instead of 24.7 KB per four tiles) -- and it is those stage bytes,
+// weights and activation tiles together, that a launch's time follows.  Eight waves: 4 x 2 output quadrants of 32 x 32;
+// 48 KB of ring, up to three workgroups per CU; a workgroup walks its K chunk one step per round and every wave stores
+// its whole quadrant (no exchange).  Rounds and waits as in gemm_ring.
+// WF 0: the 24 pieces of a stage are requested three per wave.  WF 1, 2 (Q8_0 tiles, quantised up to LDS as in gemm_ring):
+// waves 0 .. 3 request one weight tile each (four loads: a quantised tile's 2 KB and its scales, twice; or the four
+// pieces of an F16 tile that the operand carries), waves 4 .. 7 two pieces each of the activation blocks; the waits count
+// per wave.
+template <int SCALE, int HALFP, int WF = 0>
 __global__ __launch_bounds__(512) void gemm_ring_wide(KARGS24)
 {
     static_assert(!(SCALE && HALFP), "final outputs stay fp32");
+    static_assert(WF >= 0 && WF <= 2, "weight format");
     const uint64_t kw[24] = {KLIST24};
     const GemmKArgs g = kargs_unpack<GemmKArgs>(kw);
     constexpr int WB = 4, LOADS_PER_ROUND = 3, STAGE = (WB + 2) * 256;      // half8 elements per stage (24 KB)
@@ -468,7 +473,8 @@ __global__ __launch_bounds__(512) void gemm_ring_wide(KARGS24)
     const int tile = blockIdx.x % g.n_tiles, chunk = blockIdx.x / g.n_tiles;
     const int kb_beg = chunk * g.steps_per_chunk;
     const int nsteps = min(g.Kb, kb_beg + g.steps_per_chunk) - kb_beg;
-    // wave q requests the pieces 3 q .. 3 q + 2 of a stage: piece p = slice p % 4 of block p / 4 (blocks 0 .. 3: weight
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)wring;
+    // WF 0: wave q requests the pieces 3 q .. 3 q + 2 of a stage: piece p = slice p % 4 of block p / 4 (blocks 0 .. 3: weight
     // row blocks 4 tile + b; 4, 5: activation row blocks; clamped: rows beyond M or N are not stored)
     const half8 *src[LOADS_PER_ROUND];
     uint32_t off[LOADS_PER_ROUND];
@@ -481,13 +487,54 @@ __global__ __launch_bounds__(512) void gemm_ring_wide(KARGS24)
                          : g.A + ((size_t)min(b - WB, g.Mb - 1) * g.Kb + kb_beg) * 256 + j * 64 + a_lane(lane);
         off[i] = (uint32_t)(b * 4096 + j * 1024);
     }
-    const uint32_t base = (uint32_t)(uintptr_t)(lds_void_t *)wring;
+    // WF 1, 2: the weight row block wave q < 4 requests, the one this wave multiplies (fmt 1: from nbq on they are F16
+    // tiles), and for q >= 4 the two activation pieces (slices 2 (q & 1), + 1 of block (q - 4) / 2)
+    const int wb_req = min(WB * tile + qn, g.Nb - 1);     // (q < 4: qn = q; also the block that waves qn and 4 + qn multiply)
+    const bool q8_rows = WF == 1 && wb_req < g.W.nbq;
+    const half8 *qsrc = nullptr;
+    uint32_t qoff = 0;
+    if constexpr (WF != 0) {
+        if (q < WB) {
+            qsrc = WF == 1 ? reinterpret_cast<const half8 *>(g.W.w16) + ((size_t)max(wb_req - g.W.nbq, 0) * g.Kb + kb_beg) * 256 + lane
+                           : reinterpret_cast<const half8 *>(g.W.w16) + (size_t)wb_req * (g.Kb - g.W.kbq) * 256 + lane;    // (+ the F16 step's index)
+            qoff = (uint32_t)(q * 4096);
+        } else {
+            const int b = (q - WB) >> 1, s0 = 2 * (q & 1);
+            qsrc = g.A + ((size_t)min(b, g.Mb - 1) * g.Kb + kb_beg) * 256 + s0 * 64 + a_lane(lane);
+            qoff = (uint32_t)((WB + b) * 4096 + s0 * 1024);
+        }
+    }
+    // a quantised tile: int8 at slot + 0 .. 2047, scales at + 2048 .. 2175 (and once more at + 2304)
+    auto request_q8 = [&](uint32_t sb, size_t tile_index) __attribute__((always_inline)) {
+        const uint8_t *qp = g.W.q + tile_index * 2048 + lane * 16;
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(qp), "s"(sb) : "m0", "memory");
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(qp + 1024), "s"(sb + 1024u) : "m0", "memory");
+        const half_t *dp = g.W.d + tile_index * 64 + (lane & 7) * 8;
+        if (lane < 8) {
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(dp), "s"(sb + 2048u) : "m0", "memory");
+            asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(dp), "s"(sb + 2304u) : "m0", "memory");
+        }
+    };
     auto request = [&](int step) __attribute__((always_inline)) {
         const uint32_t sb = base + (uint32_t)((step & 1) * STAGE * 16);
+        if constexpr (WF == 0) {
 #pragma unroll
-        for (int i = 0; i < LOADS_PER_ROUND; i++) {
-            if (is_w[i]) asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src[i] + (size_t)step * 256), "s"(sb + off[i]) : "m0", "memory");
-            else asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[i] + (size_t)step * 256), "s"(sb + off[i]) : "m0", "memory");
+            for (int i = 0; i < LOADS_PER_ROUND; i++) {
+                if (is_w[i]) asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(src[i] + (size_t)step * 256), "s"(sb + off[i]) : "m0", "memory");
+                else asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(src[i] + (size_t)step * 256), "s"(sb + off[i]) : "m0", "memory");
+            }
+        } else if (q < WB) {
+            const int kt = kb_beg + step;
+            if (WF == 1 && q8_rows) { request_q8(sb + qoff, (size_t)wb_req * g.Kb + kt); return; }
+            if (WF == 2 && kt < g.W.kbq) { request_q8(sb + qoff, (size_t)wb_req * g.W.kbq + kt); return; }
+            const half8 *f = WF == 1 ? qsrc + (size_t)step * 256 : qsrc + (size_t)(kt - g.W.kbq) * 256;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(f + j * 64), "s"(sb + qoff + (uint32_t)(j * 1024)) : "m0", "memory");
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(qsrc + (size_t)step * 256 + j * 64), "s"(sb + qoff + (uint32_t)(j * 1024)) : "m0", "memory");
         }
     };
     float16v acc;
@@ -496,14 +543,32 @@ __global__ __launch_bounds__(512) void gemm_ring_wide(KARGS24)
     request(0);
     if (nsteps > 1) request(1);
     for (int rd = 0; rd < nsteps; rd++) {
-        // in flight: this wave's three loads of step rd and, if there is one, of step rd + 1 (loads retire in order)
-        if (rd + 1 < nsteps) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS_PER_ROUND) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // in flight: this wave's loads of step rd and, if there is one, of step rd + 1 (loads retire in order)
+        if (rd + 1 < nsteps) {
+            if constexpr (WF == 0) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS_PER_ROUND) : "memory");
+            else if (q < WB) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        } else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         const half8 *st = wring + (rd & 1) * STAGE;
         half8 w[4], a[4];
+        if ((WF == 1 && q8_rows) || (WF == 2 && kb_beg + rd < g.W.kbq)) {
+            const uint8_t *sq = reinterpret_cast<const uint8_t *>(st) + qn * 4096;
+            const uint4v r0 = *reinterpret_cast<const uint4v *>(sq + lane * 16), r1 = *reinterpret_cast<const uint4v *>(sq + 1024 + lane * 16);
+            const half_t *sd = reinterpret_cast<const half_t *>(sq + 2048);
+            if (WF == 1) {
+                const half8 d = bcast8(sd[lane]);
+                w[0] = q8_unpack8(r0[0], r0[1]) * d; w[1] = q8_unpack8(r0[2], r0[3]) * d;
+                w[2] = q8_unpack8(r1[0], r1[1]) * d; w[3] = q8_unpack8(r1[2], r1[3]) * d;
+            } else {
+                const half8 *sc = reinterpret_cast<const half8 *>(sd + (lane >> 5) * 32);
+                w[0] = q8_unpack8(r0[0], r0[1]) * sc[0]; w[1] = q8_unpack8(r0[2], r0[3]) * sc[1];
+                w[2] = q8_unpack8(r1[0], r1[1]) * sc[2]; w[3] = q8_unpack8(r1[2], r1[3]) * sc[3];
+            }
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; j++) w[j] = st[(qn * 4 + j) * 64 + lane];
+            for (int j = 0; j < 4; j++) w[j] = st[(qn * 4 + j) * 64 + lane];
+        }
 #pragma unroll
         for (int j = 0; j < 4; j++) a[j] = st[((WB + qm) * 4 + j) * 64 + lane];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

@@ -118,10 +118,15 @@ CASES = [
     C1.with_(name="wide_ffn_groups_f32_planes", NL=1, IS=4224, V=1024, seq=64),
     C1.with_(name="hd128_f32_planes", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
     C1.with_(name="c1_q8_f32_planes", weight_format="q8_0"),
-    # gemm_ring_wide (four weight row blocks per workgroup) forced onto every F16 product of 33 to 64 rows: whole tiles,
-    # ragged row counts, matrices whose last tile is partial, half and fp32 planes
+    # gemm_ring_wide (four weight row blocks per workgroup) forced onto every product of 33 to 64 rows: whole tiles,
+    # ragged row counts, matrices whose last tile is partial, half and fp32 planes, F16 and Q8_0 weights (with the F16
+    # adapter tiles behind the fused Q | K | V rows, and row / K block counts that are not multiples of four)
     C1.with_(name="c1_ringwide"),
-    TINY_GEMMA3.with_(name="gemma_ringwide"),
+    TINY_GEMMA3.with_(name="gemma_ringwide", seq=48),
+    C1.with_(name="c1_q8_ringwide", weight_format="q8_0"),
+    C1.with_(name="q8_odd_blocks_ringwide", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format="q8_0"),
+    TINY_GEMMA3.with_(name="gemma_q8_ringwide", seq=48, weight_format="q8_0"),
+    C1.with_(name="c1_q8_ringwide_f32_planes", weight_format="q8_0"),
     C1.with_(name="wide_ffn_groups_ringwide", NL=1, IS=4224, V=1024, seq=64),
     C1.with_(name="ragged_seq40_ringwide", NL=2, batch=1, seq=40, R=4, alpha=8.0),
     C1.with_(name="hd128_ringwide_f32_planes", NL=2, D=256, Hq=4, Hkv=2, hd=128, IS=512, V=2048, seq=64),
@@ -185,6 +190,35 @@ def test_train_steps_match_oracle(cfg):
     lib.load().hip_gemm_large_m_block(0)
     lib.load().hip_attention_flash(-1)
     lib.load().hip_gemm_image_budget_mb(65536)
+
+
+@pytest.mark.parametrize("half_planes", [0, 1], ids=["f32_planes", "half_planes"])
+@pytest.mark.parametrize("fmt", ["f16", "q8_0"])
+def test_both_workgroup_shapes_of_the_ring_kernel_give_the_same_step(fmt, half_planes):
+    """gemm_ring (64 weight rows per workgroup, two K groups) and gemm_ring_wide (128 rows, one K group) form the same
+    products from the same tiles and differ only in the order of a chunk's fp32 sums.  Every product's activation operand
+    is rounded to fp16 (and, with planes of halves, five chunk sums per layer as well), so a last-bit difference in fp32
+    becomes an fp16 rounding step here and there: the logits and adapter gradients of one step (learning rate 0) agree
+    to a few fp16 steps, ten times closer than the bar against the oracle."""
+    cfg = C1.with_(name="ring_shapes", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format=fmt)
+    model = make_model(cfg, seed=21, gamma_jitter=0.1)
+    tok, tgt = make_batch(cfg, seed=30)
+    from llm_metal_amd import lib
+    L = lib.load()
+    L.hip_gemm_half_planes(half_planes)
+    out = {}
+    with SFTState(cfg, model) as st:
+        for wide in (0, 2):
+            L.hip_gemm_ring_wide(wide)
+            st.set_lora(model["lora"])
+            loss = st.train_step(tok, tgt, 0.0)
+            out[wide] = (loss, st.logits().copy(), st.lora_grads().copy())
+    L.hip_gemm_ring_wide(1)
+    L.hip_gemm_half_planes(1)
+    tol = 1e-3
+    assert abs(out[0][0] - out[2][0]) <= tol * abs(out[0][0]), (out[0][0], out[2][0])
+    assert rel(out[2][1], out[0][1]) < tol, rel(out[2][1], out[0][1])
+    assert rel(out[2][2], out[0][2]) < 5 * tol, rel(out[2][2], out[0][2])
 
 
 @pytest.mark.parametrize("bad", [dict(hd=516, Hq=1, Hkv=1), dict(seq=4097), dict(Hq=120, Hkv=8, hd=128, D=256), dict(R=18)],
