@@ -81,6 +81,7 @@ struct GemmPlan {
 // nbq: Q8_0 row blocks of a fmt-1 operand (an odd count forces one row block per wave); fmt: WeightOp::fmt of the operand
 GemmPlan plan_gemm(int M, int N, int K, int nbq = 0, int fmt = 0);
 void set_gemm_ring(int on);
+int gemm_ring_wide_mode();
 void set_gemm_ring_wide(int on);     // 1: products with enough row tiles take gemm_ring_wide; 2: every F16 product of 33 to 64 rows (tests)
 int gemm_ring_enabled();            // 1 (default): products of up to 64 rows take gemm_ring (Q8_0 tiles stay quantised up to LDS); 0: gemm_tiled
 

@@ -315,8 +315,9 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
         p.rotate = 0;
         // four weight row blocks per workgroup (up to three workgroups per CU) with the same K chunks, when every CU
         // still gets such a workgroup (with 0.9 of them -- 9728 x 2560 and 6176 x 2560 in three and five chunks -- the
-        // products alone gain 2-7 %, the step nothing with F16 weights and it loses 1 % with Q8_0); both activation
-        // blocks in use
+        // products alone gain 2-7 %, the step nothing with F16 weights and it loses 1 % with Q8_0); more than 32 rows: with one
+        // activation block (20 KB stages, two waves requesting nothing) batched generation on a training state's tiles
+        // took 3.66 instead of 3.63 ms per step of eight tokens
         if (g_ring_wide && M > 32 && (!g_force_S || g_ring_wide == 2)) {
             const int nt4 = (Nb + 3) / 4;
             bool wide = g_ring_wide == 2 || (long)nt4 * p.S >= (long)cus;
@@ -612,6 +613,7 @@ int gemm_half_planes_enabled() { return g_half_planes; }
 
 void set_gemm_ring(int on) { g_ring = on; }
 void set_gemm_ring_wide(int on) { g_ring_wide = on; }
+int gemm_ring_wide_mode() { return g_ring_wide; }
 int gemm_ring_enabled() { return g_ring; }
 
 // Which kernel multiplies an [M, K] activation block with an [N, K] weight.  Measured on MI355X (Qwen3-4B shapes):

@@ -190,10 +190,12 @@ size_t max_planes_elems(SFTState *s)
     const Sh shapes[] = {{s->nq_ext, s->D}, {s->D, s->qd}, {2 * s->IS, s->D}, {s->D, s->IS}, {s->V, s->D},
                          {s->D, s->V}, {s->IS, s->D}, {s->D, 2 * s->IS}, {s->qd, s->D}, {s->D, s->nq_ext}};
     size_t mx = 0;
-    const int ring_was = gemm_ring_enabled();             // the kernel family can be switched at run time: room for either
+    const int ring_was = gemm_ring_enabled(), wide_was = gemm_ring_wide_mode();   // the kernel family can be switched at run time: room for either
     for (int ring = 0; ring < 2; ring++)
+    for (int wide = 0; wide <= ring; wide++)              // (the wide workgroups may take twice the K chunks)
     for (const Sh &sh : shapes) {
         set_gemm_ring(ring);
+        set_gemm_ring_wide(wide);
         GemmPlan p = plan_gemm(s->BN, sh.N, sh.K, (s->q8_native && s->R > 0 && sh.N == s->nq_ext && sh.K == s->D) ? (s->qd + 2 * s->kd) / 32 : 0, s->q8_native ? 1 : 0);
         // whichever kernel the product takes (the choice can be forced at run time): the planes of the streaming kernel, or
         // up to four K chunks of the large-M one; the LM head writes the logits directly unless the streaming kernel splits K
@@ -202,6 +204,7 @@ size_t max_planes_elems(SFTState *s)
         if (e > mx) mx = e;
     }
     set_gemm_ring(ring_was);
+    set_gemm_ring_wide(wide_was);
     return mx;
 }
 

@@ -221,6 +221,27 @@ def test_both_workgroup_shapes_of_the_ring_kernel_give_the_same_step(fmt, half_p
     assert rel(out[2][2], out[0][2]) < 5 * tol, rel(out[2][2], out[0][2])
 
 
+def test_the_workgroup_shape_can_be_switched_on_a_live_state_whose_lm_head_backward_takes_twice_the_chunks():
+    """Under a vocabulary of 32 768 the LM head's backward takes gemm_ring_wide at twice gemm_ring's K chunks, hence twice
+    the planes: a state created while the switch was off has room for them (the plane buffer is sized for either shape),
+    and the step gives the same loss and gradient norm both ways."""
+    cfg = C1.with_(name="long_head_switch", NL=1, D=1792, Hq=14, Hkv=2, hd=128, IS=2048, V=32768, seq=64, tied=False)
+    model = make_model(cfg, seed=5)
+    tok, tgt = make_batch(cfg, seed=6)
+    from llm_metal_amd import lib
+    L = lib.load()
+    L.hip_gemm_ring_wide(0)
+    out = {}
+    with SFTState(cfg, model) as st:
+        for wide in (0, 1):
+            L.hip_gemm_ring_wide(wide)
+            st.set_lora(model["lora"])
+            out[wide] = (st.train_step(tok, tgt, 0.0), st.grad_norm())
+    L.hip_gemm_ring_wide(1)
+    assert np.isfinite(out[0][0]) and abs(out[0][0] - out[1][0]) <= 1e-4 * abs(out[0][0]), out
+    assert abs(out[0][1] - out[1][1]) <= 2e-3 * out[0][1], out
+
+
 @pytest.mark.parametrize("bad", [dict(hd=516, Hq=1, Hkv=1), dict(seq=4097), dict(Hq=120, Hkv=8, hd=128, D=256), dict(R=18)],
                          ids=["head_dim_516", "seq_4097", "qkv_row_beyond_lds", "rank_18"])
 def test_dimensions_beyond_the_limits_are_refused_at_creation(bad, capfd):
