@@ -321,9 +321,11 @@ GemmPlan plan_gemm(int M, int N, int K, int nbq, int fmt)
         if (g_ring_wide && M > 32 && (!g_force_S || g_ring_wide == 2)) {
             const int nt4 = (Nb + 3) / 4;
             bool wide = g_ring_wide == 2 || (long)nt4 * p.S >= (long)cus;
-            // under a very long K (the lm_head backward) twice the chunks, up to 16, cost little: the planes stay a few percent of
-            // the weights (2560 x 151936: 157 -> 139 us; with 28 chunks on 1152 x 262144 it loses, 122 -> 126 us)
-            if (!wide && !g_force_S && K >= 32768 && 2 * p.S <= 16) {
+            // under a long K twice the chunks, up to 16, cost little: the planes stay a few percent of the weights.  The
+            // lm_head backward (2560 x 151936: 157 -> 139 us alone; with 28 chunks on 1152 x 262144 it loses, 122 -> 126 us),
+            // and with F16 weights the down forward and the gate|up backward (K = 9728, 19456; six -> twelve chunks: the
+            // step 7.17 -> 7.09 ms; from K = 4096 on the same; with Q8_0 weights the step loses 0.4 %)
+            if (!wide && !g_force_S && K >= (fmt == 0 ? 8192 : 32768) && 2 * p.S <= 16) {
                 const int steps2 = (Kb + 2 * p.S - 1) / (2 * p.S), S2 = (Kb + steps2 - 1) / steps2;
                 if ((long)nt4 * S2 >= (long)cus * 7 / 8) { wide = true; p.steps = steps2; p.S = S2; }
             }
