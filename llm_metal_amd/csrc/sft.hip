@@ -595,7 +595,9 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
         qb.dq_f = at<float>(s->dq_f, keepL * BN * qd); qb.dv_f = nullptr; qb.dh = at<float>(s->dh, keepL * BN * (R ? 2 * R : 1));
         if (kv_shares) { qb.dkp = ab.dkp; qb.dvp = ab.dvp; qb.rows_total = BN; qb.dv_f = ab.dv; }
         qb.out16 = d16[3]; qb.inv_scale = dinv[3];
-        if (mode == BWD_LORA) qb.pf = prefetch_for(s, wop(s, W_QKV, L, true), D, s->nq_ext, 1024);
+        // (adapters only: the gradient of the first layer's input has no consumer, so its product and norm backward are not run)
+        const bool input_grad = mode != BWD_LORA || L > 0;
+        if (mode == BWD_LORA && input_grad) qb.pf = prefetch_for(s, wop(s, W_QKV, L, true), D, s->nq_ext, 1024);
         launch_qkv_bwd(qb, BN);
         if (defer) {
             // the layer's four weight gradients: eight transposes in one launch, then G += dY^T X for the four matrices in one
@@ -625,6 +627,7 @@ void backward_impl(SFTState *s, int mode = BWD_LORA, float lr = 0.f)
                         s->wqkv, s->wqkvT, s->gqkv, L * s->st_qkv, L * s->st_qkvT);
 
         // dln1 = [dq|dk|dv|dh] [Wq;Wk;Wv;A_q;A_v]; dx += RNB(x_in, dln1; g_in); clamp     [:956-980]
+        if (!input_grad) break;
         Planes pl = gemm(s, d16[3], dinv[3], wop(s, W_QKV, L, true), D, s->nq_ext);
         NormBwdArgs n1{};
         n1.dy = pl; n1.x_saved = at<float>(s->xs, (size_t)(2 * L) * xsz); n1.g = at<float>(s->g_in, (size_t)L * D);
