@@ -177,6 +177,29 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
     const bool lora = RK != 0 && a.R > 0 && kind != 1;
     const float *B = kind == 0 ? a.Bq : a.Bv;
 
+    // what the epilogue needs and nothing computed here decides -- the norm weights, the rotation, the rows of B --
+    // is requested before the planes, so that all of it is one round trip
+    const int pos = (int)(row % a.seq);
+    float g0[NP], g1[NP]; float2 cs[NP];
+    if (kind != 2) {
+        const float *g = kind == 0 ? a.g_q : a.g_k;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int d = min(lane + 64 * p, half - 1);
+            g0[p] = g[d]; g1[p] = g[d + half]; cs[p] = a.rope[(size_t)pos * half + d];
+        }
+    }
+    constexpr bool B_AHEAD = NP == 1 && RK == 16;          // (more pairs per lane would hold too many registers)
+    float4 bw0[4], bw1[4];
+    if constexpr (B_AHEAD) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) bw0[i] = bw1[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (lora && lane < half) {
+            const float *b0 = B + (size_t)(h * hd + lane) * a.R, *b1 = b0 + (size_t)half * a.R;
+#pragma unroll
+            for (int i = 0; i < 4; i++) { bw0[i] = ld4(b0 + 4 * i); bw1[i] = ld4(b1 + 4 * i); }
+        }
+    }
     // everything this lane reads from the planes in one go: positions p (first half of the head), NP + p (second
     // half) and 2 NP (the lane's entry of x A^T)
     float x0[NP], x1[NP], tval;
@@ -206,7 +229,10 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
             if constexpr (RK == 16) {                          // t through scalar registers, whole rows of B as 16-byte loads
                 float4 w0[4], w1[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) { w0[i] = w1[i] = make_float4(0.f, 0.f, 0.f, 0.f); if (d < half) { w0[i] = ld4(b0 + 4 * i); w1[i] = ld4(b1 + 4 * i); } }
+                for (int i = 0; i < 4; i++) {
+                    if constexpr (B_AHEAD) { w0[i] = bw0[i]; w1[i] = bw1[i]; }
+                    else { w0[i] = w1[i] = make_float4(0.f, 0.f, 0.f, 0.f); if (d < half) { w0[i] = ld4(b0 + 4 * i); w1[i] = ld4(b1 + 4 * i); } }
+                }
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float t0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tval), 4 * i));
@@ -254,10 +280,8 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
     }
     ss = wave_sum(ss);
     const float inv = rsqrtf(ss / (float)hd + a.eps);
-    const float *g = kind == 0 ? a.g_q : a.g_k;
     float *pre = kind == 0 ? a.q_pre : a.k_pre, *fin = kind == 0 ? a.q_fin : a.k_fin;
     const int W = kind == 0 ? qd : kd;
-    const int pos = (int)(row % a.seq);
 #pragma unroll
     for (int p = 0; p < NP; p++) {
         const int d = lane + 64 * p;
@@ -265,9 +289,8 @@ __global__ __launch_bounds__(TB) void k_qkv_post(QkvPostArgs a)
         const size_t o = row * W + h * hd + d;
         pre[o] = x0[p];
         pre[o + half] = x1[p];
-        const float n0 = x0[p] * inv * g[d], n1 = x1[p] * inv * g[d + half];
-        const float2 cs = a.rope[(size_t)pos * half + d];
-        const float f0 = n0 * cs.x - n1 * cs.y, f1 = n0 * cs.y + n1 * cs.x;
+        const float n0 = x0[p] * inv * g0[p], n1 = x1[p] * inv * g1[p];
+        const float f0 = n0 * cs[p].x - n1 * cs[p].y, f1 = n0 * cs[p].y + n1 * cs[p].x;
         fin[o] = f0;
         fin[o + half] = f1;
         if (kind == 1 && a.kT) {
