@@ -80,6 +80,16 @@ __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv && !padded) x[t] = ld4(base + 4 * v);
     }
+    // one value per thread: the norm weights are requested with the row, not after the reductions they do not depend on
+    // (a round trip each); with more values per thread the registers are worth more
+    constexpr bool AHEAD = MAXV == 1;
+    float4 gn[MAXV], gb[MAXV];
+    if constexpr (AHEAD) {
+        const int v = threadIdx.x;
+        gn[0] = gb[0] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv && a.g_norm) gn[0] = ld4(a.g_norm + 4 * v);
+        if (v < nv && a.branch.S > 0 && a.g_branch) gb[0] = ld4(a.g_branch + 4 * v);
+    }
     if (a.branch.S > 0) // (many rows: a plane per round trip and 48 registers, so that eight workgroups fit a CU: 25.5 -> 22.7 us at 2048 x 2560)
     planes_at4_multi<MAXV, (MAXV == 1 ? 20 : NT == RB ? 6 : 1), GROUPED>(a.branch, rows, cols, ok, b);
     if (gather && a.emb_scale != 1.0f) {
@@ -101,7 +111,8 @@ __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
             if (v >= nv) continue;
             if (a.g_branch) {
                 if (a.branch_raw_out) st4(a.branch_raw_out + r * D + 4 * v, b[t]);
-                const float4 g = ld4(a.g_branch + 4 * v);
+                float4 g;
+                if constexpr (AHEAD) g = gb[t]; else g = ld4(a.g_branch + 4 * v);
                 x[t].x += b[t].x * inv * g.x; x[t].y += b[t].y * inv * g.y;
                 x[t].z += b[t].z * inv * g.z; x[t].w += b[t].w * inv * g.w;
             } else {
@@ -124,7 +135,8 @@ __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
     for (int t = 0; t < MAXV; t++) {
         const int v = threadIdx.x + t * NT;
         if (v >= nv) continue;
-        const float4 g = ld4(a.g_norm + 4 * v);
+        float4 g;
+        if constexpr (AHEAD) g = gn[t]; else g = ld4(a.g_norm + 4 * v);
         x[t].x = x[t].x * inv * g.x; x[t].y = x[t].y * inv * g.y; x[t].z = x[t].z * inv * g.z; x[t].w = x[t].w * inv * g.w;
         amax = fmaxf(amax, amax4(x[t]));
     }
@@ -1111,9 +1123,23 @@ __global__ __launch_bounds__(NT) void k_norm_bwd_rows(KARGS24)
         rows[t] = r; cols[t] = 4 * v; ok[t] = v < nv;
         if (v < nv) x[t] = ld4(a.x_saved + r * D + 4 * v);
     }
+    // one value per thread: the norm weights and the gradient to add to are requested with the row, not after the planes
+    // and the reduction (a round trip each); with more values per thread the registers are worth more
+    constexpr bool AHEAD = MAXV == 1;
+    float4 dprev[MAXV], xb[MAXV], gb[MAXV];
+    if constexpr (AHEAD) {
+        const int v = threadIdx.x;
+        dprev[0] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv) g[0] = ld4(a.g + 4 * v);
+        if (v < nv && a.dx_prev) dprev[0] = ld4(a.dx_prev + r * D + 4 * v);
+        xb[0] = gb[0] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < nv && a.d16 && a.branch_raw) { xb[0] = ld4(a.branch_raw + r * D + 4 * v); gb[0] = ld4(a.g_branch + 4 * v); }
+    }
     planes_at4_multi<MAXV, (MAXV == 1 ? 20 : NT == RB ? 4 : 3), GROUPED>(a.dy, rows, cols, ok, dy);      // (many rows: 92 registers instead of 108)
+    if constexpr (!AHEAD) {
 #pragma unroll
-    for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) g[t] = ld4(a.g + 4 * v); }
+        for (int t = 0; t < MAXV; t++) { const int v = threadIdx.x + t * NT; if (v < nv) g[t] = ld4(a.g + 4 * v); }
+    }
 #pragma unroll
     for (int t = 0; t < MAXV; t++) {
         ss += sumsq4(x[t]);
@@ -1130,7 +1156,11 @@ __global__ __launch_bounds__(NT) void k_norm_bwd_rows(KARGS24)
         if (v >= nv) continue;
         dx[t] = make_float4((g[t].x * dy[t].x - coeff * x[t].x) * inv, (g[t].y * dy[t].y - coeff * x[t].y) * inv,
                             (g[t].z * dy[t].z - coeff * x[t].z) * inv, (g[t].w * dy[t].w - coeff * x[t].w) * inv);
-        if (a.dx_prev) { const float4 p = ld4(a.dx_prev + r * D + 4 * v); dx[t].x += p.x; dx[t].y += p.y; dx[t].z += p.z; dx[t].w += p.w; }
+        if (a.dx_prev) {
+            float4 p;
+            if constexpr (AHEAD) p = dprev[t]; else p = ld4(a.dx_prev + r * D + 4 * v);
+            dx[t].x += p.x; dx[t].y += p.y; dx[t].z += p.z; dx[t].w += p.w;
+        }
         if (a.clamp > 0.f) {
             dx[t].x = fminf(fmaxf(dx[t].x, -a.clamp), a.clamp); dx[t].y = fminf(fmaxf(dx[t].y, -a.clamp), a.clamp);
             dx[t].z = fminf(fmaxf(dx[t].z, -a.clamp), a.clamp); dx[t].w = fminf(fmaxf(dx[t].w, -a.clamp), a.clamp);
@@ -1145,8 +1175,8 @@ __global__ __launch_bounds__(NT) void k_norm_bwd_rows(KARGS24)
         for (int t = 0; t < MAXV; t++) {
             const int v = threadIdx.x + t * NT;
             if (v >= nv) continue;
-            x[t] = ld4(a.branch_raw + r * D + 4 * v);
-            g[t] = ld4(a.g_branch + 4 * v);
+            if constexpr (AHEAD) { x[t] = xb[t]; g[t] = gb[t]; }
+            else { x[t] = ld4(a.branch_raw + r * D + 4 * v); g[t] = ld4(a.g_branch + 4 * v); }
             ssb += sumsq4(x[t]);
             dotb += dx[t].x * g[t].x * x[t].x + dx[t].y * g[t].y * x[t].y + dx[t].z * g[t].z * x[t].z + dx[t].w * g[t].w * x[t].w;
         }
