@@ -259,8 +259,8 @@ def main():
 def _main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: 200 training steps, or 20 decoded tokens with --decode)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: 20, or 3 with --decode)")
     ap.add_argument("--config", default="c3_qwen3_4b_f16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seq", type=int, default=0, help="override the configuration's sequence length (experiments only)")
@@ -292,6 +292,10 @@ def _main():
                     help="only run the library's plain copy kernel (1 GiB in, 1 GiB out, 5 launches): "
                          "the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
+    if args.steps is None:
+        args.steps = 20 if args.decode else 200
+    if args.warmup is None:
+        args.warmup = 3 if args.decode else 20
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the step has no multi-GPU path); use --gpus 1",
               file=sys.stderr)
@@ -376,7 +380,7 @@ def _main():
         loss = float(np.mean(loss[:, 32:]))                # mean log-probability of the sampled tokens
 
     # dominant kernel: the weight-streaming GEMM, timed launch by launch with HIP events on the library's stream
-    prof_steps = max(1, min(5, args.steps))
+    prof_steps = max(1, min(20, args.steps))
     L.hip_gemm_profile_enable(1)
     for i in range(prof_steps):
         step(i)
