@@ -870,13 +870,16 @@ BatchRun &batch_acquire(InferenceState *s, BatchRun *&slot, int B)
     const int fmt = s->borrows_tiles ? s->borrowed_lm.fmt : 0;
     for (const auto &nk : shapes) {
         a16_elems = std::max(a16_elems, tiled_elems(2 * B, nk[1]));
-        for (int ring = 0; ring < 2; ring++) {                           // either kernel policy may be switched in later
-            const int was = gemm_ring_enabled();
-            set_gemm_ring(ring);
-            const int nbq = !fmt ? 0 : &nk == &shapes[0] ? tiled_rb(qd + 2 * kd) : tiled_rb(nk[0]);   // the adapter rows are F16 tiles
-            plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1], nbq, fmt).S * 2 * B * nk[0]);
-            set_gemm_ring(was);
-        }
+        for (int ring = 0; ring < 2; ring++)                             // either kernel policy may be switched in later
+            for (int wide = 0; wide <= ring; wide++) {                   // (the wide workgroups of the ring kernel may take twice the K chunks)
+                const int was = gemm_ring_enabled(), wide_was = gemm_ring_wide_mode();
+                set_gemm_ring(ring);
+                set_gemm_ring_wide(wide);
+                const int nbq = !fmt ? 0 : &nk == &shapes[0] ? tiled_rb(qd + 2 * kd) : tiled_rb(nk[0]);   // the adapter rows are F16 tiles
+                plane_floats = std::max(plane_floats, (size_t)plan_gemm(2 * B, nk[0], nk[1], nbq, fmt).S * 2 * B * nk[0]);
+                set_gemm_ring(was);
+                set_gemm_ring_wide(wide_was);
+            }
     }
     r.a16 = metal_buf_create(a16_elems * sizeof(half_t)); r.planes = fbuf(plane_floats);
     r.inv_ln = fbuf((size_t)2 * B); r.inv_br = fbuf((size_t)2 * B);

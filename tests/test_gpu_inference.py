@@ -212,6 +212,13 @@ def test_decode_at_the_benchmarked_widths(fmt, with_lora, from_sft):
             for b in range(8):
                 assert np.array_equal(got8[b], got8[0])
                 assert [int(t) for t in got8[b, :first_tie]] == gen[:first_tie], b
+            # twenty copies: 40 split rows, where the wide products of the streaming kernel take 128 weight rows per
+            # workgroup (gate|up, and down at twice the K chunks)
+            got20 = inf.generate_batch(prompt, 8, 20)
+            assert got20.shape == (20, 8)
+            for b in range(20):
+                assert np.array_equal(got20[b], got20[0])
+                assert [int(t) for t in got20[b, :first_tie]] == gen[:first_tie], b
 
     if from_sft:
         # the state reads the training state's tiles in place: it allocates caches, scratch and planes, nothing weight-sized
