@@ -214,8 +214,16 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
     __shared__ float sm[16];
     const int b = blockIdx.x, Kb = tiled_kb(D);
     x += (size_t)b * D;
-    float bv[EPT], v[EPT];
+    float bv[EPT], v[EPT], xv[EPT], gv[EPT], gbv[EPT];
     float inv_b = 1.f;
+    // the row, the norm weights and the branch norm's weights are requested with the planes, not after the reductions
+    // (a round trip each)
+#pragma unroll
+    for (int u = 0; u < EPT; u++) {
+        const int i = threadIdx.x + 1024 * u;
+        xv[u] = gv[u] = gbv[u] = 0.f;
+        if (i < D) { xv[u] = x[i]; gv[u] = g[i]; if (br.P && g_branch) gbv[u] = g_branch[i]; }
+    }
     if (br.P) {
 #pragma unroll
         for (int u = 0; u < EPT; u++) { const int i = threadIdx.x + 1024 * u; bv[u] = i < D ? planes_at(br, B, b, i) : 0.f; }
@@ -232,8 +240,8 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
         const int i = threadIdx.x + 1024 * u;
         v[u] = 0.f;
         if (i < D) {
-            v[u] = x[i];
-            if (br.P) { v[u] += g_branch ? bv[u] * inv_b * g_branch[i] : bv[u]; x[i] = v[u]; }
+            v[u] = xv[u];
+            if (br.P) { v[u] += g_branch ? bv[u] * inv_b * gbv[u] : bv[u]; x[i] = v[u]; }
         }
         ss += v[u] * v[u];
     }
@@ -242,7 +250,7 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
 #pragma unroll
     for (int u = 0; u < EPT; u++) {
         const int i = threadIdx.x + 1024 * u;
-        v[u] = i < D ? v[u] * inv * g[i] : 0.f;
+        v[u] = i < D ? v[u] * inv * gv[u] : 0.f;
         if (ln && i < D) ln[(size_t)b * D + i] = v[u];
         amax = fmaxf(amax, fabsf(v[u]));
     }
