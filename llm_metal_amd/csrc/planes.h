@@ -54,6 +54,10 @@ __device__ __forceinline__ float4 planes_at4(const Planes &P, size_t row, int co
 template <int T, int NB, bool GROUPED = false, int NBH = NB>
 __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (&row)[T], const int (&col)[T], const bool (&ok)[T], float4 (&s)[T])
 {
+    // the rows' factors are requested before the planes (after the sums they would cost a round trip of their own)
+    float rs[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) rs[t] = (!GROUPED && P.row_scale && ok[t]) ? P.row_scale[row[t]] : 1.0f;
     if (P.half_unscale != 0.f) {                          // uniform
         typedef _Float16 half4v __attribute__((ext_vector_type(4)));
         const half_t *ph[T];
@@ -90,7 +94,7 @@ __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (
         for (int i0 = 0; i0 < P.S; i0 += NBH) hbatch(i0);
 #pragma unroll
         for (int t = 0; t < T; t++) {
-            const float f = P.half_unscale * ((!GROUPED && P.row_scale && ok[t]) ? P.row_scale[row[t]] : 1.0f);
+            const float f = P.half_unscale * rs[t];
             s[t].x *= f; s[t].y *= f; s[t].z *= f; s[t].w *= f;
         }
         return;
@@ -133,7 +137,7 @@ __device__ __forceinline__ void planes_at4_multi(const Planes &P, const size_t (
     if (!GROUPED && P.row_scale) {
 #pragma unroll
         for (int t = 0; t < T; t++)
-            if (ok[t]) { const float f = P.row_scale[row[t]]; s[t].x *= f; s[t].y *= f; s[t].z *= f; s[t].w *= f; }
+            if (ok[t]) { const float f = rs[t]; s[t].x *= f; s[t].y *= f; s[t].z *= f; s[t].w *= f; }
     }
 }
 
@@ -142,6 +146,7 @@ template <int T, int NB>
 __device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, const int (&col)[T], const bool (&ok)[T], float (&s)[T])
 {
     const float *p[T];
+    const float rs = P.row_scale ? P.row_scale[row] : 1.0f;   // requested before the planes, not after their sums
 #pragma unroll
     for (int t = 0; t < T; t++) { p[t] = P.p + row * P.ld + col[t]; s[t] = 0.f; }
     auto batch = [&](int i0) __attribute__((always_inline)) {
@@ -157,9 +162,8 @@ __device__ __forceinline__ void planes_at_multi(const Planes &P, size_t row, con
     };
     for (int i0 = 0; i0 < P.S; i0 += NB) batch(i0);
     if (P.row_scale) {
-        const float f = P.row_scale[row];
 #pragma unroll
-        for (int t = 0; t < T; t++) s[t] *= f;
+        for (int t = 0; t < T; t++) s[t] *= rs;
     }
 }
 
