@@ -55,6 +55,19 @@ __device__ __forceinline__ void block_sum2(float &a, float &b, float *smem)
     a = ra; b = rb;
 }
 
+// A sum and a maximum for one pair of barriers; `smem` must hold 32 floats.  The sum is formed in the order block_sum forms it.
+__device__ __forceinline__ void block_sum_max(float &a, float &m, float *smem)
+{
+    a = wave_sum(a); m = wave_max(m);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    if (lane == 0) { smem[w] = a; smem[16 + w] = m; }
+    __syncthreads();
+    float ra = 0.f, rm = smem[16];
+    for (int i = 0; i < nw; i++) { ra += smem[i]; rm = fmaxf(rm, smem[16 + i]); }
+    __syncthreads();
+    a = ra; m = rm;
+}
+
 __device__ __forceinline__ float block_max(float v, float *smem)
 {
     v = wave_max(v);

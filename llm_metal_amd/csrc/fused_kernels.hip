@@ -59,7 +59,7 @@ template <int MAXV, bool GROUPED, int NT = RB>
 __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
 {
     KARGS_HOT(NormRowsArgs, a);                           // rows_launched, D, pf
-    __shared__ float sm[16];
+    __shared__ float sm[32];
     if (blockIdx.x >= a.rows_launched) {                  // workgroups beyond the rows fetch weights; they are the last
         prefetch_weight_tiles<NT>(a.pf, blockIdx.x - a.rows_launched);      // to finish and have nothing to wait for
         return;
@@ -128,19 +128,35 @@ __global__ __launch_bounds__(NT) void k_norm_rows(KARGS24)
     float ss = 0.f;
 #pragma unroll
     for (int t = 0; t < MAXV; t++) ss += sumsq4(x[t]);
-    ss = block_sum(ss, sm);
-    const float inv = rsqrtf(ss / (float)D + a.eps);
-    float amax = 0.f;
+    float amax = 0.f, inv;
+    if constexpr (AHEAD) {
+        // the norm weights are here already: the row maximum of x g, which the factor 1 / rms scales like every entry,
+        // goes through the same pair of barriers as the sum of squares
+        float mxg = 0.f;
 #pragma unroll
-    for (int t = 0; t < MAXV; t++) {
-        const int v = threadIdx.x + t * NT;
-        if (v >= nv) continue;
-        float4 g;
-        if constexpr (AHEAD) g = gn[t]; else g = ld4(a.g_norm + 4 * v);
-        x[t].x = x[t].x * inv * g.x; x[t].y = x[t].y * inv * g.y; x[t].z = x[t].z * inv * g.z; x[t].w = x[t].w * inv * g.w;
-        amax = fmaxf(amax, amax4(x[t]));
+        for (int t = 0; t < MAXV; t++)
+            mxg = fmaxf(mxg, amax4(make_float4(x[t].x * gn[t].x, x[t].y * gn[t].y, x[t].z * gn[t].z, x[t].w * gn[t].w)));
+        block_sum_max(ss, mxg, sm);
+        inv = rsqrtf(ss / (float)D + a.eps);
+        amax = mxg * inv;
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const float4 g = gn[t];
+            x[t].x = x[t].x * inv * g.x; x[t].y = x[t].y * inv * g.y; x[t].z = x[t].z * inv * g.z; x[t].w = x[t].w * inv * g.w;
+        }
+    } else {
+        ss = block_sum(ss, sm);
+        inv = rsqrtf(ss / (float)D + a.eps);
+#pragma unroll
+        for (int t = 0; t < MAXV; t++) {
+            const int v = threadIdx.x + t * NT;
+            if (v >= nv) continue;
+            const float4 g = ld4(a.g_norm + 4 * v);
+            x[t].x = x[t].x * inv * g.x; x[t].y = x[t].y * inv * g.y; x[t].z = x[t].z * inv * g.z; x[t].w = x[t].w * inv * g.w;
+            amax = fmaxf(amax, amax4(x[t]));
+        }
+        amax = block_max(amax, sm);
     }
-    amax = block_max(amax, sm);
     const float s = row_scale_for(amax);
     const int Kb = tiled_kb(D);
 #pragma unroll

@@ -211,7 +211,7 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
                                                          const float *__restrict__ g, float *__restrict__ ln,
                                                          half_t *__restrict__ a16, float *__restrict__ inv_out, int B, int D, float eps)
 {
-    __shared__ float sm[16];
+    __shared__ float sm[32];
     const int b = blockIdx.x, Kb = tiled_kb(D);
     x += (size_t)b * D;
     float bv[EPT], v[EPT], xv[EPT], gv[EPT], gbv[EPT];
@@ -245,17 +245,20 @@ __global__ __launch_bounds__(1024) void k_add_norm_split(float *__restrict__ x, 
         }
         ss += v[u] * v[u];
     }
-    const float inv = rsqrtf(block_sum(ss, sm) / (float)D + eps);
-    float amax = 0.f;
+    // the row maximum of v g, which the factor 1 / rms scales like every entry, goes through the same pair of barriers
+    // as the sum of squares
+    float mxg = 0.f;
+#pragma unroll
+    for (int u = 0; u < EPT; u++) mxg = fmaxf(mxg, fabsf(v[u] * gv[u]));
+    block_sum_max(ss, mxg, sm);
+    const float inv = rsqrtf(ss / (float)D + eps);
 #pragma unroll
     for (int u = 0; u < EPT; u++) {
         const int i = threadIdx.x + 1024 * u;
         v[u] = i < D ? v[u] * inv * gv[u] : 0.f;
         if (ln && i < D) ln[(size_t)b * D + i] = v[u];
-        amax = fmaxf(amax, fabsf(v[u]));
     }
-    amax = block_max(amax, sm);
-    const float s = row_scale_for(amax), is = 1.0f / s;
+    const float s = row_scale_for(mxg * inv), is = 1.0f / s;
     float lmax = 0.f;
 #pragma unroll
     for (int u = 0; u < EPT; u++) {
