@@ -447,3 +447,34 @@ def test_ids_outside_the_vocabulary_launch_nothing_and_two_enqueues_do_not_race(
         st.train_step(tok, tgt, 1e-4)
         assert st.train_step(tok2, tgt2, 1e-4) == loss2
         assert np.array_equal(st.lora(), after2)
+
+
+def test_states_give_their_device_memory_back():
+    """sft_state_free / inference_state_free: a second and a third state of the same shape, each stepped once, leave as
+    much device memory free as the first did (the library's scratch arenas only grow, so the first round sets the level)."""
+    import ctypes
+    from llm_metal_amd import lib
+    from llm_metal_amd.sft import InferenceState
+    L = lib.load()
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        L.hip_mem_info(ctypes.byref(free), ctypes.byref(total))
+        return free.value
+
+    cfg = C1.with_(name="leak_check", NL=2)
+    model = make_model(cfg, seed=3)
+    tok, tgt = make_batch(cfg, seed=4)
+    levels = []
+    for _ in range(3):
+        with SFTState(cfg, model) as st:
+            st.train_step(tok, tgt, 1e-4)
+            with InferenceState(sft=st, max_seq=32) as inf:
+                inf.forward_token(int(tok[0]))
+                inf.generate_batch([int(t) for t in tok[:4]], 3, 2)
+        with InferenceState(cfg, model, max_seq=32, use_fp16=True) as inf:
+            inf.generate([int(t) for t in tok[:4]], 3)
+        L.metal_flush()
+        levels.append(free_bytes())
+    assert levels[2] >= levels[1] - (1 << 20), levels              # nothing kept from round to round
+    assert levels[1] >= levels[0] - (64 << 20), levels             # (arenas may still grow once after the first round)
