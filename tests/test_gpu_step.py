@@ -478,3 +478,20 @@ def test_states_give_their_device_memory_back():
         levels.append(free_bytes())
     assert levels[2] >= levels[1] - (1 << 20), levels              # nothing kept from round to round
     assert levels[1] >= levels[0] - (64 << 20), levels             # (arenas may still grow once after the first round)
+
+
+@pytest.mark.parametrize("fmt", ["f16", "q8_0"])
+def test_the_step_is_deterministic(fmt):
+    """No kernel of the step adds through atomics or depends on the order in which workgroups finish: two states made from
+    the same model, stepped on the same batches, hold bit-identical losses, logits, gradients and adapters."""
+    cfg = C1.with_(name="twice", NL=2, D=320, Hq=5, Hkv=1, hd=64, IS=416, V=1056, seq=48, weight_format=fmt)
+    model = make_model(cfg, seed=11, gamma_jitter=0.1)
+    batches = [make_batch(cfg, seed=12 + i) for i in range(3)]
+    runs = []
+    for _ in range(2):
+        with SFTState(cfg, model) as st:
+            losses = [st.train_step(tok, tgt, 1e-3) for tok, tgt in batches]
+            runs.append((losses, st.logits().copy(), st.lora_grads().copy(), st.lora().copy()))
+    assert runs[0][0] == runs[1][0], (runs[0][0], runs[1][0])
+    for a, b in zip(runs[0][1:], runs[1][1:]):
+        assert np.array_equal(a, b)
