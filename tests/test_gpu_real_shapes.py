@@ -212,6 +212,25 @@ def test_config3_as_benchmarked(qwen3_4b_model):
         _zero_b_properties(C3, st, qwen3_4b_model)
 
 
+def test_config3_as_benchmarked_on_both_workgroup_shapes_of_the_ring_kernel(qwen3_4b_model):
+    """1 x 64 rows on F16 weights, all layers: with gemm_ring_wide on five product shapes (the default) and with gemm_ring
+    alone the step gives the same loss and gradient norm; so does the register-staged kernel."""
+    L = lib.load()
+    with SFTState(C3, qwen3_4b_model) as st:
+        tok, tgt = make_batch(C3, seed=100)
+        out = {}
+        for ring, wide in ((1, 1), (1, 0), (0, 0)):
+            L.hip_gemm_ring(ring)
+            L.hip_gemm_ring_wide(wide)
+            st.set_lora(qwen3_4b_model["lora"])
+            out[ring, wide] = (st.train_step(tok, tgt, 0.0), st.grad_norm())   # lr 0: the adapters stay put
+        L.hip_gemm_ring(1)
+        L.hip_gemm_ring_wide(1)
+        for other in ((1, 0), (0, 0)):
+            assert abs(out[other][0] - out[1, 1][0]) <= 1e-3 * out[1, 1][0], out
+            assert abs(out[other][1] - out[1, 1][1]) <= 1e-2 * out[1, 1][1], out
+
+
 def test_config3_with_q8_weights_as_benchmarked_and_the_two_streaming_kernels_agree(qwen3_4b_model):
     """1 x 64 rows on Q8_0 weights, all layers: the products take gemm_ring and gemm_ring_wide with the tiles quantised up to
     LDS (and planes of halves); on gemm_ring alone, and on the register-staged kernel, the step must give the same loss and
